@@ -1,0 +1,249 @@
+"""ctypes front end of the CPU oracle (``kge_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY.  Importable from ``tests/``, the smoke check and the
+bench's ``cpu_baseline`` leg; never from the product package.  ``build()``
+compiles the two libraries with the Makefile beside this file.
+"""
+
+import ctypes as C
+import os
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+HERE = Path(__file__).resolve().parent
+
+SCORE = {"TransE": 0, "DistMult": 1}
+DIST = {"L1": 0, "L2": 1, "MatMul": 2}
+LOSS = {"logsigmoid": 0, "softmax": 1}
+STORE = {"float32": 0, "float16": 1, "bfloat16_embedding": 2}
+
+
+class Cfg(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "n_shard", "n_entity", "n_relation", "dim", "feature", "batch", "a2a", "score_fn",
+        "distance_fn", "loss_fn", "shared_table", "storage")] + [(n, C.c_float) for n in (
+            "gamma", "beta_m", "beta_v", "epsilon", "weight_decay", "loss_scale",
+            "softmax_correction_weight", "negative_adversarial_scale", "lr_mod_entity",
+            "lr_mod_relation", "lr_mod_projection")]
+
+
+def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score_fn="TransE",
+             distance_fn="L1", loss_fn="logsigmoid", shared_table=False, storage="float32",
+             gamma=0.0, beta_m=0.9, beta_v=0.999, epsilon=1e-8, weight_decay=0.0,
+             loss_scale=None, softmax_correction_weight=0.0, negative_adversarial_scale=0.0,
+             lr_mod_entity=1.0, lr_mod_relation=1.0, lr_mod_projection=1.0):
+    if loss_scale is None:  # src/python/poplar_kge.py:259-262
+        loss_scale = float(batch * n_shard * a2a)
+    return Cfg(n_shard, n_entity, n_relation, dim, feature, batch, a2a, SCORE[score_fn],
+               DIST[distance_fn], LOSS[loss_fn], int(shared_table), STORE[storage], gamma, beta_m,
+               beta_v, epsilon, weight_decay, loss_scale, softmax_correction_weight,
+               negative_adversarial_scale, lr_mod_entity, lr_mod_relation, lr_mod_projection)
+
+
+def build(force=False):
+    libs = [HERE / "libkge_oracle_f64.so", HERE / "libkge_oracle_f32.so"]
+    src = HERE / "kge_oracle.c"
+    if force or any(not p.exists() or p.stat().st_mtime < src.stat().st_mtime for p in libs):
+        subprocess.run(["make", "-C", str(HERE), "-B" if force else "-s", "all"], check=True)
+    return libs
+
+
+def _f32(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a
+
+
+def _u32(a):
+    return np.ascontiguousarray(a, dtype=np.uint32)
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class Oracle:
+    """One loaded oracle library; ``precision`` is "f64" (truth) or "f32"."""
+
+    def __init__(self, precision="f64"):
+        path = HERE / f"libkge_oracle_{precision}.so"
+        if not path.exists():
+            build()
+        self.lib = C.CDLL(os.fspath(path))
+        self.lib.kge_oracle_loss.restype = C.c_float
+        self.lib.kge_oracle_adam_step_size.restype = C.c_float
+        self.lib.kge_oracle_round.restype = C.c_float
+        self.lib.kge_oracle_round.argtypes = [C.c_float, C.c_int]
+        self.precision = precision
+
+    # -- ops ---------------------------------------------------------------
+    def buffer_read(self, buf, idx):
+        buf, idx = _f32(buf), _u32(idx)
+        out = np.empty((idx.size, buf.shape[1]), np.float32)
+        self.lib.kge_oracle_buffer_read(_p(buf), C.c_int64(buf.shape[1]), _p(idx),
+                                        C.c_int64(idx.size), _p(out))
+        return out
+
+    def buffer_write(self, buf, idx, data):
+        assert buf.dtype == np.float32 and buf.flags.c_contiguous
+        idx, data = _u32(idx), _f32(data)
+        self.lib.kge_oracle_buffer_write(_p(buf), C.c_int64(buf.shape[1]), _p(idx),
+                                         C.c_int64(idx.size), _p(data))
+
+    def multi_slice(self, t, idx):
+        t, idx = _f32(t), _u32(idx)
+        out = np.empty((idx.size, t.shape[1]), np.float32)
+        self.lib.kge_oracle_multi_slice(_p(t), C.c_int64(t.shape[1]), _p(idx),
+                                        C.c_int64(idx.size), _p(out))
+        return out
+
+    def multi_update_add(self, rows, idx, grad_out):
+        idx, grad_out = _u32(idx), _f32(grad_out)
+        out = np.empty((rows, grad_out.shape[1]), np.float32)
+        self.lib.kge_oracle_multi_update_add(_p(out), C.c_int64(rows),
+                                             C.c_int64(grad_out.shape[1]), _p(idx),
+                                             C.c_int64(idx.size), _p(grad_out))
+        return out
+
+    def _dist(self, fn, a, b):
+        a, b = _f32(a), _f32(b)
+        out = np.empty((a.shape[0], b.shape[0]), np.float32)
+        fn(_p(a), _p(b), C.c_int64(a.shape[0]), C.c_int64(b.shape[0]), C.c_int64(a.shape[1]),
+           _p(out))
+        return out
+
+    def l1_distance(self, a, b):
+        return self._dist(self.lib.kge_oracle_l1_distance, a, b)
+
+    def l2_distance(self, a, b):
+        return self._dist(self.lib.kge_oracle_l2_distance, a, b)
+
+    def dot_score(self, a, b):
+        return self._dist(self.lib.kge_oracle_dot_score, a, b)
+
+    def l1_distance_grad(self, a, b, g):
+        """Gradient of the first operand; call with (b, a, g.T) for the second."""
+        a, b, g = _f32(a), _f32(b), _f32(g)
+        out = np.empty_like(a)
+        self.lib.kge_oracle_l1_distance_grad(_p(a), _p(b), _p(g), C.c_int64(a.shape[0]),
+                                             C.c_int64(b.shape[0]), C.c_int64(a.shape[1]), _p(out))
+        return out
+
+    def l2_distance_grad(self, a, b, dist, g):
+        a, b, dist, g = _f32(a), _f32(b), _f32(dist), _f32(g)
+        out = np.empty_like(a)
+        self.lib.kge_oracle_l2_distance_grad(_p(a), _p(b), _p(dist), _p(g),
+                                             C.c_int64(a.shape[0]), C.c_int64(b.shape[0]),
+                                             C.c_int64(a.shape[1]), _p(out))
+        return out
+
+    def log_sigmoid(self, x):
+        x = _f32(x)
+        y = np.empty_like(x)
+        self.lib.kge_oracle_log_sigmoid(_p(x), C.c_int64(x.size), _p(y))
+        return y
+
+    def log_sigmoid_grad(self, x, dy):
+        x, dy = _f32(x), _f32(dy)
+        dx = np.empty_like(x)
+        self.lib.kge_oracle_log_sigmoid_grad(_p(x), _p(dy), C.c_int64(x.size), _p(dx))
+        return dx
+
+    def log_softmax(self, x):
+        x = _f32(x)
+        x2 = x.reshape(-1, x.shape[-1])
+        y = np.empty_like(x2)
+        self.lib.kge_oracle_log_softmax(_p(x2), C.c_int64(x2.shape[0]), C.c_int64(x2.shape[1]),
+                                        _p(y))
+        return y.reshape(x.shape)
+
+    def log_softmax_grad(self, y, dy):
+        y, dy = _f32(y), _f32(dy)
+        y2, dy2 = y.reshape(-1, y.shape[-1]), dy.reshape(-1, y.shape[-1])
+        dx = np.empty_like(y2)
+        self.lib.kge_oracle_log_softmax_grad(_p(y2), _p(dy2), C.c_int64(y2.shape[0]),
+                                             C.c_int64(y2.shape[1]), _p(dx))
+        return dx.reshape(y.shape)
+
+    def softmax_cross_entropy(self, logits, labels):
+        logits, labels = _f32(logits), _u32(labels)
+        l2 = logits.reshape(-1, logits.shape[-1])
+        out = np.empty(l2.shape[0], np.float32)
+        self.lib.kge_oracle_softmax_cross_entropy(_p(l2), _p(labels), C.c_int64(l2.shape[0]),
+                                                  C.c_int64(l2.shape[1]), _p(out))
+        return out
+
+    def softmax(self, x):
+        x = _f32(x)
+        x2 = x.reshape(-1, x.shape[-1])
+        y = np.empty_like(x2)
+        self.lib.kge_oracle_softmax(_p(x2), C.c_int64(x2.shape[0]), C.c_int64(x2.shape[1]), _p(y))
+        return y.reshape(x.shape)
+
+    def adam_step_size(self, step, lr, beta_m=0.9, beta_v=0.999):
+        """Returns (new_step, alpha)."""
+        st = C.c_uint32(step)
+        alpha = self.lib.kge_oracle_adam_step_size(C.byref(st), C.c_float(lr), C.c_float(beta_m),
+                                                   C.c_float(beta_v))
+        return st.value, alpha
+
+    def adam(self, p, m, v, g, alpha, beta_m=0.9, beta_v=0.999, eps=1e-8, wd=0.0,
+             v_is_sqrt=False):
+        """In-place on float32 contiguous p, m, v."""
+        for a in (p, m, v):
+            assert a.dtype == np.float32 and a.flags.c_contiguous
+        g = _f32(g)
+        self.lib.kge_oracle_adam(_p(p), _p(m), _p(v), _p(g), C.c_int64(p.size), C.c_float(alpha),
+                                 C.c_float(beta_m), C.c_float(beta_v), C.c_float(eps),
+                                 C.c_float(wd), C.c_int(int(v_is_sqrt)))
+
+    def round(self, x, storage):
+        return np.array([self.lib.kge_oracle_round(float(v), STORE[storage])
+                         for v in np.asarray(x, np.float32).ravel()],
+                        np.float32).reshape(np.shape(x))
+
+    def loss(self, cfg, score, label):
+        """Shard loss and d(loss)/d(score) (before the loss scale)."""
+        score, label = _f32(score), _u32(label)
+        ds = np.empty_like(score)
+        loss = self.lib.kge_oracle_loss(C.byref(cfg), _p(score), _p(label), _p(ds))
+        return loss, ds
+
+    # -- whole step --------------------------------------------------------
+    def train_step_loop(self, cfg, state, lr, batch):
+        """Runs n_step steps in place on ``state`` and returns loss f32[S].
+
+        state: dict with float32 C-contiguous arrays ``entity_data``
+        [n_tables*n_entity, 3D+F], ``relation_embedding`` (+ ``/adam_m``,
+        ``/adam_v``), ``feature_projection`` (+ moments; may be absent when
+        F == 0) and an int ``step``.  batch: dict of uint32 arrays laid out
+        [S, n_step, ...] as the host passes them.
+        """
+        S = cfg.n_shard
+        remote = _u32(batch["remote"])
+        n_step = remote.shape[1]
+        a2a, head = _u32(batch["a2a"]), _u32(batch["head"])
+        relation, tail = _u32(batch["relation"]), _u32(batch["tail"])
+        lr = _f32(np.broadcast_to(np.asarray(lr, np.float32), (S,)))
+        for k in ("entity_data", "relation_embedding", "relation_embedding/adam_m",
+                  "relation_embedding/adam_v"):
+            assert state[k].dtype == np.float32 and state[k].flags.c_contiguous, k
+        if cfg.feature:
+            proj = [state["feature_projection"], state["feature_projection/adam_m"],
+                    state["feature_projection/adam_v"]]
+            for a in proj:
+                assert a.dtype == np.float32 and a.flags.c_contiguous
+            proj = [_p(a) for a in proj]
+        else:
+            proj = [None, None, None]
+        step = C.c_uint32(int(state["step"]))
+        loss = np.zeros(S, np.float32)
+        rc = self.lib.kge_oracle_train_step_loop(
+            C.byref(cfg), C.c_int32(n_step), _p(state["entity_data"]),
+            _p(state["relation_embedding"]), _p(state["relation_embedding/adam_m"]),
+            _p(state["relation_embedding/adam_v"]), *proj, C.byref(step), _p(lr), _p(remote),
+            _p(a2a), _p(head), _p(relation), _p(tail), _p(loss))
+        assert rc == 0
+        state["step"] = step.value
+        return loss

@@ -1,0 +1,102 @@
+"""Seeded synthetic states and batches shared by the oracle and GPU parity tests."""
+
+import numpy as np
+
+
+def cfg_dict(**kw):
+    d = dict(n_shard=2, n_entity=90, n_relation=12, dim=8, feature=6, batch=6, a2a=5,
+             score_fn="TransE", distance_fn="L1", loss_fn="logsigmoid", shared_table=False,
+             storage="float32", gamma=2.0, beta_m=0.9, beta_v=0.999, epsilon=1e-8,
+             weight_decay=0.0, loss_scale=None, softmax_correction_weight=0.0,
+             negative_adversarial_scale=0.0)
+    d.update(kw)
+    if d["loss_scale"] is None:
+        d["loss_scale"] = float(d["batch"] * d["n_shard"] * d["a2a"])
+    return d
+
+
+def make_state(c, rng, warm=True, scale=None):
+    """Random tables.  ``warm``: non-zero Adam moments and step, so the update
+    formula is exercised away from its zero-state special case."""
+    S, NE, D, F, NR = c["n_shard"], c["n_entity"], c["dim"], c["feature"], c["n_relation"]
+    rows = NE if c["shared_table"] else S * NE
+    scale = scale if scale is not None else 1.0 / np.sqrt(D)
+    ed = np.zeros((rows, 3 * D + F), np.float32)
+    ed[:, :D] = rng.normal(0, scale, (rows, D))
+    if warm:
+        ed[:, D:2 * D] = rng.normal(0, 0.1, (rows, D))
+        ed[:, 2 * D:3 * D] = np.abs(rng.normal(0, 0.3, (rows, D)))
+    if F:
+        ed[:, 3 * D:] = rng.normal(0, 1, (rows, F)).astype(np.float16)
+    st = {
+        "entity_data": ed,
+        "relation_embedding": rng.normal(0, scale, (NR, D)).astype(np.float32),
+        "relation_embedding/adam_m": (rng.normal(0, 0.1, (NR, D)) * warm).astype(np.float32),
+        "relation_embedding/adam_v": (rng.normal(0, 0.3, (NR, D))**2 * warm).astype(np.float32),
+        "step": 7 if warm else 0,
+    }
+    if F:
+        st["feature_projection"] = rng.normal(0, scale / np.sqrt(F), (F, D)).astype(np.float32)
+        st["feature_projection/adam_m"] = (rng.normal(0, 0.1, (F, D)) * warm).astype(np.float32)
+        st["feature_projection/adam_v"] = (rng.normal(0, 0.3, (F, D))**2 * warm).astype(np.float32)
+    return st
+
+
+def copy_state(st):
+    return {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in st.items()}
+
+
+def random_batch(c, n_step, rng, pad=0):
+    """The reference test's batch shape (tests/python/test_poplar_kge.py:51-91):
+    ``remote`` sorted unique non-zero rows (the last ``pad`` entries zero
+    padding), random slots for head / a2a, random relations and labels."""
+    S, NE, B, A = c["n_shard"], c["n_entity"], c["batch"], c["a2a"]
+    NR = B + S * A
+    remote = np.zeros((S, n_step, NR), np.uint32)
+    for s in range(S):
+        for i in range(n_step):
+            remote[s, i, :NR - pad] = np.sort(rng.choice(np.arange(1, NE), NR - pad, replace=False))
+    lim = NR - pad if pad else NR
+    return dict(
+        remote=remote,
+        a2a=rng.integers(0, lim, (S, n_step, S, A)).astype(np.uint32),
+        head=rng.integers(0, lim, (S, n_step, B)).astype(np.uint32),
+        relation=rng.integers(0, c["n_relation"], (S, n_step, B)).astype(np.uint32),
+        tail=rng.integers(0, S * A, (S, n_step, B)).astype(np.uint32),
+    )
+
+
+def zipf_ids(rng, n_rows, size, s=1.1):
+    """Bounded power law P(k) ~ k^-s over ids 1..n_rows-1, inverse-CDF sampled."""
+    k = np.arange(1, n_rows, dtype=np.float64)
+    cdf = np.cumsum(k**-s)
+    cdf /= cdf[-1]
+    return (1 + np.searchsorted(cdf, rng.random(size))).astype(np.uint32)
+
+
+def raw_batch(c, n_step, rng, zipf=True):
+    """Raw (non-deduplicated) ids with identity slot maps: ``remote`` holds
+    every head id then every tail id the shard sends; duplicates allowed."""
+    S, NE, B, A = c["n_shard"], c["n_entity"], c["batch"], c["a2a"]
+    T = S * A
+    NR = B + T
+    shape = (S, n_step, NR)
+    remote = zipf_ids(rng, NE, shape) if zipf else rng.integers(1, NE, shape).astype(np.uint32)
+    head = np.broadcast_to(np.arange(B, dtype=np.uint32), (S, n_step, B)).copy()
+    a2a = np.broadcast_to((B + np.arange(T, dtype=np.uint32)).reshape(S, A),
+                          (S, n_step, S, A)).copy()
+    return dict(
+        remote=remote, a2a=a2a, head=head,
+        relation=rng.integers(0, c["n_relation"], (S, n_step, B)).astype(np.uint32),
+        tail=rng.integers(0, T, (S, n_step, B)).astype(np.uint32),
+    )
+
+
+def step_slice(batch, i):
+    return {k: v[:, i] for k, v in batch.items()}
+
+
+def rel_l2(x, ref):
+    x, ref = np.asarray(x, np.float64), np.asarray(ref, np.float64)
+    den = np.sqrt(np.sum(ref * ref))
+    return float(np.sqrt(np.sum((x - ref)**2)) / (den if den > 0 else 1.0))

@@ -1,0 +1,147 @@
+"""An independent torch-autograd restatement of one training step.
+
+Test infrastructure.  It follows the structure of the reference's own PyTorch
+oracle (tests/python/reference_model.py:113-152: gather by ``remote``, heads by
+``head``, tails by ``a2a`` then all-to-all as ``transpose(0, 1)``, broadcast
+score, weighted logsigmoid) generalised to the distance / score / loss
+variants of src/poplar_kge.cpp:469-499, 567-573, 615-660, and uses autograd
+for every gradient, so it shares no hand-derived backward with the C oracle.
+The optimiser is the reference formula (src/fructose/frnn.cpp:42-90) in
+float64 NumPy.  Everything runs in float64.
+"""
+
+import numpy as np
+import torch as T
+
+
+def log_sigmoid_clamped(x):
+    """src/pag/pag.cpp:888-910, forward and backward as the reference defines them."""
+
+    class Fn(T.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            ctx.save_for_backward(x)
+            return T.where(x > -11, -T.log1p(T.exp(-T.clamp(x, min=-11))), x)
+
+        @staticmethod
+        def backward(ctx, g):
+            (x,) = ctx.saved_tensors
+            return g / (1 + T.exp(T.clamp(x, max=11)))
+
+    return Fn.apply(x)
+
+
+def step(cfg, state, lr, batch_step):
+    """One step in place on ``state`` (float32 arrays); returns loss[S].
+
+    cfg: dict(n_shard, n_entity, n_relation, dim, feature, batch, a2a,
+    score_fn, distance_fn, loss_fn, shared_table, gamma, beta_m, beta_v,
+    epsilon, weight_decay, loss_scale, softmax_correction_weight,
+    negative_adversarial_scale).  batch_step: dict of int arrays for ONE step:
+    remote[S,B+T], a2a[S,S,A], head/relation/tail[S,B].
+    """
+    S, NE, D, F = cfg["n_shard"], cfg["n_entity"], cfg["dim"], cfg["feature"]
+    B, A = cfg["batch"], cfg["a2a"]
+    Tn = S * A
+    remote = T.tensor(batch_step["remote"].astype(np.int64))
+    a2a = T.tensor(batch_step["a2a"].astype(np.int64))
+    head = T.tensor(batch_step["head"].astype(np.int64))
+    relation = T.tensor(batch_step["relation"].astype(np.int64))
+    tail = T.tensor(batch_step["tail"].astype(np.int64))
+    shards = T.arange(S)
+
+    table = T.tensor(state["entity_data"].astype(np.float64))
+    base = T.zeros(S, dtype=T.int64) if cfg["shared_table"] else shards * NE
+    keys = base[:, None] + remote  # [S, NR] global row ids
+    # one leaf per distinct row so that duplicates share a gradient
+    uniq, inverse = T.unique(keys.reshape(-1), return_inverse=True)
+    emb = table[uniq, :D].clone().requires_grad_(True)
+    feat = table[uniq, 3 * D:]
+    rel = T.tensor(state["relation_embedding"].astype(np.float64), requires_grad=True)
+    params = [emb, rel]
+    if F:
+        proj = T.tensor(state["feature_projection"].astype(np.float64), requires_grad=True)
+        params.append(proj)
+        hidden_u = emb + feat @ proj
+    else:
+        hidden_u = emb
+    hidden = hidden_u[inverse].reshape(S, -1, D)  # [S, NR, D]
+
+    heads = hidden[shards[:, None], head]  # [S, B, D]
+    tails = hidden[shards[:, None, None], a2a]  # [S(src), S(dst), A, D]
+    tails = tails.transpose(0, 1).reshape(S, Tn, D)  # all-to-all
+    r = rel[relation]
+    if cfg["score_fn"] == "TransE":
+        pred = heads + r
+        if cfg["distance_fn"] == "L1":
+            dist = (pred[:, :, None, :] - tails[:, None, :, :]).abs().sum(-1)
+        elif cfg["distance_fn"] == "L2":
+            diff = pred[:, :, None, :] - tails[:, None, :, :]
+            sq = (diff * diff).sum(-1)
+            # the reference's L2 gradient is 0 at zero distance
+            safe = T.where(sq > 0, sq, T.ones_like(sq))
+            dist = T.where(sq > 0, T.sqrt(safe), T.zeros_like(sq))
+        else:
+            dist = pred @ tails.transpose(1, 2)
+        score = cfg["gamma"] - dist
+    else:
+        score = (heads * r) @ tails.transpose(1, 2)
+
+    onehot = T.nn.functional.one_hot(tail, Tn).to(T.float64)
+    if cfg["loss_fn"] == "logsigmoid":
+        w_pos, w_neg = 0.5 * Tn, 0.5 * Tn / (Tn - 1)
+        weight = onehot * (w_pos - w_neg) + w_neg
+        adv = cfg.get("negative_adversarial_scale", 0.0)
+        if adv > 0:
+            sm = T.softmax(adv * score.detach() - 10000.0 * onehot, dim=-1)
+            weight = weight * (onehot + (Tn - 1) * sm)
+        per_shard = -(weight * log_sigmoid_clamped((2 * onehot - 1) * score)).sum((1, 2)) / (
+            S * B * A * S)
+    else:
+        cw = cfg.get("softmax_correction_weight", 0.0)
+        corr = cw * np.float32(np.log(NE * S - 1) - np.log(S * A - 1)) if cw else 0.0
+        z = score + float(corr) * (1 - onehot)
+        per_shard = -(T.log_softmax(z, -1) * onehot).sum((1, 2)) / (S * B)
+    per_shard.sum().backward(T.tensor(float(cfg["loss_scale"]), dtype=T.float64))
+
+    # optimiser (float64 restatement of frnn.cpp:42-90)
+    state["step"] = int(state["step"]) + 1
+    st = state["step"]
+    # the hyper-parameters are float32 constants in the reference
+    bm, bv, eps, wd = (float(np.float32(cfg[k]))
+                       for k in ("beta_m", "beta_v", "epsilon", "weight_decay"))
+    lr = np.broadcast_to(np.asarray(lr, np.float64), (S,))
+    alpha = lr * np.sqrt(1 - bv**st) / (1 - bm**st)
+
+    def adam(p, m, v, g, a):
+        m[...] = bm * m + (1 - bm) * g
+        v[...] = bv * v + (1 - bv) * g * g
+        p[...] = p - a * (m / (np.sqrt(v) + eps) + wd * p)
+
+    g = emb.grad.numpy()
+    rows = uniq.numpy()
+    ed = state["entity_data"]
+    p = ed[rows, :D].astype(np.float64)
+    m = ed[rows, D:2 * D].astype(np.float64)
+    v = ed[rows, 2 * D:3 * D].astype(np.float64) ** 2
+    a_rows = alpha[0] if cfg["shared_table"] else alpha[rows // NE][:, None]
+    adam(p, m, v, g, a_rows)
+    ed[rows, :D] = p
+    ed[rows, D:2 * D] = m
+    ed[rows, 2 * D:3 * D] = np.sqrt(v)
+
+    def dense(name, grad):
+        n = state[name].shape[0]
+        a = alpha[0] if cfg["shared_table"] else alpha[np.arange(n) // (n // S)][:, None]
+        p = state[name].astype(np.float64)
+        m = state[name + "/adam_m"].astype(np.float64)
+        v = state[name + "/adam_v"].astype(np.float64)
+        adam(p, m, v, grad, a)
+        state[name][...] = p
+        state[name + "/adam_m"][...] = m
+        state[name + "/adam_v"][...] = v
+
+    dense("relation_embedding", rel.grad.numpy())
+    if F:
+        dense("feature_projection", proj.grad.numpy())
+    return per_shard.detach().numpy().astype(np.float32)
