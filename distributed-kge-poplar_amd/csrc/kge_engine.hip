@@ -1,0 +1,1095 @@
+// Host side of libkge_hip.so: settings, validation, command dispatch and the
+// step schedule behind the C-ABI of include/kge_hip.h.
+//
+// Mirrors, for the training path only, poplar_kge::Engine
+// (src/poplar_kge.cpp:914-1006): Model settings (:198-286), stream validation
+// (GetData, :69-106), the commands of EngineImpl::run (:950-998) and the order
+// of operations of Model::trainStep (:664-707) / trainStepLoop (:709-741).
+#include "../../include/kge_hip.h"
+#include "kge_kernels.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <memory>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+using namespace kge;
+
+namespace {
+
+#define HIP_CHECK(expr)                                                                      \
+    do {                                                                                     \
+        hipError_t e_ = (expr);                                                              \
+        if (e_ != hipSuccess) {                                                              \
+            std::ostringstream m_;                                                           \
+            m_ << "HIP error " << hipGetErrorString(e_) << " at " << __FILE__ << ":" << __LINE__ \
+               << " (" #expr ")";                                                            \
+            throw std::runtime_error(m_.str());                                              \
+        }                                                                                    \
+    } while (0)
+
+const char* kind_name(int kind) {
+    switch (kind) {
+        case KGE_STR: return "string";
+        case KGE_F32: return "float";
+        case KGE_U32: return "unsigned int";
+        case KGE_F16: return "half";
+        case KGE_BOOL: return "bool";
+        case KGE_FLOAT: return "float (scalar)";
+        case KGE_UINT: return "unsigned (scalar)";
+        case KGE_MAP: return "map";
+    }
+    return "<unknown>";
+}
+
+std::string shape_str(const size_t* shape, size_t rank) {
+    std::ostringstream s;
+    s << "(";
+    for (size_t i = 0; i < rank; ++i) s << (i ? ", " : "") << shape[i];
+    s << ")";
+    return s.str();
+}
+std::string shape_str(const std::vector<size_t>& v) { return shape_str(v.data(), v.size()); }
+
+// The reference's get/extract helpers (src/poplar_kge.cpp:38-67).
+struct Items {
+    const kge_item* items;
+    size_t n;
+    const kge_item* find(const std::string& key) const {
+        for (size_t i = 0; i < n; ++i)
+            if (items[i].key && key == items[i].key) return &items[i];
+        return nullptr;
+    }
+    const kge_item& get(const std::string& key) const {
+        const kge_item* it = find(key);
+        if (!it) throw std::invalid_argument("Key not found '" + key + "'");
+        return *it;
+    }
+    const kge_item& typed(const std::string& key, int kind) const {
+        const kge_item& it = get(key);
+        if (it.kind != kind) {
+            std::ostringstream msg;
+            msg << "Key '" << key << "' holds value of unexpected type. Expected: '" << kind_name(kind)
+                << "', actual: '" << kind_name(it.kind) << "'.";
+            throw std::invalid_argument(msg.str());
+        }
+        return it;
+    }
+    unsigned uint(const std::string& key) const { return (unsigned)typed(key, KGE_UINT).num; }
+    float flt(const std::string& key) const { return (float)typed(key, KGE_FLOAT).num; }
+    bool boolean(const std::string& key) const { return typed(key, KGE_BOOL).num != 0; }
+    std::string str(const std::string& key) const { return typed(key, KGE_STR).str; }
+    // stream binding with strict dtype and shape checks (GetData, :69-106)
+    void* array(const std::string& name, int kind, const std::vector<size_t>& shape) const {
+        const kge_item& it = get(name);
+        if (it.kind != KGE_F32 && it.kind != KGE_U32 && it.kind != KGE_F16) {
+            std::ostringstream msg;
+            msg << "'" << name << "' expected type " << kind_name(kind) << ", actual: <not found> ("
+                << kind_name(it.kind) << ")";
+            throw std::invalid_argument(msg.str());
+        }
+        if (it.kind != kind) {
+            std::ostringstream msg;
+            msg << "'" << name << "' expected array of type " << kind_name(kind)
+                << ", actual: " << kind_name(it.kind);
+            throw std::invalid_argument(msg.str());
+        }
+        if (it.rank != shape.size() || !std::equal(shape.begin(), shape.end(), it.shape)) {
+            std::ostringstream msg;
+            msg << "'" << name << "' expected array of shape " << shape_str(shape)
+                << ", actual: " << shape_str(it.shape, it.rank);
+            throw std::invalid_argument(msg.str());
+        }
+        return it.data;
+    }
+};
+
+template <class T>
+struct DevBuf {
+    T* p = nullptr;
+    size_t n = 0;
+    void alloc(size_t count) {
+        release();
+        n = count;
+        if (count) HIP_CHECK(hipMalloc((void**)&p, count * sizeof(T)));
+    }
+    void zero(hipStream_t s) {
+        if (n) HIP_CHECK(hipMemsetAsync(p, 0, n * sizeof(T), s));
+    }
+    void release() {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        n = 0;
+    }
+    ~DevBuf() { release(); }
+};
+
+int round_up(int x, int m) { return (x + m - 1) / m * m; }
+int elem_size(int et) { return et == ET_F32 ? 4 : 2; }
+int bit_length(uint64_t x) { int b = 0; while (x) { ++b; x >>= 1; } return b; }
+
+float half_to_float(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000) << 16;
+    uint32_t exp = (h >> 10) & 0x1f, man = h & 0x3ff, u;
+    if (exp == 0) {
+        if (man == 0) u = sign;
+        else {
+            int e = -1;
+            do { ++e; man <<= 1; } while (!(man & 0x400));
+            u = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3ff) << 13);
+        }
+    } else if (exp == 31) u = sign | 0x7f800000u | (man << 13);
+    else u = sign | ((exp + 112) << 23) | (man << 13);
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+uint16_t float_to_half(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    const uint32_t sign = (u >> 16) & 0x8000;
+    uint32_t mag = u & 0x7fffffffu;
+    if (mag >= 0x7f800000u) return (uint16_t)(sign | 0x7c00 | (mag > 0x7f800000u ? 0x200 : 0));
+    if (mag >= 0x477ff000u) return (uint16_t)(sign | 0x7c00);
+    if (mag < 0x38800000u) {  // subnormal half
+        if (mag < 0x33000000u) return (uint16_t)sign;
+        const int e = (int)(mag >> 23);
+        uint32_t man = (mag & 0x7fffffu) | 0x800000u;
+        const int shift = 126 - e;  // total right shift: 13 + (113 - e)
+        const uint32_t half = 1u << (shift - 1), rem = man & ((1u << shift) - 1);
+        man >>= shift;
+        if (rem > half || (rem == half && (man & 1))) ++man;
+        return (uint16_t)(sign | man);
+    }
+    mag += 0xfffu + ((mag >> 13) & 1u);
+    return (uint16_t)(sign | ((mag - 0x38000000u) >> 13));
+}
+
+enum KernelId {
+    K_PLAN = 0, K_HIDDEN, K_FWD, K_LOSS, K_BWD, K_REDUCE_ENT, K_ADAM_ENT, K_REDUCE_REL, K_ADAM_REL,
+    K_PROJ_GRAD, K_ADAM_PROJ, K_COUNT
+};
+
+struct Variable {
+    std::string name;
+    std::vector<size_t> shape;
+};
+
+}  // namespace
+
+struct kge_engine {
+    // ---- settings (src/poplar_kge.cpp:198-236) ----
+    int S, n_entity, n_rel, D, F, B, A, T, NR, R;
+    int score_fn, dist_fn, loss_fn;
+    bool shared_table;
+    float gamma, init_scale, beta_m, beta_v, epsilon, weight_decay, loss_scale, softmax_cw, neg_adv;
+    float lr_mod_entity = 1.f, lr_mod_rel = 1.f, lr_mod_proj = 1.f;
+    uint32_t seed;
+    int n_step, rw_batch;
+    int stream_kind;  // KGE_F32 or KGE_F16: dtype of the entity read/write streams
+    bool profile_kernels = false;
+    int chunk = 32;
+
+    RowLayout L;
+    int64_t n_rows;
+    int Dp, Fp;
+    std::vector<Variable> variables;
+
+    // ---- device state ----
+    hipStream_t stream = nullptr;
+    DevBuf<char> table;
+    DevBuf<float> rel, rel_m, rel_v, proj, proj_m, proj_v;
+    uint32_t step = 0;
+
+    // staged batch
+    DevBuf<uint32_t> d_remote, d_a2a, d_head, d_relation, d_tail;
+    bool staged = false;
+    // plan
+    DevBuf<uint32_t> ckey, crel, clabel, ek_a, ev_a, ek_b, ev_b, rk_a, rv_a, rk_b, rv_b, hist;
+    DevBuf<uint32_t> e_uniq, e_seg, e_coff, e_cpos, e_clen, e_counts, e_item_row;
+    DevBuf<uint32_t> r_uniq, r_seg, r_coff, r_cpos, r_clen, r_counts;
+    int e_ustride, e_cstride, r_ustride, r_cstride, n_rel_items;
+    uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
+    // step
+    DevBuf<float> coef, dist, grad, partial, rel_partial, hidden, gsum, gproj, loss_part, d_loss, d_alpha;
+    std::vector<float> h_alpha;  // [n_step][entity, relation, projection][S]
+    int n_part;
+    // io staging
+    DevBuf<uint64_t> io_rows;
+    DevBuf<float> io_data;
+    DevBuf<uint32_t> io_idx;
+
+    // timing
+    hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
+    float phase_ms[4] = {0, 0, 0, 0};  // upload, plan, steps, total of the last train_step_loop
+    std::vector<hipEvent_t> kev;
+    std::vector<int> kev_id;
+    double kernel_ms[K_COUNT] = {0};
+    uint32_t kernel_calls[K_COUNT] = {0};
+
+    ~kge_engine() {
+        for (auto& e : ev) if (e) (void)hipEventDestroy(e);
+        for (auto& e : kev) (void)hipEventDestroy(e);
+        if (stream) (void)hipStreamDestroy(stream);
+    }
+};
+
+namespace {
+
+void parse_settings(kge_engine& E, const Items& s) {
+    // the device: this library only drives a HIP device
+    const std::string device = s.str("execution.device");
+    if (device != "hip") {
+        std::ostringstream msg;
+        msg << "Unexpected setting \"device\": '" << device << "', expected \"hip\"";
+        throw std::invalid_argument(msg.str());
+    }
+    E.seed = s.uint("model.seed");
+    const std::string score = s.str("model.score_fn"), distance = s.str("model.distance_fn");
+    E.S = (int)s.uint("model.n_shard");
+    E.n_entity = (int)s.uint("model.n_entity");
+    E.n_rel = (int)s.uint("model.n_relation_type");
+    E.D = (int)s.uint("model.embedding_size");
+    E.F = (int)s.uint("model.entity_feature_size");
+    const unsigned mlp = s.uint("model.feature_mlp_size");
+    const float dropout = s.flt("model.feature_dropout");
+    const bool share = s.boolean("model.share_feature_networks");
+    E.gamma = s.flt("model.gamma");
+    E.init_scale = s.flt("model.init_scale");
+    E.beta_m = s.flt("training.adam_beta_m");
+    E.beta_v = s.flt("training.adam_beta_v");
+    E.epsilon = s.flt("training.adam_epsilon");
+    E.weight_decay = s.flt("training.weight_decay");
+    const kge_item& mods = s.typed("training.learning_rate_modifiers", KGE_MAP);
+    E.B = (int)s.uint("data.batch_size");
+    E.A = (int)s.uint("data.a2a_size");
+    E.neg_adv = s.flt("model.negative_adversarial_scale");
+    const std::string loss = s.str("training.loss.type");
+    float reg_w[3];
+    const char* reg_names[3] = {"training.embedding_regularisation", "training.feature_regularisation",
+                                "training.hidden_regularisation"};
+    for (int i = 0; i < 3; ++i) {
+        (void)s.flt(std::string(reg_names[i]) + ".power");
+        reg_w[i] = s.flt(std::string(reg_names[i]) + ".weight");
+    }
+    E.softmax_cw = loss == "softmax" ? s.flt("training.loss.correction_weight") : 0.f;
+    E.loss_scale = s.flt("training.loss_scale");
+    E.n_step = (int)s.uint("execution.train_steps_per_program_run");
+    E.rw_batch = (int)s.uint("execution.rw_batch_size");
+    (void)s.uint("execution.predict_hr_batch_size");
+    (void)s.uint("execution.predict_tail_batch_size");
+    (void)s.uint("execution.predict_n_best");
+
+    // dtype of the entity table (src/poplar_kge.cpp:237-246) + additive layouts
+    const std::string dtype = s.str("execution.dtype");
+    int emb_et, mom_et, feat_et;
+    if (dtype == "float32") { emb_et = mom_et = feat_et = ET_F32; E.stream_kind = KGE_F32; }
+    else if (dtype == "float16") { emb_et = mom_et = feat_et = ET_F16; E.stream_kind = KGE_F16; }
+    else {
+        throw std::invalid_argument("'execution.dtype' must either be 'float16' or 'float32', not '" +
+                                    dtype + "'");
+    }
+    auto parse_et = [&](const char* key, int& et) {
+        if (!s.find(key)) return;
+        const std::string v = s.str(key);
+        if (v == "float32") et = ET_F32;
+        else if (v == "float16") et = ET_F16;
+        else if (v == "bfloat16") et = ET_BF16;
+        else throw std::invalid_argument(std::string("'") + key + "' must be one of 'float32', 'float16', 'bfloat16', not '" + v + "'");
+    };
+    parse_et("execution.embedding_dtype", emb_et);
+    parse_et("execution.feature_dtype", feat_et);
+    if (mom_et != ET_F32)
+        throw std::invalid_argument("'execution.dtype' = 'float16' (half-precision optimiser state) is not "
+                                    "supported; use 'float32' with 'execution.embedding_dtype'");
+    E.shared_table = s.find("execution.shared_table") ? s.boolean("execution.shared_table") : false;
+    E.profile_kernels = s.find("execution.profile_kernels") ? s.boolean("execution.profile_kernels") : false;
+    if (s.find("execution.reduce_chunk")) E.chunk = (int)s.uint("execution.reduce_chunk");
+
+    if (score == "TransE") E.score_fn = SCORE_TRANSE;
+    else if (score == "DistMult") E.score_fn = SCORE_DISTMULT;
+    else if (score == "ComplEx" || score == "RotatE" || score == "TransH")
+        throw std::invalid_argument("'model.score_fn' = '" + score + "' is not implemented on the HIP device "
+                                    "(supported: 'TransE', 'DistMult')");
+    else
+        throw std::invalid_argument("'model.score_fn' must be one of 'TransE', 'ComplEx', 'RotatE', 'TransH', or "
+                                    "'DistMult', not '" + score + "'");
+    if (distance == "L1") E.dist_fn = DIST_L1;
+    else if (distance == "L2") E.dist_fn = DIST_L2;
+    else if (distance == "MatMul") E.dist_fn = DIST_DOT;
+    else if (E.score_fn == SCORE_DISTMULT) E.dist_fn = DIST_DOT;
+    else
+        throw std::invalid_argument("'model.distance_fn' must be one of 'L1', 'L2' or 'MatMul', not '" +
+                                    distance + "'");
+    if (loss == "logsigmoid") E.loss_fn = LOSS_LOGSIGMOID;
+    else if (loss == "softmax") E.loss_fn = LOSS_SOFTMAX;
+    else
+        throw std::invalid_argument("'training.loss.type' must be one of 'logsigmoid' or 'softmax', not '" +
+                                    loss + "'");
+    if (mlp > 0) throw std::invalid_argument("'model.feature_mlp_size' > 0 is not implemented on the HIP device");
+    if (dropout > 0) throw std::invalid_argument("'model.feature_dropout' > 0 is not implemented on the HIP device");
+    if (!share && E.F > 0)
+        throw std::invalid_argument("'model.share_feature_networks' = false is not implemented on the HIP device");
+    for (int i = 0; i < 3; ++i)
+        if (reg_w[i] > 0)
+            throw std::invalid_argument(std::string("'") + reg_names[i] + ".weight' > 0 is not implemented on the HIP device");
+    if (E.S < 1 || E.B < 1 || E.A < 1 || E.D < 1 || E.n_entity < 1 || E.n_rel < 1 || E.n_step < 1 || E.rw_batch < 1)
+        throw std::invalid_argument("sizes must be positive");
+    if (E.S * E.A < 2) throw std::invalid_argument("n_shard * a2a_size must be at least 2");
+
+    // parameter sharding check (addParameter, src/poplar_kge.cpp:294-300); a
+    // shared table keeps every parameter whole, so nothing needs to divide
+    if (!E.shared_table) {
+        auto check = [&](const char* name, int dim0, int dim1) {
+            if (dim0 % E.S) {
+                std::ostringstream msg;
+                msg << "Parameter '" << name << "' shape[0] (" << dim0 << ") is not divisible by n_shard ("
+                    << E.S << "). Note shape: (" << dim0 << ", " << dim1 << ")";
+                throw std::invalid_argument(msg.str());
+            }
+        };
+        check("relation_embedding", E.n_rel, E.D);
+        check("feature_projection", E.F, E.D);
+    }
+    for (size_t i = 0; i < mods.map_len; ++i) {
+        const std::string k = mods.map_keys[i];
+        if (k == "entity_embedding") E.lr_mod_entity = mods.map_vals[i];
+        else if (k == "relation_embedding") E.lr_mod_rel = mods.map_vals[i];
+        else if (k == "feature_projection") E.lr_mod_proj = mods.map_vals[i];
+        else
+            throw std::invalid_argument("Bad training.learning_rate_modifier: unknown parameter '" + k + "'");
+    }
+
+    E.T = E.S * E.A;
+    E.NR = E.B + E.T;
+    E.R = E.S * E.NR;
+    E.Dp = round_up(E.D, emb_et == ET_F32 ? 4 : 8);
+    E.Fp = E.F ? round_up(E.F, feat_et == ET_F32 ? 4 : 8) : 0;
+    RowLayout& L = E.L;
+    L.D = E.D; L.F = E.F; L.Dp = E.Dp; L.Fp = E.Fp;
+    L.emb_etype = emb_et; L.mom_etype = mom_et; L.feat_etype = feat_et;
+    L.off_m = (int64_t)E.Dp * elem_size(emb_et);
+    L.off_s = L.off_m + (int64_t)E.Dp * 4;
+    L.off_f = L.off_s + (int64_t)E.Dp * 4;
+    L.pitch = L.off_f + (int64_t)E.Fp * elem_size(feat_et);
+    E.n_rows = E.shared_table ? (int64_t)E.n_entity : (int64_t)E.S * E.n_entity;
+    if (E.n_rows >= (int64_t)1 << 32) throw std::invalid_argument("more than 2^32 table rows");
+    if ((int64_t)2 * E.R >= (int64_t)1 << 31) throw std::invalid_argument("batch too large");
+
+    auto var = [&](const std::string& name, std::vector<size_t> shape) {
+        E.variables.push_back({name, shape});
+    };
+    var("step", {(size_t)E.S});
+    for (const char* suffix : {"", "/adam_m", "/adam_v"}) {
+        var(std::string("relation_embedding") + suffix, {(size_t)E.n_rel, (size_t)E.D});
+        var(std::string("feature_projection") + suffix, {(size_t)E.F, (size_t)E.D});
+    }
+}
+
+void allocate(kge_engine& E) {
+    int n_dev = 0;
+    if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev < 1)
+        throw std::runtime_error("Could not attach to a HIP device");
+    HIP_CHECK(hipStreamCreate(&E.stream));
+    for (auto& e : E.ev) HIP_CHECK(hipEventCreate(&e));
+    const hipStream_t st = E.stream;
+
+    E.table.alloc((size_t)E.n_rows * E.L.pitch);
+    E.table.zero(st);
+    const size_t rel_n = (size_t)E.n_rel * E.Dp, proj_n = (size_t)E.Fp * E.Dp;
+    for (DevBuf<float>* b : {&E.rel, &E.rel_m, &E.rel_v}) { b->alloc(rel_n); b->zero(st); }
+    for (DevBuf<float>* b : {&E.proj, &E.proj_m, &E.proj_v}) { b->alloc(proj_n); b->zero(st); }
+
+    const size_t ns = E.n_step, S = E.S, B = E.B, A = E.A, R = E.R, SB = S * B;
+    E.d_remote.alloc(ns * R);
+    E.d_a2a.alloc(ns * S * S * A);
+    E.d_head.alloc(ns * SB);
+    E.d_relation.alloc(ns * SB);
+    E.d_tail.alloc(ns * SB);
+
+    E.ckey.alloc(ns * R);
+    E.crel.alloc(ns * SB);
+    E.clabel.alloc(ns * SB);
+    for (DevBuf<uint32_t>* b : {&E.ek_a, &E.ev_a, &E.ek_b, &E.ev_b}) b->alloc(ns * 2 * R);
+    E.n_rel_items = (int)(SB + E.n_rel);
+    for (DevBuf<uint32_t>* b : {&E.rk_a, &E.rv_a, &E.rk_b, &E.rv_b}) b->alloc(ns * E.n_rel_items);
+    const size_t tiles = (std::max<size_t>(2 * R, E.n_rel_items) + kSortTile - 1) / kSortTile;
+    E.hist.alloc(ns * 256 * tiles);
+
+    E.e_ustride = (int)R;
+    E.e_cstride = (int)(R + R / E.chunk + 1);
+    E.e_uniq.alloc(ns * E.e_ustride);
+    E.e_seg.alloc(ns * (E.e_ustride + 1));
+    E.e_coff.alloc(ns * (E.e_ustride + 1));
+    E.e_cpos.alloc(ns * E.e_cstride);
+    E.e_clen.alloc(ns * E.e_cstride);
+    E.e_counts.alloc(ns * 2);
+    if (E.F) E.e_item_row.alloc(ns * R);
+    E.r_ustride = E.n_rel;
+    E.r_cstride = (int)(E.n_rel + SB / E.chunk + 1);
+    E.r_uniq.alloc(ns * E.r_ustride);
+    E.r_seg.alloc(ns * (E.r_ustride + 1));
+    E.r_coff.alloc(ns * (E.r_ustride + 1));
+    E.r_cpos.alloc(ns * E.r_cstride);
+    E.r_clen.alloc(ns * E.r_cstride);
+    E.r_counts.alloc(ns * 2);
+
+    E.coef.alloc(SB * E.T);
+    const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f;
+    if (!fused && E.score_fn == SCORE_TRANSE && E.dist_fn == DIST_L2) E.dist.alloc(SB * E.T);
+    E.grad.alloc(R * E.Dp);
+    E.partial.alloc((size_t)E.e_cstride * E.Dp);
+    E.rel_partial.alloc((size_t)E.r_cstride * E.Dp);
+    if (E.F) {
+        E.hidden.alloc(R * E.Dp);
+        E.gsum.alloc(R * E.Dp);
+        E.gproj.alloc(proj_n);
+    }
+    ScoreShape sh = {};
+    sh.S = E.S; sh.B = E.B; sh.T = E.T;
+    E.n_part = fused ? score_fwd_parts(sh) : E.B;
+    E.loss_part.alloc(ns * S * E.n_part);
+    E.d_loss.alloc(S);
+    E.d_alpha.alloc(ns * 3 * S);
+
+    const size_t io_n = (size_t)E.S * E.rw_batch;
+    E.io_rows.alloc(io_n);
+    E.io_idx.alloc(io_n);
+    E.io_data.alloc(io_n * (3 * E.D + E.F));
+    HIP_CHECK(hipStreamSynchronize(st));
+}
+
+// ---- variables: "read" / "write" (src/poplar_kge.cpp:977-991) ----------------
+
+void run_read_write(kge_engine& E, bool write, const Items& in) {
+    const std::string name = in.str("name");
+    const Variable* var = nullptr;
+    for (auto& v : E.variables) if (v.name == name) var = &v;
+    if (!var) throw std::invalid_argument("Key not found '" + name + "'");
+    if (name == "step") {
+        uint32_t* v = (uint32_t*)in.array("value", KGE_U32, var->shape);
+        if (write) E.step = v[0];
+        else for (int s = 0; s < E.S; ++s) v[s] = E.step;
+        return;
+    }
+    float* host = (float*)in.array("value", KGE_F32, var->shape);
+    DevBuf<float>* buf = nullptr;
+    if (name == "relation_embedding") buf = &E.rel;
+    else if (name == "relation_embedding/adam_m") buf = &E.rel_m;
+    else if (name == "relation_embedding/adam_v") buf = &E.rel_v;
+    else if (name == "feature_projection") buf = &E.proj;
+    else if (name == "feature_projection/adam_m") buf = &E.proj_m;
+    else if (name == "feature_projection/adam_v") buf = &E.proj_v;
+    const size_t rows = var->shape[0], cols = var->shape[1];
+    if (rows == 0 || cols == 0) return;
+    HIP_CHECK(hipStreamSynchronize(E.stream));
+    if (write)
+        HIP_CHECK(hipMemcpy2D(buf->p, (size_t)E.Dp * 4, host, cols * 4, cols * 4, rows, hipMemcpyHostToDevice));
+    else
+        HIP_CHECK(hipMemcpy2D(host, cols * 4, buf->p, (size_t)E.Dp * 4, cols * 4, rows, hipMemcpyDeviceToHost));
+}
+
+// ---- entity rows: "write_entity", "read_entity" (:857-871) --------------------
+
+void upload_row_ids(kge_engine& E, const uint32_t* idx, size_t per_shard, std::vector<uint64_t>& rows) {
+    rows.resize((size_t)E.S * per_shard);
+    for (int s = 0; s < E.S; ++s)
+        for (size_t i = 0; i < per_shard; ++i) {
+            const uint32_t v = idx[s * per_shard + i];
+            if (v >= (uint32_t)E.n_entity) {
+                std::ostringstream msg;
+                msg << "entity index " << v << " out of range [0, " << E.n_entity << ")";
+                throw std::invalid_argument(msg.str());
+            }
+            rows[s * per_shard + i] = (E.shared_table ? 0 : (uint64_t)s * E.n_entity) + v;
+        }
+    HIP_CHECK(hipMemcpyAsync(E.io_rows.p, rows.data(), rows.size() * 8, hipMemcpyHostToDevice, E.stream));
+}
+
+void run_write_entity(kge_engine& E, const Items& in, bool raw) {
+    const size_t S = E.S, rw = E.rw_batch, W = raw ? 3 * E.D + E.F : E.F;
+    const uint32_t* idx = (const uint32_t*)in.array("write_indices", KGE_U32, {S, rw});
+    const int kind = raw ? KGE_F32 : E.stream_kind;
+    const void* data = in.array(raw ? "write_data" : "write_features", kind, {S, rw, W});
+    std::vector<uint64_t> rows;
+    upload_row_ids(E, idx, rw, rows);
+    std::vector<float> conv;
+    const float* src = (const float*)data;
+    if (kind == KGE_F16) {
+        conv.resize(S * rw * W);
+        const uint16_t* h = (const uint16_t*)data;
+        for (size_t i = 0; i < conv.size(); ++i) conv[i] = half_to_float(h[i]);
+        src = conv.data();
+    }
+    if (W) HIP_CHECK(hipMemcpyAsync(E.io_data.p, src, S * rw * W * 4, hipMemcpyHostToDevice, E.stream));
+    if (raw)
+        launch_rows_from_logical(E.L, E.table.p, E.io_rows.p, (int64_t)(S * rw), E.io_data.p, E.stream);
+    else  // random-normal embedding with sigma = init_scale / D (:865-866)
+        launch_init_rows(E.L, E.table.p, E.io_rows.p, (int64_t)(S * rw), E.io_data.p,
+                         E.init_scale / (float)E.D, E.seed, E.stream);
+    HIP_CHECK(hipGetLastError());
+    HIP_CHECK(hipStreamSynchronize(E.stream));
+}
+
+void run_read_entity(kge_engine& E, const Items& in) {
+    const size_t S = E.S, rw = E.rw_batch, W = 3 * E.D + E.F;
+    const uint32_t* idx = (const uint32_t*)in.array("read_indices", KGE_U32, {S, rw});
+    void* out = in.array("read_data", E.stream_kind, {S, rw, W});
+    std::vector<uint64_t> rows;
+    upload_row_ids(E, idx, rw, rows);
+    launch_rows_to_logical(E.L, E.table.p, E.io_rows.p, (int64_t)(S * rw), E.io_data.p, E.stream);
+    HIP_CHECK(hipGetLastError());
+    if (E.stream_kind == KGE_F32) {
+        HIP_CHECK(hipMemcpyAsync(out, E.io_data.p, S * rw * W * 4, hipMemcpyDeviceToHost, E.stream));
+        HIP_CHECK(hipStreamSynchronize(E.stream));
+    } else {
+        std::vector<float> tmp(S * rw * W);
+        HIP_CHECK(hipMemcpyAsync(tmp.data(), E.io_data.p, tmp.size() * 4, hipMemcpyDeviceToHost, E.stream));
+        HIP_CHECK(hipStreamSynchronize(E.stream));
+        uint16_t* h = (uint16_t*)out;
+        for (size_t i = 0; i < tmp.size(); ++i) h[i] = float_to_half(tmp[i]);
+    }
+}
+
+// ---- training ------------------------------------------------------------------
+
+struct BatchPtrs {
+    const uint32_t *remote, *a2a, *head, *relation, *tail;
+};
+
+BatchPtrs bind_batch(kge_engine& E, const Items& in) {
+    const size_t S = E.S, ns = E.n_step;
+    BatchPtrs b;
+    b.remote = (const uint32_t*)in.array("remote", KGE_U32, {S, ns, (size_t)E.NR});
+    b.a2a = (const uint32_t*)in.array("a2a", KGE_U32, {S, ns, S, (size_t)E.A});
+    b.head = (const uint32_t*)in.array("head", KGE_U32, {S, ns, (size_t)E.B});
+    b.relation = (const uint32_t*)in.array("relation", KGE_U32, {S, ns, (size_t)E.B});
+    b.tail = (const uint32_t*)in.array("tail", KGE_U32, {S, ns, (size_t)E.B});
+    return b;
+}
+
+// Every index a kernel will dereference is checked here, on the host.
+void validate_batch(const kge_engine& E, const BatchPtrs& b) {
+    auto check = [](const char* name, const uint32_t* v, size_t n, uint32_t limit) {
+        uint32_t worst = 0;
+        for (size_t i = 0; i < n; ++i) worst = std::max(worst, v[i]);
+        if (n && worst >= limit) {
+            std::ostringstream msg;
+            msg << "'" << name << "' holds index " << worst << " out of range [0, " << limit << ")";
+            throw std::invalid_argument(msg.str());
+        }
+    };
+    const size_t S = E.S, ns = E.n_step;
+    check("remote", b.remote, S * ns * E.NR, (uint32_t)E.n_entity);
+    check("a2a", b.a2a, S * ns * S * E.A, (uint32_t)E.NR);
+    check("head", b.head, S * ns * E.B, (uint32_t)E.NR);
+    check("relation", b.relation, S * ns * E.B, (uint32_t)E.n_rel);
+    check("tail", b.tail, S * ns * E.B, (uint32_t)E.T);
+}
+
+void upload_batch(kge_engine& E, const BatchPtrs& b) {
+    const hipStream_t st = E.stream;
+    HIP_CHECK(hipMemcpyAsync(E.d_remote.p, b.remote, E.d_remote.n * 4, hipMemcpyHostToDevice, st));
+    HIP_CHECK(hipMemcpyAsync(E.d_a2a.p, b.a2a, E.d_a2a.n * 4, hipMemcpyHostToDevice, st));
+    HIP_CHECK(hipMemcpyAsync(E.d_head.p, b.head, E.d_head.n * 4, hipMemcpyHostToDevice, st));
+    HIP_CHECK(hipMemcpyAsync(E.d_relation.p, b.relation, E.d_relation.n * 4, hipMemcpyHostToDevice, st));
+    HIP_CHECK(hipMemcpyAsync(E.d_tail.p, b.tail, E.d_tail.n * 4, hipMemcpyHostToDevice, st));
+}
+
+struct KernelTimer {
+    kge_engine& E;
+    int id;
+    KernelTimer(kge_engine& e, int id_) : E(e), id(id_) {
+        if (E.profile_kernels) push();
+    }
+    ~KernelTimer() {
+        if (E.profile_kernels) push();
+    }
+    void push() {
+        hipEvent_t ev;
+        (void)hipEventCreate(&ev);
+        (void)hipEventRecord(ev, E.stream);
+        E.kev.push_back(ev);
+        E.kev_id.push_back(id);
+    }
+};
+
+void collect_kernel_times(kge_engine& E) {
+    for (size_t i = 0; i + 1 < E.kev.size(); i += 2) {
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, E.kev[i], E.kev[i + 1]);
+        E.kernel_ms[E.kev_id[i]] += ms;
+        E.kernel_calls[E.kev_id[i]] += 1;
+    }
+    for (auto& e : E.kev) (void)hipEventDestroy(e);
+    E.kev.clear();
+    E.kev_id.clear();
+}
+
+void run_plan(kge_engine& E) {
+    KernelTimer timer(E, K_PLAN);
+    const hipStream_t st = E.stream;
+    PlanShape ps;
+    ps.n_step = E.n_step; ps.S = E.S; ps.B = E.B; ps.A = E.A; ps.NR = E.NR;
+    ps.n_entity = E.n_entity; ps.shared_table = E.shared_table; ps.n_relation = E.n_rel;
+    launch_build_items(ps, E.d_remote.p, E.d_a2a.p, E.d_head.p, E.d_relation.p, E.d_tail.p, E.ckey.p,
+                       E.crel.p, E.clabel.p, E.ek_a.p, E.ev_a.p, E.rk_a.p, E.rv_a.p, st);
+    const int ebits = std::max(1, bit_length((uint64_t)E.n_rows - 1));
+    const int rbits = std::max(1, bit_length((uint64_t)E.n_rel - 1));
+    const int N = 2 * E.R;
+    int which = launch_radix_sort(E.ek_a.p, E.ev_a.p, E.ek_b.p, E.ev_b.p, E.hist.p, N, E.n_step, ebits, st);
+    const uint32_t* ek = which ? E.ek_b.p : E.ek_a.p;
+    E.e_sorted_vals = which ? E.ev_b.p : E.ev_a.p;
+    SegPlan ep;
+    ep.uniq_key = E.e_uniq.p; ep.seg_start = E.e_seg.p; ep.chunk_off = E.e_coff.p;
+    ep.chunk_pos = E.e_cpos.p; ep.chunk_len = E.e_clen.p; ep.counts = E.e_counts.p;
+    ep.item_row = E.F ? E.e_item_row.p : nullptr;
+    ep.u_stride = E.e_ustride; ep.c_stride = E.e_cstride;
+    launch_find_segments(ek, E.e_sorted_vals, N, E.R, E.chunk, E.n_step, ep, st);
+
+    which = launch_radix_sort(E.rk_a.p, E.rv_a.p, E.rk_b.p, E.rv_b.p, E.hist.p, E.n_rel_items, E.n_step, rbits, st);
+    const uint32_t* rk = which ? E.rk_b.p : E.rk_a.p;
+    E.r_sorted_vals = which ? E.rv_b.p : E.rv_a.p;
+    SegPlan rp;
+    rp.uniq_key = E.r_uniq.p; rp.seg_start = E.r_seg.p; rp.chunk_off = E.r_coff.p;
+    rp.chunk_pos = E.r_cpos.p; rp.chunk_len = E.r_clen.p; rp.counts = E.r_counts.p;
+    rp.item_row = nullptr;
+    rp.u_stride = E.r_ustride; rp.c_stride = E.r_cstride;
+    launch_find_segments(rk, E.r_sorted_vals, E.n_rel_items, E.S * E.B, E.chunk, E.n_step, rp, st);
+    HIP_CHECK(hipGetLastError());
+}
+
+void run_step(kge_engine& E, int i) {
+    const hipStream_t st = E.stream;
+    const size_t R = E.R, SB = (size_t)E.S * E.B;
+    ScoreShape sh;
+    sh.S = E.S; sh.B = E.B; sh.T = E.T; sh.Dp = E.Dp;
+    sh.score_fn = E.score_fn; sh.dist_fn = E.dist_fn; sh.loss_fn = E.loss_fn;
+    sh.gamma = E.gamma; sh.loss_scale = E.loss_scale;
+    sh.softmax_correction = 0.f;
+    if (E.loss_fn == LOSS_SOFTMAX && E.softmax_cw != 0.f) {
+        // src/poplar_kge.cpp:644: float correction = log(nEntity*nShard - 1) - log(nShard*a2aSize - 1)
+        const float corr = (float)(std::log((double)((uint32_t)E.n_entity * (uint32_t)E.S - 1u)) -
+                                   std::log((double)((uint32_t)E.S * (uint32_t)E.A - 1u)));
+        sh.softmax_correction = E.softmax_cw * corr;
+    }
+    sh.negative_adversarial_scale = E.neg_adv;
+    const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f;
+
+    const uint32_t* ckey = E.ckey.p + i * R;
+    const uint32_t* crel = E.crel.p + i * SB;
+    const uint32_t* clabel = E.clabel.p + i * SB;
+    const uint32_t* e_counts = E.e_counts.p + 2 * (size_t)i;
+    const uint32_t* e_uniq = E.e_uniq.p + (size_t)i * E.e_ustride;
+    const uint32_t* r_counts = E.r_counts.p + 2 * (size_t)i;
+
+    RowSource table_rows;  // entity embeddings straight from the table
+    table_rows.base = E.table.p; table_rows.pitch = E.L.pitch; table_rows.etype = E.L.emb_etype;
+    table_rows.index = ckey; table_rows.count = E.Dp; table_rows.vec = 1;
+    RowSource ent = table_rows;
+
+    FeatureArgs fa = {};
+    if (E.F) {
+        fa.uniq_key = e_uniq; fa.counts = e_counts; fa.max_rows = (int)R;
+        fa.emb_base = E.table.p; fa.feat_base = E.table.p + E.L.off_f; fa.pitch = E.L.pitch;
+        fa.emb_etype = E.L.emb_etype; fa.feat_etype = E.L.feat_etype;
+        fa.Dp = E.Dp; fa.Fp = E.Fp; fa.proj = E.proj.p;
+        { KernelTimer t(E, K_HIDDEN); launch_hidden_fwd(fa, E.hidden.p, st); }
+        ent.base = (const char*)E.hidden.p; ent.pitch = (int64_t)E.Dp * 4; ent.etype = ET_F32;
+        ent.index = E.e_item_row.p + i * R;
+    }
+
+    float* loss_part = E.loss_part.p + (size_t)i * E.S * E.n_part;
+    { KernelTimer t(E, K_FWD);
+      launch_score_fwd(sh, ent, E.rel.p, crel, clabel, E.coef.p, E.dist.p, loss_part, fused, st); }
+    if (!fused) { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, E.dist.p, loss_part, st); }
+    { KernelTimer t(E, K_BWD); launch_score_bwd(sh, ent, E.rel.p, crel, E.coef.p, E.grad.p, st); }
+
+    const float* alpha = E.d_alpha.p + (size_t)i * 3 * E.S;
+    AdamArgs aa = {};
+    aa.Dp = E.Dp;
+    aa.beta_m = E.beta_m; aa.beta_v = E.beta_v;
+    aa.one_minus_beta_m = 1.f - E.beta_m; aa.one_minus_beta_v = 1.f - E.beta_v;
+    aa.epsilon = E.epsilon; aa.weight_decay = E.weight_decay;
+
+    // relation gradient first: for DistMult it needs the pre-update head rows
+    ReduceArgs rr = {};
+    rr.sorted_item = E.r_sorted_vals + (size_t)i * E.n_rel_items;
+    rr.chunk_pos = E.r_cpos.p + (size_t)i * E.r_cstride;
+    rr.chunk_len = E.r_clen.p + (size_t)i * E.r_cstride;
+    rr.counts = r_counts; rr.max_chunks = E.r_cstride;
+    rr.grad = E.grad.p; rr.partial = E.rel_partial.p; rr.Dp = E.Dp;
+    rr.transform = E.score_fn == SCORE_DISTMULT ? 2 : 0; rr.n_head = (int)SB;
+    rr.rel = E.rel.p; rr.crel = crel; rr.ent = ent;
+    { KernelTimer t(E, K_REDUCE_REL); launch_reduce_chunks(rr, st); }
+
+    ReduceArgs re = {};
+    re.sorted_item = E.e_sorted_vals + (size_t)i * 2 * R;
+    re.chunk_pos = E.e_cpos.p + (size_t)i * E.e_cstride;
+    re.chunk_len = E.e_clen.p + (size_t)i * E.e_cstride;
+    re.counts = e_counts; re.max_chunks = E.e_cstride;
+    re.grad = E.grad.p; re.partial = E.partial.p; re.Dp = E.Dp;
+    re.transform = E.score_fn == SCORE_DISTMULT ? 1 : 0; re.n_head = (int)SB;
+    re.rel = E.rel.p; re.crel = crel; re.ent = ent;
+    { KernelTimer t(E, K_REDUCE_ENT); launch_reduce_chunks(re, st); }
+
+    // dense Adam on the relation table (updateParameters, :329-339)
+    AdamArgs ar = aa;
+    ar.uniq_key = E.r_uniq.p + (size_t)i * E.r_ustride;
+    ar.chunk_off = E.r_coff.p + (size_t)i * (E.r_ustride + 1);
+    ar.counts = r_counts; ar.max_rows = E.n_rel;
+    ar.partial = E.rel_partial.p;
+    ar.p_base = (char*)E.rel.p; ar.m_base = (char*)E.rel_m.p; ar.v_base = (char*)E.rel_v.p;
+    ar.pitch = (int64_t)E.Dp * 4; ar.p_etype = ET_F32; ar.v_is_sqrt = 0;
+    ar.alpha = alpha + E.S;
+    ar.rows_per_alpha = E.shared_table ? 0u : (uint32_t)(E.n_rel / E.S);
+    { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
+
+    // entity rows: sum partials, Adam on [emb | m | sqrt v], write back in place (:695-704)
+    AdamArgs ae = aa;
+    ae.uniq_key = e_uniq;
+    ae.chunk_off = E.e_coff.p + (size_t)i * (E.e_ustride + 1);
+    ae.counts = e_counts; ae.max_rows = (int)R;
+    ae.partial = E.partial.p;
+    ae.grad_out = E.F ? E.gsum.p : nullptr;
+    ae.p_base = E.table.p; ae.m_base = E.table.p + E.L.off_m; ae.v_base = E.table.p + E.L.off_s;
+    ae.pitch = E.L.pitch; ae.p_etype = E.L.emb_etype; ae.v_is_sqrt = 1;
+    ae.alpha = alpha;
+    ae.rows_per_alpha = E.shared_table ? 0u : (uint32_t)E.n_entity;
+    { KernelTimer t(E, K_ADAM_ENT); launch_adam_rows(ae, st); }
+
+    if (E.F) {
+        { KernelTimer t(E, K_PROJ_GRAD); launch_proj_grad(fa, E.gsum.p, E.gproj.p, st); }
+        // dense Adam on the projection; shard s owns rows [s*F/S, (s+1)*F/S) and its step size
+        KernelTimer t(E, K_ADAM_PROJ);
+        const int n_slices = E.shared_table ? 1 : E.S;
+        for (int s = 0; s < n_slices; ++s) {
+            const int r0 = E.shared_table ? 0 : s * (E.F / E.S);
+            const int r1 = (E.shared_table || s == E.S - 1) ? E.Fp : (s + 1) * (E.F / E.S);
+            if (r1 <= r0) continue;
+            const size_t o = (size_t)r0 * E.Dp;
+            launch_adam_flat(E.proj.p + o, E.proj_m.p + o, E.proj_v.p + o, E.gproj.p + o,
+                             (int64_t)(r1 - r0) * E.Dp, E.h_alpha[((size_t)i * 3 + 2) * E.S + s],
+                             E.beta_m, E.beta_v, E.epsilon, E.weight_decay, 0, st);
+        }
+    }
+    HIP_CHECK(hipGetLastError());
+}
+
+// Engine.train_step_loop's device half (Model::trainStepLoop, :709-741)
+void run_train_step_loop(kge_engine& E, const Items& in) {
+    const size_t S = E.S;
+    const float* lr = (const float*)in.array("learning_rate", KGE_F32, {S});
+    float* loss = (float*)in.array("loss", KGE_F32, {S});
+    const bool staged = in.find("staged") && in.boolean("staged");
+    const hipStream_t st = E.stream;
+    HIP_CHECK(hipEventRecord(E.ev[0], st));
+    if (!staged) {
+        const BatchPtrs b = bind_batch(E, in);
+        validate_batch(E, b);
+        upload_batch(E, b);
+    } else if (!E.staged) {
+        throw std::invalid_argument("train_step_loop with staged=true needs a preceding stage_batch");
+    }
+    // step sizes of every step of this call (adamStepSizeAutoIncrement, frnn.cpp:42-59)
+    E.h_alpha.resize((size_t)E.n_step * 3 * S);
+    for (int i = 0; i < E.n_step; ++i) {
+        const double t = (double)(E.step + (uint32_t)i + 1u);
+        const double factor = std::sqrt(1.0 - std::pow((double)E.beta_v, t)) / (1.0 - std::pow((double)E.beta_m, t));
+        for (size_t s = 0; s < S; ++s) {
+            const float a = (float)(factor * (double)lr[s]);
+            E.h_alpha[((size_t)i * 3 + 0) * S + s] = a * E.lr_mod_entity;
+            E.h_alpha[((size_t)i * 3 + 1) * S + s] = a * E.lr_mod_rel;
+            E.h_alpha[((size_t)i * 3 + 2) * S + s] = a * E.lr_mod_proj;
+        }
+    }
+    HIP_CHECK(hipMemcpyAsync(E.d_alpha.p, E.h_alpha.data(), E.h_alpha.size() * 4, hipMemcpyHostToDevice, st));
+    HIP_CHECK(hipEventRecord(E.ev[1], st));
+    run_plan(E);
+    HIP_CHECK(hipEventRecord(E.ev[2], st));
+    for (int i = 0; i < E.n_step; ++i) run_step(E, i);
+    launch_loss_finalize(E.loss_part.p, E.n_step, E.S, E.n_part, 1.f / (float)E.n_step, E.d_loss.p, st);
+    HIP_CHECK(hipGetLastError());
+    HIP_CHECK(hipEventRecord(E.ev[3], st));
+    HIP_CHECK(hipMemcpyAsync(loss, E.d_loss.p, S * 4, hipMemcpyDeviceToHost, st));
+    HIP_CHECK(hipStreamSynchronize(st));
+    E.step += (uint32_t)E.n_step;
+    for (int k = 0; k < 3; ++k) HIP_CHECK(hipEventElapsedTime(&E.phase_ms[k], E.ev[k], E.ev[k + 1]));
+    HIP_CHECK(hipEventElapsedTime(&E.phase_ms[3], E.ev[0], E.ev[3]));
+    if (E.profile_kernels) collect_kernel_times(E);
+}
+
+void run_stage_batch(kge_engine& E, const Items& in) {
+    const BatchPtrs b = bind_batch(E, in);
+    validate_batch(E, b);
+    upload_batch(E, b);
+    HIP_CHECK(hipStreamSynchronize(E.stream));
+    E.staged = true;
+}
+
+// "timing": phase_ms f32[4] {upload, plan, steps, total} of the last loop;
+// kernel_ms f32[K_COUNT], kernel_calls u32[K_COUNT] accumulated since the last
+// "timing" call (only with execution.profile_kernels); plan_counts
+// u32[n_step, 4] {distinct entity rows, entity chunks, relation rows, relation chunks}.
+void run_timing(kge_engine& E, const Items& in) {
+    if (in.find("phase_ms")) {
+        float* p = (float*)in.array("phase_ms", KGE_F32, {4});
+        std::memcpy(p, E.phase_ms, sizeof(E.phase_ms));
+    }
+    if (in.find("kernel_ms")) {
+        float* p = (float*)in.array("kernel_ms", KGE_F32, {(size_t)K_COUNT});
+        uint32_t* c = (uint32_t*)in.array("kernel_calls", KGE_U32, {(size_t)K_COUNT});
+        for (int k = 0; k < K_COUNT; ++k) {
+            p[k] = (float)E.kernel_ms[k];
+            c[k] = E.kernel_calls[k];
+            E.kernel_ms[k] = 0;
+            E.kernel_calls[k] = 0;
+        }
+    }
+    if (in.find("plan_counts")) {
+        uint32_t* p = (uint32_t*)in.array("plan_counts", KGE_U32, {(size_t)E.n_step, 4});
+        std::vector<uint32_t> e(2 * E.n_step), r(2 * E.n_step);
+        HIP_CHECK(hipMemcpy(e.data(), E.e_counts.p, e.size() * 4, hipMemcpyDeviceToHost));
+        HIP_CHECK(hipMemcpy(r.data(), E.r_counts.p, r.size() * 4, hipMemcpyDeviceToHost));
+        for (int i = 0; i < E.n_step; ++i) {
+            p[4 * i + 0] = e[2 * i]; p[4 * i + 1] = e[2 * i + 1];
+            p[4 * i + 2] = r[2 * i]; p[4 * i + 3] = r[2 * i + 1];
+        }
+    }
+}
+
+// "gather_benchmark": the stand-alone row gather (fr::Buffer::read) over the
+// engine's own table: gathers `indices` u32[n] physical rows `repeats` times
+// into a scratch buffer and reports the mean kernel time in `ms` f32[1].
+void run_gather_benchmark(kge_engine& E, const Items& in) {
+    const kge_item& idx = in.typed("indices", KGE_U32);
+    if (idx.rank != 1) throw std::invalid_argument("'indices' expected a 1-D array");
+    const size_t n = idx.shape[0];
+    float* ms = (float*)in.array("ms", KGE_F32, {1});
+    const unsigned repeats = in.find("repeats") ? in.uint("repeats") : 10u;
+    const uint32_t* h = (const uint32_t*)idx.data;
+    for (size_t i = 0; i < n; ++i)
+        if ((int64_t)h[i] >= E.n_rows) throw std::invalid_argument("'indices' out of range");
+    DevBuf<uint32_t> d_idx;
+    DevBuf<char> out;
+    d_idx.alloc(n);
+    out.alloc(n * (size_t)E.L.pitch);
+    HIP_CHECK(hipMemcpy(d_idx.p, h, n * 4, hipMemcpyHostToDevice));
+    launch_rows_gather(E.table.p, d_idx.p, out.p, (int64_t)n, E.L.pitch, E.stream);
+    HIP_CHECK(hipEventRecord(E.ev[0], E.stream));
+    for (unsigned r = 0; r < repeats; ++r)
+        launch_rows_gather(E.table.p, d_idx.p, out.p, (int64_t)n, E.L.pitch, E.stream);
+    HIP_CHECK(hipEventRecord(E.ev[1], E.stream));
+    HIP_CHECK(hipStreamSynchronize(E.stream));
+    float t = 0.f;
+    HIP_CHECK(hipEventElapsedTime(&t, E.ev[0], E.ev[1]));
+    ms[0] = t / (float)repeats;
+}
+
+void set_error(char* err, size_t len, const char* what) {
+    if (err && len) {
+        std::strncpy(err, what, len - 1);
+        err[len - 1] = 0;
+    }
+}
+
+template <class Fn>
+int guarded(char* err, size_t len, Fn&& fn) {
+    try {
+        fn();
+        return KGE_OK;
+    } catch (const std::invalid_argument& e) {
+        set_error(err, len, e.what());
+        return KGE_INVALID_ARGUMENT;
+    } catch (const std::logic_error& e) {
+        set_error(err, len, e.what());
+        return KGE_LOGIC_ERROR;
+    } catch (const std::exception& e) {
+        set_error(err, len, e.what());
+        return KGE_RUNTIME_ERROR;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int kge_engine_create(const kge_item* settings, size_t n_settings, const char* gp_folder,
+                      kge_engine** out, char* err, size_t err_len) {
+    (void)gp_folder;
+    return guarded(err, err_len, [&] {
+        if (!out) throw std::invalid_argument("null output pointer");
+        std::unique_ptr<kge_engine> E(new kge_engine());
+        parse_settings(*E, Items{settings, n_settings});
+        allocate(*E);
+        *out = E.release();
+    });
+}
+
+int kge_engine_run(kge_engine* engine, const char* command, kge_item* items, size_t n_items,
+                   char* err, size_t err_len) {
+    return guarded(err, err_len, [&] {
+        if (!engine || !command) throw std::invalid_argument("null engine or command");
+        kge_engine& E = *engine;
+        const Items in{items, n_items};
+        const std::string cmd = command;
+        if (cmd == "train_step_loop") run_train_step_loop(E, in);
+        else if (cmd == "read_entity") run_read_entity(E, in);
+        else if (cmd == "write_entity") run_write_entity(E, in, false);
+        else if (cmd == "write_entity_raw") run_write_entity(E, in, true);
+        else if (cmd == "read") run_read_write(E, false, in);
+        else if (cmd == "write") run_read_write(E, true, in);
+        else if (cmd == "stage_batch") run_stage_batch(E, in);
+        else if (cmd == "timing") run_timing(E, in);
+        else if (cmd == "gather_benchmark") run_gather_benchmark(E, in);
+        else if (cmd == "variables") { /* served by kge_engine_variable_info */ }
+        else if (cmd == "predict")
+            throw std::runtime_error("command 'predict' is not implemented on the HIP device");
+        else
+            throw std::invalid_argument("Unknown command '" + cmd + "'");
+    });
+}
+
+size_t kge_engine_variable_count(const kge_engine* engine) { return engine ? engine->variables.size() : 0; }
+
+int kge_engine_variable_info(const kge_engine* engine, size_t index, const char** name,
+                             const size_t** shape, size_t* rank) {
+    if (!engine || index >= engine->variables.size()) return KGE_INVALID_ARGUMENT;
+    const Variable& v = engine->variables[index];
+    *name = v.name.c_str();
+    *shape = v.shape.data();
+    *rank = v.shape.size();
+    return KGE_OK;
+}
+
+void kge_engine_destroy(kge_engine* engine) {
+    if (!engine) return;
+    if (engine->stream) (void)hipStreamSynchronize(engine->stream);
+    delete engine;
+}
+
+// ---- device ops --------------------------------------------------------------
+
+static int op_status(const char* what) {
+    (void)what;
+    return hipGetLastError() == hipSuccess ? KGE_OK : KGE_RUNTIME_ERROR;
+}
+
+static bool bad_dims(int M, int N, int D) { return M < 0 || N < 0 || D < 1; }
+
+int kge_l1_distance(const float* a, const float* b, float* out, int M, int N, int D, void* stream) {
+    if (bad_dims(M, N, D)) return KGE_INVALID_ARGUMENT;
+    if (M == 0 || N == 0) return KGE_OK;
+    launch_distance(DIST_L1, a, b, out, M, N, D, (hipStream_t)stream);
+    return op_status("l1_distance");
+}
+int kge_l2_distance(const float* a, const float* b, float* out, int M, int N, int D, void* stream) {
+    if (bad_dims(M, N, D)) return KGE_INVALID_ARGUMENT;
+    if (M == 0 || N == 0) return KGE_OK;
+    launch_distance(DIST_L2, a, b, out, M, N, D, (hipStream_t)stream);
+    return op_status("l2_distance");
+}
+int kge_dot_score(const float* a, const float* b, float* out, int M, int N, int D, void* stream) {
+    if (bad_dims(M, N, D)) return KGE_INVALID_ARGUMENT;
+    if (M == 0 || N == 0) return KGE_OK;
+    launch_distance(DIST_DOT, a, b, out, M, N, D, (hipStream_t)stream);
+    return op_status("dot_score");
+}
+int kge_l1_distance_grad(const float* a, const float* b, const float* g, float* grad, int M, int N,
+                         int D, void* stream) {
+    if (bad_dims(M, N, D)) return KGE_INVALID_ARGUMENT;
+    if (M == 0) return KGE_OK;
+    launch_distance_grad(DIST_L1, a, b, nullptr, g, grad, M, N, D, (hipStream_t)stream);
+    return op_status("l1_distance_grad");
+}
+int kge_l2_distance_grad(const float* a, const float* b, const float* dist, const float* g,
+                         float* grad, int M, int N, int D, void* stream) {
+    if (bad_dims(M, N, D)) return KGE_INVALID_ARGUMENT;
+    if (M == 0) return KGE_OK;
+    launch_distance_grad(DIST_L2, a, b, dist, g, grad, M, N, D, (hipStream_t)stream);
+    return op_status("l2_distance_grad");
+}
+int kge_buffer_read(const void* buf, const uint32_t* idx, void* out, int64_t n, int64_t row_bytes,
+                    void* stream) {
+    if (n < 0 || row_bytes < 4 || row_bytes % 4) return KGE_INVALID_ARGUMENT;
+    launch_rows_gather(buf, idx, out, n, row_bytes, (hipStream_t)stream);
+    return op_status("buffer_read");
+}
+int kge_buffer_write(void* buf, const uint32_t* idx, const void* data, int64_t n, int64_t row_bytes,
+                     void* stream) {
+    if (n < 0 || row_bytes < 4 || row_bytes % 4) return KGE_INVALID_ARGUMENT;
+    launch_rows_scatter(buf, idx, data, n, row_bytes, (hipStream_t)stream);
+    return op_status("buffer_write");
+}
+
+namespace {
+struct ScatterLayout {
+    size_t N, tiles, cmax;
+    size_t off_keys_a, off_vals_a, off_keys_b, off_vals_b, off_hist, off_uniq, off_seg, off_coff,
+        off_cpos, off_clen, off_counts, off_partial, total;
+};
+ScatterLayout scatter_layout(int64_t n, int64_t rows, int64_t cols) {
+    ScatterLayout L;
+    L.N = (size_t)(n + rows);
+    L.tiles = (L.N + kSortTile - 1) / kSortTile;
+    L.cmax = (size_t)rows + (size_t)n / 32 + 1;
+    size_t o = 0;
+    auto take = [&](size_t words) { size_t at = o; o += (words * 4 + 15) / 16 * 16; return at; };
+    L.off_keys_a = take(L.N); L.off_vals_a = take(L.N);
+    L.off_keys_b = take(L.N); L.off_vals_b = take(L.N);
+    L.off_hist = take(256 * L.tiles);
+    L.off_uniq = take(rows); L.off_seg = take(rows + 1); L.off_coff = take(rows + 1);
+    L.off_cpos = take(L.cmax); L.off_clen = take(L.cmax); L.off_counts = take(2);
+    L.off_partial = take(L.cmax * (size_t)cols);
+    L.total = o;
+    return L;
+}
+}  // namespace
+
+size_t kge_scatter_add_workspace_bytes(int64_t n, int64_t rows, int64_t cols) {
+    if (n < 0 || rows < 1 || cols < 1) return 0;
+    return scatter_layout(n, rows, cols).total;
+}
+
+int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* idx, int64_t n,
+                    const float* grad_out, void* workspace, void* stream) {
+    if (n < 0 || rows < 1 || cols < 1 || n + rows >= ((int64_t)1 << 31)) return KGE_INVALID_ARGUMENT;
+    if (!workspace || (uintptr_t)workspace % 16) return KGE_INVALID_ARGUMENT;
+    const hipStream_t st = (hipStream_t)stream;
+    const ScatterLayout L = scatter_layout(n, rows, cols);
+    char* w = (char*)workspace;
+    auto u32 = [&](size_t off) { return (uint32_t*)(w + off); };
+    launch_iota_keys(idx, u32(L.off_keys_a), u32(L.off_vals_a), n, rows, st);
+    const int bits = std::max(1, bit_length((uint64_t)rows - 1));
+    const int which = launch_radix_sort(u32(L.off_keys_a), u32(L.off_vals_a), u32(L.off_keys_b),
+                                        u32(L.off_vals_b), u32(L.off_hist), (int)L.N, 1, bits, st);
+    SegPlan sp;
+    sp.uniq_key = u32(L.off_uniq); sp.seg_start = u32(L.off_seg); sp.chunk_off = u32(L.off_coff);
+    sp.chunk_pos = u32(L.off_cpos); sp.chunk_len = u32(L.off_clen); sp.counts = u32(L.off_counts);
+    sp.item_row = nullptr; sp.u_stride = (int)rows; sp.c_stride = (int)L.cmax;
+    const uint32_t* sk = which ? u32(L.off_keys_b) : u32(L.off_keys_a);
+    const uint32_t* sv = which ? u32(L.off_vals_b) : u32(L.off_vals_a);
+    launch_find_segments(sk, sv, (int)L.N, (int)n, 32, 1, sp, st);
+    ReduceArgs ra = {};
+    ra.sorted_item = sv; ra.chunk_pos = sp.chunk_pos; ra.chunk_len = sp.chunk_len; ra.counts = sp.counts;
+    ra.max_chunks = (int)L.cmax; ra.grad = grad_out; ra.partial = (float*)(w + L.off_partial);
+    ra.Dp = (int)cols; ra.transform = 0;
+    launch_reduce_chunks(ra, st);
+    launch_sum_partials_rows(sp.chunk_off, ra.partial, rows, cols, grad_t, st);
+    return op_status("scatter_add");
+}
+
+int kge_adam(float* p, float* m, float* v, const float* g, int64_t n, float alpha, float beta_m,
+             float beta_v, float epsilon, float weight_decay, int v_is_sqrt, void* stream) {
+    if (n < 0) return KGE_INVALID_ARGUMENT;
+    launch_adam_flat(p, m, v, g, n, alpha, beta_m, beta_v, epsilon, weight_decay, v_is_sqrt,
+                     (hipStream_t)stream);
+    return op_status("adam");
+}
+
+}  // extern "C"

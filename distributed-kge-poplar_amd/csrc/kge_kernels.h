@@ -1,0 +1,207 @@
+// Internal launcher interface between the engine (host logic) and the gfx950
+// kernels.  Everything here takes device pointers; nothing allocates.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+namespace kge {
+
+enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1 };
+enum { DIST_L1 = 0, DIST_L2 = 1, DIST_DOT = 2 };
+enum { LOSS_LOGSIGMOID = 0, LOSS_SOFTMAX = 1 };
+enum { ET_F32 = 0, ET_BF16 = 1, ET_F16 = 2 };
+
+constexpr int kSortTile = 2048;  // items per workgroup in one radix pass
+constexpr int kScoreTile = 64;   // score tile edge (rows of either operand)
+
+// Indexed rows: logical row r is `count` elements of type `etype` starting at
+// base + index[r] * pitch (bytes).
+struct RowSource {
+    const char* base;
+    int64_t pitch;
+    int etype;
+    const uint32_t* index;  // null: identity
+    int count;              // elements per row
+    int vec;                // rows 16-byte aligned and count % 4 == 0: float4 access allowed
+};
+
+// ---- plan phase (index-only work, batched over the steps of one call) ----
+
+struct PlanShape {
+    int n_step, S, B, A, NR;  // NR = B + S*A slots per shard
+    int n_entity;             // rows per shard table
+    int shared_table;
+    int n_relation;
+};
+
+// Compact per-step arrays + the items to sort for the entity plan and the
+// relation plan.  Item layout, entity plan (2R items, R = S*NR):
+//   [0, S*B)          head contributions  c = d*B + b
+//   [S*B, R)          tail contributions  c = S*B + d*T + (j*A + i)
+//   [R, 2R)           every remote slot, as a zero-gradient member of the update set
+// relation plan (S*B + n_relation items): head contributions, then every relation id.
+void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
+                        const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
+                        uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
+                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals,
+                        hipStream_t stream);
+
+// Stable LSD radix sort of n_seg independent arrays of N (key, value) pairs on
+// the low `key_bits` bits.  Result is in keys_a/vals_a if the return value is
+// 0, in keys_b/vals_b if it is 1.  hist must hold n_seg * 256 * ceil(N/kSortTile) words.
+int launch_radix_sort(uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
+                      uint32_t* hist, int N, int n_seg, int key_bits, hipStream_t stream);
+
+// Per-segment outputs of the segment finder, all with a per-step stride.
+struct SegPlan {
+    uint32_t* uniq_key;   // [n_seg, u_stride]      key of each distinct row, ascending
+    uint32_t* seg_start;  // [n_seg, u_stride + 1]  first sorted position of each row
+    uint32_t* chunk_off;  // [n_seg, u_stride + 1]  first chunk of each row
+    uint32_t* chunk_pos;  // [n_seg, c_stride]      first sorted position of each chunk
+    uint32_t* chunk_len;  // [n_seg, c_stride]      real items in the chunk (<= chunk size)
+    uint32_t* counts;     // [n_seg, 2]             {distinct rows, chunks}
+    uint32_t* item_row;   // [n_seg, n_real] or null: distinct-row index of each real item
+    int u_stride, c_stride;
+};
+
+void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sorted, int N,
+                          int n_real, int chunk, int n_seg, const SegPlan& plan,
+                          hipStream_t stream);
+
+// ---- step phase ----------------------------------------------------------
+
+struct ScoreShape {
+    int S, B, T, Dp;   // Dp: embedding size rounded up to a multiple of 4
+    int score_fn, dist_fn, loss_fn;
+    float gamma, loss_scale;
+    float softmax_correction;      // already multiplied by the correction weight
+    float negative_adversarial_scale;
+};
+
+// Scores of every block: a-operand row (d,b) = entity row of contribution
+// d*B+b combined with relation crel[d*B+b]; b-operand row (d,t) = entity row of
+// contribution S*B + d*T + t.  With `fused_loss` the logsigmoid loss and the
+// backward coefficient are produced in the epilogue; otherwise the raw score is
+// stored in `coef` (and the L2 distance in `dist`) for launch_loss_rows.
+// loss_part receives S * n_part partial sums (n_part = tiles per block).
+void launch_score_fwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
+                      const uint32_t* crel, const uint32_t* clabel, float* coef, float* dist,
+                      float* loss_part, bool fused_loss, hipStream_t stream);
+int score_fwd_parts(const ScoreShape& sh);
+
+// Row-wise losses (softmax; logsigmoid with adversarial weighting): converts
+// the raw scores in `coef` to backward coefficients in place; loss_part gets
+// S * B partial sums.
+void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef, const float* dist,
+                      float* loss_part, hipStream_t stream);
+
+// Gradient rows of every contribution: grad[c, :] for head contributions
+// (w.r.t. the predicted tail / the head-times-relation product) and tail
+// contributions, from the coefficient matrix.
+void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
+                      const uint32_t* crel, const float* coef, float* grad, hipStream_t stream);
+
+// Deterministic segmented reduction, first level: one wave per chunk sums the
+// chunk's gradient rows in sorted order into partial[chunk, :].
+// transform: 0 none; 1 multiply head rows (c < n_head) by rel[crel[c]]
+// (DistMult, entity plan); 2 multiply by the head entity row (DistMult,
+// relation plan).
+struct ReduceArgs {
+    const uint32_t* sorted_item;  // this step's sorted values
+    const uint32_t* chunk_pos;
+    const uint32_t* chunk_len;
+    const uint32_t* counts;       // {rows, chunks}
+    int max_chunks;
+    const float* grad;            // [R, Dp]
+    float* partial;               // [max_chunks, Dp]
+    int Dp;
+    int transform, n_head;
+    const float* rel;
+    const uint32_t* crel;
+    RowSource ent;
+};
+void launch_reduce_chunks(const ReduceArgs& a, hipStream_t stream);
+
+// Second level fused with Adam: one wave per distinct row sums its chunk
+// partials in order, applies the update in place and (optionally) stores the
+// summed gradient.
+struct AdamArgs {
+    const uint32_t* uniq_key;
+    const uint32_t* chunk_off;
+    const uint32_t* counts;
+    int max_rows;
+    const float* partial;      // [chunks, Dp] or null
+    const float* grad_direct;  // [rows, Dp] used instead of partial when non-null
+    float* grad_out;           // [rows, Dp] or null
+    char* p_base;              // parameter rows: p_base + key * pitch
+    char* m_base;
+    char* v_base;
+    int64_t pitch;
+    int p_etype;               // ET_* of the parameter (moments are float32)
+    int Dp;
+    int v_is_sqrt;
+    const float* alpha;        // [n_alpha] step sizes
+    uint32_t rows_per_alpha;   // alpha index = key / rows_per_alpha (0: always alpha[0])
+    float beta_m, beta_v, one_minus_beta_m, one_minus_beta_v, epsilon, weight_decay;
+};
+void launch_adam_rows(const AdamArgs& a, hipStream_t stream);
+
+// loss[s] = sum over steps and parts of loss_part / n_step, in a fixed order.
+void launch_loss_finalize(const float* loss_part, int n_step, int S, int n_part, float scale,
+                          float* loss, hipStream_t stream);
+
+// ---- feature projection (hidden = emb + feature * W) -----------------------
+struct FeatureArgs {
+    const uint32_t* uniq_key;
+    const uint32_t* counts;
+    int max_rows;
+    const char* emb_base;   // table + emb offset
+    const char* feat_base;  // table + feature offset
+    int64_t pitch;
+    int emb_etype, feat_etype;
+    int Dp, Fp;
+    const float* proj;      // [Fp, Dp]
+};
+void launch_hidden_fwd(const FeatureArgs& a, float* hidden, hipStream_t stream);
+// gproj[f, :] = sum_u feature[u, f] * grad_rows[u, :]
+void launch_proj_grad(const FeatureArgs& a, const float* grad_rows, float* gproj,
+                      hipStream_t stream);
+
+// ---- table access ----------------------------------------------------------
+void launch_rows_gather(const void* buf, const uint32_t* idx, void* out, int64_t n,
+                        int64_t row_bytes, hipStream_t stream);
+void launch_rows_scatter(void* buf, const uint32_t* idx, const void* data, int64_t n,
+                         int64_t row_bytes, hipStream_t stream);
+
+struct RowLayout {
+    int D, F, Dp, Fp;
+    int emb_etype, mom_etype, feat_etype;
+    int64_t off_m, off_s, off_f, pitch;  // bytes; embedding at offset 0
+};
+// logical float32 rows [n, 3D+F] <-> physical rows at base + idx[i]*pitch
+void launch_rows_to_logical(const RowLayout& L, const char* base, const uint64_t* rows, int64_t n,
+                            float* out, hipStream_t stream);
+void launch_rows_from_logical(const RowLayout& L, char* base, const uint64_t* rows, int64_t n,
+                              const float* in, hipStream_t stream);
+// write_entity: embedding ~ N(0, sigma) from a counter-based generator keyed by
+// (seed, row, column); zero moments; features from `features` [n, F] float32.
+void launch_init_rows(const RowLayout& L, char* base, const uint64_t* rows, int64_t n,
+                      const float* features, float sigma, uint32_t seed, hipStream_t stream);
+
+// ---- standalone ops --------------------------------------------------------
+void launch_distance(int dist_fn, const float* a, const float* b, float* out, int M, int N, int D,
+                     hipStream_t stream);
+void launch_distance_grad(int dist_fn, const float* a, const float* b, const float* dist,
+                          const float* g, float* grad, int M, int N, int D, hipStream_t stream);
+void launch_adam_flat(float* p, float* m, float* v, const float* g, int64_t n, float alpha,
+                      float beta_m, float beta_v, float epsilon, float weight_decay, int v_is_sqrt,
+                      hipStream_t stream);
+void launch_fill_u32(uint32_t* p, uint32_t value, int64_t n, hipStream_t stream);
+void launch_iota_keys(const uint32_t* idx, uint32_t* keys, uint32_t* vals, int64_t n, int64_t rows,
+                      hipStream_t stream);
+void launch_sum_partials_rows(const uint32_t* chunk_off, const float* partial, int64_t rows,
+                              int64_t cols, float* out, hipStream_t stream);
+
+}  // namespace kge

@@ -1,0 +1,1279 @@
+// gfx950 (CDNA4, wave64) kernels of the per-shard KGE training step.
+//
+// Reference semantics, by kernel:
+//   build_items / radix sort / find_segments  host np.unique + multiUpdateAdd grouping
+//       (src/python/poplar_kge_dataset.py:161-164, src/pag/pag.cpp:721-743)
+//   score_fwd      predictTail + score + logsigmoid loss (src/poplar_kge.cpp:488-499,
+//                  567-573, 615-636; l1/l2distance codelets)
+//   loss_rows      softmax / adversarial loss (src/poplar_kge.cpp:623-652)
+//   score_bwd      l1/l2distancegrad, matMul backward (src/pag/pag.cpp:685-700, 777-836)
+//   reduce_chunks + adam_rows   multiUpdateAdd + fr::nn::adam + Buffer::write
+//                  (src/fructose/frnn.cpp:61-90, src/poplar_kge.cpp:695-704)
+#include "kge_kernels.h"
+
+#include <algorithm>
+
+namespace kge {
+
+#define DEVINL __device__ __forceinline__
+
+// --------------------------------------------------------------------------
+// element access
+
+DEVINL float bf16_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+DEVINL uint16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// four consecutive elements starting at element k (k % 4 == 0) of a row
+DEVINL float4 load4(const char* row, int k, int etype) {
+    if (etype == ET_F32) return *reinterpret_cast<const float4*>(row + (size_t)k * 4);
+    const uint2 raw = *reinterpret_cast<const uint2*>(row + (size_t)k * 2);
+    if (etype == ET_BF16)
+        return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                           __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u));
+    const __half2 h0 = *reinterpret_cast<const __half2*>(&raw.x);
+    const __half2 h1 = *reinterpret_cast<const __half2*>(&raw.y);
+    const float2 f0 = __half22float2(h0), f1 = __half22float2(h1);
+    return make_float4(f0.x, f0.y, f1.x, f1.y);
+}
+
+DEVINL void store4(char* row, int k, int etype, float4 v) {
+    if (etype == ET_F32) {
+        *reinterpret_cast<float4*>(row + (size_t)k * 4) = v;
+        return;
+    }
+    uint2 raw;
+    if (etype == ET_BF16) {
+        raw.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+        raw.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+    } else {
+        const __half2 h0 = __floats2half2_rn(v.x, v.y), h1 = __floats2half2_rn(v.z, v.w);
+        raw.x = *reinterpret_cast<const uint32_t*>(&h0);
+        raw.y = *reinterpret_cast<const uint32_t*>(&h1);
+    }
+    *reinterpret_cast<uint2*>(row + (size_t)k * 2) = raw;
+}
+
+// guarded variant for sources whose rows are not 16-byte aligned or whose
+// length is not a multiple of four (standalone ops on arbitrary shapes)
+DEVINL float load1(const char* sec, int k, int etype) {
+    if (etype == ET_F32) return reinterpret_cast<const float*>(sec)[k];
+    if (etype == ET_BF16) return bf16_to_f32(reinterpret_cast<const uint16_t*>(sec)[k]);
+    return __half2float(reinterpret_cast<const __half*>(sec)[k]);
+}
+DEVINL float4 load4(const char* row, int k, const RowSource& s) {
+    if (s.vec) return load4(row, k, s.etype);
+    float v[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) v[x] = (k + x < s.count) ? load1(row, k + x, s.etype) : 0.f;
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+
+DEVINL const char* row_ptr(const RowSource& s, uint32_t r) {
+    const uint32_t key = s.index ? s.index[r] : r;
+    return s.base + (int64_t)key * s.pitch;
+}
+
+DEVINL float4 f4add(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+DEVINL float4 f4mul(float4 a, float4 b) { return make_float4(a.x * b.x, a.y * b.y, a.z * b.z, a.w * b.w); }
+
+// rel_mode: 0 none, 1 add (TransE), 2 multiply (DistMult)
+DEVINL float4 combine_rel(float4 e, const float* relrow, int k, int rel_mode) {
+    if (rel_mode == 0) return e;
+    const float4 r = *reinterpret_cast<const float4*>(relrow + k);
+    return rel_mode == 1 ? f4add(e, r) : f4mul(e, r);
+}
+
+DEVINL float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+DEVINL float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// --------------------------------------------------------------------------
+// plan phase
+
+__global__ __launch_bounds__(256) void k_build_items(PlanShape ps, const uint32_t* __restrict__ remote,
+                                                     const uint32_t* __restrict__ a2a,
+                                                     const uint32_t* __restrict__ head,
+                                                     const uint32_t* __restrict__ relation,
+                                                     const uint32_t* __restrict__ tail,
+                                                     uint32_t* __restrict__ ckey,
+                                                     uint32_t* __restrict__ crel,
+                                                     uint32_t* __restrict__ clabel,
+                                                     uint32_t* __restrict__ ent_keys,
+                                                     uint32_t* __restrict__ ent_vals,
+                                                     uint32_t* __restrict__ rel_keys,
+                                                     uint32_t* __restrict__ rel_vals) {
+    const int step = blockIdx.y;
+    const int S = ps.S, B = ps.B, A = ps.A, NR = ps.NR, T = S * A, nst = ps.n_step;
+    const int R = S * NR, SB = S * B;
+    const int item = blockIdx.x * 256 + threadIdx.x;
+    const int n_rel_items = SB + ps.n_relation;
+    if (item < 2 * R) {
+        int src, slot;
+        if (item < SB) {
+            const int d = item / B, b = item - d * B;
+            src = d;
+            slot = head[((size_t)d * nst + step) * B + b];
+        } else if (item < R) {
+            const int cc = item - SB;
+            const int d = cc / T, t = cc - d * T;
+            const int j = t / A, i = t - j * A;
+            src = j;
+            slot = a2a[(((size_t)j * nst + step) * S + d) * A + i];
+        } else {
+            const int sl = item - R;
+            src = sl / NR;
+            slot = sl - src * NR;
+        }
+        const uint32_t base = ps.shared_table ? 0u : (uint32_t)src * (uint32_t)ps.n_entity;
+        const uint32_t key = base + remote[((size_t)src * nst + step) * NR + slot];
+        if (item < R) ckey[(size_t)step * R + item] = key;
+        ent_keys[(size_t)step * 2 * R + item] = key;
+        ent_vals[(size_t)step * 2 * R + item] = item;
+    }
+    if (item < n_rel_items) {
+        uint32_t key;
+        if (item < SB) {
+            const int d = item / B, b = item - d * B;
+            key = relation[((size_t)d * nst + step) * B + b];
+            crel[(size_t)step * SB + item] = key;
+            clabel[(size_t)step * SB + item] = tail[((size_t)d * nst + step) * B + b];
+        } else {
+            key = item - SB;
+        }
+        rel_keys[(size_t)step * n_rel_items + item] = key;
+        rel_vals[(size_t)step * n_rel_items + item] = item;
+    }
+}
+
+void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
+                        const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
+                        uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
+                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals,
+                        hipStream_t stream) {
+    const int R = ps.S * ps.NR;
+    const int n = std::max(2 * R, ps.S * ps.B + ps.n_relation);
+    dim3 grid((n + 255) / 256, ps.n_step);
+    hipLaunchKernelGGL(k_build_items, grid, dim3(256), 0, stream, ps, remote, a2a, head, relation,
+                       tail, ckey, crel, clabel, ent_keys, ent_vals, rel_keys, rel_vals);
+}
+
+// ---- stable LSD radix sort, 8 bits per pass --------------------------------
+// hist layout: [seg][digit][tile]
+
+__global__ __launch_bounds__(256) void k_sort_hist(const uint32_t* __restrict__ keys, int N,
+                                                   int n_tiles, int shift,
+                                                   uint32_t* __restrict__ hist) {
+    __shared__ uint32_t h[256];
+    const int seg = blockIdx.y, tile = blockIdx.x;
+    h[threadIdx.x] = 0;
+    __syncthreads();
+    const uint32_t* k = keys + (size_t)seg * N;
+    const int base = tile * kSortTile;
+#pragma unroll
+    for (int r = 0; r < kSortTile / 256; ++r) {
+        const int i = base + r * 256 + threadIdx.x;
+        if (i < N) atomicAdd(&h[(k[i] >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    hist[((size_t)seg * 256 + threadIdx.x) * n_tiles + tile] = h[threadIdx.x];
+}
+
+// exclusive scan over (digit-major, tile-minor) for one segment per block
+__global__ __launch_bounds__(256) void k_sort_scan(uint32_t* __restrict__ hist, int n_tiles) {
+    __shared__ uint32_t tot[256];
+    const int seg = blockIdx.x, d = threadIdx.x;
+    uint32_t* h = hist + ((size_t)seg * 256 + d) * n_tiles;
+    uint32_t sum = 0;
+    for (int t = 0; t < n_tiles; ++t) sum += h[t];
+    tot[d] = sum;
+    __syncthreads();
+    // Hillis-Steele inclusive scan over the 256 digit totals
+    for (int off = 1; off < 256; off <<= 1) {
+        uint32_t v = d >= off ? tot[d - off] : 0;
+        __syncthreads();
+        tot[d] += v;
+        __syncthreads();
+    }
+    uint32_t run = tot[d] - sum;  // exclusive base of digit d
+    for (int t = 0; t < n_tiles; ++t) {
+        const uint32_t c = h[t];
+        h[t] = run;
+        run += c;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_sort_scatter(const uint32_t* __restrict__ keys_in,
+                                                      const uint32_t* __restrict__ vals_in,
+                                                      uint32_t* __restrict__ keys_out,
+                                                      uint32_t* __restrict__ vals_out, int N,
+                                                      int n_tiles, int shift,
+                                                      const uint32_t* __restrict__ hist) {
+    // run[w][digit]: next output position for wave w's items with that digit
+    __shared__ uint32_t run[4][256];
+    const int seg = blockIdx.y, tile = blockIdx.x;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const uint32_t* kin = keys_in + (size_t)seg * N;
+    const uint32_t* vin = vals_in + (size_t)seg * N;
+    constexpr int ROUNDS = kSortTile / 256;  // rounds of 64 items per wave
+    const int wbase = tile * kSortTile + wave * (kSortTile / 4);
+
+    for (int i = tid; i < 4 * 256; i += 256) (&run[0][0])[i] = 0;
+    __syncthreads();
+    uint32_t key[ROUNDS], val[ROUNDS];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        const int i = wbase + r * 64 + lane;
+        key[r] = i < N ? kin[i] : 0xffffffffu;
+        val[r] = i < N ? vin[i] : 0u;
+        if (i < N) atomicAdd(&run[wave][(key[r] >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    {   // per digit: exclusive prefix over the four waves + the tile's global base
+        const int d = tid;
+        uint32_t base = hist[((size_t)seg * 256 + d) * n_tiles + tile];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t c = run[w][d];
+            run[w][d] = base;
+            base += c;
+        }
+    }
+    __syncthreads();
+    uint32_t* kout = keys_out + (size_t)seg * N;
+    uint32_t* vout = vals_out + (size_t)seg * N;
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        const int i = wbase + r * 64 + lane;
+        const bool valid = i < N;
+        const uint32_t digit = (key[r] >> shift) & 255u;
+        // lanes of this wave holding the same digit (match-any by 8 ballots)
+        uint64_t peers = __ballot(valid);
+#pragma unroll
+        for (int bit = 0; bit < 8; ++bit) {
+            const uint64_t m = __ballot((digit >> bit) & 1u);
+            peers &= ((digit >> bit) & 1u) ? m : ~m;
+        }
+        const uint64_t lt = (1ull << lane) - 1ull;
+        const uint32_t rank = __popcll(peers & lt);
+        uint32_t off = 0;
+        if (valid) off = run[wave][digit];
+        __syncthreads();
+        if (valid && rank == 0) run[wave][digit] = off + (uint32_t)__popcll(peers);
+        __syncthreads();
+        if (valid) {
+            kout[off + rank] = key[r];
+            vout[off + rank] = val[r];
+        }
+    }
+}
+
+int launch_radix_sort(uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
+                      uint32_t* hist, int N, int n_seg, int key_bits, hipStream_t stream) {
+    const int n_tiles = (N + kSortTile - 1) / kSortTile;
+    int passes = (key_bits + 7) / 8;
+    if (passes < 1) passes = 1;
+    uint32_t *kin = keys_a, *vin = vals_a, *kout = keys_b, *vout = vals_b;
+    for (int p = 0; p < passes; ++p) {
+        const int shift = 8 * p;
+        hipLaunchKernelGGL(k_sort_hist, dim3(n_tiles, n_seg), dim3(256), 0, stream, kin, N, n_tiles,
+                           shift, hist);
+        hipLaunchKernelGGL(k_sort_scan, dim3(n_seg), dim3(256), 0, stream, hist, n_tiles);
+        hipLaunchKernelGGL(k_sort_scatter, dim3(n_tiles, n_seg), dim3(256), 0, stream, kin, vin,
+                           kout, vout, N, n_tiles, shift, hist);
+        uint32_t* t = kin; kin = kout; kout = t;
+        t = vin; vin = vout; vout = t;
+    }
+    return (passes & 1);  // odd number of passes: result is in the b buffers
+}
+
+// ---- segments and chunks ---------------------------------------------------
+
+// exclusive scan of one value per thread over a 1024-thread block
+DEVINL uint32_t block_scan_1024(uint32_t v, uint32_t* lds /*[16]*/, uint32_t* total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t t = __shfl_up(inc, off, 64);
+        if (lane >= off) inc += t;
+    }
+    __syncthreads();
+    if (lane == 63) lds[wave] = inc;
+    __syncthreads();
+    uint32_t wbase = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+        const uint32_t c = lds[w];
+        if (w < wave) wbase += c;
+        tot += c;
+    }
+    *total = tot;
+    return wbase + inc - v;
+}
+
+__global__ __launch_bounds__(1024) void k_find_segments(const uint32_t* __restrict__ keys,
+                                                        const uint32_t* __restrict__ vals, int N,
+                                                        int n_real, int chunk, SegPlan plan) {
+    __shared__ uint32_t lds[16];
+    const int seg = blockIdx.x, tid = threadIdx.x;
+    keys += (size_t)seg * N;
+    vals += (size_t)seg * N;
+    uint32_t* uniq_key = plan.uniq_key + (size_t)seg * plan.u_stride;
+    uint32_t* seg_start = plan.seg_start + (size_t)seg * (plan.u_stride + 1);
+    uint32_t* chunk_off = plan.chunk_off + (size_t)seg * (plan.u_stride + 1);
+    uint32_t* chunk_pos = plan.chunk_pos + (size_t)seg * plan.c_stride;
+    uint32_t* chunk_len = plan.chunk_len + (size_t)seg * plan.c_stride;
+    uint32_t* item_row = plan.item_row ? plan.item_row + (size_t)seg * n_real : nullptr;
+
+    const int per = (N + 1023) / 1024;
+    const int lo = min(N, tid * per), hi = min(N, lo + per);
+    uint32_t cnt = 0;
+    for (int i = lo; i < hi; ++i) cnt += (i == 0 || keys[i] != keys[i - 1]) ? 1u : 0u;
+    uint32_t U;
+    const uint32_t ubase = block_scan_1024(cnt, lds, &U);
+    {
+        uint32_t u = ubase;  // index of the next distinct row to start
+        for (int i = lo; i < hi; ++i) {
+            if (i == 0 || keys[i] != keys[i - 1]) {
+                uniq_key[u] = keys[i];
+                seg_start[u] = i;
+                ++u;
+            }
+            if (item_row && vals[i] < (uint32_t)n_real) item_row[vals[i]] = u - 1;
+        }
+    }
+    if (tid == 0) seg_start[U] = N;
+    __syncthreads();
+
+    const int uper = ((int)U + 1023) / 1024;
+    const int ulo = min((int)U, tid * uper), uhi = min((int)U, ulo + uper);
+    uint32_t nch = 0;
+    for (int u = ulo; u < uhi; ++u) {
+        const uint32_t s = seg_start[u], e = seg_start[u + 1];
+        // real items (value < n_real) precede the others within a segment
+        uint32_t a = s, b = e;
+        while (a < b) {
+            const uint32_t mid = (a + b) >> 1;
+            if (vals[mid] < (uint32_t)n_real) a = mid + 1; else b = mid;
+        }
+        nch += (a - s + chunk - 1) / chunk;
+    }
+    uint32_t NC;
+    uint32_t cb = block_scan_1024(nch, lds, &NC);
+    for (int u = ulo; u < uhi; ++u) {
+        const uint32_t s = seg_start[u], e = seg_start[u + 1];
+        uint32_t a = s, b = e;
+        while (a < b) {
+            const uint32_t mid = (a + b) >> 1;
+            if (vals[mid] < (uint32_t)n_real) a = mid + 1; else b = mid;
+        }
+        const uint32_t real = a - s;
+        chunk_off[u] = cb;
+        for (uint32_t l = 0; l * chunk < real; ++l) {
+            chunk_pos[cb] = s + l * chunk;
+            chunk_len[cb] = min((uint32_t)chunk, real - l * chunk);
+            ++cb;
+        }
+    }
+    if (tid == 0) {
+        chunk_off[U] = NC;
+        plan.counts[2 * seg] = U;
+        plan.counts[2 * seg + 1] = NC;
+    }
+}
+
+void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sorted, int N,
+                          int n_real, int chunk, int n_seg, const SegPlan& plan,
+                          hipStream_t stream) {
+    hipLaunchKernelGGL(k_find_segments, dim3(n_seg), dim3(1024), 0, stream, keys_sorted,
+                       vals_sorted, N, n_real, chunk, plan);
+}
+
+// --------------------------------------------------------------------------
+// scoring: forward
+
+// logSigmoid and its derivative exactly as src/pag/pag.cpp:894-903
+DEVINL float log_sigmoid(float z) { return z > -11.f ? -log1pf(expf(-z)) : z; }
+DEVINL float log_sigmoid_grad(float z) { return 1.f / (1.f + expf(fminf(z, 11.f))); }
+
+struct FwdParams {
+    ScoreShape sh;
+    RowSource ent_a, ent_b;
+    const float* rel;
+    const uint32_t* crel;
+    const uint32_t* clabel;
+    float* coef;
+    float* dist;
+    float* loss_part;
+    int a_rel_mode;   // how the a-operand combines with its relation row
+    int out_mode;     // 0 fused logsigmoid -> coefficient; 1 raw score (+dist); 2 raw distance
+    int a_c0, b_c0;   // contribution index of block 0's first a / b row
+};
+
+constexpr int BK = 32;         // embedding columns staged per iteration
+constexpr int LDP = kScoreTile + 4;  // padded LDS row (floats), keeps float4 reads aligned
+
+template <int DIST>
+__global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
+    __shared__ __attribute__((aligned(16))) float As[BK][LDP];
+    __shared__ __attribute__((aligned(16))) float Bs[BK][LDP];
+    __shared__ float red[4];
+    const ScoreShape& sh = p.sh;
+    const int d = blockIdx.z, m0 = blockIdx.y * kScoreTile, n0 = blockIdx.x * kScoreTile;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int B = sh.B, T = sh.T, Dp = sh.Dp;
+
+    // staging assignment: row lr (+32) of each operand, float4 column k4
+    const int lr = tid >> 3, k4 = (tid & 7) * 4;
+    const char* arow[2];
+    const char* brow[2];
+    const float* rrow[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int m = m0 + lr + 32 * h, n = n0 + lr + 32 * h;
+        arow[h] = m < B ? row_ptr(p.ent_a, p.a_c0 + d * B + m) : nullptr;
+        rrow[h] = (m < B && p.a_rel_mode) ? p.rel + (size_t)p.crel[d * B + m] * Dp : nullptr;
+        brow[h] = n < T ? row_ptr(p.ent_b, p.b_c0 + d * T + n) : nullptr;
+    }
+
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+    for (int k0 = 0; k0 < Dp; k0 += BK) {
+        const int k = k0 + k4;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float4 a = make_float4(0, 0, 0, 0), b = a;
+            if (k < Dp) {
+                if (arow[h]) a = combine_rel(load4(arow[h], k, p.ent_a), rrow[h], k, p.a_rel_mode);
+                if (brow[h]) b = load4(brow[h], k, p.ent_b);
+            }
+            const int r = lr + 32 * h;
+            As[k4 + 0][r] = a.x; As[k4 + 1][r] = a.y; As[k4 + 2][r] = a.z; As[k4 + 3][r] = a.w;
+            Bs[k4 + 0][r] = b.x; Bs[k4 + 1][r] = b.y; Bs[k4 + 2][r] = b.z; Bs[k4 + 3][r] = b.w;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK; ++kk) {
+            const float4 a4 = *reinterpret_cast<const float4*>(&As[kk][ty * 4]);
+            const float4 b4 = *reinterpret_cast<const float4*>(&Bs[kk][tx * 4]);
+            const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+            const float bv[4] = {b4.x, b4.y, b4.z, b4.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (DIST == DIST_L1) {
+                        acc[i][j] += fabsf(av[i] - bv[j]);
+                    } else if (DIST == DIST_L2) {
+                        const float t = av[i] - bv[j];
+                        acc[i][j] = fmaf(t, t, acc[i][j]);
+                    } else {
+                        acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+                    }
+                }
+        }
+        __syncthreads();
+    }
+
+    // epilogue
+    const float Tn = (float)T;
+    const float w_pos = 0.5f * Tn, w_neg = (0.5f * Tn) / (float)(T - 1);
+    const float inv_norm = 1.f / ((float)sh.S * (float)B * Tn);
+    float loss_acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= B) continue;
+        const uint32_t label = p.out_mode == 0 ? p.clabel[d * B + m] : 0u;
+        float outv[4], distv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            const float dist = DIST == DIST_L2 ? sqrtf(acc[i][j]) : acc[i][j];
+            distv[j] = dist;
+            if (p.out_mode == 2) { outv[j] = dist; continue; }
+            const float score = sh.score_fn == SCORE_DISTMULT ? dist : sh.gamma - dist;
+            if (p.out_mode == 1) { outv[j] = score; continue; }
+            const bool pos = (uint32_t)n == label;
+            const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
+            const float z = sign * score;
+            if (n < T) loss_acc -= w * log_sigmoid(z);
+            // d loss / d score, times the loss scale
+            const float ds = -w * sign * log_sigmoid_grad(z) * inv_norm * sh.loss_scale;
+            float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;  // score = gamma - dist
+            if (DIST == DIST_L2) c = dist != 0.f ? c / dist : 0.f;
+            outv[j] = c;
+        }
+        const int n = n0 + tx * 4;
+        float* crow = p.coef + ((size_t)d * B + m) * T;
+        float* drow = (p.out_mode == 1 && DIST == DIST_L2 && p.dist) ? p.dist + ((size_t)d * B + m) * T : nullptr;
+        if (n + 3 < T && (T & 3) == 0) {
+            *reinterpret_cast<float4*>(crow + n) = make_float4(outv[0], outv[1], outv[2], outv[3]);
+            if (drow) *reinterpret_cast<float4*>(drow + n) = make_float4(distv[0], distv[1], distv[2], distv[3]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (n + j < T) {
+                    crow[n + j] = outv[j];
+                    if (drow) drow[n + j] = distv[j];
+                }
+        }
+    }
+    if (p.out_mode == 0) {
+        loss_acc = wave_sum(loss_acc);
+        if ((tid & 63) == 0) red[tid >> 6] = loss_acc;
+        __syncthreads();
+        if (tid == 0) {
+            const int n_part = gridDim.x * gridDim.y;
+            p.loss_part[(size_t)d * n_part + blockIdx.y * gridDim.x + blockIdx.x] =
+                (red[0] + red[1] + red[2] + red[3]) * inv_norm;
+        }
+    }
+}
+
+int score_fwd_parts(const ScoreShape& sh) {
+    return ((sh.T + kScoreTile - 1) / kScoreTile) * ((sh.B + kScoreTile - 1) / kScoreTile);
+}
+
+static void launch_fwd(const FwdParams& p, hipStream_t stream) {
+    dim3 grid((p.sh.T + kScoreTile - 1) / kScoreTile, (p.sh.B + kScoreTile - 1) / kScoreTile, p.sh.S);
+    if (p.sh.dist_fn == DIST_L1)
+        hipLaunchKernelGGL(k_score_fwd<DIST_L1>, grid, dim3(256), 0, stream, p);
+    else if (p.sh.dist_fn == DIST_L2)
+        hipLaunchKernelGGL(k_score_fwd<DIST_L2>, grid, dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL(k_score_fwd<DIST_DOT>, grid, dim3(256), 0, stream, p);
+}
+
+void launch_score_fwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
+                      const uint32_t* crel, const uint32_t* clabel, float* coef, float* dist,
+                      float* loss_part, bool fused_loss, hipStream_t stream) {
+    FwdParams p;
+    p.sh = sh;
+    if (sh.score_fn == SCORE_DISTMULT) p.sh.dist_fn = DIST_DOT;
+    p.ent_a = ent; p.ent_b = ent; p.rel = rel; p.crel = crel; p.clabel = clabel;
+    p.coef = coef; p.dist = dist; p.loss_part = loss_part;
+    p.a_rel_mode = sh.score_fn == SCORE_DISTMULT ? 2 : 1;
+    p.out_mode = fused_loss ? 0 : 1;
+    p.a_c0 = 0; p.b_c0 = sh.S * sh.B;
+    launch_fwd(p, stream);
+}
+
+// --------------------------------------------------------------------------
+// row-wise losses: softmax cross entropy with the sampling correction
+// (src/poplar_kge.cpp:638-652) and logsigmoid with self-adversarial negative
+// weights (src/poplar_kge.cpp:623-633).  One wave per (block, positive).
+
+__global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t* __restrict__ clabel,
+                                                   float* __restrict__ coef,
+                                                   const float* __restrict__ dist,
+                                                   float* __restrict__ loss_part) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // d*B + b
+    if (row >= sh.S * sh.B) return;
+    const int T = sh.T;
+    float* s = coef + (size_t)row * T;
+    const float* dr = dist ? dist + (size_t)row * T : nullptr;
+    const uint32_t label = clabel[row];
+    float loss = 0.f;
+    if (sh.loss_fn == LOSS_SOFTMAX) {
+        const float corr = sh.softmax_correction;
+        float mx = -INFINITY;
+        for (int t = lane; t < T; t += 64) mx = fmaxf(mx, s[t] + ((uint32_t)t == label ? 0.f : corr));
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int t = lane; t < T; t += 64) sum += expf(s[t] + ((uint32_t)t == label ? 0.f : corr) - mx);
+        sum = wave_sum(sum);
+        const float lse = mx + logf(sum);
+        const float inv_norm = 1.f / ((float)sh.S * (float)sh.B);
+        for (int t = lane; t < T; t += 64) {
+            const bool pos = (uint32_t)t == label;
+            const float z = s[t] + (pos ? 0.f : corr);
+            if (pos) loss = -(z - lse) * inv_norm;
+            const float ds = (expf(z - lse) - (pos ? 1.f : 0.f)) * inv_norm * sh.loss_scale;
+            float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;
+            if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
+            s[t] = c;
+        }
+    } else {
+        const float adv = sh.negative_adversarial_scale;
+        const float Tn = (float)T;
+        const float w_pos = 0.5f * Tn, w_neg = (0.5f * Tn) / (float)(T - 1);
+        const float inv_norm = 1.f / ((float)sh.S * (float)sh.B * Tn);
+        float mx = -INFINITY, sum = 1.f;
+        if (adv > 0.f) {
+            for (int t = lane; t < T; t += 64)
+                mx = fmaxf(mx, adv * s[t] + ((uint32_t)t == label ? -10000.f : 0.f));
+            mx = wave_max(mx);
+            sum = 0.f;
+            for (int t = lane; t < T; t += 64)
+                sum += expf(adv * s[t] + ((uint32_t)t == label ? -10000.f : 0.f) - mx);
+            sum = wave_sum(sum);
+        }
+        for (int t = lane; t < T; t += 64) {
+            const bool pos = (uint32_t)t == label;
+            const float sc = s[t];
+            float w = pos ? w_pos : w_neg;
+            if (adv > 0.f) {
+                const float sm = expf(adv * sc + (pos ? -10000.f : 0.f) - mx) / sum;
+                w *= (pos ? 1.f : 0.f) + (Tn - 1.f) * sm;
+            }
+            const float sign = pos ? 1.f : -1.f, z = sign * sc;
+            loss -= w * log_sigmoid(z) * inv_norm;
+            const float ds = -w * sign * log_sigmoid_grad(z) * inv_norm * sh.loss_scale;
+            float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;
+            if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
+            s[t] = c;
+        }
+    }
+    loss = wave_sum(loss);
+    if (lane == 0) loss_part[row] = loss;
+}
+
+void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef, const float* dist,
+                      float* loss_part, hipStream_t stream) {
+    const int rows = sh.S * sh.B;
+    const bool l2 = sh.score_fn == SCORE_TRANSE && sh.dist_fn == DIST_L2;
+    hipLaunchKernelGGL(k_loss_rows, dim3((rows + 3) / 4), dim3(256), 0, stream, sh, clabel, coef,
+                       l2 ? dist : nullptr, loss_part);
+}
+
+// --------------------------------------------------------------------------
+// scoring: backward.  out[i, k] = sum_j c[i, j] * phi(self[i, k], other[j, k])
+//   L1   phi = signum(self - other)
+//   L2   phi = self - other              (c already holds g / dist)
+//   DOT  phi = other
+
+struct BwdParams {
+    RowSource ent_a, ent_b;
+    const float* rel;
+    const uint32_t* crel;
+    const float* coef;     // [S, B, T]
+    const float* coef_div; // null, or [S, B, T]: coefficient = coef / coef_div, 0 where coef_div == 0
+    float* grad;           // [R, Dp]
+    int S, B, T, Dp;
+    int side_b;            // 0: self = a-operand rows (heads), 1: self = b-operand rows (tails)
+    int grad_c0;           // output row of block 0's first self row
+    int vec_out;           // output rows allow aligned float4 stores
+    int a_rel_mode;        // relation combine of the a-operand
+    int a_c0, b_c0;
+};
+
+constexpr int BJ = 32;  // rows of `other` staged per iteration
+
+template <int DIST>
+__global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
+    __shared__ __attribute__((aligned(16))) float Cs[BJ][LDP];  // Cs[j][i]
+    __shared__ __attribute__((aligned(16))) float Os[BJ][LDP];  // Os[j][k]
+    const int d = blockIdx.z, i0 = blockIdx.y * kScoreTile, kt0 = blockIdx.x * kScoreTile;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int B = p.B, T = p.T, Dp = p.Dp;
+    const int n_self = p.side_b ? T : B, n_other = p.side_b ? B : T;
+    const int self_c0 = (p.side_b ? p.b_c0 + d * T : p.a_c0 + d * B);
+    const int other_c0 = (p.side_b ? p.a_c0 + d * B : p.b_c0 + d * T);
+    const int self_rel = p.side_b ? 0 : p.a_rel_mode, other_rel = p.side_b ? p.a_rel_mode : 0;
+    const RowSource& self_src = p.side_b ? p.ent_b : p.ent_a;
+    const RowSource& other_src = p.side_b ? p.ent_a : p.ent_b;
+    const float* coef = p.coef + (size_t)d * B * T;
+    const float* cdiv = p.coef_div ? p.coef_div + (size_t)d * B * T : nullptr;
+
+    // this thread's 4x4 block of `self` (needed by L1 in the loop, by L2 at the end)
+    float sv[4][4];
+    const int kcol = kt0 + tx * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i0 + ty * 4 + i;
+        float4 v = make_float4(0, 0, 0, 0);
+        if (DIST != DIST_DOT && r < n_self && kcol < Dp) {
+            v = load4(row_ptr(self_src, self_c0 + r), kcol, self_src);
+            if (self_rel) v = combine_rel(v, p.rel + (size_t)p.crel[d * B + r] * Dp, kcol, self_rel);
+        }
+        sv[i][0] = v.x; sv[i][1] = v.y; sv[i][2] = v.z; sv[i][3] = v.w;
+    }
+    float acc[4][4], csum[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        csum[i] = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[i][k] = 0.f;
+    }
+
+    for (int j0 = 0; j0 < n_other; j0 += BJ) {
+        // coefficient tile -> Cs[j][i]
+        if (!p.side_b) {
+            // c[i][j] = coef[i0+i][j0+j], contiguous over j: transposing store
+            const int li = tid >> 3, j4 = (tid & 7) * 4;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int i = li + 32 * h, gi = i0 + i, gj = j0 + j4;
+                float v[4] = {0.f, 0.f, 0.f, 0.f};
+                if (gi < B) {
+                    const float* src = coef + (size_t)gi * T + gj;
+                    if (cdiv) {
+                        const float* dv = cdiv + (size_t)gi * T + gj;
+#pragma unroll
+                        for (int x = 0; x < 4; ++x)
+                            if (gj + x < T) v[x] = dv[x] != 0.f ? src[x] / dv[x] : 0.f;
+                    } else if (gj + 3 < T && (T & 3) == 0) {
+                        const float4 t = *reinterpret_cast<const float4*>(src);
+                        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+                    } else {
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) if (gj + x < T) v[x] = src[x];
+                    }
+                }
+#pragma unroll
+                for (int x = 0; x < 4; ++x) Cs[j4 + x][i] = v[x];
+            }
+        } else {
+            // c[i][j] = coef[j0+j][i0+i], contiguous over i: direct store
+            const int lj = tid >> 4, i4 = (tid & 15) * 4;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int j = lj + 16 * h, gj = j0 + j, gi = i0 + i4;
+                float4 t = make_float4(0, 0, 0, 0);
+                if (gj < B) {
+                    const float* src = coef + (size_t)gj * T + gi;
+                    if (cdiv) {
+                        const float* dv = cdiv + (size_t)gj * T + gi;
+                        if (gi + 0 < T) t.x = dv[0] != 0.f ? src[0] / dv[0] : 0.f;
+                        if (gi + 1 < T) t.y = dv[1] != 0.f ? src[1] / dv[1] : 0.f;
+                        if (gi + 2 < T) t.z = dv[2] != 0.f ? src[2] / dv[2] : 0.f;
+                        if (gi + 3 < T) t.w = dv[3] != 0.f ? src[3] / dv[3] : 0.f;
+                    } else if (gi + 3 < T && (T & 3) == 0) {
+                        t = *reinterpret_cast<const float4*>(src);
+                    } else {
+                        if (gi + 0 < T) t.x = src[0];
+                        if (gi + 1 < T) t.y = src[1];
+                        if (gi + 2 < T) t.z = src[2];
+                        if (gi + 3 < T) t.w = src[3];
+                    }
+                }
+                *reinterpret_cast<float4*>(&Cs[j][i4]) = t;
+            }
+        }
+        // other rows -> Os[j][k]
+        {
+            const int lj = tid >> 4, kk4 = (tid & 15) * 4;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int j = lj + 16 * h, gj = j0 + j, gk = kt0 + kk4;
+                float4 t = make_float4(0, 0, 0, 0);
+                if (gj < n_other && gk < Dp) {
+                    t = load4(row_ptr(other_src, other_c0 + gj), gk, other_src);
+                    if (other_rel)
+                        t = combine_rel(t, p.rel + (size_t)p.crel[d * B + gj] * Dp, gk, other_rel);
+                }
+                *reinterpret_cast<float4*>(&Os[j][kk4]) = t;
+            }
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int jj = 0; jj < BJ; ++jj) {
+            const float4 c4 = *reinterpret_cast<const float4*>(&Cs[jj][ty * 4]);
+            const float4 o4 = *reinterpret_cast<const float4*>(&Os[jj][tx * 4]);
+            const float cv[4] = {c4.x, c4.y, c4.z, c4.w};
+            const float ov[4] = {o4.x, o4.y, o4.z, o4.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (DIST == DIST_L2) csum[i] += cv[i];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (DIST == DIST_L1) {
+                        const float t = sv[i][k] - ov[k];
+                        const float sg = (t > 0.f ? 1.f : 0.f) - (t < 0.f ? 1.f : 0.f);
+                        acc[i][k] = fmaf(cv[i], sg, acc[i][k]);
+                    } else {
+                        acc[i][k] = fmaf(cv[i], ov[k], acc[i][k]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i0 + ty * 4 + i;
+        if (r >= n_self || kcol >= Dp) continue;
+        float o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (DIST == DIST_L2) o[k] = sv[i][k] * csum[i] - acc[i][k];
+            else o[k] = acc[i][k];
+        }
+        float* dst = p.grad + (size_t)(p.grad_c0 + d * n_self + r) * Dp + kcol;
+        if (p.vec_out) {
+            *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) if (kcol + k < Dp) dst[k] = o[k];
+        }
+    }
+}
+
+static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
+    const int n_self = p.side_b ? p.T : p.B;
+    dim3 grid((p.Dp + kScoreTile - 1) / kScoreTile, (n_self + kScoreTile - 1) / kScoreTile, p.S);
+    if (dist_fn == DIST_L1)
+        hipLaunchKernelGGL(k_score_bwd<DIST_L1>, grid, dim3(256), 0, stream, p);
+    else if (dist_fn == DIST_L2)
+        hipLaunchKernelGGL(k_score_bwd<DIST_L2>, grid, dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL(k_score_bwd<DIST_DOT>, grid, dim3(256), 0, stream, p);
+}
+
+void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
+                      const uint32_t* crel, const float* coef, float* grad, hipStream_t stream) {
+    BwdParams p;
+    p.ent_a = ent; p.ent_b = ent; p.rel = rel; p.crel = crel; p.coef = coef; p.grad = grad;
+    p.coef_div = nullptr;
+    p.S = sh.S; p.B = sh.B; p.T = sh.T; p.Dp = sh.Dp; p.vec_out = 1;
+    p.a_rel_mode = sh.score_fn == SCORE_DISTMULT ? 2 : 1;
+    p.a_c0 = 0; p.b_c0 = sh.S * sh.B;
+    const int dist_fn = sh.score_fn == SCORE_DISTMULT ? DIST_DOT : sh.dist_fn;
+    p.side_b = 0; p.grad_c0 = p.a_c0;
+    launch_bwd(p, dist_fn, stream);
+    p.side_b = 1; p.grad_c0 = p.b_c0;
+    launch_bwd(p, dist_fn, stream);
+}
+
+// --------------------------------------------------------------------------
+// segmented reduction + Adam
+
+__global__ __launch_bounds__(256) void k_reduce_chunks(ReduceArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int q = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (q >= (int)a.counts[1]) return;
+    const uint32_t pos = a.chunk_pos[q], len = a.chunk_len[q];
+    const int Dp = a.Dp;
+    if (Dp & 3) {  // unaligned rows (standalone scatter-add on arbitrary widths)
+        for (int k = lane; k < Dp; k += 64) {
+            float acc = 0.f;
+            for (uint32_t j = 0; j < len; ++j)
+                acc += a.grad[(size_t)a.sorted_item[pos + j] * Dp + k];
+            a.partial[(size_t)q * Dp + k] = acc;
+        }
+        return;
+    }
+    for (int k = lane * 4; k < Dp; k += 256) {
+        float4 acc = make_float4(0, 0, 0, 0);
+        for (uint32_t j = 0; j < len; ++j) {
+            const uint32_t c = a.sorted_item[pos + j];
+            float4 g = *reinterpret_cast<const float4*>(a.grad + (size_t)c * Dp + k);
+            if (a.transform == 1) {
+                if (c < (uint32_t)a.n_head)
+                    g = f4mul(g, *reinterpret_cast<const float4*>(a.rel + (size_t)a.crel[c] * Dp + k));
+            } else if (a.transform == 2) {
+                g = f4mul(g, load4(row_ptr(a.ent, c), k, a.ent));
+            }
+            acc = f4add(acc, g);
+        }
+        *reinterpret_cast<float4*>(a.partial + (size_t)q * Dp + k) = acc;
+    }
+}
+
+void launch_reduce_chunks(const ReduceArgs& a, hipStream_t stream) {
+    hipLaunchKernelGGL(k_reduce_chunks, dim3((a.max_chunks + 3) / 4), dim3(256), 0, stream, a);
+}
+
+// fr::nn::adam (src/fructose/frnn.cpp:74-89) on one float4
+DEVINL void adam4(float4& p, float4& m, float4& v, float4 g, const AdamArgs& a, float alpha) {
+    float* pp = &p.x; float* mm = &m.x; float* vv = &v.x; const float* gg = &g.x;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        float vi = vv[x];
+        if (a.v_is_sqrt) vi = vi * vi;
+        const float mi = a.beta_m * mm[x] + a.one_minus_beta_m * gg[x];
+        vi = a.beta_v * vi + a.one_minus_beta_v * gg[x] * gg[x];
+        pp[x] = pp[x] - alpha * (mi / (sqrtf(vi) + a.epsilon) + a.weight_decay * pp[x]);
+        mm[x] = mi;
+        vv[x] = a.v_is_sqrt ? sqrtf(vi) : vi;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (u >= (int)a.counts[0]) return;
+    const uint32_t key = a.uniq_key[u];
+    const float alpha = a.alpha[a.rows_per_alpha ? key / a.rows_per_alpha : 0u];
+    const int Dp = a.Dp;
+    uint32_t q0 = 0, q1 = 0;
+    if (a.partial) { q0 = a.chunk_off[u]; q1 = a.chunk_off[u + 1]; }
+    char* prow = a.p_base + (int64_t)key * a.pitch;
+    char* mrow = a.m_base + (int64_t)key * a.pitch;
+    char* vrow = a.v_base + (int64_t)key * a.pitch;
+    for (int k = lane * 4; k < Dp; k += 256) {
+        float4 g = make_float4(0, 0, 0, 0);
+        if (a.grad_direct) {
+            g = *reinterpret_cast<const float4*>(a.grad_direct + (size_t)u * Dp + k);
+        } else {
+            for (uint32_t q = q0; q < q1; ++q)
+                g = f4add(g, *reinterpret_cast<const float4*>(a.partial + (size_t)q * Dp + k));
+        }
+        if (a.grad_out) *reinterpret_cast<float4*>(a.grad_out + (size_t)u * Dp + k) = g;
+        float4 p = load4(prow, k, a.p_etype);
+        float4 m = *reinterpret_cast<const float4*>(mrow + (size_t)k * 4);
+        float4 v = *reinterpret_cast<const float4*>(vrow + (size_t)k * 4);
+        adam4(p, m, v, g, a, alpha);
+        store4(prow, k, a.p_etype, p);
+        *reinterpret_cast<float4*>(mrow + (size_t)k * 4) = m;
+        *reinterpret_cast<float4*>(vrow + (size_t)k * 4) = v;
+    }
+}
+
+void launch_adam_rows(const AdamArgs& a, hipStream_t stream) {
+    hipLaunchKernelGGL(k_adam_rows, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a);
+}
+
+__global__ __launch_bounds__(64) void k_loss_finalize(const float* __restrict__ loss_part, int n_step,
+                                                      int S, int n_part, float scale,
+                                                      float* __restrict__ loss) {
+    const int s = blockIdx.x, lane = threadIdx.x;
+    float acc = 0.f;
+    for (int i = 0; i < n_step; ++i) {
+        const float* p = loss_part + ((size_t)i * S + s) * n_part;
+        float part = 0.f;
+        for (int t = lane; t < n_part; t += 64) part += p[t];
+        acc += wave_sum(part);
+    }
+    if (lane == 0) loss[s] = acc * scale;
+}
+
+void launch_loss_finalize(const float* loss_part, int n_step, int S, int n_part, float scale,
+                          float* loss, hipStream_t stream) {
+    hipLaunchKernelGGL(k_loss_finalize, dim3(S), dim3(64), 0, stream, loss_part, n_step, S, n_part,
+                       scale, loss);
+}
+
+// --------------------------------------------------------------------------
+// feature projection (src/poplar_kge.cpp:451-462): one wave per distinct row
+
+__global__ __launch_bounds__(256) void k_hidden_fwd(FeatureArgs a, float* __restrict__ hidden) {
+    const int lane = threadIdx.x & 63;
+    const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (u >= (int)a.counts[0]) return;
+    const uint32_t key = a.uniq_key[u];
+    const char* erow = a.emb_base + (int64_t)key * a.pitch;
+    const char* frow = a.feat_base + (int64_t)key * a.pitch;
+    for (int k = lane * 4; k < a.Dp; k += 256) {
+        float4 h = load4(erow, k, a.emb_etype);
+        for (int f = 0; f < a.Fp; f += 4) {
+            const float4 x = load4(frow, f, a.feat_etype);
+            const float xv[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float4 w = *reinterpret_cast<const float4*>(a.proj + (size_t)(f + i) * a.Dp + k);
+                h.x = fmaf(xv[i], w.x, h.x); h.y = fmaf(xv[i], w.y, h.y);
+                h.z = fmaf(xv[i], w.z, h.z); h.w = fmaf(xv[i], w.w, h.w);
+            }
+        }
+        *reinterpret_cast<float4*>(hidden + (size_t)u * a.Dp + k) = h;
+    }
+}
+
+void launch_hidden_fwd(const FeatureArgs& a, float* hidden, hipStream_t stream) {
+    hipLaunchKernelGGL(k_hidden_fwd, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, hidden);
+}
+
+// gproj[f, k] = sum_u feature[u, f] * grad_rows[u, k]; block = 4 feature rows x 64 float4 columns
+__global__ __launch_bounds__(256) void k_proj_grad(FeatureArgs a, const float* __restrict__ grad_rows,
+                                                   float* __restrict__ gproj) {
+    const int lane = threadIdx.x & 63;
+    const int f = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int k = (blockIdx.x * 64 + lane) * 4;
+    if (f >= a.Fp || k >= a.Dp) return;
+    const int U = a.counts[0];
+    float4 acc = make_float4(0, 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+        const char* frow = a.feat_base + (int64_t)a.uniq_key[u] * a.pitch;
+        float x;
+        if (a.feat_etype == ET_F32) x = reinterpret_cast<const float*>(frow)[f];
+        else if (a.feat_etype == ET_F16) x = __half2float(reinterpret_cast<const __half*>(frow)[f]);
+        else x = bf16_to_f32(reinterpret_cast<const uint16_t*>(frow)[f]);
+        const float4 g = *reinterpret_cast<const float4*>(grad_rows + (size_t)u * a.Dp + k);
+        acc.x = fmaf(x, g.x, acc.x); acc.y = fmaf(x, g.y, acc.y);
+        acc.z = fmaf(x, g.z, acc.z); acc.w = fmaf(x, g.w, acc.w);
+    }
+    *reinterpret_cast<float4*>(gproj + (size_t)f * a.Dp + k) = acc;
+}
+
+void launch_proj_grad(const FeatureArgs& a, const float* grad_rows, float* gproj,
+                      hipStream_t stream) {
+    dim3 grid((a.Dp / 4 + 63) / 64, (a.Fp + 3) / 4);
+    hipLaunchKernelGGL(k_proj_grad, grid, dim3(256), 0, stream, a, grad_rows, gproj);
+}
+
+// --------------------------------------------------------------------------
+// table access
+
+// One wave per row, 16 bytes per lane per iteration when the row allows it.
+__global__ __launch_bounds__(256) void k_rows_copy(const char* __restrict__ src,
+                                                   char* __restrict__ dst,
+                                                   const uint32_t* __restrict__ idx, int64_t n,
+                                                   int64_t row_bytes, int scatter, int vec16) {
+    const int lane = threadIdx.x & 63;
+    const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= n) return;
+    const int64_t r = idx[i];
+    const char* s = scatter ? src + i * row_bytes : src + r * row_bytes;
+    char* d = scatter ? dst + r * row_bytes : dst + i * row_bytes;
+    if (vec16) {
+        for (int64_t b = (int64_t)lane * 16; b < row_bytes; b += 64 * 16)
+            *reinterpret_cast<uint4*>(d + b) = *reinterpret_cast<const uint4*>(s + b);
+    } else {
+        for (int64_t b = (int64_t)lane * 4; b < row_bytes; b += 64 * 4)
+            *reinterpret_cast<uint32_t*>(d + b) = *reinterpret_cast<const uint32_t*>(s + b);
+    }
+}
+
+void launch_rows_gather(const void* buf, const uint32_t* idx, void* out, int64_t n,
+                        int64_t row_bytes, hipStream_t stream) {
+    if (n == 0) return;
+    const int vec16 = (row_bytes % 16 == 0) && ((uintptr_t)buf % 16 == 0) && ((uintptr_t)out % 16 == 0);
+    hipLaunchKernelGGL(k_rows_copy, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream,
+                       (const char*)buf, (char*)out, idx, n, row_bytes, 0, vec16);
+}
+
+void launch_rows_scatter(void* buf, const uint32_t* idx, const void* data, int64_t n,
+                         int64_t row_bytes, hipStream_t stream) {
+    if (n == 0) return;
+    const int vec16 = (row_bytes % 16 == 0) && ((uintptr_t)buf % 16 == 0) && ((uintptr_t)data % 16 == 0);
+    hipLaunchKernelGGL(k_rows_copy, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream,
+                       (const char*)data, (char*)buf, idx, n, row_bytes, 1, vec16);
+}
+
+DEVINL void store1(char* sec, int k, int etype, float v) {
+    if (etype == ET_F32) reinterpret_cast<float*>(sec)[k] = v;
+    else if (etype == ET_BF16) reinterpret_cast<uint16_t*>(sec)[k] = f32_to_bf16(v);
+    else reinterpret_cast<__half*>(sec)[k] = __float2half_rn(v);
+}
+
+// logical column c of [emb D | m D | sqrt v D | feature F] -> (section byte offset, index, type)
+DEVINL void locate(const RowLayout& L, int c, int64_t& off, int& k, int& et) {
+    if (c < L.D) { off = 0; k = c; et = L.emb_etype; }
+    else if (c < 2 * L.D) { off = L.off_m; k = c - L.D; et = L.mom_etype; }
+    else if (c < 3 * L.D) { off = L.off_s; k = c - 2 * L.D; et = L.mom_etype; }
+    else { off = L.off_f; k = c - 3 * L.D; et = L.feat_etype; }
+}
+
+__global__ __launch_bounds__(256) void k_rows_to_logical(RowLayout L, const char* __restrict__ base,
+                                                         const uint64_t* __restrict__ rows, int64_t n,
+                                                         float* __restrict__ out) {
+    const int W = 3 * L.D + L.F;
+    const int64_t i = blockIdx.x;
+    if (i >= n) return;
+    const char* row = base + (int64_t)rows[i] * L.pitch;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        int64_t off; int k, et;
+        locate(L, c, off, k, et);
+        out[i * W + c] = load1(row + off, k, et);
+    }
+}
+
+__global__ __launch_bounds__(256) void k_rows_from_logical(RowLayout L, char* __restrict__ base,
+                                                           const uint64_t* __restrict__ rows,
+                                                           int64_t n, const float* __restrict__ in) {
+    const int W = 3 * L.D + L.F;
+    const int64_t i = blockIdx.x;
+    if (i >= n) return;
+    char* row = base + (int64_t)rows[i] * L.pitch;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        int64_t off; int k, et;
+        locate(L, c, off, k, et);
+        store1(row + off, k, et, in[i * W + c]);
+    }
+}
+
+void launch_rows_to_logical(const RowLayout& L, const char* base, const uint64_t* rows, int64_t n,
+                            float* out, hipStream_t stream) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(k_rows_to_logical, dim3((unsigned)n), dim3(256), 0, stream, L, base, rows, n, out);
+}
+void launch_rows_from_logical(const RowLayout& L, char* base, const uint64_t* rows, int64_t n,
+                              const float* in, hipStream_t stream) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(k_rows_from_logical, dim3((unsigned)n), dim3(256), 0, stream, L, base, rows, n, in);
+}
+
+// counter-based normal generator: two rounds of a 64-bit mix, then Box-Muller
+DEVINL uint64_t mix64(uint64_t x) {
+    x ^= x >> 30; x *= 0xbf58476d1ce4e5b9ull;
+    x ^= x >> 27; x *= 0x94d049bb133111ebull;
+    x ^= x >> 31;
+    return x;
+}
+DEVINL float normal_at(uint32_t seed, uint64_t row, uint32_t col) {
+    const uint64_t h = mix64(mix64(((uint64_t)seed << 32) ^ row * 0x9e3779b97f4a7c15ull) + col);
+    const float u1 = ((uint32_t)(h >> 40) + 1u) * (1.0f / 16777217.0f);  // (0, 1)
+    const float u2 = (uint32_t)(h & 0xffffffu) * (1.0f / 16777216.0f);   // [0, 1)
+    return sqrtf(-2.f * logf(u1)) * cospif(2.f * u2);
+}
+
+// Model::writeEntity (src/poplar_kge.cpp:864-871): emb ~ N(0, sigma), zero
+// moments, host features; padding columns are zero.
+__global__ __launch_bounds__(256) void k_init_rows(RowLayout L, char* __restrict__ base,
+                                                   const uint64_t* __restrict__ rows, int64_t n,
+                                                   const float* __restrict__ features, float sigma,
+                                                   uint32_t seed) {
+    const int64_t i = blockIdx.x;
+    if (i >= n) return;
+    const uint64_t r = rows[i];
+    char* row = base + (int64_t)r * L.pitch;
+    for (int k = threadIdx.x; k < L.Dp; k += 256) {
+        store1(row, k, L.emb_etype, k < L.D ? sigma * normal_at(seed, r, k) : 0.f);
+        store1(row + L.off_m, k, L.mom_etype, 0.f);
+        store1(row + L.off_s, k, L.mom_etype, 0.f);
+    }
+    for (int f = threadIdx.x; f < L.Fp; f += 256)
+        store1(row + L.off_f, f, L.feat_etype, f < L.F ? features[i * L.F + f] : 0.f);
+}
+
+void launch_init_rows(const RowLayout& L, char* base, const uint64_t* rows, int64_t n,
+                      const float* features, float sigma, uint32_t seed, hipStream_t stream) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(k_init_rows, dim3((unsigned)n), dim3(256), 0, stream, L, base, rows, n,
+                       features, sigma, seed);
+}
+
+// --------------------------------------------------------------------------
+// standalone ops
+
+static RowSource plain_rows(const float* ptr, int D) {
+    RowSource r;
+    r.base = (const char*)ptr; r.pitch = (int64_t)D * 4; r.etype = ET_F32; r.index = nullptr;
+    r.count = D; r.vec = (D % 4 == 0) && ((uintptr_t)ptr % 16 == 0);
+    return r;
+}
+
+void launch_distance(int dist_fn, const float* a, const float* b, float* out, int M, int N, int D,
+                     hipStream_t stream) {
+    FwdParams p;
+    p.sh.S = 1; p.sh.B = M; p.sh.T = N; p.sh.Dp = D;
+    p.sh.score_fn = SCORE_TRANSE; p.sh.dist_fn = dist_fn; p.sh.loss_fn = LOSS_LOGSIGMOID;
+    p.sh.gamma = 0.f; p.sh.loss_scale = 1.f; p.sh.softmax_correction = 0.f;
+    p.sh.negative_adversarial_scale = 0.f;
+    p.ent_a = plain_rows(a, D); p.ent_b = plain_rows(b, D);
+    p.rel = nullptr; p.crel = nullptr; p.clabel = nullptr;
+    p.coef = out; p.dist = nullptr; p.loss_part = nullptr;
+    p.a_rel_mode = 0; p.out_mode = 2;
+    p.a_c0 = 0; p.b_c0 = 0;
+    launch_fwd(p, stream);
+}
+
+// g [M, N]; dist [M, N] (L2 only, else null): gradient of the first operand
+void launch_distance_grad(int dist_fn, const float* a, const float* b, const float* dist,
+                          const float* g, float* grad, int M, int N, int D, hipStream_t stream) {
+    BwdParams p;
+    p.ent_a = plain_rows(a, D); p.ent_b = plain_rows(b, D);
+    p.rel = nullptr; p.crel = nullptr;
+    p.coef = g;
+    p.coef_div = dist_fn == DIST_L2 ? dist : nullptr;
+    p.grad = grad;
+    p.S = 1; p.B = M; p.T = N; p.Dp = D;
+    p.side_b = 0; p.a_rel_mode = 0;
+    p.a_c0 = 0; p.b_c0 = 0; p.grad_c0 = 0;
+    p.vec_out = (D % 4 == 0) && ((uintptr_t)grad % 16 == 0);
+    launch_bwd(p, dist_fn, stream);
+}
+
+__global__ __launch_bounds__(256) void k_adam_flat(float* __restrict__ p, float* __restrict__ m,
+                                                   float* __restrict__ v, const float* __restrict__ g,
+                                                   int64_t n, AdamArgs a, float alpha) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float vi = v[i];
+    if (a.v_is_sqrt) vi = vi * vi;
+    const float mi = a.beta_m * m[i] + a.one_minus_beta_m * g[i];
+    vi = a.beta_v * vi + a.one_minus_beta_v * g[i] * g[i];
+    p[i] = p[i] - alpha * (mi / (sqrtf(vi) + a.epsilon) + a.weight_decay * p[i]);
+    m[i] = mi;
+    v[i] = a.v_is_sqrt ? sqrtf(vi) : vi;
+}
+
+void launch_adam_flat(float* p, float* m, float* v, const float* g, int64_t n, float alpha,
+                      float beta_m, float beta_v, float epsilon, float weight_decay, int v_is_sqrt,
+                      hipStream_t stream) {
+    if (n == 0) return;
+    AdamArgs a = {};
+    a.beta_m = beta_m; a.beta_v = beta_v;
+    a.one_minus_beta_m = 1.f - beta_m; a.one_minus_beta_v = 1.f - beta_v;
+    a.epsilon = epsilon; a.weight_decay = weight_decay; a.v_is_sqrt = v_is_sqrt;
+    hipLaunchKernelGGL(k_adam_flat, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, m, v,
+                       g, n, a, alpha);
+}
+
+__global__ __launch_bounds__(256) void k_fill_u32(uint32_t* p, uint32_t value, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = value;
+}
+void launch_fill_u32(uint32_t* p, uint32_t value, int64_t n, hipStream_t stream) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, value, n);
+}
+
+// items for a plain scatter-add: n real items keyed by idx, then one
+// zero-gradient item per table row so that every row forms a segment
+__global__ __launch_bounds__(256) void k_iota_keys(const uint32_t* __restrict__ idx,
+                                                   uint32_t* __restrict__ keys,
+                                                   uint32_t* __restrict__ vals, int64_t n,
+                                                   int64_t rows) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n + rows) return;
+    keys[i] = i < n ? idx[i] : (uint32_t)(i - n);
+    vals[i] = (uint32_t)i;
+}
+void launch_iota_keys(const uint32_t* idx, uint32_t* keys, uint32_t* vals, int64_t n, int64_t rows,
+                      hipStream_t stream) {
+    hipLaunchKernelGGL(k_iota_keys, dim3((unsigned)((n + rows + 255) / 256)), dim3(256), 0, stream,
+                       idx, keys, vals, n, rows);
+}
+
+// out[r, :] = sum of the partial rows of table row r's chunks (second level
+// of the segmented reduction without an optimiser step)
+__global__ __launch_bounds__(256) void k_sum_partials_rows(const uint32_t* __restrict__ chunk_off,
+                                                           const float* __restrict__ partial,
+                                                           int64_t rows, int64_t cols,
+                                                           float* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const uint32_t q0 = chunk_off[r], q1 = chunk_off[r + 1];
+    if (cols & 3) {
+        for (int64_t k = lane; k < cols; k += 64) {
+            float g = 0.f;
+            for (uint32_t q = q0; q < q1; ++q) g += partial[(size_t)q * cols + k];
+            out[r * cols + k] = g;
+        }
+        return;
+    }
+    for (int64_t k = lane * 4; k < cols; k += 256) {
+        float4 g = make_float4(0, 0, 0, 0);
+        for (uint32_t q = q0; q < q1; ++q)
+            g = f4add(g, *reinterpret_cast<const float4*>(partial + (size_t)q * cols + k));
+        *reinterpret_cast<float4*>(out + r * cols + k) = g;
+    }
+}
+void launch_sum_partials_rows(const uint32_t* chunk_off, const float* partial, int64_t rows,
+                              int64_t cols, float* out, hipStream_t stream) {
+    hipLaunchKernelGGL(k_sum_partials_rows, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
+                       chunk_off, partial, rows, cols, out);
+}
+
+}  // namespace kge
