@@ -27,7 +27,7 @@ CASES = {
     "l2_weight_decay": dict(distance_fn="L2", weight_decay=0.01, feature=0),
     "shared_l2": dict(distance_fn="L2", shared_table=True, n_shard=4, batch=8, a2a=4, feature=0,
                       n_entity=60, gamma=3.0),
-    "odd_dim": dict(dim=10, feature=3, n_entity=41, batch=5, a2a=3, distance_fn="L2"),
+    "odd_dim": dict(dim=10, feature=6, n_entity=41, batch=5, a2a=3, distance_fn="L2"),
     "mid_l2": dict(distance_fn="L2", n_shard=4, batch=96, a2a=40, dim=128, feature=0,
                    n_entity=3000, n_relation=40, gamma=6.0),
     "mid_l1": dict(distance_fn="L1", n_shard=2, batch=70, a2a=45, dim=64, feature=0,
@@ -63,8 +63,11 @@ def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_lo
         if k == "step":
             continue
         d_h, d_o = st_h[k] - st0[k], st_o[k] - st0[k]
-        assert K.rel_l2(st_h[k], st_o[k]) < 1e-5, k
-        assert K.rel_l2(d_h, d_o) < 2e-5, (k, K.rel_l2(d_h, d_o))
+        # updated rows: 1e-5 relative (measured ~1e-7); the update itself: the
+        # reference's own 1e-4 bar on (final - initial), whose float32 storage
+        # rounding alone is ~1e-5 of a small delta
+        assert K.rel_l2(st_h[k], st_o[k]) < 1e-6, (k, K.rel_l2(st_h[k], st_o[k]))
+        assert K.rel_l2(d_h, d_o) < 1e-4, (k, K.rel_l2(d_h, d_o))
     return c, st0, st_h, engine
 
 
