@@ -1,0 +1,318 @@
+#!/usr/bin/env python3
+"""Throughput of the per-shard KGE training step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+
+One "step" is one training step over one batch: gather -> BESS scoring ->
+loss forward/backward -> deterministic scatter-add -> sparse Adam write-back.
+The index arrays of all W + K steps (fresh ids every step) are resident in HBM
+before the timed region, which runs exactly K steps through the engine's
+``train_step_loop`` (device plan phase included) and ends with the loss copied
+back and the stream synchronised.  Prints ONE JSON line.
+
+Extra objects in that line:
+  roofline      the kernel with the largest share of the step time: algorithmic
+                bytes or flops per launch over its mean launch duration, measured
+                with HIP events on the engine's stream in a second (untimed) pass
+  kernels       the same figures for every kernel of the step
+  cpu_baseline  the sequential float32 CPU oracle on the first steps of the same
+                workload, on this host's cores (1 thread)
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+for p in (ROOT, ROOT / "distributed-kge-poplar_amd", ROOT / "tests"):
+    sys.path.insert(0, os.fspath(p))
+
+# Synthetic workloads (ids Zipf s=1.1 over 1..N-1, relations uniform, one shared
+# table addressed by K blocks = K virtual shards).  c2 is the configuration the
+# headline metric is quoted on.
+WORKLOADS = {
+    "c1": dict(desc="TransE-L2 D=64 fp32, 10k entities, 1 block x (256 positives, 64 shared tails)",
+               n_entity=10_000, n_relation=50, dim=64, blocks=1, batch=256, tails=64,
+               distance_fn="L2", uniform=True),
+    "c2": dict(desc="TransE-L2 D=256 fp32, 1M entities, 32 blocks x (256 positives, 256 shared tails)",
+               n_entity=1_000_000, n_relation=1000, dim=256, blocks=32, batch=256, tails=256,
+               distance_fn="L2"),
+    "c3": dict(desc="TransE-L1 D=256 fp32, 22.8M entities, 64 blocks x (256 positives, 512 shared tails)",
+               n_entity=22_800_000, n_relation=1387, dim=256, blocks=64, batch=256, tails=512,
+               distance_fn="L1"),
+    "c3l2": dict(desc="TransE-L2 D=256 fp32, 22.8M entities, 64 blocks x (256 positives, 512 shared tails)",
+                 n_entity=22_800_000, n_relation=1387, dim=256, blocks=64, batch=256, tails=512,
+                 distance_fn="L2"),
+    "c5": dict(desc="TransE-L2 D=256 bf16 embedding + fp32 moments, 91.2M entities, "
+                    "32 blocks x (512 positives, 512 shared tails)",
+               n_entity=91_200_000, n_relation=1387, dim=256, blocks=32, batch=512, tails=512,
+               distance_fn="L2", embedding_dtype="bfloat16"),
+}
+
+PEAK_HBM_GBPS = 8000.0
+PEAK_FP32_TFLOPS = 157.3
+
+
+def make_settings(w, n_step, kge):
+    s = kge.Settings.create_demo()
+    s.seed = 20240611
+    m, d, t, e = s.model, s.data, s.training, s.execution
+    m.score_fn, m.distance_fn = "TransE", w["distance_fn"]
+    m.n_shard, m.n_entity, m.n_relation_type = w["blocks"], w["n_entity"], w["n_relation"]
+    m.embedding_size, m.entity_feature_size, m.gamma = w["dim"], 0, 10.0
+    m.init_scale = float(np.sqrt(w["dim"]))  # embeddings ~ N(0, 1/sqrt(D)): sigma = init_scale / D
+    d.batch_size, d.a2a_size = w["batch"], w["tails"] // w["blocks"]
+    t.learning_rate, t.loss = 1e-3, kge.LogSigmoidLoss()
+    e.device, e.dtype, e.shared_table = "hip", "float32", True
+    e.embedding_dtype = w.get("embedding_dtype")
+    e.train_steps_per_program_run = n_step
+    e.rw_batch_size = 8192
+    return s.prepare()
+
+
+def make_batch(w, n_step, kge, K):
+    """Raw ids with identity slot maps: every block lists its heads then the
+    tails it contributes; the device does all the de-duplication."""
+    c = dict(n_shard=w["blocks"], n_entity=w["n_entity"], batch=w["batch"],
+             a2a=w["tails"] // w["blocks"], n_relation=w["n_relation"])
+    rng = np.random.Generator(np.random.PCG64(20240611 + 1))
+    return kge.Batch(**K.raw_batch(c, n_step, rng, zipf=not w.get("uniform", False)))
+
+
+def init_tables(engine, settings):
+    """write_entity over the whole table (random-normal embeddings drawn on the
+    device).  The table is shared, so each of the n_shard index rows of one call
+    covers a different range of table rows."""
+    engine.initialise_variables()
+    m, e = settings.model, settings.execution
+    per_call = m.n_shard * e.rw_batch_size
+    feat = np.zeros(settings.entity_data_w_shape, np.float32)
+    for off in range(0, m.n_entity, per_call):
+        idx = np.arange(off, off + per_call, dtype=np.int64)
+        idx[idx >= m.n_entity] = 0
+        engine.engine.run("write_entity", dict(
+            write_indices=idx.astype(np.uint32).reshape(m.n_shard, -1), write_features=feat))
+    # row 0 last, so that the overflow of the final chunk does not decide its content
+    idx = np.zeros(per_call, np.uint32)
+    engine.engine.run("write_entity", dict(write_indices=idx.reshape(m.n_shard, -1), write_features=feat))
+    engine.uninitialized_entity_data[:] = False
+
+
+def read_rows(engine, settings, ids):
+    """Rows `ids` of the shared table as float32 [len(ids), 3D+F] (read_entity)."""
+    m, e = settings.model, settings.execution
+    per_call = m.n_shard * e.rw_batch_size
+    out = np.zeros((len(ids), settings.entity_data_r_size), np.float32)
+    for off in range(0, len(ids), per_call):
+        chunk = ids[off:off + per_call]
+        idx = np.zeros(per_call, np.uint32)
+        idx[:len(chunk)] = chunk
+        data = np.zeros(settings.entity_data_r_shape, np.float32)
+        engine.engine.run("read_entity", dict(read_indices=idx.reshape(m.n_shard, -1), read_data=data))
+        out[off:off + len(chunk)] = data.reshape(per_call, -1)[:len(chunk)]
+    return out
+
+
+def cpu_baseline(engine, settings, w, batch, n_check, n_cpu_steps):
+    """Times the sequential float32 oracle on the first `n_cpu_steps` steps of
+    the workload, starting from the device's own initial rows.  The first
+    `n_check` of them are run as a separate call so that their mean loss can be
+    compared with the GPU's.  Returns (json object, loss of the first call)."""
+    from oracle.kge_oracle import Oracle, make_cfg
+
+    m, d = settings.model, settings.data
+    sub = {k: np.ascontiguousarray(v[:, :n_cpu_steps]) for k, v in vars(batch).items()}
+    ids = np.unique(sub["remote"])
+    rows = read_rows(engine, settings, ids)
+    table = np.zeros((m.n_entity, settings.entity_data_r_size), np.float32)  # untouched pages stay virtual
+    table[ids] = rows
+    state = {"entity_data": table, "step": 0,
+             "relation_embedding": engine.read_variable("relation_embedding"),
+             "relation_embedding/adam_m": engine.read_variable("relation_embedding/adam_m"),
+             "relation_embedding/adam_v": engine.read_variable("relation_embedding/adam_v")}
+    cfg = make_cfg(n_shard=m.n_shard, n_entity=m.n_entity, n_relation=m.n_relation_type,
+                   dim=m.embedding_size, feature=0, batch=d.batch_size, a2a=d.a2a_size,
+                   score_fn=m.score_fn, distance_fn=m.distance_fn, loss_fn="logsigmoid",
+                   shared_table=True, gamma=m.gamma, loss_scale=settings.training.loss_scale,
+                   storage="bfloat16_embedding" if w.get("embedding_dtype") == "bfloat16" else "float32")
+    oracle = Oracle("f32")
+    lr = settings.training.learning_rate
+    t0 = time.perf_counter()
+    first = {k: np.ascontiguousarray(v[:, :n_check]) for k, v in sub.items()}
+    loss = oracle.train_step_loop(cfg, state, lr, first)
+    if n_cpu_steps > n_check:
+        rest = {k: np.ascontiguousarray(v[:, n_check:]) for k, v in sub.items()}
+        oracle.train_step_loop(cfg, state, lr, rest)
+    dt = time.perf_counter() - t0
+    triples = n_cpu_steps * m.n_shard * d.batch_size
+    return dict(value=triples / dt, unit="triples/s", cores=1, kind="port",
+                sample=f"{n_cpu_steps} step(s) of the same workload ({triples} triples) in {dt:.1f} s, "
+                       f"sequential float32 C oracle, 1 thread of {os.cpu_count()} host cpus"), loss
+
+
+def kernel_table(w, timing, n_steps, uniq_rows):
+    """Algorithmic bytes / flops per launch and achieved rates of every kernel."""
+    K_, B, T, D = w["blocks"], w["batch"], w["tails"], w["dim"]
+    R = K_ * (B + T)
+    U = float(np.mean(uniq_rows))
+    emb_bytes = 2 if w.get("embedding_dtype") == "bfloat16" else 4
+    row_state = D * emb_bytes + 2 * D * 4           # emb + m + sqrt v, read and written
+    pair_dims = K_ * B * T * D
+    work = {
+        # flops: 3 per pair-dim forward (sub, abs|mul, add); backward = 2x forward
+        "score_fwd": ("flops", 3.0 * pair_dims),
+        "score_bwd": ("flops", 6.0 * pair_dims),
+        # bytes: contributions in, one summed row out per distinct row
+        "reduce_entity": ("bytes", R * D * 4 + U * D * 4),
+        "adam_entity": ("bytes", U * 2 * row_state),
+        "reduce_relation": ("bytes", K_ * B * D * 4 + w["n_relation"] * D * 4),
+        "adam_relation": ("bytes", 2 * 3 * w["n_relation"] * D * 4),
+        "plan": ("bytes", 4.0 * (R + 2 * K_ * B) + 4 * U),
+    }
+    out = {}
+    for name, rec in timing["kernels"].items():
+        if rec["calls"] == 0 or name not in work:
+            continue
+        kind, amount = work[name]
+        ms = rec["ms"] / n_steps  # per step (plan: one launch group per call, shared by its steps)
+        entry = dict(ms_per_step=ms, launches_per_step=rec["calls"] / n_steps)
+        if kind == "bytes":
+            entry.update(bound="hbm", achieved=amount / (ms * 1e-3) / 1e9, peak=PEAK_HBM_GBPS, unit="GB/s")
+        else:
+            entry.update(bound="mfma", achieved=amount / (ms * 1e-3) / 1e12, peak=PEAK_FP32_TFLOPS,
+                         unit="TFLOP/s")
+        entry["frac"] = entry["achieved"] / entry["peak"]
+        entry["algorithmic_per_step"] = amount
+        out[name] = entry
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-steps", type=int, default=None,
+                    help="steps the CPU baseline times (default: sized for ~10-30 s)")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU holding one shard's whole table: --gpus must be 1 "
+                 "(the step has no collectives; nothing here uses a second GPU)")
+    if args.steps < 1 or args.warmup < 0:
+        sys.exit("--steps must be >= 1 and --warmup >= 0")
+
+    import torch  # device discovery only; all device memory is the engine's own
+
+    if not torch.cuda.is_available():
+        sys.exit("no HIP device visible")
+    import kge_cases as K
+    import poplar_kge as kge
+
+    w = WORKLOADS[args.workload]
+    n_total = args.warmup + args.steps
+    settings = make_settings(w, n_total, kge)
+    m, d = settings.model, settings.data
+    engine = kge.Engine(settings, np.full(m.n_shard, m.n_entity - 1))
+    init_tables(engine, settings)
+    batch = make_batch(w, n_total, kge, K)
+    engine.stage_batch(batch)
+
+    # CPU baseline on the first steps, from the same initial state the GPU starts from
+    # (about 15 s of CPU work: ~2e9 pair-dims per second for the whole step on one core)
+    pair_dims = m.n_shard * d.batch_size * settings.n_tail * m.embedding_size
+    n_cpu = args.cpu_steps or int(np.clip(round(15 * 2e9 / pair_dims), 1, n_total))
+    n_cpu = min(n_cpu, n_total)
+    n_check = max(1, min(n_cpu, args.warmup))
+    cpu, cpu_loss = (None, None) if args.no_cpu else cpu_baseline(engine, settings, w, batch, n_check, n_cpu)
+
+    # warm-up: W untimed steps; the first n_cpu of them double as the parity check
+    check = None
+    done = 0
+    if args.warmup > 0:
+        first = n_check if cpu is not None else args.warmup
+        loss, _ = engine.train_step_loop(None, step_begin=0, step_count=first)
+        done = first
+        if cpu is not None:
+            check = dict(gpu_loss=loss, cpu_loss=float(np.sum(cpu_loss)),
+                         rel_err=abs(loss - float(np.sum(cpu_loss))) / abs(float(np.sum(cpu_loss))))
+        if args.warmup > done:
+            engine.train_step_loop(None, step_begin=done, step_count=args.warmup - done)
+
+    # timed region: exactly K steps, device idle on both sides
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    loss, _ = engine.train_step_loop(None, step_begin=args.warmup, step_count=args.steps)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    timing = engine.timing()
+    uniq_rows = timing["unique_entity_rows"][args.warmup:args.warmup + args.steps].astype(np.float64)
+
+    # second pass over the same steps with an event pair around every kernel
+    engine.train_step_loop(None, step_begin=args.warmup, step_count=args.steps, profile_kernels=True)
+    prof = engine.timing()
+    kernels = kernel_table(w, prof, args.steps, uniq_rows)
+    step_kernels = {k: v for k, v in kernels.items() if k != "plan"}
+    dominant = max(step_kernels, key=lambda k: step_kernels[k]["ms_per_step"])
+    dom = kernels[dominant]
+    roofline = dict(kernel=dominant, bound=dom["bound"], achieved=dom["achieved"], peak=dom["peak"],
+                    unit=dom["unit"], frac=dom["frac"], traffic=None,
+                    launch_ms=dom["ms_per_step"] / dom["launches_per_step"])
+
+    # stand-alone row gather (fr::Buffer::read) over one step's distinct rows
+    ids = np.unique(batch.remote[:, args.warmup]).astype(np.uint32)
+    gms = np.zeros(1, np.float32)
+    engine.engine.run("gather_benchmark", dict(indices=ids, ms=gms, repeats=20))
+    row_bytes = (2 if w.get("embedding_dtype") == "bfloat16" else 4) * m.embedding_size + 8 * m.embedding_size
+    gather = dict(rows=int(ids.size), ms=float(gms[0]),
+                  achieved=2 * ids.size * row_bytes / (gms[0] * 1e-3) / 1e9, unit="GB/s (read + write)")
+
+    triples = args.steps * m.n_shard * d.batch_size
+    U = float(np.mean(uniq_rows))
+    R = m.n_shard * settings.n_remote
+    step_bytes = (U * 2 * row_bytes + 4 * (R + 2 * m.n_shard * d.batch_size) + 4 * U
+                  + 2 * 3 * m.n_relation_type * m.embedding_size * 4)
+    out = {
+        "metric": "train triples/sec (fwd+bwd+sparse Adam) at dim 256; achieved HBM GB/s",
+        "value": triples / dt,
+        "unit": "triples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 rows / f32 math" if w.get("embedding_dtype") == "bfloat16" else "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {w['desc']}; Zipf s=1.1 ids, logsigmoid loss, "
+                               f"Adam lr 1e-3, raw ids de-duplicated on the device",
+                   "positives_per_step": m.n_shard * d.batch_size, "row_refs_per_step": R,
+                   "unique_rows_per_step": U},
+        "step_hbm": {"algorithmic_bytes_per_step": step_bytes,
+                     "achieved": step_bytes / (dt / args.steps) / 1e9, "unit": "GB/s"},
+        "device_ms": {"plan_per_step": timing["plan_ms"] / args.steps,
+                      "kernels_per_step": timing["steps_ms"] / args.steps},
+        "loss": loss,
+        "roofline": roofline,
+        "kernels": kernels,
+        "row_gather": gather,
+        "cpu_baseline": cpu,
+        "check": check,
+    }
+    def plain(o):  # numpy scalars -> Python numbers
+        if isinstance(o, np.generic):
+            return o.item()
+        raise TypeError(type(o))
+
+    print(json.dumps(out, default=plain))
+
+
+if __name__ == "__main__":
+    main()

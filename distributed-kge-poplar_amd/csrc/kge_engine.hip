@@ -631,36 +631,49 @@ void collect_kernel_times(kge_engine& E) {
     E.kev_id.clear();
 }
 
-void run_plan(kge_engine& E) {
+// Index-only work for steps [s0, s0 + sn) of the resident batch: contribution
+// keys, the two sorts and the segment / chunk tables.
+void run_plan(kge_engine& E, int s0, int sn) {
     KernelTimer timer(E, K_PLAN);
     const hipStream_t st = E.stream;
+    const size_t R = E.R, SB = (size_t)E.S * E.B, N = 2 * R, NRI = E.n_rel_items;
     PlanShape ps;
     ps.n_step = E.n_step; ps.S = E.S; ps.B = E.B; ps.A = E.A; ps.NR = E.NR;
     ps.n_entity = E.n_entity; ps.shared_table = E.shared_table; ps.n_relation = E.n_rel;
+    ps.step0 = s0; ps.step_count = sn;
     launch_build_items(ps, E.d_remote.p, E.d_a2a.p, E.d_head.p, E.d_relation.p, E.d_tail.p, E.ckey.p,
                        E.crel.p, E.clabel.p, E.ek_a.p, E.ev_a.p, E.rk_a.p, E.rv_a.p, st);
     const int ebits = std::max(1, bit_length((uint64_t)E.n_rows - 1));
     const int rbits = std::max(1, bit_length((uint64_t)E.n_rel - 1));
-    const int N = 2 * E.R;
-    int which = launch_radix_sort(E.ek_a.p, E.ev_a.p, E.ek_b.p, E.ev_b.p, E.hist.p, N, E.n_step, ebits, st);
+    int which = launch_radix_sort(E.ek_a.p + s0 * N, E.ev_a.p + s0 * N, E.ek_b.p + s0 * N, E.ev_b.p + s0 * N,
+                                  E.hist.p, (int)N, sn, ebits, st);
     const uint32_t* ek = which ? E.ek_b.p : E.ek_a.p;
     E.e_sorted_vals = which ? E.ev_b.p : E.ev_a.p;
     SegPlan ep;
-    ep.uniq_key = E.e_uniq.p; ep.seg_start = E.e_seg.p; ep.chunk_off = E.e_coff.p;
-    ep.chunk_pos = E.e_cpos.p; ep.chunk_len = E.e_clen.p; ep.counts = E.e_counts.p;
-    ep.item_row = E.F ? E.e_item_row.p : nullptr;
     ep.u_stride = E.e_ustride; ep.c_stride = E.e_cstride;
-    launch_find_segments(ek, E.e_sorted_vals, N, E.R, E.chunk, E.n_step, ep, st);
+    ep.uniq_key = E.e_uniq.p + (size_t)s0 * ep.u_stride;
+    ep.seg_start = E.e_seg.p + (size_t)s0 * (ep.u_stride + 1);
+    ep.chunk_off = E.e_coff.p + (size_t)s0 * (ep.u_stride + 1);
+    ep.chunk_pos = E.e_cpos.p + (size_t)s0 * ep.c_stride;
+    ep.chunk_len = E.e_clen.p + (size_t)s0 * ep.c_stride;
+    ep.counts = E.e_counts.p + 2 * (size_t)s0;
+    ep.item_row = E.F ? E.e_item_row.p + s0 * R : nullptr;
+    launch_find_segments(ek + s0 * N, E.e_sorted_vals + s0 * N, (int)N, (int)R, E.chunk, sn, ep, st);
 
-    which = launch_radix_sort(E.rk_a.p, E.rv_a.p, E.rk_b.p, E.rv_b.p, E.hist.p, E.n_rel_items, E.n_step, rbits, st);
+    which = launch_radix_sort(E.rk_a.p + s0 * NRI, E.rv_a.p + s0 * NRI, E.rk_b.p + s0 * NRI,
+                              E.rv_b.p + s0 * NRI, E.hist.p, (int)NRI, sn, rbits, st);
     const uint32_t* rk = which ? E.rk_b.p : E.rk_a.p;
     E.r_sorted_vals = which ? E.rv_b.p : E.rv_a.p;
     SegPlan rp;
-    rp.uniq_key = E.r_uniq.p; rp.seg_start = E.r_seg.p; rp.chunk_off = E.r_coff.p;
-    rp.chunk_pos = E.r_cpos.p; rp.chunk_len = E.r_clen.p; rp.counts = E.r_counts.p;
-    rp.item_row = nullptr;
     rp.u_stride = E.r_ustride; rp.c_stride = E.r_cstride;
-    launch_find_segments(rk, E.r_sorted_vals, E.n_rel_items, E.S * E.B, E.chunk, E.n_step, rp, st);
+    rp.uniq_key = E.r_uniq.p + (size_t)s0 * rp.u_stride;
+    rp.seg_start = E.r_seg.p + (size_t)s0 * (rp.u_stride + 1);
+    rp.chunk_off = E.r_coff.p + (size_t)s0 * (rp.u_stride + 1);
+    rp.chunk_pos = E.r_cpos.p + (size_t)s0 * rp.c_stride;
+    rp.chunk_len = E.r_clen.p + (size_t)s0 * rp.c_stride;
+    rp.counts = E.r_counts.p + 2 * (size_t)s0;
+    rp.item_row = nullptr;
+    launch_find_segments(rk + s0 * NRI, E.r_sorted_vals + s0 * NRI, (int)NRI, (int)SB, E.chunk, sn, rp, st);
     HIP_CHECK(hipGetLastError());
 }
 
@@ -787,7 +800,19 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     const float* lr = (const float*)in.array("learning_rate", KGE_F32, {S});
     float* loss = (float*)in.array("loss", KGE_F32, {S});
     const bool staged = in.find("staged") && in.boolean("staged");
+    // additive: run only steps [step_begin, step_begin + step_count) of a staged batch
+    int s0 = 0, sn = E.n_step;
+    if (in.find("step_begin") || in.find("step_count")) {
+        if (!staged) throw std::invalid_argument("'step_begin' / 'step_count' need staged=true");
+        s0 = (int)in.uint("step_begin");
+        sn = (int)in.uint("step_count");
+        if (sn < 1 || s0 + sn > E.n_step) throw std::invalid_argument("step range outside the staged batch");
+    }
     const hipStream_t st = E.stream;
+    // additive: per-kernel event timing for this call only
+    const bool profile_saved = E.profile_kernels;
+    if (in.find("profile_kernels")) E.profile_kernels = in.boolean("profile_kernels");
+    struct Restore { bool& ref; bool v; ~Restore() { ref = v; } } restore{E.profile_kernels, profile_saved};
     HIP_CHECK(hipEventRecord(E.ev[0], st));
     if (!staged) {
         const BatchPtrs b = bind_batch(E, in);
@@ -798,8 +823,8 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     }
     // step sizes of every step of this call (adamStepSizeAutoIncrement, frnn.cpp:42-59)
     E.h_alpha.resize((size_t)E.n_step * 3 * S);
-    for (int i = 0; i < E.n_step; ++i) {
-        const double t = (double)(E.step + (uint32_t)i + 1u);
+    for (int i = s0; i < s0 + sn; ++i) {
+        const double t = (double)(E.step + (uint32_t)(i - s0) + 1u);
         const double factor = std::sqrt(1.0 - std::pow((double)E.beta_v, t)) / (1.0 - std::pow((double)E.beta_m, t));
         for (size_t s = 0; s < S; ++s) {
             const float a = (float)(factor * (double)lr[s]);
@@ -810,15 +835,16 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     }
     HIP_CHECK(hipMemcpyAsync(E.d_alpha.p, E.h_alpha.data(), E.h_alpha.size() * 4, hipMemcpyHostToDevice, st));
     HIP_CHECK(hipEventRecord(E.ev[1], st));
-    run_plan(E);
+    run_plan(E, s0, sn);
     HIP_CHECK(hipEventRecord(E.ev[2], st));
-    for (int i = 0; i < E.n_step; ++i) run_step(E, i);
-    launch_loss_finalize(E.loss_part.p, E.n_step, E.S, E.n_part, 1.f / (float)E.n_step, E.d_loss.p, st);
+    for (int i = s0; i < s0 + sn; ++i) run_step(E, i);
+    launch_loss_finalize(E.loss_part.p + (size_t)s0 * E.S * E.n_part, sn, E.S, E.n_part, 1.f / (float)sn,
+                         E.d_loss.p, st);
     HIP_CHECK(hipGetLastError());
     HIP_CHECK(hipEventRecord(E.ev[3], st));
     HIP_CHECK(hipMemcpyAsync(loss, E.d_loss.p, S * 4, hipMemcpyDeviceToHost, st));
     HIP_CHECK(hipStreamSynchronize(st));
-    E.step += (uint32_t)E.n_step;
+    E.step += (uint32_t)sn;
     for (int k = 0; k < 3; ++k) HIP_CHECK(hipEventElapsedTime(&E.phase_ms[k], E.ev[k], E.ev[k + 1]));
     HIP_CHECK(hipEventElapsedTime(&E.phase_ms[3], E.ev[0], E.ev[3]));
     if (E.profile_kernels) collect_kernel_times(E);

@@ -34,6 +34,7 @@ struct PlanShape {
     int n_entity;             // rows per shard table
     int shared_table;
     int n_relation;
+    int step0, step_count;    // the steps of the resident batch to plan
 };
 
 // Compact per-step arrays + the items to sort for the entity plan and the

@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void k_build_items(PlanShape ps, const uint32_
                                                      uint32_t* __restrict__ ent_vals,
                                                      uint32_t* __restrict__ rel_keys,
                                                      uint32_t* __restrict__ rel_vals) {
-    const int step = blockIdx.y;
+    const int step = ps.step0 + blockIdx.y;
     const int S = ps.S, B = ps.B, A = ps.A, NR = ps.NR, T = S * A, nst = ps.n_step;
     const int R = S * NR, SB = S * B;
     const int item = blockIdx.x * 256 + threadIdx.x;
@@ -164,7 +164,7 @@ void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint3
                         hipStream_t stream) {
     const int R = ps.S * ps.NR;
     const int n = std::max(2 * R, ps.S * ps.B + ps.n_relation);
-    dim3 grid((n + 255) / 256, ps.n_step);
+    dim3 grid((n + 255) / 256, ps.step_count);
     hipLaunchKernelGGL(k_build_items, grid, dim3(256), 0, stream, ps, remote, a2a, head, relation,
                        tail, ckey, crel, clabel, ent_keys, ent_vals, rel_keys, rel_vals);
 }

@@ -413,20 +413,29 @@ class Engine:
             raise ValueError("Calling train_step() with uninitialised variables "
                              f"{sorted(self.uninitialized_variables)}")
 
-    def train_step_loop(self, batch: Optional[Batch]) -> Tuple[float, float]:
+    def train_step_loop(self, batch: Optional[Batch], step_begin: Optional[int] = None,
+                        step_count: Optional[int] = None,
+                        profile_kernels: Optional[bool] = None) -> Tuple[float, float]:
         """``train_steps_per_program_run`` steps; returns (loss summed over
         shards and averaged over steps, learning rate used).  ``batch=None``
-        (additive) reuses the index arrays left in HBM by ``stage_batch``."""
+        (additive) reuses the index arrays left in HBM by ``stage_batch``,
+        optionally only its steps [step_begin, step_begin + step_count)."""
         self._check_initialised()
         n_shard = self.settings.model.n_shard
         lr = self._next_learning_rate()
-        self.step += self.settings.execution.train_steps_per_program_run
+        n_run = self.settings.execution.train_steps_per_program_run
         loss = np.full(n_shard, np.nan, dtype=np.float32)
         data: Dict[str, Any] = dict(learning_rate=np.full(n_shard, lr, dtype=np.float32), loss=loss)
         if batch is None:
             data["staged"] = True
+            if step_count is not None:
+                data["step_begin"], data["step_count"] = int(step_begin or 0), int(step_count)
+                n_run = int(step_count)
         else:
             data.update({k: np.ascontiguousarray(v) for k, v in vars(batch).items()})
+        if profile_kernels is not None:  # additive: HIP-event timing of every kernel
+            data["profile_kernels"] = bool(profile_kernels)
+        self.step += n_run
         self.engine.run("train_step_loop", data)
         return float(np.sum(loss)), lr
 
