@@ -168,10 +168,12 @@ def kernel_table(w, timing, n_steps, uniq_rows):
         "score_fwd": ("flops", 3.0 * pair_dims),
         "score_bwd": ("flops", 6.0 * pair_dims),
         # bytes: contributions in, one summed row out per distinct row
-        "reduce_entity": ("bytes", R * D * 4 + U * D * 4),
-        "adam_entity": ("bytes", U * 2 * row_state),
-        "reduce_relation": ("bytes", K_ * B * D * 4 + w["n_relation"] * D * 4),
-        "adam_relation": ("bytes", 2 * 3 * w["n_relation"] * D * 4),
+        # one wave per contribution: row in (from the table), float32 operand row out
+        "gather_operands": ("bytes", R * D * (emb_bytes + 4)),
+        # the two launches below each serve the entity rows and the relation table:
+        # contributions in, one summed row out per distinct row; rows read + written
+        "reduce_entity": ("bytes", (R + K_ * B) * D * 4 + (U + w["n_relation"]) * D * 4),
+        "adam_entity": ("bytes", U * 2 * row_state + 2 * 3 * w["n_relation"] * D * 4),
         "plan": ("bytes", 4.0 * (R + 2 * K_ * B) + 4 * U),
     }
     out = {}
@@ -201,6 +203,8 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=None,
                     help="steps the CPU baseline times (default: sized for ~10-30 s)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--n-entity", type=int, default=None, help="override the table size (experiments)")
+    ap.add_argument("--scoring", default=None, choices=["mfma", "valu"], help="scoring kernels (default mfma)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU holding one shard's whole table: --gpus must be 1 "
@@ -215,9 +219,14 @@ def main():
     import kge_cases as K
     import poplar_kge as kge
 
-    w = WORKLOADS[args.workload]
+    w = dict(WORKLOADS[args.workload])
+    if args.n_entity:
+        w["n_entity"] = args.n_entity
+        w["desc"] += f" [table size overridden: {args.n_entity}]"
     n_total = args.warmup + args.steps
     settings = make_settings(w, n_total, kge)
+    if args.scoring:
+        settings.execution.scoring = args.scoring
     m, d = settings.model, settings.data
     engine = kge.Engine(settings, np.full(m.n_shard, m.n_entity - 1))
     init_tables(engine, settings)

@@ -171,7 +171,7 @@ uint16_t float_to_half(float f) {
 }
 
 enum KernelId {
-    K_PLAN = 0, K_HIDDEN, K_FWD, K_LOSS, K_BWD, K_REDUCE_ENT, K_ADAM_ENT, K_REDUCE_REL, K_ADAM_REL,
+    K_PLAN = 0, K_HIDDEN, K_GATHER, K_FWD, K_LOSS, K_BWD, K_REDUCE_ENT, K_ADAM_ENT, K_REDUCE_REL, K_ADAM_REL,
     K_PROJ_GRAD, K_ADAM_PROJ, K_COUNT
 };
 
@@ -193,7 +193,9 @@ struct kge_engine {
     int n_step, rw_batch;
     int stream_kind;  // KGE_F32 or KGE_F16: dtype of the entity read/write streams
     bool profile_kernels = false;
-    int chunk = 32;
+    int use_mfma = 1;  // additive setting execution.scoring = "mfma" | "valu"
+    int chunk = 64;       // contributions per first-level chunk (rows with many contributions)
+    int direct_max = 16;  // rows with at most this many contributions are summed by their Adam wave
 
     RowLayout L;
     int64_t n_rows;
@@ -211,12 +213,13 @@ struct kge_engine {
     bool staged = false;
     // plan
     DevBuf<uint32_t> ckey, crel, clabel, ek_a, ev_a, ek_b, ev_b, rk_a, rv_a, rk_b, rv_b, hist;
-    DevBuf<uint32_t> e_uniq, e_seg, e_coff, e_cpos, e_clen, e_counts, e_item_row;
-    DevBuf<uint32_t> r_uniq, r_seg, r_coff, r_cpos, r_clen, r_counts;
+    DevBuf<uint32_t> e_uniq, e_seg, e_coff, e_cpos, e_clen, e_counts, e_item_row, e_real;
+    DevBuf<uint32_t> r_uniq, r_seg, r_coff, r_cpos, r_clen, r_counts, r_real;
+    DevBuf<uint32_t> nearflag;
     int e_ustride, e_cstride, r_ustride, r_cstride, n_rel_items;
     uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
     // step
-    DevBuf<float> coef, dist, grad, partial, rel_partial, hidden, gsum, gproj, loss_part, d_loss, d_alpha;
+    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, loss_part, d_loss, d_alpha;
     std::vector<float> h_alpha;  // [n_step][entity, relation, projection][S]
     int n_part;
     // io staging
@@ -310,6 +313,12 @@ void parse_settings(kge_engine& E, const Items& s) {
     E.shared_table = s.find("execution.shared_table") ? s.boolean("execution.shared_table") : false;
     E.profile_kernels = s.find("execution.profile_kernels") ? s.boolean("execution.profile_kernels") : false;
     if (s.find("execution.reduce_chunk")) E.chunk = (int)s.uint("execution.reduce_chunk");
+    if (s.find("execution.scoring")) {
+        const std::string v = s.str("execution.scoring");
+        if (v == "mfma") E.use_mfma = 1;
+        else if (v == "valu") E.use_mfma = 0;
+        else throw std::invalid_argument("'execution.scoring' must be 'mfma' or 'valu', not '" + v + "'");
+    }
 
     if (score == "TransE") E.score_fn = SCORE_TRANSE;
     else if (score == "DistMult") E.score_fn = SCORE_DISTMULT;
@@ -422,7 +431,8 @@ void allocate(kge_engine& E) {
     E.hist.alloc(ns * 256 * tiles);
 
     E.e_ustride = (int)R;
-    E.e_cstride = (int)(R + R / E.chunk + 1);
+    E.e_cstride = (int)(R / std::min(E.chunk, E.direct_max + 1) + 2);
+    E.e_real.alloc(ns * E.e_ustride);
     E.e_uniq.alloc(ns * E.e_ustride);
     E.e_seg.alloc(ns * (E.e_ustride + 1));
     E.e_coff.alloc(ns * (E.e_ustride + 1));
@@ -431,7 +441,8 @@ void allocate(kge_engine& E) {
     E.e_counts.alloc(ns * 2);
     if (E.F) E.e_item_row.alloc(ns * R);
     E.r_ustride = E.n_rel;
-    E.r_cstride = (int)(E.n_rel + SB / E.chunk + 1);
+    E.r_cstride = (int)(SB / std::min(E.chunk, E.direct_max + 1) + 2);
+    E.r_real.alloc(ns * E.r_ustride);
     E.r_uniq.alloc(ns * E.r_ustride);
     E.r_seg.alloc(ns * (E.r_ustride + 1));
     E.r_coff.alloc(ns * (E.r_ustride + 1));
@@ -443,8 +454,10 @@ void allocate(kge_engine& E) {
     const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f;
     if (!fused && E.score_fn == SCORE_TRANSE && E.dist_fn == DIST_L2) E.dist.alloc(SB * E.T);
     E.grad.alloc(R * E.Dp);
+    E.opnd.alloc(R * E.Dp);
     E.partial.alloc((size_t)E.e_cstride * E.Dp);
     E.rel_partial.alloc((size_t)E.r_cstride * E.Dp);
+    if (E.score_fn == SCORE_DISTMULT) E.rel_gsum.alloc((size_t)E.n_rel * E.Dp);
     if (E.F) {
         E.hidden.alloc(R * E.Dp);
         E.gsum.alloc(R * E.Dp);
@@ -452,7 +465,12 @@ void allocate(kge_engine& E) {
     }
     ScoreShape sh = {};
     sh.S = E.S; sh.B = E.B; sh.T = E.T;
+    sh.score_fn = E.score_fn; sh.dist_fn = E.dist_fn; sh.use_mfma = E.use_mfma;
     E.n_part = fused ? score_fwd_parts(sh) : E.B;
+    if (E.use_mfma && E.score_fn == SCORE_TRANSE && E.dist_fn == DIST_L2) {
+        E.nearflag.alloc(nearflag_words(sh));
+        E.nearflag.zero(st);
+    }
     E.loss_part.alloc(ns * S * E.n_part);
     E.d_loss.alloc(S);
     E.d_alpha.alloc(ns * 3 * S);
@@ -658,7 +676,8 @@ void run_plan(kge_engine& E, int s0, int sn) {
     ep.chunk_len = E.e_clen.p + (size_t)s0 * ep.c_stride;
     ep.counts = E.e_counts.p + 2 * (size_t)s0;
     ep.item_row = E.F ? E.e_item_row.p + s0 * R : nullptr;
-    launch_find_segments(ek + s0 * N, E.e_sorted_vals + s0 * N, (int)N, (int)R, E.chunk, sn, ep, st);
+    ep.seg_real = E.e_real.p + (size_t)s0 * ep.u_stride;
+    launch_find_segments(ek + s0 * N, E.e_sorted_vals + s0 * N, (int)N, (int)R, E.chunk, E.direct_max, sn, ep, st);
 
     which = launch_radix_sort(E.rk_a.p + s0 * NRI, E.rv_a.p + s0 * NRI, E.rk_b.p + s0 * NRI,
                               E.rv_b.p + s0 * NRI, E.hist.p, (int)NRI, sn, rbits, st);
@@ -673,7 +692,8 @@ void run_plan(kge_engine& E, int s0, int sn) {
     rp.chunk_len = E.r_clen.p + (size_t)s0 * rp.c_stride;
     rp.counts = E.r_counts.p + 2 * (size_t)s0;
     rp.item_row = nullptr;
-    launch_find_segments(rk + s0 * NRI, E.r_sorted_vals + s0 * NRI, (int)NRI, (int)SB, E.chunk, sn, rp, st);
+    rp.seg_real = E.r_real.p + (size_t)s0 * rp.u_stride;
+    launch_find_segments(rk + s0 * NRI, E.r_sorted_vals + s0 * NRI, (int)NRI, (int)SB, E.chunk, E.direct_max, sn, rp, st);
     HIP_CHECK(hipGetLastError());
 }
 
@@ -692,6 +712,8 @@ void run_step(kge_engine& E, int i) {
         sh.softmax_correction = E.softmax_cw * corr;
     }
     sh.negative_adversarial_scale = E.neg_adv;
+    sh.use_mfma = E.use_mfma;
+    sh.operands_dense = 0;
     const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f;
 
     const uint32_t* ckey = E.ckey.p + i * R;
@@ -717,11 +739,20 @@ void run_step(kge_engine& E, int i) {
         ent.index = E.e_item_row.p + i * R;
     }
 
+    // dense operands: every contribution's row, float32, relation applied to the heads
+    { KernelTimer t(E, K_GATHER);
+      launch_gather_operands(ent, E.rel.p, crel, E.score_fn == SCORE_DISTMULT ? 2 : 1, (int)SB, (int)R, E.Dp,
+                             E.opnd.p, st); }
+    RowSource dense;
+    dense.base = (const char*)E.opnd.p; dense.pitch = (int64_t)E.Dp * 4; dense.etype = ET_F32;
+    dense.index = nullptr; dense.count = E.Dp; dense.vec = 1;
+    sh.operands_dense = 1;
+
     float* loss_part = E.loss_part.p + (size_t)i * E.S * E.n_part;
     { KernelTimer t(E, K_FWD);
-      launch_score_fwd(sh, ent, E.rel.p, crel, clabel, E.coef.p, E.dist.p, loss_part, fused, st); }
+      launch_score_fwd(sh, dense, E.rel.p, crel, clabel, E.coef.p, E.dist.p, E.nearflag.p, loss_part, fused, st); }
     if (!fused) { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, E.dist.p, loss_part, st); }
-    { KernelTimer t(E, K_BWD); launch_score_bwd(sh, ent, E.rel.p, crel, E.coef.p, E.grad.p, st); }
+    { KernelTimer t(E, K_BWD); launch_score_bwd(sh, dense, E.rel.p, crel, E.coef.p, E.nearflag.p, E.grad.p, st); }
 
     const float* alpha = E.d_alpha.p + (size_t)i * 3 * E.S;
     AdamArgs aa = {};
@@ -730,30 +761,41 @@ void run_step(kge_engine& E, int i) {
     aa.one_minus_beta_m = 1.f - E.beta_m; aa.one_minus_beta_v = 1.f - E.beta_v;
     aa.epsilon = E.epsilon; aa.weight_decay = E.weight_decay;
 
-    // relation gradient first: for DistMult it needs the pre-update head rows
+    // both reductions read pre-update rows (DistMult multiplies by them), so they
+    // come before both updates
+    ContribSrc rsrc = {};
+    rsrc.sorted_item = E.r_sorted_vals + (size_t)i * E.n_rel_items;
+    rsrc.grad = E.grad.p;
+    rsrc.transform = E.score_fn == SCORE_DISTMULT ? 2 : 0; rsrc.n_head = (int)SB;
+    rsrc.rel = E.rel.p; rsrc.crel = crel; rsrc.ent = ent;
+    ContribSrc esrc = rsrc;
+    esrc.sorted_item = E.e_sorted_vals + (size_t)i * 2 * R;
+    esrc.transform = E.score_fn == SCORE_DISTMULT ? 1 : 0;
+
     ReduceArgs rr = {};
-    rr.sorted_item = E.r_sorted_vals + (size_t)i * E.n_rel_items;
+    rr.src = rsrc;
     rr.chunk_pos = E.r_cpos.p + (size_t)i * E.r_cstride;
     rr.chunk_len = E.r_clen.p + (size_t)i * E.r_cstride;
     rr.counts = r_counts; rr.max_chunks = E.r_cstride;
-    rr.grad = E.grad.p; rr.partial = E.rel_partial.p; rr.Dp = E.Dp;
-    rr.transform = E.score_fn == SCORE_DISTMULT ? 2 : 0; rr.n_head = (int)SB;
-    rr.rel = E.rel.p; rr.crel = crel; rr.ent = ent;
-    { KernelTimer t(E, K_REDUCE_REL); launch_reduce_chunks(rr, st); }
+    rr.partial = E.rel_partial.p; rr.Dp = E.Dp;
 
     ReduceArgs re = {};
-    re.sorted_item = E.e_sorted_vals + (size_t)i * 2 * R;
+    re.src = esrc;
     re.chunk_pos = E.e_cpos.p + (size_t)i * E.e_cstride;
     re.chunk_len = E.e_clen.p + (size_t)i * E.e_cstride;
     re.counts = e_counts; re.max_chunks = E.e_cstride;
-    re.grad = E.grad.p; re.partial = E.partial.p; re.Dp = E.Dp;
-    re.transform = E.score_fn == SCORE_DISTMULT ? 1 : 0; re.n_head = (int)SB;
-    re.rel = E.rel.p; re.crel = crel; re.ent = ent;
-    { KernelTimer t(E, K_REDUCE_ENT); launch_reduce_chunks(re, st); }
+    re.partial = E.partial.p; re.Dp = E.Dp;
+    { KernelTimer t(E, K_REDUCE_ENT); launch_reduce_chunks2(re, rr, st); }
 
-    // dense Adam on the relation table (updateParameters, :329-339)
+    // With DistMult the relation rows' direct contributions read entity rows and
+    // the entity rows' read relation rows, so neither table may be updated before
+    // the other's gradient is complete: materialise the relation gradient first.
+    // (TransE contributions do not depend on either table.)
     AdamArgs ar = aa;
+    ar.src = rsrc;
     ar.uniq_key = E.r_uniq.p + (size_t)i * E.r_ustride;
+    ar.seg_start = E.r_seg.p + (size_t)i * (E.r_ustride + 1);
+    ar.seg_real = E.r_real.p + (size_t)i * E.r_ustride;
     ar.chunk_off = E.r_coff.p + (size_t)i * (E.r_ustride + 1);
     ar.counts = r_counts; ar.max_rows = E.n_rel;
     ar.partial = E.rel_partial.p;
@@ -761,11 +803,12 @@ void run_step(kge_engine& E, int i) {
     ar.pitch = (int64_t)E.Dp * 4; ar.p_etype = ET_F32; ar.v_is_sqrt = 0;
     ar.alpha = alpha + E.S;
     ar.rows_per_alpha = E.shared_table ? 0u : (uint32_t)(E.n_rel / E.S);
-    { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
 
-    // entity rows: sum partials, Adam on [emb | m | sqrt v], write back in place (:695-704)
     AdamArgs ae = aa;
+    ae.src = esrc;
     ae.uniq_key = e_uniq;
+    ae.seg_start = E.e_seg.p + (size_t)i * (E.e_ustride + 1);
+    ae.seg_real = E.e_real.p + (size_t)i * E.e_ustride;
     ae.chunk_off = E.e_coff.p + (size_t)i * (E.e_ustride + 1);
     ae.counts = e_counts; ae.max_rows = (int)R;
     ae.partial = E.partial.p;
@@ -774,7 +817,22 @@ void run_step(kge_engine& E, int i) {
     ae.pitch = E.L.pitch; ae.p_etype = E.L.emb_etype; ae.v_is_sqrt = 1;
     ae.alpha = alpha;
     ae.rows_per_alpha = E.shared_table ? 0u : (uint32_t)E.n_entity;
-    { KernelTimer t(E, K_ADAM_ENT); launch_adam_rows(ae, st); }
+
+    if (E.score_fn == SCORE_DISTMULT) {
+        // entity update first (reads pre-update relation rows), writing its summed
+        // gradient is not needed; then the relation update reads POST-update entity
+        // rows unless its gradient was materialised: do that with a zero-step pass
+        ar.grad_out = E.rel_gsum.p;
+        ar.no_update = 1;
+        { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
+        { KernelTimer t(E, K_ADAM_ENT); launch_adam_rows(ae, st); }
+        ar.grad_out = nullptr; ar.no_update = 0;
+        ar.grad_direct = E.rel_gsum.p;
+        { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
+    } else {
+        KernelTimer t(E, K_ADAM_ENT);
+        launch_adam_rows2(ae, ar, st);
+    }
 
     if (E.F) {
         { KernelTimer t(E, K_PROJ_GRAD); launch_proj_grad(fa, E.gsum.p, E.gproj.p, st); }
@@ -1100,11 +1158,13 @@ int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* i
     sp.item_row = nullptr; sp.u_stride = (int)rows; sp.c_stride = (int)L.cmax;
     const uint32_t* sk = which ? u32(L.off_keys_b) : u32(L.off_keys_a);
     const uint32_t* sv = which ? u32(L.off_vals_b) : u32(L.off_vals_a);
-    launch_find_segments(sk, sv, (int)L.N, (int)n, 32, 1, sp, st);
+    sp.seg_real = nullptr;
+    launch_find_segments(sk, sv, (int)L.N, (int)n, 32, 0, 1, sp, st);
     ReduceArgs ra = {};
-    ra.sorted_item = sv; ra.chunk_pos = sp.chunk_pos; ra.chunk_len = sp.chunk_len; ra.counts = sp.counts;
-    ra.max_chunks = (int)L.cmax; ra.grad = grad_out; ra.partial = (float*)(w + L.off_partial);
-    ra.Dp = (int)cols; ra.transform = 0;
+    ra.src.sorted_item = sv; ra.src.grad = grad_out; ra.src.transform = 0;
+    ra.chunk_pos = sp.chunk_pos; ra.chunk_len = sp.chunk_len; ra.counts = sp.counts;
+    ra.max_chunks = (int)L.cmax; ra.partial = (float*)(w + L.off_partial);
+    ra.Dp = (int)cols;
     launch_reduce_chunks(ra, st);
     launch_sum_partials_rows(sp.chunk_off, ra.partial, rows, cols, grad_t, st);
     return op_status("scatter_add");

@@ -64,11 +64,14 @@ struct SegPlan {
     uint32_t* chunk_len;  // [n_seg, c_stride]      real items in the chunk (<= chunk size)
     uint32_t* counts;     // [n_seg, 2]             {distinct rows, chunks}
     uint32_t* item_row;   // [n_seg, n_real] or null: distinct-row index of each real item
+    uint32_t* seg_real;   // [n_seg, u_stride] or null: real items of each row
     int u_stride, c_stride;
 };
 
+// Rows with at most `direct_max` real items get no chunks (their consumer sums
+// the items itself); longer rows are cut into chunks of `chunk` items.
 void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sorted, int N,
-                          int n_real, int chunk, int n_seg, const SegPlan& plan,
+                          int n_real, int chunk, int direct_max, int n_seg, const SegPlan& plan,
                           hipStream_t stream);
 
 // ---- step phase ----------------------------------------------------------
@@ -79,7 +82,14 @@ struct ScoreShape {
     float gamma, loss_scale;
     float softmax_correction;      // already multiplied by the correction weight
     float negative_adversarial_scale;
+    int use_mfma;                  // L2 / dot scoring on the matrix cores (else the VALU kernels)
+    int operands_dense;            // a-operand rows already hold the predicted tails (launch_gather_operands)
 };
+
+// Dense float32 operand matrix [n_rows, Dp] from indexed rows: rows [0, n_head)
+// combined with their relation row (rel_mode 1 add, 2 multiply).
+void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
+                            int n_head, int n_rows, int Dp, float* out, hipStream_t stream);
 
 // Scores of every block: a-operand row (d,b) = entity row of contribution
 // d*B+b combined with relation crel[d*B+b]; b-operand row (d,t) = entity row of
@@ -89,7 +99,11 @@ struct ScoreShape {
 // loss_part receives S * n_part partial sums (n_part = tiles per block).
 void launch_score_fwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
                       const uint32_t* crel, const uint32_t* clabel, float* coef, float* dist,
-                      float* loss_part, bool fused_loss, hipStream_t stream);
+                      uint32_t* nearflag, float* loss_part, bool fused_loss, hipStream_t stream);
+// words of the near-identical-pair flag matrix the L2 matrix-core path needs
+inline size_t nearflag_words(const ScoreShape& sh) {
+    return (size_t)sh.S * ((sh.B + 31) / 32) * ((sh.T + 31) / 32);
+}
 int score_fwd_parts(const ScoreShape& sh);
 
 // Row-wise losses (softmax; logsigmoid with adversarial weighting): converts
@@ -102,39 +116,49 @@ void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef,
 // (w.r.t. the predicted tail / the head-times-relation product) and tail
 // contributions, from the coefficient matrix.
 void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
-                      const uint32_t* crel, const float* coef, float* grad, hipStream_t stream);
+                      const uint32_t* crel, const float* coef, const uint32_t* nearflag, float* grad,
+                      hipStream_t stream);
 
-// Deterministic segmented reduction, first level: one wave per chunk sums the
-// chunk's gradient rows in sorted order into partial[chunk, :].
-// transform: 0 none; 1 multiply head rows (c < n_head) by rel[crel[c]]
-// (DistMult, entity plan); 2 multiply by the head entity row (DistMult,
-// relation plan).
-struct ReduceArgs {
+// Where gradient contributions come from.  transform: 0 none; 1 multiply head
+// rows (c < n_head) by rel[crel[c]] (DistMult, entity plan); 2 multiply by the
+// head entity row (DistMult, relation plan).
+struct ContribSrc {
     const uint32_t* sorted_item;  // this step's sorted values
-    const uint32_t* chunk_pos;
-    const uint32_t* chunk_len;
-    const uint32_t* counts;       // {rows, chunks}
-    int max_chunks;
     const float* grad;            // [R, Dp]
-    float* partial;               // [max_chunks, Dp]
-    int Dp;
     int transform, n_head;
     const float* rel;
     const uint32_t* crel;
     RowSource ent;
 };
-void launch_reduce_chunks(const ReduceArgs& a, hipStream_t stream);
 
-// Second level fused with Adam: one wave per distinct row sums its chunk
-// partials in order, applies the update in place and (optionally) stores the
-// summed gradient.
+// Deterministic segmented reduction, first level (rows with many
+// contributions only): one workgroup per chunk sums the chunk's gradient rows
+// in a fixed order into partial[chunk, :].
+struct ReduceArgs {
+    ContribSrc src;
+    const uint32_t* chunk_pos;
+    const uint32_t* chunk_len;
+    const uint32_t* counts;       // {rows, chunks}
+    int max_chunks;
+    float* partial;               // [max_chunks, Dp]
+    int Dp;
+};
+void launch_reduce_chunks(const ReduceArgs& a, hipStream_t stream);
+void launch_reduce_chunks2(const ReduceArgs& a0, const ReduceArgs& a1, hipStream_t stream);  // one launch
+
+// Second level fused with Adam: one wave per distinct row sums its
+// contributions (few: directly; many: its chunk partials) in order, applies the
+// update in place and (optionally) stores the summed gradient.
 struct AdamArgs {
+    ContribSrc src;
     const uint32_t* uniq_key;
+    const uint32_t* seg_start;
+    const uint32_t* seg_real;
     const uint32_t* chunk_off;
     const uint32_t* counts;
     int max_rows;
-    const float* partial;      // [chunks, Dp] or null
-    const float* grad_direct;  // [rows, Dp] used instead of partial when non-null
+    const float* partial;      // [chunks, Dp]
+    const float* grad_direct;  // [rows, Dp] used instead of the contributions when non-null
     float* grad_out;           // [rows, Dp] or null
     char* p_base;              // parameter rows: p_base + key * pitch
     char* m_base;
@@ -143,11 +167,13 @@ struct AdamArgs {
     int p_etype;               // ET_* of the parameter (moments are float32)
     int Dp;
     int v_is_sqrt;
+    int no_update;             // only form the summed gradient (grad_out), leave the rows alone
     const float* alpha;        // [n_alpha] step sizes
     uint32_t rows_per_alpha;   // alpha index = key / rows_per_alpha (0: always alpha[0])
     float beta_m, beta_v, one_minus_beta_m, one_minus_beta_v, epsilon, weight_decay;
 };
 void launch_adam_rows(const AdamArgs& a, hipStream_t stream);
+void launch_adam_rows2(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream);  // one launch
 
 // loss[s] = sum over steps and parts of loss_part / n_step, in a fixed order.
 void launch_loss_finalize(const float* loss_part, int n_step, int S, int n_part, float scale,

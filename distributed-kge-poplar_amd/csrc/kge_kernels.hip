@@ -325,7 +325,8 @@ DEVINL uint32_t block_scan_1024(uint32_t v, uint32_t* lds /*[16]*/, uint32_t* to
 
 __global__ __launch_bounds__(1024) void k_find_segments(const uint32_t* __restrict__ keys,
                                                         const uint32_t* __restrict__ vals, int N,
-                                                        int n_real, int chunk, SegPlan plan) {
+                                                        int n_real, int chunk, int direct_max,
+                                                        SegPlan plan) {
     __shared__ uint32_t lds[16];
     const int seg = blockIdx.x, tid = threadIdx.x;
     keys += (size_t)seg * N;
@@ -336,6 +337,7 @@ __global__ __launch_bounds__(1024) void k_find_segments(const uint32_t* __restri
     uint32_t* chunk_pos = plan.chunk_pos + (size_t)seg * plan.c_stride;
     uint32_t* chunk_len = plan.chunk_len + (size_t)seg * plan.c_stride;
     uint32_t* item_row = plan.item_row ? plan.item_row + (size_t)seg * n_real : nullptr;
+    uint32_t* seg_real = plan.seg_real ? plan.seg_real + (size_t)seg * plan.u_stride : nullptr;
 
     const int per = (N + 1023) / 1024;
     const int lo = min(N, tid * per), hi = min(N, lo + per);
@@ -368,7 +370,9 @@ __global__ __launch_bounds__(1024) void k_find_segments(const uint32_t* __restri
             const uint32_t mid = (a + b) >> 1;
             if (vals[mid] < (uint32_t)n_real) a = mid + 1; else b = mid;
         }
-        nch += (a - s + chunk - 1) / chunk;
+        const uint32_t real = a - s;
+        if (seg_real) seg_real[u] = real;
+        if (real > (uint32_t)direct_max) nch += (real + chunk - 1) / chunk;
     }
     uint32_t NC;
     uint32_t cb = block_scan_1024(nch, lds, &NC);
@@ -381,6 +385,7 @@ __global__ __launch_bounds__(1024) void k_find_segments(const uint32_t* __restri
         }
         const uint32_t real = a - s;
         chunk_off[u] = cb;
+        if (real <= (uint32_t)direct_max) continue;
         for (uint32_t l = 0; l * chunk < real; ++l) {
             chunk_pos[cb] = s + l * chunk;
             chunk_len[cb] = min((uint32_t)chunk, real - l * chunk);
@@ -395,10 +400,37 @@ __global__ __launch_bounds__(1024) void k_find_segments(const uint32_t* __restri
 }
 
 void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sorted, int N,
-                          int n_real, int chunk, int n_seg, const SegPlan& plan,
+                          int n_real, int chunk, int direct_max, int n_seg, const SegPlan& plan,
                           hipStream_t stream) {
     hipLaunchKernelGGL(k_find_segments, dim3(n_seg), dim3(1024), 0, stream, keys_sorted,
-                       vals_sorted, N, n_real, chunk, plan);
+                       vals_sorted, N, n_real, chunk, direct_max, plan);
+}
+
+// --------------------------------------------------------------------------
+// operand gather: one wave per contribution copies its entity (or hidden) row,
+// converted to float32 and with the relation already applied for the heads
+// (predicted tail h + r, or h * r), into the dense operand matrix the scoring
+// kernels read: rows [0, n_head) = a-operands, the rest = b-operands.
+__global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const float* __restrict__ rel,
+                                                         const uint32_t* __restrict__ crel,
+                                                         int rel_mode, int n_head, int n_rows, int Dp,
+                                                         float* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (c >= n_rows) return;
+    const char* row = row_ptr(ent, c);
+    const float* rrow = (c < n_head && rel_mode) ? rel + (size_t)crel[c] * Dp : nullptr;
+    for (int k = lane * 4; k < Dp; k += 256) {
+        float4 v = load4(row, k, ent);
+        if (rrow) v = combine_rel(v, rrow, k, rel_mode);
+        *reinterpret_cast<float4*>(out + (size_t)c * Dp + k) = v;
+    }
+}
+
+void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
+                            int n_head, int n_rows, int Dp, float* out, hipStream_t stream) {
+    hipLaunchKernelGGL(k_gather_operands, dim3((n_rows + 3) / 4), dim3(256), 0, stream, ent, rel, crel,
+                       rel_mode, n_head, n_rows, Dp, out);
 }
 
 // --------------------------------------------------------------------------
@@ -407,6 +439,27 @@ void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sort
 // logSigmoid and its derivative exactly as src/pag/pag.cpp:894-903
 DEVINL float log_sigmoid(float z) { return z > -11.f ? -log1pf(expf(-z)) : z; }
 DEVINL float log_sigmoid_grad(float z) { return 1.f / (1.f + expf(fminf(z, 11.f))); }
+
+// The same two functions from ONE hardware exponential (the scoring epilogues
+// evaluate them once per score): with u = exp(-|z|) in (0, 1],
+//   z >= 0:        logsig = -log1p(u),     dlogsig = u' / (1 + u'),  u' = max(u, e^-11)  (the +11 clamp)
+//   -11 < z < 0:   logsig = z - log1p(u),  dlogsig = 1 / (1 + u)
+//   z <= -11:      logsig = z              (the reference drops the log1p term there)
+// log1p(u) = log(w) - ((w - 1) - u) / w with w = 1 + u keeps the low bits of u.
+DEVINL void log_sigmoid_both(float z, float& value, float& grad) {
+    const float u = __expf(-fabsf(z));
+    const float w = 1.f + u;
+    const float rw = __frcp_rn(w);
+    const float l1p = __logf(w) - ((w - 1.f) - u) * rw;
+    if (z >= 0.f) {
+        const float uc = fmaxf(u, 1.670170079e-5f);  // exp(-11)
+        value = -l1p;
+        grad = uc * __frcp_rn(1.f + uc);
+    } else {
+        value = z > -11.f ? z - l1p : z;
+        grad = rw;
+    }
+}
 
 struct FwdParams {
     ScoreShape sh;
@@ -420,6 +473,7 @@ struct FwdParams {
     int a_rel_mode;   // how the a-operand combines with its relation row
     int out_mode;     // 0 fused logsigmoid -> coefficient; 1 raw score (+dist); 2 raw distance
     int a_c0, b_c0;   // contribution index of block 0's first a / b row
+    uint32_t* nearflag;  // [S, ceil(B/32), ceil(T/32)] or null: 32x32 sub-blocks holding near-identical pairs
 };
 
 constexpr int BK = 32;         // embedding columns staged per iteration
@@ -430,10 +484,12 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
     __shared__ __attribute__((aligned(16))) float As[BK][LDP];
     __shared__ __attribute__((aligned(16))) float Bs[BK][LDP];
     __shared__ float red[4];
+    __shared__ uint32_t label_s[kScoreTile];
     const ScoreShape& sh = p.sh;
     const int d = blockIdx.z, m0 = blockIdx.y * kScoreTile, n0 = blockIdx.x * kScoreTile;
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int B = sh.B, T = sh.T, Dp = sh.Dp;
+    if (p.out_mode == 0 && tid < kScoreTile) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
 
     // staging assignment: row lr (+32) of each operand, float4 column k4
     const int lr = tid >> 3, k4 = (tid & 7) * 4;
@@ -500,7 +556,7 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
     for (int i = 0; i < 4; ++i) {
         const int m = m0 + ty * 4 + i;
         if (m >= B) continue;
-        const uint32_t label = p.out_mode == 0 ? p.clabel[d * B + m] : 0u;
+        const uint32_t label = p.out_mode == 0 ? label_s[ty * 4 + i] : 0u;
         float outv[4], distv[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -513,11 +569,13 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
             const bool pos = (uint32_t)n == label;
             const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
             const float z = sign * score;
-            if (n < T) loss_acc -= w * log_sigmoid(z);
+            float lsig, dlsig;
+            log_sigmoid_both(z, lsig, dlsig);
+            if (n < T) loss_acc -= w * lsig;
             // d loss / d score, times the loss scale
-            const float ds = -w * sign * log_sigmoid_grad(z) * inv_norm * sh.loss_scale;
+            const float ds = -w * sign * dlsig * inv_norm * sh.loss_scale;
             float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;  // score = gamma - dist
-            if (DIST == DIST_L2) c = dist != 0.f ? c / dist : 0.f;
+            if (DIST == DIST_L2) c = dist != 0.f ? c * __frcp_rn(dist) : 0.f;
             outv[j] = c;
         }
         const int n = n0 + tx * 4;
@@ -547,11 +605,306 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
     }
 }
 
+// --------------------------------------------------------------------------
+// scoring forward on the matrix cores (L2 and dot): S[m,n] = sum_k a[m,k] b[n,k]
+// with v_mfma_f32_32x32x2_f32.  Workgroup tile 128 (a rows) x 64 (b rows), four
+// waves as 2 x 2, each wave two 32x32 accumulators.  For L2,
+// d^2 = |a|^2 + |b|^2 - 2 a.b; where that cancels (d^2 small against the norms)
+// the pair is recomputed directly as sum (a-b)^2 by the whole wave, so the
+// result keeps float32 accuracy and is exactly 0 for identical rows.
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int FM_TM = 128, FM_TN = 64, FM_LDA = FM_TM + 1, FM_LDB = FM_TN + 1;
+constexpr float kCancelRatio = 0.125f;  // recompute when d^2 < ratio * (|a|^2 + |b|^2)
+// Below this ratio the backward's product form self*sum(c) - sum(c*other) would
+// lose accuracy against the reference's c*(self-other); such 32x32 sub-blocks
+// are flagged for the backward kernel, which handles them in the direct form.
+constexpr float kNearRatio = 1.f / 4096.f;
+
+// BKT = embedding columns staged per iteration: with 128 a whole D = 256 row
+// takes two iterations, the loads of the second in flight under the first's
+// matrix work (one workgroup per CU, 99 KB of LDS).
+// ALIGNED: B % 128 == 0, T % 64 == 0, Dp % BKT == 0, float32 operands with the
+// relation already applied: the
+// staging loads carry no bounds checks (and so no branches that would force
+// the prefetch to complete before the matrix work starts).
+template <int DIST, int BKT, bool ALIGNED>
+__global__ __launch_bounds__(256) void k_score_fwd_mfma(FwdParams p) {
+    constexpr int NC = BKT / 32;  // float4 columns per staged row per thread
+    __shared__ float As[BKT][FM_LDA];
+    __shared__ float Bs[BKT][FM_LDB];
+    __shared__ float na_s[FM_TM], nb_s[FM_TN];
+    __shared__ float red[4];
+    __shared__ uint32_t label_s[FM_TM];
+    const ScoreShape& sh = p.sh;
+    const int d = blockIdx.z, m0 = blockIdx.y * FM_TM, n0 = blockIdx.x * FM_TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 32;
+    const int B = sh.B, T = sh.T, Dp = sh.Dp;
+    if (p.out_mode == 0 && tid < FM_TM) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
+
+    // staging: a tile = 128 rows x 32 columns = 1024 float4 (4 per thread),
+    // b tile = 64 x 32 = 512 float4 (2 per thread); 8 consecutive threads share a row
+    const int srow = tid >> 3, k4 = (tid & 7) * 4;
+    const char* arow[4];
+    const float* rrow[4];
+    const char* brow[2];
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+        const int m = m0 + srow + 32 * h;
+        if (ALIGNED) {  // dense, un-indexed operands: plain address arithmetic
+            arow[h] = p.ent_a.base + (int64_t)(p.a_c0 + d * B + m) * p.ent_a.pitch;
+            rrow[h] = nullptr;
+        } else {
+            arow[h] = m < B ? row_ptr(p.ent_a, p.a_c0 + d * B + m) : nullptr;
+            rrow[h] = (m < B && p.a_rel_mode) ? p.rel + (size_t)p.crel[d * B + m] * Dp : nullptr;
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int n = n0 + srow + 32 * h;
+        if (ALIGNED) brow[h] = p.ent_b.base + (int64_t)(p.b_c0 + d * T + n) * p.ent_b.pitch;
+        else brow[h] = n < T ? row_ptr(p.ent_b, p.b_c0 + d * T + n) : nullptr;
+    }
+    float na_acc[4] = {0.f, 0.f, 0.f, 0.f}, nb_acc[2] = {0.f, 0.f};
+    floatx16 acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+
+    float4 areg[4][NC], breg[2][NC];
+    auto prefetch = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int k = k0 + 32 * c + k4;
+            if (ALIGNED) {
+#pragma unroll
+                for (int h = 0; h < 4; ++h) areg[h][c] = *reinterpret_cast<const float4*>(arow[h] + (size_t)k * 4);
+#pragma unroll
+                for (int h = 0; h < 2; ++h) breg[h][c] = *reinterpret_cast<const float4*>(brow[h] + (size_t)k * 4);
+                continue;
+            }
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+                areg[h][c] = make_float4(0, 0, 0, 0);
+                if (arow[h] && k < Dp)
+                    areg[h][c] = combine_rel(load4(arow[h], k, p.ent_a), rrow[h], k, p.a_rel_mode);
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                breg[h][c] = make_float4(0, 0, 0, 0);
+                if (brow[h] && k < Dp) breg[h][c] = load4(brow[h], k, p.ent_b);
+            }
+        }
+    };
+    prefetch(0);
+    for (int k0 = 0; k0 < Dp; k0 += BKT) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int kc = 32 * c + k4;
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+                const float4 a = areg[h][c];
+                const int r = srow + 32 * h;
+                As[kc + 0][r] = a.x; As[kc + 1][r] = a.y; As[kc + 2][r] = a.z; As[kc + 3][r] = a.w;
+                if (DIST == DIST_L2) na_acc[h] += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const float4 b = breg[h][c];
+                const int r = srow + 32 * h;
+                Bs[kc + 0][r] = b.x; Bs[kc + 1][r] = b.y; Bs[kc + 2][r] = b.z; Bs[kc + 3][r] = b.w;
+                if (DIST == DIST_L2) nb_acc[h] += b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+            }
+        }
+        __syncthreads();
+        if (k0 + BKT < Dp) prefetch(k0 + BKT);
+        // operands of four k-pairs at a time, fetched from LDS one group ahead of
+        // the matrix instructions that consume them
+        {
+            constexpr int NG = BKT / 8;
+            float ra0[2][4], ra1[2][4], rb[2][4];
+            const int hl = lane >> 5, cl = lane & 31;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                rb[0][x] = Bs[2 * x + hl][wn + cl];
+                ra0[0][x] = As[2 * x + hl][wm + cl];
+                ra1[0][x] = As[2 * x + hl][wm + 32 + cl];
+            }
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                if (g + 1 < NG) {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const int kk = 8 * (g + 1) + 2 * x + hl;
+                        rb[(g + 1) & 1][x] = Bs[kk][wn + cl];
+                        ra0[(g + 1) & 1][x] = As[kk][wm + cl];
+                        ra1[(g + 1) & 1][x] = As[kk][wm + 32 + cl];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra0[g & 1][x], rb[g & 1][x], acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra1[g & 1][x], rb[g & 1][x], acc[1], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();
+    }
+    if (DIST == DIST_L2) {
+        // the 8 threads of a row hold partial sums of squares: combine in a fixed order
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+            float v = na_acc[h];
+            v += __shfl_xor(v, 1, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 4, 64);
+            if ((tid & 7) == 0) na_s[srow + 32 * h] = v;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float v = nb_acc[h];
+            v += __shfl_xor(v, 1, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 4, 64);
+            if ((tid & 7) == 0) nb_s[srow + 32 * h] = v;
+        }
+        __syncthreads();
+    }
+
+    // epilogue.  Accumulator layout of v_mfma_f32_32x32x2_f32: register r of
+    // lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+    const float Tn = (float)T;
+    const float w_pos = 0.5f * Tn, w_neg = (0.5f * Tn) / (float)(T - 1);
+    const float inv_norm = 1.f / ((float)sh.S * (float)B * Tn);
+    float loss_acc = 0.f;
+    const int n_loc = wn + (lane & 31), n = n0 + n_loc;
+    const float nb = DIST == DIST_L2 ? nb_s[n_loc] : 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        // phase 1 (straight-line): squared distances and which of them cancelled
+        float val[16];
+        uint32_t cancel = 0u, near = 0u;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m_loc = wm + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const bool live = ALIGNED || (m0 + m_loc < B && n < T);
+            val[r] = acc[t][r];
+            if (DIST == DIST_L2) {
+                const float na = na_s[m_loc];
+                val[r] = na + nb - 2.f * acc[t][r];
+                if (live && val[r] < kCancelRatio * (na + nb)) cancel |= 1u << r;
+                if (live && val[r] < kNearRatio * (na + nb)) near |= 1u << r;
+            }
+        }
+        // phase 2 (rare): the wave recomputes the cancelled pairs directly
+        if (DIST == DIST_L2 && __ballot(cancel != 0u)) {
+            near = 0u;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m_loc = wm + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const int m = m0 + m_loc;
+                uint64_t todo = __ballot((cancel >> r) & 1u);
+                while (todo) {
+                    const int src = __ffsll((long long)todo) - 1;
+                    todo &= todo - 1;
+                    const int fm = __shfl(m, src, 64), fn = __shfl(n, src, 64);
+                    const char* ar = row_ptr(p.ent_a, p.a_c0 + d * B + fm);
+                    const float* rr = p.a_rel_mode ? p.rel + (size_t)p.crel[d * B + fm] * Dp : nullptr;
+                    const char* br = row_ptr(p.ent_b, p.b_c0 + d * T + fn);
+                    float part = 0.f;
+                    for (int k = lane * 4; k < Dp; k += 256) {
+                        const float4 a = combine_rel(load4(ar, k, p.ent_a), rr, k, p.a_rel_mode);
+                        const float4 b = load4(br, k, p.ent_b);
+                        const float dx = a.x - b.x, dy = a.y - b.y, dz = a.z - b.z, dw = a.w - b.w;
+                        part += dx * dx + dy * dy + dz * dz + dw * dw;
+                    }
+                    part = wave_sum(part);
+                    if (lane == src) val[r] = part;
+                }
+                const bool live = ALIGNED || (m < B && n < T);
+                if (live && val[r] < kNearRatio * (na_s[m_loc] + nb)) near |= 1u << r;
+            }
+        }
+        // phase 3 (straight-line): distance, score, loss, backward coefficient
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m_loc = wm + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int m = m0 + m_loc;
+            const bool live = ALIGNED || (m < B && n < T);
+            const float dist = DIST == DIST_L2 ? __builtin_amdgcn_sqrtf(fmaxf(val[r], 0.f)) : val[r];
+            float outv;
+            if (p.out_mode == 2) {
+                outv = dist;
+            } else {
+                const float score = sh.score_fn == SCORE_DISTMULT ? dist : sh.gamma - dist;
+                if (p.out_mode == 1) {
+                    outv = score;
+                    if (live && DIST == DIST_L2 && p.dist) p.dist[((size_t)d * B + m) * T + n] = dist;
+                } else {
+                    const bool pos = (uint32_t)n == label_s[m_loc];
+                    const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
+                    const float z = sign * score;
+                    float lsig, dlsig;
+                    log_sigmoid_both(z, lsig, dlsig);
+                    if (live) loss_acc -= w * lsig;
+                    const float ds = -w * sign * dlsig * inv_norm * sh.loss_scale;
+                    outv = sh.score_fn == SCORE_DISTMULT ? ds : -ds;
+                    if (DIST == DIST_L2) outv = dist != 0.f ? outv * __frcp_rn(dist) : 0.f;
+                }
+            }
+            if (live) p.coef[((size_t)d * B + m) * T + n] = outv;
+        }
+        if (DIST == DIST_L2 && p.nearflag) {
+            // this wave owns the whole 32x32 sub-block: a plain store, no atomics
+            const bool any = __ballot(near != 0u) != 0;
+            const int mt = (m0 + wm + 32 * t) >> 5, nt = (n0 + wn) >> 5;
+            const int MT = (B + 31) >> 5, NT = (T + 31) >> 5;
+            if (lane == 0 && mt < MT && nt < NT) p.nearflag[((size_t)d * MT + mt) * NT + nt] = any ? 1u : 0u;
+        }
+    }
+    if (p.out_mode == 0) {
+        loss_acc = wave_sum(loss_acc);
+        if (lane == 0) red[wave] = loss_acc;
+        __syncthreads();
+        if (tid == 0) {
+            const int n_part = gridDim.x * gridDim.y;
+            p.loss_part[(size_t)d * n_part + blockIdx.y * gridDim.x + blockIdx.x] =
+                (red[0] + red[1] + red[2] + red[3]) * inv_norm;
+        }
+    }
+}
+
+static bool fwd_uses_mfma(const FwdParams& p) {
+    return p.sh.use_mfma && p.sh.dist_fn != DIST_L1 && p.ent_a.vec && p.ent_b.vec && (p.sh.Dp & 3) == 0;
+}
+
 int score_fwd_parts(const ScoreShape& sh) {
-    return ((sh.T + kScoreTile - 1) / kScoreTile) * ((sh.B + kScoreTile - 1) / kScoreTile);
+    const bool mfma = sh.use_mfma && !(sh.score_fn == SCORE_TRANSE && sh.dist_fn == DIST_L1);
+    const int tm = mfma ? FM_TM : kScoreTile, tn = mfma ? FM_TN : kScoreTile;
+    return ((sh.T + tn - 1) / tn) * ((sh.B + tm - 1) / tm);
 }
 
 static void launch_fwd(const FwdParams& p, hipStream_t stream) {
+    if (fwd_uses_mfma(p)) {
+        dim3 grid((p.sh.T + FM_TN - 1) / FM_TN, (p.sh.B + FM_TM - 1) / FM_TM, p.sh.S);
+        const bool f32 = p.ent_a.etype == ET_F32 && p.ent_b.etype == ET_F32;
+        const bool aligned = f32 && p.a_rel_mode == 0 && !p.ent_a.index && !p.ent_b.index &&
+                             p.sh.B % FM_TM == 0 && p.sh.T % FM_TN == 0;
+        // few workgroups: stage 128 columns per iteration so that one workgroup per
+        // CU still overlaps its loads with its matrix work; many: 32, for occupancy
+        const bool wide = aligned && p.sh.Dp % 128 == 0 && (int)(grid.x * grid.y * grid.z) <= 512;
+#define KGE_FWD(D_)                                                                                       \
+    do {                                                                                                  \
+        if (wide) hipLaunchKernelGGL((k_score_fwd_mfma<D_, 128, true>), grid, dim3(256), 0, stream, p);    \
+        else if (aligned && p.sh.Dp % 32 == 0)                                                             \
+            hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true>), grid, dim3(256), 0, stream, p);           \
+        else hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, false>), grid, dim3(256), 0, stream, p);         \
+    } while (0)
+        if (p.sh.dist_fn == DIST_L2) KGE_FWD(DIST_L2); else KGE_FWD(DIST_DOT);
+#undef KGE_FWD
+        return;
+    }
     dim3 grid((p.sh.T + kScoreTile - 1) / kScoreTile, (p.sh.B + kScoreTile - 1) / kScoreTile, p.sh.S);
     if (p.sh.dist_fn == DIST_L1)
         hipLaunchKernelGGL(k_score_fwd<DIST_L1>, grid, dim3(256), 0, stream, p);
@@ -563,13 +916,14 @@ static void launch_fwd(const FwdParams& p, hipStream_t stream) {
 
 void launch_score_fwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
                       const uint32_t* crel, const uint32_t* clabel, float* coef, float* dist,
-                      float* loss_part, bool fused_loss, hipStream_t stream) {
+                      uint32_t* nearflag, float* loss_part, bool fused_loss, hipStream_t stream) {
     FwdParams p;
+    p.nearflag = nearflag;
     p.sh = sh;
     if (sh.score_fn == SCORE_DISTMULT) p.sh.dist_fn = DIST_DOT;
     p.ent_a = ent; p.ent_b = ent; p.rel = rel; p.crel = crel; p.clabel = clabel;
     p.coef = coef; p.dist = dist; p.loss_part = loss_part;
-    p.a_rel_mode = sh.score_fn == SCORE_DISTMULT ? 2 : 1;
+    p.a_rel_mode = sh.operands_dense ? 0 : (sh.score_fn == SCORE_DISTMULT ? 2 : 1);
     p.out_mode = fused_loss ? 0 : 1;
     p.a_c0 = 0; p.b_c0 = sh.S * sh.B;
     launch_fwd(p, stream);
@@ -673,6 +1027,8 @@ struct BwdParams {
     int vec_out;           // output rows allow aligned float4 stores
     int a_rel_mode;        // relation combine of the a-operand
     int a_c0, b_c0;
+    int use_mfma;
+    const uint32_t* nearflag;  // from the forward pass (L2 on the matrix cores), or null
 };
 
 constexpr int BJ = 32;  // rows of `other` staged per iteration
@@ -706,13 +1062,11 @@ __global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
         }
         sv[i][0] = v.x; sv[i][1] = v.y; sv[i][2] = v.z; sv[i][3] = v.w;
     }
-    float acc[4][4], csum[4];
+    float acc[4][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        csum[i] = 0.f;
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int k = 0; k < 4; ++k) acc[i][k] = 0.f;
-    }
 
     for (int j0 = 0; j0 < n_other; j0 += BJ) {
         // coefficient tile -> Cs[j][i]
@@ -792,13 +1146,14 @@ __global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
             const float ov[4] = {o4.x, o4.y, o4.z, o4.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                if (DIST == DIST_L2) csum[i] += cv[i];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     if (DIST == DIST_L1) {
                         const float t = sv[i][k] - ov[k];
                         const float sg = (t > 0.f ? 1.f : 0.f) - (t < 0.f ? 1.f : 0.f);
                         acc[i][k] = fmaf(cv[i], sg, acc[i][k]);
+                    } else if (DIST == DIST_L2) {
+                        acc[i][k] = fmaf(cv[i], sv[i][k] - ov[k], acc[i][k]);
                     } else {
                         acc[i][k] = fmaf(cv[i], ov[k], acc[i][k]);
                     }
@@ -814,8 +1169,7 @@ __global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
         float o[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            if (DIST == DIST_L2) o[k] = sv[i][k] * csum[i] - acc[i][k];
-            else o[k] = acc[i][k];
+            o[k] = acc[i][k];
         }
         float* dst = p.grad + (size_t)(p.grad_c0 + d * n_self + r) * Dp + kcol;
         if (p.vec_out) {
@@ -827,8 +1181,280 @@ __global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
     }
 }
 
+// --------------------------------------------------------------------------
+// scoring backward on the matrix cores (L2 and dot):
+//   out[i,k] = sum_j c[i,j] other[j,k]          (a [I x J] . [J x Dp] product)
+//   L2: out[i,k] = self[i,k] * sum_j c[i,j] - that product
+// Workgroup tile 128 (self rows) x 64 (embedding columns), waves 2 x 2, each
+// wave two 32x32 accumulators; the next chunk of c and `other` is fetched into
+// registers while the matrix cores work on the current one.
+
+constexpr int BM_TI = 128, BM_TK = 64, BM_LDK = BM_TK + 4;
+
+// BJT = rows of `other` staged per iteration (32 or 128, see the forward kernel).
+// ALIGNED: n_self % 128 == 0, n_other % BJT == 0, Dp % 64 == 0, T % 4 == 0,
+// float32 operands without a relation to apply: branch-free staging loads.
+template <int DIST, int SIDE_B, int BJT, bool ALIGNED>
+__global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
+    // head side stores the coefficient tile transposed (scalar stores, odd
+    // pitch); tail side copies float4 along i (16-byte aligned pitch)
+    constexpr int LDI = SIDE_B ? BM_TI + 4 : BM_TI + 1;
+    constexpr int NCH = BJT / 32;  // 32-row sub-chunks per iteration
+    __shared__ __attribute__((aligned(16))) float Cs[BJT][LDI];
+    __shared__ __attribute__((aligned(16))) float Os[BJT][BM_LDK];
+    __shared__ float csum_s[BM_TI];
+    const int d = blockIdx.z, i0 = blockIdx.y * BM_TI, kt0 = blockIdx.x * BM_TK;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wi = (wave >> 1) * 64, wk = (wave & 1) * 32;
+    const int B = p.B, T = p.T, Dp = p.Dp;
+    const int n_self = SIDE_B ? T : B, n_other = SIDE_B ? B : T;
+    const int self_c0 = SIDE_B ? p.b_c0 + d * T : p.a_c0 + d * B;
+    const int other_c0 = SIDE_B ? p.a_c0 + d * B : p.b_c0 + d * T;
+    const int self_rel = SIDE_B ? 0 : p.a_rel_mode, other_rel = SIDE_B ? p.a_rel_mode : 0;
+    const RowSource& self_src = SIDE_B ? p.ent_b : p.ent_a;
+    const RowSource& other_src = SIDE_B ? p.ent_a : p.ent_b;
+    const float* coef = p.coef + (size_t)d * B * T;
+
+    floatx16 acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+    float cs_acc = 0.f;
+    const int kcol = kt0 + wk + (lane & 31);
+
+    // L2: this lane's 2 x 16 `self` values, in accumulator layout
+    float sv[2][16];
+    if (DIST == DIST_L2) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = i0 + wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (ALIGNED) {
+                    sv[t][r] = reinterpret_cast<const float*>(
+                        self_src.base + (int64_t)(self_c0 + i) * self_src.pitch)[kcol];
+                    continue;
+                }
+                float v = 0.f;
+                if (i < n_self && kcol < Dp) {
+                    v = load1(row_ptr(self_src, self_c0 + i), kcol, self_src.etype);
+                    if (self_rel) {
+                        const float rv = p.rel[(size_t)p.crel[d * B + i] * Dp + kcol];
+                        v = self_rel == 1 ? v + rv : v * rv;
+                    }
+                }
+                sv[t][r] = v;
+            }
+    }
+    // near-identical-pair flags of the (self sub-tile, other chunk) blocks
+    const int MT = (B + 31) >> 5, NT = (T + 31) >> 5;
+    const uint32_t* nflag = (DIST == DIST_L2 && p.nearflag) ? p.nearflag + (size_t)d * MT * NT : nullptr;
+    auto flag_of = [&](int i_tile, int j_tile) -> uint32_t {
+        if (!nflag) return 0u;
+        const int mt = SIDE_B ? j_tile : i_tile, nt = SIDE_B ? i_tile : j_tile;
+        if (ALIGNED) return nflag[(size_t)mt * NT + nt];
+        return (mt < MT && nt < NT) ? nflag[(size_t)mt * NT + nt] : 0u;
+    };
+    uint32_t nf_next[NCH][2], nf_row_next[NCH];
+    float4 creg[NCH][4], oreg[NCH][2];
+    auto prefetch = [&](int jbase) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int j0 = jbase + 32 * c;
+            nf_next[c][0] = flag_of((i0 + wi) >> 5, j0 >> 5);
+            nf_next[c][1] = flag_of((i0 + wi + 32) >> 5, j0 >> 5);
+            nf_row_next[c] = flag_of((i0 + (tid & (BM_TI - 1))) >> 5, j0 >> 5);
+            if (ALIGNED) {
+#pragma unroll
+                for (int h = 0; h < 4; ++h) {
+                    const int idx = tid + 256 * h;
+                    const float* src = SIDE_B ? coef + (size_t)(j0 + (idx >> 5)) * T + i0 + (idx & 31) * 4
+                                              : coef + (size_t)(i0 + (idx >> 3)) * T + j0 + (idx & 7) * 4;
+                    creg[c][h] = *reinterpret_cast<const float4*>(src);
+                }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int idx = tid + 256 * h;
+                    oreg[c][h] = *reinterpret_cast<const float4*>(
+                        other_src.base + (int64_t)(other_c0 + j0 + (idx >> 4)) * other_src.pitch +
+                        (size_t)(kt0 + (idx & 15) * 4) * 4);
+                }
+                continue;
+            }
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+                const int idx = tid + 256 * h;
+                creg[c][h] = make_float4(0, 0, 0, 0);
+                if (!SIDE_B) {  // c[i][j] = coef[i0+i][j0+j]: float4 along j
+                    const int gi = i0 + (idx >> 3), gj = j0 + (idx & 7) * 4;
+                    if (gi < B && gj < T) {
+                        const float* src = coef + (size_t)gi * T + gj;
+                        if (gj + 3 < T && (T & 3) == 0) creg[c][h] = *reinterpret_cast<const float4*>(src);
+                        else {
+                            creg[c][h].x = src[0];
+                            if (gj + 1 < T) creg[c][h].y = src[1];
+                            if (gj + 2 < T) creg[c][h].z = src[2];
+                            if (gj + 3 < T) creg[c][h].w = src[3];
+                        }
+                    }
+                } else {        // c[i][j] = coef[j0+j][i0+i]: float4 along i
+                    const int gj = j0 + (idx >> 5), gi = i0 + (idx & 31) * 4;
+                    if (gj < B && gi < T) {
+                        const float* src = coef + (size_t)gj * T + gi;
+                        if (gi + 3 < T && (T & 3) == 0) creg[c][h] = *reinterpret_cast<const float4*>(src);
+                        else {
+                            creg[c][h].x = src[0];
+                            if (gi + 1 < T) creg[c][h].y = src[1];
+                            if (gi + 2 < T) creg[c][h].z = src[2];
+                            if (gi + 3 < T) creg[c][h].w = src[3];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int idx = tid + 256 * h;
+                const int gj = j0 + (idx >> 4), gk = kt0 + (idx & 15) * 4;
+                oreg[c][h] = make_float4(0, 0, 0, 0);
+                if (gj < n_other && gk < Dp) {
+                    oreg[c][h] = load4(row_ptr(other_src, other_c0 + gj), gk, other_src);
+                    if (other_rel)
+                        oreg[c][h] = combine_rel(oreg[c][h], p.rel + (size_t)p.crel[d * B + gj] * Dp, gk, other_rel);
+                }
+            }
+        }
+    };
+    prefetch(0);
+    for (int jbase = 0; jbase < n_other; jbase += BJT) {
+        bool direct0[NCH], direct1[NCH], direct_row[NCH];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            direct0[c] = nf_next[c][0] != 0u; direct1[c] = nf_next[c][1] != 0u; direct_row[c] = nf_row_next[c] != 0u;
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+                const int idx = tid + 256 * h;
+                if (!SIDE_B) {
+                    const int i = idx >> 3, j4 = 32 * c + (idx & 7) * 4;
+                    Cs[j4 + 0][i] = creg[c][h].x; Cs[j4 + 1][i] = creg[c][h].y;
+                    Cs[j4 + 2][i] = creg[c][h].z; Cs[j4 + 3][i] = creg[c][h].w;
+                } else {
+                    *reinterpret_cast<float4*>(&Cs[32 * c + (idx >> 5)][(idx & 31) * 4]) = creg[c][h];
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int idx = tid + 256 * h;
+                *reinterpret_cast<float4*>(&Os[32 * c + (idx >> 4)][(idx & 15) * 4]) = oreg[c][h];
+            }
+        }
+        __syncthreads();
+        if (jbase + BJT < n_other) prefetch(jbase + BJT);
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int jo = 32 * c;
+            if (DIST == DIST_L2 && tid < BM_TI && !direct_row[c]) {
+#pragma unroll
+                for (int jj = 0; jj < 32; ++jj) cs_acc += Cs[jo + jj][tid];
+            }
+            if (!direct0[c] && !direct1[c]) {
+                float ra0[2][4], ra1[2][4], rb[2][4];
+                const int hl = lane >> 5, cl = lane & 31;
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    rb[0][x] = Os[jo + 2 * x + hl][wk + cl];
+                    ra0[0][x] = Cs[jo + 2 * x + hl][wi + cl];
+                    ra1[0][x] = Cs[jo + 2 * x + hl][wi + 32 + cl];
+                }
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    if (g + 1 < 4) {
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) {
+                            const int jj = jo + 8 * (g + 1) + 2 * x + hl;
+                            rb[(g + 1) & 1][x] = Os[jj][wk + cl];
+                            ra0[(g + 1) & 1][x] = Cs[jj][wi + cl];
+                            ra1[(g + 1) & 1][x] = Cs[jj][wi + 32 + cl];
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra0[g & 1][x], rb[g & 1][x], acc[0], 0, 0, 0);
+                        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra1[g & 1][x], rb[g & 1][x], acc[1], 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                // some pair of this block is nearly identical: c * (self - other) directly,
+                // as the reference codelet does (acc holds the negated sum, see the epilogue)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    if (t == 0 ? direct0[c] : direct1[c]) {
+                        for (int jj = jo; jj < jo + 32; ++jj) {
+                            const float o = Os[jj][wk + (lane & 31)];
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                const float cc = Cs[jj][wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
+                                acc[t][r] = fmaf(-cc, sv[t][r] - o, acc[t][r]);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 16; ++q) {
+                            const int jj = jo + 2 * q + (lane >> 5);
+                            const float b = Os[jj][wk + (lane & 31)];
+                            const float a = Cs[jj][wi + 32 * t + (lane & 31)];
+                            acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[t], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (DIST == DIST_L2) {
+        if (tid < BM_TI) csum_s[tid] = cs_acc;
+        __syncthreads();
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i_loc = wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int i = i0 + i_loc;
+            if (i >= n_self || kcol >= Dp) continue;
+            float o = acc[t][r];
+            if (DIST == DIST_L2) o = sv[t][r] * csum_s[i_loc] - o;
+            p.grad[(size_t)(p.grad_c0 + d * n_self + i) * Dp + kcol] = o;
+        }
+}
+
 static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
     const int n_self = p.side_b ? p.T : p.B;
+    const bool mfma_ok = p.use_mfma && !p.coef_div && p.ent_a.vec && p.ent_b.vec && (p.Dp & 3) == 0 &&
+                         (dist_fn == DIST_DOT || (dist_fn == DIST_L2 && p.nearflag));
+    if (mfma_ok) {
+        dim3 grid((p.Dp + BM_TK - 1) / BM_TK, (n_self + BM_TI - 1) / BM_TI, p.S);
+        const int n_other = p.side_b ? p.B : p.T;
+        const bool plain = p.ent_a.etype == ET_F32 && p.ent_b.etype == ET_F32 && !p.ent_a.index &&
+                           !p.ent_b.index && p.a_rel_mode == 0;
+        const bool aligned = plain && n_self % BM_TI == 0 && p.Dp % BM_TK == 0 && p.T % 4 == 0 && n_other % 32 == 0;
+        const bool wide = aligned && n_other % 128 == 0 && (int)(grid.x * grid.y * grid.z) <= 512;
+#define KGE_BWD(D_, S_)                                                                                     \
+    do {                                                                                                    \
+        if (wide) hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 128, true>), grid, dim3(256), 0, stream, p);  \
+        else if (aligned) hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 32, true>), grid, dim3(256), 0, stream, p); \
+        else hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 32, false>), grid, dim3(256), 0, stream, p);       \
+    } while (0)
+        if (dist_fn == DIST_L2) {
+            if (p.side_b) KGE_BWD(DIST_L2, 1); else KGE_BWD(DIST_L2, 0);
+        } else {
+            if (p.side_b) KGE_BWD(DIST_DOT, 1); else KGE_BWD(DIST_DOT, 0);
+        }
+#undef KGE_BWD
+        return;
+    }
     dim3 grid((p.Dp + kScoreTile - 1) / kScoreTile, (n_self + kScoreTile - 1) / kScoreTile, p.S);
     if (dist_fn == DIST_L1)
         hipLaunchKernelGGL(k_score_bwd<DIST_L1>, grid, dim3(256), 0, stream, p);
@@ -839,12 +1465,14 @@ static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
 }
 
 void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
-                      const uint32_t* crel, const float* coef, float* grad, hipStream_t stream) {
+                      const uint32_t* crel, const float* coef, const uint32_t* nearflag, float* grad,
+                      hipStream_t stream) {
     BwdParams p;
     p.ent_a = ent; p.ent_b = ent; p.rel = rel; p.crel = crel; p.coef = coef; p.grad = grad;
     p.coef_div = nullptr;
-    p.S = sh.S; p.B = sh.B; p.T = sh.T; p.Dp = sh.Dp; p.vec_out = 1;
-    p.a_rel_mode = sh.score_fn == SCORE_DISTMULT ? 2 : 1;
+    p.S = sh.S; p.B = sh.B; p.T = sh.T; p.Dp = sh.Dp; p.vec_out = 1; p.use_mfma = sh.use_mfma;
+    p.nearflag = nearflag;
+    p.a_rel_mode = sh.operands_dense ? 0 : (sh.score_fn == SCORE_DISTMULT ? 2 : 1);
     p.a_c0 = 0; p.b_c0 = sh.S * sh.B;
     const int dist_fn = sh.score_fn == SCORE_DISTMULT ? DIST_DOT : sh.dist_fn;
     p.side_b = 0; p.grad_c0 = p.a_c0;
@@ -856,40 +1484,85 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
 // --------------------------------------------------------------------------
 // segmented reduction + Adam
 
-__global__ __launch_bounds__(256) void k_reduce_chunks(ReduceArgs a) {
-    const int lane = threadIdx.x & 63;
-    const int q = blockIdx.x * 4 + (threadIdx.x >> 6);
+// One gradient contribution (row c of the contribution-gradient matrix), four
+// columns from k, with the DistMult product rule applied on load.
+DEVINL float4 load_contrib(const ContribSrc& cs, uint32_t c, int k, int Dp) {
+    float4 g = *reinterpret_cast<const float4*>(cs.grad + (size_t)c * Dp + k);
+    if (cs.transform == 1) {
+        if (c < (uint32_t)cs.n_head)
+            g = f4mul(g, *reinterpret_cast<const float4*>(cs.rel + (size_t)cs.crel[c] * Dp + k));
+    } else if (cs.transform == 2) {
+        g = f4mul(g, load4(row_ptr(cs.ent, c), k, cs.ent));
+    }
+    return g;
+}
+
+// Ordered sum of the contributions at sorted positions [pos, pos + n), columns
+// k..k+3: eight independent row loads in flight, added in position order.
+// Must be called by every lane of the wave (the item indices travel by
+// shuffle); lanes with `active` false load nothing and return zero.
+DEVINL float4 sum_contribs(const ContribSrc& cs, uint32_t pos, uint32_t n, int k, int Dp, int lane,
+                           bool active) {
+    float4 acc = make_float4(0, 0, 0, 0);
+    for (uint32_t j = 0; j < n; j += 8) {
+        const uint32_t mine = (j + (lane & 7) < n) ? cs.sorted_item[pos + j + (lane & 7)] : 0u;
+        float4 v[8];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            const uint32_t c = __shfl(mine, x, 64);
+            v[x] = (active && j + x < n) ? load_contrib(cs, c, k, Dp) : make_float4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int x = 0; x < 8; ++x) acc = f4add(acc, v[x]);
+    }
+    return acc;
+}
+
+// First level for rows with many contributions: one workgroup per chunk, each
+// wave sums a quarter of the chunk, the four quarters are added in wave order.
+__global__ __launch_bounds__(256) void k_reduce_chunks(ReduceArgs a0, ReduceArgs a1) {
+    __shared__ __attribute__((aligned(16))) float part[3][256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // two reductions share the launch: blocks [0, a0.max_chunks) serve the first
+    const bool second = (int)blockIdx.x >= a0.max_chunks;
+    const ReduceArgs& a = second ? a1 : a0;
+    const int q = second ? blockIdx.x - a0.max_chunks : blockIdx.x;
     if (q >= (int)a.counts[1]) return;
     const uint32_t pos = a.chunk_pos[q], len = a.chunk_len[q];
     const int Dp = a.Dp;
-    if (Dp & 3) {  // unaligned rows (standalone scatter-add on arbitrary widths)
-        for (int k = lane; k < Dp; k += 64) {
-            float acc = 0.f;
-            for (uint32_t j = 0; j < len; ++j)
-                acc += a.grad[(size_t)a.sorted_item[pos + j] * Dp + k];
-            a.partial[(size_t)q * Dp + k] = acc;
-        }
+    if (Dp & 3) {  // unaligned rows (stand-alone scatter-add on arbitrary widths): wave 0 only
+        if (wave == 0)
+            for (int k = lane; k < Dp; k += 64) {
+                float acc = 0.f;
+                for (uint32_t j = 0; j < len; ++j)
+                    acc += a.src.grad[(size_t)a.src.sorted_item[pos + j] * Dp + k];
+                a.partial[(size_t)q * Dp + k] = acc;
+            }
         return;
     }
-    for (int k = lane * 4; k < Dp; k += 256) {
-        float4 acc = make_float4(0, 0, 0, 0);
-        for (uint32_t j = 0; j < len; ++j) {
-            const uint32_t c = a.sorted_item[pos + j];
-            float4 g = *reinterpret_cast<const float4*>(a.grad + (size_t)c * Dp + k);
-            if (a.transform == 1) {
-                if (c < (uint32_t)a.n_head)
-                    g = f4mul(g, *reinterpret_cast<const float4*>(a.rel + (size_t)a.crel[c] * Dp + k));
-            } else if (a.transform == 2) {
-                g = f4mul(g, load4(row_ptr(a.ent, c), k, a.ent));
-            }
-            acc = f4add(acc, g);
+    const uint32_t quarter = (len + 3) / 4;
+    const uint32_t w0 = min(len, wave * quarter), w1 = min(len, w0 + quarter);
+    for (int k0 = 0; k0 < Dp; k0 += 256) {
+        const int k = k0 + lane * 4;
+        float4 acc = sum_contribs(a.src, pos + w0, w1 - w0, k, Dp, lane, k < Dp);
+        if (wave > 0) *reinterpret_cast<float4*>(&part[wave - 1][lane * 4]) = acc;
+        __syncthreads();
+        if (wave == 0 && k < Dp) {
+#pragma unroll
+            for (int w = 0; w < 3; ++w) acc = f4add(acc, *reinterpret_cast<const float4*>(&part[w][lane * 4]));
+            *reinterpret_cast<float4*>(a.partial + (size_t)q * Dp + k) = acc;
         }
-        *reinterpret_cast<float4*>(a.partial + (size_t)q * Dp + k) = acc;
+        __syncthreads();
     }
 }
 
 void launch_reduce_chunks(const ReduceArgs& a, hipStream_t stream) {
-    hipLaunchKernelGGL(k_reduce_chunks, dim3((a.max_chunks + 3) / 4), dim3(256), 0, stream, a);
+    ReduceArgs none = a;
+    none.max_chunks = 0;
+    hipLaunchKernelGGL(k_reduce_chunks, dim3(a.max_chunks), dim3(256), 0, stream, a, none);
+}
+void launch_reduce_chunks2(const ReduceArgs& a0, const ReduceArgs& a1, hipStream_t stream) {
+    hipLaunchKernelGGL(k_reduce_chunks, dim3(a0.max_chunks + a1.max_chunks), dim3(256), 0, stream, a0, a1);
 }
 
 // fr::nn::adam (src/fructose/frnn.cpp:74-89) on one float4
@@ -907,30 +1580,52 @@ DEVINL void adam4(float4& p, float4& m, float4& v, float4 g, const AdamArgs& a, 
     }
 }
 
-__global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a) {
+// One wave per distinct row: gather its gradient (directly from its few
+// contributions, or from its chunk partials), Adam, write the row back.
+__global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
     const int lane = threadIdx.x & 63;
-    const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
+    // two tables share the launch: blocks [0, ceil(a0.max_rows / 4)) serve the first
+    const int blocks0 = (a0.max_rows + 3) / 4;
+    const bool second = (int)blockIdx.x >= blocks0;
+    const AdamArgs& a = second ? a1 : a0;
+    const int u = (second ? blockIdx.x - blocks0 : blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (u >= (int)a.counts[0]) return;
     const uint32_t key = a.uniq_key[u];
     const float alpha = a.alpha[a.rows_per_alpha ? key / a.rows_per_alpha : 0u];
     const int Dp = a.Dp;
-    uint32_t q0 = 0, q1 = 0;
-    if (a.partial) { q0 = a.chunk_off[u]; q1 = a.chunk_off[u + 1]; }
+    uint32_t q0 = 0, q1 = 0, pos = 0, n_real = 0;
+    if (!a.grad_direct) {
+        q0 = a.chunk_off[u]; q1 = a.chunk_off[u + 1];
+        pos = a.seg_start[u]; n_real = a.seg_real[u];
+    }
     char* prow = a.p_base + (int64_t)key * a.pitch;
     char* mrow = a.m_base + (int64_t)key * a.pitch;
     char* vrow = a.v_base + (int64_t)key * a.pitch;
-    for (int k = lane * 4; k < Dp; k += 256) {
+    for (int k0 = 0; k0 < Dp; k0 += 256) {
+        const int k = k0 + lane * 4;
+        const bool active = k < Dp;
         float4 g = make_float4(0, 0, 0, 0);
-        if (a.grad_direct) {
-            g = *reinterpret_cast<const float4*>(a.grad_direct + (size_t)u * Dp + k);
-        } else {
-            for (uint32_t q = q0; q < q1; ++q)
-                g = f4add(g, *reinterpret_cast<const float4*>(a.partial + (size_t)q * Dp + k));
-        }
-        if (a.grad_out) *reinterpret_cast<float4*>(a.grad_out + (size_t)u * Dp + k) = g;
+        if (!a.grad_direct && q1 == q0 && n_real)  // wave-uniform: all lanes take part in the shuffles
+            g = sum_contribs(a.src, pos, n_real, k, Dp, lane, active);
+        if (!active) continue;
         float4 p = load4(prow, k, a.p_etype);
         float4 m = *reinterpret_cast<const float4*>(mrow + (size_t)k * 4);
         float4 v = *reinterpret_cast<const float4*>(vrow + (size_t)k * 4);
+        if (a.grad_direct) {
+            g = *reinterpret_cast<const float4*>(a.grad_direct + (size_t)u * Dp + k);
+        } else if (q1 > q0) {
+            for (uint32_t q = q0; q < q1; q += 8) {
+                float4 t[8];
+#pragma unroll
+                for (int x = 0; x < 8; ++x)
+                    t[x] = (q + x < q1) ? *reinterpret_cast<const float4*>(a.partial + (size_t)(q + x) * Dp + k)
+                                        : make_float4(0, 0, 0, 0);
+#pragma unroll
+                for (int x = 0; x < 8; ++x) g = f4add(g, t[x]);
+            }
+        }
+        if (a.grad_out) *reinterpret_cast<float4*>(a.grad_out + (size_t)u * Dp + k) = g;
+        if (a.no_update) continue;
         adam4(p, m, v, g, a, alpha);
         store4(prow, k, a.p_etype, p);
         *reinterpret_cast<float4*>(mrow + (size_t)k * 4) = m;
@@ -939,7 +1634,13 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a) {
 }
 
 void launch_adam_rows(const AdamArgs& a, hipStream_t stream) {
-    hipLaunchKernelGGL(k_adam_rows, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a);
+    AdamArgs none = a;
+    none.max_rows = 0;
+    hipLaunchKernelGGL(k_adam_rows, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, none);
+}
+void launch_adam_rows2(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream) {
+    hipLaunchKernelGGL(k_adam_rows, dim3((a0.max_rows + 3) / 4 + (a1.max_rows + 3) / 4), dim3(256), 0,
+                       stream, a0, a1);
 }
 
 __global__ __launch_bounds__(64) void k_loss_finalize(const float* __restrict__ loss_part, int n_step,
@@ -1169,11 +1870,12 @@ void launch_distance(int dist_fn, const float* a, const float* b, float* out, in
     p.sh.score_fn = SCORE_TRANSE; p.sh.dist_fn = dist_fn; p.sh.loss_fn = LOSS_LOGSIGMOID;
     p.sh.gamma = 0.f; p.sh.loss_scale = 1.f; p.sh.softmax_correction = 0.f;
     p.sh.negative_adversarial_scale = 0.f;
+    p.sh.use_mfma = 1; p.sh.operands_dense = 0;
     p.ent_a = plain_rows(a, D); p.ent_b = plain_rows(b, D);
     p.rel = nullptr; p.crel = nullptr; p.clabel = nullptr;
     p.coef = out; p.dist = nullptr; p.loss_part = nullptr;
     p.a_rel_mode = 0; p.out_mode = 2;
-    p.a_c0 = 0; p.b_c0 = 0;
+    p.a_c0 = 0; p.b_c0 = 0; p.nearflag = nullptr;
     launch_fwd(p, stream);
 }
 
@@ -1188,7 +1890,7 @@ void launch_distance_grad(int dist_fn, const float* a, const float* b, const flo
     p.grad = grad;
     p.S = 1; p.B = M; p.T = N; p.Dp = D;
     p.side_b = 0; p.a_rel_mode = 0;
-    p.a_c0 = 0; p.b_c0 = 0; p.grad_c0 = 0;
+    p.a_c0 = 0; p.b_c0 = 0; p.grad_c0 = 0; p.use_mfma = 1; p.nearflag = nullptr;
     p.vec_out = (D % 4 == 0) && ((uintptr_t)grad % 16 == 0);
     launch_bwd(p, dist_fn, stream);
 }

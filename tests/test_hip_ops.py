@@ -122,6 +122,25 @@ def test_distance_vs_oracle(oracle64, kind, shape):
     assert K.rel_l2(gb, gb_ref) < 1e-5
 
 
+def test_l2_distance_near_duplicates(oracle64):
+    """Rows that nearly coincide: |a|^2 + |b|^2 - 2ab would lose every digit;
+    the result must still be within 1e-5 relative, and exactly 0 for equal rows."""
+    rng = np.random.default_rng(9)
+    M, N, D = 200, 150, 256
+    a = rng.normal(size=(M, D)).astype(np.float32)
+    b = rng.normal(size=(N, D)).astype(np.float32)
+    for j, scale in enumerate([0.0, 1e-6, 1e-4, 1e-3, 1e-2, 0.1, 0.3, 0.5]):
+        b[j::8][:M // 8 + 1] = (a[j::8][:N // 8 + 1][:len(b[j::8])] *
+                                (1 + scale * rng.normal(size=(len(b[j::8]), D)))).astype(np.float32)[:len(b[j::8])]
+    out = _distance("kge_l2_distance", a, b)
+    ref = oracle64.l2_distance(a, b)
+    np.testing.assert_allclose(out, ref, rtol=1e-5, atol=0)
+    assert np.all(out[ref == 0] == 0) and np.any(ref == 0)
+    g = rng.normal(size=(M, N)).astype(np.float32)
+    ga, ga_ref = _distance_grad("l2", a, b, g, out), oracle64.l2_distance_grad(a, b, out, g)
+    assert K.rel_l2(ga, ga_ref) < 1e-5
+
+
 def test_buffer_kat():
     # tests/fructose/testFructose.cpp:121-139
     buf = torch.zeros(3, 4, device="cuda")

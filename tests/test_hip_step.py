@@ -35,7 +35,8 @@ CASES = {
 }
 
 
-def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_loop=1, warm=True):
+def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_loop=1, warm=True,
+             **settings):
     import libpoplar_kge
 
     c = K.cfg_dict(**kw)
@@ -44,7 +45,7 @@ def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_lo
     lr = np.resize(np.asarray(lr, np.float32), c["n_shard"])
     if c["shared_table"]:
         lr[:] = lr[0]
-    engine = libpoplar_kge.Engine(H.engine_settings(c, n_step), "")
+    engine = libpoplar_kge.Engine(H.engine_settings(c, n_step, **settings), "")
     H.load_state(engine, c, st0)
     # the state round-trips bit-exactly through write_entity_raw / read_entity
     rt = H.read_state(engine, c)
@@ -74,6 +75,39 @@ def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_lo
 @pytest.mark.parametrize("name", list(CASES))
 def test_step_vs_oracle(oracle64, name):
     run_case(oracle64, CASES[name])
+
+
+@pytest.mark.parametrize("name", ["l2_logsigmoid", "l2_softmax", "distmult_softmax_feat", "mid_l2",
+                                  "transe_matmul", "shared_l2"])
+def test_step_vs_oracle_valu_scoring(oracle64, name):
+    # the same cases on the VALU scoring kernels (default: matrix cores)
+    run_case(oracle64, CASES[name], **{"execution.scoring": "valu"})
+
+
+def test_step_near_duplicate_rows(oracle64):
+    # head + relation almost equal to some tails: the L2 forward must not cancel
+    import libpoplar_kge
+
+    c = K.cfg_dict(distance_fn="L2", feature=0, gamma=1.0, n_shard=2, batch=40, a2a=30, dim=64,
+                   n_entity=400, n_relation=4)
+    rng = np.random.default_rng(3)
+    st0 = K.make_state(c, rng)
+    D = c["dim"]
+    st0["relation_embedding"] *= 1e-3
+    base = st0["entity_data"][1, :D].copy()
+    for r in range(2, st0["entity_data"].shape[0], 3):  # a third of the rows cluster tightly
+        st0["entity_data"][r, :D] = base * (1 + 1e-3 * rng.normal(size=D))
+    st0["entity_data"][5, :D] = st0["entity_data"][8, :D]  # and two are identical
+    batch = K.random_batch(c, 2, rng)
+    engine = libpoplar_kge.Engine(H.engine_settings(c, 2), "")
+    H.load_state(engine, c, st0)
+    st_o = K.copy_state(st0)
+    loss_o = oracle64.train_step_loop(make_cfg(**c), st_o, 0.05, batch)
+    loss_h = H.train(engine, c, 0.05, batch)
+    np.testing.assert_allclose(loss_h, loss_o, rtol=1e-5)
+    st_h = H.read_state(engine, c)
+    for k in ("entity_data", "relation_embedding"):
+        assert K.rel_l2(st_h[k] - st0[k], st_o[k] - st0[k]) < 1e-4, k
 
 
 def test_step_padding_rows(oracle64):
