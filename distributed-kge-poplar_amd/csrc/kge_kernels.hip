@@ -615,7 +615,7 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int FM_TM = 128, FM_TN = 64, FM_LDA = FM_TM + 1, FM_LDB = FM_TN + 1;
+constexpr int FM_TM = 128, FM_TN = 64;
 constexpr float kCancelRatio = 0.125f;  // recompute when d^2 < ratio * (|a|^2 + |b|^2)
 // Below this ratio the backward's product form self*sum(c) - sum(c*other) would
 // lose accuracy against the reference's c*(self-other); such 32x32 sub-blocks
@@ -624,35 +624,45 @@ constexpr float kNearRatio = 1.f / 4096.f;
 
 // BKT = embedding columns staged per iteration: with 128 a whole D = 256 row
 // takes two iterations, the loads of the second in flight under the first's
-// matrix work (one workgroup per CU, 99 KB of LDS).
-// ALIGNED: B % 128 == 0, T % 64 == 0, Dp % BKT == 0, float32 operands with the
-// relation already applied: the
-// staging loads carry no bounds checks (and so no branches that would force
-// the prefetch to complete before the matrix work starts).
-template <int DIST, int BKT, bool ALIGNED>
-__global__ __launch_bounds__(256) void k_score_fwd_mfma(FwdParams p) {
-    constexpr int NC = BKT / 32;  // float4 columns per staged row per thread
-    __shared__ float As[BKT][FM_LDA];
-    __shared__ float Bs[BKT][FM_LDB];
+// matrix work (99 KB of LDS).  NW = waves per workgroup: 8 (two per SIMD, each
+// one 32x32 accumulator) when a launch has so few workgroups that each CU gets
+// one, so that a second wave hides the other's LDS and epilogue latencies; 4
+// (each two accumulators) otherwise.
+// ALIGNED: B % 128 == 0, T % 64 == 0, Dp % BKT == 0, dense float32 operands with
+// the relation already applied: the staging loads carry no bounds checks (and
+// so no branches that would force the prefetch to complete before the matrix
+// work starts).
+template <int DIST, int BKT, bool ALIGNED, int NW>
+__global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
+    constexpr int NT = NW * 64;       // threads
+    constexpr int AT = 8 / NW;        // 32-row accumulator tiles per wave (NW/2 waves cover 128 rows)
+    constexpr int RP = NT / 8;        // rows staged per pass (8 threads share a row)
+    constexpr int HA = FM_TM / RP, HB = FM_TN / RP;
+    constexpr int NC = BKT / 32;      // float4 columns per staged row per thread
+    // tiles keep the operands' own layout (row = entity row, columns contiguous):
+    // staging is a float4 copy, and a lane fetches four consecutive columns of
+    // its row in one 16-byte LDS read that feeds four matrix instructions.  The
+    // pitch of BKT + 4 floats spreads eight consecutive rows over all banks.
+    constexpr int LDT = BKT + 4;
+    __shared__ __attribute__((aligned(16))) float As[FM_TM][LDT];
+    __shared__ __attribute__((aligned(16))) float Bs[FM_TN][LDT];
     __shared__ float na_s[FM_TM], nb_s[FM_TN];
-    __shared__ float red[4];
+    __shared__ float red[NW];
     __shared__ uint32_t label_s[FM_TM];
     const ScoreShape& sh = p.sh;
     const int d = blockIdx.z, m0 = blockIdx.y * FM_TM, n0 = blockIdx.x * FM_TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 32;
+    const int wm = (wave >> 1) * (32 * AT), wn = (wave & 1) * 32;
     const int B = sh.B, T = sh.T, Dp = sh.Dp;
     if (p.out_mode == 0 && tid < FM_TM) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
 
-    // staging: a tile = 128 rows x 32 columns = 1024 float4 (4 per thread),
-    // b tile = 64 x 32 = 512 float4 (2 per thread); 8 consecutive threads share a row
     const int srow = tid >> 3, k4 = (tid & 7) * 4;
-    const char* arow[4];
-    const float* rrow[4];
-    const char* brow[2];
+    const char* arow[HA];
+    const float* rrow[HA];
+    const char* brow[HB];
 #pragma unroll
-    for (int h = 0; h < 4; ++h) {
-        const int m = m0 + srow + 32 * h;
+    for (int h = 0; h < HA; ++h) {
+        const int m = m0 + srow + RP * h;
         if (ALIGNED) {  // dense, un-indexed operands: plain address arithmetic
             arow[h] = p.ent_a.base + (int64_t)(p.a_c0 + d * B + m) * p.ent_a.pitch;
             rrow[h] = nullptr;
@@ -662,38 +672,42 @@ __global__ __launch_bounds__(256) void k_score_fwd_mfma(FwdParams p) {
         }
     }
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int n = n0 + srow + 32 * h;
+    for (int h = 0; h < HB; ++h) {
+        const int n = n0 + srow + RP * h;
         if (ALIGNED) brow[h] = p.ent_b.base + (int64_t)(p.b_c0 + d * T + n) * p.ent_b.pitch;
         else brow[h] = n < T ? row_ptr(p.ent_b, p.b_c0 + d * T + n) : nullptr;
     }
-    float na_acc[4] = {0.f, 0.f, 0.f, 0.f}, nb_acc[2] = {0.f, 0.f};
-    floatx16 acc[2];
+    float na_acc[HA], nb_acc[HB];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int h = 0; h < HA; ++h) na_acc[h] = 0.f;
+#pragma unroll
+    for (int h = 0; h < HB; ++h) nb_acc[h] = 0.f;
+    floatx16 acc[AT];
+#pragma unroll
+    for (int t = 0; t < AT; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
 
-    float4 areg[4][NC], breg[2][NC];
+    float4 areg[HA][NC], breg[HB][NC];
     auto prefetch = [&](int k0) {
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int k = k0 + 32 * c + k4;
             if (ALIGNED) {
 #pragma unroll
-                for (int h = 0; h < 4; ++h) areg[h][c] = *reinterpret_cast<const float4*>(arow[h] + (size_t)k * 4);
+                for (int h = 0; h < HA; ++h) areg[h][c] = *reinterpret_cast<const float4*>(arow[h] + (size_t)k * 4);
 #pragma unroll
-                for (int h = 0; h < 2; ++h) breg[h][c] = *reinterpret_cast<const float4*>(brow[h] + (size_t)k * 4);
+                for (int h = 0; h < HB; ++h) breg[h][c] = *reinterpret_cast<const float4*>(brow[h] + (size_t)k * 4);
                 continue;
             }
 #pragma unroll
-            for (int h = 0; h < 4; ++h) {
+            for (int h = 0; h < HA; ++h) {
                 areg[h][c] = make_float4(0, 0, 0, 0);
                 if (arow[h] && k < Dp)
                     areg[h][c] = combine_rel(load4(arow[h], k, p.ent_a), rrow[h], k, p.a_rel_mode);
             }
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            for (int h = 0; h < HB; ++h) {
                 breg[h][c] = make_float4(0, 0, 0, 0);
                 if (brow[h] && k < Dp) breg[h][c] = load4(brow[h], k, p.ent_b);
             }
@@ -705,50 +719,47 @@ __global__ __launch_bounds__(256) void k_score_fwd_mfma(FwdParams p) {
         for (int c = 0; c < NC; ++c) {
             const int kc = 32 * c + k4;
 #pragma unroll
-            for (int h = 0; h < 4; ++h) {
+            for (int h = 0; h < HA; ++h) {
                 const float4 a = areg[h][c];
-                const int r = srow + 32 * h;
-                As[kc + 0][r] = a.x; As[kc + 1][r] = a.y; As[kc + 2][r] = a.z; As[kc + 3][r] = a.w;
+                *reinterpret_cast<float4*>(&As[srow + RP * h][kc]) = a;
                 if (DIST == DIST_L2) na_acc[h] += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
             }
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            for (int h = 0; h < HB; ++h) {
                 const float4 b = breg[h][c];
-                const int r = srow + 32 * h;
-                Bs[kc + 0][r] = b.x; Bs[kc + 1][r] = b.y; Bs[kc + 2][r] = b.z; Bs[kc + 3][r] = b.w;
+                *reinterpret_cast<float4*>(&Bs[srow + RP * h][kc]) = b;
                 if (DIST == DIST_L2) nb_acc[h] += b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
             }
         }
         __syncthreads();
         if (k0 + BKT < Dp) prefetch(k0 + BKT);
-        // operands of four k-pairs at a time, fetched from LDS one group ahead of
-        // the matrix instructions that consume them
+        // Each group of four matrix instructions covers eight columns: instruction
+        // x takes column 8g + x from the lower half-wave and 8g + 4 + x from the
+        // upper one.  Operands are fetched one group ahead of their use.
         {
             constexpr int NG = BKT / 8;
-            float ra0[2][4], ra1[2][4], rb[2][4];
+            float4 ra[2][AT], rb[2];
             const int hl = lane >> 5, cl = lane & 31;
+            rb[0] = *reinterpret_cast<const float4*>(&Bs[wn + cl][4 * hl]);
 #pragma unroll
-            for (int x = 0; x < 4; ++x) {
-                rb[0][x] = Bs[2 * x + hl][wn + cl];
-                ra0[0][x] = As[2 * x + hl][wm + cl];
-                ra1[0][x] = As[2 * x + hl][wm + 32 + cl];
-            }
+            for (int t = 0; t < AT; ++t) ra[0][t] = *reinterpret_cast<const float4*>(&As[wm + 32 * t + cl][4 * hl]);
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
                 if (g + 1 < NG) {
+                    rb[(g + 1) & 1] = *reinterpret_cast<const float4*>(&Bs[wn + cl][8 * (g + 1) + 4 * hl]);
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        const int kk = 8 * (g + 1) + 2 * x + hl;
-                        rb[(g + 1) & 1][x] = Bs[kk][wn + cl];
-                        ra0[(g + 1) & 1][x] = As[kk][wm + cl];
-                        ra1[(g + 1) & 1][x] = As[kk][wm + 32 + cl];
-                    }
+                    for (int t = 0; t < AT; ++t)
+                        ra[(g + 1) & 1][t] =
+                            *reinterpret_cast<const float4*>(&As[wm + 32 * t + cl][8 * (g + 1) + 4 * hl]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
+                const float bx[4] = {rb[g & 1].x, rb[g & 1].y, rb[g & 1].z, rb[g & 1].w};
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra0[g & 1][x], rb[g & 1][x], acc[0], 0, 0, 0);
-                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra1[g & 1][x], rb[g & 1][x], acc[1], 0, 0, 0);
+                for (int t = 0; t < AT; ++t) {
+                    const float ax[4] = {ra[g & 1][t].x, ra[g & 1][t].y, ra[g & 1][t].z, ra[g & 1][t].w};
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+                        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(ax[x], bx[x], acc[t], 0, 0, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -758,16 +769,16 @@ __global__ __launch_bounds__(256) void k_score_fwd_mfma(FwdParams p) {
     if (DIST == DIST_L2) {
         // the 8 threads of a row hold partial sums of squares: combine in a fixed order
 #pragma unroll
-        for (int h = 0; h < 4; ++h) {
+        for (int h = 0; h < HA; ++h) {
             float v = na_acc[h];
             v += __shfl_xor(v, 1, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 4, 64);
-            if ((tid & 7) == 0) na_s[srow + 32 * h] = v;
+            if ((tid & 7) == 0) na_s[srow + RP * h] = v;
         }
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int h = 0; h < HB; ++h) {
             float v = nb_acc[h];
             v += __shfl_xor(v, 1, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 4, 64);
-            if ((tid & 7) == 0) nb_s[srow + 32 * h] = v;
+            if ((tid & 7) == 0) nb_s[srow + RP * h] = v;
         }
         __syncthreads();
     }
@@ -781,7 +792,7 @@ __global__ __launch_bounds__(256) void k_score_fwd_mfma(FwdParams p) {
     const int n_loc = wn + (lane & 31), n = n0 + n_loc;
     const float nb = DIST == DIST_L2 ? nb_s[n_loc] : 0.f;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < AT; ++t) {
         // phase 1 (straight-line): squared distances and which of them cancelled
         float val[16];
         uint32_t cancel = 0u, near = 0u;
@@ -859,8 +870,8 @@ __global__ __launch_bounds__(256) void k_score_fwd_mfma(FwdParams p) {
             // this wave owns the whole 32x32 sub-block: a plain store, no atomics
             const bool any = __ballot(near != 0u) != 0;
             const int mt = (m0 + wm + 32 * t) >> 5, nt = (n0 + wn) >> 5;
-            const int MT = (B + 31) >> 5, NT = (T + 31) >> 5;
-            if (lane == 0 && mt < MT && nt < NT) p.nearflag[((size_t)d * MT + mt) * NT + nt] = any ? 1u : 0u;
+            const int MT = (B + 31) >> 5, NTL = (T + 31) >> 5;
+            if (lane == 0 && mt < MT && nt < NTL) p.nearflag[((size_t)d * MT + mt) * NTL + nt] = any ? 1u : 0u;
         }
     }
     if (p.out_mode == 0) {
@@ -869,8 +880,10 @@ __global__ __launch_bounds__(256) void k_score_fwd_mfma(FwdParams p) {
         __syncthreads();
         if (tid == 0) {
             const int n_part = gridDim.x * gridDim.y;
-            p.loss_part[(size_t)d * n_part + blockIdx.y * gridDim.x + blockIdx.x] =
-                (red[0] + red[1] + red[2] + red[3]) * inv_norm;
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) tot += red[w];
+            p.loss_part[(size_t)d * n_part + blockIdx.y * gridDim.x + blockIdx.x] = tot * inv_norm;
         }
     }
 }
@@ -891,15 +904,11 @@ static void launch_fwd(const FwdParams& p, hipStream_t stream) {
         const bool f32 = p.ent_a.etype == ET_F32 && p.ent_b.etype == ET_F32;
         const bool aligned = f32 && p.a_rel_mode == 0 && !p.ent_a.index && !p.ent_b.index &&
                              p.sh.B % FM_TM == 0 && p.sh.T % FM_TN == 0;
-        // few workgroups: stage 128 columns per iteration so that one workgroup per
-        // CU still overlaps its loads with its matrix work; many: 32, for occupancy
-        const bool wide = aligned && p.sh.Dp % 128 == 0 && (int)(grid.x * grid.y * grid.z) <= 512;
-#define KGE_FWD(D_)                                                                                       \
-    do {                                                                                                  \
-        if (wide) hipLaunchKernelGGL((k_score_fwd_mfma<D_, 128, true>), grid, dim3(256), 0, stream, p);    \
-        else if (aligned && p.sh.Dp % 32 == 0)                                                             \
-            hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true>), grid, dim3(256), 0, stream, p);           \
-        else hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, false>), grid, dim3(256), 0, stream, p);         \
+#define KGE_FWD(D_)                                                                                          \
+    do {                                                                                                     \
+        if (aligned && p.sh.Dp % 32 == 0) /* eight waves: two per SIMD hide each other's latencies */   \
+            hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true, 8>), grid, dim3(512), 0, stream, p);           \
+        else hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, false, 4>), grid, dim3(256), 0, stream, p);         \
     } while (0)
         if (p.sh.dist_fn == DIST_L2) KGE_FWD(DIST_L2); else KGE_FWD(DIST_DOT);
 #undef KGE_FWD
@@ -1191,23 +1200,32 @@ __global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
 
 constexpr int BM_TI = 128, BM_TK = 64, BM_LDK = BM_TK + 4;
 
-// BJT = rows of `other` staged per iteration (32 or 128, see the forward kernel).
+// BJT = rows of `other` staged per iteration (32 or 128) and NW = waves per
+// workgroup (4 or 8), chosen as in the forward kernel.
 // ALIGNED: n_self % 128 == 0, n_other % BJT == 0, Dp % 64 == 0, T % 4 == 0,
-// float32 operands without a relation to apply: branch-free staging loads.
-template <int DIST, int SIDE_B, int BJT, bool ALIGNED>
-__global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
-    // head side stores the coefficient tile transposed (scalar stores, odd
-    // pitch); tail side copies float4 along i (16-byte aligned pitch)
-    constexpr int LDI = SIDE_B ? BM_TI + 4 : BM_TI + 1;
-    constexpr int NCH = BJT / 32;  // 32-row sub-chunks per iteration
-    __shared__ __attribute__((aligned(16))) float Cs[BJT][LDI];
+// dense float32 operands without a relation to apply: branch-free staging loads.
+template <int DIST, int SIDE_B, int BJT, bool ALIGNED, int NW>
+DEVINL void bwd_mfma_body(const BwdParams& p, const int d) {
+    // Both tiles are float4 copies of global memory.  Head side: Cs[i][j] (the
+    // coefficient rows as stored), a lane reads four consecutive j of its row i
+    // in one 16-byte LDS read.  Tail side: Cs[j][i] (coefficient rows are the
+    // other operand's rows), a lane reads its column i of four rows j.
+    constexpr int NT = NW * 64;
+    constexpr int AT = 8 / NW;        // 32-row accumulator tiles per wave
+    constexpr int NCH = BJT / 32;     // 32-row sub-chunks per iteration
+    constexpr int HC = 1024 / NT;     // float4 of a 32 x 128 coefficient sub-tile per thread
+    constexpr int HO = 512 / NT;      // float4 of a 32 x 64 `other` sub-tile per thread
+    constexpr int CS_ROWS = SIDE_B ? BJT : BM_TI, CS_LD = SIDE_B ? BM_TI + 4 : BJT + 4;
+    __shared__ __attribute__((aligned(16))) float Cs[CS_ROWS][CS_LD];
     __shared__ __attribute__((aligned(16))) float Os[BJT][BM_LDK];
     __shared__ float csum_s[BM_TI];
-    const int d = blockIdx.z, i0 = blockIdx.y * BM_TI, kt0 = blockIdx.x * BM_TK;
+    const int i0 = blockIdx.y * BM_TI, kt0 = blockIdx.x * BM_TK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wi = (wave >> 1) * 64, wk = (wave & 1) * 32;
+    const int wi = (wave >> 1) * (32 * AT), wk = (wave & 1) * 32;
     const int B = p.B, T = p.T, Dp = p.Dp;
     const int n_self = SIDE_B ? T : B, n_other = SIDE_B ? B : T;
+    if (i0 >= n_self) return;  // the grid is sized for the longer side
+    const int grad_c0 = SIDE_B ? p.b_c0 : p.a_c0;
     const int self_c0 = SIDE_B ? p.b_c0 + d * T : p.a_c0 + d * B;
     const int other_c0 = SIDE_B ? p.a_c0 + d * B : p.b_c0 + d * T;
     const int self_rel = SIDE_B ? 0 : p.a_rel_mode, other_rel = SIDE_B ? p.a_rel_mode : 0;
@@ -1215,19 +1233,19 @@ __global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
     const RowSource& other_src = SIDE_B ? p.ent_a : p.ent_b;
     const float* coef = p.coef + (size_t)d * B * T;
 
-    floatx16 acc[2];
+    floatx16 acc[AT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < AT; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
     float cs_acc = 0.f;
     const int kcol = kt0 + wk + (lane & 31);
 
-    // L2: this lane's 2 x 16 `self` values, in accumulator layout
-    float sv[2][16];
+    // L2: this lane's `self` values, in accumulator layout
+    float sv[AT][16];
     if (DIST == DIST_L2) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < AT; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int i = i0 + wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
@@ -1248,34 +1266,34 @@ __global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
             }
     }
     // near-identical-pair flags of the (self sub-tile, other chunk) blocks
-    const int MT = (B + 31) >> 5, NT = (T + 31) >> 5;
-    const uint32_t* nflag = (DIST == DIST_L2 && p.nearflag) ? p.nearflag + (size_t)d * MT * NT : nullptr;
+    const int MT = (B + 31) >> 5, NTL = (T + 31) >> 5;
+    const uint32_t* nflag = (DIST == DIST_L2 && p.nearflag) ? p.nearflag + (size_t)d * MT * NTL : nullptr;
     auto flag_of = [&](int i_tile, int j_tile) -> uint32_t {
         if (!nflag) return 0u;
         const int mt = SIDE_B ? j_tile : i_tile, nt = SIDE_B ? i_tile : j_tile;
-        if (ALIGNED) return nflag[(size_t)mt * NT + nt];
-        return (mt < MT && nt < NT) ? nflag[(size_t)mt * NT + nt] : 0u;
+        if (ALIGNED) return nflag[(size_t)mt * NTL + nt];
+        return (mt < MT && nt < NTL) ? nflag[(size_t)mt * NTL + nt] : 0u;
     };
-    uint32_t nf_next[NCH][2], nf_row_next[NCH];
-    float4 creg[NCH][4], oreg[NCH][2];
+    uint32_t nf_next[NCH][AT], nf_row_next[NCH];
+    float4 creg[NCH][HC], oreg[NCH][HO];
     auto prefetch = [&](int jbase) {
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int j0 = jbase + 32 * c;
-            nf_next[c][0] = flag_of((i0 + wi) >> 5, j0 >> 5);
-            nf_next[c][1] = flag_of((i0 + wi + 32) >> 5, j0 >> 5);
+#pragma unroll
+            for (int t = 0; t < AT; ++t) nf_next[c][t] = flag_of((i0 + wi + 32 * t) >> 5, j0 >> 5);
             nf_row_next[c] = flag_of((i0 + (tid & (BM_TI - 1))) >> 5, j0 >> 5);
             if (ALIGNED) {
 #pragma unroll
-                for (int h = 0; h < 4; ++h) {
-                    const int idx = tid + 256 * h;
+                for (int h = 0; h < HC; ++h) {
+                    const int idx = tid + NT * h;
                     const float* src = SIDE_B ? coef + (size_t)(j0 + (idx >> 5)) * T + i0 + (idx & 31) * 4
                                               : coef + (size_t)(i0 + (idx >> 3)) * T + j0 + (idx & 7) * 4;
                     creg[c][h] = *reinterpret_cast<const float4*>(src);
                 }
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const int idx = tid + 256 * h;
+                for (int h = 0; h < HO; ++h) {
+                    const int idx = tid + NT * h;
                     oreg[c][h] = *reinterpret_cast<const float4*>(
                         other_src.base + (int64_t)(other_c0 + j0 + (idx >> 4)) * other_src.pitch +
                         (size_t)(kt0 + (idx & 15) * 4) * 4);
@@ -1283,8 +1301,8 @@ __global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
                 continue;
             }
 #pragma unroll
-            for (int h = 0; h < 4; ++h) {
-                const int idx = tid + 256 * h;
+            for (int h = 0; h < HC; ++h) {
+                const int idx = tid + NT * h;
                 creg[c][h] = make_float4(0, 0, 0, 0);
                 if (!SIDE_B) {  // c[i][j] = coef[i0+i][j0+j]: float4 along j
                     const int gi = i0 + (idx >> 3), gj = j0 + (idx & 7) * 4;
@@ -1313,8 +1331,8 @@ __global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
                 }
             }
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int idx = tid + 256 * h;
+            for (int h = 0; h < HO; ++h) {
+                const int idx = tid + NT * h;
                 const int gj = j0 + (idx >> 4), gk = kt0 + (idx & 15) * 4;
                 oreg[c][h] = make_float4(0, 0, 0, 0);
                 if (gj < n_other && gk < Dp) {
@@ -1327,24 +1345,28 @@ __global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
     };
     prefetch(0);
     for (int jbase = 0; jbase < n_other; jbase += BJT) {
-        bool direct0[NCH], direct1[NCH], direct_row[NCH];
+        bool direct[NCH][AT], direct_row[NCH], any_direct[NCH];
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            direct0[c] = nf_next[c][0] != 0u; direct1[c] = nf_next[c][1] != 0u; direct_row[c] = nf_row_next[c] != 0u;
+            any_direct[c] = false;
 #pragma unroll
-            for (int h = 0; h < 4; ++h) {
-                const int idx = tid + 256 * h;
+            for (int t = 0; t < AT; ++t) {
+                direct[c][t] = nf_next[c][t] != 0u;
+                any_direct[c] = any_direct[c] || direct[c][t];
+            }
+            direct_row[c] = nf_row_next[c] != 0u;
+#pragma unroll
+            for (int h = 0; h < HC; ++h) {
+                const int idx = tid + NT * h;
                 if (!SIDE_B) {
-                    const int i = idx >> 3, j4 = 32 * c + (idx & 7) * 4;
-                    Cs[j4 + 0][i] = creg[c][h].x; Cs[j4 + 1][i] = creg[c][h].y;
-                    Cs[j4 + 2][i] = creg[c][h].z; Cs[j4 + 3][i] = creg[c][h].w;
+                    *reinterpret_cast<float4*>(&Cs[idx >> 3][32 * c + (idx & 7) * 4]) = creg[c][h];
                 } else {
                     *reinterpret_cast<float4*>(&Cs[32 * c + (idx >> 5)][(idx & 31) * 4]) = creg[c][h];
                 }
             }
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int idx = tid + 256 * h;
+            for (int h = 0; h < HO; ++h) {
+                const int idx = tid + NT * h;
                 *reinterpret_cast<float4*>(&Os[32 * c + (idx >> 4)][(idx & 15) * 4]) = oreg[c][h];
             }
         }
@@ -1354,48 +1376,60 @@ __global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
         for (int c = 0; c < NCH; ++c) {
             const int jo = 32 * c;
             if (DIST == DIST_L2 && tid < BM_TI && !direct_row[c]) {
+                if (SIDE_B) {
 #pragma unroll
-                for (int jj = 0; jj < 32; ++jj) cs_acc += Cs[jo + jj][tid];
-            }
-            if (!direct0[c] && !direct1[c]) {
-                float ra0[2][4], ra1[2][4], rb[2][4];
-                const int hl = lane >> 5, cl = lane & 31;
+                    for (int jj = 0; jj < 32; ++jj) cs_acc += Cs[jo + jj][tid];
+                } else {
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    rb[0][x] = Os[jo + 2 * x + hl][wk + cl];
-                    ra0[0][x] = Cs[jo + 2 * x + hl][wi + cl];
-                    ra1[0][x] = Cs[jo + 2 * x + hl][wi + 32 + cl];
+                    for (int jj = 0; jj < 32; jj += 4) {
+                        const float4 v = *reinterpret_cast<const float4*>(&Cs[tid][jo + jj]);
+                        cs_acc += v.x; cs_acc += v.y; cs_acc += v.z; cs_acc += v.w;
+                    }
                 }
+            }
+            if (!any_direct[c]) {
+                // group g covers rows j = jo + 8g .. 8g+7 of `other`: instruction x
+                // takes row 8g + x (lower half-wave) and 8g + 4 + x (upper)
+                float ra[2][AT][4], rb[2][4];
+                const int hl = lane >> 5, cl = lane & 31;
+                auto fetch = [&](int buf, int g) {
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    if (g + 1 < 4) {
+                    for (int x = 0; x < 4; ++x) rb[buf][x] = Os[jo + 8 * g + 4 * hl + x][wk + cl];
 #pragma unroll
-                        for (int x = 0; x < 4; ++x) {
-                            const int jj = jo + 8 * (g + 1) + 2 * x + hl;
-                            rb[(g + 1) & 1][x] = Os[jj][wk + cl];
-                            ra0[(g + 1) & 1][x] = Cs[jj][wi + cl];
-                            ra1[(g + 1) & 1][x] = Cs[jj][wi + 32 + cl];
+                    for (int t = 0; t < AT; ++t) {
+                        if (SIDE_B) {
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) ra[buf][t][x] = Cs[jo + 8 * g + 4 * hl + x][wi + 32 * t + cl];
+                        } else {
+                            const float4 v = *reinterpret_cast<const float4*>(&Cs[wi + 32 * t + cl][jo + 8 * g + 4 * hl]);
+                            ra[buf][t][0] = v.x; ra[buf][t][1] = v.y; ra[buf][t][2] = v.z; ra[buf][t][3] = v.w;
                         }
                     }
+                };
+                fetch(0, 0);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    if (g + 1 < 4) fetch((g + 1) & 1, g + 1);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra0[g & 1][x], rb[g & 1][x], acc[0], 0, 0, 0);
-                        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra1[g & 1][x], rb[g & 1][x], acc[1], 0, 0, 0);
-                    }
+                    for (int x = 0; x < 4; ++x)
+#pragma unroll
+                        for (int t = 0; t < AT; ++t)
+                            acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[g & 1][t][x], rb[g & 1][x], acc[t], 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
                 // some pair of this block is nearly identical: c * (self - other) directly,
                 // as the reference codelet does (acc holds the negated sum, see the epilogue)
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    if (t == 0 ? direct0[c] : direct1[c]) {
+                for (int t = 0; t < AT; ++t) {
+                    if (direct[c][t]) {
                         for (int jj = jo; jj < jo + 32; ++jj) {
                             const float o = Os[jj][wk + (lane & 31)];
 #pragma unroll
                             for (int r = 0; r < 16; ++r) {
-                                const float cc = Cs[jj][wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
+                                const int il = wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                                const float cc = SIDE_B ? Cs[jj][il] : Cs[il][jj];
                                 acc[t][r] = fmaf(-cc, sv[t][r] - o, acc[t][r]);
                             }
                         }
@@ -1404,7 +1438,7 @@ __global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
                         for (int q = 0; q < 16; ++q) {
                             const int jj = jo + 2 * q + (lane >> 5);
                             const float b = Os[jj][wk + (lane & 31)];
-                            const float a = Cs[jj][wi + 32 * t + (lane & 31)];
+                            const float a = SIDE_B ? Cs[jj][wi + 32 * t + (lane & 31)] : Cs[wi + 32 * t + (lane & 31)][jj];
                             acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[t], 0, 0, 0);
                         }
                     }
@@ -1418,16 +1452,28 @@ __global__ __launch_bounds__(256) void k_score_bwd_mfma(BwdParams p) {
         __syncthreads();
     }
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < AT; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int i_loc = wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             const int i = i0 + i_loc;
-            if (i >= n_self || kcol >= Dp) continue;
+            if (!ALIGNED && (i >= n_self || kcol >= Dp)) continue;
             float o = acc[t][r];
             if (DIST == DIST_L2) o = sv[t][r] * csum_s[i_loc] - o;
-            p.grad[(size_t)(p.grad_c0 + d * n_self + i) * Dp + kcol] = o;
+            p.grad[(size_t)(grad_c0 + d * n_self + i) * Dp + kcol] = o;
         }
+}
+
+// one side per launch (p.side_b), or both sides in one launch: blocks with
+// blockIdx.z < S do the head side, the others the tail side
+template <int DIST, int SIDE_B, int BJT, bool ALIGNED, int NW>
+__global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma(BwdParams p) {
+    bwd_mfma_body<DIST, SIDE_B, BJT, ALIGNED, NW>(p, blockIdx.z);
+}
+template <int DIST, int BJT, bool ALIGNED, int NW>
+__global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma_both(BwdParams p) {
+    if ((int)blockIdx.z < p.S) bwd_mfma_body<DIST, 0, BJT, ALIGNED, NW>(p, blockIdx.z);
+    else bwd_mfma_body<DIST, 1, BJT, ALIGNED, NW>(p, blockIdx.z - p.S);
 }
 
 static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
@@ -1440,12 +1486,10 @@ static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
         const bool plain = p.ent_a.etype == ET_F32 && p.ent_b.etype == ET_F32 && !p.ent_a.index &&
                            !p.ent_b.index && p.a_rel_mode == 0;
         const bool aligned = plain && n_self % BM_TI == 0 && p.Dp % BM_TK == 0 && p.T % 4 == 0 && n_other % 32 == 0;
-        const bool wide = aligned && n_other % 128 == 0 && (int)(grid.x * grid.y * grid.z) <= 512;
 #define KGE_BWD(D_, S_)                                                                                     \
     do {                                                                                                    \
-        if (wide) hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 128, true>), grid, dim3(256), 0, stream, p);  \
-        else if (aligned) hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 32, true>), grid, dim3(256), 0, stream, p); \
-        else hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 32, false>), grid, dim3(256), 0, stream, p);       \
+        if (aligned) hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 32, true, 8>), grid, dim3(512), 0, stream, p); \
+        else hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 32, false, 4>), grid, dim3(256), 0, stream, p);    \
     } while (0)
         if (dist_fn == DIST_L2) {
             if (p.side_b) KGE_BWD(DIST_L2, 1); else KGE_BWD(DIST_L2, 0);
@@ -1475,6 +1519,20 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
     p.a_rel_mode = sh.operands_dense ? 0 : (sh.score_fn == SCORE_DISTMULT ? 2 : 1);
     p.a_c0 = 0; p.b_c0 = sh.S * sh.B;
     const int dist_fn = sh.score_fn == SCORE_DISTMULT ? DIST_DOT : sh.dist_fn;
+    // matrix-core path: both sides in one launch (tile-aligned shapes)
+    const bool plain = ent.etype == ET_F32 && !ent.index && p.a_rel_mode == 0 && ent.vec;
+    const bool both = sh.use_mfma && plain && sh.B % BM_TI == 0 && sh.T % BM_TI == 0 && sh.Dp % BM_TK == 0 &&
+                      (dist_fn == DIST_DOT || (dist_fn == DIST_L2 && nearflag));
+    if (both) {
+        dim3 grid(sh.Dp / BM_TK, std::max(sh.B, sh.T) / BM_TI, 2 * sh.S);
+        // eight waves per workgroup (two per SIMD): measured faster than four at
+        // every BASELINE shape, few workgroups (c2) or many (c3)
+        if (dist_fn == DIST_L2)
+            hipLaunchKernelGGL((k_score_bwd_mfma_both<DIST_L2, 32, true, 8>), grid, dim3(512), 0, stream, p);
+        else
+            hipLaunchKernelGGL((k_score_bwd_mfma_both<DIST_DOT, 32, true, 8>), grid, dim3(512), 0, stream, p);
+        return;
+    }
     p.side_b = 0; p.grad_c0 = p.a_c0;
     launch_bwd(p, dist_fn, stream);
     p.side_b = 1; p.grad_c0 = p.b_c0;

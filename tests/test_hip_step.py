@@ -32,6 +32,19 @@ CASES = {
                    n_entity=3000, n_relation=40, gamma=6.0),
     "mid_l1": dict(distance_fn="L1", n_shard=2, batch=70, a2a=45, dim=64, feature=0,
                    n_entity=2000, n_relation=10, gamma=6.0),
+    # tile-aligned shapes (positives % 128, tails % 128, dim % 64): the matrix-core fast path
+    "aligned_l2": dict(distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
+                       n_entity=3000, n_relation=8, gamma=6.0),
+    "aligned_l2_wide": dict(distance_fn="L2", n_shard=4, batch=256, a2a=64, dim=128, feature=0,
+                            n_entity=5000, n_relation=8, gamma=6.0, shared_table=True),
+    "aligned_distmult": dict(score_fn="DistMult", distance_fn="MatMul", loss_fn="softmax",
+                             softmax_correction_weight=1.0, n_shard=2, batch=128, a2a=64, dim=64,
+                             feature=0, n_entity=3000, n_relation=8),
+    "aligned_l2_softmax": dict(distance_fn="L2", loss_fn="softmax", softmax_correction_weight=1.0,
+                               n_shard=2, batch=128, a2a=64, dim=64, feature=0, n_entity=3000,
+                               n_relation=8, gamma=6.0),
+    "bf16_embedding_l2": dict(distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
+                              n_entity=3000, n_relation=8, gamma=6.0, storage="bfloat16_embedding"),
 }
 
 
@@ -42,6 +55,10 @@ def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_lo
     c = K.cfg_dict(**kw)
     rng = np.random.default_rng(11)
     st0 = K.make_state(c, rng, warm=warm)
+    bf16 = c["storage"] == "bfloat16_embedding"
+    if bf16:  # the table stores bfloat16 embeddings: start from representable values
+        D = c["dim"]
+        st0["entity_data"][:, :D] = oracle.round(st0["entity_data"][:, :D], "bfloat16_embedding")
     lr = np.resize(np.asarray(lr, np.float32), c["n_shard"])
     if c["shared_table"]:
         lr[:] = lr[0]
@@ -64,10 +81,20 @@ def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_lo
         if k == "step":
             continue
         d_h, d_o = st_h[k] - st0[k], st_o[k] - st0[k]
-        # updated rows: 1e-5 relative (measured ~1e-7); the update itself: the
+        # updated rows: 1e-5 relative (measured ~1e-6 at lr 0.1); the update itself: the
         # reference's own 1e-4 bar on (final - initial), whose float32 storage
         # rounding alone is ~1e-5 of a small delta
-        assert K.rel_l2(st_h[k], st_o[k]) < 1e-6, (k, K.rel_l2(st_h[k], st_o[k]))
+        if bf16 and k == "entity_data":
+            # bfloat16 rows: 2e-2 relative; a float32 difference of one part in 1e7 may
+            # round an element to the other bfloat16 neighbour (2^-8 relative), so the
+            # moments (float32) are held to the tight bar and the embedding to bf16's
+            D = c["dim"]
+            assert K.rel_l2(st_h[k][:, D:], st_o[k][:, D:]) < 1e-5
+            assert K.rel_l2(st_h[k][:, :D], st_o[k][:, :D]) < 2e-3
+            mism = np.mean(st_h[k][:, :D] != st_o[k][:, :D])
+            assert mism < 1e-3, mism  # all but a handful of elements are bit-identical
+            continue
+        assert K.rel_l2(st_h[k], st_o[k]) < 1e-5, (k, K.rel_l2(st_h[k], st_o[k]))
         assert K.rel_l2(d_h, d_o) < 1e-4, (k, K.rel_l2(d_h, d_o))
     return c, st0, st_h, engine
 
@@ -110,6 +137,34 @@ def test_step_near_duplicate_rows(oracle64):
         assert K.rel_l2(st_h[k] - st0[k], st_o[k] - st0[k]) < 1e-4, k
 
 
+@pytest.mark.parametrize("scoring", ["mfma", "valu"])
+def test_step_near_duplicate_rows_aligned(oracle64, scoring):
+    # the same hazard at tile-aligned shapes: the fast path flags the 32x32 score
+    # sub-blocks that hold near-identical pairs and the backward treats them directly
+    import libpoplar_kge
+
+    c = K.cfg_dict(distance_fn="L2", feature=0, gamma=1.0, n_shard=2, batch=128, a2a=64, dim=64,
+                   n_entity=600, n_relation=4)
+    rng = np.random.default_rng(4)
+    st0 = K.make_state(c, rng)
+    D = c["dim"]
+    st0["relation_embedding"] *= 1e-4
+    base = st0["entity_data"][1, :D].copy()
+    for r in range(2, st0["entity_data"].shape[0], 5):  # a fifth of the rows cluster tightly
+        st0["entity_data"][r, :D] = base * (1 + 3e-4 * rng.normal(size=D))
+    st0["entity_data"][7, :D] = st0["entity_data"][12, :D]
+    batch = K.random_batch(c, 2, rng)
+    engine = libpoplar_kge.Engine(H.engine_settings(c, 2, **{"execution.scoring": scoring}), "")
+    H.load_state(engine, c, st0)
+    st_o = K.copy_state(st0)
+    loss_o = oracle64.train_step_loop(make_cfg(**c), st_o, 0.05, batch)
+    loss_h = H.train(engine, c, 0.05, batch)
+    np.testing.assert_allclose(loss_h, loss_o, rtol=1e-5)
+    st_h = H.read_state(engine, c)
+    for k in ("entity_data", "relation_embedding"):
+        assert K.rel_l2(st_h[k] - st0[k], st_o[k] - st0[k]) < 1e-4, k
+
+
 def test_step_padding_rows(oracle64):
     # zero-padded `remote`: row 0 gathered several times, updated once with g = 0
     run_case(oracle64, dict(feature=0), batch_fn=lambda c, n, r: K.random_batch(c, n, r, pad=4))
@@ -130,7 +185,7 @@ def test_step_cold_start(oracle64):
 def test_step_deterministic():
     import libpoplar_kge
 
-    c = K.cfg_dict(distance_fn="L2", shared_table=True, n_shard=8, batch=64, a2a=8, dim=64,
+    c = K.cfg_dict(distance_fn="L2", shared_table=True, n_shard=8, batch=128, a2a=16, dim=64,
                    feature=0, n_entity=300, n_relation=20, gamma=5.0)
     rng = np.random.default_rng(5)
     st0 = K.make_state(c, rng)
