@@ -402,8 +402,12 @@ void parse_settings(kge_engine& E, const Items& s) {
 
 void allocate(kge_engine& E) {
     int n_dev = 0;
-    if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev < 1)
-        throw std::runtime_error("Could not attach to a HIP device");
+    const hipError_t dev_err = hipGetDeviceCount(&n_dev);
+    if (dev_err != hipSuccess || n_dev < 1) {
+        (void)hipGetLastError();
+        throw std::runtime_error(std::string("Could not attach to a HIP device (") +
+                                 (dev_err != hipSuccess ? hipGetErrorString(dev_err) : "no device") + ")");
+    }
     HIP_CHECK(hipStreamCreate(&E.stream));
     for (auto& e : E.ev) HIP_CHECK(hipEventCreate(&e));
     const hipStream_t st = E.stream;

@@ -6,6 +6,12 @@ from pathlib import Path
 
 import pytest
 
+# PyTorch-ROCm bundles its own copy of the HIP runtime.  Two copies in one
+# process cannot both initialise the device, so torch (used by the GPU tests
+# for device memory) is loaded before anything pulls in libkge_hip.so, which
+# then binds to the copy already present.
+import torch  # noqa: F401,E402
+
 ROOT = Path(__file__).resolve().parent.parent
 PKG = ROOT / "distributed-kge-poplar_amd"
 for p in (ROOT, PKG, ROOT / "tests"):
