@@ -614,6 +614,9 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
 // result keeps float32 accuracy and is exactly 0 for identical rows.
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+DEVINL floatx4 as_x4(float4 v) { return floatx4{v.x, v.y, v.z, v.w}; }
+DEVINL float4 as_f4(floatx4 v) { return make_float4(v.x, v.y, v.z, v.w); }
 
 constexpr int FM_TM = 128, FM_TN = 64;
 constexpr float kCancelRatio = 0.125f;  // recompute when d^2 < ratio * (|a|^2 + |b|^2)
@@ -1275,40 +1278,39 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d) {
         return (mt < MT && nt < NTL) ? nflag[(size_t)mt * NTL + nt] : 0u;
     };
     uint32_t nf_next[NCH][AT], nf_row_next[NCH];
-    float4 creg[NCH][HC], oreg[NCH][HO];
-    auto prefetch = [&](int jbase) {
+    floatx4 creg[NCH][HC], oreg[NCH][HO];
+    auto prefetch = [&](int jbase) __attribute__((always_inline)) {
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int j0 = jbase + 32 * c;
 #pragma unroll
             for (int t = 0; t < AT; ++t) nf_next[c][t] = flag_of((i0 + wi + 32 * t) >> 5, j0 >> 5);
             nf_row_next[c] = flag_of((i0 + (tid & (BM_TI - 1))) >> 5, j0 >> 5);
-            if (ALIGNED) {
+            if constexpr (ALIGNED) {
 #pragma unroll
                 for (int h = 0; h < HC; ++h) {
                     const int idx = tid + NT * h;
                     const float* src = SIDE_B ? coef + (size_t)(j0 + (idx >> 5)) * T + i0 + (idx & 31) * 4
                                               : coef + (size_t)(i0 + (idx >> 3)) * T + j0 + (idx & 7) * 4;
-                    creg[c][h] = *reinterpret_cast<const float4*>(src);
+                    creg[c][h] = *reinterpret_cast<const floatx4*>(src);
                 }
 #pragma unroll
                 for (int h = 0; h < HO; ++h) {
                     const int idx = tid + NT * h;
-                    oreg[c][h] = *reinterpret_cast<const float4*>(
+                    oreg[c][h] = *reinterpret_cast<const floatx4*>(
                         other_src.base + (int64_t)(other_c0 + j0 + (idx >> 4)) * other_src.pitch +
                         (size_t)(kt0 + (idx & 15) * 4) * 4);
                 }
-                continue;
-            }
+            } else {
 #pragma unroll
             for (int h = 0; h < HC; ++h) {
                 const int idx = tid + NT * h;
-                creg[c][h] = make_float4(0, 0, 0, 0);
+                creg[c][h] = floatx4{0.f, 0.f, 0.f, 0.f};
                 if (!SIDE_B) {  // c[i][j] = coef[i0+i][j0+j]: float4 along j
                     const int gi = i0 + (idx >> 3), gj = j0 + (idx & 7) * 4;
                     if (gi < B && gj < T) {
                         const float* src = coef + (size_t)gi * T + gj;
-                        if (gj + 3 < T && (T & 3) == 0) creg[c][h] = *reinterpret_cast<const float4*>(src);
+                        if (gj + 3 < T && (T & 3) == 0) creg[c][h] = *reinterpret_cast<const floatx4*>(src);
                         else {
                             creg[c][h].x = src[0];
                             if (gj + 1 < T) creg[c][h].y = src[1];
@@ -1320,7 +1322,7 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d) {
                     const int gj = j0 + (idx >> 5), gi = i0 + (idx & 31) * 4;
                     if (gj < B && gi < T) {
                         const float* src = coef + (size_t)gj * T + gi;
-                        if (gi + 3 < T && (T & 3) == 0) creg[c][h] = *reinterpret_cast<const float4*>(src);
+                        if (gi + 3 < T && (T & 3) == 0) creg[c][h] = *reinterpret_cast<const floatx4*>(src);
                         else {
                             creg[c][h].x = src[0];
                             if (gi + 1 < T) creg[c][h].y = src[1];
@@ -1334,12 +1336,13 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d) {
             for (int h = 0; h < HO; ++h) {
                 const int idx = tid + NT * h;
                 const int gj = j0 + (idx >> 4), gk = kt0 + (idx & 15) * 4;
-                oreg[c][h] = make_float4(0, 0, 0, 0);
+                oreg[c][h] = floatx4{0.f, 0.f, 0.f, 0.f};
                 if (gj < n_other && gk < Dp) {
-                    oreg[c][h] = load4(row_ptr(other_src, other_c0 + gj), gk, other_src);
+                    oreg[c][h] = as_x4(load4(row_ptr(other_src, other_c0 + gj), gk, other_src));
                     if (other_rel)
-                        oreg[c][h] = combine_rel(oreg[c][h], p.rel + (size_t)p.crel[d * B + gj] * Dp, gk, other_rel);
+                        oreg[c][h] = as_x4(combine_rel(as_f4(oreg[c][h]), p.rel + (size_t)p.crel[d * B + gj] * Dp, gk, other_rel));
                 }
+            }
             }
         }
     };
@@ -1359,15 +1362,15 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d) {
             for (int h = 0; h < HC; ++h) {
                 const int idx = tid + NT * h;
                 if (!SIDE_B) {
-                    *reinterpret_cast<float4*>(&Cs[idx >> 3][32 * c + (idx & 7) * 4]) = creg[c][h];
+                    *reinterpret_cast<floatx4*>(&Cs[idx >> 3][32 * c + (idx & 7) * 4]) = creg[c][h];
                 } else {
-                    *reinterpret_cast<float4*>(&Cs[32 * c + (idx >> 5)][(idx & 31) * 4]) = creg[c][h];
+                    *reinterpret_cast<floatx4*>(&Cs[32 * c + (idx >> 5)][(idx & 31) * 4]) = creg[c][h];
                 }
             }
 #pragma unroll
             for (int h = 0; h < HO; ++h) {
                 const int idx = tid + NT * h;
-                *reinterpret_cast<float4*>(&Os[32 * c + (idx >> 4)][(idx & 15) * 4]) = oreg[c][h];
+                *reinterpret_cast<floatx4*>(&Os[32 * c + (idx >> 4)][(idx & 15) * 4]) = oreg[c][h];
             }
         }
         __syncthreads();
