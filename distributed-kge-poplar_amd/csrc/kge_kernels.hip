@@ -423,6 +423,9 @@ __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const fl
     for (int k = lane * 4; k < Dp; k += 256) {
         float4 v = load4(row, k, ent);
         if (rrow) v = combine_rel(v, rrow, k, rel_mode);
+        // + 0 turns a -0 into +0, so that a difference of stored operands is never -0
+        // (the paired L1 backward reads the sign off the difference's bit pattern)
+        v.x += 0.f; v.y += 0.f; v.z += 0.f; v.w += 0.f;
         *reinterpret_cast<float4*>(out + (size_t)c * Dp + k) = v;
     }
 }
@@ -1511,6 +1514,78 @@ static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
         hipLaunchKernelGGL(k_score_bwd<DIST_DOT>, grid, dim3(256), 0, stream, p);
 }
 
+
+// --------------------------------------------------------------------------
+// L1 backward, both sides in one pass over the pairs.  c * signum(a - b) has no
+// contraction form, so this is vector-ALU work; computing the term once and
+// adding it to the head's sum and (negated) to the tail's sum halves it.
+// One workgroup of 16 waves per (block, 64-column slice); a lane owns one
+// column.  Wave w keeps tails [w*TW, (w+1)*TW) and their gradient sums in
+// registers and walks over all heads; a head's sum over one wave's tails is a
+// partial, the 16 partials of a head meet in LDS and are added in wave order
+// (deterministic).  The coefficients of a (head, tail range) are wave-uniform
+// and come in through scalar loads.
+constexpr int L1P_CB = 16;     // heads per chunk (one per wave in the reduction)
+constexpr int L1P_WAVES = 16;
+
+template <int TW>
+__global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restrict__ operands,
+                                                            const float* __restrict__ coef,
+                                                            float* __restrict__ grad, int B, int T,
+                                                            int Dp, int a_c0, int b_c0) {
+    __shared__ float part[2][L1P_WAVES][L1P_CB][64];
+    const int d = blockIdx.y, k = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int t0 = w * TW;
+    const float* a_rows = operands + (size_t)(a_c0 + d * B) * Dp + k;
+    const float* b_rows = operands + (size_t)(b_c0 + d * T + t0) * Dp + k;
+    const float* crow = coef + (size_t)d * B * T + t0;
+
+    float bt[TW], gt[TW];
+#pragma unroll
+    for (int j = 0; j < TW; ++j) {
+        bt[j] = b_rows[(size_t)j * Dp];
+        gt[j] = 0.f;
+    }
+    for (int b0 = 0, buf = 0; b0 < B; b0 += L1P_CB, buf ^= 1) {
+        float a_next = a_rows[(size_t)b0 * Dp];
+        for (int bi = 0; bi < L1P_CB; ++bi) {
+            const float a = a_next;
+            if (bi + 1 < L1P_CB) a_next = a_rows[(size_t)(b0 + bi + 1) * Dp];
+            const float* c = crow + (size_t)(b0 + bi) * T;
+            float gp = 0.f;
+#pragma unroll
+            for (int j = 0; j < TW; ++j) {
+                // signum(a - b) with signum(0) = 0 (poplar_extensions l1distance.codelet.cpp:76-79):
+                // the difference's bit pattern read as an integer has its sign and is zero
+                // only for +0; converted to float (magnitude >= 1 unless zero) and clamped
+                // to [-1, 1].  (-0 never appears: the dense operands are stored with +0 added.)
+                const float sg = __builtin_amdgcn_fmed3f((float)__float_as_int(a - bt[j]), -1.f, 1.f);
+                gp = fmaf(c[j], sg, gp);
+                gt[j] = fmaf(-c[j], sg, gt[j]);
+            }
+            part[buf][w][bi][lane] = gp;
+        }
+        __syncthreads();
+        // wave w adds the 16 partials of head b0 + w
+        float sum = 0.f;
+#pragma unroll
+        for (int v = 0; v < L1P_WAVES; ++v) sum += part[buf][v][w][lane];
+        grad[(size_t)(a_c0 + d * B + b0 + w) * Dp + k] = sum;
+    }
+#pragma unroll
+    for (int j = 0; j < TW; ++j) grad[(size_t)(b_c0 + d * T + t0 + j) * Dp + k] = gt[j];
+}
+
+// shapes the paired L1 kernel takes: tails split evenly over 16 waves, whole
+// chunks of heads, whole 64-column slices, and enough workgroups for the chip
+static bool l1_pair_ok(const ScoreShape& sh) {
+    const int tw = sh.T / L1P_WAVES;
+    return sh.T % L1P_WAVES == 0 && (tw == 8 || tw == 16 || tw == 32) && sh.B % L1P_CB == 0 &&
+           sh.Dp % 64 == 0 && sh.S * (sh.Dp / 64) >= 128;
+}
+
 void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
                       const uint32_t* crel, const float* coef, const uint32_t* nearflag, float* grad,
                       hipStream_t stream) {
@@ -1534,6 +1609,18 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
             hipLaunchKernelGGL((k_score_bwd_mfma_both<DIST_L2, 32, true, 8>), grid, dim3(512), 0, stream, p);
         else
             hipLaunchKernelGGL((k_score_bwd_mfma_both<DIST_DOT, 32, true, 8>), grid, dim3(512), 0, stream, p);
+        return;
+    }
+    if (dist_fn == DIST_L1 && sh.use_mfma && sh.operands_dense && plain && ent.pitch == (int64_t)sh.Dp * 4 && l1_pair_ok(sh)) {
+        const float* ops = reinterpret_cast<const float*>(ent.base);
+        dim3 grid(sh.Dp / 64, sh.S);
+        const int tw = sh.T / L1P_WAVES;
+        if (tw == 32)
+            hipLaunchKernelGGL(k_score_bwd_l1_pair<32>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
+        else if (tw == 16)
+            hipLaunchKernelGGL(k_score_bwd_l1_pair<16>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
+        else
+            hipLaunchKernelGGL(k_score_bwd_l1_pair<8>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
         return;
     }
     p.side_b = 0; p.grad_c0 = p.a_c0;

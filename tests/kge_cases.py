@@ -17,7 +17,10 @@ def cfg_dict(**kw):
 
 def make_state(c, rng, warm=True, scale=None):
     """Random tables.  ``warm``: non-zero Adam moments and step, so the update
-    formula is exercised away from its zero-state special case."""
+    formula is exercised away from its zero-state special case.  The second
+    moments stay away from zero: m / (sqrt(v) + eps) with sqrt(v) ~ 1e-5 turns a
+    float32 rounding difference in a cancelling gradient sum into a visible
+    change of the parameter, in any implementation."""
     S, NE, D, F, NR = c["n_shard"], c["n_entity"], c["dim"], c["feature"], c["n_relation"]
     rows = NE if c["shared_table"] else S * NE
     scale = scale if scale is not None else 1.0 / np.sqrt(D)
@@ -25,20 +28,20 @@ def make_state(c, rng, warm=True, scale=None):
     ed[:, :D] = rng.normal(0, scale, (rows, D))
     if warm:
         ed[:, D:2 * D] = rng.normal(0, 0.1, (rows, D))
-        ed[:, 2 * D:3 * D] = np.abs(rng.normal(0, 0.3, (rows, D)))
+        ed[:, 2 * D:3 * D] = 0.05 + np.abs(rng.normal(0, 0.3, (rows, D)))
     if F:
         ed[:, 3 * D:] = rng.normal(0, 1, (rows, F)).astype(np.float16)
     st = {
         "entity_data": ed,
         "relation_embedding": rng.normal(0, scale, (NR, D)).astype(np.float32),
         "relation_embedding/adam_m": (rng.normal(0, 0.1, (NR, D)) * warm).astype(np.float32),
-        "relation_embedding/adam_v": (rng.normal(0, 0.3, (NR, D))**2 * warm).astype(np.float32),
+        "relation_embedding/adam_v": ((0.05 + np.abs(rng.normal(0, 0.3, (NR, D))))**2 * warm).astype(np.float32),
         "step": 7 if warm else 0,
     }
     if F:
         st["feature_projection"] = rng.normal(0, scale / np.sqrt(F), (F, D)).astype(np.float32)
         st["feature_projection/adam_m"] = (rng.normal(0, 0.1, (F, D)) * warm).astype(np.float32)
-        st["feature_projection/adam_v"] = (rng.normal(0, 0.3, (F, D))**2 * warm).astype(np.float32)
+        st["feature_projection/adam_v"] = ((0.05 + np.abs(rng.normal(0, 0.3, (F, D))))**2 * warm).astype(np.float32)
     return st
 
 

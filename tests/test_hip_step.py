@@ -43,6 +43,13 @@ CASES = {
     "aligned_l2_softmax": dict(distance_fn="L2", loss_fn="softmax", softmax_correction_weight=1.0,
                                n_shard=2, batch=128, a2a=64, dim=64, feature=0, n_entity=3000,
                                n_relation=8, gamma=6.0),
+    # L1 with tails split over 16 waves of 8 / 16 / 32: the one-pass backward for both sides
+    "paired_l1_t128": dict(distance_fn="L1", n_shard=32, batch=16, a2a=4, dim=256, feature=0,
+                           n_entity=4000, n_relation=8, gamma=6.0, shared_table=True),
+    "paired_l1_t256": dict(distance_fn="L1", n_shard=32, batch=32, a2a=8, dim=256, feature=0,
+                           n_entity=4000, n_relation=8, gamma=6.0, shared_table=True),
+    "paired_l1_t512": dict(distance_fn="L1", n_shard=32, batch=16, a2a=16, dim=256, feature=0,
+                           n_entity=4000, n_relation=8, gamma=6.0, shared_table=True),
     "bf16_embedding_l2": dict(distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
                               n_entity=3000, n_relation=8, gamma=6.0, storage="bfloat16_embedding"),
 }
@@ -105,10 +112,41 @@ def test_step_vs_oracle(oracle64, name):
 
 
 @pytest.mark.parametrize("name", ["l2_logsigmoid", "l2_softmax", "distmult_softmax_feat", "mid_l2",
-                                  "transe_matmul", "shared_l2"])
+                                  "transe_matmul", "shared_l2", "paired_l1_t256"])
 def test_step_vs_oracle_valu_scoring(oracle64, name):
     # the same cases on the VALU scoring kernels (default: matrix cores)
     run_case(oracle64, CASES[name], **{"execution.scoring": "valu"})
+
+
+def test_step_l1_equal_and_signed_zero_entries(oracle64):
+    # signum(0) = 0 on the one-pass L1 backward: identical rows under a zero
+    # relation, zero entries of either sign, and rows that differ in a few columns
+    import libpoplar_kge
+
+    c = K.cfg_dict(distance_fn="L1", n_shard=32, batch=16, a2a=4, dim=256, feature=0, n_entity=300,
+                   n_relation=4, gamma=6.0, shared_table=True)
+    rng = np.random.default_rng(9)
+    st0 = K.make_state(c, rng)
+    D = c["dim"]
+    st0["relation_embedding"][:2] = 0.0
+    st0["relation_embedding"][1, ::2] = -0.0
+    rows = st0["entity_data"]
+    for r in range(2, rows.shape[0], 2):       # half of the rows are near-copies of row 1
+        rows[r, :D] = rows[1, :D]
+        rows[r, rng.integers(0, D, 5)] += 0.01
+    rows[:, 3] = 0.0
+    rows[::3, 3] = -0.0
+    rows[:, 7] = np.where(rng.random(rows.shape[0]) < 0.5, 0.0, -0.0)
+    batch = K.random_batch(c, 2, rng)
+    engine = libpoplar_kge.Engine(H.engine_settings(c, 2), "")
+    H.load_state(engine, c, st0)
+    st_o = K.copy_state(st0)
+    loss_o = oracle64.train_step_loop(make_cfg(**c), st_o, 0.05, batch)
+    loss_h = H.train(engine, c, 0.05, batch)
+    np.testing.assert_allclose(loss_h, loss_o, rtol=1e-5)
+    st_h = H.read_state(engine, c)
+    for k in ("entity_data", "relation_embedding"):
+        assert K.rel_l2(st_h[k] - st0[k], st_o[k] - st0[k]) < 1e-4, k
 
 
 def test_step_near_duplicate_rows(oracle64):
