@@ -17,6 +17,10 @@ Extra objects in that line:
   kernels       the same figures for every kernel of the step
   cpu_baseline  the sequential float32 CPU oracle on the first steps of the same
                 workload, on this host's cores (1 thread)
+  host_batches  the same steps with the index arrays handed over as host buffers
+                every call (PCIe-inclusive; never the headline value)
+  copy_calibration  one plain row copy much larger than the caches, whose known
+                size scales the FETCH_SIZE / WRITE_SIZE counters of a profiler run
 """
 
 import argparse
@@ -56,6 +60,14 @@ WORKLOADS = {
 
 PEAK_HBM_GBPS = 8000.0
 PEAK_FP32_TFLOPS = 157.3
+
+# HBM bytes per launch (fetched + written) of the dominant kernel, from two
+# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each
+# scaled by what the same counter reads for the calibration copy below.
+# Counters cannot be read from inside this process, so the figures are carried
+# here and refreshed together with the committed profiler summaries.
+MEASURED_TRAFFIC_BYTES = {
+}
 
 
 def make_settings(w, n_step, kge):
@@ -282,7 +294,23 @@ def main():
     gather = dict(rows=int(ids.size), ms=float(gms[0]),
                   achieved=2 * ids.size * row_bytes / (gms[0] * 1e-3) / 1e9, unit="GB/s (read + write)")
 
+    # one large plain copy (distinct rows, > 1 GB each way): scales the profiler's byte counters
+    n_cal = min(m.n_entity - 1, 400_000)
+    cal_ids = (1 + np.random.default_rng(5).permutation(m.n_entity - 1)[:n_cal]).astype(np.uint32)
+    engine.engine.run("gather_benchmark", dict(indices=cal_ids, ms=gms, repeats=1))
+    calibration = dict(kernel="k_rows_copy", rows=int(n_cal), bytes_read=int(n_cal * row_bytes),
+                       bytes_written=int(n_cal * row_bytes), ms=float(gms[0]),
+                       achieved=2 * n_cal * row_bytes / (gms[0] * 1e-3) / 1e9, unit="GB/s (read + write)")
+
+    # one call over all W + K steps with the index arrays passed as host buffers
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    engine.train_step_loop(batch)
+    torch.cuda.synchronize()
+    dt_host = (time.perf_counter() - t1) / n_total
+
     triples = args.steps * m.n_shard * d.batch_size
+    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get((args.workload, dominant))
     U = float(np.mean(uniq_rows))
     R = m.n_shard * settings.n_remote
     step_bytes = (U * 2 * row_bytes + 4 * (R + 2 * m.n_shard * d.batch_size) + 4 * U
@@ -312,6 +340,11 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
         "row_gather": gather,
+        "copy_calibration": calibration,
+        "host_batches": {"value": m.n_shard * d.batch_size / dt_host, "unit": "triples/s",
+                         "ms_per_step": dt_host * 1e3,
+                         "note": f"one call over {n_total} steps, index arrays uploaded from host "
+                                 "memory inside the timed call"},
         "cpu_baseline": cpu,
         "check": check,
     }

@@ -436,6 +436,37 @@ void launch_gather_operands(const RowSource& ent, const float* rel, const uint32
                        rel_mode, n_head, n_rows, Dp, out);
 }
 
+
+// --------------------------------------------------------------------------
+// Tile order.  The scoring kernels run gx * gy tiles for each of gz blocks; a
+// block's tiles all read that block's operand rows (and coefficient matrix).
+// Workgroups go to the 8 XCDs round-robin by linear id and every XCD has its own
+// L2, so with the plain (x, y, z) order each XCD would fetch every block's
+// operands.  Launching a 1-D grid and decoding it this way keeps a block's
+// tiles on one XCD (block z on XCD z % 8), in consecutive slots of that XCD.
+struct TileId { int x, y, z, gx, gy; };
+constexpr int kXcdGroup = 2;
+DEVINL TileId xcd_tile(int gx, int gy, int gz) {
+    const int L = blockIdx.x, n = gx * gy;
+    int z, t;
+    if ((gz & 7) == 0) {
+        // kXcdGroup blocks of an XCD are interleaved tile by tile, so that the CUs of
+        // an XCD do not all start on a new block's cold rows at the same moment
+        const int j = L >> 3;
+        const int G = ((gz >> 3) % kXcdGroup) == 0 ? kXcdGroup : 1;
+        const int chunk = j / (G * n), r = j - chunk * (G * n);
+        z = (L & 7) + 8 * (chunk * G + r % G);
+        t = r / G;
+    } else {
+        z = L / n;
+        t = L - z * n;
+    }
+    TileId id;
+    id.y = t / gx; id.x = t - id.y * gx; id.z = z; id.gx = gx; id.gy = gy;
+    return id;
+}
+static dim3 tile_grid(int gx, int gy, int gz) { return dim3((unsigned)(gx * gy * gz)); }
+
 // --------------------------------------------------------------------------
 // scoring: forward
 
@@ -489,7 +520,8 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
     __shared__ float red[4];
     __shared__ uint32_t label_s[kScoreTile];
     const ScoreShape& sh = p.sh;
-    const int d = blockIdx.z, m0 = blockIdx.y * kScoreTile, n0 = blockIdx.x * kScoreTile;
+    const TileId tile = xcd_tile((sh.T + kScoreTile - 1) / kScoreTile, (sh.B + kScoreTile - 1) / kScoreTile, sh.S);
+    const int d = tile.z, m0 = tile.y * kScoreTile, n0 = tile.x * kScoreTile;
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int B = sh.B, T = sh.T, Dp = sh.Dp;
     if (p.out_mode == 0 && tid < kScoreTile) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
@@ -601,8 +633,8 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
         if ((tid & 63) == 0) red[tid >> 6] = loss_acc;
         __syncthreads();
         if (tid == 0) {
-            const int n_part = gridDim.x * gridDim.y;
-            p.loss_part[(size_t)d * n_part + blockIdx.y * gridDim.x + blockIdx.x] =
+            const int n_part = tile.gx * tile.gy;
+            p.loss_part[(size_t)d * n_part + tile.y * tile.gx + tile.x] =
                 (red[0] + red[1] + red[2] + red[3]) * inv_norm;
         }
     }
@@ -656,7 +688,8 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     __shared__ float red[NW];
     __shared__ uint32_t label_s[FM_TM];
     const ScoreShape& sh = p.sh;
-    const int d = blockIdx.z, m0 = blockIdx.y * FM_TM, n0 = blockIdx.x * FM_TN;
+    const TileId tile = xcd_tile((sh.T + FM_TN - 1) / FM_TN, (sh.B + FM_TM - 1) / FM_TM, sh.S);
+    const int d = tile.z, m0 = tile.y * FM_TM, n0 = tile.x * FM_TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * (32 * AT), wn = (wave & 1) * 32;
     const int B = sh.B, T = sh.T, Dp = sh.Dp;
@@ -885,11 +918,11 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
         if (lane == 0) red[wave] = loss_acc;
         __syncthreads();
         if (tid == 0) {
-            const int n_part = gridDim.x * gridDim.y;
+            const int n_part = tile.gx * tile.gy;
             float tot = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) tot += red[w];
-            p.loss_part[(size_t)d * n_part + blockIdx.y * gridDim.x + blockIdx.x] = tot * inv_norm;
+            p.loss_part[(size_t)d * n_part + tile.y * tile.gx + tile.x] = tot * inv_norm;
         }
     }
 }
@@ -906,7 +939,7 @@ int score_fwd_parts(const ScoreShape& sh) {
 
 static void launch_fwd(const FwdParams& p, hipStream_t stream) {
     if (fwd_uses_mfma(p)) {
-        dim3 grid((p.sh.T + FM_TN - 1) / FM_TN, (p.sh.B + FM_TM - 1) / FM_TM, p.sh.S);
+        const dim3 grid = tile_grid((p.sh.T + FM_TN - 1) / FM_TN, (p.sh.B + FM_TM - 1) / FM_TM, p.sh.S);
         const bool f32 = p.ent_a.etype == ET_F32 && p.ent_b.etype == ET_F32;
         const bool aligned = f32 && p.a_rel_mode == 0 && !p.ent_a.index && !p.ent_b.index &&
                              p.sh.B % FM_TM == 0 && p.sh.T % FM_TN == 0;
@@ -920,7 +953,7 @@ static void launch_fwd(const FwdParams& p, hipStream_t stream) {
 #undef KGE_FWD
         return;
     }
-    dim3 grid((p.sh.T + kScoreTile - 1) / kScoreTile, (p.sh.B + kScoreTile - 1) / kScoreTile, p.sh.S);
+    const dim3 grid = tile_grid((p.sh.T + kScoreTile - 1) / kScoreTile, (p.sh.B + kScoreTile - 1) / kScoreTile, p.sh.S);
     if (p.sh.dist_fn == DIST_L1)
         hipLaunchKernelGGL(k_score_fwd<DIST_L1>, grid, dim3(256), 0, stream, p);
     else if (p.sh.dist_fn == DIST_L2)
@@ -1052,10 +1085,11 @@ template <int DIST>
 __global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
     __shared__ __attribute__((aligned(16))) float Cs[BJ][LDP];  // Cs[j][i]
     __shared__ __attribute__((aligned(16))) float Os[BJ][LDP];  // Os[j][k]
-    const int d = blockIdx.z, i0 = blockIdx.y * kScoreTile, kt0 = blockIdx.x * kScoreTile;
-    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int B = p.B, T = p.T, Dp = p.Dp;
     const int n_self = p.side_b ? T : B, n_other = p.side_b ? B : T;
+    const TileId tile = xcd_tile((Dp + kScoreTile - 1) / kScoreTile, (n_self + kScoreTile - 1) / kScoreTile, p.S);
+    const int d = tile.z, i0 = tile.y * kScoreTile, kt0 = tile.x * kScoreTile;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int self_c0 = (p.side_b ? p.b_c0 + d * T : p.a_c0 + d * B);
     const int other_c0 = (p.side_b ? p.a_c0 + d * B : p.b_c0 + d * T);
     const int self_rel = p.side_b ? 0 : p.a_rel_mode, other_rel = p.side_b ? p.a_rel_mode : 0;
@@ -1211,7 +1245,7 @@ constexpr int BM_TI = 128, BM_TK = 64, BM_LDK = BM_TK + 4;
 // ALIGNED: n_self % 128 == 0, n_other % BJT == 0, Dp % 64 == 0, T % 4 == 0,
 // dense float32 operands without a relation to apply: branch-free staging loads.
 template <int DIST, int SIDE_B, int BJT, bool ALIGNED, int NW>
-DEVINL void bwd_mfma_body(const BwdParams& p, const int d) {
+DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, const int tile_y) {
     // Both tiles are float4 copies of global memory.  Head side: Cs[i][j] (the
     // coefficient rows as stored), a lane reads four consecutive j of its row i
     // in one 16-byte LDS read.  Tail side: Cs[j][i] (coefficient rows are the
@@ -1225,7 +1259,7 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d) {
     __shared__ __attribute__((aligned(16))) float Cs[CS_ROWS][CS_LD];
     __shared__ __attribute__((aligned(16))) float Os[BJT][BM_LDK];
     __shared__ float csum_s[BM_TI];
-    const int i0 = blockIdx.y * BM_TI, kt0 = blockIdx.x * BM_TK;
+    const int i0 = tile_y * BM_TI, kt0 = tile_x * BM_TK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wi = (wave >> 1) * (32 * AT), wk = (wave & 1) * 32;
     const int B = p.B, T = p.T, Dp = p.Dp;
@@ -1470,16 +1504,21 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d) {
         }
 }
 
-// one side per launch (p.side_b), or both sides in one launch: blocks with
-// blockIdx.z < S do the head side, the others the tail side
+// one side per launch (p.side_b), or both sides in one launch
 template <int DIST, int SIDE_B, int BJT, bool ALIGNED, int NW>
 __global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma(BwdParams p) {
-    bwd_mfma_body<DIST, SIDE_B, BJT, ALIGNED, NW>(p, blockIdx.z);
+    const int n_self = SIDE_B ? p.T : p.B;
+    const TileId tile = xcd_tile((p.Dp + BM_TK - 1) / BM_TK, (n_self + BM_TI - 1) / BM_TI, p.S);
+    bwd_mfma_body<DIST, SIDE_B, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y);
 }
 template <int DIST, int BJT, bool ALIGNED, int NW>
 __global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma_both(BwdParams p) {
-    if ((int)blockIdx.z < p.S) bwd_mfma_body<DIST, 0, BJT, ALIGNED, NW>(p, blockIdx.z);
-    else bwd_mfma_body<DIST, 1, BJT, ALIGNED, NW>(p, blockIdx.z - p.S);
+    // a block's head-side tiles and then its tail-side tiles, back to back on one XCD:
+    // both sides read the same operand rows and coefficient matrix
+    const int gy = (p.B > p.T ? p.B : p.T) / BM_TI;
+    const TileId tile = xcd_tile(p.Dp / BM_TK, 2 * gy, p.S);
+    if (tile.y < gy) bwd_mfma_body<DIST, 0, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y);
+    else bwd_mfma_body<DIST, 1, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y - gy);
 }
 
 static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
@@ -1487,7 +1526,7 @@ static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
     const bool mfma_ok = p.use_mfma && !p.coef_div && p.ent_a.vec && p.ent_b.vec && (p.Dp & 3) == 0 &&
                          (dist_fn == DIST_DOT || (dist_fn == DIST_L2 && p.nearflag));
     if (mfma_ok) {
-        dim3 grid((p.Dp + BM_TK - 1) / BM_TK, (n_self + BM_TI - 1) / BM_TI, p.S);
+        const dim3 grid = tile_grid((p.Dp + BM_TK - 1) / BM_TK, (n_self + BM_TI - 1) / BM_TI, p.S);
         const int n_other = p.side_b ? p.B : p.T;
         const bool plain = p.ent_a.etype == ET_F32 && p.ent_b.etype == ET_F32 && !p.ent_a.index &&
                            !p.ent_b.index && p.a_rel_mode == 0;
@@ -1505,7 +1544,7 @@ static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
 #undef KGE_BWD
         return;
     }
-    dim3 grid((p.Dp + kScoreTile - 1) / kScoreTile, (n_self + kScoreTile - 1) / kScoreTile, p.S);
+    const dim3 grid = tile_grid((p.Dp + kScoreTile - 1) / kScoreTile, (n_self + kScoreTile - 1) / kScoreTile, p.S);
     if (dist_fn == DIST_L1)
         hipLaunchKernelGGL(k_score_bwd<DIST_L1>, grid, dim3(256), 0, stream, p);
     else if (dist_fn == DIST_L2)
@@ -1534,7 +1573,8 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
                                                             float* __restrict__ grad, int B, int T,
                                                             int Dp, int a_c0, int b_c0) {
     __shared__ float part[2][L1P_WAVES][L1P_CB][64];
-    const int d = blockIdx.y, k = blockIdx.x * 64 + (threadIdx.x & 63);
+    const TileId tile = xcd_tile(Dp / 64, 1, (int)gridDim.x / (Dp / 64));
+    const int d = tile.z, k = tile.x * 64 + (threadIdx.x & 63);
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int t0 = w * TW;
@@ -1602,7 +1642,7 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
     const bool both = sh.use_mfma && plain && sh.B % BM_TI == 0 && sh.T % BM_TI == 0 && sh.Dp % BM_TK == 0 &&
                       (dist_fn == DIST_DOT || (dist_fn == DIST_L2 && nearflag));
     if (both) {
-        dim3 grid(sh.Dp / BM_TK, std::max(sh.B, sh.T) / BM_TI, 2 * sh.S);
+        const dim3 grid = tile_grid(sh.Dp / BM_TK, 2 * (std::max(sh.B, sh.T) / BM_TI), sh.S);
         // eight waves per workgroup (two per SIMD): measured faster than four at
         // every BASELINE shape, few workgroups (c2) or many (c3)
         if (dist_fn == DIST_L2)
@@ -1613,7 +1653,7 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
     }
     if (dist_fn == DIST_L1 && sh.use_mfma && sh.operands_dense && plain && ent.pitch == (int64_t)sh.Dp * 4 && l1_pair_ok(sh)) {
         const float* ops = reinterpret_cast<const float*>(ent.base);
-        dim3 grid(sh.Dp / 64, sh.S);
+        const dim3 grid = tile_grid(sh.Dp / 64, 1, sh.S);
         const int tw = sh.T / L1P_WAVES;
         if (tw == 32)
             hipLaunchKernelGGL(k_score_bwd_l1_pair<32>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
