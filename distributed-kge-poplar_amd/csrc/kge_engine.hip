@@ -172,7 +172,9 @@ uint16_t float_to_half(float f) {
 
 enum KernelId {
     K_PLAN = 0, K_HIDDEN, K_GATHER, K_FWD, K_LOSS, K_BWD, K_REDUCE_ENT, K_ADAM_ENT, K_REDUCE_REL, K_ADAM_REL,
-    K_PROJ_GRAD, K_ADAM_PROJ, K_COUNT
+    K_PROJ_GRAD, K_ADAM_PROJ,
+    K_EVENT_PAIR,  // an event pair with nothing between: what the pairs around the kernels add
+    K_COUNT
 };
 
 struct Variable {
@@ -838,6 +840,7 @@ void run_step(kge_engine& E, int i) {
         launch_adam_rows2(ae, ar, st);
     }
 
+    { KernelTimer t(E, K_EVENT_PAIR); }
     if (E.F) {
         { KernelTimer t(E, K_PROJ_GRAD); launch_proj_grad(fa, E.gsum.p, E.gproj.p, st); }
         // dense Adam on the projection; shard s owns rows [s*F/S, (s+1)*F/S) and its step size
