@@ -52,6 +52,11 @@ WORKLOADS = {
     "c3l2": dict(desc="TransE-L2 D=256 fp32, 22.8M entities, 64 blocks x (256 positives, 512 shared tails)",
                  n_entity=22_800_000, n_relation=1387, dim=256, blocks=64, batch=256, tails=512,
                  distance_fn="L2"),
+    "c4": dict(desc="DistMult D=512 + 768-dim fp16 feature projected 768->512, 4M entities, "
+                    "1 block x (8192 positives, 2048 shared tails), softmax CE",
+               n_entity=4_000_000, n_relation=1387, dim=512, blocks=1, batch=8192, tails=2048,
+               score_fn="DistMult", distance_fn="MatMul", loss="softmax", feature=768,
+               feature_dtype="float16"),
     "c5": dict(desc="TransE-L2 D=256 bf16 embedding + fp32 moments, 91.2M entities, "
                     "32 blocks x (512 positives, 512 shared tails)",
                n_entity=91_200_000, n_relation=1387, dim=256, blocks=32, batch=512, tails=512,
@@ -76,14 +81,15 @@ def make_settings(w, n_step, kge):
     s = kge.Settings.create_demo()
     s.seed = 20240611
     m, d, t, e = s.model, s.data, s.training, s.execution
-    m.score_fn, m.distance_fn = "TransE", w["distance_fn"]
+    m.score_fn, m.distance_fn = w.get("score_fn", "TransE"), w["distance_fn"]
     m.n_shard, m.n_entity, m.n_relation_type = w["blocks"], w["n_entity"], w["n_relation"]
-    m.embedding_size, m.entity_feature_size, m.gamma = w["dim"], 0, 10.0
+    m.embedding_size, m.entity_feature_size, m.gamma = w["dim"], w.get("feature", 0), 10.0
     m.init_scale = float(np.sqrt(w["dim"]))  # embeddings ~ N(0, 1/sqrt(D)): sigma = init_scale / D
     d.batch_size, d.a2a_size = w["batch"], w["tails"] // w["blocks"]
-    t.learning_rate, t.loss = 1e-3, kge.LogSigmoidLoss()
+    t.learning_rate = 1e-3
+    t.loss = kge.SoftmaxLoss(correction_weight=1.0) if w.get("loss") == "softmax" else kge.LogSigmoidLoss()
     e.device, e.dtype, e.shared_table = "hip", "float32", True
-    e.embedding_dtype = w.get("embedding_dtype")
+    e.embedding_dtype, e.feature_dtype = w.get("embedding_dtype"), w.get("feature_dtype")
     e.train_steps_per_program_run = n_step
     e.rw_batch_size = 8192
     return s.prepare()
@@ -106,6 +112,9 @@ def init_tables(engine, settings):
     m, e = settings.model, settings.execution
     per_call = m.n_shard * e.rw_batch_size
     feat = np.zeros(settings.entity_data_w_shape, np.float32)
+    if m.entity_feature_size:
+        # N(0, 1) features; one block of them serves every call (rows per_call apart share features)
+        feat = np.random.default_rng(settings.seed + 5).normal(size=feat.shape).astype(np.float32)
     for off in range(0, m.n_entity, per_call):
         idx = np.arange(off, off + per_call, dtype=np.int64)
         idx[idx >= m.n_entity] = 0
@@ -145,13 +154,17 @@ def cpu_baseline(engine, settings, w, batch, n_check, n_cpu_steps):
     rows = read_rows(engine, settings, ids)
     table = np.zeros((m.n_entity, settings.entity_data_r_size), np.float32)  # untouched pages stay virtual
     table[ids] = rows
-    state = {"entity_data": table, "step": 0,
-             "relation_embedding": engine.read_variable("relation_embedding"),
-             "relation_embedding/adam_m": engine.read_variable("relation_embedding/adam_m"),
-             "relation_embedding/adam_v": engine.read_variable("relation_embedding/adam_v")}
+    state = {"entity_data": table, "step": 0}
+    names = ["relation_embedding"] + (["feature_projection"] if m.entity_feature_size else [])
+    for name in names:
+        for suffix in ("", "/adam_m", "/adam_v"):
+            state[name + suffix] = engine.read_variable(name + suffix)
+    softmax = w.get("loss") == "softmax"
     cfg = make_cfg(n_shard=m.n_shard, n_entity=m.n_entity, n_relation=m.n_relation_type,
-                   dim=m.embedding_size, feature=0, batch=d.batch_size, a2a=d.a2a_size,
-                   score_fn=m.score_fn, distance_fn=m.distance_fn, loss_fn="logsigmoid",
+                   dim=m.embedding_size, feature=m.entity_feature_size, batch=d.batch_size, a2a=d.a2a_size,
+                   score_fn=m.score_fn, distance_fn=m.distance_fn,
+                   loss_fn="softmax" if softmax else "logsigmoid",
+                   softmax_correction_weight=1.0 if softmax else 0.0,
                    shared_table=True, gamma=m.gamma, loss_scale=settings.training.loss_scale,
                    storage="bfloat16_embedding" if w.get("embedding_dtype") == "bfloat16" else "float32")
     oracle = Oracle("f32")
@@ -190,16 +203,20 @@ def kernel_table(w, timing, n_steps, uniq_rows):
         "adam_entity": ("bytes", U * 2 * row_state + 2 * 3 * w["n_relation"] * D * 4),
         "plan": ("bytes", 4.0 * (R + 2 * K_ * B) + 4 * U),
     }
+    F = w.get("feature", 0)
+    if F:
+        work["hidden_fwd"] = ("flops", 2.0 * U * F * D)
+        work["proj_grad"] = ("flops", 2.0 * U * F * D)
+        work["loss_rows"] = ("bytes", 2.0 * K_ * B * T * 4)
+    if w.get("score_fn") == "DistMult":  # 2 flop per pair-dim forward (mul, add); backward = 2x
+        work["score_fwd"] = ("flops", 2.0 * pair_dims)
+        work["score_bwd"] = ("flops", 4.0 * pair_dims)
     out = {}
-    # what an event pair reads with nothing between its events: taken off every launch
-    pair = timing["kernels"]["event_pair"]
-    pair_ms = pair["ms"] / pair["calls"] if pair["calls"] else 0.0
     for name, rec in timing["kernels"].items():
         if rec["calls"] == 0 or name not in work:
             continue
         kind, amount = work[name]
-        # per step (plan: one launch group per call, shared by its steps)
-        ms = (rec["ms"] - (pair_ms * rec["calls"] if name != "plan" else 0.0)) / n_steps
+        ms = rec["ms"] / n_steps  # per step (plan: one launch group per call, shared by its steps)
         entry = dict(ms_per_step=ms, launches_per_step=rec["calls"] / n_steps)
         if kind == "bytes":
             entry.update(bound="hbm", achieved=amount / (ms * 1e-3) / 1e9, peak=PEAK_HBM_GBPS, unit="GB/s")
@@ -288,17 +305,16 @@ def main():
     step_kernels = {k: v for k, v in kernels.items() if k != "plan"}
     dominant = max(step_kernels, key=lambda k: step_kernels[k]["ms_per_step"])
     dom = kernels[dominant]
-    pair = prof["kernels"]["event_pair"]
     roofline = dict(kernel=dominant, bound=dom["bound"], achieved=dom["achieved"], peak=dom["peak"],
                     unit=dom["unit"], frac=dom["frac"], traffic=None,
-                    launch_ms=dom["ms_per_step"] / dom["launches_per_step"],
-                    event_pair_ms=pair["ms"] / max(pair["calls"], 1))
+                    launch_ms=dom["ms_per_step"] / dom["launches_per_step"])
 
     # stand-alone row gather (fr::Buffer::read) over one step's distinct rows
     ids = np.unique(batch.remote[:, args.warmup]).astype(np.uint32)
     gms = np.zeros(1, np.float32)
     engine.engine.run("gather_benchmark", dict(indices=ids, ms=gms, repeats=20))
-    row_bytes = (2 if w.get("embedding_dtype") == "bfloat16" else 4) * m.embedding_size + 8 * m.embedding_size
+    row_bytes = ((2 if w.get("embedding_dtype") == "bfloat16" else 4) * m.embedding_size + 8 * m.embedding_size
+                 + (2 if w.get("feature_dtype") == "float16" else 4) * m.entity_feature_size)
     gather = dict(rows=int(ids.size), ms=float(gms[0]),
                   achieved=2 * ids.size * row_bytes / (gms[0] * 1e-3) / 1e9, unit="GB/s (read + write)")
 
@@ -336,7 +352,8 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16 rows / f32 math" if w.get("embedding_dtype") == "bfloat16" else "f32",
         "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {w['desc']}; Zipf s=1.1 ids, logsigmoid loss, "
+        "config": {"workload": f"{args.workload}: {w['desc']}; Zipf s=1.1 ids, "
+                               f"{w.get('loss', 'logsigmoid')} loss, "
                                f"Adam lr 1e-3, raw ids de-duplicated on the device",
                    "positives_per_step": m.n_shard * d.batch_size, "row_refs_per_step": R,
                    "unique_rows_per_step": U},

@@ -172,9 +172,7 @@ uint16_t float_to_half(float f) {
 
 enum KernelId {
     K_PLAN = 0, K_HIDDEN, K_GATHER, K_FWD, K_LOSS, K_BWD, K_REDUCE_ENT, K_ADAM_ENT, K_REDUCE_REL, K_ADAM_REL,
-    K_PROJ_GRAD, K_ADAM_PROJ,
-    K_EVENT_PAIR,  // an event pair with nothing between: what the pairs around the kernels add
-    K_COUNT
+    K_PROJ_GRAD, K_ADAM_PROJ, K_COUNT
 };
 
 struct Variable {
@@ -221,7 +219,7 @@ struct kge_engine {
     int e_ustride, e_cstride, r_ustride, r_cstride, n_rel_items;
     uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
     // step
-    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, loss_part, d_loss, d_alpha;
+    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, loss_part, d_loss, d_alpha;
     std::vector<float> h_alpha;  // [n_step][entity, relation, projection][S]
     int n_part;
     // io staging
@@ -467,6 +465,9 @@ void allocate(kge_engine& E) {
     if (E.F) {
         E.hidden.alloc(R * E.Dp);
         E.gsum.alloc(R * E.Dp);
+        E.gsum.zero(E.stream);  // rows past a step's distinct count are read (times zero): keep them finite
+        E.featd.alloc(R * E.Fp);
+        E.gproj_part.alloc((size_t)16 * E.Fp * E.Dp);
         E.gproj.alloc(proj_n);
     }
     ScoreShape sh = {};
@@ -740,6 +741,7 @@ void run_step(kge_engine& E, int i) {
         fa.emb_base = E.table.p; fa.feat_base = E.table.p + E.L.off_f; fa.pitch = E.L.pitch;
         fa.emb_etype = E.L.emb_etype; fa.feat_etype = E.L.feat_etype;
         fa.Dp = E.Dp; fa.Fp = E.Fp; fa.proj = E.proj.p;
+        fa.featd = E.featd.p; fa.gproj_part = E.gproj_part.p; fa.use_mfma = E.use_mfma;
         { KernelTimer t(E, K_HIDDEN); launch_hidden_fwd(fa, E.hidden.p, st); }
         ent.base = (const char*)E.hidden.p; ent.pitch = (int64_t)E.Dp * 4; ent.etype = ET_F32;
         ent.index = E.e_item_row.p + i * R;
@@ -840,7 +842,6 @@ void run_step(kge_engine& E, int i) {
         launch_adam_rows2(ae, ar, st);
     }
 
-    { KernelTimer t(E, K_EVENT_PAIR); }
     if (E.F) {
         { KernelTimer t(E, K_PROJ_GRAD); launch_proj_grad(fa, E.gsum.p, E.gproj.p, st); }
         // dense Adam on the projection; shard s owns rows [s*F/S, (s+1)*F/S) and its step size

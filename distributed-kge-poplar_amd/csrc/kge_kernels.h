@@ -190,6 +190,9 @@ struct FeatureArgs {
     int emb_etype, feat_etype;
     int Dp, Fp;
     const float* proj;      // [Fp, Dp]
+    float* featd;           // scratch [max_rows, Fp]: the distinct rows' features, float32
+    float* gproj_part;      // scratch [16, Fp, Dp]: split-contraction partials of the projection gradient
+    int use_mfma;
 };
 void launch_hidden_fwd(const FeatureArgs& a, float* hidden, hipStream_t stream);
 // gproj[f, :] = sum_u feature[u, f] * grad_rows[u, :]

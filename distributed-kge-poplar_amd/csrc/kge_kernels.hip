@@ -1077,6 +1077,13 @@ struct BwdParams {
     int a_c0, b_c0;
     int use_mfma;
     const uint32_t* nearflag;  // from the forward pass (L2 on the matrix cores), or null
+    // optional rows added to the output (the feature projection's `embedding + ...`):
+    // output row i gets row add_index[i] of add_base, row 0 for i >= *add_count
+    const char* add_base;
+    int64_t add_pitch;
+    int add_etype;
+    const uint32_t* add_index;
+    const uint32_t* add_count;
 };
 
 constexpr int BJ = 32;  // rows of `other` staged per iteration
@@ -1500,6 +1507,10 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
             if (!ALIGNED && (i >= n_self || kcol >= Dp)) continue;
             float o = acc[t][r];
             if (DIST == DIST_L2) o = sv[t][r] * csum_s[i_loc] - o;
+            if (DIST == DIST_DOT && p.add_base) {
+                const uint32_t row = (uint32_t)i < *p.add_count ? p.add_index[i] : 0u;
+                o += load1(p.add_base + (int64_t)row * p.add_pitch, kcol, p.add_etype);
+            }
             p.grad[(size_t)(grad_c0 + d * n_self + i) * Dp + kcol] = o;
         }
 }
@@ -1631,7 +1642,7 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
                       hipStream_t stream) {
     BwdParams p;
     p.ent_a = ent; p.ent_b = ent; p.rel = rel; p.crel = crel; p.coef = coef; p.grad = grad;
-    p.coef_div = nullptr;
+    p.coef_div = nullptr; p.add_base = nullptr;
     p.S = sh.S; p.B = sh.B; p.T = sh.T; p.Dp = sh.Dp; p.vec_out = 1; p.use_mfma = sh.use_mfma;
     p.nearflag = nearflag;
     p.a_rel_mode = sh.operands_dense ? 0 : (sh.score_fn == SCORE_DISTMULT ? 2 : 1);
@@ -1877,8 +1888,48 @@ __global__ __launch_bounds__(256) void k_hidden_fwd(FeatureArgs a, float* __rest
     }
 }
 
+// The distinct rows' features as dense float32 [max_rows, Fp], rows past the
+// count zero: the operand both feature products read.  One wave per row.
+__global__ __launch_bounds__(256) void k_gather_features(FeatureArgs a, float* __restrict__ featd) {
+    const int lane = threadIdx.x & 63;
+    const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (u >= a.max_rows) return;
+    const bool live = u < (int)a.counts[0];
+    const char* frow = a.feat_base + (int64_t)(live ? a.uniq_key[u] : 0u) * a.pitch;
+    for (int f = lane * 4; f < a.Fp; f += 256) {
+        const float4 x = live ? load4(frow, f, a.feat_etype) : make_float4(0, 0, 0, 0);
+        *reinterpret_cast<float4*>(featd + (size_t)u * a.Fp + f) = x;
+    }
+}
+
+static bool feature_mfma_ok(const FeatureArgs& a) {
+    return a.use_mfma && a.featd && (a.Dp & 3) == 0 && (a.Fp & 3) == 0;
+}
+
+static RowSource dense_rows(const float* base, int cols) {
+    RowSource r;
+    r.base = reinterpret_cast<const char*>(base); r.pitch = (int64_t)cols * 4; r.etype = ET_F32;
+    r.index = nullptr; r.count = cols; r.vec = 1;
+    return r;
+}
+
+// hidden[u, :] = embedding[key u, :] + feature[u, :] . W as a [U x Fp] . [Fp x Dp]
+// product on the matrix cores (the scoring backward's dot kernel: coefficient
+// matrix = dense features, other rows = W), the embedding added in its epilogue.
 void launch_hidden_fwd(const FeatureArgs& a, float* hidden, hipStream_t stream) {
-    hipLaunchKernelGGL(k_hidden_fwd, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, hidden);
+    if (!feature_mfma_ok(a)) {
+        hipLaunchKernelGGL(k_hidden_fwd, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, hidden);
+        return;
+    }
+    hipLaunchKernelGGL(k_gather_features, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, a.featd);
+    BwdParams p = {};
+    p.ent_a = p.ent_b = dense_rows(a.proj, a.Dp);
+    p.coef = a.featd; p.grad = hidden;
+    p.S = 1; p.B = a.max_rows; p.T = a.Fp; p.Dp = a.Dp;
+    p.side_b = 0; p.vec_out = 1; p.use_mfma = 1;
+    p.add_base = a.emb_base; p.add_pitch = a.pitch; p.add_etype = a.emb_etype;
+    p.add_index = a.uniq_key; p.add_count = a.counts;
+    launch_bwd(p, DIST_DOT, stream);
 }
 
 // gproj[f, k] = sum_u feature[u, f] * grad_rows[u, k]; block = 4 feature rows x 64 float4 columns
@@ -1903,8 +1954,39 @@ __global__ __launch_bounds__(256) void k_proj_grad(FeatureArgs a, const float* _
     *reinterpret_cast<float4*>(gproj + (size_t)f * a.Dp + k) = acc;
 }
 
+// out[i] = sum over the `ns` partial arrays of part[s][i], in order (n % 4 == 0)
+__global__ __launch_bounds__(256) void k_sum_splits(const float* __restrict__ part, int ns, int64_t n,
+                                                    float* __restrict__ out) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n) return;
+    float4 acc = *reinterpret_cast<const float4*>(part + i);
+    for (int s = 1; s < ns; ++s) acc = f4add(acc, *reinterpret_cast<const float4*>(part + (size_t)s * n + i));
+    *reinterpret_cast<float4*>(out + i) = acc;
+}
+
 void launch_proj_grad(const FeatureArgs& a, const float* grad_rows, float* gproj,
                       hipStream_t stream) {
+    if (feature_mfma_ok(a)) {
+        // gproj = features^T . grad_rows, [Fp x U] . [U x Dp]: the dot kernel's tail side
+        // (coefficient rows run along the contraction).  Rows past the distinct count
+        // are zero in the dense features and finite in grad_rows, so they add nothing.
+        // The output has few tiles, so the contraction is split over `ns` blocks of
+        // rows whose partial products are then added in block order.
+        int ns = 1;
+        while (ns < 16 && a.max_rows % (2 * ns * 32) == 0 && a.gproj_part) ns *= 2;
+        BwdParams p = {};
+        p.ent_a = p.ent_b = dense_rows(grad_rows, a.Dp);
+        p.coef = a.featd; p.grad = ns > 1 ? a.gproj_part : gproj;
+        p.S = ns; p.B = a.max_rows / ns; p.T = a.Fp; p.Dp = a.Dp;
+        p.side_b = 1; p.vec_out = 1; p.use_mfma = 1;
+        launch_bwd(p, DIST_DOT, stream);
+        if (ns > 1) {
+            const int64_t n = (int64_t)a.Fp * a.Dp;
+            hipLaunchKernelGGL(k_sum_splits, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, stream,
+                               a.gproj_part, ns, n, gproj);
+        }
+        return;
+    }
     dim3 grid((a.Dp / 4 + 63) / 64, (a.Fp + 3) / 4);
     hipLaunchKernelGGL(k_proj_grad, grid, dim3(256), 0, stream, a, grad_rows, gproj);
 }

@@ -250,7 +250,7 @@ class Batch:
 
 
 KERNEL_NAMES = ("plan", "hidden_fwd", "gather_operands", "score_fwd", "loss_rows", "score_bwd", "reduce_entity",
-                "adam_entity", "reduce_relation", "adam_relation", "proj_grad", "adam_proj", "event_pair")
+                "adam_entity", "reduce_relation", "adam_relation", "proj_grad", "adam_proj")
 
 
 class Engine:
