@@ -1,5 +1,6 @@
 """GPU parity at the BASELINE sizes (c2: 1M-row float32 table; c3: 22.8M rows,
-70 GB; c5: 91.2M rows with bfloat16 embeddings, 233 GB): the table is
+70 GB; c4: 4M rows with 768 float16 features, DistMult, softmax; c5: 91.2M rows
+with bfloat16 embeddings, 233 GB): the table is
 initialised on the device, the rows a few steps touch are read back, the CPU
 oracle runs the same steps on a compacted copy of exactly those rows, and the
 updated rows, the relation table and the loss are compared.  Also: rows nobody
@@ -38,7 +39,8 @@ def _run(workload, n_step, rng_rows=2000):
     import poplar_kge as kge
 
     w = bench.WORKLOADS[workload]
-    row_bytes = (2 if w.get("embedding_dtype") else 4) * w["dim"] + 8 * w["dim"]
+    row_bytes = ((2 if w.get("embedding_dtype") else 4) * w["dim"] + 8 * w["dim"]
+                 + (2 if w.get("feature_dtype") else 4) * w.get("feature", 0))
     need = w["n_entity"] * row_bytes + (4 << 30)
     if _free_gpu_bytes() < need:
         pytest.skip(f"needs {need >> 30} GiB of free HBM")
@@ -56,9 +58,10 @@ def _run(workload, n_step, rng_rows=2000):
     # the generator gives N(0, init_scale / D) embeddings and zero moments
     D = m.embedding_size
     assert abs(before[:, :D].std() * np.sqrt(D) - 1.0) < 0.02 and abs(before[:, :D].mean()) < 1e-3
-    assert np.all(before[:, D:] == 0)
+    assert np.all(before[:, D:3 * D] == 0)
 
-    relation_before = engine.read_variable("relation_embedding")
+    dense = ["relation_embedding"] + (["feature_projection"] if m.entity_feature_size else [])
+    dense_before = {k + sfx: engine.read_variable(k + sfx) for k in dense for sfx in ("", "/adam_m", "/adam_v")}
     loss, _ = engine.train_step_loop(batch)
     after = bench.read_rows(engine, settings, ids)
     after_others = bench.read_rows(engine, settings, others)
@@ -69,12 +72,16 @@ def _run(workload, n_step, rng_rows=2000):
     compact[1:] = before
     remap = lambda a: (1 + np.searchsorted(ids, a)).astype(np.uint32)
     state = {"entity_data": compact, "step": 0}
-    state["relation_embedding"] = relation_before
-    state["relation_embedding/adam_m"] = np.zeros_like(state["relation_embedding"])
-    state["relation_embedding/adam_v"] = np.zeros_like(state["relation_embedding"])
+    state.update(dense_before)
     storage = "bfloat16_embedding" if w.get("embedding_dtype") == "bfloat16" else "float32"
-    cfg = make_cfg(n_shard=m.n_shard, n_entity=compact.shape[0], n_relation=m.n_relation_type, dim=D,
-                   feature=0, batch=d.batch_size, a2a=d.a2a_size, distance_fn=m.distance_fn,
+    softmax = w.get("loss") == "softmax"
+    # the softmax correction term reads n_entity: the oracle gets the real table size for it
+    cfg = make_cfg(n_shard=m.n_shard, n_entity=m.n_entity if softmax else compact.shape[0],
+                   n_relation=m.n_relation_type, dim=D,
+                   feature=m.entity_feature_size, batch=d.batch_size, a2a=d.a2a_size,
+                   score_fn=m.score_fn, distance_fn=m.distance_fn,
+                   loss_fn="softmax" if softmax else "logsigmoid",
+                   softmax_correction_weight=1.0 if softmax else 0.0,
                    shared_table=True, gamma=m.gamma, loss_scale=settings.training.loss_scale,
                    storage=storage)
     ob = {k: v for k, v in vars(batch).items()}
@@ -89,11 +96,11 @@ def _run(workload, n_step, rng_rows=2000):
         assert K.rel_l2(after[:, D:], ref[:, D:]) < 1e-5          # float32 moments
         assert K.rel_l2(after[:, :D], ref[:, :D]) < 2e-3          # bfloat16 embedding (bar: 2e-2)
         assert np.mean(after[:, :D] != ref[:, :D]) < 2e-3
-    _close_but_for_sign_flips(engine.read_variable("relation_embedding"), state["relation_embedding"],
-                              "relation_embedding")
-    # the dense table keeps v = E[g^2]; the bar is on |g|-like quantities, as for the rows' sqrt(v)
-    assert K.rel_l2(np.sqrt(engine.read_variable("relation_embedding/adam_v")),
-                    np.sqrt(state["relation_embedding/adam_v"])) < 1e-5
+    for name in dense:
+        _close_but_for_sign_flips(engine.read_variable(name), state[name], name)
+        # the dense tables keep v = E[g^2]; the bar is on |g|-like quantities, as for the rows' sqrt(v)
+        assert K.rel_l2(np.sqrt(engine.read_variable(name + "/adam_v")),
+                        np.sqrt(state[name + "/adam_v"])) < 1e-5, name
     return settings, batch, ids, after, loss
 
 
@@ -119,6 +126,11 @@ def test_c3_full_size_vs_oracle():
 
 def test_c3_l2_full_size_vs_oracle():
     _run("c3l2", n_step=2)
+
+
+def test_c4_full_size_vs_oracle():
+    # DistMult + 768 -> 512 feature projection + softmax CE, 8192 x 2048 scores
+    _run("c4", n_step=1)
 
 
 def test_c5_full_size_vs_oracle():
