@@ -56,7 +56,7 @@ WORKLOADS = {
                     "1 block x (8192 positives, 2048 shared tails), softmax CE",
                n_entity=4_000_000, n_relation=1387, dim=512, blocks=1, batch=8192, tails=2048,
                score_fn="DistMult", distance_fn="MatMul", loss="softmax", feature=768,
-               feature_dtype="float16"),
+               feature_dtype="float16", scoring_dtype="bfloat16"),
     "c5": dict(desc="TransE-L2 D=256 bf16 embedding + fp32 moments, 91.2M entities, "
                     "32 blocks x (512 positives, 512 shared tails)",
                n_entity=91_200_000, n_relation=1387, dim=256, blocks=32, batch=512, tails=512,
@@ -90,6 +90,7 @@ def make_settings(w, n_step, kge):
     t.loss = kge.SoftmaxLoss(correction_weight=1.0) if w.get("loss") == "softmax" else kge.LogSigmoidLoss()
     e.device, e.dtype, e.shared_table = "hip", "float32", True
     e.embedding_dtype, e.feature_dtype = w.get("embedding_dtype"), w.get("feature_dtype")
+    e.scoring_dtype = w.get("scoring_dtype")
     e.train_steps_per_program_run = n_step
     e.rw_batch_size = 8192
     return s.prepare()
@@ -166,6 +167,7 @@ def cpu_baseline(engine, settings, w, batch, n_check, n_cpu_steps):
                    loss_fn="softmax" if softmax else "logsigmoid",
                    softmax_correction_weight=1.0 if softmax else 0.0,
                    shared_table=True, gamma=m.gamma, loss_scale=settings.training.loss_scale,
+                   scoring_bf16=settings.execution.scoring_dtype == "bfloat16",
                    storage="bfloat16_embedding" if w.get("embedding_dtype") == "bfloat16" else "float32")
     oracle = Oracle("f32")
     lr = settings.training.learning_rate
@@ -350,7 +352,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16 rows / f32 math" if w.get("embedding_dtype") == "bfloat16" else "f32",
+        "dtype": ("bf16 scoring operands / f32 accumulate" if w.get("scoring_dtype") == "bfloat16" else
+                  "bf16 rows / f32 math" if w.get("embedding_dtype") == "bfloat16" else "f32"),
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {w['desc']}; Zipf s=1.1 ids, "
                                f"{w.get('loss', 'logsigmoid')} loss, "

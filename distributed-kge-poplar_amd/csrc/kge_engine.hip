@@ -194,6 +194,7 @@ struct kge_engine {
     int stream_kind;  // KGE_F32 or KGE_F16: dtype of the entity read/write streams
     bool profile_kernels = false;
     int use_mfma = 1;  // additive setting execution.scoring = "mfma" | "valu"
+    bool score_bf16 = false;  // additive setting execution.scoring_dtype = "float32" | "bfloat16"
     int chunk = 64;       // contributions per first-level chunk (rows with many contributions)
     int direct_max = 16;  // rows with at most this many contributions are summed by their Adam wave
 
@@ -219,6 +220,7 @@ struct kge_engine {
     int e_ustride, e_cstride, r_ustride, r_cstride, n_rel_items;
     uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
     // step
+    DevBuf<uint16_t> opnd16, opndT16, coef16, coefT16;  // bfloat16 scoring operands
     DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, loss_part, d_loss, d_alpha;
     std::vector<float> h_alpha;  // [n_step][entity, relation, projection][S]
     int n_part;
@@ -318,6 +320,16 @@ void parse_settings(kge_engine& E, const Items& s) {
         if (v == "mfma") E.use_mfma = 1;
         else if (v == "valu") E.use_mfma = 0;
         else throw std::invalid_argument("'execution.scoring' must be 'mfma' or 'valu', not '" + v + "'");
+    }
+
+    if (s.find("execution.scoring_dtype")) {
+        const std::string v = s.str("execution.scoring_dtype");
+        if (v == "bfloat16") E.score_bf16 = true;
+        else if (v != "float32")
+            throw std::invalid_argument("'execution.scoring_dtype' must be 'float32' or 'bfloat16', not '" + v + "'");
+        if (E.score_bf16 && score != "DistMult")
+            throw std::invalid_argument("'execution.scoring_dtype' = 'bfloat16' is implemented for "
+                                        "'model.score_fn' = 'DistMult' (dot-product scores) only");
     }
 
     if (score == "TransE") E.score_fn = SCORE_TRANSE;
@@ -455,8 +467,14 @@ void allocate(kge_engine& E) {
     E.r_counts.alloc(ns * 2);
 
     E.coef.alloc(SB * E.T);
-    const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f;
+    const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f && !E.score_bf16;
     if (!fused && E.score_fn == SCORE_TRANSE && E.dist_fn == DIST_L2) E.dist.alloc(SB * E.T);
+    if (E.score_bf16) {
+        E.opnd16.alloc(R * E.Dp);
+        E.opndT16.alloc(R * E.Dp);
+        E.coef16.alloc(SB * E.T);
+        E.coefT16.alloc(SB * E.T);
+    }
     E.grad.alloc(R * E.Dp);
     E.opnd.alloc(R * E.Dp);
     E.partial.alloc((size_t)E.e_cstride * E.Dp);
@@ -721,7 +739,7 @@ void run_step(kge_engine& E, int i) {
     sh.negative_adversarial_scale = E.neg_adv;
     sh.use_mfma = E.use_mfma;
     sh.operands_dense = 0;
-    const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f;
+    const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f && !E.score_bf16;
 
     const uint32_t* ckey = E.ckey.p + i * R;
     const uint32_t* crel = E.crel.p + i * SB;
@@ -750,17 +768,53 @@ void run_step(kge_engine& E, int i) {
     // dense operands: every contribution's row, float32, relation applied to the heads
     { KernelTimer t(E, K_GATHER);
       launch_gather_operands(ent, E.rel.p, crel, E.score_fn == SCORE_DISTMULT ? 2 : 1, (int)SB, (int)R, E.Dp,
-                             E.opnd.p, st); }
+                             E.opnd.p, E.score_bf16 ? E.opnd16.p : nullptr, st); }
     RowSource dense;
     dense.base = (const char*)E.opnd.p; dense.pitch = (int64_t)E.Dp * 4; dense.etype = ET_F32;
     dense.index = nullptr; dense.count = E.Dp; dense.vec = 1;
     sh.operands_dense = 1;
 
     float* loss_part = E.loss_part.p + (size_t)i * E.S * E.n_part;
-    { KernelTimer t(E, K_FWD);
-      launch_score_fwd(sh, dense, E.rel.p, crel, clabel, E.coef.p, E.dist.p, E.nearflag.p, loss_part, fused, st); }
-    if (!fused) { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, E.dist.p, loss_part, st); }
-    { KernelTimer t(E, K_BWD); launch_score_bwd(sh, dense, E.rel.p, crel, E.coef.p, E.nearflag.p, E.grad.p, st); }
+    // bfloat16 dot-product scoring on the matrix cores: three batched products
+    //   scores = q . tails^T,   d q = c . tails,   d tails = c^T . q
+    // each in the form C = A . Bt^T, which needs tails^T, q^T and c^T: transposing casts
+    const int Bn = E.B, Tn = E.T, Dp = E.Dp;
+    const bool bf16_fast = E.score_bf16 && E.use_mfma && gemm_nt_bf16_ok(Bn, Tn, Dp) &&
+                           gemm_nt_bf16_ok(Bn, Dp, Tn) && gemm_nt_bf16_ok(Tn, Dp, Bn);
+    if (bf16_fast) {
+        const size_t head_n = SB * (size_t)Dp;
+        GemmNT g = {};
+        g.batches = E.S;
+        { KernelTimer t(E, K_FWD);
+          g.A = E.opnd16.p; g.lda = Dp; g.a_batch = (int64_t)Bn * Dp;
+          g.Bt = E.opnd16.p + head_n; g.ldb = Dp; g.b_batch = (int64_t)Tn * Dp;
+          g.C = E.coef.p; g.ldc = Tn; g.c_batch = (int64_t)Bn * Tn;
+          g.M = Bn; g.N = Tn; g.K = Dp;
+          launch_gemm_nt_bf16(g, st); }
+        { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, nullptr, loss_part, st); }
+        { KernelTimer t(E, K_BWD);
+          launch_transpose_bf16(E.opnd16.p, false, E.S, Bn, Dp, Dp, (int64_t)Bn * Dp, E.opndT16.p, nullptr, st);
+          launch_transpose_bf16(E.opnd16.p + head_n, false, E.S, Tn, Dp, Dp, (int64_t)Tn * Dp,
+                                E.opndT16.p + head_n, nullptr, st);
+          launch_transpose_bf16(E.coef.p, true, E.S, Bn, Tn, Tn, (int64_t)Bn * Tn, E.coefT16.p, E.coef16.p, st);
+          // d q [B, Dp] = c [B, T] . tails [T, Dp]
+          g.A = E.coef16.p; g.lda = Tn; g.a_batch = (int64_t)Bn * Tn;
+          g.Bt = E.opndT16.p + head_n; g.ldb = Tn; g.b_batch = (int64_t)Dp * Tn;
+          g.C = E.grad.p; g.ldc = Dp; g.c_batch = (int64_t)Bn * Dp;
+          g.M = Bn; g.N = Dp; g.K = Tn;
+          launch_gemm_nt_bf16(g, st);
+          // d tails [T, Dp] = c^T [T, B] . q [B, Dp]
+          g.A = E.coefT16.p; g.lda = Bn; g.a_batch = (int64_t)Tn * Bn;
+          g.Bt = E.opndT16.p; g.ldb = Bn; g.b_batch = (int64_t)Dp * Bn;
+          g.C = E.grad.p + head_n; g.ldc = Dp; g.c_batch = (int64_t)Tn * Dp;
+          g.M = Tn; g.N = Dp; g.K = Bn;
+          launch_gemm_nt_bf16(g, st); }
+    } else {
+        { KernelTimer t(E, K_FWD);
+          launch_score_fwd(sh, dense, E.rel.p, crel, clabel, E.coef.p, E.dist.p, E.nearflag.p, loss_part, fused, st); }
+        if (!fused) { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, E.dist.p, loss_part, st); }
+        { KernelTimer t(E, K_BWD); launch_score_bwd(sh, dense, E.rel.p, crel, E.coef.p, E.nearflag.p, E.grad.p, st); }
+    }
 
     const float* alpha = E.d_alpha.p + (size_t)i * 3 * E.S;
     AdamArgs aa = {};

@@ -88,8 +88,29 @@ struct ScoreShape {
 
 // Dense float32 operand matrix [n_rows, Dp] from indexed rows: rows [0, n_head)
 // combined with their relation row (rel_mode 1 add, 2 multiply).
+// With `out16` the values are rounded to bfloat16, stored there, and the float32
+// copy holds the same rounded values.
 void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
-                            int n_head, int n_rows, int Dp, float* out, hipStream_t stream);
+                            int n_head, int n_rows, int Dp, float* out, uint16_t* out16,
+                            hipStream_t stream);
+
+// Batched bfloat16 product on the matrix cores: C[z] = A[z] . Bt[z]^T, float32 out.
+// Strides in elements.  Optional rows added to the output: output row m gets row
+// add_index[m] of add_base (row 0 for m >= *add_count), columns as C's.
+struct GemmNT {
+    const uint16_t* A;  int64_t lda, a_batch;   // [M, K]
+    const uint16_t* Bt; int64_t ldb, b_batch;   // [N, K]
+    float* C;           int64_t ldc, c_batch;   // [M, N]
+    int M, N, K, batches;
+    const char* add_base; int64_t add_pitch; int add_etype;
+    const uint32_t* add_index; const uint32_t* add_count;
+};
+bool gemm_nt_bf16_ok(int M, int N, int K);
+void launch_gemm_nt_bf16(const GemmNT& g, hipStream_t stream);
+// in[z][rows, cols] (float32 or bfloat16) -> out_t[z][cols, rows] bfloat16 and, unless null,
+// out[z][rows, cols] bfloat16; rows % 64 == 0, cols % 64 == 0
+void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, int cols, int64_t ld_in,
+                           int64_t in_batch, uint16_t* out_t, uint16_t* out, hipStream_t stream);
 
 // Scores of every block: a-operand row (d,b) = entity row of contribution
 // d*B+b combined with relation crel[d*B+b]; b-operand row (d,t) = entity row of

@@ -414,7 +414,8 @@ void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sort
 __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const float* __restrict__ rel,
                                                          const uint32_t* __restrict__ crel,
                                                          int rel_mode, int n_head, int n_rows, int Dp,
-                                                         float* __restrict__ out) {
+                                                         float* __restrict__ out,
+                                                         uint16_t* __restrict__ out16) {
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (c >= n_rows) return;
@@ -426,16 +427,26 @@ __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const fl
         // + 0 turns a -0 into +0, so that a difference of stored operands is never -0
         // (the paired L1 backward reads the sign off the difference's bit pattern)
         v.x += 0.f; v.y += 0.f; v.z += 0.f; v.w += 0.f;
+        if (out16) {
+            // bfloat16 scoring: the operands are rounded once, here; the float32 copy holds
+            // the same rounded values, so every scoring kernel computes the same products
+            const uint16_t h0 = f32_to_bf16(v.x), h1 = f32_to_bf16(v.y), h2 = f32_to_bf16(v.z), h3 = f32_to_bf16(v.w);
+            uint2 raw;
+            raw.x = (uint32_t)h0 | ((uint32_t)h1 << 16);
+            raw.y = (uint32_t)h2 | ((uint32_t)h3 << 16);
+            *reinterpret_cast<uint2*>(out16 + (size_t)c * Dp + k) = raw;
+            v = make_float4(bf16_to_f32(h0), bf16_to_f32(h1), bf16_to_f32(h2), bf16_to_f32(h3));
+        }
         *reinterpret_cast<float4*>(out + (size_t)c * Dp + k) = v;
     }
 }
 
 void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
-                            int n_head, int n_rows, int Dp, float* out, hipStream_t stream) {
+                            int n_head, int n_rows, int Dp, float* out, uint16_t* out16,
+                            hipStream_t stream) {
     hipLaunchKernelGGL(k_gather_operands, dim3((n_rows + 3) / 4), dim3(256), 0, stream, ent, rel, crel,
-                       rel_mode, n_head, n_rows, Dp, out);
+                       rel_mode, n_head, n_rows, Dp, out, out16);
 }
-
 
 // --------------------------------------------------------------------------
 // Tile order.  The scoring kernels run gx * gy tiles for each of gz blocks; a
@@ -975,6 +986,137 @@ void launch_score_fwd(const ScoreShape& sh, const RowSource& ent, const float* r
     p.out_mode = fused_loss ? 0 : 1;
     p.a_c0 = 0; p.b_c0 = sh.S * sh.B;
     launch_fwd(p, stream);
+}
+
+
+// --------------------------------------------------------------------------
+// bfloat16 matrix-core products (execution.scoring_dtype = "bfloat16"):
+//   C[z][m, n] = sum_k A[z][m, k] * Bt[z][n, k],  bfloat16 in, float32 out,
+// with v_mfma_f32_32x32x16_bf16 (lane l supplies row l%32, columns
+// 8*(l/32) .. +7 of the 16-column step, for both operands).  Workgroup tile
+// 128 x 128, four waves as 2 x 2, each 2 x 2 accumulators of 32 x 32; K slabs of
+// 64 staged through LDS with 16-byte copies, the next slab in registers while
+// the current one is multiplied.  LDS rows are padded to 72 elements (144 B) so
+// that eight consecutive rows' 16-byte reads fall in different banks.
+// Shapes: M % 128 == 0, N % 128 == 0, K % 64 == 0, rows 16-byte aligned.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int GB_T = 128, GB_K = 64, GB_LD = GB_K + 8;
+
+__global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
+    __shared__ __attribute__((aligned(16))) uint16_t As[GB_T][GB_LD];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[GB_T][GB_LD];
+    const TileId tile = xcd_tile(g.N / GB_T, g.M / GB_T, g.batches);
+    const int z = tile.z, m0 = tile.y * GB_T, n0 = tile.x * GB_T;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int hl = lane >> 5, cl = lane & 31;
+    const uint16_t* A = g.A + (size_t)z * g.a_batch + (size_t)m0 * g.lda;
+    const uint16_t* Bt = g.Bt + (size_t)z * g.b_batch + (size_t)n0 * g.ldb;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // staging: 128 rows x 64 columns = 1024 16-byte pieces per operand, four per thread
+    floatx4 areg[4], breg[4];
+    auto prefetch = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+            const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
+            areg[h] = *reinterpret_cast<const floatx4*>(A + (size_t)row * g.lda + k0 + col);
+            breg[h] = *reinterpret_cast<const floatx4*>(Bt + (size_t)row * g.ldb + k0 + col);
+        }
+    };
+    prefetch(0);
+    for (int k0 = 0; k0 < g.K; k0 += GB_K) {
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+            const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
+            *reinterpret_cast<floatx4*>(&As[row][col]) = areg[h];
+            *reinterpret_cast<floatx4*>(&Bs[row][col]) = breg[h];
+        }
+        __syncthreads();
+        if (k0 + GB_K < g.K) prefetch(k0 + GB_K);
+        floatx4 fa[2][2], fb[2][2];
+        auto fetch = [&](int buf, int ks) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[buf][i] = *reinterpret_cast<const floatx4*>(&As[wm + 32 * i + cl][16 * ks + 8 * hl]);
+                fb[buf][i] = *reinterpret_cast<const floatx4*>(&Bs[wn + 32 * i + cl][16 * ks + 8 * hl]);
+            }
+        };
+        fetch(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < GB_K / 16; ++ks) {
+            if (ks + 1 < GB_K / 16) fetch((ks + 1) & 1, ks + 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8, fa[ks & 1][i]), __builtin_bit_cast(bf16x8, fb[ks & 1][j]),
+                        acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+    }
+    // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32
+    float* C = g.C + (size_t)z * g.c_batch;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = m0 + wm + 32 * i + 8 * (r >> 2) + 4 * hl + (r & 3);
+            uint32_t add_row = 0;
+            if (g.add_base) add_row = (uint32_t)m < *g.add_count ? g.add_index[m] : 0u;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int n = n0 + wn + 32 * j + cl;
+                float o = acc[i][j][r];
+                if (g.add_base) o += load1(g.add_base + (int64_t)add_row * g.add_pitch, n, g.add_etype);
+                C[(size_t)m * g.ldc + n] = o;
+            }
+        }
+}
+
+bool gemm_nt_bf16_ok(int M, int N, int K) { return M % GB_T == 0 && N % GB_T == 0 && K % GB_K == 0; }
+
+void launch_gemm_nt_bf16(const GemmNT& g, hipStream_t stream) {
+    hipLaunchKernelGGL(k_gemm_nt_bf16, tile_grid(g.N / GB_T, g.M / GB_T, g.batches), dim3(256), 0, stream, g);
+}
+
+// Transposing cast: in[z][r, c] (float32 or bfloat16, row pitch ld_in) ->
+// out_t[z][c, r] bfloat16 (dense) and, if asked, out[z][r, c] bfloat16 (dense).
+// 64 x 64 tiles through LDS; rows and cols multiples of 64.
+__global__ __launch_bounds__(256) void k_transpose_bf16(const void* __restrict__ in, int in_f32,
+                                                        int rows, int cols, int64_t ld_in,
+                                                        int64_t in_batch, uint16_t* __restrict__ out_t,
+                                                        uint16_t* __restrict__ out) {
+    __shared__ uint16_t tile[64][66];
+    const int z = blockIdx.z, r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4) {
+        const size_t off = (size_t)z * in_batch + (size_t)(r0 + r) * ld_in + c0 + tx;
+        const uint16_t h = in_f32 ? f32_to_bf16(reinterpret_cast<const float*>(in)[off])
+                                  : reinterpret_cast<const uint16_t*>(in)[off];
+        tile[r][tx] = h;
+        if (out) out[((size_t)z * rows + r0 + r) * cols + c0 + tx] = h;
+    }
+    __syncthreads();
+    for (int c = ty; c < 64; c += 4)
+        out_t[((size_t)z * cols + c0 + c) * rows + r0 + tx] = tile[tx][c];
+}
+
+void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, int cols, int64_t ld_in,
+                           int64_t in_batch, uint16_t* out_t, uint16_t* out, hipStream_t stream) {
+    hipLaunchKernelGGL(k_transpose_bf16, dim3(cols / 64, rows / 64, batches), dim3(256), 0, stream, in,
+                       in_f32 ? 1 : 0, rows, cols, ld_in, in_batch, out_t, out);
 }
 
 // --------------------------------------------------------------------------

@@ -48,6 +48,9 @@ typedef struct {
     int32_t loss_fn;        /* LOSS_*                                           */
     int32_t shared_table;   /* 1: every shard addresses the same n_entity rows  */
     int32_t storage;        /* STORE_*: rounding applied on row write-back      */
+    int32_t scoring_bf16;   /* 1: predicted tails and tails rounded to bfloat16
+                             * before the dot product (products exact, sums in
+                             * REAL); gradients pass straight through the rounding */
     float gamma;
     float beta_m, beta_v, epsilon, weight_decay;
     float loss_scale;
@@ -457,6 +460,11 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             for (int64_t i = 0; i < A; ++i)
                 memcpy(tl + (j * A + i) * D, hidden + (j * NR + a2a[(j * S + d) * A + i]) * D,
                        sizeof(REAL) * (size_t)D);
+
+        if (c->scoring_bf16) {
+            for (int64_t x = 0; x < B * D; ++x) p[x] = (REAL)round_bf16((float)p[x]);
+            for (int64_t x = 0; x < T * D; ++x) tl[x] = (REAL)round_bf16((float)tl[x]);
+        }
 
         /* 3. scores (:492-499, :571-573, :469-486) */
         const int dot = (c->score_fn == SCORE_DISTMULT) || c->distance_fn == DIST_DOT;

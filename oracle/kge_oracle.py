@@ -23,7 +23,7 @@ STORE = {"float32": 0, "float16": 1, "bfloat16_embedding": 2}
 class Cfg(C.Structure):
     _fields_ = [(n, C.c_int32) for n in (
         "n_shard", "n_entity", "n_relation", "dim", "feature", "batch", "a2a", "score_fn",
-        "distance_fn", "loss_fn", "shared_table", "storage")] + [(n, C.c_float) for n in (
+        "distance_fn", "loss_fn", "shared_table", "storage", "scoring_bf16")] + [(n, C.c_float) for n in (
             "gamma", "beta_m", "beta_v", "epsilon", "weight_decay", "loss_scale",
             "softmax_correction_weight", "negative_adversarial_scale", "lr_mod_entity",
             "lr_mod_relation", "lr_mod_projection")]
@@ -31,13 +31,14 @@ class Cfg(C.Structure):
 
 def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score_fn="TransE",
              distance_fn="L1", loss_fn="logsigmoid", shared_table=False, storage="float32",
-             gamma=0.0, beta_m=0.9, beta_v=0.999, epsilon=1e-8, weight_decay=0.0,
+             scoring_bf16=False, gamma=0.0, beta_m=0.9, beta_v=0.999, epsilon=1e-8, weight_decay=0.0,
              loss_scale=None, softmax_correction_weight=0.0, negative_adversarial_scale=0.0,
              lr_mod_entity=1.0, lr_mod_relation=1.0, lr_mod_projection=1.0):
     if loss_scale is None:  # src/python/poplar_kge.py:259-262
         loss_scale = float(batch * n_shard * a2a)
     return Cfg(n_shard, n_entity, n_relation, dim, feature, batch, a2a, SCORE[score_fn],
-               DIST[distance_fn], LOSS[loss_fn], int(shared_table), STORE[storage], gamma, beta_m,
+               DIST[distance_fn], LOSS[loss_fn], int(shared_table), STORE[storage], int(scoring_bf16),
+               gamma, beta_m,
                beta_v, epsilon, weight_decay, loss_scale, softmax_correction_weight,
                negative_adversarial_scale, lr_mod_entity, lr_mod_relation, lr_mod_projection)
 

@@ -69,6 +69,8 @@ def engine_settings(c, n_step, rw_batch=64, **extra):
     }
     if c.get("storage") == "bfloat16_embedding":
         s["execution.embedding_dtype"] = "bfloat16"
+    if c.get("scoring_bf16"):
+        s["execution.scoring_dtype"] = "bfloat16"
     s.update(extra)
     return s
 

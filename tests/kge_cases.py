@@ -6,7 +6,7 @@ import numpy as np
 def cfg_dict(**kw):
     d = dict(n_shard=2, n_entity=90, n_relation=12, dim=8, feature=6, batch=6, a2a=5,
              score_fn="TransE", distance_fn="L1", loss_fn="logsigmoid", shared_table=False,
-             storage="float32", gamma=2.0, beta_m=0.9, beta_v=0.999, epsilon=1e-8,
+             storage="float32", scoring_bf16=False, gamma=2.0, beta_m=0.9, beta_v=0.999, epsilon=1e-8,
              weight_decay=0.0, loss_scale=None, softmax_correction_weight=0.0,
              negative_adversarial_scale=0.0)
     d.update(kw)

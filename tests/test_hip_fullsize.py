@@ -23,22 +23,22 @@ def _free_gpu_bytes():
     return torch.cuda.mem_get_info()[0]
 
 
-def _close_but_for_sign_flips(got, ref, what, max_flip_fraction=5e-4):
+def _close_but_for_sign_flips(got, ref, what, max_flip_fraction=5e-4, tol=1e-5):
     """Adam's first steps from zero moments move a parameter by about
     lr * sign(g): where a gradient element is an exact cancellation (common for
     L1, whose terms are +-c) its sign is decided by rounding, and float32 and
     float64 may disagree.  Such elements are allowed, rarely; all the others
     must agree to 1e-5."""
     scale = np.sqrt(np.mean(np.asarray(ref, np.float64)**2))
-    bad = np.abs(got - ref) > 1e-4 * scale
+    bad = np.abs(got - ref) > 10 * tol * scale
     assert bad.mean() < max_flip_fraction, (what, bad.mean())
-    assert K.rel_l2(np.where(bad, 0, got), np.where(bad, 0, ref)) < 1e-5, what
+    assert K.rel_l2(np.where(bad, 0, got), np.where(bad, 0, ref)) < tol, what
 
 
-def _run(workload, n_step, rng_rows=2000):
+def _run(workload, n_step, rng_rows=2000, **override):
     import poplar_kge as kge
 
-    w = bench.WORKLOADS[workload]
+    w = dict(bench.WORKLOADS[workload], **override)
     row_bytes = ((2 if w.get("embedding_dtype") else 4) * w["dim"] + 8 * w["dim"]
                  + (2 if w.get("feature_dtype") else 4) * w.get("feature", 0))
     need = w["n_entity"] * row_bytes + (4 << 30)
@@ -83,24 +83,30 @@ def _run(workload, n_step, rng_rows=2000):
                    loss_fn="softmax" if softmax else "logsigmoid",
                    softmax_correction_weight=1.0 if softmax else 0.0,
                    shared_table=True, gamma=m.gamma, loss_scale=settings.training.loss_scale,
-                   storage=storage)
+                   scoring_bf16=w.get("scoring_dtype") == "bfloat16", storage=storage)
     ob = {k: v for k, v in vars(batch).items()}
     ob["remote"] = remap(batch.remote)
     loss_o = Oracle("f64").train_step_loop(cfg, state, settings.training.learning_rate, ob)
-    np.testing.assert_allclose(loss, float(np.sum(loss_o)), rtol=1e-5)
+    # bfloat16 scoring: the oracle rounds the same operands, so the loss stays tight; the
+    # coefficient matrix is a bfloat16 operand of the backward products on the device only
+    # (2^-9 relative per element): gradients, and with them the moments, hold bf16's 2e-2 bar
+    bf16_scoring = w.get("scoring_dtype") == "bfloat16"
+    tol = 2e-2 if bf16_scoring else 1e-5
+    flips = 2e-2 if bf16_scoring else 5e-4   # cold-start sign flips of near-zero gradient elements
+    np.testing.assert_allclose(loss, float(np.sum(loss_o)), rtol=1e-4 if bf16_scoring else 1e-5)
     ref = state["entity_data"][1:]
     assert np.all(np.any(after != before, axis=1))       # every touched row moved
     if storage == "float32":
-        _close_but_for_sign_flips(after, ref, "entity rows")
+        _close_but_for_sign_flips(after, ref, "entity rows", flips, tol)
     else:
         assert K.rel_l2(after[:, D:], ref[:, D:]) < 1e-5          # float32 moments
         assert K.rel_l2(after[:, :D], ref[:, :D]) < 2e-3          # bfloat16 embedding (bar: 2e-2)
         assert np.mean(after[:, :D] != ref[:, :D]) < 2e-3
     for name in dense:
-        _close_but_for_sign_flips(engine.read_variable(name), state[name], name)
+        _close_but_for_sign_flips(engine.read_variable(name), state[name], name, flips, tol)
         # the dense tables keep v = E[g^2]; the bar is on |g|-like quantities, as for the rows' sqrt(v)
         assert K.rel_l2(np.sqrt(engine.read_variable(name + "/adam_v")),
-                        np.sqrt(state[name + "/adam_v"])) < 1e-5, name
+                        np.sqrt(state[name + "/adam_v"])) < tol, name
     return settings, batch, ids, after, loss
 
 
@@ -129,8 +135,13 @@ def test_c3_l2_full_size_vs_oracle():
 
 
 def test_c4_full_size_vs_oracle():
-    # DistMult + 768 -> 512 feature projection + softmax CE, 8192 x 2048 scores
+    # DistMult + 768 -> 512 feature projection + softmax CE, 8192 x 2048 scores,
+    # bfloat16 scoring operands on the matrix cores
     _run("c4", n_step=1)
+
+
+def test_c4_float32_scoring_full_size_vs_oracle():
+    _run("c4", n_step=1, scoring_dtype=None)
 
 
 def test_c5_full_size_vs_oracle():

@@ -55,6 +55,54 @@ CASES = {
 }
 
 
+# bfloat16 scoring (DistMult): operands rounded to bfloat16, float32 accumulation.  The oracle
+# rounds the same operands; the coefficient matrix is a bfloat16 operand of the two backward
+# products on the device only (2^-9 relative per element), hence the bar of 2e-2 on the update.
+BF16_SCORING_CASES = {
+    "aligned": dict(score_fn="DistMult", distance_fn="MatMul", loss_fn="softmax", softmax_correction_weight=1.0,
+                    n_shard=2, batch=128, a2a=64, dim=128, feature=0, n_entity=3000, n_relation=8,
+                    scoring_bf16=True),
+    "aligned_logsigmoid_shared": dict(score_fn="DistMult", distance_fn="MatMul", n_shard=4, batch=128, a2a=32,
+                                      dim=128, feature=0, n_entity=2000, n_relation=8, shared_table=True,
+                                      scoring_bf16=True),
+    "aligned_features": dict(score_fn="DistMult", distance_fn="MatMul", loss_fn="softmax",
+                             softmax_correction_weight=1.0, n_shard=1, batch=256, a2a=128, dim=128,
+                             feature=64, n_entity=3000, n_relation=8, shared_table=True, scoring_bf16=True),
+    "ragged_fallback": dict(score_fn="DistMult", distance_fn="MatMul", loss_fn="softmax",
+                            softmax_correction_weight=1.0, n_shard=2, batch=40, a2a=30, dim=64, feature=0,
+                            n_entity=1000, n_relation=8, scoring_bf16=True),
+}
+
+
+@pytest.mark.parametrize("name", list(BF16_SCORING_CASES))
+def test_step_bf16_scoring(oracle64, name):
+    import libpoplar_kge
+
+    c = K.cfg_dict(**BF16_SCORING_CASES[name])
+    rng = np.random.default_rng(21)
+    st0 = K.make_state(c, rng)
+    batch = K.random_batch(c, 2, rng)
+    lr = np.full(c["n_shard"], 0.05, np.float32)
+    engine = libpoplar_kge.Engine(H.engine_settings(c, 2), "")
+    H.load_state(engine, c, st0)
+    st_o = K.copy_state(st0)
+    loss_o = oracle64.train_step_loop(make_cfg(**c), st_o, lr, batch)
+    loss_h = H.train(engine, c, lr, batch)
+    np.testing.assert_allclose(loss_h, loss_o, rtol=1e-4)   # forward: same rounded operands
+    st_h = H.read_state(engine, c)
+    for k in st0:
+        if k == "step":
+            continue
+        assert K.rel_l2(st_h[k] - st0[k], st_o[k] - st0[k]) < 2e-2, k
+    # and the rounding is really what is compared: without it the oracle's update differs
+    # from the device's by more than the device differs from the rounding oracle
+    c32 = dict(c, scoring_bf16=False)
+    st_f = K.copy_state(st0)
+    oracle64.train_step_loop(make_cfg(**c32), st_f, lr, batch)
+    k = "relation_embedding"
+    assert K.rel_l2(st_f[k] - st0[k], st_o[k] - st0[k]) > 1e-4
+
+
 def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_loop=1, warm=True,
              **settings):
     import libpoplar_kge
