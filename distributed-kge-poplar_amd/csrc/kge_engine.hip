@@ -221,7 +221,7 @@ struct kge_engine {
     uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
     // step
     DevBuf<uint16_t> opnd16, opndT16, coef16, coefT16;  // bfloat16 scoring operands
-    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, loss_part, d_loss, d_alpha;
+    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, loss_part, d_loss, d_alpha;
     std::vector<float> h_alpha;  // [n_step][entity, relation, projection][S]
     int n_part;
     // io staging
@@ -474,6 +474,10 @@ void allocate(kge_engine& E) {
         E.opndT16.alloc(R * E.Dp);
         E.coef16.alloc(SB * E.T);
         E.coefT16.alloc(SB * E.T);
+        // split-contraction partials of the two backward products
+        const size_t p_head = (size_t)E.S * gemm_nt_bf16_ksplit(E.B, E.Dp, E.T, E.S) * E.B * E.Dp;
+        const size_t p_tail = (size_t)E.S * gemm_nt_bf16_ksplit(E.T, E.Dp, E.B, E.S) * E.T * E.Dp;
+        E.gemm_part.alloc(std::max(p_head, p_tail));
     }
     E.grad.alloc(R * E.Dp);
     E.opnd.alloc(R * E.Dp);
@@ -791,17 +795,17 @@ void run_step(kge_engine& E, int i) {
           g.C = E.coef.p; g.ldc = Tn; g.c_batch = (int64_t)Bn * Tn;
           g.M = Bn; g.N = Tn; g.K = Dp;
           launch_gemm_nt_bf16(g, st); }
-        { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, nullptr, loss_part, st); }
+        { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, nullptr, loss_part, E.coef16.p, st); }
         { KernelTimer t(E, K_BWD);
           launch_transpose_bf16(E.opnd16.p, false, E.S, Bn, Dp, Dp, (int64_t)Bn * Dp, E.opndT16.p, nullptr, st);
           launch_transpose_bf16(E.opnd16.p + head_n, false, E.S, Tn, Dp, Dp, (int64_t)Tn * Dp,
                                 E.opndT16.p + head_n, nullptr, st);
-          launch_transpose_bf16(E.coef.p, true, E.S, Bn, Tn, Tn, (int64_t)Bn * Tn, E.coefT16.p, E.coef16.p, st);
+          launch_transpose_bf16(E.coef16.p, false, E.S, Bn, Tn, Tn, (int64_t)Bn * Tn, E.coefT16.p, nullptr, st);
           // d q [B, Dp] = c [B, T] . tails [T, Dp]
           g.A = E.coef16.p; g.lda = Tn; g.a_batch = (int64_t)Bn * Tn;
           g.Bt = E.opndT16.p + head_n; g.ldb = Tn; g.b_batch = (int64_t)Dp * Tn;
           g.C = E.grad.p; g.ldc = Dp; g.c_batch = (int64_t)Bn * Dp;
-          g.M = Bn; g.N = Dp; g.K = Tn;
+          g.M = Bn; g.N = Dp; g.K = Tn; g.part = E.gemm_part.p;
           launch_gemm_nt_bf16(g, st);
           // d tails [T, Dp] = c^T [T, B] . q [B, Dp]
           g.A = E.coefT16.p; g.lda = Bn; g.a_batch = (int64_t)Tn * Bn;
@@ -812,7 +816,7 @@ void run_step(kge_engine& E, int i) {
     } else {
         { KernelTimer t(E, K_FWD);
           launch_score_fwd(sh, dense, E.rel.p, crel, clabel, E.coef.p, E.dist.p, E.nearflag.p, loss_part, fused, st); }
-        if (!fused) { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, E.dist.p, loss_part, st); }
+        if (!fused) { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, E.dist.p, loss_part, nullptr, st); }
         { KernelTimer t(E, K_BWD); launch_score_bwd(sh, dense, E.rel.p, crel, E.coef.p, E.nearflag.p, E.grad.p, st); }
     }
 

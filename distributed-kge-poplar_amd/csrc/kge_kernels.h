@@ -102,10 +102,12 @@ struct GemmNT {
     const uint16_t* Bt; int64_t ldb, b_batch;   // [N, K]
     float* C;           int64_t ldc, c_batch;   // [M, N]
     int M, N, K, batches;
+    float* part; int ksplit;                    // scratch for split contractions (or null); set by the launcher
     const char* add_base; int64_t add_pitch; int add_etype;
     const uint32_t* add_index; const uint32_t* add_count;
 };
 bool gemm_nt_bf16_ok(int M, int N, int K);
+int gemm_nt_bf16_ksplit(int M, int N, int K, int batches);  // partials needed: batches * ksplit * M * N floats
 void launch_gemm_nt_bf16(const GemmNT& g, hipStream_t stream);
 // in[z][rows, cols] (float32 or bfloat16) -> out_t[z][cols, rows] bfloat16 and, unless null,
 // out[z][rows, cols] bfloat16; rows % 64 == 0, cols % 64 == 0
@@ -131,7 +133,7 @@ int score_fwd_parts(const ScoreShape& sh);
 // the raw scores in `coef` to backward coefficients in place; loss_part gets
 // S * B partial sums.
 void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef, const float* dist,
-                      float* loss_part, hipStream_t stream);
+                      float* loss_part, uint16_t* coef16, hipStream_t stream);
 
 // Gradient rows of every contribution: grad[c, :] for head contributions
 // (w.r.t. the predicted tail / the head-times-relation product) and tail

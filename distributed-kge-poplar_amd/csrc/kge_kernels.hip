@@ -1006,13 +1006,17 @@ constexpr int GB_T = 128, GB_K = 64, GB_LD = GB_K + 8;
 __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     __shared__ __attribute__((aligned(16))) uint16_t As[GB_T][GB_LD];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[GB_T][GB_LD];
-    const TileId tile = xcd_tile(g.N / GB_T, g.M / GB_T, g.batches);
-    const int z = tile.z, m0 = tile.y * GB_T, n0 = tile.x * GB_T;
+    // z = batch * ksplit + split: with ksplit > 1 every split multiplies its own K / ksplit
+    // columns into its own partial output [batch][split][M, N]
+    const TileId tile = xcd_tile(g.N / GB_T, g.M / GB_T, g.batches * g.ksplit);
+    const int zb = tile.z / g.ksplit, zs = tile.z - zb * g.ksplit;
+    const int m0 = tile.y * GB_T, n0 = tile.x * GB_T;
+    const int K = g.K / g.ksplit;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
     const int hl = lane >> 5, cl = lane & 31;
-    const uint16_t* A = g.A + (size_t)z * g.a_batch + (size_t)m0 * g.lda;
-    const uint16_t* Bt = g.Bt + (size_t)z * g.b_batch + (size_t)n0 * g.ldb;
+    const uint16_t* A = g.A + (size_t)zb * g.a_batch + (size_t)m0 * g.lda + (size_t)zs * K;
+    const uint16_t* Bt = g.Bt + (size_t)zb * g.b_batch + (size_t)n0 * g.ldb + (size_t)zs * K;
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -1033,7 +1037,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
         }
     };
     prefetch(0);
-    for (int k0 = 0; k0 < g.K; k0 += GB_K) {
+    for (int k0 = 0; k0 < K; k0 += GB_K) {
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
             const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
@@ -1041,7 +1045,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
             *reinterpret_cast<floatx4*>(&Bs[row][col]) = breg[h];
         }
         __syncthreads();
-        if (k0 + GB_K < g.K) prefetch(k0 + GB_K);
+        if (k0 + GB_K < K) prefetch(k0 + GB_K);
         floatx4 fa[2][2], fb[2][2];
         auto fetch = [&](int buf, int ks) __attribute__((always_inline)) {
 #pragma unroll
@@ -1067,7 +1071,8 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
         __syncthreads();
     }
     // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32
-    float* C = g.C + (size_t)z * g.c_batch;
+    float* C = g.ksplit > 1 ? g.part + ((size_t)zb * g.ksplit + zs) * ((size_t)g.M * g.ldc)
+                            : g.C + (size_t)zb * g.c_batch;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -1087,8 +1092,38 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
 
 bool gemm_nt_bf16_ok(int M, int N, int K) { return M % GB_T == 0 && N % GB_T == 0 && K % GB_K == 0; }
 
-void launch_gemm_nt_bf16(const GemmNT& g, hipStream_t stream) {
-    hipLaunchKernelGGL(k_gemm_nt_bf16, tile_grid(g.N / GB_T, g.M / GB_T, g.batches), dim3(256), 0, stream, g);
+// How many ways to split the contraction so that the launch has at least two
+// workgroups per CU (a power of two, at most 16, each split at least 256 columns).
+int gemm_nt_bf16_ksplit(int M, int N, int K, int batches) {
+    const long tiles = (long)(M / GB_T) * (N / GB_T) * batches;
+    int ks = 1;
+    while (ks < 16 && tiles * ks < 512 && K % (2 * ks * GB_K) == 0 && K / (2 * ks) >= 256) ks *= 2;
+    return ks;
+}
+
+// out[b][i] = sum over s of part[b][s][i], in order (n % 4 == 0); blockIdx.y = b
+__global__ __launch_bounds__(256) void k_sum_split_batches(const float* __restrict__ part, int ns, int64_t n,
+                                                           float* __restrict__ out, int64_t out_batch) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n) return;
+    const float* p = part + (size_t)blockIdx.y * ns * n + i;
+    float4 acc = *reinterpret_cast<const float4*>(p);
+    for (int s = 1; s < ns; ++s) acc = f4add(acc, *reinterpret_cast<const float4*>(p + (size_t)s * n));
+    *reinterpret_cast<float4*>(out + (size_t)blockIdx.y * out_batch + i) = acc;
+}
+
+// With g.part set the contraction may be split (gemm_nt_bf16_ksplit); the partial
+// products are added in split order.  Splitting needs ldc == N (dense partials).
+void launch_gemm_nt_bf16(const GemmNT& g0, hipStream_t stream) {
+    GemmNT g = g0;
+    g.ksplit = (g.part && g.ldc == g.N && !g.add_base) ? gemm_nt_bf16_ksplit(g.M, g.N, g.K, g.batches) : 1;
+    hipLaunchKernelGGL(k_gemm_nt_bf16, tile_grid(g.N / GB_T, g.M / GB_T, g.batches * g.ksplit), dim3(256), 0,
+                       stream, g);
+    if (g.ksplit > 1) {
+        const int64_t n = (int64_t)g.M * g.N;
+        hipLaunchKernelGGL(k_sum_split_batches, dim3((unsigned)((n / 4 + 255) / 256), g.batches), dim3(256), 0,
+                           stream, g.part, g.ksplit, n, g.C, g.c_batch);
+    }
 }
 
 // Transposing cast: in[z][r, c] (float32 or bfloat16, row pitch ld_in) ->
@@ -1098,19 +1133,35 @@ __global__ __launch_bounds__(256) void k_transpose_bf16(const void* __restrict__
                                                         int rows, int cols, int64_t ld_in,
                                                         int64_t in_batch, uint16_t* __restrict__ out_t,
                                                         uint16_t* __restrict__ out) {
-    __shared__ uint16_t tile[64][66];
+    // pitch of 66 elements: a column walk (the transposed read) steps 33 banks per row
+    __shared__ __attribute__((aligned(4))) uint16_t tile[64][66];
     const int z = blockIdx.z, r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    for (int r = ty; r < 64; r += 4) {
-        const size_t off = (size_t)z * in_batch + (size_t)(r0 + r) * ld_in + c0 + tx;
-        const uint16_t h = in_f32 ? f32_to_bf16(reinterpret_cast<const float*>(in)[off])
-                                  : reinterpret_cast<const uint16_t*>(in)[off];
-        tile[r][tx] = h;
-        if (out) out[((size_t)z * rows + r0 + r) * cols + c0 + tx] = h;
+    const int q = (threadIdx.x & 15) * 4, lr = threadIdx.x >> 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = lr + 16 * i;
+        const size_t off = (size_t)z * in_batch + (size_t)(r0 + r) * ld_in + c0 + q;
+        uint2 raw;
+        if (in_f32) {
+            const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(in) + off);
+            raw.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+            raw.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+        } else {
+            raw = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(in) + off);
+        }
+        *reinterpret_cast<uint32_t*>(&tile[r][q]) = raw.x;
+        *reinterpret_cast<uint32_t*>(&tile[r][q + 2]) = raw.y;
+        if (out) *reinterpret_cast<uint2*>(out + ((size_t)z * rows + r0 + r) * cols + c0 + q) = raw;
     }
     __syncthreads();
-    for (int c = ty; c < 64; c += 4)
-        out_t[((size_t)z * cols + c0 + c) * rows + r0 + tx] = tile[tx][c];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = lr + 16 * i;
+        uint2 raw;
+        raw.x = (uint32_t)tile[q][c] | ((uint32_t)tile[q + 1][c] << 16);
+        raw.y = (uint32_t)tile[q + 2][c] | ((uint32_t)tile[q + 3][c] << 16);
+        *reinterpret_cast<uint2*>(out_t + ((size_t)z * cols + c0 + c) * rows + r0 + q) = raw;
+    }
 }
 
 void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, int cols, int64_t ld_in,
@@ -1127,12 +1178,14 @@ void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, i
 __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t* __restrict__ clabel,
                                                    float* __restrict__ coef,
                                                    const float* __restrict__ dist,
-                                                   float* __restrict__ loss_part) {
+                                                   float* __restrict__ loss_part,
+                                                   uint16_t* __restrict__ coef16) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // d*B + b
     if (row >= sh.S * sh.B) return;
     const int T = sh.T;
     float* s = coef + (size_t)row * T;
+    uint16_t* s16 = coef16 ? coef16 + (size_t)row * T : nullptr;  // bfloat16 copy for the matrix cores
     const float* dr = dist ? dist + (size_t)row * T : nullptr;
     const uint32_t label = clabel[row];
     float loss = 0.f;
@@ -1154,6 +1207,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
             float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;
             if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
             s[t] = c;
+            if (s16) s16[t] = f32_to_bf16(c);
         }
     } else {
         const float adv = sh.negative_adversarial_scale;
@@ -1184,6 +1238,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
             float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;
             if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
             s[t] = c;
+            if (s16) s16[t] = f32_to_bf16(c);
         }
     }
     loss = wave_sum(loss);
@@ -1191,11 +1246,11 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
 }
 
 void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef, const float* dist,
-                      float* loss_part, hipStream_t stream) {
+                      float* loss_part, uint16_t* coef16, hipStream_t stream) {
     const int rows = sh.S * sh.B;
     const bool l2 = sh.score_fn == SCORE_TRANSE && sh.dist_fn == DIST_L2;
     hipLaunchKernelGGL(k_loss_rows, dim3((rows + 3) / 4), dim3(256), 0, stream, sh, clabel, coef,
-                       l2 ? dist : nullptr, loss_part);
+                       l2 ? dist : nullptr, loss_part, coef16);
 }
 
 // --------------------------------------------------------------------------
