@@ -220,8 +220,8 @@ struct kge_engine {
     int e_ustride, e_cstride, r_ustride, r_cstride, n_rel_items;
     uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
     // step
-    DevBuf<uint16_t> opnd16, opndT16, coef16, coefT16;  // bfloat16 scoring operands
-    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, loss_part, d_loss, d_alpha;
+    DevBuf<uint16_t> opnd16, opndT16, coef16, coefT16, feat16, featT16, projT16, gT16;  // bfloat16 scoring operands
+    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, d_loss, d_alpha;
     std::vector<float> h_alpha;  // [n_step][entity, relation, projection][S]
     int n_part;
     // io staging
@@ -490,6 +490,13 @@ void allocate(kge_engine& E) {
         E.gsum.zero(E.stream);  // rows past a step's distinct count are read (times zero): keep them finite
         E.featd.alloc(R * E.Fp);
         E.gproj_part.alloc((size_t)16 * E.Fp * E.Dp);
+        if (E.score_bf16) {
+            E.feat16.alloc(R * E.Fp);
+            E.featT16.alloc(R * E.Fp);
+            E.projT16.alloc((size_t)E.Fp * E.Dp);
+            E.gT16.alloc(R * E.Dp);
+            E.projR.alloc((size_t)E.Fp * E.Dp);
+        }
         E.gproj.alloc(proj_n);
     }
     ScoreShape sh = {};
@@ -764,6 +771,8 @@ void run_step(kge_engine& E, int i) {
         fa.emb_etype = E.L.emb_etype; fa.feat_etype = E.L.feat_etype;
         fa.Dp = E.Dp; fa.Fp = E.Fp; fa.proj = E.proj.p;
         fa.featd = E.featd.p; fa.gproj_part = E.gproj_part.p; fa.use_mfma = E.use_mfma;
+        fa.round_bf16 = E.score_bf16 ? 1 : 0; fa.projR = E.projR.p;
+        fa.feat16 = E.feat16.p; fa.featT16 = E.featT16.p; fa.projT16 = E.projT16.p; fa.gT16 = E.gT16.p;
         { KernelTimer t(E, K_HIDDEN); launch_hidden_fwd(fa, E.hidden.p, st); }
         ent.base = (const char*)E.hidden.p; ent.pitch = (int64_t)E.Dp * 4; ent.etype = ET_F32;
         ent.index = E.e_item_row.p + i * R;

@@ -216,6 +216,11 @@ struct FeatureArgs {
     float* featd;           // scratch [max_rows, Fp]: the distinct rows' features, float32
     float* gproj_part;      // scratch [16, Fp, Dp]: split-contraction partials of the projection gradient
     int use_mfma;
+    // bfloat16 products (null without bfloat16 scoring): features [max_rows, Fp] and their
+    // transpose, W^T [Dp, Fp], grad_rows^T [Dp, max_rows]
+    uint16_t *feat16, *featT16, *projT16, *gT16;
+    int round_bf16;         // features and W enter their products rounded to bfloat16
+    float* projR;           // scratch [Fp, Dp]: W rounded, for the float32 kernels
 };
 void launch_hidden_fwd(const FeatureArgs& a, float* hidden, hipStream_t stream);
 // gproj[f, :] = sum_u feature[u, f] * grad_rows[u, :]

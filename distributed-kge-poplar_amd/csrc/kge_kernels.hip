@@ -60,6 +60,10 @@ DEVINL void store4(char* row, int k, int etype, float4 v) {
 
 // guarded variant for sources whose rows are not 16-byte aligned or whose
 // length is not a multiple of four (standalone ops on arbitrary shapes)
+DEVINL float4 round4_bf16(float4 v) {
+    return make_float4(bf16_to_f32(f32_to_bf16(v.x)), bf16_to_f32(f32_to_bf16(v.y)),
+                       bf16_to_f32(f32_to_bf16(v.z)), bf16_to_f32(f32_to_bf16(v.w)));
+}
 DEVINL float load1(const char* sec, int k, int etype) {
     if (etype == ET_F32) return reinterpret_cast<const float*>(sec)[k];
     if (etype == ET_BF16) return bf16_to_f32(reinterpret_cast<const uint16_t*>(sec)[k]);
@@ -2072,11 +2076,13 @@ __global__ __launch_bounds__(256) void k_hidden_fwd(FeatureArgs a, float* __rest
     for (int k = lane * 4; k < a.Dp; k += 256) {
         float4 h = load4(erow, k, a.emb_etype);
         for (int f = 0; f < a.Fp; f += 4) {
-            const float4 x = load4(frow, f, a.feat_etype);
+            float4 x = load4(frow, f, a.feat_etype);
+            if (a.round_bf16) x = round4_bf16(x);
             const float xv[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float4 w = *reinterpret_cast<const float4*>(a.proj + (size_t)(f + i) * a.Dp + k);
+                float4 w = *reinterpret_cast<const float4*>(a.proj + (size_t)(f + i) * a.Dp + k);
+                if (a.round_bf16) w = round4_bf16(w);
                 h.x = fmaf(xv[i], w.x, h.x); h.y = fmaf(xv[i], w.y, h.y);
                 h.z = fmaf(xv[i], w.z, h.z); h.w = fmaf(xv[i], w.w, h.w);
             }
@@ -2087,7 +2093,8 @@ __global__ __launch_bounds__(256) void k_hidden_fwd(FeatureArgs a, float* __rest
 
 // The distinct rows' features as dense float32 [max_rows, Fp], rows past the
 // count zero: the operand both feature products read.  One wave per row.
-__global__ __launch_bounds__(256) void k_gather_features(FeatureArgs a, float* __restrict__ featd) {
+__global__ __launch_bounds__(256) void k_gather_features(FeatureArgs a, float* __restrict__ featd,
+                                                         uint16_t* __restrict__ feat16) {
     const int lane = threadIdx.x & 63;
     const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (u >= a.max_rows) return;
@@ -2095,8 +2102,28 @@ __global__ __launch_bounds__(256) void k_gather_features(FeatureArgs a, float* _
     const char* frow = a.feat_base + (int64_t)(live ? a.uniq_key[u] : 0u) * a.pitch;
     for (int f = lane * 4; f < a.Fp; f += 256) {
         const float4 x = live ? load4(frow, f, a.feat_etype) : make_float4(0, 0, 0, 0);
-        *reinterpret_cast<float4*>(featd + (size_t)u * a.Fp + f) = x;
+        if (feat16) {
+            uint2 raw;
+            raw.x = (uint32_t)f32_to_bf16(x.x) | ((uint32_t)f32_to_bf16(x.y) << 16);
+            raw.y = (uint32_t)f32_to_bf16(x.z) | ((uint32_t)f32_to_bf16(x.w) << 16);
+            *reinterpret_cast<uint2*>(feat16 + (size_t)u * a.Fp + f) = raw;
+        } else {
+            *reinterpret_cast<float4*>(featd + (size_t)u * a.Fp + f) = a.round_bf16 ? round4_bf16(x) : x;
+        }
     }
+}
+
+// out = in rounded to bfloat16 (kept as float32); n % 4 == 0
+__global__ __launch_bounds__(256) void k_round_bf16_copy(const float* __restrict__ in, int64_t n,
+                                                         float* __restrict__ out) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i < n) *reinterpret_cast<float4*>(out + i) = round4_bf16(*reinterpret_cast<const float4*>(in + i));
+}
+
+// bfloat16 feature products (with bfloat16 scoring): both are C = A . Bt^T products
+static bool feature_bf16_ok(const FeatureArgs& a) {
+    return a.use_mfma && a.feat16 && gemm_nt_bf16_ok(a.max_rows, a.Dp, a.Fp) &&
+           gemm_nt_bf16_ok(a.Fp, a.Dp, a.max_rows);
 }
 
 static bool feature_mfma_ok(const FeatureArgs& a) {
@@ -2114,13 +2141,34 @@ static RowSource dense_rows(const float* base, int cols) {
 // product on the matrix cores (the scoring backward's dot kernel: coefficient
 // matrix = dense features, other rows = W), the embedding added in its epilogue.
 void launch_hidden_fwd(const FeatureArgs& a, float* hidden, hipStream_t stream) {
+    if (feature_bf16_ok(a)) {
+        // hidden [U, Dp] = features [U, Fp] . W [Fp, Dp] + embedding: A = features, Bt = W^T
+        hipLaunchKernelGGL(k_gather_features, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a,
+                           (float*)nullptr, a.feat16);
+        launch_transpose_bf16(a.proj, true, 1, a.Fp, a.Dp, a.Dp, 0, a.projT16, nullptr, stream);
+        GemmNT g = {};
+        g.A = a.feat16; g.lda = a.Fp; g.Bt = a.projT16; g.ldb = a.Fp; g.C = hidden; g.ldc = a.Dp;
+        g.M = a.max_rows; g.N = a.Dp; g.K = a.Fp; g.batches = 1;
+        g.add_base = a.emb_base; g.add_pitch = a.pitch; g.add_etype = a.emb_etype;
+        g.add_index = a.uniq_key; g.add_count = a.counts;
+        launch_gemm_nt_bf16(g, stream);
+        return;
+    }
     if (!feature_mfma_ok(a)) {
         hipLaunchKernelGGL(k_hidden_fwd, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, hidden);
         return;
     }
-    hipLaunchKernelGGL(k_gather_features, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, a.featd);
+    hipLaunchKernelGGL(k_gather_features, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, a.featd,
+                       (uint16_t*)nullptr);
+    const float* w = a.proj;
+    if (a.round_bf16) {  // bfloat16 operands at shapes the bfloat16 product does not take
+        const int64_t n = (int64_t)a.Fp * a.Dp;
+        hipLaunchKernelGGL(k_round_bf16_copy, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, stream,
+                           a.proj, n, a.projR);
+        w = a.projR;
+    }
     BwdParams p = {};
-    p.ent_a = p.ent_b = dense_rows(a.proj, a.Dp);
+    p.ent_a = p.ent_b = dense_rows(w, a.Dp);
     p.coef = a.featd; p.grad = hidden;
     p.S = 1; p.B = a.max_rows; p.T = a.Fp; p.Dp = a.Dp;
     p.side_b = 0; p.vec_out = 1; p.use_mfma = 1;
@@ -2144,6 +2192,7 @@ __global__ __launch_bounds__(256) void k_proj_grad(FeatureArgs a, const float* _
         if (a.feat_etype == ET_F32) x = reinterpret_cast<const float*>(frow)[f];
         else if (a.feat_etype == ET_F16) x = __half2float(reinterpret_cast<const __half*>(frow)[f]);
         else x = bf16_to_f32(reinterpret_cast<const uint16_t*>(frow)[f]);
+        if (a.round_bf16) x = bf16_to_f32(f32_to_bf16(x));
         const float4 g = *reinterpret_cast<const float4*>(grad_rows + (size_t)u * a.Dp + k);
         acc.x = fmaf(x, g.x, acc.x); acc.y = fmaf(x, g.y, acc.y);
         acc.z = fmaf(x, g.z, acc.z); acc.w = fmaf(x, g.w, acc.w);
@@ -2163,6 +2212,18 @@ __global__ __launch_bounds__(256) void k_sum_splits(const float* __restrict__ pa
 
 void launch_proj_grad(const FeatureArgs& a, const float* grad_rows, float* gproj,
                       hipStream_t stream) {
+    if (feature_bf16_ok(a)) {
+        // gproj [Fp, Dp] = features^T [Fp, U] . grad_rows [U, Dp]: A = features^T, Bt = grad_rows^T;
+        // rows past the distinct count are zero in the features and finite in grad_rows
+        launch_transpose_bf16(a.feat16, false, 1, a.max_rows, a.Fp, a.Fp, 0, a.featT16, nullptr, stream);
+        launch_transpose_bf16(grad_rows, true, 1, a.max_rows, a.Dp, a.Dp, 0, a.gT16, nullptr, stream);
+        GemmNT g = {};
+        g.A = a.featT16; g.lda = a.max_rows; g.Bt = a.gT16; g.ldb = a.max_rows; g.C = gproj; g.ldc = a.Dp;
+        g.M = a.Fp; g.N = a.Dp; g.K = a.max_rows; g.batches = 1;
+        g.part = a.gproj_part;  // [16, Fp, Dp]: room for every split
+        launch_gemm_nt_bf16(g, stream);
+        return;
+    }
     if (feature_mfma_ok(a)) {
         // gproj = features^T . grad_rows, [Fp x U] . [U x Dp]: the dot kernel's tail side
         // (coefficient rows run along the contraction).  Rows past the distinct count

@@ -49,8 +49,9 @@ typedef struct {
     int32_t shared_table;   /* 1: every shard addresses the same n_entity rows  */
     int32_t storage;        /* STORE_*: rounding applied on row write-back      */
     int32_t scoring_bf16;   /* 1: predicted tails and tails rounded to bfloat16
-                             * before the dot product (products exact, sums in
-                             * REAL); gradients pass straight through the rounding */
+                             * before the dot product, features and projection
+                             * before theirs (products exact, sums in REAL);
+                             * gradients pass straight through the rounding      */
     float gamma;
     float beta_m, beta_v, epsilon, weight_decay;
     float loss_scale;
@@ -431,9 +432,11 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             REAL* h = hidden + (s * NR + j) * D;
             for (int64_t k = 0; k < D; ++k) h[k] = row[k];
             for (int64_t f = 0; f < F; ++f) {
-                const REAL x = row[3 * D + f];
+                /* bfloat16 scoring also takes the projection's operands in bfloat16 */
+                const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
                 if (x != 0)
-                    for (int64_t k = 0; k < D; ++k) h[k] += x * (REAL)proj[f * D + k];
+                    for (int64_t k = 0; k < D; ++k)
+                        h[k] += x * (REAL)(c->scoring_bf16 ? round_bf16(proj[f * D + k]) : proj[f * D + k]);
             }
         }
 
@@ -575,7 +578,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                 const float* row = table + KEY(s, j) * ROW;
                 const REAL* gh = ghid + (s * NR + j) * D;
                 for (int64_t f = 0; f < F; ++f) {
-                    const REAL x = row[3 * D + f];
+                    const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
                     if (x != 0)
                         for (int64_t k = 0; k < D; ++k) gproj[f * D + k] += x * gh[k];
                 }
