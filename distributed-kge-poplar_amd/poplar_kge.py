@@ -250,6 +250,31 @@ class Batch:
     tail: np.ndarray
 
 
+@dataclasses.dataclass
+class Predictions:
+    """Best tails per query, as (shard, row) pairs (reference :435-470).
+
+    shard_idx  uint32[..., n_best, 2]
+    score      float32[..., n_best]
+    """
+
+    shard_idx: np.ndarray
+    score: np.ndarray
+
+    def _take(self, order: np.ndarray) -> "Predictions":
+        # order: int[..., k] positions along the n_best axis
+        return Predictions(shard_idx=np.take_along_axis(self.shard_idx, order[..., None], axis=-2),
+                           score=np.take_along_axis(self.score, order, axis=-1))
+
+    def topk(self, k: int) -> "Predictions":
+        """The k best of every item, in no particular order."""
+        return self._take(np.argpartition(self.score, -k, axis=-1)[..., -k:])
+
+    def sort(self) -> "Predictions":
+        """Every item's predictions by descending score."""
+        return self._take(np.argsort(self.score, axis=-1)[..., ::-1])
+
+
 KERNEL_NAMES = ("plan", "hidden_fwd", "gather_operands", "score_fwd", "loss_rows", "score_bwd", "reduce_entity",
                 "adam_entity", "reduce_relation", "adam_relation", "proj_grad", "adam_proj")
 
