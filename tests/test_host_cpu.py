@@ -102,3 +102,22 @@ def test_learning_rate_schedules():
     np.testing.assert_allclose(
         _schedule(kge.SteppedLearningRateDecay(step=20, multiplier=0.5), 6),
         [0.1, 0.1, 0.05, 0.025, 0.025, 0.0125])
+
+
+def test_predictions_topk():
+    # the known-answer vector of the reference's test (tests/python/test_poplar_kge.py:15-46)
+    import poplar_kge as kge
+
+    pre = kge.Predictions(
+        shard_idx=np.array([[[10, 100], [20, 200], [30, 300], [40, 400]],
+                            [[50, 500], [60, 600], [70, 700], [80, 800]]]),
+        score=np.array([[2, 1, 3, 0], [-4, -3, -2, -1]]))
+    post = pre.topk(k=3).sort()
+    assert post.shard_idx.shape == (2, 3, 2) and post.score.shape == (2, 3)
+    np.testing.assert_equal(post.shard_idx, [[[30, 300], [10, 100], [20, 200]],
+                                             [[80, 800], [70, 700], [60, 600]]])
+    np.testing.assert_equal(post.score, [[3, 2, 1], [-1, -2, -3]])
+    multi = kge.Predictions(pre.shard_idx[:, np.newaxis], pre.score[:, np.newaxis]).topk(k=3).sort()
+    assert multi.shard_idx.shape == (2, 1, 3, 2) and multi.score.shape == (2, 1, 3)
+    np.testing.assert_equal(multi.shard_idx[:, 0], post.shard_idx)
+    np.testing.assert_equal(multi.score[:, 0], post.score)
