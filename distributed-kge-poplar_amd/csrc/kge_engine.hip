@@ -191,6 +191,7 @@ struct kge_engine {
     float lr_mod_entity = 1.f, lr_mod_rel = 1.f, lr_mod_proj = 1.f;
     uint32_t seed;
     int n_step, rw_batch;
+    int predict_hr_batch = 0, predict_n_best = 0;
     int stream_kind;  // KGE_F32 or KGE_F16: dtype of the entity read/write streams
     bool profile_kernels = false;
     int use_mfma = 1;  // additive setting execution.scoring = "mfma" | "valu"
@@ -220,6 +221,9 @@ struct kge_engine {
     int e_ustride, e_cstride, r_ustride, r_cstride, n_rel_items;
     uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
     // step
+    // predict scratch (allocated by the first predict call)
+    DevBuf<uint32_t> p_idx, p_rel, p_count, p_best_i;
+    DevBuf<float> p_opnd, p_scores, p_best_s, p_hidden, p_featd;
     DevBuf<uint16_t> opnd16, opndT16, coef16, coefT16, feat16, featT16, projT16, gT16;  // bfloat16 scoring operands
     DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, d_loss, d_alpha;
     std::vector<float> h_alpha;  // [n_step][entity, relation, projection][S]
@@ -286,9 +290,9 @@ void parse_settings(kge_engine& E, const Items& s) {
     E.loss_scale = s.flt("training.loss_scale");
     E.n_step = (int)s.uint("execution.train_steps_per_program_run");
     E.rw_batch = (int)s.uint("execution.rw_batch_size");
-    (void)s.uint("execution.predict_hr_batch_size");
-    (void)s.uint("execution.predict_tail_batch_size");
-    (void)s.uint("execution.predict_n_best");
+    E.predict_hr_batch = (int)s.uint("execution.predict_hr_batch_size");
+    (void)s.uint("execution.predict_tail_batch_size");  // the device picks its own chunk of tails
+    E.predict_n_best = (int)s.uint("execution.predict_n_best");
 
     // dtype of the entity table (src/poplar_kge.cpp:237-246) + additive layouts
     const std::string dtype = s.str("execution.dtype");
@@ -1022,6 +1026,123 @@ void run_timing(kge_engine& E, const Items& in) {
     }
 }
 
+// "predict" (Model::predict, src/poplar_kge.cpp:811-855): for every (head row,
+// relation) of every shard the n_best best-scoring tails of every shard's table.
+//   predict_head, predict_relation  u32[S, Hb]   rows inside the query's own shard
+//   predict_entity_count            u32[S]       real rows per shard (rows 1..count)
+//   predict_scores  f32[S, S, Hb, n_best], predict_indices u32[S, S, Hb, n_best]:
+//       [query shard, tail shard, query, rank], best first (ties: lower row first)
+// Rows past the count never enter; when a shard has fewer than n_best rows the
+// rest reads score -1e6, row 0 (the collector's initial content in the reference).
+// With execution.shared_table the one table is scanned in S contiguous row
+// ranges ("tail shards"), indices are table rows, the count is element 0.
+void run_predict(kge_engine& E, const Items& in) {
+    const size_t S = E.S, Hb = (size_t)E.predict_hr_batch, nb = (size_t)E.predict_n_best;
+    if (nb < 1 || nb > 1024) throw std::invalid_argument("'execution.predict_n_best' must be in [1, 1024]");
+    const uint32_t* head = (const uint32_t*)in.array("predict_head", KGE_U32, {S, Hb});
+    const uint32_t* relation = (const uint32_t*)in.array("predict_relation", KGE_U32, {S, Hb});
+    const uint32_t* count = (const uint32_t*)in.array("predict_entity_count", KGE_U32, {S});
+    float* out_s = (float*)in.array("predict_scores", KGE_F32, {S, S, Hb, nb});
+    uint32_t* out_i = (uint32_t*)in.array("predict_indices", KGE_U32, {S, S, Hb, nb});
+    const hipStream_t st = E.stream;
+    const int Q = (int)(S * Hb), Qp = round_up(Q, 128), Dp = E.Dp;
+    const int chunk = round_up((int)std::min<int64_t>(E.n_entity, 8192), 64);
+
+    std::vector<uint32_t> rows(Qp, 0u), rels(Qp, 0u);
+    for (size_t s = 0; s < S; ++s) {
+        if (count[s] >= (uint32_t)E.n_entity)
+            throw std::invalid_argument("'predict_entity_count' must be < model.n_entity (row 0 is padding)");
+        for (size_t j = 0; j < Hb; ++j) {
+            const uint32_t h = head[s * Hb + j], r = relation[s * Hb + j];
+            if (h >= (uint32_t)E.n_entity) throw std::invalid_argument("'predict_head' index out of range");
+            if (r >= (uint32_t)E.n_rel) throw std::invalid_argument("'predict_relation' index out of range");
+            rows[s * Hb + j] = (E.shared_table ? 0u : (uint32_t)s * (uint32_t)E.n_entity) + h;
+            rels[s * Hb + j] = r;
+        }
+    }
+    if (E.p_idx.n < (size_t)(Qp + chunk)) {
+        E.p_idx.alloc(Qp + chunk);
+        E.p_rel.alloc(Qp);
+        E.p_count.alloc(1);
+        E.p_opnd.alloc((size_t)(Qp + chunk) * Dp);
+        E.p_scores.alloc((size_t)Qp * chunk);
+        E.p_best_s.alloc((size_t)Q * nb);
+        E.p_best_i.alloc((size_t)Q * nb);
+        if (E.F) {
+            E.p_hidden.alloc((size_t)std::max(Qp, chunk) * Dp);
+            E.p_featd.alloc((size_t)std::max(Qp, chunk) * E.Fp);
+        }
+    }
+    HIP_CHECK(hipMemcpyAsync(E.p_idx.p, rows.data(), (size_t)Qp * 4, hipMemcpyHostToDevice, st));
+    HIP_CHECK(hipMemcpyAsync(E.p_rel.p, rels.data(), (size_t)Qp * 4, hipMemcpyHostToDevice, st));
+
+    // rows `idx[0..n)` of the table as a row source: the embeddings, or hidden = emb + feature . W
+    auto rows_of = [&](const uint32_t* idx, int n) {
+        RowSource r;
+        r.base = E.table.p; r.pitch = E.L.pitch; r.etype = E.L.emb_etype;
+        r.index = idx; r.count = Dp; r.vec = 1;
+        if (E.F) {
+            const uint32_t n_u = (uint32_t)n;
+            HIP_CHECK(hipMemcpyAsync(E.p_count.p, &n_u, 4, hipMemcpyHostToDevice, st));
+            HIP_CHECK(hipStreamSynchronize(st));  // n_u leaves scope
+            FeatureArgs fa = {};
+            fa.uniq_key = idx; fa.counts = E.p_count.p; fa.max_rows = n;
+            fa.emb_base = E.table.p; fa.feat_base = E.table.p + E.L.off_f; fa.pitch = E.L.pitch;
+            fa.emb_etype = E.L.emb_etype; fa.feat_etype = E.L.feat_etype;
+            fa.Dp = Dp; fa.Fp = E.Fp; fa.proj = E.proj.p;
+            fa.featd = E.p_featd.p; fa.use_mfma = E.use_mfma;
+            launch_hidden_fwd(fa, E.p_hidden.p, st);
+            r.base = (const char*)E.p_hidden.p; r.pitch = (int64_t)Dp * 4; r.etype = ET_F32; r.index = nullptr;
+        }
+        return r;
+    };
+    // predicted tails of all queries: dense rows [0, Qp)
+    launch_gather_operands(rows_of(E.p_idx.p, Qp), E.rel.p, E.p_rel.p, E.score_fn == SCORE_DISTMULT ? 2 : 1, Qp,
+                           Qp, Dp, E.p_opnd.p, nullptr, st);
+
+    ScoreShape sh = {};
+    sh.S = 1; sh.B = Qp; sh.T = chunk; sh.Dp = Dp;
+    sh.score_fn = E.score_fn; sh.dist_fn = E.dist_fn; sh.loss_fn = E.loss_fn;
+    sh.gamma = E.gamma; sh.loss_scale = 1.f; sh.use_mfma = E.use_mfma; sh.operands_dense = 1;
+    RowSource dense;
+    dense.base = (const char*)E.p_opnd.p; dense.pitch = (int64_t)Dp * 4; dense.etype = ET_F32;
+    dense.index = nullptr; dense.count = Dp; dense.vec = 1;
+
+    std::vector<float> init_s((size_t)Q * nb, -1e6f), got_s((size_t)Q * nb);
+    std::vector<uint32_t> init_i((size_t)Q * nb, 0u), got_i((size_t)Q * nb);
+    const int64_t per_range = ((int64_t)E.n_entity - 1 + (int64_t)S - 1) / (int64_t)S;
+    for (size_t ts = 0; ts < S; ++ts) {
+        HIP_CHECK(hipMemcpyAsync(E.p_best_s.p, init_s.data(), init_s.size() * 4, hipMemcpyHostToDevice, st));
+        HIP_CHECK(hipMemcpyAsync(E.p_best_i.p, init_i.data(), init_i.size() * 4, hipMemcpyHostToDevice, st));
+        int64_t lo, hi, table_off;
+        if (E.shared_table) {
+            lo = 1 + (int64_t)ts * per_range;
+            hi = std::min<int64_t>(lo + per_range, 1 + (int64_t)count[0]);
+            table_off = 0;
+        } else {
+            lo = 1; hi = 1 + (int64_t)count[ts]; table_off = (int64_t)ts * E.n_entity;
+        }
+        for (int64_t r0 = lo; r0 < hi; r0 += chunk) {
+            const int live = (int)std::min<int64_t>(chunk, hi - r0);
+            uint32_t* tail_idx = E.p_idx.p + Qp;
+            launch_row_range((uint32_t)(table_off + r0), live, chunk, tail_idx, st);
+            launch_gather_operands(rows_of(tail_idx, chunk), E.rel.p, nullptr, 0, 0, chunk, Dp,
+                                   E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
+            launch_score_fwd(sh, dense, E.rel.p, nullptr, nullptr, E.p_scores.p, nullptr, nullptr, nullptr,
+                             false, st);
+            launch_topk_merge(E.p_scores.p, chunk, Q, live, (uint32_t)r0, (int)nb, E.p_best_s.p, E.p_best_i.p, st);
+        }
+        HIP_CHECK(hipGetLastError());
+        HIP_CHECK(hipMemcpyAsync(got_s.data(), E.p_best_s.p, got_s.size() * 4, hipMemcpyDeviceToHost, st));
+        HIP_CHECK(hipMemcpyAsync(got_i.data(), E.p_best_i.p, got_i.size() * 4, hipMemcpyDeviceToHost, st));
+        HIP_CHECK(hipStreamSynchronize(st));
+        for (size_t hs = 0; hs < S; ++hs) {
+            std::memcpy(out_s + (hs * S + ts) * Hb * nb, got_s.data() + hs * Hb * nb, Hb * nb * 4);
+            std::memcpy(out_i + (hs * S + ts) * Hb * nb, got_i.data() + hs * Hb * nb, Hb * nb * 4);
+        }
+    }
+}
+
 // "gather_benchmark": the stand-alone row gather (fr::Buffer::read) over the
 // engine's own table: gathers `indices` u32[n] physical rows `repeats` times
 // into a scratch buffer and reports the mean kernel time in `ms` f32[1].
@@ -1107,8 +1228,7 @@ int kge_engine_run(kge_engine* engine, const char* command, kge_item* items, siz
         else if (cmd == "timing") run_timing(E, in);
         else if (cmd == "gather_benchmark") run_gather_benchmark(E, in);
         else if (cmd == "variables") { /* served by kge_engine_variable_info */ }
-        else if (cmd == "predict")
-            throw std::runtime_error("command 'predict' is not implemented on the HIP device");
+        else if (cmd == "predict") run_predict(E, in);
         else
             throw std::invalid_argument("Unknown command '" + cmd + "'");
     });

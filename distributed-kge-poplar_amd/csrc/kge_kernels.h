@@ -227,6 +227,13 @@ void launch_hidden_fwd(const FeatureArgs& a, float* hidden, hipStream_t stream);
 void launch_proj_grad(const FeatureArgs& a, const float* grad_rows, float* gproj,
                       hipStream_t stream);
 
+// ---- predict -----------------------------------------------------------------
+// Merge scores[q, 0..n_valid) (indices first_index + column) into each query's
+// n_best best (score descending, index ascending; n_best <= 1024).
+void launch_topk_merge(const float* scores, int64_t ld, int n_queries, int n_valid, uint32_t first_index,
+                       int n_best, float* best_score, uint32_t* best_index, hipStream_t stream);
+void launch_row_range(uint32_t base, int n_live, int n, uint32_t* out, hipStream_t stream);
+
 // ---- table access ----------------------------------------------------------
 void launch_rows_gather(const void* buf, const uint32_t* idx, void* out, int64_t n,
                         int64_t row_bytes, hipStream_t stream);

@@ -1881,6 +1881,111 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
     launch_bwd(p, dist_fn, stream);
 }
 
+
+// --------------------------------------------------------------------------
+// predict: running top-k over a stream of score chunks
+// (TopKCollector, src/poplar_kge.cpp:743-809).  One workgroup per query keeps
+// its n_best (score, index) pairs sorted by (score descending, index
+// ascending); a block of 1024 new scores is merged only if one of them beats
+// the current n_best-th score, by a bitonic sort of the 2048-entry union in LDS.
+// Ties therefore resolve to the lower index, whatever the chunking.
+
+constexpr int TK_BLOCK = 1024, TK_SORT = 2048, TK_MAX_BEST = 1024;
+
+DEVINL bool topk_before(float sa, uint32_t ia, float sb, uint32_t ib) {
+    return sa > sb || (sa == sb && ia < ib);
+}
+
+__global__ __launch_bounds__(256) void k_topk_merge(const float* __restrict__ scores, int64_t ld,
+                                                    int n_valid, uint32_t first_index, int n_best,
+                                                    float* __restrict__ best_score,
+                                                    uint32_t* __restrict__ best_index) {
+    __shared__ float ks[TK_SORT];
+    __shared__ uint32_t vs[TK_SORT];
+    const int q = blockIdx.x, tid = threadIdx.x;
+    const float* row = scores + (size_t)q * ld;
+    float* bs = best_score + (size_t)q * n_best;
+    uint32_t* bi = best_index + (size_t)q * n_best;
+    // the current best live in ks / vs [TK_BLOCK, TK_BLOCK + n_best)
+    for (int i = tid; i < TK_BLOCK; i += 256) {
+        ks[TK_BLOCK + i] = i < n_best ? bs[i] : -INFINITY;
+        vs[TK_BLOCK + i] = i < n_best ? bi[i] : 0xffffffffu;
+    }
+    __syncthreads();
+    bool changed = false;
+    for (int base = 0; base < n_valid; base += TK_BLOCK) {
+        const float kth = ks[TK_BLOCK + n_best - 1];
+        float v[4];
+        bool beats = false;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = base + tid + 256 * j;
+            v[j] = i < n_valid ? row[i] : -INFINITY;
+            beats = beats || v[j] > kth;
+        }
+        if (!__syncthreads_or(beats)) continue;
+        changed = true;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            ks[tid + 256 * j] = v[j];
+            vs[tid + 256 * j] = first_index + (uint32_t)(base + tid + 256 * j);
+        }
+        __syncthreads();
+        // bitonic sort of all TK_SORT entries, best first
+        for (int size = 2; size <= TK_SORT; size <<= 1)
+            for (int stride = size >> 1; stride > 0; stride >>= 1) {
+                for (int t = tid; t < TK_SORT / 2; t += 256) {
+                    const int lo = 2 * t - (t & (stride - 1)), hi = lo + stride;
+                    const bool up = (lo & size) == 0;  // this run sorts best-first
+                    const float sa = ks[lo], sb = ks[hi];
+                    const uint32_t ia = vs[lo], ib = vs[hi];
+                    const bool ordered = topk_before(sa, ia, sb, ib) || (sa == sb && ia == ib);
+                    if (ordered != up) {
+                        ks[lo] = sb; ks[hi] = sa;
+                        vs[lo] = ib; vs[hi] = ia;
+                    }
+                }
+                __syncthreads();
+            }
+        // the n_best winners move back to their place, the rest is dropped
+        float ws[4];
+        uint32_t wi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = tid + 256 * j;
+            ws[j] = i < n_best ? ks[i] : -INFINITY;
+            wi[j] = i < n_best ? vs[i] : 0xffffffffu;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            ks[TK_BLOCK + tid + 256 * j] = ws[j];
+            vs[TK_BLOCK + tid + 256 * j] = wi[j];
+        }
+        __syncthreads();
+    }
+    if (changed)
+        for (int i = tid; i < n_best; i += 256) {
+            bs[i] = ks[TK_BLOCK + i];
+            bi[i] = vs[TK_BLOCK + i];
+        }
+}
+
+void launch_topk_merge(const float* scores, int64_t ld, int n_queries, int n_valid, uint32_t first_index,
+                       int n_best, float* best_score, uint32_t* best_index, hipStream_t stream) {
+    hipLaunchKernelGGL(k_topk_merge, dim3(n_queries), dim3(256), 0, stream, scores, ld, n_valid, first_index,
+                       n_best, best_score, best_index);
+}
+
+// out[i] = base + i for i < n_live, 0 (the padding row) after that
+__global__ __launch_bounds__(256) void k_row_range(uint32_t base, int n_live, int n, uint32_t* __restrict__ out) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = i < n_live ? base + (uint32_t)i : 0u;
+}
+void launch_row_range(uint32_t base, int n_live, int n, uint32_t* out, hipStream_t stream) {
+    hipLaunchKernelGGL(k_row_range, dim3((n + 255) / 256), dim3(256), 0, stream, base, n_live, n, out);
+}
+
 // --------------------------------------------------------------------------
 // segmented reduction + Adam
 

@@ -484,5 +484,45 @@ class Engine:
             kernels={k: dict(ms=float(kms[i]), calls=int(calls[i])) for i, k in enumerate(KERNEL_NAMES)},
             unique_entity_rows=counts[:, 0].copy(), entity_chunks=counts[:, 1].copy())
 
-    def predict(self, shard_idx_relation: np.ndarray) -> Any:
-        raise NotImplementedError("predict is outside the training-step path this engine covers")
+    # ---- prediction ------------------------------------------------------------
+    def _predict_hr_chunk(self, idx_relation: np.ndarray) -> Predictions:
+        """One ``predict`` program run (reference :781-817): idx_relation
+        uint32[n_shard, predict_hr_batch_size, 2] = (head row, relation) per
+        query shard.  The device returns every tail shard's n_best per query;
+        they are merged to the overall n_best here, best first."""
+        ex, S = self.settings.execution, self.settings.model.n_shard
+        Hb, n_best = ex.predict_hr_batch_size, ex.predict_n_best
+        scores = np.full((S, S, Hb, n_best), np.nan, np.float32)  # [query shard, tail shard, query, rank]
+        rows = np.zeros(scores.shape, np.uint32)
+        self.engine.run("predict", dict(
+            predict_head=np.ascontiguousarray(idx_relation[:, :, 0], np.uint32),
+            predict_relation=np.ascontiguousarray(idx_relation[:, :, 1], np.uint32),
+            predict_entity_count=np.ascontiguousarray(self.shard_to_entity_count, np.uint32),
+            predict_scores=scores, predict_indices=rows))
+        tail_shard = np.broadcast_to(np.arange(S, dtype=np.uint32)[None, :, None, None], rows.shape)
+        shard_idx = np.stack([tail_shard, rows], axis=-1)          # [S, S, Hb, n_best, 2]
+        pooled = Predictions(shard_idx=shard_idx.transpose(0, 2, 1, 3, 4).reshape(S, Hb, S * n_best, 2),
+                             score=scores.transpose(0, 2, 1, 3).reshape(S, Hb, S * n_best))
+        return pooled.topk(n_best).sort()
+
+    def predict(self, shard_idx_relation: np.ndarray) -> Predictions:
+        """Best tails for queries uint32[n, 3] = (head shard, head row, relation)
+        (reference :820-861): queries are dealt to their shards' slots in chunks
+        of predict_hr_batch_size, unused slots query row 0."""
+        shard_idx_relation = np.asarray(shard_idx_relation)
+        if shard_idx_relation.shape[1:] != (3,):
+            raise ValueError("shard_idx_relation should be of shape (n, 3)")
+        ex, S = self.settings.execution, self.settings.model.n_shard
+        Hb, n_best, n = ex.predict_hr_batch_size, ex.predict_n_best, shard_idx_relation.shape[0]
+        out = Predictions(shard_idx=np.zeros((n, n_best, 2), np.uint32), score=np.zeros((n, n_best), np.float32))
+        of_shard = [np.flatnonzero(shard_idx_relation[:, 0] == s) for s in range(S)]
+        for start in range(0, max(len(x) for x in of_shard), Hb):
+            slots = np.zeros((S, Hb, 2), np.uint32)
+            part = [x[start:start + Hb] for x in of_shard]
+            for s, which in enumerate(part):
+                slots[s, :len(which)] = shard_idx_relation[which, 1:3]
+            found = self._predict_hr_chunk(slots)
+            for s, which in enumerate(part):
+                out.shard_idx[which] = found.shard_idx[s, :len(which)]
+                out.score[which] = found.score[s, :len(which)]
+        return out

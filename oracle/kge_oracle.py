@@ -248,3 +248,37 @@ class Oracle:
         assert rc == 0
         state["step"] = step.value
         return loss
+
+
+def predict_reference(cfg, state, queries, shard_to_count, n_best):
+    """Brute-force tail prediction in float64 (tests/python/reference_model.py:169-206):
+    score every (head shard, head row, relation) query against every real row of
+    every shard's table and return the n_best best as (shard, row) and score,
+    best first, ties to the lower (shard, row).
+
+    state as for ``train_step_loop`` with private tables (``entity_data``
+    [n_shard * n_entity, 3D+F]); queries int[n, 3]."""
+    S, NE, D, F = cfg.n_shard, cfg.n_entity, cfg.dim, cfg.feature
+    rows = np.asarray(state["entity_data"], np.float64).reshape(S * NE, -1)
+    hidden = rows[:, :D].copy()
+    if F:
+        hidden += rows[:, 3 * D:3 * D + F] @ np.asarray(state["feature_projection"], np.float64)
+    rel = np.asarray(state["relation_embedding"], np.float64)
+    q = np.asarray(queries, np.int64)
+    h = hidden[q[:, 0] * NE + q[:, 1]]
+    dot = cfg.score_fn == SCORE["DistMult"] or cfg.distance_fn == DIST["MatMul"]
+    p = h * rel[q[:, 2]] if cfg.score_fn == SCORE["DistMult"] else h + rel[q[:, 2]]
+    if dot:
+        dist = p @ hidden.T
+    elif cfg.distance_fn == DIST["L1"]:
+        dist = np.stack([np.abs(x[None, :] - hidden).sum(-1) for x in p])
+    else:
+        dist = np.stack([np.sqrt(((x[None, :] - hidden) ** 2).sum(-1)) for x in p])
+    score = dist if cfg.score_fn == SCORE["DistMult"] else cfg.gamma - dist
+    live = np.zeros((S, NE), bool)
+    for s, n in enumerate(shard_to_count):
+        live[s, 1:1 + int(n)] = True
+    score = np.where(live.reshape(-1)[None, :], score, -np.inf)
+    order = np.argsort(-score, axis=1, kind="stable")[:, :n_best]
+    best = np.take_along_axis(score, order, axis=1)
+    return np.stack(np.divmod(order, NE), axis=-1), best

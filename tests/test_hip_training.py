@@ -148,3 +148,86 @@ def test_training_from_sampled_batches():
     # raw ids visit the same entities in the same roles; rows that are gathered but carry no
     # gradient differ (padding slots do not exist in raw mode), trained rows agree
     np.testing.assert_allclose(results[0][0], results[1][0], rtol=1e-5)
+
+
+def _random_queries(engine, n):
+    s = engine.settings
+    return np.stack([engine.random_integers(s.model.n_shard, (n,)),
+                     1 + engine.random_integers(s.model.n_entity - 1, (n,)),
+                     engine.random_integers(s.model.n_relation_type, (n,))], axis=-1)
+
+
+@pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "no_features_big"])
+def test_predict_vs_brute_force(variant):
+    """Engine.predict against a float64 brute force over every row of every shard
+    (the reference checks shapes, ranges and ordering, tests/python/test_poplar_kge.py:155-175,
+    and the MRR against its torch model, :214-236)."""
+    import poplar_kge as kge
+    from oracle.kge_oracle import predict_reference
+
+    settings = kge.Settings.create_demo()
+    settings.seed = 100
+    m, ex = settings.model, settings.execution
+    if variant == "l2":
+        m.distance_fn = "L2"
+    elif variant == "distmult":
+        m.score_fn, m.distance_fn = "DistMult", "MatMul"
+    elif variant == "no_features_big":
+        # several chunks of tails per shard, several query chunks, ragged counts
+        m.n_entity, m.entity_feature_size, m.embedding_size, m.n_shard = 20000, 0, 32, 3
+        settings.data.batch_size, ex.rw_batch_size, ex.predict_n_best = 6, 4096, 20
+        m.distance_fn = "L2"
+    settings.prepare()
+    S = m.n_shard
+    counts = np.array([m.n_entity - 1 - 7 * s for s in range(S)])
+    engine = kge.Engine(settings, counts)
+    features = engine.random_normal((S, m.n_entity, m.entity_feature_size), np.float16)
+    engine.initialise_all(features)
+    state = _oracle_state(engine.read_all())
+
+    n = ex.predict_hr_batch_size + 5
+    queries = _random_queries(engine, n)
+    found = engine.predict(queries)
+    assert found.shard_idx.shape == (n, ex.predict_n_best, 2) and found.score.shape == (n, ex.predict_n_best)
+    assert np.all(found.shard_idx[:, :, 0] < S)
+    assert np.all((found.shard_idx[:, :, 1] >= 1) & (found.shard_idx[:, :, 1] <= counts[found.shard_idx[:, :, 0]]))
+    assert not np.any(np.isnan(found.score))
+    np.testing.assert_equal(found.score, np.sort(found.score, axis=-1)[..., ::-1])
+
+    want_idx, want_score = predict_reference(_oracle_cfg(settings), state, queries, counts, ex.predict_n_best)
+    np.testing.assert_allclose(found.score, want_score, rtol=1e-5, atol=1e-5)
+    # the same entities, up to swaps between scores closer than float32 resolves
+    agree = np.all(found.shard_idx == want_idx, axis=-1)
+    close = np.abs(found.score - want_score) <= 1e-5 * np.maximum(1.0, np.abs(want_score))
+    assert np.all(agree | close)
+    assert agree.mean() > 0.99
+
+
+def test_training_mrr_matches_brute_force():
+    """The reference's MRR check (tests/python/test_poplar_kge.py:214-236): after every
+    program run the validation MRR from Engine.predict equals the brute-force one."""
+    import poplar_kge as kge
+    import poplar_kge_dataset as kge_data
+    from oracle.kge_oracle import predict_reference
+
+    settings = kge.Settings.create_demo()
+    settings.seed = 100
+    settings.prepare()
+    data = kge_data.RawData.load(settings)
+    dataset = kge_data.Dataset.load(data, settings)
+    engine = kge.Engine(settings, dataset.shard_to_count)
+    engine.initialise_all(dataset.entity_features(settings.model.entity_feature_size))
+    cfg, n_best = _oracle_cfg(settings), settings.execution.predict_n_best
+
+    def brute_force(queries):
+        idx, score = predict_reference(cfg, _oracle_state(engine.read_all()), queries, dataset.shard_to_count, n_best)
+        return kge.Predictions(shard_idx=idx.astype(np.uint32), score=score)
+
+    seen = []
+    for _ in range(6):
+        engine.train_step_loop(dataset.sample_batch())
+        for part in ("valid", "train"):
+            got, want = dataset.mrr(part, engine.predict), dataset.mrr(part, brute_force)
+            np.testing.assert_allclose(got, want, rtol=1e-4)
+            seen.append(want)
+    assert max(seen) > 0.05   # the training triples are being learnt: the comparison is not 0 == 0
