@@ -196,7 +196,7 @@ struct kge_engine {
     bool profile_kernels = false;
     int use_mfma = 1;  // additive setting execution.scoring = "mfma" | "valu"
     bool score_bf16 = false;  // additive setting execution.scoring_dtype = "float32" | "bfloat16"
-    int chunk = 64;       // contributions per first-level chunk (rows with many contributions)
+    int chunk = 64;       // contributions per first-level chunk (rows with many contributions; 256 measured no faster)
     int direct_max = 16;  // rows with at most this many contributions are summed by their Adam wave
 
     RowLayout L;
@@ -855,14 +855,14 @@ void run_step(kge_engine& E, int i) {
     rr.src = rsrc;
     rr.chunk_pos = E.r_cpos.p + (size_t)i * E.r_cstride;
     rr.chunk_len = E.r_clen.p + (size_t)i * E.r_cstride;
-    rr.counts = r_counts; rr.max_chunks = E.r_cstride;
+    rr.counts = r_counts; rr.max_chunks = E.r_cstride; rr.chunk = E.chunk;
     rr.partial = E.rel_partial.p; rr.Dp = E.Dp;
 
     ReduceArgs re = {};
     re.src = esrc;
     re.chunk_pos = E.e_cpos.p + (size_t)i * E.e_cstride;
     re.chunk_len = E.e_clen.p + (size_t)i * E.e_cstride;
-    re.counts = e_counts; re.max_chunks = E.e_cstride;
+    re.counts = e_counts; re.max_chunks = E.e_cstride; re.chunk = E.chunk;
     re.partial = E.partial.p; re.Dp = E.Dp;
     { KernelTimer t(E, K_REDUCE_ENT); launch_reduce_chunks2(re, rr, st); }
 
@@ -1358,7 +1358,7 @@ int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* i
     ReduceArgs ra = {};
     ra.src.sorted_item = sv; ra.src.grad = grad_out; ra.src.transform = 0;
     ra.chunk_pos = sp.chunk_pos; ra.chunk_len = sp.chunk_len; ra.counts = sp.counts;
-    ra.max_chunks = (int)L.cmax; ra.partial = (float*)(w + L.off_partial);
+    ra.max_chunks = (int)L.cmax; ra.chunk = 32; ra.partial = (float*)(w + L.off_partial);
     ra.Dp = (int)cols;
     launch_reduce_chunks(ra, st);
     launch_sum_partials_rows(sp.chunk_off, ra.partial, rows, cols, grad_t, st);

@@ -163,6 +163,7 @@ struct ReduceArgs {
     const uint32_t* chunk_len;
     const uint32_t* counts;       // {rows, chunks}
     int max_chunks;
+    int chunk;                    // most contributions a chunk holds
     float* partial;               // [max_chunks, Dp]
     int Dp;
 };

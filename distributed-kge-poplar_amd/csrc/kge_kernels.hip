@@ -2006,27 +2006,32 @@ DEVINL float4 load_contrib(const ContribSrc& cs, uint32_t c, int k, int Dp) {
 // k..k+3: eight independent row loads in flight, added in position order.
 // Must be called by every lane of the wave (the item indices travel by
 // shuffle); lanes with `active` false load nothing and return zero.
+template <int NB>
 DEVINL float4 sum_contribs(const ContribSrc& cs, uint32_t pos, uint32_t n, int k, int Dp, int lane,
                            bool active) {
     float4 acc = make_float4(0, 0, 0, 0);
-    for (uint32_t j = 0; j < n; j += 8) {
-        const uint32_t mine = (j + (lane & 7) < n) ? cs.sorted_item[pos + j + (lane & 7)] : 0u;
-        float4 v[8];
+    for (uint32_t j = 0; j < n; j += NB) {
+        const uint32_t mine = (j + (lane & (NB - 1)) < n) ? cs.sorted_item[pos + j + (lane & (NB - 1))] : 0u;
+        float4 v[NB];
 #pragma unroll
-        for (int x = 0; x < 8; ++x) {
+        for (int x = 0; x < NB; ++x) {
             const uint32_t c = __shfl(mine, x, 64);
             v[x] = (active && j + x < n) ? load_contrib(cs, c, k, Dp) : make_float4(0, 0, 0, 0);
         }
 #pragma unroll
-        for (int x = 0; x < 8; ++x) acc = f4add(acc, v[x]);
+        for (int x = 0; x < NB; ++x) acc = f4add(acc, v[x]);
     }
     return acc;
 }
 
 // First level for rows with many contributions: one workgroup per chunk, each
-// wave sums a quarter of the chunk, the four quarters are added in wave order.
-__global__ __launch_bounds__(256) void k_reduce_chunks(ReduceArgs a0, ReduceArgs a1) {
-    __shared__ __attribute__((aligned(16))) float part[3][256];
+// of its NW waves sums an NW-th of the chunk, the NW sums are added in wave order.
+// NW = 16 serves chunks of up to 256 contributions with the same two rounds of
+// eight loads per wave that NW = 4 needs for 64: four times fewer partials for
+// the second level to walk through.
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void k_reduce_chunks(ReduceArgs a0, ReduceArgs a1) {
+    __shared__ __attribute__((aligned(16))) float part[NW - 1][256];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // two reductions share the launch: blocks [0, a0.max_chunks) serve the first
     const bool second = (int)blockIdx.x >= a0.max_chunks;
@@ -2045,29 +2050,37 @@ __global__ __launch_bounds__(256) void k_reduce_chunks(ReduceArgs a0, ReduceArgs
             }
         return;
     }
-    const uint32_t quarter = (len + 3) / 4;
-    const uint32_t w0 = min(len, wave * quarter), w1 = min(len, w0 + quarter);
+    const uint32_t share = (len + NW - 1) / NW;
+    const uint32_t w0 = min(len, wave * share), w1 = min(len, w0 + share);
     for (int k0 = 0; k0 < Dp; k0 += 256) {
         const int k = k0 + lane * 4;
-        float4 acc = sum_contribs(a.src, pos + w0, w1 - w0, k, Dp, lane, k < Dp);
+        float4 acc = sum_contribs<8>(a.src, pos + w0, w1 - w0, k, Dp, lane, k < Dp);
         if (wave > 0) *reinterpret_cast<float4*>(&part[wave - 1][lane * 4]) = acc;
         __syncthreads();
         if (wave == 0 && k < Dp) {
 #pragma unroll
-            for (int w = 0; w < 3; ++w) acc = f4add(acc, *reinterpret_cast<const float4*>(&part[w][lane * 4]));
+            for (int w = 0; w < NW - 1; ++w) acc = f4add(acc, *reinterpret_cast<const float4*>(&part[w][lane * 4]));
             *reinterpret_cast<float4*>(a.partial + (size_t)q * Dp + k) = acc;
         }
         __syncthreads();
     }
 }
 
+static void launch_reduce_kernel(const ReduceArgs& a0, const ReduceArgs& a1, hipStream_t stream) {
+    const int n = a0.max_chunks + a1.max_chunks;
+    if (n == 0) return;
+    if (std::max(a0.chunk, a1.chunk) > 64)
+        hipLaunchKernelGGL(k_reduce_chunks<16>, dim3(n), dim3(1024), 0, stream, a0, a1);
+    else
+        hipLaunchKernelGGL(k_reduce_chunks<4>, dim3(n), dim3(256), 0, stream, a0, a1);
+}
 void launch_reduce_chunks(const ReduceArgs& a, hipStream_t stream) {
     ReduceArgs none = a;
     none.max_chunks = 0;
-    hipLaunchKernelGGL(k_reduce_chunks, dim3(a.max_chunks), dim3(256), 0, stream, a, none);
+    launch_reduce_kernel(a, none, stream);
 }
 void launch_reduce_chunks2(const ReduceArgs& a0, const ReduceArgs& a1, hipStream_t stream) {
-    hipLaunchKernelGGL(k_reduce_chunks, dim3(a0.max_chunks + a1.max_chunks), dim3(256), 0, stream, a0, a1);
+    launch_reduce_kernel(a0, a1, stream);
 }
 
 // fr::nn::adam (src/fructose/frnn.cpp:74-89) on one float4
@@ -2111,7 +2124,7 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
         const bool active = k < Dp;
         float4 g = make_float4(0, 0, 0, 0);
         if (!a.grad_direct && q1 == q0 && n_real)  // wave-uniform: all lanes take part in the shuffles
-            g = sum_contribs(a.src, pos, n_real, k, Dp, lane, active);
+            g = sum_contribs<8>(a.src, pos, n_real, k, Dp, lane, active);
         if (!active) continue;
         float4 p = load4(prow, k, a.p_etype);
         float4 m = *reinterpret_cast<const float4*>(mrow + (size_t)k * 4);
