@@ -1856,7 +1856,7 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
     if (both) {
         const dim3 grid = tile_grid(sh.Dp / BM_TK, 2 * (std::max(sh.B, sh.T) / BM_TI), sh.S);
         // eight waves per workgroup (two per SIMD): measured faster than four at
-        // every BASELINE shape, few workgroups (c2) or many (c3)
+        // every benchmark shape, few workgroups (1M-row workload) or many (22.8M-row workload)
         if (dist_fn == DIST_L2)
             hipLaunchKernelGGL((k_score_bwd_mfma_both<DIST_L2, 32, true, 8>), grid, dim3(512), 0, stream, p);
         else

@@ -1,4 +1,4 @@
-"""GPU parity at the BASELINE sizes (c2: 1M-row float32 table; c3: 22.8M rows,
+"""GPU parity at the full benchmark sizes (c2: 1M-row float32 table; c3: 22.8M rows,
 70 GB; c4: 4M rows with 768 float16 features, DistMult, softmax; c5: 91.2M rows
 with bfloat16 embeddings, 233 GB): the table is
 initialised on the device, the rows a few steps touch are read back, the CPU

@@ -290,6 +290,12 @@ STEP_CASES = {
     "l2_weight_decay": dict(distance_fn="L2", weight_decay=0.01, feature=0),
     "shared_table_l2": dict(distance_fn="L2", shared_table=True, n_shard=4, batch=8, a2a=4,
                             feature=0, n_entity=60, gamma=3.0),
+    # bfloat16 scoring operands (this build's option): rounding placement and the
+    # straight-through gradient against autograd
+    "distmult_bf16_scoring_feat": dict(score_fn="DistMult", distance_fn="MatMul", loss_fn="softmax",
+                                       softmax_correction_weight=1.0, feature=4, scoring_bf16=True),
+    "distmult_bf16_scoring_logsigmoid": dict(score_fn="DistMult", distance_fn="MatMul", feature=0,
+                                             scoring_bf16=True),
 }
 
 
@@ -361,3 +367,59 @@ def test_storage_rounding(orc):
     np.testing.assert_array_equal(orc.round(x, "float16"), x.astype(np.float16).astype(np.float32))
     bf = T.tensor(x).to(T.bfloat16).to(T.float32).numpy()
     np.testing.assert_array_equal(orc.round(x, "bfloat16_embedding"), bf)
+
+
+# ---- predict reference ------------------------------------------------------
+
+def test_predict_reference_by_hand():
+    # two shards of three rows (row 0 padding), D = 1: scores are gamma - |h + r - t|
+    from oracle.kge_oracle import predict_reference
+
+    cfg = make_cfg(n_shard=2, n_entity=3, n_relation=2, dim=1, feature=0, batch=1, a2a=1, gamma=10.0)
+    rows = np.zeros((6, 3), np.float32)
+    rows[:, 0] = [99, 1.0, 2.0,      # shard 0: padding, rows 1, 2
+                  99, 4.0, -1.0]     # shard 1: padding, rows 1, 2
+    state = {"entity_data": rows, "relation_embedding": np.array([[0.5], [-3.0]], np.float32)}
+    queries = np.array([[0, 1, 0],    # h = 1.0, r = 0.5 -> 1.5: 1.0 and 2.0 tie at 0.5, 4.0 and -1.0 at 2.5
+                        [1, 1, 1]])   # h = 4.0, r = -3 -> 1.0: nearest 1.0, then 2.0, -1.0, 4.0
+    idx, score = predict_reference(cfg, state, queries, [2, 2], 3)
+    np.testing.assert_array_equal(idx[0], [[0, 1], [0, 2], [1, 1]])   # ties -> lower (shard, row)
+    np.testing.assert_allclose(score[0], [9.5, 9.5, 7.5])
+    np.testing.assert_array_equal(idx[1], [[0, 1], [0, 2], [1, 2]])
+    np.testing.assert_allclose(score[1], [10.0, 9.0, 8.0])
+    # rows past a shard's count never appear, nor does the padding row
+    idx, score = predict_reference(cfg, state, queries, [1, 2], 3)
+    np.testing.assert_array_equal(idx[1], [[0, 1], [1, 2], [1, 1]])
+    np.testing.assert_allclose(score[1], [10.0, 8.0, 7.0])
+
+
+def test_predict_reference_vs_torch_topk():
+    # against the form of tests/python/reference_model.py:169-206: mask, broadcast score, topk
+    import torch as T
+    from oracle.kge_oracle import predict_reference
+
+    rng = np.random.default_rng(5)
+    S, NE, D, F, NR = 3, 40, 8, 4, 6
+    for kw in (dict(distance_fn="L1"), dict(distance_fn="L2"), dict(score_fn="DistMult", distance_fn="MatMul")):
+        cfg = make_cfg(n_shard=S, n_entity=NE, n_relation=NR, dim=D, feature=F, batch=2, a2a=2, gamma=3.0, **kw)
+        st = {"entity_data": rng.normal(size=(S * NE, 3 * D + F)).astype(np.float32),
+              "relation_embedding": rng.normal(size=(NR, D)).astype(np.float32),
+              "feature_projection": rng.normal(size=(F, D)).astype(np.float32)}
+        counts = [NE - 1, NE - 5, NE - 9]
+        q = np.stack([rng.integers(0, S, 17), rng.integers(1, NE - 9, 17), rng.integers(0, NR, 17)], -1)
+        idx, score = predict_reference(cfg, st, q, counts, 7)
+        e = T.tensor(st["entity_data"], dtype=T.float64)
+        hid = e[:, :D] + e[:, 3 * D:] @ T.tensor(st["feature_projection"], dtype=T.float64)
+        rel = T.tensor(st["relation_embedding"], dtype=T.float64)[q[:, 2]]
+        h = hid[q[:, 0] * NE + q[:, 1]]
+        if kw.get("score_fn") == "DistMult":
+            sc = (h * rel) @ hid.T
+        else:
+            sc = 3.0 - T.cdist(h + rel, hid, p=1 if kw["distance_fn"] == "L1" else 2)
+        mask = T.zeros(S, NE, dtype=T.float64)
+        for i, n in enumerate(counts):
+            mask[i, 0] = -1e4
+            mask[i, 1 + n:] = -1e4
+        top = T.topk(sc + mask.reshape(-1), k=7)
+        np.testing.assert_allclose(score, top.values.numpy(), rtol=1e-12, atol=1e-12)
+        np.testing.assert_array_equal(idx[..., 0] * NE + idx[..., 1], top.indices.numpy())

@@ -31,6 +31,12 @@ def log_sigmoid_clamped(x):
     return Fn.apply(x)
 
 
+def round_bf16_ste(x):
+    """x rounded to bfloat16 (nearest even) in the forward pass, identity in the
+    backward pass: how the bfloat16 scoring mode treats its operands."""
+    return x + (x.detach().to(T.float32).to(T.bfloat16).to(T.float64) - x.detach())
+
+
 def step(cfg, state, lr, batch_step):
     """One step in place on ``state`` (float32 arrays); returns loss[S].
 
@@ -62,7 +68,10 @@ def step(cfg, state, lr, batch_step):
     if F:
         proj = T.tensor(state["feature_projection"].astype(np.float64), requires_grad=True)
         params.append(proj)
-        hidden_u = emb + feat @ proj
+        if cfg.get("scoring_bf16"):
+            hidden_u = emb + round_bf16_ste(feat) @ round_bf16_ste(proj)
+        else:
+            hidden_u = emb + feat @ proj
     else:
         hidden_u = emb
     hidden = hidden_u[inverse].reshape(S, -1, D)  # [S, NR, D]
@@ -85,7 +94,10 @@ def step(cfg, state, lr, batch_step):
             dist = pred @ tails.transpose(1, 2)
         score = cfg["gamma"] - dist
     else:
-        score = (heads * r) @ tails.transpose(1, 2)
+        pred = heads * r
+        if cfg.get("scoring_bf16"):
+            pred, tails = round_bf16_ste(pred), round_bf16_ste(tails)
+        score = pred @ tails.transpose(1, 2)
 
     onehot = T.nn.functional.one_hot(tail, Tn).to(T.float64)
     if cfg["loss_fn"] == "logsigmoid":
