@@ -313,9 +313,6 @@ void parse_settings(kge_engine& E, const Items& s) {
     };
     parse_et("execution.embedding_dtype", emb_et);
     parse_et("execution.feature_dtype", feat_et);
-    if (mom_et != ET_F32)
-        throw std::invalid_argument("'execution.dtype' = 'float16' (half-precision optimiser state) is not "
-                                    "supported; use 'float32' with 'execution.embedding_dtype'");
     E.shared_table = s.find("execution.shared_table") ? s.boolean("execution.shared_table") : false;
     E.profile_kernels = s.find("execution.profile_kernels") ? s.boolean("execution.profile_kernels") : false;
     if (s.find("execution.reduce_chunk")) E.chunk = (int)s.uint("execution.reduce_chunk");
@@ -393,14 +390,14 @@ void parse_settings(kge_engine& E, const Items& s) {
     E.T = E.S * E.A;
     E.NR = E.B + E.T;
     E.R = E.S * E.NR;
-    E.Dp = round_up(E.D, emb_et == ET_F32 ? 4 : 8);
+    E.Dp = round_up(E.D, (emb_et == ET_F32 && mom_et == ET_F32) ? 4 : 8);
     E.Fp = E.F ? round_up(E.F, feat_et == ET_F32 ? 4 : 8) : 0;
     RowLayout& L = E.L;
     L.D = E.D; L.F = E.F; L.Dp = E.Dp; L.Fp = E.Fp;
     L.emb_etype = emb_et; L.mom_etype = mom_et; L.feat_etype = feat_et;
     L.off_m = (int64_t)E.Dp * elem_size(emb_et);
-    L.off_s = L.off_m + (int64_t)E.Dp * 4;
-    L.off_f = L.off_s + (int64_t)E.Dp * 4;
+    L.off_s = L.off_m + (int64_t)E.Dp * elem_size(mom_et);
+    L.off_f = L.off_s + (int64_t)E.Dp * elem_size(mom_et);
     L.pitch = L.off_f + (int64_t)E.Fp * elem_size(feat_et);
     E.n_rows = E.shared_table ? (int64_t)E.n_entity : (int64_t)E.S * E.n_entity;
     if (E.n_rows >= (int64_t)1 << 32) throw std::invalid_argument("more than 2^32 table rows");
@@ -879,7 +876,7 @@ void run_step(kge_engine& E, int i) {
     ar.counts = r_counts; ar.max_rows = E.n_rel;
     ar.partial = E.rel_partial.p;
     ar.p_base = (char*)E.rel.p; ar.m_base = (char*)E.rel_m.p; ar.v_base = (char*)E.rel_v.p;
-    ar.pitch = (int64_t)E.Dp * 4; ar.p_etype = ET_F32; ar.v_is_sqrt = 0;
+    ar.pitch = (int64_t)E.Dp * 4; ar.p_etype = ET_F32; ar.m_etype = ET_F32; ar.v_is_sqrt = 0;
     ar.alpha = alpha + E.S;
     ar.rows_per_alpha = E.shared_table ? 0u : (uint32_t)(E.n_rel / E.S);
 
@@ -893,7 +890,7 @@ void run_step(kge_engine& E, int i) {
     ae.partial = E.partial.p;
     ae.grad_out = E.F ? E.gsum.p : nullptr;
     ae.p_base = E.table.p; ae.m_base = E.table.p + E.L.off_m; ae.v_base = E.table.p + E.L.off_s;
-    ae.pitch = E.L.pitch; ae.p_etype = E.L.emb_etype; ae.v_is_sqrt = 1;
+    ae.pitch = E.L.pitch; ae.p_etype = E.L.emb_etype; ae.m_etype = E.L.mom_etype; ae.v_is_sqrt = 1;
     ae.alpha = alpha;
     ae.rows_per_alpha = E.shared_table ? 0u : (uint32_t)E.n_entity;
 

@@ -188,7 +188,7 @@ struct AdamArgs {
     char* m_base;
     char* v_base;
     int64_t pitch;
-    int p_etype;               // ET_* of the parameter (moments are float32)
+    int p_etype, m_etype;      // ET_* of the parameter and of the two moments
     int Dp;
     int v_is_sqrt;
     int no_update;             // only form the summed gradient (grad_out), leave the rows alone

@@ -2127,8 +2127,8 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
             g = sum_contribs<8>(a.src, pos, n_real, k, Dp, lane, active);
         if (!active) continue;
         float4 p = load4(prow, k, a.p_etype);
-        float4 m = *reinterpret_cast<const float4*>(mrow + (size_t)k * 4);
-        float4 v = *reinterpret_cast<const float4*>(vrow + (size_t)k * 4);
+        float4 m = load4(mrow, k, a.m_etype);
+        float4 v = load4(vrow, k, a.m_etype);
         if (a.grad_direct) {
             g = *reinterpret_cast<const float4*>(a.grad_direct + (size_t)u * Dp + k);
         } else if (q1 > q0) {
@@ -2146,8 +2146,8 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
         if (a.no_update) continue;
         adam4(p, m, v, g, a, alpha);
         store4(prow, k, a.p_etype, p);
-        *reinterpret_cast<float4*>(mrow + (size_t)k * 4) = m;
-        *reinterpret_cast<float4*>(vrow + (size_t)k * 4) = v;
+        store4(mrow, k, a.m_etype, m);
+        store4(vrow, k, a.m_etype, v);
     }
 }
 

@@ -69,6 +69,8 @@ def engine_settings(c, n_step, rw_batch=64, **extra):
     }
     if c.get("storage") == "bfloat16_embedding":
         s["execution.embedding_dtype"] = "bfloat16"
+    if c.get("storage") == "float16":
+        s["execution.dtype"] = "float16"
     if c.get("scoring_bf16"):
         s["execution.scoring_dtype"] = "bfloat16"
     s.update(extra)
@@ -107,9 +109,10 @@ def read_state(engine, c, rw=64):
     S, NE, D, F = c["n_shard"], c["n_entity"], c["dim"], c["feature"]
     n_tables = 1 if c["shared_table"] else S
     ed = np.zeros((n_tables, NE, 3 * D + F), np.float32)
+    half = c.get("storage") == "float16"   # the read stream carries execution.dtype, float16 as int16 bits
     for off, idx in _chunks(c, rw):
-        out = np.zeros((S, rw, 3 * D + F), np.float32)
-        engine.run("read_entity", dict(read_indices=idx, read_data=out))
+        out = np.zeros((S, rw, 3 * D + F), np.float16 if half else np.float32)
+        engine.run("read_entity", dict(read_indices=idx, read_data=out.view(np.int16) if half else out))
         n = min(rw, NE - off)
         ed[:, off:off + n] = out[:n_tables, :n]
     st = {"entity_data": ed.reshape(-1, 3 * D + F)}

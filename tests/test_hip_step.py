@@ -103,6 +103,39 @@ def test_step_bf16_scoring(oracle64, name):
     assert K.rel_l2(st_f[k] - st0[k], st_o[k] - st0[k]) > 1e-4
 
 
+@pytest.mark.parametrize("name", ["demo", "l2_aligned"])
+def test_step_float16_table(oracle64, name):
+    """execution.dtype = "float16" (src/poplar_kge.cpp:237-246): embedding, both
+    moments and features stored as float16, read / write streams in float16.  The
+    oracle rounds on write-back as the reference's cast does (:412-417); a float32
+    difference of 1e-7 may round an element to the other float16 neighbour
+    (2^-11 relative), hence the bars (the reference's own: loss 2e-3, update 1e-1)."""
+    import libpoplar_kge
+
+    kw = dict(storage="float16", feature=6) if name == "demo" else dict(
+        storage="float16", distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
+        n_entity=3000, n_relation=8, gamma=6.0)
+    c = K.cfg_dict(**kw)
+    rng = np.random.default_rng(13)
+    st0 = K.make_state(c, rng)
+    st0["entity_data"] = oracle64.round(st0["entity_data"], "float16")   # representable start
+    batch = K.random_batch(c, 3, rng)
+    engine = libpoplar_kge.Engine(H.engine_settings(c, 3), "")
+    H.load_state(engine, c, st0)
+    np.testing.assert_array_equal(H.read_state(engine, c)["entity_data"], st0["entity_data"])
+    st_o = K.copy_state(st0)
+    lr = np.full(c["n_shard"], 0.02, np.float32)
+    loss_o = oracle64.train_step_loop(make_cfg(**c), st_o, lr, batch)
+    loss_h = H.train(engine, c, lr, batch)
+    np.testing.assert_allclose(loss_h, loss_o, rtol=2e-3)
+    st_h = H.read_state(engine, c)
+    for k in st0:
+        if k == "step":
+            continue
+        assert K.rel_l2(st_h[k] - st0[k], st_o[k] - st0[k]) < 2e-2, k
+    assert np.mean(st_h["entity_data"] != st_o["entity_data"]) < 1e-2
+
+
 def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_loop=1, warm=True,
              **settings):
     import libpoplar_kge

@@ -37,11 +37,13 @@ def _random_batch(engine):
 
 def _oracle_cfg(settings):
     m, d, t = settings.model, settings.data, settings.training
+    storage = "float16" if settings.execution.dtype == "float16" else "float32"
     return make_cfg(n_shard=m.n_shard, n_entity=m.n_entity, n_relation=m.n_relation_type,
                     dim=m.embedding_size, feature=m.entity_feature_size, batch=d.batch_size,
                     a2a=d.a2a_size, score_fn=m.score_fn, distance_fn=m.distance_fn,
                     loss_fn=t.loss.type, gamma=m.gamma, beta_m=t.adam_beta_m, beta_v=t.adam_beta_v,
-                    epsilon=t.adam_epsilon, weight_decay=t.weight_decay, loss_scale=t.loss_scale)
+                    epsilon=t.adam_epsilon, weight_decay=t.weight_decay, loss_scale=t.loss_scale,
+                    storage=storage)
 
 
 def _oracle_state(state):
@@ -77,12 +79,16 @@ def test_engine_ops():
     np.testing.assert_allclose(engine.read_entity_all()[:, :, -m.entity_feature_size:], features)
 
 
-def test_training():
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_training(dtype):
     import poplar_kge as kge
     import poplar_kge_dataset as kge_data
 
     settings = kge.Settings.create_demo()
     settings.seed = 100
+    settings.execution.dtype = dtype
+    if dtype == "float16":
+        settings.training.n_step = 20  # "since numerical errors compound" (the reference, :184-185)
     settings.prepare()
     data = kge_data.RawData.load(settings)
     dataset = kge_data.Dataset.load(data, settings)
@@ -98,24 +104,25 @@ def test_training():
     for b in batches:
         b.remote[...] = batches[0].remote[:, 0, np.newaxis, :]
     n_loop = settings.program_runs_per_log * settings.logs_per_training_run
-    assert n_loop == 20
+    assert n_loop == dict(float32=20, float16=4)[dtype]
 
     loss, ref_loss = [], []
     for b in itertools.islice(itertools.cycle(batches), n_loop):
         step_loss, lr = engine.train_step_loop(b)
         loss.append(step_loss)
         ref_loss.append(float(np.sum(oracle.train_step_loop(cfg, ref, lr, vars(b)))))
-    np.testing.assert_allclose(loss, ref_loss, rtol=1e-4)
+    np.testing.assert_allclose(loss, ref_loss, rtol=dict(float16=2e-3, float32=1e-4)[dtype])
 
     final = engine.read_all()
-    assert set(np.ravel(final.pop("step"))) == {ref["step"]} == {100}
+    assert set(np.ravel(final.pop("step"))) == {ref["step"]} == {5 * n_loop}
     first = _oracle_state(initial)
     for key, value in final.items():
         value = value.reshape(ref[key].shape)
         delta, ref_delta = value - first[key], ref[key] - first[key]
         assert np.any(ref_delta != 0), key
         distance = K.rel_l2(delta, ref_delta)
-        assert distance <= 1e-4, f"(final - initial) of '{key}' is {distance:.2g} away from the oracle's"
+        tolerance = dict(float16=1e-1, float32=1e-4)[dtype]   # the reference's bars (:251)
+        assert distance <= tolerance, f"(final - initial) of '{key}' is {distance:.2g} away from the oracle's"
 
 
 def test_training_from_sampled_batches():
