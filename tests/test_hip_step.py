@@ -230,6 +230,50 @@ def test_step_l1_equal_and_signed_zero_entries(oracle64):
         assert K.rel_l2(st_h[k] - st0[k], st_o[k] - st0[k]) < 1e-4, k
 
 
+EDGE_CASES = {
+    # the smallest shapes the formulas allow (T >= 2: the negative weight divides by T - 1)
+    "one_shard_one_positive": dict(n_shard=1, batch=1, a2a=2, dim=4, feature=0, n_entity=5, n_relation=1),
+    "one_column": dict(n_shard=2, batch=3, a2a=2, dim=1, feature=0, n_entity=9, n_relation=2),
+    "one_column_l2_features": dict(n_shard=2, batch=3, a2a=2, dim=1, feature=2, n_entity=9, n_relation=2,
+                                   distance_fn="L2"),
+    "single_relation_distmult": dict(score_fn="DistMult", distance_fn="MatMul", n_shard=1, batch=4, a2a=3,
+                                     dim=12, feature=0, n_entity=30, n_relation=1, loss_fn="softmax",
+                                     softmax_correction_weight=0.5),
+    "wide_rows": dict(n_shard=2, batch=4, a2a=3, dim=1027, feature=0, n_entity=20, n_relation=4,
+                      distance_fn="L2"),
+    "many_shards": dict(n_shard=16, batch=2, a2a=1, dim=8, feature=0, n_entity=40, n_relation=16),
+}
+
+
+@pytest.mark.parametrize("name", list(EDGE_CASES))
+def test_step_edge_shapes(oracle64, name):
+    run_case(oracle64, EDGE_CASES[name], n_step=2)
+
+
+def test_step_all_padding(oracle64):
+    # a batch that gathers only the padding row: every slot is row 0, which is updated once per
+    # shard with the sum of all its (non-zero) gradients, as any other row would be
+    import libpoplar_kge
+
+    c = K.cfg_dict(feature=0, n_shard=2, batch=4, a2a=3, dim=8, n_entity=20, n_relation=2)
+    rng = np.random.default_rng(17)
+    st0 = K.make_state(c, rng)
+    batch = K.random_batch(c, 2, rng)
+    batch["remote"][...] = 0
+    engine = libpoplar_kge.Engine(H.engine_settings(c, 2), "")
+    H.load_state(engine, c, st0)
+    st_o = K.copy_state(st0)
+    loss_o = oracle64.train_step_loop(make_cfg(**c), st_o, 0.05, batch)
+    loss_h = H.train(engine, c, 0.05, batch)
+    np.testing.assert_allclose(loss_h, loss_o, rtol=1e-5)
+    st_h = H.read_state(engine, c)
+    ne = c["n_entity"]
+    for s in range(c["n_shard"]):   # only row 0 of each shard moved
+        np.testing.assert_array_equal(st_h["entity_data"][s * ne + 1:(s + 1) * ne],
+                                      st0["entity_data"][s * ne + 1:(s + 1) * ne])
+    assert K.rel_l2(st_h["entity_data"], st_o["entity_data"]) < 1e-5
+
+
 def test_step_near_duplicate_rows(oracle64):
     # head + relation almost equal to some tails: the L2 forward must not cancel
     import libpoplar_kge
