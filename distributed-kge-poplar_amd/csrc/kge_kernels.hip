@@ -1447,13 +1447,16 @@ __global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
 // registers while the matrix cores work on the current one.
 
 constexpr int BM_TI = 128, BM_TK = 64, BM_LDK = BM_TK + 4;
+// LDS of a backward workgroup: two coefficient tiles (the larger layout: 128 x 36 floats),
+// two `other` tiles (32 x 68 floats) and the 128 coefficient row sums
+constexpr int kBwdSmemBytes = 2 * (BM_TI * 36 * 4) + 2 * (32 * BM_LDK * 4) + BM_TI * 4;
 
 // BJT = rows of `other` staged per iteration (32 or 128) and NW = waves per
 // workgroup (4 or 8), chosen as in the forward kernel.
 // ALIGNED: n_self % 128 == 0, n_other % BJT == 0, Dp % 64 == 0, T % 4 == 0,
 // dense float32 operands without a relation to apply: branch-free staging loads.
 template <int DIST, int SIDE_B, int BJT, bool ALIGNED, int NW>
-DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, const int tile_y) {
+DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, const int tile_y, char* smem) {
     // Both tiles are float4 copies of global memory.  Head side: Cs[i][j] (the
     // coefficient rows as stored), a lane reads four consecutive j of its row i
     // in one 16-byte LDS read.  Tail side: Cs[j][i] (coefficient rows are the
@@ -1464,9 +1467,14 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
     constexpr int HC = 1024 / NT;     // float4 of a 32 x 128 coefficient sub-tile per thread
     constexpr int HO = 512 / NT;      // float4 of a 32 x 64 `other` sub-tile per thread
     constexpr int CS_ROWS = SIDE_B ? BJT : BM_TI, CS_LD = SIDE_B ? BM_TI + 4 : BJT + 4;
-    __shared__ __attribute__((aligned(16))) float Cs[CS_ROWS][CS_LD];
-    __shared__ __attribute__((aligned(16))) float Os[BJT][BM_LDK];
-    __shared__ float csum_s[BM_TI];
+    // two copies of each tile: while the matrix cores work on one slab the next is
+    // staged into the other copy, with a single barrier per slab
+    typedef float CsTile[CS_ROWS][CS_LD];
+    typedef float OsTile[BJT][BM_LDK];
+    static_assert(2 * sizeof(CsTile) + 2 * sizeof(OsTile) + BM_TI * 4 <= kBwdSmemBytes, "LDS carve-up");
+    CsTile* Cs2 = reinterpret_cast<CsTile*>(smem);
+    OsTile* Os2 = reinterpret_cast<OsTile*>(smem + 2 * sizeof(CsTile));
+    float* csum_s = reinterpret_cast<float*>(smem + 2 * sizeof(CsTile) + 2 * sizeof(OsTile));
     const int i0 = tile_y * BM_TI, kt0 = tile_x * BM_TK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wi = (wave >> 1) * (32 * AT), wk = (wave & 1) * 32;
@@ -1591,46 +1599,66 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
             }
         }
     };
-    prefetch(0);
-    for (int jbase = 0; jbase < n_other; jbase += BJT) {
-        bool direct[NCH][AT], direct_row[NCH], any_direct[NCH];
+    bool direct_next[NCH][AT], direct_row_next[NCH], any_direct_next[NCH];
+    // writes the prefetched slab into tile copy `nb` and latches its near-pair flags
+    auto stage = [&](int nb) __attribute__((always_inline)) {
+        CsTile& Cn = Cs2[nb];
+        OsTile& On = Os2[nb];
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            any_direct[c] = false;
+            any_direct_next[c] = false;
 #pragma unroll
             for (int t = 0; t < AT; ++t) {
-                direct[c][t] = nf_next[c][t] != 0u;
-                any_direct[c] = any_direct[c] || direct[c][t];
+                direct_next[c][t] = nf_next[c][t] != 0u;
+                any_direct_next[c] = any_direct_next[c] || direct_next[c][t];
             }
-            direct_row[c] = nf_row_next[c] != 0u;
+            direct_row_next[c] = nf_row_next[c] != 0u;
 #pragma unroll
             for (int h = 0; h < HC; ++h) {
                 const int idx = tid + NT * h;
                 if (!SIDE_B) {
-                    *reinterpret_cast<floatx4*>(&Cs[idx >> 3][32 * c + (idx & 7) * 4]) = creg[c][h];
+                    *reinterpret_cast<floatx4*>(&Cn[idx >> 3][32 * c + (idx & 7) * 4]) = creg[c][h];
                 } else {
-                    *reinterpret_cast<floatx4*>(&Cs[32 * c + (idx >> 5)][(idx & 31) * 4]) = creg[c][h];
+                    *reinterpret_cast<floatx4*>(&Cn[32 * c + (idx >> 5)][(idx & 31) * 4]) = creg[c][h];
                 }
             }
 #pragma unroll
             for (int h = 0; h < HO; ++h) {
                 const int idx = tid + NT * h;
-                *reinterpret_cast<floatx4*>(&Os[32 * c + (idx >> 4)][(idx & 15) * 4]) = oreg[c][h];
+                *reinterpret_cast<floatx4*>(&On[32 * c + (idx >> 4)][(idx & 15) * 4]) = oreg[c][h];
             }
         }
-        __syncthreads();
-        if (jbase + BJT < n_other) prefetch(jbase + BJT);
+    };
+    prefetch(0);
+    stage(0);
+    __syncthreads();
+    if (BJT < n_other) prefetch(BJT);
+    for (int jbase = 0, buf = 0; jbase < n_other; jbase += BJT, buf ^= 1) {
+        bool direct[NCH][AT], direct_row[NCH], any_direct[NCH];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            any_direct[c] = any_direct_next[c];
+            direct_row[c] = direct_row_next[c];
+#pragma unroll
+            for (int t = 0; t < AT; ++t) direct[c][t] = direct_next[c][t];
+        }
+        if (jbase + BJT < n_other) {
+            stage(buf ^ 1);  // the other copy: last read one slab ago, before the barrier
+            if (jbase + 2 * BJT < n_other) prefetch(jbase + 2 * BJT);
+        }
+        const CsTile& Cc = Cs2[buf];
+        const OsTile& Oc = Os2[buf];
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int jo = 32 * c;
             if (DIST == DIST_L2 && tid < BM_TI && !direct_row[c]) {
                 if (SIDE_B) {
 #pragma unroll
-                    for (int jj = 0; jj < 32; ++jj) cs_acc += Cs[jo + jj][tid];
+                    for (int jj = 0; jj < 32; ++jj) cs_acc += Cc[jo + jj][tid];
                 } else {
 #pragma unroll
                     for (int jj = 0; jj < 32; jj += 4) {
-                        const float4 v = *reinterpret_cast<const float4*>(&Cs[tid][jo + jj]);
+                        const float4 v = *reinterpret_cast<const float4*>(&Cc[tid][jo + jj]);
                         cs_acc += v.x; cs_acc += v.y; cs_acc += v.z; cs_acc += v.w;
                     }
                 }
@@ -1642,14 +1670,14 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
                 const int hl = lane >> 5, cl = lane & 31;
                 auto fetch = [&](int buf, int g) {
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) rb[buf][x] = Os[jo + 8 * g + 4 * hl + x][wk + cl];
+                    for (int x = 0; x < 4; ++x) rb[buf][x] = Oc[jo + 8 * g + 4 * hl + x][wk + cl];
 #pragma unroll
                     for (int t = 0; t < AT; ++t) {
                         if (SIDE_B) {
 #pragma unroll
-                            for (int x = 0; x < 4; ++x) ra[buf][t][x] = Cs[jo + 8 * g + 4 * hl + x][wi + 32 * t + cl];
+                            for (int x = 0; x < 4; ++x) ra[buf][t][x] = Cc[jo + 8 * g + 4 * hl + x][wi + 32 * t + cl];
                         } else {
-                            const float4 v = *reinterpret_cast<const float4*>(&Cs[wi + 32 * t + cl][jo + 8 * g + 4 * hl]);
+                            const float4 v = *reinterpret_cast<const float4*>(&Cc[wi + 32 * t + cl][jo + 8 * g + 4 * hl]);
                             ra[buf][t][0] = v.x; ra[buf][t][1] = v.y; ra[buf][t][2] = v.z; ra[buf][t][3] = v.w;
                         }
                     }
@@ -1673,11 +1701,11 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
                 for (int t = 0; t < AT; ++t) {
                     if (direct[c][t]) {
                         for (int jj = jo; jj < jo + 32; ++jj) {
-                            const float o = Os[jj][wk + (lane & 31)];
+                            const float o = Oc[jj][wk + (lane & 31)];
 #pragma unroll
                             for (int r = 0; r < 16; ++r) {
                                 const int il = wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                                const float cc = SIDE_B ? Cs[jj][il] : Cs[il][jj];
+                                const float cc = SIDE_B ? Cc[jj][il] : Cc[il][jj];
                                 acc[t][r] = fmaf(-cc, sv[t][r] - o, acc[t][r]);
                             }
                         }
@@ -1685,8 +1713,8 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
 #pragma unroll
                         for (int q = 0; q < 16; ++q) {
                             const int jj = jo + 2 * q + (lane >> 5);
-                            const float b = Os[jj][wk + (lane & 31)];
-                            const float a = SIDE_B ? Cs[jj][wi + 32 * t + (lane & 31)] : Cs[wi + 32 * t + (lane & 31)][jj];
+                            const float b = Oc[jj][wk + (lane & 31)];
+                            const float a = SIDE_B ? Cc[jj][wi + 32 * t + (lane & 31)] : Cc[wi + 32 * t + (lane & 31)][jj];
                             acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[t], 0, 0, 0);
                         }
                     }
@@ -1719,18 +1747,20 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
 // one side per launch (p.side_b), or both sides in one launch
 template <int DIST, int SIDE_B, int BJT, bool ALIGNED, int NW>
 __global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma(BwdParams p) {
+    __shared__ __attribute__((aligned(16))) char smem[kBwdSmemBytes];
     const int n_self = SIDE_B ? p.T : p.B;
     const TileId tile = xcd_tile((p.Dp + BM_TK - 1) / BM_TK, (n_self + BM_TI - 1) / BM_TI, p.S);
-    bwd_mfma_body<DIST, SIDE_B, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y);
+    bwd_mfma_body<DIST, SIDE_B, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y, smem);
 }
 template <int DIST, int BJT, bool ALIGNED, int NW>
 __global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma_both(BwdParams p) {
     // a block's head-side tiles and then its tail-side tiles, back to back on one XCD:
     // both sides read the same operand rows and coefficient matrix
+    __shared__ __attribute__((aligned(16))) char smem[kBwdSmemBytes];  // one allocation serves either side
     const int gy = (p.B > p.T ? p.B : p.T) / BM_TI;
     const TileId tile = xcd_tile(p.Dp / BM_TK, 2 * gy, p.S);
-    if (tile.y < gy) bwd_mfma_body<DIST, 0, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y);
-    else bwd_mfma_body<DIST, 1, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y - gy);
+    if (tile.y < gy) bwd_mfma_body<DIST, 0, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y, smem);
+    else bwd_mfma_body<DIST, 1, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y - gy, smem);
 }
 
 static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
