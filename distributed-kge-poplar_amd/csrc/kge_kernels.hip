@@ -1495,6 +1495,8 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
     float cs_acc = 0.f;
+    constexpr int NQ = NT / BM_TI, QL = 32 / NQ;  // threads per coefficient row, coefficients per thread and slab
+    const int crow = tid & (BM_TI - 1), cq = tid / BM_TI;
     const int kcol = kt0 + wk + (lane & 31);
 
     // L2: this lane's `self` values, in accumulator layout
@@ -1651,14 +1653,16 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int jo = 32 * c;
-            if (DIST == DIST_L2 && tid < BM_TI && !direct_row[c]) {
+            // coefficient row sums (L2): NQ threads share a row, each adds its QL of the slab's
+            // 32 coefficients, so that every wave carries the same small load
+            if (DIST == DIST_L2 && !direct_row[c]) {
                 if (SIDE_B) {
 #pragma unroll
-                    for (int jj = 0; jj < 32; ++jj) cs_acc += Cc[jo + jj][tid];
+                    for (int jj = 0; jj < QL; ++jj) cs_acc += Cc[jo + cq * QL + jj][crow];
                 } else {
 #pragma unroll
-                    for (int jj = 0; jj < 32; jj += 4) {
-                        const float4 v = *reinterpret_cast<const float4*>(&Cc[tid][jo + jj]);
+                    for (int jj = 0; jj < QL; jj += 4) {
+                        const float4 v = *reinterpret_cast<const float4*>(&Cc[crow][jo + cq * QL + jj]);
                         cs_acc += v.x; cs_acc += v.y; cs_acc += v.z; cs_acc += v.w;
                     }
                 }
@@ -1724,7 +1728,16 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
         __syncthreads();
     }
     if (DIST == DIST_L2) {
-        if (tid < BM_TI) csum_s[tid] = cs_acc;
+        // the NQ partial sums of a row, added in a fixed order (the tiles are no longer read)
+        float* part = reinterpret_cast<float*>(smem);
+        part[cq * BM_TI + crow] = cs_acc;
+        __syncthreads();
+        if (tid < BM_TI) {
+            float sum = part[tid];
+#pragma unroll
+            for (int q = 1; q < NQ; ++q) sum += part[q * BM_TI + tid];
+            csum_s[tid] = sum;
+        }
         __syncthreads();
     }
 #pragma unroll
@@ -2130,6 +2143,8 @@ DEVINL void adam4(float4& p, float4& m, float4& v, float4 g, const AdamArgs& a, 
 
 // One wave per distinct row: gather its gradient (directly from its few
 // contributions, or from its chunk partials), Adam, write the row back.
+// MF32: both moments float32 (the usual layout), accessed as plain 16-byte words
+template <bool MF32>
 __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
     const int lane = threadIdx.x & 63;
     // two tables share the launch: blocks [0, ceil(a0.max_rows / 4)) serve the first
@@ -2157,8 +2172,14 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
             g = sum_contribs<8>(a.src, pos, n_real, k, Dp, lane, active);
         if (!active) continue;
         float4 p = load4(prow, k, a.p_etype);
-        float4 m = load4(mrow, k, a.m_etype);
-        float4 v = load4(vrow, k, a.m_etype);
+        float4 m, v;
+        if constexpr (MF32) {
+            m = *reinterpret_cast<const float4*>(mrow + (size_t)k * 4);
+            v = *reinterpret_cast<const float4*>(vrow + (size_t)k * 4);
+        } else {
+            m = load4(mrow, k, a.m_etype);
+            v = load4(vrow, k, a.m_etype);
+        }
         if (a.grad_direct) {
             g = *reinterpret_cast<const float4*>(a.grad_direct + (size_t)u * Dp + k);
         } else if (q1 > q0) {
@@ -2176,19 +2197,30 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
         if (a.no_update) continue;
         adam4(p, m, v, g, a, alpha);
         store4(prow, k, a.p_etype, p);
-        store4(mrow, k, a.m_etype, m);
-        store4(vrow, k, a.m_etype, v);
+        if constexpr (MF32) {
+            *reinterpret_cast<float4*>(mrow + (size_t)k * 4) = m;
+            *reinterpret_cast<float4*>(vrow + (size_t)k * 4) = v;
+        } else {
+            store4(mrow, k, a.m_etype, m);
+            store4(vrow, k, a.m_etype, v);
+        }
     }
 }
 
+static void launch_adam_kernel(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream) {
+    const dim3 grid((a0.max_rows + 3) / 4 + (a1.max_rows + 3) / 4);
+    if (grid.x == 0) return;
+    const bool f32 = (a0.max_rows == 0 || a0.m_etype == ET_F32) && (a1.max_rows == 0 || a1.m_etype == ET_F32);
+    if (f32) hipLaunchKernelGGL(k_adam_rows<true>, grid, dim3(256), 0, stream, a0, a1);
+    else hipLaunchKernelGGL(k_adam_rows<false>, grid, dim3(256), 0, stream, a0, a1);
+}
 void launch_adam_rows(const AdamArgs& a, hipStream_t stream) {
     AdamArgs none = a;
     none.max_rows = 0;
-    hipLaunchKernelGGL(k_adam_rows, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, none);
+    launch_adam_kernel(a, none, stream);
 }
 void launch_adam_rows2(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream) {
-    hipLaunchKernelGGL(k_adam_rows, dim3((a0.max_rows + 3) / 4 + (a1.max_rows + 3) / 4), dim3(256), 0,
-                       stream, a0, a1);
+    launch_adam_kernel(a0, a1, stream);
 }
 
 __global__ __launch_bounds__(64) void k_loss_finalize(const float* __restrict__ loss_part, int n_step,
