@@ -491,7 +491,8 @@ DEVINL float log_sigmoid_grad(float z) { return 1.f / (1.f + expf(fminf(z, 11.f)
 
 // The same two functions from ONE hardware exponential (the scoring epilogues
 // evaluate them once per score): with u = exp(-|z|) in (0, 1],
-//   z >= 0:        logsig = -log1p(u),     dlogsig = u' / (1 + u'),  u' = max(u, e^-11)  (the +11 clamp)
+//   z >= 0:        logsig = -log1p(u),     dlogsig = u' / (1 + u'),  u' = max(u, e^-11)  (the +11 clamp;
+//                  u / (1 + u) grows with u, so the clamp can move to the quotient)
 //   -11 < z < 0:   logsig = z - log1p(u),  dlogsig = 1 / (1 + u)
 //   z <= -11:      logsig = z              (the reference drops the log1p term there)
 // log1p(u) = log(w) - ((w - 1) - u) / w with w = 1 + u keeps the low bits of u.
@@ -500,14 +501,12 @@ DEVINL void log_sigmoid_both(float z, float& value, float& grad) {
     const float w = 1.f + u;
     const float rw = __frcp_rn(w);
     const float l1p = __logf(w) - ((w - 1.f) - u) * rw;
-    if (z >= 0.f) {
-        const float uc = fmaxf(u, 1.670170079e-5f);  // exp(-11)
-        value = -l1p;
-        grad = uc * __frcp_rn(1.f + uc);
-    } else {
-        value = z > -11.f ? z - l1p : z;
-        grad = rw;
-    }
+    // straight-line selects (lanes of a wave mix both signs of z):
+    //   value = min(z, 0) - log1p(u), without the log1p term for z <= -11
+    //   grad  = u / (1 + u) clamped below at its value for u = e^-11 (z >= 0), 1 / (1 + u) (z < 0)
+    value = fminf(z, 0.f) - (z > -11.f ? l1p : 0.f);
+    const float g_pos = fmaxf(u * rw, 1.670142184e-5f);  // e^-11 / (1 + e^-11)
+    grad = z >= 0.f ? g_pos : rw;
 }
 
 struct FwdParams {
