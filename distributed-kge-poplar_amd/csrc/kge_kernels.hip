@@ -97,6 +97,8 @@ DEVINL float wave_sum(float v) {
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
 }
+// a wave-uniform float pinned to a scalar register
+DEVINL float uniform_f32(float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); }
 DEVINL float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
@@ -497,10 +499,12 @@ DEVINL float log_sigmoid_grad(float z) { return 1.f / (1.f + expf(fminf(z, 11.f)
 //   z <= -11:      logsig = z              (the reference drops the log1p term there)
 // log1p(u) = log(w) - ((w - 1) - u) / w with w = 1 + u keeps the low bits of u.
 DEVINL void log_sigmoid_both(float z, float& value, float& grad) {
-    const float u = __expf(-fabsf(z));
+    // single hardware instructions: exp2, rcp and log2 (about 1 ulp each; w is in [1, 2], so
+    // none of the range fix-ups of the library forms is needed)
+    const float u = __builtin_amdgcn_exp2f(-1.44269504089f * fabsf(z));
     const float w = 1.f + u;
-    const float rw = __frcp_rn(w);
-    const float l1p = __logf(w) - ((w - 1.f) - u) * rw;
+    const float rw = __builtin_amdgcn_rcpf(w);
+    const float l1p = 0.69314718056f * __builtin_amdgcn_logf(w) - ((w - 1.f) - u) * rw;
     // straight-line selects (lanes of a wave mix both signs of z):
     //   value = min(z, 0) - log1p(u), without the log1p term for z <= -11
     //   grad  = u / (1 + u) clamped below at its value for u = e^-11 (z >= 0), 1 / (1 + u) (z < 0)
@@ -598,8 +602,10 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
 
     // epilogue
     const float Tn = (float)T;
-    const float w_pos = 0.5f * Tn, w_neg = (0.5f * Tn) / (float)(T - 1);
-    const float inv_norm = 1.f / ((float)sh.S * (float)B * Tn);
+    // kept in scalar registers (see the matrix-core kernel's epilogue)
+    const float w_pos = uniform_f32(0.5f * Tn), w_neg = uniform_f32((0.5f * Tn) / (float)(T - 1));
+    const float inv_norm = uniform_f32(1.f / ((float)sh.S * (float)B * Tn));
+    const float grad_scale = uniform_f32(inv_norm * sh.loss_scale);
     float loss_acc = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -622,9 +628,9 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
             log_sigmoid_both(z, lsig, dlsig);
             if (n < T) loss_acc -= w * lsig;
             // d loss / d score, times the loss scale
-            const float ds = -w * sign * dlsig * inv_norm * sh.loss_scale;
+            const float ds = -w * sign * dlsig * grad_scale;
             float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;  // score = gamma - dist
-            if (DIST == DIST_L2) c = dist != 0.f ? c * __frcp_rn(dist) : 0.f;
+            if (DIST == DIST_L2) c = dist != 0.f ? c * __builtin_amdgcn_rcpf(dist) : 0.f;
             outv[j] = c;
         }
         const int n = n0 + tx * 4;
@@ -839,10 +845,16 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     // epilogue.  Accumulator layout of v_mfma_f32_32x32x2_f32: register r of
     // lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32.
     const float Tn = (float)T;
-    const float w_pos = 0.5f * Tn, w_neg = (0.5f * Tn) / (float)(T - 1);
-    const float inv_norm = 1.f / ((float)sh.S * (float)B * Tn);
+    // loss weights and the gradient scale, kept in scalar registers so that the compiler
+    // does not re-derive them (a division each) at every output
+    const float w_pos = uniform_f32(0.5f * Tn), w_neg = uniform_f32((0.5f * Tn) / (float)(T - 1));
+    const float inv_norm = uniform_f32(1.f / ((float)sh.S * (float)B * Tn));
+    const float grad_scale = uniform_f32(inv_norm * sh.loss_scale);
     float loss_acc = 0.f;
     const int n_loc = wn + (lane & 31), n = n0 + n_loc;
+    // outputs of this block: 32-bit offsets inside the block's [B, T] matrix
+    float* const coef_blk = p.coef + (size_t)d * B * T;
+    float* const dist_blk = p.dist ? p.dist + (size_t)d * B * T : nullptr;
     const float nb = DIST == DIST_L2 ? nb_s[n_loc] : 0.f;
 #pragma unroll
     for (int t = 0; t < AT; ++t) {
@@ -904,7 +916,7 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
                 const float score = sh.score_fn == SCORE_DISTMULT ? dist : sh.gamma - dist;
                 if (p.out_mode == 1) {
                     outv = score;
-                    if (live && DIST == DIST_L2 && p.dist) p.dist[((size_t)d * B + m) * T + n] = dist;
+                    if (live && DIST == DIST_L2 && dist_blk) dist_blk[m * T + n] = dist;
                 } else {
                     const bool pos = (uint32_t)n == label_s[m_loc];
                     const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
@@ -912,12 +924,12 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
                     float lsig, dlsig;
                     log_sigmoid_both(z, lsig, dlsig);
                     if (live) loss_acc -= w * lsig;
-                    const float ds = -w * sign * dlsig * inv_norm * sh.loss_scale;
+                    const float ds = -w * sign * dlsig * grad_scale;
                     outv = sh.score_fn == SCORE_DISTMULT ? ds : -ds;
-                    if (DIST == DIST_L2) outv = dist != 0.f ? outv * __frcp_rn(dist) : 0.f;
+                    if (DIST == DIST_L2) outv = dist != 0.f ? outv * __builtin_amdgcn_rcpf(dist) : 0.f;
                 }
             }
-            if (live) p.coef[((size_t)d * B + m) * T + n] = outv;
+            if (live) coef_blk[m * T + n] = outv;
         }
         if (DIST == DIST_L2 && p.nearflag) {
             // this wave owns the whole 32x32 sub-block: a plain store, no atomics
