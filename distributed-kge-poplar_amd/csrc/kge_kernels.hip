@@ -531,7 +531,7 @@ struct FwdParams {
 constexpr int BK = 32;         // embedding columns staged per iteration
 constexpr int LDP = kScoreTile + 4;  // padded LDS row (floats), keeps float4 reads aligned
 
-template <int DIST>
+template <int DIST, int OM>  // OM: FwdParams::out_mode, fixed at compile time
 __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
     __shared__ __attribute__((aligned(16))) float As[BK][LDP];
     __shared__ __attribute__((aligned(16))) float Bs[BK][LDP];
@@ -542,7 +542,7 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
     const int d = tile.z, m0 = tile.y * kScoreTile, n0 = tile.x * kScoreTile;
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int B = sh.B, T = sh.T, Dp = sh.Dp;
-    if (p.out_mode == 0 && tid < kScoreTile) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
+    if (OM == 0 && tid < kScoreTile) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
 
     // staging assignment: row lr (+32) of each operand, float4 column k4
     const int lr = tid >> 3, k4 = (tid & 7) * 4;
@@ -611,16 +611,16 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
     for (int i = 0; i < 4; ++i) {
         const int m = m0 + ty * 4 + i;
         if (m >= B) continue;
-        const uint32_t label = p.out_mode == 0 ? label_s[ty * 4 + i] : 0u;
+        const uint32_t label = OM == 0 ? label_s[ty * 4 + i] : 0u;
         float outv[4], distv[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
             const float dist = DIST == DIST_L2 ? sqrtf(acc[i][j]) : acc[i][j];
             distv[j] = dist;
-            if (p.out_mode == 2) { outv[j] = dist; continue; }
+            if (OM == 2) { outv[j] = dist; continue; }
             const float score = sh.score_fn == SCORE_DISTMULT ? dist : sh.gamma - dist;
-            if (p.out_mode == 1) { outv[j] = score; continue; }
+            if (OM == 1) { outv[j] = score; continue; }
             const bool pos = (uint32_t)n == label;
             const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
             const float z = sign * score;
@@ -635,7 +635,7 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
         }
         const int n = n0 + tx * 4;
         float* crow = p.coef + ((size_t)d * B + m) * T;
-        float* drow = (p.out_mode == 1 && DIST == DIST_L2 && p.dist) ? p.dist + ((size_t)d * B + m) * T : nullptr;
+        float* drow = (OM == 1 && DIST == DIST_L2 && p.dist) ? p.dist + ((size_t)d * B + m) * T : nullptr;
         if (n + 3 < T && (T & 3) == 0) {
             *reinterpret_cast<float4*>(crow + n) = make_float4(outv[0], outv[1], outv[2], outv[3]);
             if (drow) *reinterpret_cast<float4*>(drow + n) = make_float4(distv[0], distv[1], distv[2], distv[3]);
@@ -648,7 +648,7 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
                 }
         }
     }
-    if (p.out_mode == 0) {
+    if (OM == 0) {
         loss_acc = wave_sum(loss_acc);
         if ((tid & 63) == 0) red[tid >> 6] = loss_acc;
         __syncthreads();
@@ -690,7 +690,9 @@ constexpr float kNearRatio = 1.f / 4096.f;
 // the relation already applied: the staging loads carry no bounds checks (and
 // so no branches that would force the prefetch to complete before the matrix
 // work starts).
-template <int DIST, int BKT, bool ALIGNED, int NW>
+// OM: what the epilogue stores (FwdParams::out_mode), a template parameter so that the
+// sixteen outputs of a lane form one straight-line block the scheduler can interleave
+template <int DIST, int BKT, bool ALIGNED, int NW, int OM>
 __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     constexpr int NT = NW * 64;       // threads
     constexpr int AT = 8 / NW;        // 32-row accumulator tiles per wave (NW/2 waves cover 128 rows)
@@ -713,7 +715,7 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * (32 * AT), wn = (wave & 1) * 32;
     const int B = sh.B, T = sh.T, Dp = sh.Dp;
-    if (p.out_mode == 0 && tid < FM_TM) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
+    if (OM == 0 && tid < FM_TM) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
 
     const int srow = tid >> 3, k4 = (tid & 7) * 4;
     const char* arow[HA];
@@ -903,6 +905,10 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
             }
         }
         // phase 3 (straight-line): distance, score, loss, backward coefficient
+        uint32_t label_r[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            label_r[r] = OM == 0 ? label_s[wm + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)] : 0u;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int m_loc = wm + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
@@ -910,15 +916,15 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
             const bool live = ALIGNED || (m < B && n < T);
             const float dist = DIST == DIST_L2 ? __builtin_amdgcn_sqrtf(fmaxf(val[r], 0.f)) : val[r];
             float outv;
-            if (p.out_mode == 2) {
+            if (OM == 2) {
                 outv = dist;
             } else {
                 const float score = sh.score_fn == SCORE_DISTMULT ? dist : sh.gamma - dist;
-                if (p.out_mode == 1) {
+                if (OM == 1) {
                     outv = score;
                     if (live && DIST == DIST_L2 && dist_blk) dist_blk[m * T + n] = dist;
                 } else {
-                    const bool pos = (uint32_t)n == label_s[m_loc];
+                    const bool pos = (uint32_t)n == label_r[r];
                     const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
                     const float z = sign * score;
                     float lsig, dlsig;
@@ -939,7 +945,7 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
             if (lane == 0 && mt < MT && nt < NTL) p.nearflag[((size_t)d * MT + mt) * NTL + nt] = any ? 1u : 0u;
         }
     }
-    if (p.out_mode == 0) {
+    if (OM == 0) {
         loss_acc = wave_sum(loss_acc);
         if (lane == 0) red[wave] = loss_acc;
         __syncthreads();
@@ -969,23 +975,34 @@ static void launch_fwd(const FwdParams& p, hipStream_t stream) {
         const bool f32 = p.ent_a.etype == ET_F32 && p.ent_b.etype == ET_F32;
         const bool aligned = f32 && p.a_rel_mode == 0 && !p.ent_a.index && !p.ent_b.index &&
                              p.sh.B % FM_TM == 0 && p.sh.T % FM_TN == 0;
-#define KGE_FWD(D_)                                                                                          \
+#define KGE_FWD_OM(D_, OM_)                                                                                  \
     do {                                                                                                     \
         if (aligned && p.sh.Dp % 32 == 0) /* eight waves: two per SIMD hide each other's latencies */   \
-            hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true, 8>), grid, dim3(512), 0, stream, p);           \
-        else hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, false, 4>), grid, dim3(256), 0, stream, p);         \
+            hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true, 8, OM_>), grid, dim3(512), 0, stream, p);      \
+        else hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, false, 4, OM_>), grid, dim3(256), 0, stream, p);    \
+    } while (0)
+#define KGE_FWD(D_)                                                                                          \
+    do {                                                                                                     \
+        if (p.out_mode == 0) KGE_FWD_OM(D_, 0);                                                              \
+        else if (p.out_mode == 1) KGE_FWD_OM(D_, 1);                                                         \
+        else KGE_FWD_OM(D_, 2);                                                                              \
     } while (0)
         if (p.sh.dist_fn == DIST_L2) KGE_FWD(DIST_L2); else KGE_FWD(DIST_DOT);
+#undef KGE_FWD_OM
 #undef KGE_FWD
         return;
     }
     const dim3 grid = tile_grid((p.sh.T + kScoreTile - 1) / kScoreTile, (p.sh.B + kScoreTile - 1) / kScoreTile, p.sh.S);
-    if (p.sh.dist_fn == DIST_L1)
-        hipLaunchKernelGGL(k_score_fwd<DIST_L1>, grid, dim3(256), 0, stream, p);
-    else if (p.sh.dist_fn == DIST_L2)
-        hipLaunchKernelGGL(k_score_fwd<DIST_L2>, grid, dim3(256), 0, stream, p);
-    else
-        hipLaunchKernelGGL(k_score_fwd<DIST_DOT>, grid, dim3(256), 0, stream, p);
+#define KGE_FWD_VALU(D_)                                                                                     \
+    do {                                                                                                     \
+        if (p.out_mode == 0) hipLaunchKernelGGL((k_score_fwd<D_, 0>), grid, dim3(256), 0, stream, p);         \
+        else if (p.out_mode == 1) hipLaunchKernelGGL((k_score_fwd<D_, 1>), grid, dim3(256), 0, stream, p);    \
+        else hipLaunchKernelGGL((k_score_fwd<D_, 2>), grid, dim3(256), 0, stream, p);                         \
+    } while (0)
+    if (p.sh.dist_fn == DIST_L1) KGE_FWD_VALU(DIST_L1);
+    else if (p.sh.dist_fn == DIST_L2) KGE_FWD_VALU(DIST_L2);
+    else KGE_FWD_VALU(DIST_DOT);
+#undef KGE_FWD_VALU
 }
 
 void launch_score_fwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
