@@ -319,8 +319,9 @@ void parse_settings(kge_engine& E, const Items& s) {
     if (s.find("execution.scoring")) {
         const std::string v = s.str("execution.scoring");
         if (v == "mfma") E.use_mfma = 1;
+        else if (v == "mfma_bf16x3") E.use_mfma = 2;
         else if (v == "valu") E.use_mfma = 0;
-        else throw std::invalid_argument("'execution.scoring' must be 'mfma' or 'valu', not '" + v + "'");
+        else throw std::invalid_argument("'execution.scoring' must be 'mfma', 'mfma_bf16x3' or 'valu', not '" + v + "'");
     }
 
     if (s.find("execution.scoring_dtype")) {

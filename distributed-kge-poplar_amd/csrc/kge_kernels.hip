@@ -673,6 +673,44 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 DEVINL floatx4 as_x4(float4 v) { return floatx4{v.x, v.y, v.z, v.w}; }
 DEVINL float4 as_f4(floatx4 v) { return make_float4(v.x, v.y, v.z, v.w); }
 
+// float32 products from bfloat16 matrix instructions.  Every float32 value is
+// the exact sum of three bfloat16 pieces (round to nearest of the value, of what
+// that leaves, and of what that leaves: 8 + 8 + 8 significant bits), and
+//   a * b = a0 b0 + (a0 b1 + a1 b0) + (a1 b1 + a0 b2 + a2 b0) + O(2^-24 |a b|):
+// six v_mfma_f32_32x32x16_bf16 (float32 accumulate) per sixteen columns instead
+// of eight v_mfma_f32_32x32x2_f32, at sixteen times the rate per instruction.
+// Measured against float64 the sums are as accurate as the float32 instruction's.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+DEVINL uint32_t pack_bf16(float a, float b) {
+    return __builtin_bit_cast(uint32_t, bf16x2{(__bf16)a, (__bf16)b});
+}
+DEVINL float bf16_lo_f32(uint32_t pair) { return __uint_as_float(pair << 16); }
+DEVINL float bf16_hi_f32(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
+// four values -> their three pieces, four bfloat16 (8 bytes) per piece
+DEVINL void split4_bf16(floatx4 v, uint2 piece[3]) {
+    float r[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+        const uint32_t p0 = pack_bf16(r[0], r[1]), p1 = pack_bf16(r[2], r[3]);
+        piece[q] = make_uint2(p0, p1);
+        if (q < 2) {
+            r[0] -= bf16_lo_f32(p0); r[1] -= bf16_hi_f32(p0);
+            r[2] -= bf16_lo_f32(p1); r[3] -= bf16_hi_f32(p1);
+        }
+    }
+}
+// the six products of one 16-column step, smallest first; a[q], b[q] hold piece q of
+// eight consecutive columns of this lane's row
+DEVINL floatx16 mfma_split6(const floatx4 a[3], const floatx4 b[3], floatx16 acc) {
+#define KGE_MM(x_, y_)                                                                                \
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[x_]),                  \
+                                                  __builtin_bit_cast(bf16x8, b[y_]), acc, 0, 0, 0)
+    KGE_MM(0, 2); KGE_MM(2, 0); KGE_MM(1, 1); KGE_MM(0, 1); KGE_MM(1, 0); KGE_MM(0, 0);
+#undef KGE_MM
+    return acc;
+}
+
 constexpr int FM_TM = 128, FM_TN = 64;
 constexpr float kCancelRatio = 0.125f;  // recompute when d^2 < ratio * (|a|^2 + |b|^2)
 // Below this ratio the backward's product form self*sum(c) - sum(c*other) would
@@ -692,7 +730,9 @@ constexpr float kNearRatio = 1.f / 4096.f;
 // work starts).
 // OM: what the epilogue stores (FwdParams::out_mode), a template parameter so that the
 // sixteen outputs of a lane form one straight-line block the scheduler can interleave
-template <int DIST, int BKT, bool ALIGNED, int NW, int OM>
+// SPLIT: the products run as six bfloat16 matrix instructions on three-piece operands
+// (split4_bf16): the tiles hold the three pieces of every value, split while staging.
+template <int DIST, int BKT, bool ALIGNED, int NW, int OM, bool SPLIT = false>
 __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     constexpr int NT = NW * 64;       // threads
     constexpr int AT = 8 / NW;        // 32-row accumulator tiles per wave (NW/2 waves cover 128 rows)
@@ -704,8 +744,13 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     // its row in one 16-byte LDS read that feeds four matrix instructions.  The
     // pitch of BKT + 4 floats spreads eight consecutive rows over all banks.
     constexpr int LDT = BKT + 4;
-    __shared__ __attribute__((aligned(16))) float As[FM_TM][LDT];
-    __shared__ __attribute__((aligned(16))) float Bs[FM_TN][LDT];
+    __shared__ __attribute__((aligned(16))) float As[SPLIT ? 1 : FM_TM][LDT];
+    __shared__ __attribute__((aligned(16))) float Bs[SPLIT ? 1 : FM_TN][LDT];
+    // SPLIT: piece q of row r, columns contiguous; the pitch of BKT + 8 bfloat16 (80 bytes
+    // for BKT = 32) puts sixteen consecutive rows' 16-byte reads in different banks
+    constexpr int LDH = BKT + 8;
+    __shared__ __attribute__((aligned(16))) uint16_t Ap[SPLIT ? 3 : 1][SPLIT ? FM_TM : 1][LDH];
+    __shared__ __attribute__((aligned(16))) uint16_t Bp[SPLIT ? 3 : 1][SPLIT ? FM_TN : 1][LDH];
     __shared__ float na_s[FM_TM], nb_s[FM_TN];
     __shared__ float red[NW];
     __shared__ uint32_t label_s[FM_TM];
@@ -782,18 +827,57 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
 #pragma unroll
             for (int h = 0; h < HA; ++h) {
                 const float4 a = areg[h][c];
-                *reinterpret_cast<float4*>(&As[srow + RP * h][kc]) = a;
+                if constexpr (SPLIT) {
+                    uint2 piece[3];
+                    split4_bf16(as_x4(a), piece);
+#pragma unroll
+                    for (int q = 0; q < 3; ++q) *reinterpret_cast<uint2*>(&Ap[q][srow + RP * h][kc]) = piece[q];
+                } else {
+                    *reinterpret_cast<float4*>(&As[srow + RP * h][kc]) = a;
+                }
                 if (DIST == DIST_L2) na_acc[h] += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
             }
 #pragma unroll
             for (int h = 0; h < HB; ++h) {
                 const float4 b = breg[h][c];
-                *reinterpret_cast<float4*>(&Bs[srow + RP * h][kc]) = b;
+                if constexpr (SPLIT) {
+                    uint2 piece[3];
+                    split4_bf16(as_x4(b), piece);
+#pragma unroll
+                    for (int q = 0; q < 3; ++q) *reinterpret_cast<uint2*>(&Bp[q][srow + RP * h][kc]) = piece[q];
+                } else {
+                    *reinterpret_cast<float4*>(&Bs[srow + RP * h][kc]) = b;
+                }
                 if (DIST == DIST_L2) nb_acc[h] += b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
             }
         }
         __syncthreads();
         if (k0 + BKT < Dp) prefetch(k0 + BKT);
+        if constexpr (SPLIT) {
+            // a step covers sixteen columns: a lane supplies columns 8 * (lane / 32) .. + 7 of its
+            // row, for both operands; the pieces of the next step are fetched under this one's work
+            constexpr int NS = BKT / 16;
+            floatx4 fa[2][AT][3], fb[2][3];
+            const int hl = lane >> 5, cl = lane & 31;
+            auto fetch = [&](int buf, int ks) __attribute__((always_inline)) {
+#pragma unroll
+                for (int q = 0; q < 3; ++q) {
+                    fb[buf][q] = *reinterpret_cast<const floatx4*>(&Bp[q][wn + cl][16 * ks + 8 * hl]);
+#pragma unroll
+                    for (int t = 0; t < AT; ++t)
+                        fa[buf][t][q] = *reinterpret_cast<const floatx4*>(&Ap[q][wm + 32 * t + cl][16 * ks + 8 * hl]);
+                }
+            };
+            fetch(0, 0);
+#pragma unroll
+            for (int ks = 0; ks < NS; ++ks) {
+                if (ks + 1 < NS) fetch((ks + 1) & 1, ks + 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < AT; ++t) acc[t] = mfma_split6(fa[ks & 1][t], fb[ks & 1], acc[t]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else
         // Each group of four matrix instructions covers eight columns: instruction
         // x takes column 8g + x from the lower half-wave and 8g + 4 + x from the
         // upper one.  Operands are fetched one group ahead of their use.
@@ -977,7 +1061,9 @@ static void launch_fwd(const FwdParams& p, hipStream_t stream) {
                              p.sh.B % FM_TM == 0 && p.sh.T % FM_TN == 0;
 #define KGE_FWD_OM(D_, OM_)                                                                                  \
     do {                                                                                                     \
-        if (aligned && p.sh.Dp % 32 == 0) /* eight waves: two per SIMD hide each other's latencies */   \
+        if (aligned && p.sh.Dp % 32 == 0 && p.sh.use_mfma == 2)                                              \
+            hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true, 4, OM_, true>), grid, dim3(256), 0, stream, p); \
+        else if (aligned && p.sh.Dp % 32 == 0) /* eight waves: two per SIMD hide each other's latencies */ \
             hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true, 8, OM_>), grid, dim3(512), 0, stream, p);      \
         else hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, false, 4, OM_>), grid, dim3(256), 0, stream, p);    \
     } while (0)
@@ -1031,8 +1117,6 @@ void launch_score_fwd(const ScoreShape& sh, const RowSource& ent, const float* r
 // the current one is multiplied.  LDS rows are padded to 72 elements (144 B) so
 // that eight consecutive rows' 16-byte reads fall in different banks.
 // Shapes: M % 128 == 0, N % 128 == 0, K % 64 == 0, rows 16-byte aligned.
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-
 constexpr int GB_T = 128, GB_K = 64, GB_LD = GB_K + 8;
 
 __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {

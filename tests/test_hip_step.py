@@ -199,6 +199,14 @@ def test_step_vs_oracle_valu_scoring(oracle64, name):
     run_case(oracle64, CASES[name], **{"execution.scoring": "valu"})
 
 
+@pytest.mark.parametrize("name", ["aligned_l2", "aligned_l2_wide", "aligned_distmult", "aligned_l2_softmax",
+                                  "bf16_embedding_l2", "l2_feat", "mid_l2"])
+def test_step_vs_oracle_split_scoring(oracle64, name):
+    # float32 products from six bfloat16 matrix instructions on three-piece operands: the same
+    # float32 bars (ragged shapes fall back to the float32 instruction)
+    run_case(oracle64, CASES[name], **{"execution.scoring": "mfma_bf16x3"})
+
+
 def test_step_l1_equal_and_signed_zero_entries(oracle64):
     # signum(0) = 0 on the one-pass L1 backward: identical rows under a zero
     # relation, zero entries of either sign, and rows that differ in a few columns
@@ -300,7 +308,7 @@ def test_step_near_duplicate_rows(oracle64):
         assert K.rel_l2(st_h[k] - st0[k], st_o[k] - st0[k]) < 1e-4, k
 
 
-@pytest.mark.parametrize("scoring", ["mfma", "valu"])
+@pytest.mark.parametrize("scoring", ["mfma", "mfma_bf16x3", "valu"])
 def test_step_near_duplicate_rows_aligned(oracle64, scoring):
     # the same hazard at tile-aligned shapes: the fast path flags the 32x32 score
     # sub-blocks that hold near-identical pairs and the backward treats them directly
