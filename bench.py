@@ -241,7 +241,7 @@ def main():
                     help="steps the CPU baseline times (default: sized for ~10-30 s)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--n-entity", type=int, default=None, help="override the table size (experiments)")
-    ap.add_argument("--scoring", default=None, choices=["mfma", "mfma_bf16x3", "valu"], help="scoring kernels (default mfma)")
+    ap.add_argument("--scoring", default=None, choices=["mfma", "mfma_bf16x3", "valu"], help="scoring kernels (default mfma_bf16x3)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU holding one shard's whole table: --gpus must be 1 "

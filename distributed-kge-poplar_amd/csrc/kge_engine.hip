@@ -194,7 +194,10 @@ struct kge_engine {
     int predict_hr_batch = 0, predict_n_best = 0;
     int stream_kind;  // KGE_F32 or KGE_F16: dtype of the entity read/write streams
     bool profile_kernels = false;
-    int use_mfma = 1;  // additive setting execution.scoring = "mfma" | "valu"
+    // additive setting execution.scoring: "mfma_bf16x3" (2, the default: matrix cores, the forward
+    // products from six bfloat16 instructions on three-piece float32 operands where shapes are
+    // aligned), "mfma" (1: float32 matrix instructions only), "valu" (0)
+    int use_mfma = 2;
     bool score_bf16 = false;  // additive setting execution.scoring_dtype = "float32" | "bfloat16"
     int chunk = 64;       // contributions per first-level chunk (rows with many contributions; 256 measured no faster)
     int direct_max = 16;  // rows with at most this many contributions are summed by their Adam wave

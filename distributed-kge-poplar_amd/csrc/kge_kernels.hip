@@ -12,6 +12,7 @@
 #include "kge_kernels.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace kge {
 
@@ -668,6 +669,15 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
 // the pair is recomputed directly as sum (a-b)^2 by the whole wave, so the
 // result keeps float32 accuracy and is exactly 0 for identical rows.
 
+// f(integral_constant<0>) ... f(integral_constant<N-1>): a loop whose index is a compile-time constant
+template <int N, int I = 0, class F>
+DEVINL void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
+
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 DEVINL floatx4 as_x4(float4 v) { return floatx4{v.x, v.y, v.z, v.w}; }
@@ -732,7 +742,9 @@ constexpr float kNearRatio = 1.f / 4096.f;
 // sixteen outputs of a lane form one straight-line block the scheduler can interleave
 // SPLIT: the products run as six bfloat16 matrix instructions on three-piece operands
 // (split4_bf16): the tiles hold the three pieces of every value, split while staging.
-template <int DIST, int BKT, bool ALIGNED, int NW, int OM, bool SPLIT = false>
+// PF: slabs of operand loads in flight (register sets).  A slab's loads take a round trip to the
+// memory-side cache however little work the slab is, so with PF = 1 that latency is paid per slab.
+template <int DIST, int BKT, bool ALIGNED, int NW, int OM, bool SPLIT = false, int PF = 1>
 __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     constexpr int NT = NW * 64;       // threads
     constexpr int AT = 8 / NW;        // 32-row accumulator tiles per wave (NW/2 waves cover 128 rows)
@@ -746,11 +758,11 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     constexpr int LDT = BKT + 4;
     __shared__ __attribute__((aligned(16))) float As[SPLIT ? 1 : FM_TM][LDT];
     __shared__ __attribute__((aligned(16))) float Bs[SPLIT ? 1 : FM_TN][LDT];
-    // SPLIT: piece q of row r, columns contiguous; the pitch of BKT + 8 bfloat16 (80 bytes
-    // for BKT = 32) puts sixteen consecutive rows' 16-byte reads in different banks
-    constexpr int LDH = BKT + 8;
-    __shared__ __attribute__((aligned(16))) uint16_t Ap[SPLIT ? 3 : 1][SPLIT ? FM_TM : 1][LDH];
-    __shared__ __attribute__((aligned(16))) uint16_t Bp[SPLIT ? 3 : 1][SPLIT ? FM_TN : 1][LDH];
+    // SPLIT: two copies of [piece][row][32 columns] bfloat16; rows of 64 bytes whose four
+    // 16-byte chunks are stored at position chunk ^ ((row / 4) % 4), which puts sixteen
+    // consecutive rows' reads of one chunk in different banks without padding
+    __shared__ __attribute__((aligned(16))) uint16_t Ap[SPLIT ? 2 : 1][SPLIT ? 3 : 1][SPLIT ? FM_TM : 1][BKT];
+    __shared__ __attribute__((aligned(16))) uint16_t Bp[SPLIT ? 2 : 1][SPLIT ? 3 : 1][SPLIT ? FM_TN : 1][BKT];
     __shared__ float na_s[FM_TM], nb_s[FM_TN];
     __shared__ float red[NW];
     __shared__ uint32_t label_s[FM_TM];
@@ -794,90 +806,140 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
 
-    float4 areg[HA][NC], breg[HB][NC];
-    auto prefetch = [&](int k0) {
+    floatx4 areg[PF][HA][NC], breg[PF][HB][NC];
+    auto prefetch = [&](auto set, int k0) __attribute__((always_inline)) {
+        constexpr int s = decltype(set)::value;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int k = k0 + 32 * c + k4;
             if (ALIGNED) {
 #pragma unroll
-                for (int h = 0; h < HA; ++h) areg[h][c] = *reinterpret_cast<const float4*>(arow[h] + (size_t)k * 4);
+                for (int h = 0; h < HA; ++h) areg[s][h][c] = *reinterpret_cast<const floatx4*>(arow[h] + (size_t)k * 4);
 #pragma unroll
-                for (int h = 0; h < HB; ++h) breg[h][c] = *reinterpret_cast<const float4*>(brow[h] + (size_t)k * 4);
+                for (int h = 0; h < HB; ++h) breg[s][h][c] = *reinterpret_cast<const floatx4*>(brow[h] + (size_t)k * 4);
                 continue;
             }
 #pragma unroll
             for (int h = 0; h < HA; ++h) {
-                areg[h][c] = make_float4(0, 0, 0, 0);
+                areg[s][h][c] = floatx4{0.f, 0.f, 0.f, 0.f};
                 if (arow[h] && k < Dp)
-                    areg[h][c] = combine_rel(load4(arow[h], k, p.ent_a), rrow[h], k, p.a_rel_mode);
+                    areg[s][h][c] = as_x4(combine_rel(load4(arow[h], k, p.ent_a), rrow[h], k, p.a_rel_mode));
             }
 #pragma unroll
             for (int h = 0; h < HB; ++h) {
-                breg[h][c] = make_float4(0, 0, 0, 0);
-                if (brow[h] && k < Dp) breg[h][c] = load4(brow[h], k, p.ent_b);
+                breg[s][h][c] = floatx4{0.f, 0.f, 0.f, 0.f};
+                if (brow[h] && k < Dp) breg[s][h][c] = as_x4(load4(brow[h], k, p.ent_b));
             }
         }
     };
-    prefetch(0);
-    for (int k0 = 0; k0 < Dp; k0 += BKT) {
+    static_for<PF>([&](auto set) {
+        if (ALIGNED || decltype(set)::value * BKT < Dp) prefetch(set, decltype(set)::value * BKT);
+    });
+    if constexpr (SPLIT) {
+        static_assert(BKT == 32 && PF % 2 == 0 && ALIGNED, "the three-piece path: aligned shapes, slabs of 32");
+        const int hl = lane >> 5, cl = lane & 31;
+        // writes one register set (a slab) into tile copy `buf`, as pieces; `live` = 0 for the
+        // slab past the end (its squares must not count)
+        auto stage = [&](auto set, auto bufc, float live) __attribute__((always_inline)) {
+            constexpr int s = decltype(set)::value, buf = decltype(bufc)::value;
+#pragma unroll
+            for (int h = 0; h < HA; ++h) {
+                const int row = srow + RP * h;
+                const int col = (((k4 >> 3) ^ ((row >> 2) & 3)) << 3) + (k4 & 4);
+                const floatx4 a = areg[s][h][0];
+                uint2 piece[3];
+                split4_bf16(a, piece);
+#pragma unroll
+                for (int q = 0; q < 3; ++q) *reinterpret_cast<uint2*>(&Ap[buf][q][row][col]) = piece[q];
+                if (DIST == DIST_L2) na_acc[h] += live * (a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w);
+            }
+#pragma unroll
+            for (int h = 0; h < HB; ++h) {
+                const int row = srow + RP * h;
+                const int col = (((k4 >> 3) ^ ((row >> 2) & 3)) << 3) + (k4 & 4);
+                const floatx4 b = breg[s][h][0];
+                uint2 piece[3];
+                split4_bf16(b, piece);
+#pragma unroll
+                for (int q = 0; q < 3; ++q) *reinterpret_cast<uint2*>(&Bp[buf][q][row][col]) = piece[q];
+                if (DIST == DIST_L2) nb_acc[h] += live * (b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w);
+            }
+        };
+        using I0 = std::integral_constant<int, 0>;
+        stage(I0{}, I0{}, 1.f);
+        prefetch(I0{}, min(PF * BKT, Dp - BKT));
+        __syncthreads();
+        // One barrier per slab: while the matrix cores work on one tile copy the next slab is
+        // split into the other, the splitting instructions issued between the matrix
+        // instructions (each of which depends on the one before it).
+        for (int kb = 0; kb < Dp; kb += PF * BKT)
+        static_for<PF>([&](auto sc) {
+            constexpr int s = decltype(sc)::value;
+            using Next = std::integral_constant<int, (s + 1) % PF>;
+            using Other = std::integral_constant<int, (s + 1) & 1>;
+            constexpr int buf = s & 1;
+            const int k0 = kb + s * BKT;
+            // the slab in tile copy `buf`: two steps of sixteen columns; a lane supplies columns
+            // 8 * (lane / 32) .. + 7 of a step, of its row, for both operands
+            floatx4 fa[2][AT][3], fb[2][3];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const int chunk = 2 * ks + hl;
+#pragma unroll
+                for (int q = 0; q < 3; ++q) {
+                    const int rb = wn + cl;
+                    fb[ks][q] = *reinterpret_cast<const floatx4*>(&Bp[buf][q][rb][(chunk ^ ((rb >> 2) & 3)) << 3]);
+#pragma unroll
+                    for (int t = 0; t < AT; ++t) {
+                        const int ra = wm + 32 * t + cl;
+                        fa[ks][t][q] = *reinterpret_cast<const floatx4*>(&Ap[buf][q][ra][(chunk ^ ((ra >> 2) & 3)) << 3]);
+                    }
+                }
+            }
+            stage(Next{}, Other{}, k0 + BKT < Dp ? 1.f : 0.f);
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int t = 0; t < AT; ++t) acc[t] = mfma_split6(fa[ks][t], fb[ks], acc[t]);
+            // the order asked of the scheduler: the LDS reads, then one matrix instruction,
+            // a share of the vector work and an LDS write, in turn
+            __builtin_amdgcn_sched_group_barrier(0x100, 6 * (AT + 1), 0);
+#pragma unroll
+            for (int i = 0; i < 12 * AT; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, (30 * (HA + HB) + 12 * AT - 1) / (12 * AT), 0);
+                if (i < 3 * (HA + HB)) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            }
+            prefetch(Next{}, min(k0 + BKT + PF * BKT, Dp - BKT));
+            __syncthreads();
+        });
+    } else
+    for (int kb = 0; kb < Dp; kb += PF * BKT)
+    static_for<PF>([&](auto set) {
+        constexpr int s = decltype(set)::value;
+        const int k0 = kb + s * BKT;
+        if (!ALIGNED && PF > 1 && k0 >= Dp) return;  // ALIGNED: Dp % (PF * BKT) == 0
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int kc = 32 * c + k4;
 #pragma unroll
             for (int h = 0; h < HA; ++h) {
-                const float4 a = areg[h][c];
-                if constexpr (SPLIT) {
-                    uint2 piece[3];
-                    split4_bf16(as_x4(a), piece);
-#pragma unroll
-                    for (int q = 0; q < 3; ++q) *reinterpret_cast<uint2*>(&Ap[q][srow + RP * h][kc]) = piece[q];
-                } else {
-                    *reinterpret_cast<float4*>(&As[srow + RP * h][kc]) = a;
-                }
+                const float4 a = as_f4(areg[s][h][c]);
+                *reinterpret_cast<float4*>(&As[srow + RP * h][kc]) = a;
                 if (DIST == DIST_L2) na_acc[h] += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
             }
 #pragma unroll
             for (int h = 0; h < HB; ++h) {
-                const float4 b = breg[h][c];
-                if constexpr (SPLIT) {
-                    uint2 piece[3];
-                    split4_bf16(as_x4(b), piece);
-#pragma unroll
-                    for (int q = 0; q < 3; ++q) *reinterpret_cast<uint2*>(&Bp[q][srow + RP * h][kc]) = piece[q];
-                } else {
-                    *reinterpret_cast<float4*>(&Bs[srow + RP * h][kc]) = b;
-                }
+                const float4 b = as_f4(breg[s][h][c]);
+                *reinterpret_cast<float4*>(&Bs[srow + RP * h][kc]) = b;
                 if (DIST == DIST_L2) nb_acc[h] += b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
             }
         }
         __syncthreads();
-        if (k0 + BKT < Dp) prefetch(k0 + BKT);
-        if constexpr (SPLIT) {
-            // a step covers sixteen columns: a lane supplies columns 8 * (lane / 32) .. + 7 of its
-            // row, for both operands; the pieces of the next step are fetched under this one's work
-            constexpr int NS = BKT / 16;
-            floatx4 fa[2][AT][3], fb[2][3];
-            const int hl = lane >> 5, cl = lane & 31;
-            auto fetch = [&](int buf, int ks) __attribute__((always_inline)) {
-#pragma unroll
-                for (int q = 0; q < 3; ++q) {
-                    fb[buf][q] = *reinterpret_cast<const floatx4*>(&Bp[q][wn + cl][16 * ks + 8 * hl]);
-#pragma unroll
-                    for (int t = 0; t < AT; ++t)
-                        fa[buf][t][q] = *reinterpret_cast<const floatx4*>(&Ap[q][wm + 32 * t + cl][16 * ks + 8 * hl]);
-                }
-            };
-            fetch(0, 0);
-#pragma unroll
-            for (int ks = 0; ks < NS; ++ks) {
-                if (ks + 1 < NS) fetch((ks + 1) & 1, ks + 1);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int t = 0; t < AT; ++t) acc[t] = mfma_split6(fa[ks & 1][t], fb[ks & 1], acc[t]);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        } else
+        // ALIGNED: branch-free (a branch here would merge the register set's old and new
+        // contents and wait for the loads at once); past the end the last slab is loaded again
+        if (ALIGNED) prefetch(set, min(k0 + PF * BKT, Dp - BKT));
+        else if (k0 + PF * BKT < Dp) prefetch(set, k0 + PF * BKT);
         // Each group of four matrix instructions covers eight columns: instruction
         // x takes column 8g + x from the lower half-wave and 8g + 4 + x from the
         // upper one.  Operands are fetched one group ahead of their use.
@@ -910,7 +972,7 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
             }
         }
         __syncthreads();
-    }
+    });
     if (DIST == DIST_L2) {
         // the 8 threads of a row hold partial sums of squares: combine in a fixed order
 #pragma unroll
@@ -1061,8 +1123,9 @@ static void launch_fwd(const FwdParams& p, hipStream_t stream) {
                              p.sh.B % FM_TM == 0 && p.sh.T % FM_TN == 0;
 #define KGE_FWD_OM(D_, OM_)                                                                                  \
     do {                                                                                                     \
-        if (aligned && p.sh.Dp % 32 == 0 && p.sh.use_mfma == 2)                                              \
-            hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true, 4, OM_, true>), grid, dim3(256), 0, stream, p); \
+        if (aligned && p.sh.Dp % 64 == 0 && p.sh.use_mfma == 2) {                                            \
+            hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true, 8, OM_, true, 2>), grid, dim3(512), 0, stream, p); \
+        }                                                                                                    \
         else if (aligned && p.sh.Dp % 32 == 0) /* eight waves: two per SIMD hide each other's latencies */ \
             hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, true, 8, OM_>), grid, dim3(512), 0, stream, p);      \
         else hipLaunchKernelGGL((k_score_fwd_mfma<D_, 32, false, 4, OM_>), grid, dim3(256), 0, stream, p);    \

@@ -199,12 +199,14 @@ def test_step_vs_oracle_valu_scoring(oracle64, name):
     run_case(oracle64, CASES[name], **{"execution.scoring": "valu"})
 
 
+@pytest.mark.parametrize("scoring", ["mfma", "mfma_bf16x3"])
 @pytest.mark.parametrize("name", ["aligned_l2", "aligned_l2_wide", "aligned_distmult", "aligned_l2_softmax",
                                   "bf16_embedding_l2", "l2_feat", "mid_l2"])
-def test_step_vs_oracle_split_scoring(oracle64, name):
-    # float32 products from six bfloat16 matrix instructions on three-piece operands: the same
-    # float32 bars (ragged shapes fall back to the float32 instruction)
-    run_case(oracle64, CASES[name], **{"execution.scoring": "mfma_bf16x3"})
+def test_step_vs_oracle_matrix_scoring(oracle64, name, scoring):
+    # the two matrix-core forms of the float32 products, named explicitly: float32 instructions
+    # ("mfma"), and six bfloat16 instructions on three-piece operands in the forward kernel
+    # ("mfma_bf16x3", the default; ragged shapes fall back to the float32 instruction): same bars
+    run_case(oracle64, CASES[name], **{"execution.scoring": scoring})
 
 
 def test_step_l1_equal_and_signed_zero_entries(oracle64):
