@@ -65,6 +65,7 @@ WORKLOADS = {
 
 PEAK_HBM_GBPS = 8000.0
 PEAK_FP32_TFLOPS = 157.3
+PEAK_BF16_TFLOPS = 2500.0
 
 # HBM bytes per launch (fetched + written) of the dominant kernel, from two
 # `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each
@@ -73,7 +74,7 @@ PEAK_FP32_TFLOPS = 157.3
 # here and refreshed together with the committed profiler summaries.
 MEASURED_TRAFFIC_BYTES = {
     ("c2", "score_bwd"): 41.8e6,     # 25.1 MB fetched + 16.8 MB written
-    ("c3l2", "score_bwd"): 151.3e6,  # 101.0 MB fetched + 50.3 MB written
+    ("c3l2", "score_bwd"): 148.4e6,  # 98.0 MB fetched + 50.3 MB written
 }
 
 
@@ -184,6 +185,14 @@ def cpu_baseline(engine, settings, w, batch, n_check, n_cpu_steps):
                        f"sequential float32 C oracle, 1 thread of {os.cpu_count()} host cpus"), loss
 
 
+def split_forward(w):
+    """Whether the forward kernel takes the three-piece bfloat16 path: the engine's default for
+    L2 / dot scoring on float32 operands at shapes aligned to its tiles."""
+    return (w.get("scoring") in (None, "mfma_bf16x3") and w.get("distance_fn", "L2") != "L1"
+            and w.get("scoring_dtype") != "bfloat16"
+            and w["batch"] % 128 == 0 and w["tails"] % 64 == 0 and w["dim"] % 64 == 0)
+
+
 def kernel_table(w, timing, n_steps, uniq_rows):
     """Algorithmic bytes / flops per launch and achieved rates of every kernel."""
     K_, B, T, D = w["blocks"], w["batch"], w["tails"], w["dim"]
@@ -223,8 +232,16 @@ def kernel_table(w, timing, n_steps, uniq_rows):
         if kind == "bytes":
             entry.update(bound="hbm", achieved=amount / (ms * 1e-3) / 1e9, peak=PEAK_HBM_GBPS, unit="GB/s")
         else:
-            entry.update(bound="mfma", achieved=amount / (ms * 1e-3) / 1e12, peak=PEAK_FP32_TFLOPS,
-                         unit="TFLOP/s")
+            # the published peak of the instruction the kernel issues: float32 matrix / vector
+            # instructions 157.3; bfloat16 matrix instructions 2500, of which the float32-product
+            # forward kernel issues six per product (three-piece operands)
+            peak, instr = PEAK_FP32_TFLOPS, "f32"
+            if w.get("scoring_dtype") == "bfloat16":
+                peak, instr = PEAK_BF16_TFLOPS, "bf16"
+            elif name == "score_fwd" and split_forward(w):
+                peak, instr = PEAK_BF16_TFLOPS / 6.0, "bf16 x6 (float32 products)"
+            entry.update(bound="mfma", achieved=amount / (ms * 1e-3) / 1e12, peak=peak, unit="TFLOP/s",
+                         instructions=instr)
         entry["frac"] = entry["achieved"] / entry["peak"]
         entry["algorithmic_per_step"] = amount
         out[name] = entry
@@ -263,7 +280,7 @@ def main():
     n_total = args.warmup + args.steps
     settings = make_settings(w, n_total, kge)
     if args.scoring:
-        settings.execution.scoring = args.scoring
+        settings.execution.scoring = w["scoring"] = args.scoring
     m, d = settings.model, settings.data
     engine = kge.Engine(settings, np.full(m.n_shard, m.n_entity - 1))
     init_tables(engine, settings)
