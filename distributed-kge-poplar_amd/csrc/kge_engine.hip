@@ -339,9 +339,10 @@ void parse_settings(kge_engine& E, const Items& s) {
 
     if (score == "TransE") E.score_fn = SCORE_TRANSE;
     else if (score == "DistMult") E.score_fn = SCORE_DISTMULT;
-    else if (score == "ComplEx" || score == "RotatE" || score == "TransH")
+    else if (score == "ComplEx") E.score_fn = SCORE_COMPLEX;
+    else if (score == "RotatE" || score == "TransH")
         throw std::invalid_argument("'model.score_fn' = '" + score + "' is not implemented on the HIP device "
-                                    "(supported: 'TransE', 'DistMult')");
+                                    "(supported: 'TransE', 'DistMult', 'ComplEx')");
     else
         throw std::invalid_argument("'model.score_fn' must be one of 'TransE', 'ComplEx', 'RotatE', 'TransH', or "
                                     "'DistMult', not '" + score + "'");
@@ -352,6 +353,10 @@ void parse_settings(kge_engine& E, const Items& s) {
     else
         throw std::invalid_argument("'model.distance_fn' must be one of 'L1', 'L2' or 'MatMul', not '" +
                                     distance + "'");
+    if (E.score_fn == SCORE_DISTMULT) E.dist_fn = DIST_DOT;  // distMultScore ignores the setting (:571-573)
+    if (E.score_fn == SCORE_COMPLEX && E.D % 2)
+        throw std::invalid_argument("'model.score_fn' = 'ComplEx' needs an even 'model.embedding_size' "
+                                    "(real and imaginary halves)");
     if (loss == "logsigmoid") E.loss_fn = LOSS_LOGSIGMOID;
     else if (loss == "softmax") E.loss_fn = LOSS_SOFTMAX;
     else
@@ -473,7 +478,7 @@ void allocate(kge_engine& E) {
 
     E.coef.alloc(SB * E.T);
     const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f && !E.score_bf16;
-    if (!fused && E.score_fn == SCORE_TRANSE && E.dist_fn == DIST_L2) E.dist.alloc(SB * E.T);
+    if (!fused && E.dist_fn == DIST_L2) E.dist.alloc(SB * E.T);
     if (E.score_bf16) {
         E.opnd16.alloc(R * E.Dp);
         E.opndT16.alloc(R * E.Dp);
@@ -488,7 +493,7 @@ void allocate(kge_engine& E) {
     E.opnd.alloc(R * E.Dp);
     E.partial.alloc((size_t)E.e_cstride * E.Dp);
     E.rel_partial.alloc((size_t)E.r_cstride * E.Dp);
-    if (E.score_fn == SCORE_DISTMULT) E.rel_gsum.alloc((size_t)E.n_rel * E.Dp);
+    if (E.score_fn != SCORE_TRANSE) E.rel_gsum.alloc((size_t)E.n_rel * E.Dp);
     if (E.F) {
         E.hidden.alloc(R * E.Dp);
         E.gsum.alloc(R * E.Dp);
@@ -508,7 +513,7 @@ void allocate(kge_engine& E) {
     sh.S = E.S; sh.B = E.B; sh.T = E.T;
     sh.score_fn = E.score_fn; sh.dist_fn = E.dist_fn; sh.use_mfma = E.use_mfma;
     E.n_part = fused ? score_fwd_parts(sh) : E.B;
-    if (E.use_mfma && E.score_fn == SCORE_TRANSE && E.dist_fn == DIST_L2) {
+    if (E.use_mfma && E.dist_fn == DIST_L2) {
         E.nearflag.alloc(nearflag_words(sh));
         E.nearflag.zero(st);
     }
@@ -738,6 +743,11 @@ void run_plan(kge_engine& E, int s0, int sn) {
     HIP_CHECK(hipGetLastError());
 }
 
+// how the gather combines a head row with its relation row (launch_gather_operands)
+static int rel_mode_of(const kge_engine& E) {
+    return E.score_fn == SCORE_DISTMULT ? 2 : E.score_fn == SCORE_COMPLEX ? 3 : 1;
+}
+
 void run_step(kge_engine& E, int i) {
     const hipStream_t st = E.stream;
     const size_t R = E.R, SB = (size_t)E.S * E.B;
@@ -785,7 +795,7 @@ void run_step(kge_engine& E, int i) {
 
     // dense operands: every contribution's row, float32, relation applied to the heads
     { KernelTimer t(E, K_GATHER);
-      launch_gather_operands(ent, E.rel.p, crel, E.score_fn == SCORE_DISTMULT ? 2 : 1, (int)SB, (int)R, E.Dp,
+      launch_gather_operands(ent, E.rel.p, crel, rel_mode_of(E), E.D / 2, (int)SB, (int)R, E.Dp,
                              E.opnd.p, E.score_bf16 ? E.opnd16.p : nullptr, st); }
     RowSource dense;
     dense.base = (const char*)E.opnd.p; dense.pitch = (int64_t)E.Dp * 4; dense.etype = ET_F32;
@@ -841,16 +851,17 @@ void run_step(kge_engine& E, int i) {
     aa.one_minus_beta_m = 1.f - E.beta_m; aa.one_minus_beta_v = 1.f - E.beta_v;
     aa.epsilon = E.epsilon; aa.weight_decay = E.weight_decay;
 
-    // both reductions read pre-update rows (DistMult multiplies by them), so they
+    // both reductions read pre-update rows (DistMult and ComplEx multiply by them), so they
     // come before both updates
     ContribSrc rsrc = {};
     rsrc.sorted_item = E.r_sorted_vals + (size_t)i * E.n_rel_items;
     rsrc.grad = E.grad.p;
-    rsrc.transform = E.score_fn == SCORE_DISTMULT ? 2 : 0; rsrc.n_head = (int)SB;
+    rsrc.transform = E.score_fn == SCORE_DISTMULT ? 2 : E.score_fn == SCORE_COMPLEX ? 4 : 0;
+    rsrc.n_head = (int)SB; rsrc.half = E.D / 2;
     rsrc.rel = E.rel.p; rsrc.crel = crel; rsrc.ent = ent;
     ContribSrc esrc = rsrc;
     esrc.sorted_item = E.e_sorted_vals + (size_t)i * 2 * R;
-    esrc.transform = E.score_fn == SCORE_DISTMULT ? 1 : 0;
+    esrc.transform = E.score_fn == SCORE_DISTMULT ? 1 : E.score_fn == SCORE_COMPLEX ? 3 : 0;
 
     ReduceArgs rr = {};
     rr.src = rsrc;
@@ -867,7 +878,7 @@ void run_step(kge_engine& E, int i) {
     re.partial = E.partial.p; re.Dp = E.Dp;
     { KernelTimer t(E, K_REDUCE_ENT); launch_reduce_chunks2(re, rr, st); }
 
-    // With DistMult the relation rows' direct contributions read entity rows and
+    // With DistMult / ComplEx the relation rows' direct contributions read entity rows and
     // the entity rows' read relation rows, so neither table may be updated before
     // the other's gradient is complete: materialise the relation gradient first.
     // (TransE contributions do not depend on either table.)
@@ -898,7 +909,7 @@ void run_step(kge_engine& E, int i) {
     ae.alpha = alpha;
     ae.rows_per_alpha = E.shared_table ? 0u : (uint32_t)E.n_entity;
 
-    if (E.score_fn == SCORE_DISTMULT) {
+    if (E.score_fn != SCORE_TRANSE) {
         // entity update first (reads pre-update relation rows), writing its summed
         // gradient is not needed; then the relation update reads POST-update entity
         // rows unless its gradient was materialised: do that with a zero-step pass
@@ -1098,7 +1109,7 @@ void run_predict(kge_engine& E, const Items& in) {
         return r;
     };
     // predicted tails of all queries: dense rows [0, Qp)
-    launch_gather_operands(rows_of(E.p_idx.p, Qp), E.rel.p, E.p_rel.p, E.score_fn == SCORE_DISTMULT ? 2 : 1, Qp,
+    launch_gather_operands(rows_of(E.p_idx.p, Qp), E.rel.p, E.p_rel.p, rel_mode_of(E), E.D / 2, Qp,
                            Qp, Dp, E.p_opnd.p, nullptr, st);
 
     ScoreShape sh = {};
@@ -1127,7 +1138,7 @@ void run_predict(kge_engine& E, const Items& in) {
             const int live = (int)std::min<int64_t>(chunk, hi - r0);
             uint32_t* tail_idx = E.p_idx.p + Qp;
             launch_row_range((uint32_t)(table_off + r0), live, chunk, tail_idx, st);
-            launch_gather_operands(rows_of(tail_idx, chunk), E.rel.p, nullptr, 0, 0, chunk, Dp,
+            launch_gather_operands(rows_of(tail_idx, chunk), E.rel.p, nullptr, 0, 0, 0, chunk, Dp,
                                    E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
             launch_score_fwd(sh, dense, E.rel.p, nullptr, nullptr, E.p_scores.p, nullptr, nullptr, nullptr,
                              false, st);

@@ -8,7 +8,10 @@
 
 namespace kge {
 
-enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1 };
+// TransE: score = gamma - distance(h + r, t).  DistMult: score = (h * r) . t.  ComplEx: the
+// complex product of h and r on the (real | imaginary) halves of the row, scored by the
+// distance function's value itself (src/poplar_kge.cpp:501-514).
+enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2 };
 enum { DIST_L1 = 0, DIST_L2 = 1, DIST_DOT = 2 };
 enum { LOSS_LOGSIGMOID = 0, LOSS_SOFTMAX = 1 };
 enum { ET_F32 = 0, ET_BF16 = 1, ET_F16 = 2 };
@@ -87,11 +90,12 @@ struct ScoreShape {
 };
 
 // Dense float32 operand matrix [n_rows, Dp] from indexed rows: rows [0, n_head)
-// combined with their relation row (rel_mode 1 add, 2 multiply).
+// combined with their relation row (rel_mode 1 add, 2 multiply, 3 complex product on the
+// halves [0, half) | [half, 2 half) of the row).
 // With `out16` the values are rounded to bfloat16, stored there, and the float32
 // copy holds the same rounded values.
 void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
-                            int n_head, int n_rows, int Dp, float* out, uint16_t* out16,
+                            int half, int n_head, int n_rows, int Dp, float* out, uint16_t* out16,
                             hipStream_t stream);
 
 // Batched bfloat16 product on the matrix cores: C[z] = A[z] . Bt[z]^T, float32 out.
@@ -144,11 +148,12 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
 
 // Where gradient contributions come from.  transform: 0 none; 1 multiply head
 // rows (c < n_head) by rel[crel[c]] (DistMult, entity plan); 2 multiply by the
-// head entity row (DistMult, relation plan).
+// head entity row (DistMult, relation plan); 3 / 4 the same two for ComplEx: the
+// product with the complex conjugate on the halves [0, half) | [half, 2 half).
 struct ContribSrc {
     const uint32_t* sorted_item;  // this step's sorted values
     const float* grad;            // [R, Dp]
-    int transform, n_head;
+    int transform, n_head, half;
     const float* rel;
     const uint32_t* crel;
     RowSource ent;

@@ -420,8 +420,8 @@ void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sort
 // kernels read: rows [0, n_head) = a-operands, the rest = b-operands.
 __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const float* __restrict__ rel,
                                                          const uint32_t* __restrict__ crel,
-                                                         int rel_mode, int n_head, int n_rows, int Dp,
-                                                         float* __restrict__ out,
+                                                         int rel_mode, int half, int n_head, int n_rows,
+                                                         int Dp, float* __restrict__ out,
                                                          uint16_t* __restrict__ out16) {
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -430,7 +430,19 @@ __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const fl
     const float* rrow = (c < n_head && rel_mode) ? rel + (size_t)crel[c] * Dp : nullptr;
     for (int k = lane * 4; k < Dp; k += 256) {
         float4 v = load4(row, k, ent);
-        if (rrow) v = combine_rel(v, rrow, k, rel_mode);
+        if (rrow && rel_mode == 3) {
+            // complex product: column kk pairs with kk +- half (src/poplar_kge.cpp:501-510)
+            float* vv = &v.x;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const int kk = k + x;
+                if (kk >= 2 * half) { vv[x] = 0.f; continue; }
+                const int pp = kk < half ? kk + half : kk - half;
+                const float e2 = load1(row, pp, ent.etype);
+                vv[x] = kk < half ? vv[x] * rrow[kk] - e2 * rrow[pp]    // re = h_re r_re - h_im r_im
+                                  : e2 * rrow[kk] + vv[x] * rrow[pp];   // im = h_re r_im + h_im r_re
+            }
+        } else if (rrow) v = combine_rel(v, rrow, k, rel_mode);
         // + 0 turns a -0 into +0, so that a difference of stored operands is never -0
         // (the paired L1 backward reads the sign off the difference's bit pattern)
         v.x += 0.f; v.y += 0.f; v.z += 0.f; v.w += 0.f;
@@ -449,10 +461,10 @@ __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const fl
 }
 
 void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
-                            int n_head, int n_rows, int Dp, float* out, uint16_t* out16,
+                            int half, int n_head, int n_rows, int Dp, float* out, uint16_t* out16,
                             hipStream_t stream) {
     hipLaunchKernelGGL(k_gather_operands, dim3((n_rows + 3) / 4), dim3(256), 0, stream, ent, rel, crel,
-                       rel_mode, n_head, n_rows, Dp, out, out16);
+                       rel_mode, half, n_head, n_rows, Dp, out, out16);
 }
 
 // --------------------------------------------------------------------------
@@ -620,7 +632,7 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
             const float dist = DIST == DIST_L2 ? sqrtf(acc[i][j]) : acc[i][j];
             distv[j] = dist;
             if (OM == 2) { outv[j] = dist; continue; }
-            const float score = sh.score_fn == SCORE_DISTMULT ? dist : sh.gamma - dist;
+            const float score = sh.score_fn != SCORE_TRANSE ? dist : sh.gamma - dist;
             if (OM == 1) { outv[j] = score; continue; }
             const bool pos = (uint32_t)n == label;
             const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
@@ -630,7 +642,7 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
             if (n < T) loss_acc -= w * lsig;
             // d loss / d score, times the loss scale
             const float ds = -w * sign * dlsig * grad_scale;
-            float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;  // score = gamma - dist
+            float c = sh.score_fn != SCORE_TRANSE ? ds : -ds;  // score = gamma - dist
             if (DIST == DIST_L2) c = dist != 0.f ? c * __builtin_amdgcn_rcpf(dist) : 0.f;
             outv[j] = c;
         }
@@ -1065,7 +1077,7 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
             if (OM == 2) {
                 outv = dist;
             } else {
-                const float score = sh.score_fn == SCORE_DISTMULT ? dist : sh.gamma - dist;
+                const float score = sh.score_fn != SCORE_TRANSE ? dist : sh.gamma - dist;
                 if (OM == 1) {
                     outv = score;
                     if (live && DIST == DIST_L2 && dist_blk) dist_blk[m * T + n] = dist;
@@ -1077,7 +1089,7 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
                     log_sigmoid_both(z, lsig, dlsig);
                     if (live) loss_acc -= w * lsig;
                     const float ds = -w * sign * dlsig * grad_scale;
-                    outv = sh.score_fn == SCORE_DISTMULT ? ds : -ds;
+                    outv = sh.score_fn != SCORE_TRANSE ? ds : -ds;
                     if (DIST == DIST_L2) outv = dist != 0.f ? outv * __builtin_amdgcn_rcpf(dist) : 0.f;
                 }
             }
@@ -1110,7 +1122,7 @@ static bool fwd_uses_mfma(const FwdParams& p) {
 }
 
 int score_fwd_parts(const ScoreShape& sh) {
-    const bool mfma = sh.use_mfma && !(sh.score_fn == SCORE_TRANSE && sh.dist_fn == DIST_L1);
+    const bool mfma = sh.use_mfma && !(sh.score_fn != SCORE_DISTMULT && sh.dist_fn == DIST_L1);
     const int tm = mfma ? FM_TM : kScoreTile, tn = mfma ? FM_TN : kScoreTile;
     return ((sh.T + tn - 1) / tn) * ((sh.B + tm - 1) / tm);
 }
@@ -1383,7 +1395,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
             const float z = s[t] + (pos ? 0.f : corr);
             if (pos) loss = -(z - lse) * inv_norm;
             const float ds = (expf(z - lse) - (pos ? 1.f : 0.f)) * inv_norm * sh.loss_scale;
-            float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;
+            float c = sh.score_fn != SCORE_TRANSE ? ds : -ds;
             if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
             s[t] = c;
             if (s16) s16[t] = f32_to_bf16(c);
@@ -1414,7 +1426,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
             const float sign = pos ? 1.f : -1.f, z = sign * sc;
             loss -= w * log_sigmoid(z) * inv_norm;
             const float ds = -w * sign * log_sigmoid_grad(z) * inv_norm * sh.loss_scale;
-            float c = sh.score_fn == SCORE_DISTMULT ? ds : -ds;
+            float c = sh.score_fn != SCORE_TRANSE ? ds : -ds;
             if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
             s[t] = c;
             if (s16) s16[t] = f32_to_bf16(c);
@@ -1427,7 +1439,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
 void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef, const float* dist,
                       float* loss_part, uint16_t* coef16, hipStream_t stream) {
     const int rows = sh.S * sh.B;
-    const bool l2 = sh.score_fn == SCORE_TRANSE && sh.dist_fn == DIST_L2;
+    const bool l2 = sh.score_fn != SCORE_DISTMULT && sh.dist_fn == DIST_L2;
     hipLaunchKernelGGL(k_loss_rows, dim3((rows + 3) / 4), dim3(256), 0, stream, sh, clabel, coef,
                        l2 ? dist : nullptr, loss_part, coef16);
 }
@@ -2108,7 +2120,7 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
 // the current n_best-th score, by a bitonic sort of the 2048-entry union in LDS.
 // Ties therefore resolve to the lower index, whatever the chunking.
 
-constexpr int TK_BLOCK = 1024, TK_SORT = 2048, TK_MAX_BEST = 1024;
+constexpr int TK_BLOCK = 1024, TK_SORT = 2048;
 
 DEVINL bool topk_before(float sa, uint32_t ia, float sb, uint32_t ib) {
     return sa > sb || (sa == sb && ia < ib);
@@ -2211,7 +2223,27 @@ void launch_row_range(uint32_t base, int n_live, int n, uint32_t* out, hipStream
 // columns from k, with the DistMult product rule applied on load.
 DEVINL float4 load_contrib(const ContribSrc& cs, uint32_t c, int k, int Dp) {
     float4 g = *reinterpret_cast<const float4*>(cs.grad + (size_t)c * Dp + k);
-    if (cs.transform == 1) {
+    if (cs.transform >= 3) {
+        // ComplEx: the predicted tail is the complex product h r, so the head's gradient is
+        // g conj(r) and the relation's g conj(h) (column kk pairs with kk +- half):
+        //   re: g_re o_re + g_im o_im      im: g_im o_re - g_re o_im      (o = r or h)
+        if (c < (uint32_t)cs.n_head) {
+            const float* gr = cs.grad + (size_t)c * Dp;
+            const float* rr = cs.rel + (size_t)cs.crel[c] * Dp;
+            const char* er = row_ptr(cs.ent, c);
+            float* gg = &g.x;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const int kk = k + x;
+                if (kk >= 2 * cs.half) { gg[x] = 0.f; continue; }
+                const int pp = kk < cs.half ? kk + cs.half : kk - cs.half;
+                const float o_k = cs.transform == 3 ? rr[kk] : load1(er, kk, cs.ent.etype);
+                const float o_p = cs.transform == 3 ? rr[pp] : load1(er, pp, cs.ent.etype);
+                const float g_p = gr[pp];
+                gg[x] = kk < cs.half ? gg[x] * o_k + g_p * o_p : gg[x] * o_p - g_p * o_k;
+            }
+        }
+    } else if (cs.transform == 1) {
         if (c < (uint32_t)cs.n_head)
             g = f4mul(g, *reinterpret_cast<const float4*>(cs.rel + (size_t)cs.crel[c] * Dp + k));
     } else if (cs.transform == 2) {

@@ -30,7 +30,7 @@
 
 #define API __attribute__((visibility("default")))
 
-enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1 };
+enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2 };
 enum { DIST_L1 = 0, DIST_L2 = 1, DIST_DOT = 2 };
 enum { LOSS_LOGSIGMOID = 0, LOSS_SOFTMAX = 1 };
 enum { STORE_F32 = 0, STORE_F16 = 1, STORE_BF16_EMB = 2 };
@@ -45,6 +45,7 @@ typedef struct {
     int32_t a2a;            /* A tails sent to each shard; T = S*A              */
     int32_t score_fn;       /* SCORE_*                                          */
     int32_t distance_fn;    /* DIST_* (ignored for DistMult, which is a dot)    */
+                            /* ComplEx: dim even; score = distance_fn's value   */
     int32_t loss_fn;        /* LOSS_*                                           */
     int32_t shared_table;   /* 1: every shard addresses the same n_entity rows  */
     int32_t storage;        /* STORE_*: rounding applied on row write-back      */
@@ -454,6 +455,15 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
         for (int64_t b = 0; b < B; ++b) {
             const REAL* h = hidden + (d * NR + head[d * B + b]) * D;
             const float* r = rel + (int64_t)relation[d * B + b] * D;
+            if (c->score_fn == SCORE_COMPLEX) {
+                /* complExPredict (:501-510): halves are real | imaginary parts, (h_re + i h_im)(r_re + i r_im) */
+                const int64_t H = D / 2;
+                for (int64_t k = 0; k < H; ++k) {
+                    p[b * D + k] = h[k] * (REAL)r[k] - h[k + H] * (REAL)r[k + H];
+                    p[b * D + k + H] = h[k] * (REAL)r[k + H] + h[k + H] * (REAL)r[k];
+                }
+                continue;
+            }
             for (int64_t k = 0; k < D; ++k)
                 p[b * D + k] = c->score_fn == SCORE_TRANSE ? h[k] + (REAL)r[k] : h[k] * (REAL)r[k];
         }
@@ -484,7 +494,9 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                     acc = (REAL)sqrt((double)acc);
                 }
                 dist[b * T + t] = acc;
-                if (c->score_fn == SCORE_DISTMULT)
+                /* distMultScore / complExScore return the distance function's value itself
+                 * (:512-514, :571-573); TransE gamma minus it (:492-499) */
+                if (c->score_fn != SCORE_TRANSE)
                     score[b * T + t] = acc;
                 else
                     score[b * T + t] = (REAL)c->gamma - acc;
@@ -510,7 +522,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                     }
                     continue;
                 }
-                g = -g; /* score = gamma - distance (pag.cpp sub: :323-345) */
+                if (c->score_fn == SCORE_TRANSE) g = -g; /* score = gamma - distance (pag.cpp sub: :323-345) */
                 if (dot) {
                     for (int64_t k = 0; k < D; ++k) {
                         gx[k] += g * y[k];
@@ -538,6 +550,19 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             REAL* gh = ghid + (d * NR + head[d * B + b]) * D;
             const REAL* h = hidden + (d * NR + head[d * B + b]) * D;
             const int64_t r = relation[d * B + b];
+            if (c->score_fn == SCORE_COMPLEX) {
+                /* p_re = h_re r_re - h_im r_im, p_im = h_re r_im + h_im r_re */
+                const int64_t H = D / 2;
+                for (int64_t k = 0; k < H; ++k) {
+                    const REAL gre = dp[b * D + k], gim = dp[b * D + k + H];
+                    const REAL rre = rel[r * D + k], rim = rel[r * D + k + H];
+                    gh[k] += gre * rre + gim * rim;
+                    gh[k + H] += gim * rre - gre * rim;
+                    grel[r * D + k] += gre * h[k] + gim * h[k + H];
+                    grel[r * D + k + H] += gim * h[k] - gre * h[k + H];
+                }
+                continue;
+            }
             for (int64_t k = 0; k < D; ++k) {
                 if (c->score_fn == SCORE_TRANSE) {
                     gh[k] += dp[b * D + k];

@@ -14,7 +14,7 @@ import numpy as np
 
 HERE = Path(__file__).resolve().parent
 
-SCORE = {"TransE": 0, "DistMult": 1}
+SCORE = {"TransE": 0, "DistMult": 1, "ComplEx": 2}
 DIST = {"L1": 0, "L2": 1, "MatMul": 2}
 LOSS = {"logsigmoid": 0, "softmax": 1}
 STORE = {"float32": 0, "float16": 1, "bfloat16_embedding": 2}
@@ -267,14 +267,20 @@ def predict_reference(cfg, state, queries, shard_to_count, n_best):
     q = np.asarray(queries, np.int64)
     h = hidden[q[:, 0] * NE + q[:, 1]]
     dot = cfg.score_fn == SCORE["DistMult"] or cfg.distance_fn == DIST["MatMul"]
-    p = h * rel[q[:, 2]] if cfg.score_fn == SCORE["DistMult"] else h + rel[q[:, 2]]
+    r = rel[q[:, 2]]
+    if cfg.score_fn == SCORE["ComplEx"]:  # src/poplar_kge.cpp:501-510
+        H = D // 2
+        p = np.concatenate([h[:, :H] * r[:, :H] - h[:, H:] * r[:, H:],
+                            h[:, :H] * r[:, H:] + h[:, H:] * r[:, :H]], axis=1)
+    else:
+        p = h * r if cfg.score_fn == SCORE["DistMult"] else h + r
     if dot:
         dist = p @ hidden.T
     elif cfg.distance_fn == DIST["L1"]:
         dist = np.stack([np.abs(x[None, :] - hidden).sum(-1) for x in p])
     else:
         dist = np.stack([np.sqrt(((x[None, :] - hidden) ** 2).sum(-1)) for x in p])
-    score = dist if cfg.score_fn == SCORE["DistMult"] else cfg.gamma - dist
+    score = cfg.gamma - dist if cfg.score_fn == SCORE["TransE"] else dist
     live = np.zeros((S, NE), bool)
     for s, n in enumerate(shard_to_count):
         live[s, 1:1 + int(n)] = True

@@ -52,6 +52,20 @@ CASES = {
                            n_entity=4000, n_relation=8, gamma=6.0, shared_table=True),
     "bf16_embedding_l2": dict(distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
                               n_entity=3000, n_relation=8, gamma=6.0, storage="bfloat16_embedding"),
+    # ComplEx (src/poplar_kge.cpp:501-514): complex product of head and relation on the row's
+    # halves, scored by the distance function's value itself
+    "complex_matmul_softmax": dict(score_fn="ComplEx", distance_fn="MatMul", loss_fn="softmax",
+                                   softmax_correction_weight=1.0, feature=0),
+    "complex_matmul_feat": dict(score_fn="ComplEx", distance_fn="MatMul", feature=4),
+    "complex_l2": dict(score_fn="ComplEx", distance_fn="L2", feature=0),
+    "complex_l1": dict(score_fn="ComplEx", distance_fn="L1", feature=0),
+    "complex_odd_half": dict(score_fn="ComplEx", distance_fn="MatMul", dim=10, feature=0, n_entity=41,
+                             batch=5, a2a=3),
+    "aligned_complex": dict(score_fn="ComplEx", distance_fn="MatMul", loss_fn="softmax",
+                            softmax_correction_weight=1.0, n_shard=2, batch=128, a2a=64, dim=64,
+                            feature=0, n_entity=3000, n_relation=8),
+    "aligned_complex_l2_shared": dict(score_fn="ComplEx", distance_fn="L2", n_shard=4, batch=128, a2a=32,
+                                      dim=128, feature=0, n_entity=2000, n_relation=8, shared_table=True),
 }
 
 

@@ -290,6 +290,13 @@ STEP_CASES = {
     "l2_weight_decay": dict(distance_fn="L2", weight_decay=0.01, feature=0),
     "shared_table_l2": dict(distance_fn="L2", shared_table=True, n_shard=4, batch=8, a2a=4,
                             feature=0, n_entity=60, gamma=3.0),
+    # ComplEx (src/poplar_kge.cpp:501-514): complex product of head and relation on the
+    # (real | imaginary) halves, scored by the distance function's value itself
+    "complex_matmul_softmax": dict(score_fn="ComplEx", distance_fn="MatMul", loss_fn="softmax",
+                                   softmax_correction_weight=1.0, feature=0),
+    "complex_matmul_logsigmoid_feat": dict(score_fn="ComplEx", distance_fn="MatMul", feature=4),
+    "complex_l2": dict(score_fn="ComplEx", distance_fn="L2", feature=0),
+    "complex_l1": dict(score_fn="ComplEx", distance_fn="L1", feature=0),
     # bfloat16 scoring operands (this build's option): rounding placement and the
     # straight-through gradient against autograd
     "distmult_bf16_scoring_feat": dict(score_fn="DistMult", distance_fn="MatMul", loss_fn="softmax",
@@ -328,6 +335,25 @@ def _run_case(orc, kw, batch_fn, n_step=3, pad=0, lr=(0.1, 0.07)):
 @pytest.mark.parametrize("name", list(STEP_CASES))
 def test_train_step_vs_autograd(orc, name):
     _run_case(orc, STEP_CASES[name], K.random_batch)
+
+
+def test_complex_score_is_real_part_of_hermitian_product(orc):
+    """ComplEx with the dot product scores Re(<h r, conj t>): checked against numpy's complex
+    arithmetic through the loss of a one-positive, two-tail step (softmax cross entropy of
+    the two scores, closed form)."""
+    c = K.cfg_dict(score_fn="ComplEx", distance_fn="MatMul", loss_fn="softmax", feature=0, n_shard=1,
+                   batch=1, a2a=2, dim=6, n_entity=5, n_relation=2)
+    rng = np.random.default_rng(5)
+    st = K.make_state(c, rng)
+    batch = dict(remote=np.array([[[1, 2, 3]]], np.uint32), a2a=np.array([[[[1, 2]]]], np.uint32),
+                 head=np.array([[[0]]], np.uint32), relation=np.array([[[1]]], np.uint32),
+                 tail=np.array([[[1]]], np.uint32))
+    e, r = st["entity_data"][:, :6].astype(np.float64), st["relation_embedding"][1].astype(np.float64)
+    z = lambda v: v[:3] + 1j * v[3:]  # noqa: E731
+    scores = np.array([np.real(np.sum(z(e[1]) * z(r) * np.conj(z(e[t])))) for t in (2, 3)])
+    want = -(scores[1] - np.log(np.exp(scores).sum()))
+    got = orc.train_step_loop(make_cfg(**c), K.copy_state(st), 0.01, batch)
+    np.testing.assert_allclose(got, [want], rtol=2e-6 if orc.precision == "f64" else 1e-5)
 
 
 def test_train_step_padding_rows(orc):

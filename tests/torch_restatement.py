@@ -80,8 +80,12 @@ def step(cfg, state, lr, batch_step):
     tails = hidden[shards[:, None, None], a2a]  # [S(src), S(dst), A, D]
     tails = tails.transpose(0, 1).reshape(S, Tn, D)  # all-to-all
     r = rel[relation]
-    if cfg["score_fn"] == "TransE":
-        pred = heads + r
+    if cfg["score_fn"] in ("TransE", "ComplEx"):
+        if cfg["score_fn"] == "ComplEx":  # complex product on (real | imaginary) halves
+            hc = T.complex(heads[..., :D // 2], heads[..., D // 2:]) * T.complex(r[..., :D // 2], r[..., D // 2:])
+            pred = T.cat([hc.real, hc.imag], -1)
+        else:
+            pred = heads + r
         if cfg["distance_fn"] == "L1":
             dist = (pred[:, :, None, :] - tails[:, None, :, :]).abs().sum(-1)
         elif cfg["distance_fn"] == "L2":
@@ -92,7 +96,7 @@ def step(cfg, state, lr, batch_step):
             dist = T.where(sq > 0, T.sqrt(safe), T.zeros_like(sq))
         else:
             dist = pred @ tails.transpose(1, 2)
-        score = cfg["gamma"] - dist
+        score = cfg["gamma"] - dist if cfg["score_fn"] == "TransE" else dist
     else:
         pred = heads * r
         if cfg.get("scoring_bf16"):
