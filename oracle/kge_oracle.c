@@ -16,7 +16,12 @@
  * against the reference's own inline known-answer vectors
  * (tests/pag/testPag.cpp, tests/fructose/testFructose.cpp,
  * tests/testPoplarKge.cpp), against torch autograd / closed forms, and the
- * whole step against an independent torch-autograd restatement.
+ * whole step against an independent torch-autograd restatement (every score
+ * function incl. ComplEx, whose restatement there is torch.complex arithmetic,
+ * plus a closed-form Re<h r, conj t> check in numpy).  The one option that is
+ * not the reference's, cfg.scoring_bf16 (operands of the scoring and projection
+ * products rounded to bfloat16, float32 accumulation), is pinned the same way
+ * with a straight-through rounding in the autograd restatement.
  * "parity unpinned": none of the functions in this file.
  */
 #include <math.h>
