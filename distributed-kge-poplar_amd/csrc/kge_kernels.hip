@@ -1202,12 +1202,17 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     const TileId tile = xcd_tile(g.N / GB_T, g.M / GB_T, g.batches * g.ksplit);
     const int zb = tile.z / g.ksplit, zs = tile.z - zb * g.ksplit;
     const int m0 = tile.y * GB_T, n0 = tile.x * GB_T;
-    const int K = g.K / g.ksplit;
+    if (g.m_limit && (uint32_t)m0 >= *g.m_limit) return;
+    int K = g.K / g.ksplit;
+    if (g.k_limit) {  // this split's share of the live columns, in whole slabs
+        const int live = (int)((*g.k_limit + GB_K - 1) / GB_K) * GB_K;
+        K = max(0, min(K, live - zs * K));
+    }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
     const int hl = lane >> 5, cl = lane & 31;
-    const uint16_t* A = g.A + (size_t)zb * g.a_batch + (size_t)m0 * g.lda + (size_t)zs * K;
-    const uint16_t* Bt = g.Bt + (size_t)zb * g.b_batch + (size_t)n0 * g.ldb + (size_t)zs * K;
+    const uint16_t* A = g.A + (size_t)zb * g.a_batch + (size_t)m0 * g.lda + (size_t)zs * (g.K / g.ksplit);
+    const uint16_t* Bt = g.Bt + (size_t)zb * g.b_batch + (size_t)n0 * g.ldb + (size_t)zs * (g.K / g.ksplit);
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -1227,7 +1232,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
             breg[h] = *reinterpret_cast<const floatx4*>(Bt + (size_t)row * g.ldb + k0 + col);
         }
     };
-    prefetch(0);
+    if (K > 0) prefetch(0);
     for (int k0 = 0; k0 < K; k0 += GB_K) {
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
@@ -1264,20 +1269,45 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32
     float* C = g.ksplit > 1 ? g.part + ((size_t)zb * g.ksplit + zs) * ((size_t)g.M * g.ldc)
                             : g.C + (size_t)zb * g.c_batch;
+    float* __restrict__ const Cr = C;
+    if (g.add_base) {
+        // the added rows: all row ids first, then all values, then the stores, so that the
+        // loads of one 32-row half are in flight together (in the natural order every row's
+        // value waits for its id, 32 round trips one after the other)
+        const char* __restrict__ const ab = g.add_base;
+        const uint32_t* __restrict__ const ai = g.add_index;
+        const uint32_t cnt = *g.add_count;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            uint32_t add_row[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm + 32 * i + 8 * (r >> 2) + 4 * hl + (r & 3);
+                add_row[r] = (uint32_t)m < cnt ? ai[m] : 0u;
+            }
+            float addv[16][2];
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    addv[r][j] = load1(ab + (int64_t)add_row[r] * g.add_pitch, n0 + wn + 32 * j + cl, g.add_etype);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm + 32 * i + 8 * (r >> 2) + 4 * hl + (r & 3);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    Cr[(size_t)m * g.ldc + n0 + wn + 32 * j + cl] = acc[i][j][r] + addv[r][j];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int m = m0 + wm + 32 * i + 8 * (r >> 2) + 4 * hl + (r & 3);
-            uint32_t add_row = 0;
-            if (g.add_base) add_row = (uint32_t)m < *g.add_count ? g.add_index[m] : 0u;
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int n = n0 + wn + 32 * j + cl;
-                float o = acc[i][j][r];
-                if (g.add_base) o += load1(g.add_base + (int64_t)add_row * g.add_pitch, n, g.add_etype);
-                C[(size_t)m * g.ldc + n] = o;
-            }
+            for (int j = 0; j < 2; ++j) Cr[(size_t)m * g.ldc + n0 + wn + 32 * j + cl] = acc[i][j][r];
         }
 }
 
@@ -1323,10 +1353,12 @@ void launch_gemm_nt_bf16(const GemmNT& g0, hipStream_t stream) {
 __global__ __launch_bounds__(256) void k_transpose_bf16(const void* __restrict__ in, int in_f32,
                                                         int rows, int cols, int64_t ld_in,
                                                         int64_t in_batch, uint16_t* __restrict__ out_t,
-                                                        uint16_t* __restrict__ out) {
+                                                        uint16_t* __restrict__ out,
+                                                        const uint32_t* __restrict__ row_limit) {
     // pitch of 66 elements: a column walk (the transposed read) steps 33 banks per row
     __shared__ __attribute__((aligned(4))) uint16_t tile[64][66];
     const int z = blockIdx.z, r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    if (row_limit && (uint32_t)r0 >= *row_limit) return;
     const int q = (threadIdx.x & 15) * 4, lr = threadIdx.x >> 4;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -1356,9 +1388,10 @@ __global__ __launch_bounds__(256) void k_transpose_bf16(const void* __restrict__
 }
 
 void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, int cols, int64_t ld_in,
-                           int64_t in_batch, uint16_t* out_t, uint16_t* out, hipStream_t stream) {
+                           int64_t in_batch, uint16_t* out_t, uint16_t* out, hipStream_t stream,
+                           const uint32_t* row_limit) {
     hipLaunchKernelGGL(k_transpose_bf16, dim3(cols / 64, rows / 64, batches), dim3(256), 0, stream, in,
-                       in_f32 ? 1 : 0, rows, cols, ld_in, in_batch, out_t, out);
+                       in_f32 ? 1 : 0, rows, cols, ld_in, in_batch, out_t, out, row_limit);
 }
 
 // --------------------------------------------------------------------------
@@ -2538,6 +2571,7 @@ void launch_hidden_fwd(const FeatureArgs& a, float* hidden, hipStream_t stream) 
         g.M = a.max_rows; g.N = a.Dp; g.K = a.Fp; g.batches = 1;
         g.add_base = a.emb_base; g.add_pitch = a.pitch; g.add_etype = a.emb_etype;
         g.add_index = a.uniq_key; g.add_count = a.counts;
+        g.m_limit = a.counts;  // rows past the distinct count are never read
         launch_gemm_nt_bf16(g, stream);
         return;
     }
@@ -2602,12 +2636,15 @@ void launch_proj_grad(const FeatureArgs& a, const float* grad_rows, float* gproj
     if (feature_bf16_ok(a)) {
         // gproj [Fp, Dp] = features^T [Fp, U] . grad_rows [U, Dp]: A = features^T, Bt = grad_rows^T;
         // rows past the distinct count are zero in the features and finite in grad_rows
-        launch_transpose_bf16(a.feat16, false, 1, a.max_rows, a.Fp, a.Fp, 0, a.featT16, nullptr, stream);
-        launch_transpose_bf16(grad_rows, true, 1, a.max_rows, a.Dp, a.Dp, 0, a.gT16, nullptr, stream);
+        // (the contraction stops at the distinct count, so neither those rows nor their
+        // transposes are touched)
+        launch_transpose_bf16(a.feat16, false, 1, a.max_rows, a.Fp, a.Fp, 0, a.featT16, nullptr, stream, a.counts);
+        launch_transpose_bf16(grad_rows, true, 1, a.max_rows, a.Dp, a.Dp, 0, a.gT16, nullptr, stream, a.counts);
         GemmNT g = {};
         g.A = a.featT16; g.lda = a.max_rows; g.Bt = a.gT16; g.ldb = a.max_rows; g.C = gproj; g.ldc = a.Dp;
         g.M = a.Fp; g.N = a.Dp; g.K = a.max_rows; g.batches = 1;
         g.part = a.gproj_part;  // [16, Fp, Dp]: room for every split
+        g.k_limit = a.counts;
         launch_gemm_nt_bf16(g, stream);
         return;
     }
