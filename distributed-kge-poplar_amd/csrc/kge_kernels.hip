@@ -1413,7 +1413,62 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
     const float* dr = dist ? dist + (size_t)row * T : nullptr;
     const uint32_t label = clabel[row];
     float loss = 0.f;
-    if (sh.loss_fn == LOSS_SOFTMAX) {
+    if (sh.loss_fn == LOSS_SOFTMAX && (T & 3) == 0 && T <= 2048) {
+        // the row stays in registers (up to eight float4 per lane): one read, one write
+        const float corr = sh.softmax_correction;
+        constexpr int NV = 8;
+        floatx4 z[NV];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int t = 4 * lane + 256 * i;
+            if (t < T) {
+                z[i] = *reinterpret_cast<const floatx4*>(s + t);
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    z[i][x] += (uint32_t)(t + x) == label ? 0.f : corr;
+                    mx = fmaxf(mx, z[i][x]);
+                }
+            }
+        }
+        mx = wave_max(mx);
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (4 * lane + 256 * i < T)
+#pragma unroll
+                for (int x = 0; x < 4; ++x) sum += __expf(z[i][x] - mx);
+        sum = wave_sum(sum);
+        const float lse = mx + logf(sum);
+        const float inv_norm = 1.f / ((float)sh.S * (float)sh.B);
+        const float gs = inv_norm * sh.loss_scale;
+        const float sgn = sh.score_fn != SCORE_TRANSE ? 1.f : -1.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int t = 4 * lane + 256 * i;
+            if (t < T) {
+                floatx4 c;
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const bool pos = (uint32_t)(t + x) == label;
+                    if (pos) loss = -(z[i][x] - lse) * inv_norm;
+                    c[x] = sgn * (__expf(z[i][x] - lse) - (pos ? 1.f : 0.f)) * gs;
+                }
+                if (dr) {
+                    const floatx4 dv = *reinterpret_cast<const floatx4*>(dr + t);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) c[x] = dv[x] != 0.f ? c[x] / dv[x] : 0.f;
+                }
+                *reinterpret_cast<floatx4*>(s + t) = c;
+                if (s16) {
+                    uint2 raw;
+                    raw.x = (uint32_t)f32_to_bf16(c.x) | ((uint32_t)f32_to_bf16(c.y) << 16);
+                    raw.y = (uint32_t)f32_to_bf16(c.z) | ((uint32_t)f32_to_bf16(c.w) << 16);
+                    *reinterpret_cast<uint2*>(s16 + t) = raw;
+                }
+            }
+        }
+    } else if (sh.loss_fn == LOSS_SOFTMAX) {
         const float corr = sh.softmax_correction;
         float mx = -INFINITY;
         for (int t = lane; t < T; t += 64) mx = fmaxf(mx, s[t] + ((uint32_t)t == label ? 0.f : corr));
