@@ -2015,6 +2015,34 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
         }
         __syncthreads();
     }
+    float* __restrict__ const gout = p.grad;
+    if (DIST == DIST_DOT && p.add_base) {
+        // added rows: all row ids, then all values, then the stores, so that a tile's loads are
+        // in flight together instead of sixteen dependent round trips one after the other
+        const char* __restrict__ const ab = p.add_base;
+        const uint32_t* __restrict__ const ai = p.add_index;
+        const uint32_t cnt = *p.add_count;
+#pragma unroll
+        for (int t = 0; t < AT; ++t) {
+            uint32_t row[16];
+            float addv[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = i0 + wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                row[r] = ((ALIGNED || i < n_self) && (uint32_t)i < cnt) ? ai[i] : 0u;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                addv[r] = (ALIGNED || kcol < Dp) ? load1(ab + (int64_t)row[r] * p.add_pitch, kcol, p.add_etype) : 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = i0 + wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (!ALIGNED && (i >= n_self || kcol >= Dp)) continue;
+                gout[(size_t)(grad_c0 + d * n_self + i) * Dp + kcol] = acc[t][r] + addv[r];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int t = 0; t < AT; ++t)
 #pragma unroll
@@ -2024,11 +2052,7 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
             if (!ALIGNED && (i >= n_self || kcol >= Dp)) continue;
             float o = acc[t][r];
             if (DIST == DIST_L2) o = sv[t][r] * csum_s[i_loc] - o;
-            if (DIST == DIST_DOT && p.add_base) {
-                const uint32_t row = (uint32_t)i < *p.add_count ? p.add_index[i] : 0u;
-                o += load1(p.add_base + (int64_t)row * p.add_pitch, kcol, p.add_etype);
-            }
-            p.grad[(size_t)(grad_c0 + d * n_self + i) * Dp + kcol] = o;
+            gout[(size_t)(grad_c0 + d * n_self + i) * Dp + kcol] = o;
         }
 }
 
