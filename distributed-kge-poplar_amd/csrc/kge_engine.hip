@@ -228,6 +228,10 @@ struct kge_engine {
     DevBuf<uint32_t> p_idx, p_rel, p_count, p_best_i;
     DevBuf<float> p_opnd, p_scores, p_best_s, p_hidden, p_featd;
     DevBuf<uint16_t> opnd16, opndT16, coef16, coefT16, feat16, featT16, projT16, gT16;  // bfloat16 scoring operands
+    // norm regularisers (src/poplar_kge.cpp:430-437): per distinct row gradients and loss shares
+    float reg_p[3] = {3.f, 3.f, 3.f}, reg_w[3] = {0.f, 0.f, 0.f};
+    bool reg_on = false;
+    DevBuf<float> reg_val, reg_fh, reg_loss_row, reg_loss_part;
     DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, d_loss, d_alpha;
     std::vector<float> h_alpha;  // [n_step][entity, relation, projection][S]
     int n_part;
@@ -282,12 +286,12 @@ void parse_settings(kge_engine& E, const Items& s) {
     E.A = (int)s.uint("data.a2a_size");
     E.neg_adv = s.flt("model.negative_adversarial_scale");
     const std::string loss = s.str("training.loss.type");
-    float reg_w[3];
     const char* reg_names[3] = {"training.embedding_regularisation", "training.feature_regularisation",
                                 "training.hidden_regularisation"};
     for (int i = 0; i < 3; ++i) {
-        (void)s.flt(std::string(reg_names[i]) + ".power");
-        reg_w[i] = s.flt(std::string(reg_names[i]) + ".weight");
+        E.reg_p[i] = s.flt(std::string(reg_names[i]) + ".power");
+        E.reg_w[i] = s.flt(std::string(reg_names[i]) + ".weight");
+        if (E.reg_w[i] > 0) E.reg_on = true;
     }
     E.softmax_cw = loss == "softmax" ? s.flt("training.loss.correction_weight") : 0.f;
     E.loss_scale = s.flt("training.loss_scale");
@@ -317,6 +321,9 @@ void parse_settings(kge_engine& E, const Items& s) {
     parse_et("execution.embedding_dtype", emb_et);
     parse_et("execution.feature_dtype", feat_et);
     E.shared_table = s.find("execution.shared_table") ? s.boolean("execution.shared_table") : false;
+    if (E.reg_on && E.shared_table)
+        throw std::invalid_argument("norm regularisers (weight > 0) need private shard tables: with "
+                                    "'execution.shared_table' a row's loss share has no owning shard");
     E.profile_kernels = s.find("execution.profile_kernels") ? s.boolean("execution.profile_kernels") : false;
     if (s.find("execution.reduce_chunk")) E.chunk = (int)s.uint("execution.reduce_chunk");
     if (s.find("execution.scoring")) {
@@ -367,8 +374,8 @@ void parse_settings(kge_engine& E, const Items& s) {
     if (!share && E.F > 0)
         throw std::invalid_argument("'model.share_feature_networks' = false is not implemented on the HIP device");
     for (int i = 0; i < 3; ++i)
-        if (reg_w[i] > 0)
-            throw std::invalid_argument(std::string("'") + reg_names[i] + ".weight' > 0 is not implemented on the HIP device");
+        if (E.reg_w[i] > 0 && !(E.reg_p[i] > 0))
+            throw std::invalid_argument(std::string("'") + reg_names[i] + ".power' must be positive");
     if (E.S < 1 || E.B < 1 || E.A < 1 || E.D < 1 || E.n_entity < 1 || E.n_rel < 1 || E.n_step < 1 || E.rw_batch < 1)
         throw std::invalid_argument("sizes must be positive");
     if (E.S * E.A < 2) throw std::invalid_argument("n_shard * a2a_size must be at least 2");
@@ -516,6 +523,12 @@ void allocate(kge_engine& E) {
     if (E.use_mfma && E.dist_fn == DIST_L2) {
         E.nearflag.alloc(nearflag_words(sh));
         E.nearflag.zero(st);
+    }
+    if (E.reg_on) {
+        E.reg_val.alloc(R * E.Dp);
+        if (E.F) E.reg_fh.alloc(R * E.Dp);
+        E.reg_loss_row.alloc(R);
+        E.reg_loss_part.alloc(ns * S);
     }
     E.loss_part.alloc(ns * S * E.n_part);
     E.d_loss.alloc(S);
@@ -844,6 +857,22 @@ void run_step(kge_engine& E, int i) {
         { KernelTimer t(E, K_BWD); launch_score_bwd(sh, dense, E.rel.p, crel, E.coef.p, E.nearflag.p, E.grad.p, st); }
     }
 
+    if (E.reg_on) {
+        RegArgs ra = {};
+        ra.uniq_key = e_uniq; ra.counts = e_counts; ra.max_rows = (int)R;
+        ra.seg_start = E.e_seg.p + (size_t)i * (E.e_ustride + 1);
+        ra.seg_real = E.e_real.p + (size_t)i * E.e_ustride;
+        ra.emb_base = E.table.p; ra.pitch = E.L.pitch; ra.emb_etype = E.L.emb_etype;
+        ra.hidden = E.F ? E.hidden.p : nullptr;
+        ra.D = E.D; ra.Dp = E.Dp;
+        for (int q = 0; q < 3; ++q) { ra.power[q] = E.reg_p[q]; ra.weight[q] = E.reg_w[q]; }
+        ra.loss_scale = E.loss_scale;
+        ra.add_val = E.reg_val.p; ra.add_fh = E.reg_fh.p; ra.loss_row = E.reg_loss_row.p;
+        launch_reg_rows(ra, st);
+        launch_reg_loss(e_uniq, e_counts, E.reg_loss_row.p, (uint32_t)E.n_entity, E.S,
+                        E.reg_loss_part.p + (size_t)i * E.S, st);
+    }
+
     const float* alpha = E.d_alpha.p + (size_t)i * 3 * E.S;
     AdamArgs aa = {};
     aa.Dp = E.Dp;
@@ -904,6 +933,7 @@ void run_step(kge_engine& E, int i) {
     ae.counts = e_counts; ae.max_rows = (int)R;
     ae.partial = E.partial.p;
     ae.grad_out = E.F ? E.gsum.p : nullptr;
+    if (E.reg_on) { ae.grad_add = E.reg_val.p; ae.grad_out_add = E.reg_fh.p; }
     ae.p_base = E.table.p; ae.m_base = E.table.p + E.L.off_m; ae.v_base = E.table.p + E.L.off_s;
     ae.pitch = E.L.pitch; ae.p_etype = E.L.emb_etype; ae.m_etype = E.L.mom_etype; ae.v_is_sqrt = 1;
     ae.alpha = alpha;
@@ -988,7 +1018,7 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     HIP_CHECK(hipEventRecord(E.ev[2], st));
     for (int i = s0; i < s0 + sn; ++i) run_step(E, i);
     launch_loss_finalize(E.loss_part.p + (size_t)s0 * E.S * E.n_part, sn, E.S, E.n_part, 1.f / (float)sn,
-                         E.d_loss.p, st);
+                         E.d_loss.p, st, E.reg_on ? E.reg_loss_part.p + (size_t)s0 * E.S : nullptr);
     HIP_CHECK(hipGetLastError());
     HIP_CHECK(hipEventRecord(E.ev[3], st));
     HIP_CHECK(hipMemcpyAsync(loss, E.d_loss.p, S * 4, hipMemcpyDeviceToHost, st));

@@ -205,13 +205,40 @@ struct AdamArgs {
     const float* alpha;        // [n_alpha] step sizes
     uint32_t rows_per_alpha;   // alpha index = key / rows_per_alpha (0: always alpha[0])
     float beta_m, beta_v, one_minus_beta_m, one_minus_beta_v, epsilon, weight_decay;
+    // norm regularisers (launch_reg_rows), or null: added to the row's gradient before the
+    // update / to what grad_out receives
+    const float* grad_add;      // [rows, Dp]
+    const float* grad_out_add;  // [rows, Dp]
 };
 void launch_adam_rows(const AdamArgs& a, hipStream_t stream);
 void launch_adam_rows2(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream);  // one launch
 
-// loss[s] = sum over steps and parts of loss_part / n_step, in a fixed order.
+// loss[s] = sum over steps and parts of loss_part / n_step, in a fixed order; `extra`
+// (or null) holds one more term per (step, shard).
 void launch_loss_finalize(const float* loss_part, int n_step, int S, int n_part, float scale,
-                          float* loss, hipStream_t stream);
+                          float* loss, hipStream_t stream, const float* extra = nullptr);
+
+// Norm regularisers (src/poplar_kge.cpp:430-437, 463-465) on the distinct rows of one step:
+// weight * (sum_k |x_k^power|)^(1/power) of the embedding, of feature . W (hidden - embedding)
+// and of hidden, each counted twice per gathered slot (the reference evaluates them once
+// for the heads and once for the tails, on the same gathered rows).  A row gathered by
+// `mult` slots (segment members that are not gradient contributions) counts mult times.
+struct RegArgs {
+    const uint32_t* uniq_key; const uint32_t* seg_start; const uint32_t* seg_real; const uint32_t* counts;
+    int max_rows;
+    const char* emb_base; int64_t pitch; int emb_etype;
+    const float* hidden;        // [rows, Dp] or null (no features: hidden = embedding)
+    int D, Dp;
+    float power[3], weight[3];  // embedding, feature product, hidden
+    float loss_scale;
+    float* add_val;             // [rows, Dp] gradient for the embedding
+    float* add_fh;              // [rows, Dp] gradient for the feature product (or null)
+    float* loss_row;            // [rows] the row's share of the loss
+};
+void launch_reg_rows(const RegArgs& a, hipStream_t stream);
+// out[s] = sum of loss_row over the distinct rows owned by shard s (key / rows_per_shard), fixed order
+void launch_reg_loss(const uint32_t* uniq_key, const uint32_t* counts, const float* loss_row,
+                     uint32_t rows_per_shard, int S, float* out, hipStream_t stream);
 
 // ---- feature projection (hidden = emb + feature * W) -----------------------
 struct FeatureArgs {

@@ -2512,8 +2512,13 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
                 for (int x = 0; x < 8; ++x) g = f4add(g, t[x]);
             }
         }
-        if (a.grad_out) *reinterpret_cast<float4*>(a.grad_out + (size_t)u * Dp + k) = g;
+        if (a.grad_out) {
+            float4 go = g;
+            if (a.grad_out_add) go = f4add(go, *reinterpret_cast<const float4*>(a.grad_out_add + (size_t)u * Dp + k));
+            *reinterpret_cast<float4*>(a.grad_out + (size_t)u * Dp + k) = go;
+        }
         if (a.no_update) continue;
+        if (a.grad_add) g = f4add(g, *reinterpret_cast<const float4*>(a.grad_add + (size_t)u * Dp + k));
         adam4(p, m, v, g, a, alpha);
         store4(prow, k, a.p_etype, p);
         if constexpr (MF32) {
@@ -2544,7 +2549,8 @@ void launch_adam_rows2(const AdamArgs& a0, const AdamArgs& a1, hipStream_t strea
 
 __global__ __launch_bounds__(64) void k_loss_finalize(const float* __restrict__ loss_part, int n_step,
                                                       int S, int n_part, float scale,
-                                                      float* __restrict__ loss) {
+                                                      float* __restrict__ loss,
+                                                      const float* __restrict__ extra) {
     const int s = blockIdx.x, lane = threadIdx.x;
     float acc = 0.f;
     for (int i = 0; i < n_step; ++i) {
@@ -2552,14 +2558,83 @@ __global__ __launch_bounds__(64) void k_loss_finalize(const float* __restrict__ 
         float part = 0.f;
         for (int t = lane; t < n_part; t += 64) part += p[t];
         acc += wave_sum(part);
+        if (extra) acc += extra[(size_t)i * S + s];
     }
     if (lane == 0) loss[s] = acc * scale;
 }
 
 void launch_loss_finalize(const float* loss_part, int n_step, int S, int n_part, float scale,
-                          float* loss, hipStream_t stream) {
+                          float* loss, hipStream_t stream, const float* extra) {
     hipLaunchKernelGGL(k_loss_finalize, dim3(S), dim3(64), 0, stream, loss_part, n_step, S, n_part,
-                       scale, loss);
+                       scale, loss, extra);
+}
+
+// --------------------------------------------------------------------------
+// norm regularisers: one wave per distinct row, two passes over the row (sums, then gradients)
+
+// |x^p| and its share of the gradient |x^p| / x (0 at x = 0: the reference's pow backward
+// divides by x + (x == 0), src/pag/pag.cpp:483-503)
+DEVINL float abs_pow(float x, float p) { return fabsf(powf(x, p)); }
+
+__global__ __launch_bounds__(256) void k_reg_rows(RegArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (u >= (int)a.counts[0]) return;
+    const uint32_t key = a.uniq_key[u];
+    const float mult = (float)((a.seg_start[u + 1] - a.seg_start[u]) - a.seg_real[u]);
+    const char* erow = a.emb_base + (int64_t)key * a.pitch;
+    const float* hrow = a.hidden ? a.hidden + (size_t)u * a.Dp : nullptr;
+    float sum[3] = {0.f, 0.f, 0.f};
+    for (int k = lane; k < a.D; k += 64) {
+        const float v = load1(erow, k, a.emb_etype), h = hrow ? hrow[k] : v;
+        if (a.weight[0] > 0.f) sum[0] += abs_pow(v, a.power[0]);
+        if (a.weight[1] > 0.f) sum[1] += abs_pow(h - v, a.power[1]);
+        if (a.weight[2] > 0.f) sum[2] += abs_pow(h, a.power[2]);
+    }
+    float norm[3], coef[3], loss = 0.f;
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+        sum[q] = wave_sum(sum[q]);
+        norm[q] = a.weight[q] > 0.f ? powf(sum[q], 1.f / a.power[q]) : 0.f;
+        // d loss / d x_k = seed * (norm / sum) * |x_k^p| / x_k, seed = 2 * mult * weight * loss_scale
+        coef[q] = sum[q] != 0.f ? 2.f * mult * a.weight[q] * a.loss_scale * norm[q] / sum[q] : 0.f;
+        loss += 2.f * mult * a.weight[q] * norm[q];
+    }
+    if (lane == 0) a.loss_row[u] = loss;
+    for (int k = lane; k < a.Dp; k += 64) {
+        float gv = 0.f, gf = 0.f;
+        if (k < a.D) {
+            const float v = load1(erow, k, a.emb_etype), h = hrow ? hrow[k] : v, f = h - v;
+            if (a.weight[0] > 0.f && v != 0.f) gv += coef[0] * abs_pow(v, a.power[0]) / v;
+            if (a.weight[1] > 0.f && f != 0.f) gf += coef[1] * abs_pow(f, a.power[1]) / f;
+            if (a.weight[2] > 0.f && h != 0.f) {
+                const float gh = coef[2] * abs_pow(h, a.power[2]) / h;
+                gv += gh; gf += gh;
+            }
+        }
+        a.add_val[(size_t)u * a.Dp + k] = gv;
+        if (a.add_fh) a.add_fh[(size_t)u * a.Dp + k] = gf;
+    }
+}
+void launch_reg_rows(const RegArgs& a, hipStream_t stream) {
+    hipLaunchKernelGGL(k_reg_rows, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a);
+}
+
+__global__ __launch_bounds__(64) void k_reg_loss(const uint32_t* __restrict__ uniq_key,
+                                                 const uint32_t* __restrict__ counts,
+                                                 const float* __restrict__ loss_row, uint32_t rows_per_shard,
+                                                 float* __restrict__ out) {
+    const int s = blockIdx.x, lane = threadIdx.x;
+    const int U = (int)counts[0];
+    float part = 0.f;
+    for (int u = lane; u < U; u += 64)
+        if (uniq_key[u] / rows_per_shard == (uint32_t)s) part += loss_row[u];
+    part = wave_sum(part);
+    if (lane == 0) out[s] = part;
+}
+void launch_reg_loss(const uint32_t* uniq_key, const uint32_t* counts, const float* loss_row,
+                     uint32_t rows_per_shard, int S, float* out, hipStream_t stream) {
+    hipLaunchKernelGGL(k_reg_loss, dim3(S), dim3(64), 0, stream, uniq_key, counts, loss_row, rows_per_shard, out);
 }
 
 // --------------------------------------------------------------------------

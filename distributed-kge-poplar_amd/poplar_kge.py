@@ -213,7 +213,8 @@ class Settings:
             data=dict(batch_size=512, a2a_size=96, dataset=WikiKg90Mv2Settings()),
             training=dict(n_step=int(5e6), validation_interval=int(2.5e5),
                           loss=SoftmaxLoss(correction_weight=1.0), learning_rate=1e-3,
-                          learning_rate_decay=LinearLearningRateDecay()),
+                          learning_rate_decay=LinearLearningRateDecay(),
+                          feature_regularisation=NormRegularisation(power=3.0, weight=1e-6)),
             execution=dict(device="hip", dtype="float32", feature_dtype="float16",
                            train_steps_per_program_run=20, rw_batch_size=512,
                            predict_hr_batch_size=128, predict_tail_batch_size=1024,

@@ -64,7 +64,28 @@ typedef struct {
     float softmax_correction_weight;
     float negative_adversarial_scale;
     float lr_mod_entity, lr_mod_relation, lr_mod_projection;
+    /* norm regularisers (poplar_kge.cpp:430-437, 463-465): weight * sum over the gathered
+     * rows of (sum_k |x_k^power|)^(1/power), of the embedding, of feature . W and of
+     * their sum; weight 0 = off                                                          */
+    float reg_emb_power, reg_emb_weight, reg_feat_power, reg_feat_weight, reg_hid_power, reg_hid_weight;
 } kge_oracle_cfg;
+
+/* ------------------------------------------------------------------------ */
+/* lpnorm (poplar_kge.cpp:389-391): pow(sum(abs(pow(a, p))), 1/p) of one row, and its
+ * gradient through the reference's pow / abs backward ops (pag.cpp:483-503, 440-459):
+ *   d pow(x, e) = g * e * pow(x, e) / (x + (x == 0))     (0 at x = 0)
+ *   d abs(x)    = g * signum(x)
+ * which multiply out to  g * (n / s) * |a_k^p| / a_k  (0 where a_k = 0 or s = 0).
+ * Adds g * that to grad[0..D) (grad may be NULL) and returns n.                      */
+static REAL lpnorm_row(const REAL* a, int64_t D, float power, REAL g, REAL* grad) {
+    REAL s = 0;
+    for (int64_t k = 0; k < D; ++k) s += (REAL)fabs(pow((double)a[k], (double)power));
+    const REAL n = (REAL)pow((double)s, 1.0 / (double)power);
+    if (grad && s != 0)
+        for (int64_t k = 0; k < D; ++k)
+            if (a[k] != 0) grad[k] += g * (n / s) * (REAL)fabs(pow((double)a[k], (double)power)) / a[k];
+    return n;
+}
 
 /* ------------------------------------------------------------------------ */
 /* storage rounding helpers (write-back cast, poplar_kge.cpp:412-417)        */
@@ -446,6 +467,42 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             }
         }
 
+    /* 1b. norm regularisers over every gathered slot (:463-465).  entityHidden runs once for
+     * the heads and once for the tails on the same gathered rows and (shared networks) the
+     * same projection, so every term counts twice (:676-678).  The embedding's gradient and
+     * the feature product's gradient differ from here on: greg_val / greg_fh.              */
+    const int reg_on = c->reg_emb_weight > 0 || c->reg_feat_weight > 0 || c->reg_hid_weight > 0;
+    REAL* greg_val = reg_on ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
+    REAL* greg_fh = reg_on ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
+    REAL* reg_loss = (REAL*)calloc((size_t)S, sizeof(REAL));
+    if (reg_on) {
+        REAL* fh = (REAL*)malloc(sizeof(REAL) * (size_t)D);
+        REAL* val = (REAL*)malloc(sizeof(REAL) * (size_t)D);
+        for (int64_t s = 0; s < S; ++s)
+            for (int64_t j = 0; j < NR; ++j) {
+                const float* row = table + KEY(s, j) * ROW;
+                const REAL* h = hidden + (s * NR + j) * D;
+                REAL* gv = greg_val + (s * NR + j) * D;
+                REAL* gf = greg_fh + (s * NR + j) * D;
+                for (int64_t k = 0; k < D; ++k) { val[k] = row[k]; fh[k] = h[k] - val[k]; }
+                const REAL seed = 2 * (REAL)c->loss_scale;
+                if (c->reg_emb_weight > 0)
+                    reg_loss[s] += 2 * c->reg_emb_weight *
+                                   lpnorm_row(val, D, c->reg_emb_power, seed * c->reg_emb_weight, gv);
+                if (c->reg_feat_weight > 0)
+                    reg_loss[s] += 2 * c->reg_feat_weight *
+                                   lpnorm_row(fh, D, c->reg_feat_power, seed * c->reg_feat_weight, gf);
+                if (c->reg_hid_weight > 0) {
+                    REAL* tmp = (REAL*)calloc((size_t)D, sizeof(REAL));
+                    reg_loss[s] += 2 * c->reg_hid_weight *
+                                   lpnorm_row(h, D, c->reg_hid_power, seed * c->reg_hid_weight, tmp);
+                    for (int64_t k = 0; k < D; ++k) { gv[k] += tmp[k]; gf[k] += tmp[k]; }
+                    free(tmp);
+                }
+            }
+        free(fh); free(val);
+    }
+
     REAL* grel = (REAL*)calloc((size_t)(NREL * D), sizeof(REAL));
     REAL* p = (REAL*)malloc(sizeof(REAL) * (size_t)(B * D));
     REAL* tl = (REAL*)malloc(sizeof(REAL) * (size_t)(T * D));
@@ -508,7 +565,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             }
 
         /* 4. loss + backward seed = loss_scale (:688-691) */
-        loss_out[d] = (float)shard_loss(c, score, tail + d * B, dscore);
+        loss_out[d] = (float)(shard_loss(c, score, tail + d * B, dscore) + reg_loss[d]);  /* :688 */
         for (int64_t i = 0; i < B * T; ++i) dscore[i] *= (REAL)c->loss_scale;
 
         /* 5. backward through the score into p and tails */
@@ -607,10 +664,11 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             for (int64_t j = 0; j < NR; ++j) {
                 const float* row = table + KEY(s, j) * ROW;
                 const REAL* gh = ghid + (s * NR + j) * D;
+                const REAL* gr = greg_fh ? greg_fh + (s * NR + j) * D : NULL;
                 for (int64_t f = 0; f < F; ++f) {
                     const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
                     if (x != 0)
-                        for (int64_t k = 0; k < D; ++k) gproj[f * D + k] += x * gh[k];
+                        for (int64_t k = 0; k < D; ++k) gproj[f * D + k] += x * (gh[k] + (gr ? gr[k] : 0));
                 }
             }
     }
@@ -632,7 +690,8 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             int64_t j = i;
             for (; j < n && (int64_t)(ks[j] >> 24) == key; ++j) {
                 const REAL* gh = ghid + (int64_t)(ks[j] & 0xffffff) * D;
-                for (int64_t k = 0; k < D; ++k) g[k] += gh[k];
+                const REAL* gr = greg_val ? greg_val + (int64_t)(ks[j] & 0xffffff) * D : NULL;
+                for (int64_t k = 0; k < D; ++k) g[k] += gh[k] + (gr ? gr[k] : 0);
             }
             for (int64_t k = 0; k < D; ++k) gf[k] = (float)g[k];
             float* row = table + key * ROW;
@@ -671,6 +730,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
         free(gf);
     }
 #undef KEY
+    free(greg_val); free(greg_fh); free(reg_loss);
     free(hidden); free(ghid); free(grel); free(p); free(tl); free(score); free(dist);
     free(dscore); free(dp); free(dtl); free(alpha); free(gproj);
     return 0;

@@ -26,21 +26,26 @@ class Cfg(C.Structure):
         "distance_fn", "loss_fn", "shared_table", "storage", "scoring_bf16")] + [(n, C.c_float) for n in (
             "gamma", "beta_m", "beta_v", "epsilon", "weight_decay", "loss_scale",
             "softmax_correction_weight", "negative_adversarial_scale", "lr_mod_entity",
-            "lr_mod_relation", "lr_mod_projection")]
+            "lr_mod_relation", "lr_mod_projection", "reg_emb_power", "reg_emb_weight", "reg_feat_power",
+            "reg_feat_weight", "reg_hid_power", "reg_hid_weight")]
 
 
 def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score_fn="TransE",
              distance_fn="L1", loss_fn="logsigmoid", shared_table=False, storage="float32",
              scoring_bf16=False, gamma=0.0, beta_m=0.9, beta_v=0.999, epsilon=1e-8, weight_decay=0.0,
              loss_scale=None, softmax_correction_weight=0.0, negative_adversarial_scale=0.0,
-             lr_mod_entity=1.0, lr_mod_relation=1.0, lr_mod_projection=1.0):
+             lr_mod_entity=1.0, lr_mod_relation=1.0, lr_mod_projection=1.0,
+             embedding_regularisation=(3.0, 0.0), feature_regularisation=(3.0, 0.0),
+             hidden_regularisation=(3.0, 0.0)):
+    """The three regularisers are (power, weight) pairs (src/python/poplar_kge.py:104-108)."""
     if loss_scale is None:  # src/python/poplar_kge.py:259-262
         loss_scale = float(batch * n_shard * a2a)
     return Cfg(n_shard, n_entity, n_relation, dim, feature, batch, a2a, SCORE[score_fn],
                DIST[distance_fn], LOSS[loss_fn], int(shared_table), STORE[storage], int(scoring_bf16),
                gamma, beta_m,
                beta_v, epsilon, weight_decay, loss_scale, softmax_correction_weight,
-               negative_adversarial_scale, lr_mod_entity, lr_mod_relation, lr_mod_projection)
+               negative_adversarial_scale, lr_mod_entity, lr_mod_relation, lr_mod_projection,
+               *embedding_regularisation, *feature_regularisation, *hidden_regularisation)
 
 
 def build(force=False):

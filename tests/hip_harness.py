@@ -49,12 +49,12 @@ def engine_settings(c, n_step, rw_batch=64, **extra):
         "data.entity_feature_mapping": "full",
         "training.n_step": 100, "training.validation_interval": 50,
         **loss,
-        "training.embedding_regularisation.power": 3.0,
-        "training.embedding_regularisation.weight": 0.0,
-        "training.feature_regularisation.power": 3.0,
-        "training.feature_regularisation.weight": 0.0,
-        "training.hidden_regularisation.power": 3.0,
-        "training.hidden_regularisation.weight": 0.0,
+        "training.embedding_regularisation.power": float(c.get("embedding_regularisation", (3.0, 0.0))[0]),
+        "training.embedding_regularisation.weight": float(c.get("embedding_regularisation", (3.0, 0.0))[1]),
+        "training.feature_regularisation.power": float(c.get("feature_regularisation", (3.0, 0.0))[0]),
+        "training.feature_regularisation.weight": float(c.get("feature_regularisation", (3.0, 0.0))[1]),
+        "training.hidden_regularisation.power": float(c.get("hidden_regularisation", (3.0, 0.0))[0]),
+        "training.hidden_regularisation.weight": float(c.get("hidden_regularisation", (3.0, 0.0))[1]),
         "training.learning_rate": 0.1, "training.learning_rate_modifiers": {},
         "training.adam_beta_m": float(c["beta_m"]), "training.adam_beta_v": float(c["beta_v"]),
         "training.adam_epsilon": float(c["epsilon"]),

@@ -52,6 +52,18 @@ CASES = {
                            n_entity=4000, n_relation=8, gamma=6.0, shared_table=True),
     "bf16_embedding_l2": dict(distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
                               n_entity=3000, n_relation=8, gamma=6.0, storage="bfloat16_embedding"),
+    # norm regularisers (src/poplar_kge.cpp:430-437, 463-465): the WikiKG preset's feature
+    # regulariser, all three with different powers, and without features (hidden = embedding)
+    "feature_regularisation_p3": dict(feature_regularisation=(3.0, 1e-2), loss_fn="softmax",
+                                      softmax_correction_weight=1.0),
+    "all_regularisers_l2": dict(embedding_regularisation=(2.0, 3e-2), feature_regularisation=(3.0, 2e-2),
+                                hidden_regularisation=(4.0, 1e-2), distance_fn="L2"),
+    "regularisers_nofeat": dict(embedding_regularisation=(3.0, 5e-2), feature=0,
+                                hidden_regularisation=(2.0, 1e-2)),
+    "regularisers_distmult_aligned": dict(score_fn="DistMult", distance_fn="MatMul", n_shard=2, batch=128,
+                                          a2a=64, dim=64, feature=8, n_entity=3000, n_relation=8,
+                                          feature_regularisation=(3.0, 1e-3),
+                                          embedding_regularisation=(3.0, 1e-3)),
     # ComplEx (src/poplar_kge.cpp:501-514): complex product of head and relation on the row's
     # halves, scored by the distance function's value itself
     "complex_matmul_softmax": dict(score_fn="ComplEx", distance_fn="MatMul", loss_fn="softmax",
@@ -355,6 +367,21 @@ def test_step_near_duplicate_rows_aligned(oracle64, scoring):
 def test_step_padding_rows(oracle64):
     # zero-padded `remote`: row 0 gathered several times, updated once with g = 0
     run_case(oracle64, dict(feature=0), batch_fn=lambda c, n, r: K.random_batch(c, n, r, pad=4))
+
+
+def test_step_regularisers_with_padding_rows(oracle64):
+    # the padding row (all zeros, gathered by several slots) has norm 0 and, by the reference's
+    # guarded pow backward, zero gradient: no NaN reaches the row or the projection
+    run_case(oracle64, dict(feature_regularisation=(3.0, 1e-2), hidden_regularisation=(3.0, 1e-2)),
+             batch_fn=lambda c, n, r: K.random_batch(c, n, r, pad=4))
+
+
+def test_regularisers_need_private_tables():
+    import libpoplar_kge
+
+    c = K.cfg_dict(feature=0, shared_table=True, n_shard=2, embedding_regularisation=(3.0, 1e-2))
+    with pytest.raises(ValueError, match="private shard tables"):
+        libpoplar_kge.Engine(H.engine_settings(c, 2), "")
 
 
 def test_step_raw_zipf_duplicates(oracle64):

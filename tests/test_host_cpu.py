@@ -74,6 +74,9 @@ def test_settings_tree():
     assert w.model.n_entity == 5701915 and w.model.n_relation_type == 1392
     assert w.flatten()["training.loss.correction_weight"] == 1.0
     assert kge.Settings.create_wikikg90mv2_short().data.a2a_size == 32
+    # the preset's regularisers (reference :377-380)
+    assert (w.training.feature_regularisation.power, w.training.feature_regularisation.weight) == (3.0, 1e-6)
+    assert w.training.embedding_regularisation.weight == 0.0 and w.training.hidden_regularisation.weight == 0.0
 
 
 def _schedule(decay, n):

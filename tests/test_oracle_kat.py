@@ -297,6 +297,13 @@ STEP_CASES = {
     "complex_matmul_logsigmoid_feat": dict(score_fn="ComplEx", distance_fn="MatMul", feature=4),
     "complex_l2": dict(score_fn="ComplEx", distance_fn="L2", feature=0),
     "complex_l1": dict(score_fn="ComplEx", distance_fn="L1", feature=0),
+    # norm regularisers (src/poplar_kge.cpp:430-437, 463-465), the WikiKG preset's among them
+    "feature_regularisation_p3": dict(feature_regularisation=(3.0, 1e-2), loss_fn="softmax",
+                                      softmax_correction_weight=1.0),
+    "all_regularisers": dict(embedding_regularisation=(2.0, 3e-2), feature_regularisation=(3.0, 2e-2),
+                             hidden_regularisation=(4.0, 1e-2), distance_fn="L2"),
+    "embedding_regularisation_nofeat": dict(embedding_regularisation=(3.0, 5e-2), feature=0,
+                                            hidden_regularisation=(2.0, 1e-2)),
     # bfloat16 scoring operands (this build's option): rounding placement and the
     # straight-through gradient against autograd
     "distmult_bf16_scoring_feat": dict(score_fn="DistMult", distance_fn="MatMul", loss_fn="softmax",
@@ -354,6 +361,32 @@ def test_complex_score_is_real_part_of_hermitian_product(orc):
     want = -(scores[1] - np.log(np.exp(scores).sum()))
     got = orc.train_step_loop(make_cfg(**c), K.copy_state(st), 0.01, batch)
     np.testing.assert_allclose(got, [want], rtol=2e-6 if orc.precision == "f64" else 1e-5)
+
+
+def test_lpnorm_closed_forms(orc):
+    """One gathered row, no positives' gradient reaching it: the loss's regularisation part and the
+    row's update follow from the p-norm's closed forms (p = 2: the Euclidean norm, gradient
+    x / |x|; a zero row: norm 0 and, by the reference's guarded pow backward, zero gradient)."""
+    c = K.cfg_dict(feature=0, n_shard=1, batch=1, a2a=2, dim=4, n_entity=6, n_relation=1,
+                   embedding_regularisation=(2.0, 0.5), loss_scale=1.0)
+    rng = np.random.default_rng(2)
+    st = K.make_state(c, rng, warm=False)
+    st["entity_data"][4, :4] = [3.0, 0.0, -4.0, 0.0]       # |x| = 5, not referenced by any slot
+    st["entity_data"][5, :4] = 0.0                          # a zero row
+    batch = dict(remote=np.array([[[1, 4, 5]]], np.uint32), a2a=np.array([[[[0, 0]]]], np.uint32),
+                 head=np.array([[[0]]], np.uint32), relation=np.array([[[0]]], np.uint32),
+                 tail=np.array([[[0]]], np.uint32))
+    plain = dict(c, embedding_regularisation=(2.0, 0.0))
+    st_a, st_b = K.copy_state(st), K.copy_state(st)
+    loss_a = orc.train_step_loop(make_cfg(**c), st_a, 0.1, batch)
+    loss_b = orc.train_step_loop(make_cfg(**plain), st_b, 0.1, batch)
+    norms = np.linalg.norm(st["entity_data"][[1, 4, 5], :4].astype(np.float64), axis=1)
+    np.testing.assert_allclose(loss_a - loss_b, [2 * 0.5 * norms.sum()], rtol=1e-5)
+    # row 4: gradient 2 * 0.5 * x / |x| = (0.6, 0, -0.8, 0): the first Adam step moves each
+    # non-zero element by lr against its sign, zero elements stay
+    d4 = st_a["entity_data"][4, :4] - st["entity_data"][4, :4]
+    np.testing.assert_allclose(d4, [-0.1, 0.0, 0.1, 0.0], rtol=1e-4, atol=1e-9)
+    np.testing.assert_array_equal(st_a["entity_data"][5, :4], 0.0)
 
 
 def test_train_step_padding_rows(orc):

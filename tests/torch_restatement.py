@@ -31,6 +31,31 @@ def log_sigmoid_clamped(x):
     return Fn.apply(x)
 
 
+def safe_pow(x, e):
+    """pow with the reference's backward, g * e * pow(x, e) / (x + (x == 0)), which is 0 at
+    x = 0 where torch's own gives inf or nan (src/pag/pag.cpp:483-503).  Elsewhere the two
+    agree, so torch's autograd still checks the formula."""
+
+    class Fn(T.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            y = T.pow(x, e)
+            ctx.save_for_backward(x, y)
+            return y
+
+        @staticmethod
+        def backward(ctx, g):
+            x, y = ctx.saved_tensors
+            return g * e * y / (x + (x == 0).to(x.dtype))
+
+    return Fn.apply(x)
+
+
+def lpnorm(a, p):
+    """src/poplar_kge.cpp:389-391, per row."""
+    return safe_pow(safe_pow(a, p).abs().sum(-1), 1.0 / p)
+
+
 def round_bf16_ste(x):
     """x rounded to bfloat16 (nearest even) in the forward pass, identity in the
     backward pass: how the bfloat16 scoring mode treats its operands."""
@@ -75,6 +100,15 @@ def step(cfg, state, lr, batch_step):
     else:
         hidden_u = emb
     hidden = hidden_u[inverse].reshape(S, -1, D)  # [S, NR, D]
+    # norm regularisers over every gathered slot, once for the heads' and once for the tails'
+    # entityHidden call (src/poplar_kge.cpp:463-465, 676-678)
+    reg = T.zeros(S, dtype=T.float64)
+    value = emb[inverse].reshape(S, -1, D)
+    for key, tensor in (("embedding_regularisation", value), ("feature_regularisation", hidden - value),
+                        ("hidden_regularisation", hidden)):
+        power, weight = cfg.get(key, (3.0, 0.0))
+        if weight > 0:
+            reg = reg + 2 * weight * lpnorm(tensor, float(power)).sum(-1)
 
     heads = hidden[shards[:, None], head]  # [S, B, D]
     tails = hidden[shards[:, None, None], a2a]  # [S(src), S(dst), A, D]
@@ -118,6 +152,7 @@ def step(cfg, state, lr, batch_step):
         corr = cw * np.float32(np.log(NE * S - 1) - np.log(S * A - 1)) if cw else 0.0
         z = score + float(corr) * (1 - onehot)
         per_shard = -(T.log_softmax(z, -1) * onehot).sum((1, 2)) / (S * B)
+    per_shard = per_shard + reg  # src/poplar_kge.cpp:688
     per_shard.sum().backward(T.tensor(float(cfg["loss_scale"]), dtype=T.float64))
 
     # optimiser (float64 restatement of frnn.cpp:42-90)
