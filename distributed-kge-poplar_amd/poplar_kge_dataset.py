@@ -3,9 +3,10 @@
 Host-side counterpart of the reference's ``src/python/poplar_kge_dataset.py``
 (``RawData`` :17-157, ``unique_pad`` :161-164, ``Dataset`` :171-435): the same
 classes, attributes and array layouts, so that code written against the
-reference's module drives this engine unchanged.  What is not here: the OGB
-loader (``ogb`` is not a dependency; ``RawData.load`` raises for that dataset)
-and the torch ``DataLoader`` wrapper.
+reference's module drives this engine unchanged, ``DatasetWrapper`` (:437-475)
+for a torch ``DataLoader`` with worker processes included.  What is not here:
+the OGB loader (``ogb`` is not a dependency; ``RawData.load`` raises for that
+dataset).
 
 One addition: ``Dataset.sample_batch(deduplicate=False)`` skips the per-shard
 ``np.unique`` and hands the engine raw ids with identity slot maps -- the engine
@@ -243,3 +244,35 @@ class Dataset:
         hit = best == truth[:, None]
         rank = np.where(hit.any(axis=1), hit.argmax(axis=1) + 1, 0)
         return float(np.mean(np.where(rank > 0, 1.0 / np.maximum(rank, 1), 0.0)))
+
+
+class DatasetWrapper:
+    """A map-style dataset of sampled batches for ``torch.utils.data.DataLoader``
+    (reference :437-475): ``DataLoader(DatasetWrapper(ds), batch_size=None, num_workers=10,
+    worker_init_fn=ds.worker_init_fn)`` samples batches in worker processes, each from its
+    own random stream.  torch is only needed by the loader itself, not to define this class."""
+
+    def __init__(self, dataset: Dataset) -> None:
+        self.ds = dataset
+
+    def __len__(self) -> int:
+        return (2 ** 31) - 1
+
+    def __getitem__(self, item: int) -> Dict[str, np.ndarray]:
+        batch = self.ds.sample_batch()
+        return {name: getattr(batch, name).astype(np.int32)
+                for name in ("remote", "a2a", "head", "relation", "tail")}
+
+    @staticmethod
+    def tensors_to_batch(remote, a2a, head, relation, tail) -> "kge.Batch":
+        """What a DataLoader yields (int32 tensors) back as the engine's uint32 arrays."""
+        as_u32 = lambda t: np.ascontiguousarray(t.numpy() if hasattr(t, "numpy") else t).astype(np.uint32)  # noqa: E731
+        return kge.Batch(remote=as_u32(remote), head=as_u32(head), relation=as_u32(relation),
+                         a2a=as_u32(a2a), tail=as_u32(tail))
+
+    @staticmethod
+    def worker_init_fn(worker_id: int) -> None:
+        import torch.utils.data
+
+        unwrapped = torch.utils.data.get_worker_info().dataset.ds
+        unwrapped.random = np.random.RandomState(unwrapped.settings.seed + worker_id)

@@ -240,3 +240,37 @@ def test_training_mrr_matches_brute_force():
             np.testing.assert_allclose(got, want, rtol=1e-4)
             seen.append(want)
     assert max(seen) > 0.05   # the training triples are being learnt: the comparison is not 0 == 0
+
+
+def test_training_script_flow():
+    """The reference's training script (scripts/run_training.py:12-77) step by step, without its
+    logger: settings -> data -> dataset -> engine -> initialise_all -> a torch DataLoader over
+    DatasetWrapper -> train_step_loop per program run, validation MRR and predictions."""
+    import poplar_kge as kge
+    import poplar_kge_dataset as kge_data
+    import torch
+
+    settings = kge.Settings.create_demo()
+    settings.seed = 3
+    settings.prepare()
+    data = kge_data.RawData.load(settings)
+    dataset = kge_data.Dataset.load(data, settings)
+    engine = kge.Engine(settings, dataset.shard_to_count)
+    engine.initialise_all(dataset.entity_features(settings.model.entity_feature_size))
+    ds = kge_data.DatasetWrapper(dataset)
+    dl_iter = iter(torch.utils.data.DataLoader(ds, batch_size=None, num_workers=0,
+                                               worker_init_fn=ds.worker_init_fn))
+    losses = []
+    for n in range(settings.logs_per_training_run):
+        if n % settings.logs_per_validation == 0:
+            for part in ("train", "valid"):
+                assert 0.0 <= dataset.mrr(part, engine.predict) <= 1.0
+        loss, lr = np.mean([engine.train_step_loop(ds.tensors_to_batch(**next(dl_iter)))
+                            for _ in range(settings.program_runs_per_log)], axis=0)
+        assert np.isfinite(loss) and lr > 0
+        losses.append(loss)
+    assert losses[-1] < losses[0]
+    entity, score = dataset.predict("valid", engine.predict)
+    assert entity.shape == (len(data.eval_hr_["valid"]), settings.execution.predict_n_best)
+    assert score.shape == entity.shape and np.all(np.diff(score, axis=1) <= 0)
+    assert dataset.mrr("train", engine.predict) > 0.05

@@ -191,3 +191,35 @@ def test_mrr_definition():
 
     expected = np.mean([1.0 / (i + 1) if i < 10 else 0.0 for i in range(len(truth))])
     assert abs(ds.mrr("valid", predict_fn) - expected) < 1e-12
+
+
+@pytest.mark.parametrize("workers", [0, 2])
+def test_dataset_wrapper_with_torch_dataloader(workers):
+    """The reference's training script feeds the engine through a torch DataLoader over
+    DatasetWrapper (scripts/run_training.py:36-41, 68-71): batches arrive as int32 tensors
+    and go back to the engine's uint32 arrays; worker processes sample from their own streams."""
+    import torch
+
+    data = kge_data.RawData.generate(n_entity=70, n_relation_type=20, feature_size=0, n_train=100,
+                                     n_eval=50, seed=7)
+    S, n = 4, 3
+    settings = _data_settings(seed=5, batch_size=8, a2a_size=5)
+    dataset = kge_data.Dataset(data, n_shard=S, train_steps_per_program_run=n, settings=settings)
+    wrapper = kge_data.DatasetWrapper(dataset)
+    assert len(wrapper) == 2 ** 31 - 1
+    loader = torch.utils.data.DataLoader(wrapper, batch_size=None, num_workers=workers,
+                                         worker_init_fn=wrapper.worker_init_fn)
+    all_hrt = set(map(tuple, data.train_hrt.astype(np.int64)))
+    seen = []
+    for tensors in itertools.islice(iter(loader), 4):
+        assert all(t.dtype == torch.int32 for t in tensors.values())
+        batch = wrapper.tensors_to_batch(**tensors)
+        assert batch.remote.shape == (S, n, settings.batch_size + S * settings.a2a_size)
+        for part in vars(batch).values():
+            assert part.dtype == np.uint32
+        positive, negative = _entities_of(dataset, batch)
+        assert set(map(tuple, positive)) <= all_hrt
+        assert negative.min() >= 0 and negative.max() < data.n_entity
+        seen.append(batch.head.tobytes())
+    if workers:   # two workers, two streams: their first batches differ
+        assert seen[0] != seen[1]
