@@ -347,9 +347,10 @@ void parse_settings(kge_engine& E, const Items& s) {
     if (score == "TransE") E.score_fn = SCORE_TRANSE;
     else if (score == "DistMult") E.score_fn = SCORE_DISTMULT;
     else if (score == "ComplEx") E.score_fn = SCORE_COMPLEX;
-    else if (score == "RotatE" || score == "TransH")
+    else if (score == "RotatE") E.score_fn = SCORE_ROTATE;
+    else if (score == "TransH")
         throw std::invalid_argument("'model.score_fn' = '" + score + "' is not implemented on the HIP device "
-                                    "(supported: 'TransE', 'DistMult', 'ComplEx')");
+                                    "(supported: 'TransE', 'DistMult', 'ComplEx', 'RotatE')");
     else
         throw std::invalid_argument("'model.score_fn' must be one of 'TransE', 'ComplEx', 'RotatE', 'TransH', or "
                                     "'DistMult', not '" + score + "'");
@@ -361,9 +362,12 @@ void parse_settings(kge_engine& E, const Items& s) {
         throw std::invalid_argument("'model.distance_fn' must be one of 'L1', 'L2' or 'MatMul', not '" +
                                     distance + "'");
     if (E.score_fn == SCORE_DISTMULT) E.dist_fn = DIST_DOT;  // distMultScore ignores the setting (:571-573)
-    if (E.score_fn == SCORE_COMPLEX && E.D % 2)
-        throw std::invalid_argument("'model.score_fn' = 'ComplEx' needs an even 'model.embedding_size' "
+    if ((E.score_fn == SCORE_COMPLEX || E.score_fn == SCORE_ROTATE) && E.D % 2)
+        throw std::invalid_argument("'model.score_fn' = '" + score + "' needs an even 'model.embedding_size' "
                                     "(real and imaginary halves)");
+    if (E.score_fn == SCORE_ROTATE && E.dist_fn == DIST_DOT)
+        throw std::invalid_argument("'model.score_fn' = 'RotatE' scores by a distance: 'model.distance_fn' "
+                                    "must be 'L1' or 'L2'");
     if (loss == "logsigmoid") E.loss_fn = LOSS_LOGSIGMOID;
     else if (loss == "softmax") E.loss_fn = LOSS_SOFTMAX;
     else
@@ -391,7 +395,7 @@ void parse_settings(kge_engine& E, const Items& s) {
                 throw std::invalid_argument(msg.str());
             }
         };
-        check("relation_embedding", E.n_rel, E.D);
+        check("relation_embedding", E.n_rel, E.score_fn == SCORE_ROTATE ? E.D / 2 : E.D);
         check("feature_projection", E.F, E.D);
     }
     for (size_t i = 0; i < mods.map_len; ++i) {
@@ -424,7 +428,10 @@ void parse_settings(kge_engine& E, const Items& s) {
     };
     var("step", {(size_t)E.S});
     for (const char* suffix : {"", "/adam_m", "/adam_v"}) {
-        var(std::string("relation_embedding") + suffix, {(size_t)E.n_rel, (size_t)E.D});
+        // RotatE's rows are D / 2 phases (src/poplar_kge.cpp:248-249); the device rows keep the
+        // full pitch, their upper half stays zero
+        var(std::string("relation_embedding") + suffix,
+            {(size_t)E.n_rel, (size_t)(E.score_fn == SCORE_ROTATE ? E.D / 2 : E.D)});
         var(std::string("feature_projection") + suffix, {(size_t)E.F, (size_t)E.D});
     }
 }
@@ -758,7 +765,7 @@ void run_plan(kge_engine& E, int s0, int sn) {
 
 // how the gather combines a head row with its relation row (launch_gather_operands)
 static int rel_mode_of(const kge_engine& E) {
-    return E.score_fn == SCORE_DISTMULT ? 2 : E.score_fn == SCORE_COMPLEX ? 3 : 1;
+    return E.score_fn == SCORE_DISTMULT ? 2 : E.score_fn == SCORE_COMPLEX ? 3 : E.score_fn == SCORE_ROTATE ? 4 : 1;
 }
 
 void run_step(kge_engine& E, int i) {
@@ -885,12 +892,12 @@ void run_step(kge_engine& E, int i) {
     ContribSrc rsrc = {};
     rsrc.sorted_item = E.r_sorted_vals + (size_t)i * E.n_rel_items;
     rsrc.grad = E.grad.p;
-    rsrc.transform = E.score_fn == SCORE_DISTMULT ? 2 : E.score_fn == SCORE_COMPLEX ? 4 : 0;
+    rsrc.transform = E.score_fn == SCORE_DISTMULT ? 2 : E.score_fn == SCORE_COMPLEX ? 4 : E.score_fn == SCORE_ROTATE ? 6 : 0;
     rsrc.n_head = (int)SB; rsrc.half = E.D / 2;
     rsrc.rel = E.rel.p; rsrc.crel = crel; rsrc.ent = ent;
     ContribSrc esrc = rsrc;
     esrc.sorted_item = E.e_sorted_vals + (size_t)i * 2 * R;
-    esrc.transform = E.score_fn == SCORE_DISTMULT ? 1 : E.score_fn == SCORE_COMPLEX ? 3 : 0;
+    esrc.transform = E.score_fn == SCORE_DISTMULT ? 1 : E.score_fn == SCORE_COMPLEX ? 3 : E.score_fn == SCORE_ROTATE ? 5 : 0;
 
     ReduceArgs rr = {};
     rr.src = rsrc;

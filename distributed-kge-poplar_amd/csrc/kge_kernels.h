@@ -11,7 +11,11 @@ namespace kge {
 // TransE: score = gamma - distance(h + r, t).  DistMult: score = (h * r) . t.  ComplEx: the
 // complex product of h and r on the (real | imaginary) halves of the row, scored by the
 // distance function's value itself (src/poplar_kge.cpp:501-514).
-enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2 };
+// RotatE: (h_re, h_im) rotated by the relation's D/2 phases, whose sine and cosine pass
+// through float16 as in the reference (src/poplar_kge.cpp:516-537); score = gamma - distance.
+enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2, SCORE_ROTATE = 3 };
+// whether the score is the distance function's value itself (else gamma minus it)
+__host__ __device__ inline bool score_is_distance_value(int score_fn) { return score_fn == SCORE_DISTMULT || score_fn == SCORE_COMPLEX; }
 enum { DIST_L1 = 0, DIST_L2 = 1, DIST_DOT = 2 };
 enum { LOSS_LOGSIGMOID = 0, LOSS_SOFTMAX = 1 };
 enum { ET_F32 = 0, ET_BF16 = 1, ET_F16 = 2 };
@@ -91,7 +95,7 @@ struct ScoreShape {
 
 // Dense float32 operand matrix [n_rows, Dp] from indexed rows: rows [0, n_head)
 // combined with their relation row (rel_mode 1 add, 2 multiply, 3 complex product on the
-// halves [0, half) | [half, 2 half) of the row).
+// halves [0, half) | [half, 2 half) of the row, 4 rotation by the row's `half` phases).
 // With `out16` the values are rounded to bfloat16, stored there, and the float32
 // copy holds the same rounded values.
 void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
@@ -154,7 +158,8 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
 // Where gradient contributions come from.  transform: 0 none; 1 multiply head
 // rows (c < n_head) by rel[crel[c]] (DistMult, entity plan); 2 multiply by the
 // head entity row (DistMult, relation plan); 3 / 4 the same two for ComplEx: the
-// product with the complex conjugate on the halves [0, half) | [half, 2 half).
+// product with the complex conjugate on the halves [0, half) | [half, 2 half); 5 / 6 for
+// RotatE: the rotation back (entity plan), the phases' gradient in float16 (relation plan).
 struct ContribSrc {
     const uint32_t* sorted_item;  // this step's sorted values
     const float* grad;            // [R, Dp]

@@ -442,6 +442,21 @@ __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const fl
                 vv[x] = kk < half ? vv[x] * rrow[kk] - e2 * rrow[pp]    // re = h_re r_re - h_im r_im
                                   : e2 * rrow[kk] + vv[x] * rrow[pp];   // im = h_re r_im + h_im r_re
             }
+        } else if (rrow && rel_mode == 4) {
+            // rotation by the relation's phases (src/poplar_kge.cpp:516-530): phase, sine and
+            // cosine in float16, the rotation itself in float32
+            float* vv = &v.x;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const int kk = k + x;
+                if (kk >= 2 * half) { vv[x] = 0.f; continue; }
+                const int kq = kk < half ? kk : kk - half, pp = kk < half ? kk + half : kk - half;
+                const float th = (float)(_Float16)rrow[kq];
+                const float sn = (float)(_Float16)sinf(th), cs = (float)(_Float16)cosf(th);
+                const float e2 = load1(row, pp, ent.etype);
+                vv[x] = kk < half ? vv[x] * cs - e2 * sn     // re = h_re cos - h_im sin
+                                  : vv[x] * cs + e2 * sn;    // im = h_im cos + h_re sin
+            }
         } else if (rrow) v = combine_rel(v, rrow, k, rel_mode);
         // + 0 turns a -0 into +0, so that a difference of stored operands is never -0
         // (the paired L1 backward reads the sign off the difference's bit pattern)
@@ -632,7 +647,7 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
             const float dist = DIST == DIST_L2 ? sqrtf(acc[i][j]) : acc[i][j];
             distv[j] = dist;
             if (OM == 2) { outv[j] = dist; continue; }
-            const float score = sh.score_fn != SCORE_TRANSE ? dist : sh.gamma - dist;
+            const float score = score_is_distance_value(sh.score_fn) ? dist : sh.gamma - dist;
             if (OM == 1) { outv[j] = score; continue; }
             const bool pos = (uint32_t)n == label;
             const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
@@ -642,7 +657,7 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
             if (n < T) loss_acc -= w * lsig;
             // d loss / d score, times the loss scale
             const float ds = -w * sign * dlsig * grad_scale;
-            float c = sh.score_fn != SCORE_TRANSE ? ds : -ds;  // score = gamma - dist
+            float c = score_is_distance_value(sh.score_fn) ? ds : -ds;  // score = gamma - dist
             if (DIST == DIST_L2) c = dist != 0.f ? c * __builtin_amdgcn_rcpf(dist) : 0.f;
             outv[j] = c;
         }
@@ -1077,7 +1092,7 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
             if (OM == 2) {
                 outv = dist;
             } else {
-                const float score = sh.score_fn != SCORE_TRANSE ? dist : sh.gamma - dist;
+                const float score = score_is_distance_value(sh.score_fn) ? dist : sh.gamma - dist;
                 if (OM == 1) {
                     outv = score;
                     if (live && DIST == DIST_L2 && dist_blk) dist_blk[m * T + n] = dist;
@@ -1089,7 +1104,7 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
                     log_sigmoid_both(z, lsig, dlsig);
                     if (live) loss_acc -= w * lsig;
                     const float ds = -w * sign * dlsig * grad_scale;
-                    outv = sh.score_fn != SCORE_TRANSE ? ds : -ds;
+                    outv = score_is_distance_value(sh.score_fn) ? ds : -ds;
                     if (DIST == DIST_L2) outv = dist != 0.f ? outv * __builtin_amdgcn_rcpf(dist) : 0.f;
                 }
             }
@@ -1442,7 +1457,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
         const float lse = mx + logf(sum);
         const float inv_norm = 1.f / ((float)sh.S * (float)sh.B);
         const float gs = inv_norm * sh.loss_scale;
-        const float sgn = sh.score_fn != SCORE_TRANSE ? 1.f : -1.f;
+        const float sgn = score_is_distance_value(sh.score_fn) ? 1.f : -1.f;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int t = 4 * lane + 256 * i;
@@ -1483,7 +1498,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
             const float z = s[t] + (pos ? 0.f : corr);
             if (pos) loss = -(z - lse) * inv_norm;
             const float ds = (expf(z - lse) - (pos ? 1.f : 0.f)) * inv_norm * sh.loss_scale;
-            float c = sh.score_fn != SCORE_TRANSE ? ds : -ds;
+            float c = score_is_distance_value(sh.score_fn) ? ds : -ds;
             if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
             s[t] = c;
             if (s16) s16[t] = f32_to_bf16(c);
@@ -1514,7 +1529,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
             const float sign = pos ? 1.f : -1.f, z = sign * sc;
             loss -= w * log_sigmoid(z) * inv_norm;
             const float ds = -w * sign * log_sigmoid_grad(z) * inv_norm * sh.loss_scale;
-            float c = sh.score_fn != SCORE_TRANSE ? ds : -ds;
+            float c = score_is_distance_value(sh.score_fn) ? ds : -ds;
             if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
             s[t] = c;
             if (s16) s16[t] = f32_to_bf16(c);
@@ -2335,7 +2350,39 @@ void launch_row_range(uint32_t base, int n_live, int n, uint32_t* out, hipStream
 // columns from k, with the DistMult product rule applied on load.
 DEVINL float4 load_contrib(const ContribSrc& cs, uint32_t c, int k, int Dp) {
     float4 g = *reinterpret_cast<const float4*>(cs.grad + (size_t)c * Dp + k);
-    if (cs.transform >= 3) {
+    if (cs.transform >= 5) {
+        // RotatE: the predicted tail is (h_re, h_im) rotated by the phases.  Entity plan: the
+        // gradient rotated back.  Relation plan: the phases' gradient, formed in float16 as the
+        // reference's float16 sine / cosine backward ops form it (src/pag/pag.cpp:552-637),
+        // in columns [0, half); zero above.
+        if (c < (uint32_t)cs.n_head) {
+            const float* gr = cs.grad + (size_t)c * Dp;
+            const float* rr = cs.rel + (size_t)cs.crel[c] * Dp;
+            const char* er = row_ptr(cs.ent, c);
+            float* gg = &g.x;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const int kk = k + x;
+                if (kk >= 2 * cs.half) { gg[x] = 0.f; continue; }
+                const int kq = kk < cs.half ? kk : kk - cs.half;
+                const float th = (float)(_Float16)rr[kq];
+                const _Float16 sn = (_Float16)sinf(th), cs16 = (_Float16)cosf(th);
+                const float g_re = gr[kq], g_im = gr[kq + cs.half];
+                if (cs.transform == 5) {
+                    gg[x] = kk < cs.half ? g_re * (float)cs16 + g_im * (float)sn
+                                         : g_im * (float)cs16 - g_re * (float)sn;
+                } else if (kk < cs.half) {
+                    const float h_re = load1(er, kq, cs.ent.etype), h_im = load1(er, kq + cs.half, cs.ent.etype);
+                    const _Float16 g_sin = (_Float16)(-g_re * h_im + g_im * h_re);
+                    const _Float16 g_cos = (_Float16)(g_re * h_re + g_im * h_im);
+                    const _Float16 from_cos = -g_cos * sn, from_sin = g_sin * cs16;
+                    gg[x] = (float)(_Float16)(from_cos + from_sin);
+                } else {
+                    gg[x] = 0.f;
+                }
+            }
+        }
+    } else if (cs.transform >= 3) {
         // ComplEx: the predicted tail is the complex product h r, so the head's gradient is
         // g conj(r) and the relation's g conj(h) (column kk pairs with kk +- half):
         //   re: g_re o_re + g_im o_im      im: g_im o_re - g_re o_im      (o = r or h)

@@ -384,16 +384,19 @@ class Engine:
     # ---- initialisation ------------------------------------------------------
     def initialise_variables(self) -> None:
         """step = 0, zero moments, scaled-normal parameters (reference :624-688):
-        relation_embedding ~ (init_scale / D) N(0, 1); feature_projection the
-        same divided by sqrt(F)."""
+        relation_embedding ~ (init_scale / D) N(0, 1) (RotatE: uniform phases); feature_projection
+        ~ N(0, 1) scaled the same way and divided by sqrt(F)."""
         m = self.settings.model
         self.write_variable("step", np.zeros(m.n_shard, np.uint32))
         for name, shape in self.variable_to_shape.items():
             if name.endswith(("/adam_m", "/adam_v")):
                 self.write_variable(name, np.zeros(shape, np.float32))
-        self.write_variable(
-            "relation_embedding",
-            self.init_scale * self.random_normal((m.n_relation_type, self.settings.relation_embedding_size)))
+        relation_shape = (m.n_relation_type, self.settings.relation_embedding_size)
+        if m.score_fn == "RotatE":   # phases, uniform in [-pi, pi) (reference :633-635)
+            relation = self.random_uniform(relation_shape, low=-np.pi, high=np.pi)
+        else:
+            relation = self.random_normal(relation_shape)
+        self.write_variable("relation_embedding", self.init_scale * relation)
         self.write_variable(
             "feature_projection",
             (self.init_scale / np.sqrt(max(m.entity_feature_size, 1)))

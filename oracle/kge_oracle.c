@@ -22,7 +22,11 @@
  * not the reference's, cfg.scoring_bf16 (operands of the scoring and projection
  * products rounded to bfloat16, float32 accumulation), is pinned the same way
  * with a straight-through rounding in the autograd restatement.
- * "parity unpinned": none of the functions in this file.
+ * "parity unpinned": RotatE's float16 sine and cosine only.  The reference takes them with
+ * the IPU's float16 instructions, whose last-bit rounding no fixture here records; this
+ * file (and the torch restatement, with torch's float16 kernels) round the correctly
+ * rounded float result to float16.  Everything around them -- the float16 cast of the
+ * phases, the rotation, the float16 gradient arithmetic -- is pinned against autograd.
  */
 #include <math.h>
 #include <stdint.h>
@@ -35,7 +39,7 @@
 
 #define API __attribute__((visibility("default")))
 
-enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2 };
+enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2, SCORE_ROTATE = 3 };
 enum { DIST_L1 = 0, DIST_L2 = 1, DIST_DOT = 2 };
 enum { LOSS_LOGSIGMOID = 0, LOSS_SOFTMAX = 1 };
 enum { STORE_F32 = 0, STORE_F16 = 1, STORE_BF16_EMB = 2 };
@@ -447,6 +451,8 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                               const uint32_t* tail, float* loss_out) {
     const int64_t S = c->n_shard, B = c->batch, A = c->a2a, T = S * A, NR = B + T;
     const int64_t D = c->dim, F = c->feature, ROW = 3 * D + F, NREL = c->n_relation;
+    /* RotatE's relation rows are D / 2 phases (poplar_kge.cpp:248-249) */
+    const int64_t RD = c->score_fn == SCORE_ROTATE ? D / 2 : D;
     const int64_t NE = c->n_entity;
 #define KEY(s, slot) ((c->shared_table ? 0 : (int64_t)(s) * NE) + (int64_t)remote[(s) * NR + (slot)])
 
@@ -503,7 +509,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
         free(fh); free(val);
     }
 
-    REAL* grel = (REAL*)calloc((size_t)(NREL * D), sizeof(REAL));
+    REAL* grel = (REAL*)calloc((size_t)(NREL * RD), sizeof(REAL));
     REAL* p = (REAL*)malloc(sizeof(REAL) * (size_t)(B * D));
     REAL* tl = (REAL*)malloc(sizeof(REAL) * (size_t)(T * D));
     REAL* score = (REAL*)malloc(sizeof(REAL) * (size_t)(B * T));
@@ -516,7 +522,19 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
         /* 2. heads / predicted tails (:676-677, :488-490, :567-569) */
         for (int64_t b = 0; b < B; ++b) {
             const REAL* h = hidden + (d * NR + head[d * B + b]) * D;
-            const float* r = rel + (int64_t)relation[d * B + b] * D;
+            const float* r = rel + (int64_t)relation[d * B + b] * RD;
+            if (c->score_fn == SCORE_ROTATE) {
+                /* rotatEPredict (:516-530): the phases pass through float16, as do their sine
+                 * and cosine, which then rotate (h_re, h_im) in float32 */
+                const int64_t H = D / 2;
+                for (int64_t k = 0; k < H; ++k) {
+                    const float th = round_f16(r[k]);
+                    const REAL sn = round_f16((float)sin((double)th)), cs = round_f16((float)cos((double)th));
+                    p[b * D + k] = h[k] * cs - h[k + H] * sn;
+                    p[b * D + k + H] = h[k + H] * cs + h[k] * sn;
+                }
+                continue;
+            }
             if (c->score_fn == SCORE_COMPLEX) {
                 /* complExPredict (:501-510): halves are real | imaginary parts, (h_re + i h_im)(r_re + i r_im) */
                 const int64_t H = D / 2;
@@ -558,7 +576,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                 dist[b * T + t] = acc;
                 /* distMultScore / complExScore return the distance function's value itself
                  * (:512-514, :571-573); TransE gamma minus it (:492-499) */
-                if (c->score_fn != SCORE_TRANSE)
+                if (c->score_fn == SCORE_DISTMULT || c->score_fn == SCORE_COMPLEX)
                     score[b * T + t] = acc;
                 else
                     score[b * T + t] = (REAL)c->gamma - acc;
@@ -584,7 +602,8 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                     }
                     continue;
                 }
-                if (c->score_fn == SCORE_TRANSE) g = -g; /* score = gamma - distance (pag.cpp sub: :323-345) */
+                if (c->score_fn == SCORE_TRANSE || c->score_fn == SCORE_ROTATE)
+                    g = -g; /* score = gamma - distance (pag.cpp sub: :323-345) */
                 if (dot) {
                     for (int64_t k = 0; k < D; ++k) {
                         gx[k] += g * y[k];
@@ -612,6 +631,26 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             REAL* gh = ghid + (d * NR + head[d * B + b]) * D;
             const REAL* h = hidden + (d * NR + head[d * B + b]) * D;
             const int64_t r = relation[d * B + b];
+            if (c->score_fn == SCORE_ROTATE) {
+                /* p_re = h_re cos - h_im sin, p_im = h_im cos + h_re sin.  The gradient of the
+                 * phase runs in float16 as the forward does (cast's backward casts the gradient,
+                 * pag.cpp:619-637; sin' = g cos, cos' = -g sin, :552-594), then back to float32 */
+                const int64_t H = D / 2;
+                for (int64_t k = 0; k < H; ++k) {
+                    const REAL gre = dp[b * D + k], gim = dp[b * D + k + H];
+                    const float th = round_f16(rel[r * RD + k]);
+                    const float sn = round_f16((float)sin((double)th)), cs = round_f16((float)cos((double)th));
+                    gh[k] += gre * cs + gim * sn;
+                    gh[k + H] += gim * cs - gre * sn;
+                    const float g_sin = round_f16((float)(-gre * h[k + H] + gim * h[k]));
+                    const float g_cos = round_f16((float)(gre * h[k] + gim * h[k + H]));
+                    /* backward ops run in reverse: cos's first, then sin's is added to it */
+                    const float from_cos = round_f16((float)(-(double)g_cos * (double)sn));
+                    const float from_sin = round_f16((float)((double)g_sin * (double)cs));
+                    grel[r * RD + k] += (REAL)round_f16((float)((double)from_cos + (double)from_sin));
+                }
+                continue;
+            }
             if (c->score_fn == SCORE_COMPLEX) {
                 /* p_re = h_re r_re - h_im r_im, p_im = h_re r_im + h_im r_re */
                 const int64_t H = D / 2;
@@ -714,9 +753,9 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
     {
         float* gf = (float*)malloc(sizeof(float) * (size_t)D);
         for (int64_t r = 0; r < NREL; ++r) {
-            for (int64_t k = 0; k < D; ++k) gf[k] = (float)grel[r * D + k];
+            for (int64_t k = 0; k < RD; ++k) gf[k] = (float)grel[r * RD + k];
             const int64_t shard = c->shared_table ? 0 : r / (NREL / S);
-            kge_oracle_adam(rel + r * D, rel_m + r * D, rel_v + r * D, gf, D,
+            kge_oracle_adam(rel + r * RD, rel_m + r * RD, rel_v + r * RD, gf, RD,
                             alpha[shard] * c->lr_mod_relation, c->beta_m, c->beta_v, c->epsilon,
                             c->weight_decay, 0);
         }

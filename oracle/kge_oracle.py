@@ -14,7 +14,7 @@ import numpy as np
 
 HERE = Path(__file__).resolve().parent
 
-SCORE = {"TransE": 0, "DistMult": 1, "ComplEx": 2}
+SCORE = {"TransE": 0, "DistMult": 1, "ComplEx": 2, "RotatE": 3}
 DIST = {"L1": 0, "L2": 1, "MatMul": 2}
 LOSS = {"logsigmoid": 0, "softmax": 1}
 STORE = {"float32": 0, "float16": 1, "bfloat16_embedding": 2}
@@ -273,7 +273,13 @@ def predict_reference(cfg, state, queries, shard_to_count, n_best):
     h = hidden[q[:, 0] * NE + q[:, 1]]
     dot = cfg.score_fn == SCORE["DistMult"] or cfg.distance_fn == DIST["MatMul"]
     r = rel[q[:, 2]]
-    if cfg.score_fn == SCORE["ComplEx"]:  # src/poplar_kge.cpp:501-510
+    if cfg.score_fn == SCORE["RotatE"]:  # src/poplar_kge.cpp:516-530: phases, sine, cosine in float16
+        H = D // 2
+        th = r[:, :H].astype(np.float32).astype(np.float16)
+        sn = np.sin(th.astype(np.float64)).astype(np.float16).astype(np.float64)
+        cs = np.cos(th.astype(np.float64)).astype(np.float16).astype(np.float64)
+        p = np.concatenate([h[:, :H] * cs - h[:, H:] * sn, h[:, H:] * cs + h[:, :H] * sn], axis=1)
+    elif cfg.score_fn == SCORE["ComplEx"]:  # src/poplar_kge.cpp:501-510
         H = D // 2
         p = np.concatenate([h[:, :H] * r[:, :H] - h[:, H:] * r[:, H:],
                             h[:, :H] * r[:, H:] + h[:, H:] * r[:, :H]], axis=1)
@@ -285,7 +291,7 @@ def predict_reference(cfg, state, queries, shard_to_count, n_best):
         dist = np.stack([np.abs(x[None, :] - hidden).sum(-1) for x in p])
     else:
         dist = np.stack([np.sqrt(((x[None, :] - hidden) ** 2).sum(-1)) for x in p])
-    score = cfg.gamma - dist if cfg.score_fn == SCORE["TransE"] else dist
+    score = cfg.gamma - dist if cfg.score_fn in (SCORE["TransE"], SCORE["RotatE"]) else dist
     live = np.zeros((S, NE), bool)
     for s, n in enumerate(shard_to_count):
         live[s, 1:1 + int(n)] = True

@@ -32,11 +32,13 @@ def make_state(c, rng, warm=True, scale=None):
         ed[:, 2 * D:3 * D] = 0.05 + np.abs(rng.normal(0, 0.3, (rows, D)))
     if F:
         ed[:, 3 * D:] = rng.normal(0, 1, (rows, F)).astype(np.float16)
+    rotate = c["score_fn"] == "RotatE"   # relation rows are D / 2 phases
+    RD = D // 2 if rotate else D
     st = {
         "entity_data": ed,
-        "relation_embedding": rng.normal(0, scale, (NR, D)).astype(np.float32),
-        "relation_embedding/adam_m": (rng.normal(0, 0.1, (NR, D)) * warm).astype(np.float32),
-        "relation_embedding/adam_v": ((0.05 + np.abs(rng.normal(0, 0.3, (NR, D))))**2 * warm).astype(np.float32),
+        "relation_embedding": rng.normal(0, 1.0 if rotate else scale, (NR, RD)).astype(np.float32),
+        "relation_embedding/adam_m": (rng.normal(0, 0.1, (NR, RD)) * warm).astype(np.float32),
+        "relation_embedding/adam_v": ((0.05 + np.abs(rng.normal(0, 0.3, (NR, RD))))**2 * warm).astype(np.float32),
         "step": 7 if warm else 0,
     }
     if F:

@@ -52,6 +52,15 @@ CASES = {
                            n_entity=4000, n_relation=8, gamma=6.0, shared_table=True),
     "bf16_embedding_l2": dict(distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
                               n_entity=3000, n_relation=8, gamma=6.0, storage="bfloat16_embedding"),
+    # RotatE (src/poplar_kge.cpp:516-537): rotation by the relation's D / 2 phases, sine / cosine
+    # and the phases' gradient in float16
+    "rotate_l1": dict(score_fn="RotatE", distance_fn="L1", feature=0),
+    "rotate_l2_feat": dict(score_fn="RotatE", distance_fn="L2", gamma=4.0),
+    "rotate_softmax_odd_half": dict(score_fn="RotatE", distance_fn="L1", loss_fn="softmax",
+                                    softmax_correction_weight=1.0, feature=0, dim=10, n_entity=41, batch=5,
+                                    a2a=3),
+    "aligned_rotate_l2": dict(score_fn="RotatE", distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64,
+                              feature=0, n_entity=3000, n_relation=8, gamma=6.0),
     # norm regularisers (src/poplar_kge.cpp:430-437, 463-465): the WikiKG preset's feature
     # regulariser, all three with different powers, and without features (hidden = embedding)
     "feature_regularisation_p3": dict(feature_regularisation=(3.0, 1e-2), loss_fn="softmax",
@@ -207,6 +216,13 @@ def run_case(oracle, kw, n_step=3, batch_fn=K.random_batch, lr=(0.1, 0.07), n_lo
             assert K.rel_l2(st_h[k][:, :D], st_o[k][:, :D]) < 2e-3
             mism = np.mean(st_h[k][:, :D] != st_o[k][:, :D])
             assert mism < 1e-3, mism  # all but a handful of elements are bit-identical
+            continue
+        if c["score_fn"] == "RotatE" and k.startswith("relation_embedding"):
+            # the phases' gradient is formed in float16 (as the reference forms it): where the
+            # float32 value it is rounded from differs in its last bits between two implementations,
+            # an element lands on the neighbouring float16 (2^-11 relative)
+            assert K.rel_l2(st_h[k], st_o[k]) < 1e-3, (k, K.rel_l2(st_h[k], st_o[k]))
+            assert K.rel_l2(d_h, d_o) < 5e-3, (k, K.rel_l2(d_h, d_o))
             continue
         assert K.rel_l2(st_h[k], st_o[k]) < 1e-5, (k, K.rel_l2(st_h[k], st_o[k]))
         assert K.rel_l2(d_h, d_o) < 1e-4, (k, K.rel_l2(d_h, d_o))

@@ -164,7 +164,7 @@ def _random_queries(engine, n):
                      engine.random_integers(s.model.n_relation_type, (n,))], axis=-1)
 
 
-@pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "complex", "no_features_big"])
+@pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "complex", "rotate", "no_features_big"])
 def test_predict_vs_brute_force(variant):
     """Engine.predict against a float64 brute force over every row of every shard
     (the reference checks shapes, ranges and ordering, tests/python/test_poplar_kge.py:155-175,
@@ -181,6 +181,8 @@ def test_predict_vs_brute_force(variant):
         m.score_fn, m.distance_fn = "DistMult", "MatMul"
     elif variant == "complex":
         m.score_fn, m.distance_fn = "ComplEx", "MatMul"
+    elif variant == "rotate":
+        m.score_fn = "RotatE"
     elif variant == "no_features_big":
         # several chunks of tails per shard, several query chunks, ragged counts
         m.n_entity, m.entity_feature_size, m.embedding_size, m.n_shard = 20000, 0, 32, 3

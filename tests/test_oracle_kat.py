@@ -297,6 +297,12 @@ STEP_CASES = {
     "complex_matmul_logsigmoid_feat": dict(score_fn="ComplEx", distance_fn="MatMul", feature=4),
     "complex_l2": dict(score_fn="ComplEx", distance_fn="L2", feature=0),
     "complex_l1": dict(score_fn="ComplEx", distance_fn="L1", feature=0),
+    # RotatE (src/poplar_kge.cpp:516-537): rotation of (h_re, h_im) by the relation's phases, whose
+    # sine and cosine (and the phases' gradient) run in float16
+    "rotate_l1": dict(score_fn="RotatE", distance_fn="L1", feature=0),
+    "rotate_l2_feat": dict(score_fn="RotatE", distance_fn="L2", gamma=4.0),
+    "rotate_softmax": dict(score_fn="RotatE", distance_fn="L1", loss_fn="softmax", softmax_correction_weight=1.0,
+                           feature=0, dim=12),
     # norm regularisers (src/poplar_kge.cpp:430-437, 463-465), the WikiKG preset's among them
     "feature_regularisation_p3": dict(feature_regularisation=(3.0, 1e-2), loss_fn="softmax",
                                       softmax_correction_weight=1.0),

@@ -114,8 +114,15 @@ def step(cfg, state, lr, batch_step):
     tails = hidden[shards[:, None, None], a2a]  # [S(src), S(dst), A, D]
     tails = tails.transpose(0, 1).reshape(S, Tn, D)  # all-to-all
     r = rel[relation]
-    if cfg["score_fn"] in ("TransE", "ComplEx"):
-        if cfg["score_fn"] == "ComplEx":  # complex product on (real | imaginary) halves
+    if cfg["score_fn"] in ("TransE", "ComplEx", "RotatE"):
+        if cfg["score_fn"] == "RotatE":
+            # the phases, their sine and cosine and the phases' gradient in float16 (torch's own
+            # float16 kernels and autograd), the rotation in float64
+            theta = r.to(T.float32).to(T.float16)
+            sn, cs = T.sin(theta).to(T.float64), T.cos(theta).to(T.float64)
+            h_re, h_im = heads[..., :D // 2], heads[..., D // 2:]
+            pred = T.cat([h_re * cs - h_im * sn, h_im * cs + h_re * sn], -1)
+        elif cfg["score_fn"] == "ComplEx":  # complex product on (real | imaginary) halves
             hc = T.complex(heads[..., :D // 2], heads[..., D // 2:]) * T.complex(r[..., :D // 2], r[..., D // 2:])
             pred = T.cat([hc.real, hc.imag], -1)
         else:
@@ -130,7 +137,7 @@ def step(cfg, state, lr, batch_step):
             dist = T.where(sq > 0, T.sqrt(safe), T.zeros_like(sq))
         else:
             dist = pred @ tails.transpose(1, 2)
-        score = cfg["gamma"] - dist if cfg["score_fn"] == "TransE" else dist
+        score = dist if cfg["score_fn"] == "ComplEx" else cfg["gamma"] - dist
     else:
         pred = heads * r
         if cfg.get("scoring_bf16"):
