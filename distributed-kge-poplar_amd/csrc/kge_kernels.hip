@@ -418,6 +418,9 @@ void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sort
 // converted to float32 and with the relation already applied for the heads
 // (predicted tail h + r, or h * r), into the dense operand matrix the scoring
 // kernels read: rows [0, n_head) = a-operands, the rest = b-operands.
+// XF: the complex-product / rotation modes (3, 4) are compiled in (their code costs the
+// plain modes registers otherwise)
+template <bool XF>
 __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const float* __restrict__ rel,
                                                          const uint32_t* __restrict__ crel,
                                                          int rel_mode, int half, int n_head, int n_rows,
@@ -430,7 +433,7 @@ __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const fl
     const float* rrow = (c < n_head && rel_mode) ? rel + (size_t)crel[c] * Dp : nullptr;
     for (int k = lane * 4; k < Dp; k += 256) {
         float4 v = load4(row, k, ent);
-        if (rrow && rel_mode == 3) {
+        if (XF && rrow && rel_mode == 3) {
             // complex product: column kk pairs with kk +- half (src/poplar_kge.cpp:501-510)
             float* vv = &v.x;
 #pragma unroll
@@ -442,7 +445,7 @@ __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const fl
                 vv[x] = kk < half ? vv[x] * rrow[kk] - e2 * rrow[pp]    // re = h_re r_re - h_im r_im
                                   : e2 * rrow[kk] + vv[x] * rrow[pp];   // im = h_re r_im + h_im r_re
             }
-        } else if (rrow && rel_mode == 4) {
+        } else if (XF && rrow && rel_mode == 4) {
             // rotation by the relation's phases (src/poplar_kge.cpp:516-530): phase, sine and
             // cosine in float16, the rotation itself in float32
             float* vv = &v.x;
@@ -478,8 +481,12 @@ __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const fl
 void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
                             int half, int n_head, int n_rows, int Dp, float* out, uint16_t* out16,
                             hipStream_t stream) {
-    hipLaunchKernelGGL(k_gather_operands, dim3((n_rows + 3) / 4), dim3(256), 0, stream, ent, rel, crel,
-                       rel_mode, half, n_head, n_rows, Dp, out, out16);
+    if (rel_mode >= 3)
+        hipLaunchKernelGGL(k_gather_operands<true>, dim3((n_rows + 3) / 4), dim3(256), 0, stream, ent, rel, crel,
+                           rel_mode, half, n_head, n_rows, Dp, out, out16);
+    else
+        hipLaunchKernelGGL(k_gather_operands<false>, dim3((n_rows + 3) / 4), dim3(256), 0, stream, ent, rel, crel,
+                           rel_mode, half, n_head, n_rows, Dp, out, out16);
 }
 
 // --------------------------------------------------------------------------
@@ -2348,9 +2355,10 @@ void launch_row_range(uint32_t base, int n_live, int n, uint32_t* out, hipStream
 
 // One gradient contribution (row c of the contribution-gradient matrix), four
 // columns from k, with the DistMult product rule applied on load.
+template <bool XF>  // XF: the ComplEx / RotatE transforms (3 .. 6) are compiled in
 DEVINL float4 load_contrib(const ContribSrc& cs, uint32_t c, int k, int Dp) {
     float4 g = *reinterpret_cast<const float4*>(cs.grad + (size_t)c * Dp + k);
-    if (cs.transform >= 5) {
+    if (XF && cs.transform >= 5) {
         // RotatE: the predicted tail is (h_re, h_im) rotated by the phases.  Entity plan: the
         // gradient rotated back.  Relation plan: the phases' gradient, formed in float16 as the
         // reference's float16 sine / cosine backward ops form it (src/pag/pag.cpp:552-637),
@@ -2382,7 +2390,7 @@ DEVINL float4 load_contrib(const ContribSrc& cs, uint32_t c, int k, int Dp) {
                 }
             }
         }
-    } else if (cs.transform >= 3) {
+    } else if (XF && cs.transform >= 3) {
         // ComplEx: the predicted tail is the complex product h r, so the head's gradient is
         // g conj(r) and the relation's g conj(h) (column kk pairs with kk +- half):
         //   re: g_re o_re + g_im o_im      im: g_im o_re - g_re o_im      (o = r or h)
@@ -2415,7 +2423,7 @@ DEVINL float4 load_contrib(const ContribSrc& cs, uint32_t c, int k, int Dp) {
 // k..k+3: eight independent row loads in flight, added in position order.
 // Must be called by every lane of the wave (the item indices travel by
 // shuffle); lanes with `active` false load nothing and return zero.
-template <int NB>
+template <int NB, bool XF>
 DEVINL float4 sum_contribs(const ContribSrc& cs, uint32_t pos, uint32_t n, int k, int Dp, int lane,
                            bool active) {
     float4 acc = make_float4(0, 0, 0, 0);
@@ -2425,7 +2433,7 @@ DEVINL float4 sum_contribs(const ContribSrc& cs, uint32_t pos, uint32_t n, int k
 #pragma unroll
         for (int x = 0; x < NB; ++x) {
             const uint32_t c = __shfl(mine, x, 64);
-            v[x] = (active && j + x < n) ? load_contrib(cs, c, k, Dp) : make_float4(0, 0, 0, 0);
+            v[x] = (active && j + x < n) ? load_contrib<XF>(cs, c, k, Dp) : make_float4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int x = 0; x < NB; ++x) acc = f4add(acc, v[x]);
@@ -2438,7 +2446,7 @@ DEVINL float4 sum_contribs(const ContribSrc& cs, uint32_t pos, uint32_t n, int k
 // NW = 16 serves chunks of up to 256 contributions with the same two rounds of
 // eight loads per wave that NW = 4 needs for 64: four times fewer partials for
 // the second level to walk through.
-template <int NW>
+template <int NW, bool XF>
 __global__ __launch_bounds__(NW * 64) void k_reduce_chunks(ReduceArgs a0, ReduceArgs a1) {
     __shared__ __attribute__((aligned(16))) float part[NW - 1][256];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -2463,7 +2471,7 @@ __global__ __launch_bounds__(NW * 64) void k_reduce_chunks(ReduceArgs a0, Reduce
     const uint32_t w0 = min(len, wave * share), w1 = min(len, w0 + share);
     for (int k0 = 0; k0 < Dp; k0 += 256) {
         const int k = k0 + lane * 4;
-        float4 acc = sum_contribs<8>(a.src, pos + w0, w1 - w0, k, Dp, lane, k < Dp);
+        float4 acc = sum_contribs<8, XF>(a.src, pos + w0, w1 - w0, k, Dp, lane, k < Dp);
         if (wave > 0) *reinterpret_cast<float4*>(&part[wave - 1][lane * 4]) = acc;
         __syncthreads();
         if (wave == 0 && k < Dp) {
@@ -2478,10 +2486,14 @@ __global__ __launch_bounds__(NW * 64) void k_reduce_chunks(ReduceArgs a0, Reduce
 static void launch_reduce_kernel(const ReduceArgs& a0, const ReduceArgs& a1, hipStream_t stream) {
     const int n = a0.max_chunks + a1.max_chunks;
     if (n == 0) return;
-    if (std::max(a0.chunk, a1.chunk) > 64)
-        hipLaunchKernelGGL(k_reduce_chunks<16>, dim3(n), dim3(1024), 0, stream, a0, a1);
-    else
-        hipLaunchKernelGGL(k_reduce_chunks<4>, dim3(n), dim3(256), 0, stream, a0, a1);
+    const bool xf = (a0.max_chunks && a0.src.transform >= 3) || (a1.max_chunks && a1.src.transform >= 3);
+    if (std::max(a0.chunk, a1.chunk) > 64) {
+        if (xf) hipLaunchKernelGGL((k_reduce_chunks<16, true>), dim3(n), dim3(1024), 0, stream, a0, a1);
+        else hipLaunchKernelGGL((k_reduce_chunks<16, false>), dim3(n), dim3(1024), 0, stream, a0, a1);
+    } else {
+        if (xf) hipLaunchKernelGGL((k_reduce_chunks<4, true>), dim3(n), dim3(256), 0, stream, a0, a1);
+        else hipLaunchKernelGGL((k_reduce_chunks<4, false>), dim3(n), dim3(256), 0, stream, a0, a1);
+    }
 }
 void launch_reduce_chunks(const ReduceArgs& a, hipStream_t stream) {
     ReduceArgs none = a;
@@ -2510,7 +2522,7 @@ DEVINL void adam4(float4& p, float4& m, float4& v, float4 g, const AdamArgs& a, 
 // One wave per distinct row: gather its gradient (directly from its few
 // contributions, or from its chunk partials), Adam, write the row back.
 // MF32: both moments float32 (the usual layout), accessed as plain 16-byte words
-template <bool MF32>
+template <bool MF32, bool XF>
 __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
     const int lane = threadIdx.x & 63;
     // two tables share the launch: blocks [0, ceil(a0.max_rows / 4)) serve the first
@@ -2535,7 +2547,7 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
         const bool active = k < Dp;
         float4 g = make_float4(0, 0, 0, 0);
         if (!a.grad_direct && q1 == q0 && n_real)  // wave-uniform: all lanes take part in the shuffles
-            g = sum_contribs<8>(a.src, pos, n_real, k, Dp, lane, active);
+            g = sum_contribs<8, XF>(a.src, pos, n_real, k, Dp, lane, active);
         if (!active) continue;
         float4 p = load4(prow, k, a.p_etype);
         float4 m, v;
@@ -2582,8 +2594,11 @@ static void launch_adam_kernel(const AdamArgs& a0, const AdamArgs& a1, hipStream
     const dim3 grid((a0.max_rows + 3) / 4 + (a1.max_rows + 3) / 4);
     if (grid.x == 0) return;
     const bool f32 = (a0.max_rows == 0 || a0.m_etype == ET_F32) && (a1.max_rows == 0 || a1.m_etype == ET_F32);
-    if (f32) hipLaunchKernelGGL(k_adam_rows<true>, grid, dim3(256), 0, stream, a0, a1);
-    else hipLaunchKernelGGL(k_adam_rows<false>, grid, dim3(256), 0, stream, a0, a1);
+    const bool xf = (a0.max_rows && a0.src.transform >= 3) || (a1.max_rows && a1.src.transform >= 3);
+    if (f32 && !xf) hipLaunchKernelGGL((k_adam_rows<true, false>), grid, dim3(256), 0, stream, a0, a1);
+    else if (f32) hipLaunchKernelGGL((k_adam_rows<true, true>), grid, dim3(256), 0, stream, a0, a1);
+    else if (!xf) hipLaunchKernelGGL((k_adam_rows<false, false>), grid, dim3(256), 0, stream, a0, a1);
+    else hipLaunchKernelGGL((k_adam_rows<false, true>), grid, dim3(256), 0, stream, a0, a1);
 }
 void launch_adam_rows(const AdamArgs& a, hipStream_t stream) {
     AdamArgs none = a;
