@@ -143,15 +143,11 @@ def read_rows(engine, settings, ids):
     return out
 
 
-def cpu_baseline(engine, settings, w, batch, n_check, n_cpu_steps):
-    """Times the sequential float32 oracle on the first `n_cpu_steps` steps of
-    the workload, starting from the device's own initial rows.  The first
-    `n_check` of them are run as a separate call so that their mean loss can be
-    compared with the GPU's.  Returns (json object, loss of the first call)."""
-    from oracle.kge_oracle import Oracle, make_cfg
-
+def cpu_start_state(engine, settings, w, sub):
+    """The oracle-side state and configuration for the steps in `sub`, from the device's own
+    initial rows (only the rows those steps touch are read back; the rest of the host table
+    stays untouched virtual memory)."""
     m, d = settings.model, settings.data
-    sub = {k: np.ascontiguousarray(v[:, :n_cpu_steps]) for k, v in vars(batch).items()}
     ids = np.unique(sub["remote"])
     rows = read_rows(engine, settings, ids)
     table = np.zeros((m.n_entity, settings.entity_data_r_size), np.float32)  # untouched pages stay virtual
@@ -162,14 +158,28 @@ def cpu_baseline(engine, settings, w, batch, n_check, n_cpu_steps):
         for suffix in ("", "/adam_m", "/adam_v"):
             state[name + suffix] = engine.read_variable(name + suffix)
     softmax = w.get("loss") == "softmax"
-    cfg = make_cfg(n_shard=m.n_shard, n_entity=m.n_entity, n_relation=m.n_relation_type,
-                   dim=m.embedding_size, feature=m.entity_feature_size, batch=d.batch_size, a2a=d.a2a_size,
-                   score_fn=m.score_fn, distance_fn=m.distance_fn,
-                   loss_fn="softmax" if softmax else "logsigmoid",
-                   softmax_correction_weight=1.0 if softmax else 0.0,
-                   shared_table=True, gamma=m.gamma, loss_scale=settings.training.loss_scale,
-                   scoring_bf16=settings.execution.scoring_dtype == "bfloat16",
-                   storage="bfloat16_embedding" if w.get("embedding_dtype") == "bfloat16" else "float32")
+    cfg = dict(n_shard=m.n_shard, n_entity=m.n_entity, n_relation=m.n_relation_type,
+               dim=m.embedding_size, feature=m.entity_feature_size, batch=d.batch_size, a2a=d.a2a_size,
+               score_fn=m.score_fn, distance_fn=m.distance_fn,
+               loss_fn="softmax" if softmax else "logsigmoid",
+               softmax_correction_weight=1.0 if softmax else 0.0,
+               shared_table=True, gamma=m.gamma, loss_scale=settings.training.loss_scale,
+               scoring_bf16=settings.execution.scoring_dtype == "bfloat16",
+               storage="bfloat16_embedding" if w.get("embedding_dtype") == "bfloat16" else "float32")
+    return cfg, state
+
+
+def cpu_baseline(engine, settings, w, batch, n_check, n_cpu_steps):
+    """Times the sequential float32 oracle on the first `n_cpu_steps` steps of
+    the workload, starting from the device's own initial rows.  The first
+    `n_check` of them are run as a separate call so that their mean loss can be
+    compared with the GPU's.  Returns (json object, loss of the first call)."""
+    from oracle.kge_oracle import Oracle, make_cfg
+
+    m, d = settings.model, settings.data
+    sub = {k: np.ascontiguousarray(v[:, :n_cpu_steps]) for k, v in vars(batch).items()}
+    cfg, state = cpu_start_state(engine, settings, w, sub)
+    cfg = make_cfg(**cfg)
     oracle = Oracle("f32")
     lr = settings.training.learning_rate
     t0 = time.perf_counter()
@@ -183,6 +193,47 @@ def cpu_baseline(engine, settings, w, batch, n_check, n_cpu_steps):
     return dict(value=triples / dt, unit="triples/s", cores=1, kind="port",
                 sample=f"{n_cpu_steps} step(s) of the same workload ({triples} triples) in {dt:.1f} s, "
                        f"sequential float32 C oracle, 1 thread of {os.cpu_count()} host cpus"), loss
+
+
+def cpu_torch_prepare(engine, settings, w, batch, n_max, threads):
+    """The reference's PyTorch CPU path (oracle/torch_demo_step.py: fancy-index gather,
+    torch.cdist, autograd, the reference's Adam on the gathered rows) set up on the device's own
+    initial rows for the first `n_max` steps of the workload; None for a workload that path does
+    not cover.  Called before the device runs a step; timed by cpu_torch_run after the device's
+    timed regions, because its worker threads would compete with the thread that launches kernels."""
+    from oracle.torch_demo_step import TorchDemoStep
+
+    sub = {k: np.ascontiguousarray(v[:, :n_max]) for k, v in vars(batch).items()}
+    cfg, state = cpu_start_state(engine, settings, w, sub)
+    try:
+        return TorchDemoStep(cfg, state, threads=threads), sub, threads
+    except ValueError:
+        return None
+
+
+def cpu_torch_run(prepared, settings, n_check, budget_s=10.0):
+    """One untimed step to start the thread pool, then steps until `budget_s` seconds have gone
+    (at most the prepared ones).  Returns (json object, mean loss of the first n_check steps)."""
+    path, sub, threads = prepared
+    m, d = settings.model, settings.data
+    lr = settings.training.learning_rate
+    losses, dt, n = [], 0.0, 0
+    for i in range(sub["remote"].shape[1]):
+        t0 = time.perf_counter()
+        losses.append(path.step(lr, {k: v[:, i] for k, v in sub.items()}))
+        if i > 0:
+            dt += time.perf_counter() - t0
+            n += 1
+        if dt > budget_s:
+            break
+    if n == 0:
+        return None, None
+    triples = n * m.n_shard * d.batch_size
+    loss = np.mean(losses[:n_check], axis=0) if len(losses) >= n_check else None
+    return dict(value=triples / dt, unit="triples/s", cores=threads, kind="port",
+                sample=f"{n} step(s) of the same workload ({triples} triples) in {dt:.1f} s after one "
+                       f"untimed step, float32 PyTorch demo path, {threads} threads of "
+                       f"{os.cpu_count()} host cpus"), loss
 
 
 def split_forward(w):
@@ -294,6 +345,9 @@ def main():
     n_cpu = min(n_cpu, n_total)
     n_check = max(1, min(n_cpu, args.warmup))
     cpu, cpu_loss = (None, None) if args.no_cpu else cpu_baseline(engine, settings, w, batch, n_check, n_cpu)
+    # the worker threads this process may use: the host's share for one GPU, not the node's core count
+    threads = int(os.environ.get("OMP_NUM_THREADS") or min(16, os.cpu_count()))
+    torch_path = None if args.no_cpu else cpu_torch_prepare(engine, settings, w, batch, n_total, threads)
 
     # warm-up: W untimed steps; the first n_cpu of them double as the parity check
     check = None
@@ -352,6 +406,13 @@ def main():
     torch.cuda.synchronize()
     dt_host = (time.perf_counter() - t1) / n_total
 
+    # the multi-threaded CPU path last: nothing of the device is timed after it
+    cpu_torch, cpu_torch_loss = cpu_torch_run(torch_path, settings, n_check) if torch_path else (None, None)
+    if check is not None and cpu_torch_loss is not None:
+        check["cpu_torch_loss"] = float(np.sum(cpu_torch_loss))
+        check["cpu_torch_rel_err"] = (abs(check["gpu_loss"] - check["cpu_torch_loss"])
+                                      / abs(check["cpu_torch_loss"]))
+
     triples = args.steps * m.n_shard * d.batch_size
     roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get((args.workload, dominant))
     U = float(np.mean(uniq_rows))
@@ -391,6 +452,7 @@ def main():
                          "note": f"one call over {n_total} steps, index arrays uploaded from host "
                                  "memory inside the timed call"},
         "cpu_baseline": cpu,
+        "cpu_baseline_torch": cpu_torch,
         "check": check,
     }
     def plain(o):  # numpy scalars -> Python numbers
