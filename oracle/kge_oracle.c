@@ -39,7 +39,7 @@
 
 #define API __attribute__((visibility("default")))
 
-enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2, SCORE_ROTATE = 3 };
+enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2, SCORE_ROTATE = 3, SCORE_TRANSH = 4 };
 enum { DIST_L1 = 0, DIST_L2 = 1, DIST_DOT = 2 };
 enum { LOSS_LOGSIGMOID = 0, LOSS_SOFTMAX = 1 };
 enum { STORE_F32 = 0, STORE_F16 = 1, STORE_BF16_EMB = 2 };
@@ -454,6 +454,10 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
     /* RotatE's relation rows are D / 2 phases (poplar_kge.cpp:248-249) */
     const int64_t RD = c->score_fn == SCORE_ROTATE ? D / 2 : D;
     const int64_t NE = c->n_entity;
+    /* TransH (poplar_kge.cpp:252-255): `rel` and its moments hold 2 * NREL rows, the
+     * relation embeddings followed by the hyperplane normals (relation_normal)       */
+    const int transh = c->score_fn == SCORE_TRANSH;
+    const int64_t NRELT = transh ? 2 * NREL : NREL;
 #define KEY(s, slot) ((c->shared_table ? 0 : (int64_t)(s) * NE) + (int64_t)remote[(s) * NR + (slot)])
 
     /* 1. gather + hidden = emb + feature * W  (:405-410, :439-467) */
@@ -509,7 +513,11 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
         free(fh); free(val);
     }
 
-    REAL* grel = (REAL*)calloc((size_t)(NREL * RD), sizeof(REAL));
+    REAL* grel = (REAL*)calloc((size_t)(NRELT * RD), sizeof(REAL));
+    /* TransH: unit normals of the positives, their gradient, norms of the raw normals */
+    REAL* nv = transh ? (REAL*)malloc(sizeof(REAL) * (size_t)(B * D)) : NULL;
+    REAL* dnv = transh ? (REAL*)malloc(sizeof(REAL) * (size_t)(B * D)) : NULL;
+    REAL* nrm = transh ? (REAL*)malloc(sizeof(REAL) * (size_t)B) : NULL;
     REAL* p = (REAL*)malloc(sizeof(REAL) * (size_t)(B * D));
     REAL* tl = (REAL*)malloc(sizeof(REAL) * (size_t)(T * D));
     REAL* score = (REAL*)malloc(sizeof(REAL) * (size_t)(B * T));
@@ -533,6 +541,18 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                     p[b * D + k] = h[k] * cs - h[k + H] * sn;
                     p[b * D + k + H] = h[k + H] * cs + h[k] * sn;
                 }
+                continue;
+            }
+            if (transh) {
+                /* transHPredict (:539-549): unit normal, head projected onto the hyperplane,
+                 * plus the relation embedding; the normal travels on to the score */
+                const float* w = rel + (NREL + (int64_t)relation[d * B + b]) * D;
+                REAL ss = 0, a = 0;
+                for (int64_t k = 0; k < D; ++k) ss += (REAL)w[k] * (REAL)w[k];
+                nrm[b] = (REAL)sqrt((double)ss);
+                for (int64_t k = 0; k < D; ++k) nv[b * D + k] = (REAL)w[k] / nrm[b];
+                for (int64_t k = 0; k < D; ++k) a += nv[b * D + k] * h[k];
+                for (int64_t k = 0; k < D; ++k) p[b * D + k] = (h[k] - nv[b * D + k] * a) + (REAL)r[k];
                 continue;
             }
             if (c->score_fn == SCORE_COMPLEX) {
@@ -565,7 +585,14 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             for (int64_t t = 0; t < T; ++t) {
                 REAL acc = 0;
                 const REAL *x = p + b * D, *y = tl + t * D;
-                if (dot)
+                if (transh) {
+                    /* transHScore (:551-565): tails projected onto the positive's hyperplane,
+                     * L1 distance whatever distance_fn says */
+                    const REAL* n = nv + b * D;
+                    REAL cn = 0;
+                    for (int64_t k = 0; k < D; ++k) cn += n[k] * y[k];
+                    for (int64_t k = 0; k < D; ++k) acc += (REAL)fabs((double)(x[k] - (y[k] - n[k] * cn)));
+                } else if (dot)
                     for (int64_t k = 0; k < D; ++k) acc += x[k] * y[k];
                 else if (c->distance_fn == DIST_L1)
                     for (int64_t k = 0; k < D; ++k) acc += (REAL)fabs((double)(x[k] - y[k]));
@@ -589,12 +616,33 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
         /* 5. backward through the score into p and tails */
         memset(dp, 0, sizeof(REAL) * (size_t)(B * D));
         memset(dtl, 0, sizeof(REAL) * (size_t)(T * D));
+        if (transh) memset(dnv, 0, sizeof(REAL) * (size_t)(B * D));
         for (int64_t b = 0; b < B; ++b)
             for (int64_t t = 0; t < T; ++t) {
                 const REAL *x = p + b * D, *y = tl + t * D;
                 REAL* gx = dp + b * D;
                 REAL* gy = dtl + t * D;
                 REAL g = dscore[b * T + t];
+                if (transh) {
+                    /* e = p - (tail - n c), c = n . tail: abs, sub, mul, matMul backward in turn */
+                    const REAL* n = nv + b * D;
+                    REAL* gn = dnv + b * D;
+                    REAL cn = 0, gc = 0;
+                    g = -g;
+                    for (int64_t k = 0; k < D; ++k) cn += n[k] * y[k];
+                    for (int64_t k = 0; k < D; ++k) {
+                        const REAL u = g * signum(x[k] - (y[k] - n[k] * cn));
+                        gx[k] += u;         /* predicted tail */
+                        gy[k] -= u;         /* projected tail -> tail */
+                        gn[k] += u * cn;    /* projected tail -> normal * c */
+                        gc += u * n[k];     /* ... -> c */
+                    }
+                    for (int64_t k = 0; k < D; ++k) {
+                        gn[k] += gc * y[k];
+                        gy[k] += gc * n[k];
+                    }
+                    continue;
+                }
                 if (c->score_fn == SCORE_DISTMULT) { /* pag.cpp:685-700 */
                     for (int64_t k = 0; k < D; ++k) {
                         gx[k] += g * y[k];
@@ -631,6 +679,21 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             REAL* gh = ghid + (d * NR + head[d * B + b]) * D;
             const REAL* h = hidden + (d * NR + head[d * B + b]) * D;
             const int64_t r = relation[d * B + b];
+            if (transh) {
+                /* p = h - n (n . h) + rel;  n = w / |w| */
+                const REAL *n = nv + b * D, *gp = dp + b * D;
+                REAL* gn = dnv + b * D;
+                REAL a = 0, sgn = 0, ngn = 0;
+                for (int64_t k = 0; k < D; ++k) { a += n[k] * h[k]; sgn += gp[k] * n[k]; }
+                for (int64_t k = 0; k < D; ++k) {
+                    gh[k] += gp[k] - n[k] * sgn;
+                    grel[r * D + k] += gp[k];
+                    gn[k] += -a * gp[k] - h[k] * sgn;
+                }
+                for (int64_t k = 0; k < D; ++k) ngn += n[k] * gn[k];
+                for (int64_t k = 0; k < D; ++k) grel[(NREL + r) * D + k] += (gn[k] - n[k] * ngn) / nrm[b];
+                continue;
+            }
             if (c->score_fn == SCORE_ROTATE) {
                 /* p_re = h_re cos - h_im sin, p_im = h_im cos + h_re sin.  The gradient of the
                  * phase runs in float16 as the forward does (cast's backward casts the gradient,
@@ -752,9 +815,9 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
      * shard s owns rows [s*n/S, (s+1)*n/S) of each parameter (:290-304)     */
     {
         float* gf = (float*)malloc(sizeof(float) * (size_t)D);
-        for (int64_t r = 0; r < NREL; ++r) {
+        for (int64_t r = 0; r < NRELT; ++r) {
             for (int64_t k = 0; k < RD; ++k) gf[k] = (float)grel[r * RD + k];
-            const int64_t shard = c->shared_table ? 0 : r / (NREL / S);
+            const int64_t shard = c->shared_table ? 0 : (r % NREL) / (NREL / S);
             kge_oracle_adam(rel + r * RD, rel_m + r * RD, rel_v + r * RD, gf, RD,
                             alpha[shard] * c->lr_mod_relation, c->beta_m, c->beta_v, c->epsilon,
                             c->weight_decay, 0);
@@ -772,6 +835,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
     free(greg_val); free(greg_fh); free(reg_loss);
     free(hidden); free(ghid); free(grel); free(p); free(tl); free(score); free(dist);
     free(dscore); free(dp); free(dtl); free(alpha); free(gproj);
+    free(nv); free(dnv); free(nrm);
     return 0;
 }
 

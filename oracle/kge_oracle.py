@@ -14,7 +14,7 @@ import numpy as np
 
 HERE = Path(__file__).resolve().parent
 
-SCORE = {"TransE": 0, "DistMult": 1, "ComplEx": 2, "RotatE": 3}
+SCORE = {"TransE": 0, "DistMult": 1, "ComplEx": 2, "RotatE": 3, "TransH": 4}
 DIST = {"L1": 0, "L2": 1, "MatMul": 2}
 LOSS = {"logsigmoid": 0, "softmax": 1}
 STORE = {"float32": 0, "float16": 1, "bfloat16_embedding": 2}
@@ -245,12 +245,24 @@ class Oracle:
             proj = [None, None, None]
         step = C.c_uint32(int(state["step"]))
         loss = np.zeros(S, np.float32)
+        suffixes = ("", "/adam_m", "/adam_v")
+        if cfg.score_fn == SCORE["TransH"]:
+            # the C side takes the hyperplane normals as rows [n_relation, 2 n_relation) of the
+            # relation arrays
+            rel = [np.concatenate([_f32(state["relation_embedding" + x]), _f32(state["relation_normal" + x])])
+                   for x in suffixes]
+        else:
+            rel = [state["relation_embedding" + x] for x in suffixes]
         rc = self.lib.kge_oracle_train_step_loop(
             C.byref(cfg), C.c_int32(n_step), _p(state["entity_data"]),
-            _p(state["relation_embedding"]), _p(state["relation_embedding/adam_m"]),
-            _p(state["relation_embedding/adam_v"]), *proj, C.byref(step), _p(lr), _p(remote),
+            _p(rel[0]), _p(rel[1]), _p(rel[2]), *proj, C.byref(step), _p(lr), _p(remote),
             _p(a2a), _p(head), _p(relation), _p(tail), _p(loss))
         assert rc == 0
+        if cfg.score_fn == SCORE["TransH"]:
+            n = cfg.n_relation
+            for x, a in zip(suffixes, rel):
+                state["relation_embedding" + x][...] = a[:n]
+                state["relation_normal" + x][...] = a[n:]
         state["step"] = step.value
         return loss
 
@@ -283,15 +295,22 @@ def predict_reference(cfg, state, queries, shard_to_count, n_best):
         H = D // 2
         p = np.concatenate([h[:, :H] * r[:, :H] - h[:, H:] * r[:, H:],
                             h[:, :H] * r[:, H:] + h[:, H:] * r[:, :H]], axis=1)
+    elif cfg.score_fn == SCORE["TransH"]:  # src/poplar_kge.cpp:539-565
+        w = np.asarray(state["relation_normal"], np.float64)[q[:, 2]]
+        n = w / np.sqrt((w * w).sum(-1, keepdims=True))
+        p = h - n * (n * h).sum(-1, keepdims=True) + r
     else:
         p = h * r if cfg.score_fn == SCORE["DistMult"] else h + r
-    if dot:
+    if cfg.score_fn == SCORE["TransH"]:
+        dist = np.stack([np.abs(x[None, :] - (hidden - nn[None, :] * (hidden @ nn)[:, None])).sum(-1)
+                         for x, nn in zip(p, n)])
+    elif dot:
         dist = p @ hidden.T
     elif cfg.distance_fn == DIST["L1"]:
         dist = np.stack([np.abs(x[None, :] - hidden).sum(-1) for x in p])
     else:
         dist = np.stack([np.sqrt(((x[None, :] - hidden) ** 2).sum(-1)) for x in p])
-    score = cfg.gamma - dist if cfg.score_fn in (SCORE["TransE"], SCORE["RotatE"]) else dist
+    score = cfg.gamma - dist if cfg.score_fn in (SCORE["TransE"], SCORE["RotatE"], SCORE["TransH"]) else dist
     live = np.zeros((S, NE), bool)
     for s, n in enumerate(shard_to_count):
         live[s, 1:1 + int(n)] = True

@@ -41,6 +41,10 @@ def make_state(c, rng, warm=True, scale=None):
         "relation_embedding/adam_v": ((0.05 + np.abs(rng.normal(0, 0.3, (NR, RD))))**2 * warm).astype(np.float32),
         "step": 7 if warm else 0,
     }
+    if c["score_fn"] == "TransH":
+        st["relation_normal"] = rng.normal(0, scale, (NR, D)).astype(np.float32)
+        st["relation_normal/adam_m"] = (rng.normal(0, 0.1, (NR, D)) * warm).astype(np.float32)
+        st["relation_normal/adam_v"] = ((0.05 + np.abs(rng.normal(0, 0.3, (NR, D))))**2 * warm).astype(np.float32)
     if F:
         st["feature_projection"] = rng.normal(0, scale / np.sqrt(F), (F, D)).astype(np.float32)
         st["feature_projection/adam_m"] = (rng.normal(0, 0.1, (F, D)) * warm).astype(np.float32)

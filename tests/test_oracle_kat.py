@@ -303,6 +303,13 @@ STEP_CASES = {
     "rotate_l2_feat": dict(score_fn="RotatE", distance_fn="L2", gamma=4.0),
     "rotate_softmax": dict(score_fn="RotatE", distance_fn="L1", loss_fn="softmax", softmax_correction_weight=1.0,
                            feature=0, dim=12),
+    # TransH (src/poplar_kge.cpp:539-565): heads and tails projected onto the relation's
+    # hyperplane (unit normal from relation_normal), L1 distance whatever distance_fn says
+    "transh": dict(score_fn="TransH", feature=0),
+    "transh_feat_softmax": dict(score_fn="TransH", distance_fn="L2", loss_fn="softmax",
+                                softmax_correction_weight=1.0),
+    "transh_shared_table": dict(score_fn="TransH", shared_table=True, n_shard=4, batch=8, a2a=4,
+                                feature=0, n_entity=60, gamma=3.0),
     # norm regularisers (src/poplar_kge.cpp:430-437, 463-465), the WikiKG preset's among them
     "feature_regularisation_p3": dict(feature_regularisation=(3.0, 1e-2), loss_fn="softmax",
                                       softmax_correction_weight=1.0),
@@ -488,3 +495,36 @@ def test_predict_reference_vs_torch_topk():
         top = T.topk(sc + mask.reshape(-1), k=7)
         np.testing.assert_allclose(score, top.values.numpy(), rtol=1e-12, atol=1e-12)
         np.testing.assert_array_equal(idx[..., 0] * NE + idx[..., 1], top.indices.numpy())
+
+
+def test_predict_reference_transh_by_hand_and_invariances():
+    # D = 2, normal along x (any length): heads and tails lose their x part, so the score is
+    # gamma - (|r_x| + |h_y + r_y - t_y|) with r's own x part surviving (src/poplar_kge.cpp:539-565)
+    from oracle.kge_oracle import predict_reference
+
+    cfg = make_cfg(n_shard=1, n_entity=4, n_relation=1, dim=2, feature=0, batch=1, a2a=1, gamma=10.0,
+                   score_fn="TransH")
+    rows = np.zeros((4, 6), np.float32)
+    rows[:, :2] = [[0, 0], [5.0, 1.0], [-7.0, 2.5], [100.0, 0.0]]
+    state = {"entity_data": rows, "relation_embedding": np.array([[0.25, 1.0]], np.float32),
+             "relation_normal": np.array([[3.0, 0.0]], np.float32)}
+    idx, score = predict_reference(cfg, state, np.array([[0, 1, 0]]), [3], 3)
+    # h = (5, 1): projected (0, 1), + r = (0.25, 2); tails projected (0, 1), (0, 2.5), (0, 0)
+    np.testing.assert_allclose(score[0], [10 - 0.75, 10 - 1.25, 10 - 2.25])
+    np.testing.assert_array_equal(idx[0], [[0, 2], [0, 1], [0, 3]])
+    # invariances on random data: the length of the raw normal, and any multiple of the normal
+    # added to an entity, leave every score as it is
+    rng = np.random.default_rng(3)
+    NE, D, NR = 30, 6, 4
+    cfg = make_cfg(n_shard=1, n_entity=NE, n_relation=NR, dim=D, feature=0, batch=1, a2a=1, gamma=2.0,
+                   score_fn="TransH")
+    st = {"entity_data": rng.normal(size=(NE, 3 * D)).astype(np.float32),
+          "relation_embedding": rng.normal(size=(NR, D)).astype(np.float32),
+          "relation_normal": rng.normal(size=(NR, D)).astype(np.float32)}
+    q = np.stack([np.zeros(5, int), rng.integers(1, NE, 5), np.full(5, 2)], -1)
+    idx0, score0 = predict_reference(cfg, st, q, [NE - 1], NE - 1)
+    st2 = {k: v.copy() for k, v in st.items()}
+    st2["relation_normal"][2] *= 4.0
+    st2["entity_data"][1:, :D] += rng.normal(size=(NE - 1, 1)).astype(np.float32) * st["relation_normal"][2]
+    idx1, score1 = predict_reference(cfg, st2, q, [NE - 1], NE - 1)
+    np.testing.assert_allclose(score1, score0, rtol=0, atol=2e-5)

@@ -90,6 +90,9 @@ def step(cfg, state, lr, batch_step):
     feat = table[uniq, 3 * D:]
     rel = T.tensor(state["relation_embedding"].astype(np.float64), requires_grad=True)
     params = [emb, rel]
+    if cfg["score_fn"] == "TransH":
+        normal = T.tensor(state["relation_normal"].astype(np.float64), requires_grad=True)
+        params.append(normal)
     if F:
         proj = T.tensor(state["feature_projection"].astype(np.float64), requires_grad=True)
         params.append(proj)
@@ -114,7 +117,16 @@ def step(cfg, state, lr, batch_step):
     tails = hidden[shards[:, None, None], a2a]  # [S(src), S(dst), A, D]
     tails = tails.transpose(0, 1).reshape(S, Tn, D)  # all-to-all
     r = rel[relation]
-    if cfg["score_fn"] in ("TransE", "ComplEx", "RotatE"):
+    if cfg["score_fn"] == "TransH":
+        # src/poplar_kge.cpp:539-565 as written there: unit normal, head and tails projected
+        # onto the relation's hyperplane, L1 distance
+        n = normal[relation]
+        n = n / T.sqrt((n * n).sum(-1, keepdim=True))
+        pred = heads - n * (n * heads).sum(-1, keepdim=True) + r
+        tails_norm = n @ tails.transpose(1, 2)  # [S, B, T]
+        projected = tails[:, None, :, :] - n[:, :, None, :] * tails_norm[..., None]
+        score = cfg["gamma"] - (pred[:, :, None, :] - projected).abs().sum(-1)
+    elif cfg["score_fn"] in ("TransE", "ComplEx", "RotatE"):
         if cfg["score_fn"] == "RotatE":
             # the phases, their sine and cosine and the phases' gradient in float16 (torch's own
             # float16 kernels and autograd), the rotation in float64
@@ -200,6 +212,8 @@ def step(cfg, state, lr, batch_step):
         state[name + "/adam_v"][...] = v
 
     dense("relation_embedding", rel.grad.numpy())
+    if cfg["score_fn"] == "TransH":
+        dense("relation_normal", normal.grad.numpy())
     if F:
         dense("feature_projection", proj.grad.numpy())
     return per_shard.detach().numpy().astype(np.float32)
