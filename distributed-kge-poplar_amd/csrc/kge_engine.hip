@@ -185,10 +185,13 @@ struct Variable {
 struct kge_engine {
     // ---- settings (src/poplar_kge.cpp:198-236) ----
     int S, n_entity, n_rel, D, F, B, A, T, NR, R;
+    // TransH keeps a second row per relation, the hyperplane normal (relation_normal), as rows
+    // [n_rel, 2 n_rel) of the relation table: rel_copies = 2, n_rel_rows = 2 n_rel
+    int rel_copies = 1, n_rel_rows = 0;
     int score_fn, dist_fn, loss_fn;
     bool shared_table;
     float gamma, init_scale, beta_m, beta_v, epsilon, weight_decay, loss_scale, softmax_cw, neg_adv;
-    float lr_mod_entity = 1.f, lr_mod_rel = 1.f, lr_mod_proj = 1.f;
+    float lr_mod_entity = 1.f, lr_mod_rel = 1.f, lr_mod_proj = 1.f, lr_mod_normal = 1.f;
     uint32_t seed;
     int n_step, rw_batch;
     int predict_hr_batch = 0, predict_n_best = 0;
@@ -232,8 +235,12 @@ struct kge_engine {
     float reg_p[3] = {3.f, 3.f, 3.f}, reg_w[3] = {0.f, 0.f, 0.f};
     bool reg_on = false;
     DevBuf<float> reg_val, reg_fh, reg_loss_row, reg_loss_part;
+    DevBuf<float> opnd_n, cmat, dcm, transh_mm, relgrad;  // TransH: [n | tails], c, d loss / d c, its products, relation contributions
     DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, d_loss, d_alpha;
-    std::vector<float> h_alpha;  // [n_step][entity, relation, projection][S]
+    // [n_step][entity, relation, normal, projection][S]; the relation update indexes its two
+    // groups as one array (key / rows_per_alpha), a shared table's [relation, normal] pair
+    // sits in the first two entries of the relation group
+    std::vector<float> h_alpha;
     int n_part;
     // io staging
     DevBuf<uint64_t> io_rows;
@@ -256,6 +263,12 @@ struct kge_engine {
 };
 
 namespace {
+
+// DistMult, ComplEx and RotatE form a row's gradient contributions from rows of the other
+// table when they are summed (TransE's and TransH's are materialised before that)
+bool contributions_read_tables(const kge_engine& E) {
+    return E.score_fn == SCORE_DISTMULT || E.score_fn == SCORE_COMPLEX || E.score_fn == SCORE_ROTATE;
+}
 
 void parse_settings(kge_engine& E, const Items& s) {
     // the device: this library only drives a HIP device
@@ -348,9 +361,7 @@ void parse_settings(kge_engine& E, const Items& s) {
     else if (score == "DistMult") E.score_fn = SCORE_DISTMULT;
     else if (score == "ComplEx") E.score_fn = SCORE_COMPLEX;
     else if (score == "RotatE") E.score_fn = SCORE_ROTATE;
-    else if (score == "TransH")
-        throw std::invalid_argument("'model.score_fn' = '" + score + "' is not implemented on the HIP device "
-                                    "(supported: 'TransE', 'DistMult', 'ComplEx', 'RotatE')");
+    else if (score == "TransH") E.score_fn = SCORE_TRANSH;
     else
         throw std::invalid_argument("'model.score_fn' must be one of 'TransE', 'ComplEx', 'RotatE', 'TransH', or "
                                     "'DistMult', not '" + score + "'");
@@ -362,6 +373,11 @@ void parse_settings(kge_engine& E, const Items& s) {
         throw std::invalid_argument("'model.distance_fn' must be one of 'L1', 'L2' or 'MatMul', not '" +
                                     distance + "'");
     if (E.score_fn == SCORE_DISTMULT) E.dist_fn = DIST_DOT;  // distMultScore ignores the setting (:571-573)
+    if (E.score_fn == SCORE_TRANSH) {  // so does transHScore: always the L1 norm (:563-564)
+        E.dist_fn = DIST_L1;
+        E.rel_copies = 2;
+        if (E.score_bf16) throw std::invalid_argument("'execution.scoring_dtype' = 'bfloat16' is not implemented for TransH");
+    }
     if ((E.score_fn == SCORE_COMPLEX || E.score_fn == SCORE_ROTATE) && E.D % 2)
         throw std::invalid_argument("'model.score_fn' = '" + score + "' needs an even 'model.embedding_size' "
                                     "(real and imaginary halves)");
@@ -398,11 +414,13 @@ void parse_settings(kge_engine& E, const Items& s) {
         check("relation_embedding", E.n_rel, E.score_fn == SCORE_ROTATE ? E.D / 2 : E.D);
         check("feature_projection", E.F, E.D);
     }
+    E.n_rel_rows = E.n_rel * E.rel_copies;
     for (size_t i = 0; i < mods.map_len; ++i) {
         const std::string k = mods.map_keys[i];
         if (k == "entity_embedding") E.lr_mod_entity = mods.map_vals[i];
         else if (k == "relation_embedding") E.lr_mod_rel = mods.map_vals[i];
         else if (k == "feature_projection") E.lr_mod_proj = mods.map_vals[i];
+        else if (k == "relation_normal" && E.score_fn == SCORE_TRANSH) E.lr_mod_normal = mods.map_vals[i];
         else
             throw std::invalid_argument("Bad training.learning_rate_modifier: unknown parameter '" + k + "'");
     }
@@ -432,6 +450,8 @@ void parse_settings(kge_engine& E, const Items& s) {
         // full pitch, their upper half stays zero
         var(std::string("relation_embedding") + suffix,
             {(size_t)E.n_rel, (size_t)(E.score_fn == SCORE_ROTATE ? E.D / 2 : E.D)});
+        if (E.score_fn == SCORE_TRANSH)  // :252-255
+            var(std::string("relation_normal") + suffix, {(size_t)E.n_rel, (size_t)E.D});
         var(std::string("feature_projection") + suffix, {(size_t)E.F, (size_t)E.D});
     }
 }
@@ -450,7 +470,7 @@ void allocate(kge_engine& E) {
 
     E.table.alloc((size_t)E.n_rows * E.L.pitch);
     E.table.zero(st);
-    const size_t rel_n = (size_t)E.n_rel * E.Dp, proj_n = (size_t)E.Fp * E.Dp;
+    const size_t rel_n = (size_t)E.n_rel_rows * E.Dp, proj_n = (size_t)E.Fp * E.Dp;
     for (DevBuf<float>* b : {&E.rel, &E.rel_m, &E.rel_v}) { b->alloc(rel_n); b->zero(st); }
     for (DevBuf<float>* b : {&E.proj, &E.proj_m, &E.proj_v}) { b->alloc(proj_n); b->zero(st); }
 
@@ -465,7 +485,7 @@ void allocate(kge_engine& E) {
     E.crel.alloc(ns * SB);
     E.clabel.alloc(ns * SB);
     for (DevBuf<uint32_t>* b : {&E.ek_a, &E.ev_a, &E.ek_b, &E.ev_b}) b->alloc(ns * 2 * R);
-    E.n_rel_items = (int)(SB + E.n_rel);
+    E.n_rel_items = (int)((SB + E.n_rel) * E.rel_copies);
     for (DevBuf<uint32_t>* b : {&E.rk_a, &E.rv_a, &E.rk_b, &E.rv_b}) b->alloc(ns * E.n_rel_items);
     const size_t tiles = (std::max<size_t>(2 * R, E.n_rel_items) + kSortTile - 1) / kSortTile;
     E.hist.alloc(ns * 256 * tiles);
@@ -480,8 +500,8 @@ void allocate(kge_engine& E) {
     E.e_clen.alloc(ns * E.e_cstride);
     E.e_counts.alloc(ns * 2);
     if (E.F) E.e_item_row.alloc(ns * R);
-    E.r_ustride = E.n_rel;
-    E.r_cstride = (int)(SB / std::min(E.chunk, E.direct_max + 1) + 2);
+    E.r_ustride = E.n_rel_rows;
+    E.r_cstride = (int)(SB * E.rel_copies / std::min(E.chunk, E.direct_max + 1) + 2);
     E.r_real.alloc(ns * E.r_ustride);
     E.r_uniq.alloc(ns * E.r_ustride);
     E.r_seg.alloc(ns * (E.r_ustride + 1));
@@ -507,7 +527,14 @@ void allocate(kge_engine& E) {
     E.opnd.alloc(R * E.Dp);
     E.partial.alloc((size_t)E.e_cstride * E.Dp);
     E.rel_partial.alloc((size_t)E.r_cstride * E.Dp);
-    if (E.score_fn != SCORE_TRANSE) E.rel_gsum.alloc((size_t)E.n_rel * E.Dp);
+    if (contributions_read_tables(E)) E.rel_gsum.alloc((size_t)E.n_rel * E.Dp);
+    if (E.score_fn == SCORE_TRANSH) {
+        E.opnd_n.alloc(R * E.Dp);
+        E.transh_mm.alloc(R * E.Dp);
+        E.cmat.alloc(SB * E.T);
+        E.dcm.alloc(SB * E.T);
+        E.relgrad.alloc(2 * SB * E.Dp);
+    }
     if (E.F) {
         E.hidden.alloc(R * E.Dp);
         E.gsum.alloc(R * E.Dp);
@@ -539,7 +566,7 @@ void allocate(kge_engine& E) {
     }
     E.loss_part.alloc(ns * S * E.n_part);
     E.d_loss.alloc(S);
-    E.d_alpha.alloc(ns * 3 * S);
+    E.d_alpha.alloc(ns * 4 * S);
 
     const size_t io_n = (size_t)E.S * E.rw_batch;
     E.io_rows.alloc(io_n);
@@ -563,9 +590,13 @@ void run_read_write(kge_engine& E, bool write, const Items& in) {
     }
     float* host = (float*)in.array("value", KGE_F32, var->shape);
     DevBuf<float>* buf = nullptr;
+    size_t row0 = 0;  // first device row of the variable
     if (name == "relation_embedding") buf = &E.rel;
     else if (name == "relation_embedding/adam_m") buf = &E.rel_m;
     else if (name == "relation_embedding/adam_v") buf = &E.rel_v;
+    else if (name == "relation_normal") { buf = &E.rel; row0 = E.n_rel; }
+    else if (name == "relation_normal/adam_m") { buf = &E.rel_m; row0 = E.n_rel; }
+    else if (name == "relation_normal/adam_v") { buf = &E.rel_v; row0 = E.n_rel; }
     else if (name == "feature_projection") buf = &E.proj;
     else if (name == "feature_projection/adam_m") buf = &E.proj_m;
     else if (name == "feature_projection/adam_v") buf = &E.proj_v;
@@ -573,9 +604,9 @@ void run_read_write(kge_engine& E, bool write, const Items& in) {
     if (rows == 0 || cols == 0) return;
     HIP_CHECK(hipStreamSynchronize(E.stream));
     if (write)
-        HIP_CHECK(hipMemcpy2D(buf->p, (size_t)E.Dp * 4, host, cols * 4, cols * 4, rows, hipMemcpyHostToDevice));
+        HIP_CHECK(hipMemcpy2D(buf->p + row0 * E.Dp, (size_t)E.Dp * 4, host, cols * 4, cols * 4, rows, hipMemcpyHostToDevice));
     else
-        HIP_CHECK(hipMemcpy2D(host, cols * 4, buf->p, (size_t)E.Dp * 4, cols * 4, rows, hipMemcpyDeviceToHost));
+        HIP_CHECK(hipMemcpy2D(host, cols * 4, buf->p + row0 * E.Dp, (size_t)E.Dp * 4, cols * 4, rows, hipMemcpyDeviceToHost));
 }
 
 // ---- entity rows: "write_entity", "read_entity" (:857-871) --------------------
@@ -724,11 +755,12 @@ void run_plan(kge_engine& E, int s0, int sn) {
     PlanShape ps;
     ps.n_step = E.n_step; ps.S = E.S; ps.B = E.B; ps.A = E.A; ps.NR = E.NR;
     ps.n_entity = E.n_entity; ps.shared_table = E.shared_table; ps.n_relation = E.n_rel;
+    ps.rel_copies = E.rel_copies;
     ps.step0 = s0; ps.step_count = sn;
     launch_build_items(ps, E.d_remote.p, E.d_a2a.p, E.d_head.p, E.d_relation.p, E.d_tail.p, E.ckey.p,
                        E.crel.p, E.clabel.p, E.ek_a.p, E.ev_a.p, E.rk_a.p, E.rv_a.p, st);
     const int ebits = std::max(1, bit_length((uint64_t)E.n_rows - 1));
-    const int rbits = std::max(1, bit_length((uint64_t)E.n_rel - 1));
+    const int rbits = std::max(1, bit_length((uint64_t)E.n_rel_rows - 1));
     int which = launch_radix_sort(E.ek_a.p + s0 * N, E.ev_a.p + s0 * N, E.ek_b.p + s0 * N, E.ev_b.p + s0 * N,
                                   E.hist.p, (int)N, sn, ebits, st);
     const uint32_t* ek = which ? E.ek_b.p : E.ek_a.p;
@@ -759,12 +791,13 @@ void run_plan(kge_engine& E, int s0, int sn) {
     rp.counts = E.r_counts.p + 2 * (size_t)s0;
     rp.item_row = nullptr;
     rp.seg_real = E.r_real.p + (size_t)s0 * rp.u_stride;
-    launch_find_segments(rk + s0 * NRI, E.r_sorted_vals + s0 * NRI, (int)NRI, (int)SB, E.chunk, E.direct_max, sn, rp, st);
+    launch_find_segments(rk + s0 * NRI, E.r_sorted_vals + s0 * NRI, (int)NRI, (int)SB * E.rel_copies, E.chunk, E.direct_max, sn, rp, st);
     HIP_CHECK(hipGetLastError());
 }
 
 // how the gather combines a head row with its relation row (launch_gather_operands)
 static int rel_mode_of(const kge_engine& E) {
+    if (E.score_fn == SCORE_TRANSH) return 0;  // launch_transh_predict turns the copied head rows into p
     return E.score_fn == SCORE_DISTMULT ? 2 : E.score_fn == SCORE_COMPLEX ? 3 : E.score_fn == SCORE_ROTATE ? 4 : 1;
 }
 
@@ -821,6 +854,14 @@ void run_step(kge_engine& E, int i) {
     dense.base = (const char*)E.opnd.p; dense.pitch = (int64_t)E.Dp * 4; dense.etype = ET_F32;
     dense.index = nullptr; dense.count = E.Dp; dense.vec = 1;
     sh.operands_dense = 1;
+    const bool transh = E.score_fn == SCORE_TRANSH;
+    if (transh) {
+        // second operand matrix [unit normals | tails]; the heads of the first become the
+        // predicted tails (transHPredict, src/poplar_kge.cpp:539-549)
+        KernelTimer t(E, K_GATHER);
+        HIP_CHECK(hipMemcpyAsync(E.opnd_n.p, E.opnd.p, R * E.Dp * 4, hipMemcpyDeviceToDevice, st));
+        launch_transh_predict(E.rel.p, crel, E.n_rel, (int)SB, E.Dp, E.opnd.p, E.opnd_n.p, st);
+    }
 
     float* loss_part = E.loss_part.p + (size_t)i * E.S * E.n_part;
     // bfloat16 dot-product scoring on the matrix cores: three batched products
@@ -857,6 +898,31 @@ void run_step(kge_engine& E, int i) {
           g.C = E.grad.p + head_n; g.ldc = Dp; g.c_batch = (int64_t)Tn * Dp;
           g.M = Tn; g.N = Dp; g.K = Bn;
           launch_gemm_nt_bf16(g, st); }
+    } else if (transh) {
+        // transHScore (:551-565): c = n . tail and its backward are dot-product scoring on
+        // [normals | tails]; the L1 part has kernels of its own
+        RowSource dense_n = dense;
+        dense_n.base = (const char*)E.opnd_n.p;
+        ScoreShape dot = sh;
+        dot.score_fn = SCORE_DISTMULT; dot.dist_fn = DIST_DOT;
+        { KernelTimer t(E, K_FWD);
+          launch_score_fwd(dot, dense_n, E.rel.p, crel, clabel, E.cmat.p, nullptr, nullptr, nullptr, false, st);
+          TranshFwd tf;
+          tf.sh = sh; tf.pt = E.opnd.p; tf.nt = E.opnd_n.p; tf.cmat = E.cmat.p; tf.clabel = clabel;
+          tf.coef = E.coef.p; tf.dcm = E.dcm.p; tf.loss_part = loss_part;
+          launch_transh_fwd(tf, fused, st); }
+        if (!fused) {
+            KernelTimer t(E, K_LOSS);
+            launch_loss_rows(sh, clabel, E.coef.p, nullptr, loss_part, nullptr, st);
+            launch_mul_rows(E.dcm.p, E.coef.p, (int64_t)SB * E.T, st);
+        }
+        { KernelTimer t(E, K_BWD);
+          launch_score_bwd(dot, dense_n, E.rel.p, crel, E.dcm.p, nullptr, E.transh_mm.p, st);
+          TranshBwd tb;
+          tb.pt = E.opnd.p; tb.nt = E.opnd_n.p; tb.coef = E.coef.p; tb.cmat = E.cmat.p;
+          tb.mm = E.transh_mm.p; tb.grad = E.grad.p; tb.S = E.S; tb.B = E.B; tb.T = E.T; tb.Dp = E.Dp;
+          launch_transh_bwd(tb, st);
+          launch_transh_back(ent, E.rel.p, crel, E.n_rel, (int)SB, E.Dp, E.grad.p, E.transh_mm.p, E.relgrad.p, st); }
     } else {
         { KernelTimer t(E, K_FWD);
           launch_score_fwd(sh, dense, E.rel.p, crel, clabel, E.coef.p, E.dist.p, E.nearflag.p, loss_part, fused, st); }
@@ -880,7 +946,7 @@ void run_step(kge_engine& E, int i) {
                         E.reg_loss_part.p + (size_t)i * E.S, st);
     }
 
-    const float* alpha = E.d_alpha.p + (size_t)i * 3 * E.S;
+    const float* alpha = E.d_alpha.p + (size_t)i * 4 * E.S;
     AdamArgs aa = {};
     aa.Dp = E.Dp;
     aa.beta_m = E.beta_m; aa.beta_v = E.beta_v;
@@ -891,12 +957,13 @@ void run_step(kge_engine& E, int i) {
     // come before both updates
     ContribSrc rsrc = {};
     rsrc.sorted_item = E.r_sorted_vals + (size_t)i * E.n_rel_items;
-    rsrc.grad = E.grad.p;
+    rsrc.grad = transh ? E.relgrad.p : E.grad.p;  // TransH: rows [0, SB) embedding, [SB, 2 SB) normal contributions
     rsrc.transform = E.score_fn == SCORE_DISTMULT ? 2 : E.score_fn == SCORE_COMPLEX ? 4 : E.score_fn == SCORE_ROTATE ? 6 : 0;
     rsrc.n_head = (int)SB; rsrc.half = E.D / 2;
     rsrc.rel = E.rel.p; rsrc.crel = crel; rsrc.ent = ent;
     ContribSrc esrc = rsrc;
     esrc.sorted_item = E.e_sorted_vals + (size_t)i * 2 * R;
+    esrc.grad = E.grad.p;
     esrc.transform = E.score_fn == SCORE_DISTMULT ? 1 : E.score_fn == SCORE_COMPLEX ? 3 : E.score_fn == SCORE_ROTATE ? 5 : 0;
 
     ReduceArgs rr = {};
@@ -924,12 +991,13 @@ void run_step(kge_engine& E, int i) {
     ar.seg_start = E.r_seg.p + (size_t)i * (E.r_ustride + 1);
     ar.seg_real = E.r_real.p + (size_t)i * E.r_ustride;
     ar.chunk_off = E.r_coff.p + (size_t)i * (E.r_ustride + 1);
-    ar.counts = r_counts; ar.max_rows = E.n_rel;
+    ar.counts = r_counts; ar.max_rows = E.n_rel_rows;
     ar.partial = E.rel_partial.p;
     ar.p_base = (char*)E.rel.p; ar.m_base = (char*)E.rel_m.p; ar.v_base = (char*)E.rel_v.p;
     ar.pitch = (int64_t)E.Dp * 4; ar.p_etype = ET_F32; ar.m_etype = ET_F32; ar.v_is_sqrt = 0;
     ar.alpha = alpha + E.S;
-    ar.rows_per_alpha = E.shared_table ? 0u : (uint32_t)(E.n_rel / E.S);
+    // the normal rows (keys >= n_rel) take the step sizes after the relation embedding's
+    ar.rows_per_alpha = E.shared_table ? (transh ? (uint32_t)E.n_rel : 0u) : (uint32_t)(E.n_rel / E.S);
 
     AdamArgs ae = aa;
     ae.src = esrc;
@@ -946,7 +1014,7 @@ void run_step(kge_engine& E, int i) {
     ae.alpha = alpha;
     ae.rows_per_alpha = E.shared_table ? 0u : (uint32_t)E.n_entity;
 
-    if (E.score_fn != SCORE_TRANSE) {
+    if (contributions_read_tables(E)) {
         // entity update first (reads pre-update relation rows), writing its summed
         // gradient is not needed; then the relation update reads POST-update entity
         // rows unless its gradient was materialised: do that with a zero-step pass
@@ -973,7 +1041,7 @@ void run_step(kge_engine& E, int i) {
             if (r1 <= r0) continue;
             const size_t o = (size_t)r0 * E.Dp;
             launch_adam_flat(E.proj.p + o, E.proj_m.p + o, E.proj_v.p + o, E.gproj.p + o,
-                             (int64_t)(r1 - r0) * E.Dp, E.h_alpha[((size_t)i * 3 + 2) * E.S + s],
+                             (int64_t)(r1 - r0) * E.Dp, E.h_alpha[((size_t)i * 4 + 3) * E.S + s],
                              E.beta_m, E.beta_v, E.epsilon, E.weight_decay, 0, st);
         }
     }
@@ -1008,16 +1076,21 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
         throw std::invalid_argument("train_step_loop with staged=true needs a preceding stage_batch");
     }
     // step sizes of every step of this call (adamStepSizeAutoIncrement, frnn.cpp:42-59)
-    E.h_alpha.resize((size_t)E.n_step * 3 * S);
+    E.h_alpha.resize((size_t)E.n_step * 4 * S);
     for (int i = s0; i < s0 + sn; ++i) {
         const double t = (double)(E.step + (uint32_t)(i - s0) + 1u);
         const double factor = std::sqrt(1.0 - std::pow((double)E.beta_v, t)) / (1.0 - std::pow((double)E.beta_m, t));
         for (size_t s = 0; s < S; ++s) {
             const float a = (float)(factor * (double)lr[s]);
-            E.h_alpha[((size_t)i * 3 + 0) * S + s] = a * E.lr_mod_entity;
-            E.h_alpha[((size_t)i * 3 + 1) * S + s] = a * E.lr_mod_rel;
-            E.h_alpha[((size_t)i * 3 + 2) * S + s] = a * E.lr_mod_proj;
+            E.h_alpha[((size_t)i * 4 + 0) * S + s] = a * E.lr_mod_entity;
+            E.h_alpha[((size_t)i * 4 + 1) * S + s] = a * E.lr_mod_rel;
+            E.h_alpha[((size_t)i * 4 + 2) * S + s] = a * E.lr_mod_normal;
+            E.h_alpha[((size_t)i * 4 + 3) * S + s] = a * E.lr_mod_proj;
         }
+        // a shared table has one step size per parameter: the relation update finds the
+        // normal rows' at index 1 of its array
+        if (E.shared_table && E.score_fn == SCORE_TRANSH)
+            E.h_alpha[((size_t)i * 4 + 1) * S + 1] = (float)(factor * (double)lr[0]) * E.lr_mod_normal;
     }
     HIP_CHECK(hipMemcpyAsync(E.d_alpha.p, E.h_alpha.data(), E.h_alpha.size() * 4, hipMemcpyHostToDevice, st));
     HIP_CHECK(hipEventRecord(E.ev[1], st));

@@ -13,7 +13,7 @@ namespace kge {
 // distance function's value itself (src/poplar_kge.cpp:501-514).
 // RotatE: (h_re, h_im) rotated by the relation's D/2 phases, whose sine and cosine pass
 // through float16 as in the reference (src/poplar_kge.cpp:516-537); score = gamma - distance.
-enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2, SCORE_ROTATE = 3 };
+enum { SCORE_TRANSE = 0, SCORE_DISTMULT = 1, SCORE_COMPLEX = 2, SCORE_ROTATE = 3, SCORE_TRANSH = 4 };
 // whether the score is the distance function's value itself (else gamma minus it)
 __host__ __device__ inline bool score_is_distance_value(int score_fn) { return score_fn == SCORE_DISTMULT || score_fn == SCORE_COMPLEX; }
 enum { DIST_L1 = 0, DIST_L2 = 1, DIST_DOT = 2 };
@@ -41,6 +41,8 @@ struct PlanShape {
     int n_entity;             // rows per shard table
     int shared_table;
     int n_relation;
+    int rel_copies;           // 1; 2 for TransH, whose relation table holds a second row (the
+                              // hyperplane normal, row n_relation + r) per relation
     int step0, step_count;    // the steps of the resident batch to plan
 };
 
@@ -49,7 +51,9 @@ struct PlanShape {
 //   [0, S*B)          head contributions  c = d*B + b
 //   [S*B, R)          tail contributions  c = S*B + d*T + (j*A + i)
 //   [R, 2R)           every remote slot, as a zero-gradient member of the update set
-// relation plan (S*B + n_relation items): head contributions, then every relation id.
+// relation plan (S*B + n_relation items): head contributions, then every relation id; with
+// rel_copies = 2 both parts twice, the second copies keyed n_relation + r (item S*B + c is the
+// normal row's contribution of positive c).
 void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
                         const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
                         uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
@@ -311,5 +315,37 @@ void launch_iota_keys(const uint32_t* idx, uint32_t* keys, uint32_t* vals, int64
                       hipStream_t stream);
 void launch_sum_partials_rows(const uint32_t* chunk_off, const float* partial, int64_t rows,
                               int64_t cols, float* out, hipStream_t stream);
+
+// ---- TransH (src/poplar_kge.cpp:539-565) ----
+// Operand matrices, dense float32 [R, Dp]: `pt` rows [0, S*B) predicted tails and rows [S*B, R)
+// tails; `nt` rows [0, S*B) the positives' unit hyperplane normals and the same tails after
+// them.  The relation table holds the raw normals as rows [n_rel, 2 n_rel).
+// Heads of `pt` hold the gathered head rows on entry.
+void launch_transh_predict(const float* rel, const uint32_t* crel, int n_rel, int n_head, int Dp, float* pt,
+                           float* nt, hipStream_t stream);
+struct TranshFwd {
+    ScoreShape sh;
+    const float* pt; const float* nt;
+    const float* cmat;       // [S, B, T] c = n . tail (the dot-product forward on `nt`)
+    const uint32_t* clabel;
+    float* coef;             // [S, B, T] coefficient d loss / d distance (fused loss) or raw score
+    float* dcm;              // [S, B, T] d loss / d c (fused loss) or q = sum_k sign(e) n
+    float* loss_part;        // as launch_score_fwd's, one part per 64 x 64 tile
+};
+void launch_transh_fwd(const TranshFwd& p, bool fused_loss, hipStream_t stream);
+void launch_mul_rows(float* a, const float* b, int64_t n, hipStream_t stream);  // a[i] *= b[i]
+struct TranshBwd {
+    const float* pt; const float* nt;
+    const float* coef; const float* cmat;  // [S, B, T]
+    float* mm;    // [R, Dp] in: the dot-product backward on `nt` with coefficient dcm;
+                  // out rows [0, S*B): d loss / d n complete
+    float* grad;  // [R, Dp] out: d loss / d p (heads), d loss / d tail (tails)
+    int S, B, T, Dp;
+};
+void launch_transh_bwd(const TranshBwd& p, hipStream_t stream);
+// heads of `grad` -> the head rows' gradient; relgrad [2 n_head, Dp]: rows [0, n_head) the relation
+// embedding rows' contributions, rows [n_head, 2 n_head) the normal rows'
+void launch_transh_back(const RowSource& ent, const float* rel, const uint32_t* crel, int n_rel, int n_head,
+                        int Dp, float* grad, const float* mm, float* relgrad, hipStream_t stream);
 
 }  // namespace kge

@@ -125,7 +125,8 @@ __global__ __launch_bounds__(256) void k_build_items(PlanShape ps, const uint32_
     const int S = ps.S, B = ps.B, A = ps.A, NR = ps.NR, T = S * A, nst = ps.n_step;
     const int R = S * NR, SB = S * B;
     const int item = blockIdx.x * 256 + threadIdx.x;
-    const int n_rel_items = SB + ps.n_relation;
+    const int SBr = SB * ps.rel_copies;
+    const int n_rel_items = SBr + ps.n_relation * ps.rel_copies;
     if (item < 2 * R) {
         int src, slot;
         if (item < SB) {
@@ -151,13 +152,17 @@ __global__ __launch_bounds__(256) void k_build_items(PlanShape ps, const uint32_
     }
     if (item < n_rel_items) {
         uint32_t key;
-        if (item < SB) {
-            const int d = item / B, b = item - d * B;
+        if (item < SBr) {
+            const int copy = item / SB, c = item - copy * SB;
+            const int d = c / B, b = c - d * B;
             key = relation[((size_t)d * nst + step) * B + b];
-            crel[(size_t)step * SB + item] = key;
-            clabel[(size_t)step * SB + item] = tail[((size_t)d * nst + step) * B + b];
+            if (copy == 0) {
+                crel[(size_t)step * SB + c] = key;
+                clabel[(size_t)step * SB + c] = tail[((size_t)d * nst + step) * B + b];
+            }
+            key += (uint32_t)(copy * ps.n_relation);
         } else {
-            key = item - SB;
+            key = item - SBr;
         }
         rel_keys[(size_t)step * n_rel_items + item] = key;
         rel_vals[(size_t)step * n_rel_items + item] = item;
@@ -170,7 +175,7 @@ void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint3
                         uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals,
                         hipStream_t stream) {
     const int R = ps.S * ps.NR;
-    const int n = std::max(2 * R, ps.S * ps.B + ps.n_relation);
+    const int n = std::max(2 * R, (ps.S * ps.B + ps.n_relation) * ps.rel_copies);
     dim3 grid((n + 255) / 256, ps.step_count);
     hipLaunchKernelGGL(k_build_items, grid, dim3(256), 0, stream, ps, remote, a2a, head, relation,
                        tail, ckey, crel, clabel, ent_keys, ent_vals, rel_keys, rel_vals);
@@ -3144,6 +3149,372 @@ void launch_sum_partials_rows(const uint32_t* chunk_off, const float* partial, i
                               int64_t cols, float* out, hipStream_t stream) {
     hipLaunchKernelGGL(k_sum_partials_rows, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
                        chunk_off, partial, rows, cols, out);
+}
+
+// --------------------------------------------------------------------------
+// TransH (src/poplar_kge.cpp:539-565).  Per positive b: the unit normal n_b = w / |w| of its
+// relation's hyperplane (w = the relation_normal row) and the predicted tail
+// p_b = h - n (n . h) + r.  Score of (b, t): gamma - sum_k |e_btk| with
+// e_btk = p_bk - (tau_tk - n_bk c_bt), c_bt = n_b . tau_t, whatever distance_fn says.
+// Two dense float32 operand matrices [R, Dp]: `pt` rows [0, SB) predicted tails, rows
+// [SB, R) tails; `nt` rows [0, SB) unit normals, rows [SB, R) the same tails, so that c and
+// its backward (d n += dc tau, d tau += dc^T n) are the ordinary dot-product scoring
+// kernels on `nt`.  The relation table holds the normals as rows [n_rel, 2 n_rel).
+
+// heads of `pt` (holding the gathered head rows h) -> p; heads of `nt` -> n.  One wave per positive.
+__global__ __launch_bounds__(256) void k_transh_predict(const float* __restrict__ rel,
+                                                        const uint32_t* __restrict__ crel, int n_rel,
+                                                        int n_head, int Dp, float* __restrict__ pt,
+                                                        float* __restrict__ nt) {
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (c >= n_head) return;
+    const uint32_t r = crel[c];
+    const float* w = rel + (size_t)(n_rel + r) * Dp;
+    const float* dr = rel + (size_t)r * Dp;
+    float* h = pt + (size_t)c * Dp;
+    float ss = 0.f;
+    for (int k = lane * 4; k < Dp; k += 256) {
+        const float4 w4 = *reinterpret_cast<const float4*>(w + k);
+        ss += w4.x * w4.x + w4.y * w4.y + w4.z * w4.z + w4.w * w4.w;
+    }
+    const float nrm = sqrtf(wave_sum(ss));
+    float a = 0.f;
+    for (int k = lane * 4; k < Dp; k += 256) {
+        const float4 w4 = *reinterpret_cast<const float4*>(w + k);
+        const float4 h4 = *reinterpret_cast<const float4*>(h + k);
+        a += (w4.x / nrm) * h4.x + (w4.y / nrm) * h4.y + (w4.z / nrm) * h4.z + (w4.w / nrm) * h4.w;
+    }
+    a = wave_sum(a);
+    for (int k = lane * 4; k < Dp; k += 256) {
+        const float4 w4 = *reinterpret_cast<const float4*>(w + k);
+        const float4 h4 = *reinterpret_cast<const float4*>(h + k);
+        const float4 d4 = *reinterpret_cast<const float4*>(dr + k);
+        const float4 n4 = make_float4(w4.x / nrm, w4.y / nrm, w4.z / nrm, w4.w / nrm);
+        float4 p4 = make_float4((h4.x - n4.x * a) + d4.x, (h4.y - n4.y * a) + d4.y, (h4.z - n4.z * a) + d4.z,
+                                (h4.w - n4.w * a) + d4.w);
+        *reinterpret_cast<float4*>(h + k) = p4;
+        *reinterpret_cast<float4*>(nt + (size_t)c * Dp + k) = n4;
+    }
+}
+void launch_transh_predict(const float* rel, const uint32_t* crel, int n_rel, int n_head, int Dp, float* pt,
+                           float* nt, hipStream_t stream) {
+    hipLaunchKernelGGL(k_transh_predict, dim3((n_head + 3) / 4), dim3(256), 0, stream, rel, crel, n_rel, n_head,
+                       Dp, pt, nt);
+}
+
+DEVINL float sign0(float t) { return (t > 0.f ? 1.f : 0.f) - (t < 0.f ? 1.f : 0.f); }
+
+// Forward over 64 x 64 score tiles.  OM 0: fused logsigmoid loss, `coef` receives the
+// coefficient G = d loss / d distance (scaled) and `dcm` G * q with q_bt = sum_k sign(e_btk) n_bk
+// (= d loss / d c_bt); OM 1: `coef` receives the raw score and `dcm` q (the loss rows turn the
+// scores into G, launch_mul_rows then forms G * q).
+template <int OM>
+__global__ __launch_bounds__(256) void k_transh_fwd(TranshFwd p) {
+    __shared__ __attribute__((aligned(16))) float As[BK][LDP];
+    __shared__ __attribute__((aligned(16))) float Ns[BK][LDP];
+    __shared__ __attribute__((aligned(16))) float Bs[BK][LDP];
+    __shared__ float red[4];
+    __shared__ uint32_t label_s[kScoreTile];
+    const ScoreShape& sh = p.sh;
+    const TileId tile = xcd_tile((sh.T + kScoreTile - 1) / kScoreTile, (sh.B + kScoreTile - 1) / kScoreTile, sh.S);
+    const int d = tile.z, m0 = tile.y * kScoreTile, n0 = tile.x * kScoreTile;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int B = sh.B, T = sh.T, Dp = sh.Dp;
+    if (OM == 0 && tid < kScoreTile) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
+    const int lr = tid >> 3, k4 = (tid & 7) * 4;
+    const int n_head = sh.S * B;
+
+    float cm[4][4], acc[4][4], q[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+            cm[i][j] = (m < B && n < T) ? p.cmat[((size_t)d * B + m) * T + n] : 0.f;
+            acc[i][j] = 0.f;
+            q[i][j] = 0.f;
+        }
+
+    for (int k0 = 0; k0 < Dp; k0 += BK) {
+        const int k = k0 + k4;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int m = m0 + lr + 32 * h, n = n0 + lr + 32 * h;
+            float4 a = make_float4(0, 0, 0, 0), nn = a, b = a;
+            if (k < Dp) {
+                if (m < B) {
+                    a = *reinterpret_cast<const float4*>(p.pt + (size_t)(d * B + m) * Dp + k);
+                    nn = *reinterpret_cast<const float4*>(p.nt + (size_t)(d * B + m) * Dp + k);
+                }
+                if (n < T) b = *reinterpret_cast<const float4*>(p.pt + (size_t)(n_head + d * T + n) * Dp + k);
+            }
+            const int r = lr + 32 * h;
+            As[k4 + 0][r] = a.x; As[k4 + 1][r] = a.y; As[k4 + 2][r] = a.z; As[k4 + 3][r] = a.w;
+            Ns[k4 + 0][r] = nn.x; Ns[k4 + 1][r] = nn.y; Ns[k4 + 2][r] = nn.z; Ns[k4 + 3][r] = nn.w;
+            Bs[k4 + 0][r] = b.x; Bs[k4 + 1][r] = b.y; Bs[k4 + 2][r] = b.z; Bs[k4 + 3][r] = b.w;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int kk = 0; kk < BK; ++kk) {
+            const float4 a4 = *reinterpret_cast<const float4*>(&As[kk][ty * 4]);
+            const float4 n4 = *reinterpret_cast<const float4*>(&Ns[kk][ty * 4]);
+            const float4 b4 = *reinterpret_cast<const float4*>(&Bs[kk][tx * 4]);
+            const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+            const float nv[4] = {n4.x, n4.y, n4.z, n4.w};
+            const float bv[4] = {b4.x, b4.y, b4.z, b4.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float e = av[i] - (bv[j] - nv[i] * cm[i][j]);  // p - (tail - n c)
+                    acc[i][j] += fabsf(e);
+                    q[i][j] = fmaf(sign0(e), nv[i], q[i][j]);
+                }
+        }
+        __syncthreads();
+    }
+
+    const float Tn = (float)T;
+    const float w_pos = uniform_f32(0.5f * Tn), w_neg = uniform_f32((0.5f * Tn) / (float)(T - 1));
+    const float inv_norm = uniform_f32(1.f / ((float)sh.S * (float)B * Tn));
+    const float grad_scale = uniform_f32(inv_norm * sh.loss_scale);
+    float loss_acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= B) continue;
+        const uint32_t label = OM == 0 ? label_s[ty * 4 + i] : 0u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= T) continue;
+            const float score = sh.gamma - acc[i][j];
+            float outv = score, dcv = q[i][j];
+            if (OM == 0) {
+                const bool pos = (uint32_t)n == label;
+                const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
+                float lsig, dlsig;
+                log_sigmoid_both(sign * score, lsig, dlsig);
+                loss_acc -= w * lsig;
+                outv = w * sign * dlsig * grad_scale;  // d loss / d distance = -d loss / d score
+                dcv = outv * q[i][j];
+            }
+            p.coef[((size_t)d * B + m) * T + n] = outv;
+            p.dcm[((size_t)d * B + m) * T + n] = dcv;
+        }
+    }
+    if (OM == 0) {
+        loss_acc = wave_sum(loss_acc);
+        if ((tid & 63) == 0) red[tid >> 6] = loss_acc;
+        __syncthreads();
+        if (tid == 0) {
+            const int n_part = tile.gx * tile.gy;
+            p.loss_part[(size_t)d * n_part + tile.y * tile.gx + tile.x] =
+                (red[0] + red[1] + red[2] + red[3]) * inv_norm;
+        }
+    }
+}
+void launch_transh_fwd(const TranshFwd& p, bool fused_loss, hipStream_t stream) {
+    const dim3 grid = tile_grid((p.sh.T + kScoreTile - 1) / kScoreTile, (p.sh.B + kScoreTile - 1) / kScoreTile, p.sh.S);
+    if (fused_loss) hipLaunchKernelGGL(k_transh_fwd<0>, grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(k_transh_fwd<1>, grid, dim3(256), 0, stream, p);
+}
+
+// a[i] *= b[i]
+__global__ __launch_bounds__(256) void k_mul_rows(float* __restrict__ a, const float* __restrict__ b, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) a[i] *= b[i];
+}
+void launch_mul_rows(float* a, const float* b, int64_t n, hipStream_t stream) {
+    hipLaunchKernelGGL(k_mul_rows, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, a, b, n);
+}
+
+// Backward through the distance, 64 self rows x 64 columns per workgroup, all rows of the
+// other side in slabs of 32.  With s = sign(e) and G = coef:
+//   SIDE_B false (self = positives):  grad[b]  = sum_t G s          (d loss / d p)
+//                                     gn[b]   += sum_t G s c        (added to d c's share, in place)
+//   SIDE_B true  (self = tails):      grad[t]  = gt[t] - sum_b G s  (gt = d c's share)
+// gn / gt are the rows of `mm` (the dot-product backward on `nt` with coefficient dcm).
+template <bool SIDE_B>
+__global__ __launch_bounds__(256) void k_transh_bwd(TranshBwd p) {
+    __shared__ __attribute__((aligned(16))) float Cs[BJ][LDP];  // G[j][i]
+    __shared__ __attribute__((aligned(16))) float Ms[BJ][LDP];  // c[j][i]
+    __shared__ __attribute__((aligned(16))) float Os[BJ][LDP];  // other side's main rows [j][k]
+    __shared__ __attribute__((aligned(16))) float Qs[SIDE_B ? BJ : 1][LDP];  // other side's normals [j][k]
+    const int B = p.B, T = p.T, Dp = p.Dp;
+    const int n_self = SIDE_B ? T : B, n_other = SIDE_B ? B : T;
+    const TileId tile = xcd_tile((Dp + kScoreTile - 1) / kScoreTile, (n_self + kScoreTile - 1) / kScoreTile, p.S);
+    const int d = tile.z, i0 = tile.y * kScoreTile, kt0 = tile.x * kScoreTile;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int n_head = p.S * B;
+    const int self_c0 = SIDE_B ? n_head + d * T : d * B, other_c0 = SIDE_B ? d * B : n_head + d * T;
+    const float* coef = p.coef + (size_t)d * B * T;
+    const float* cmat = p.cmat + (size_t)d * B * T;
+
+    float sv[4][4], sn[4][4], acc[4][4], accn[4][4];
+    const int kcol = kt0 + tx * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i0 + ty * 4 + i;
+        float4 v = make_float4(0, 0, 0, 0), n = v;
+        if (r < n_self && kcol < Dp) {
+            v = *reinterpret_cast<const float4*>(p.pt + (size_t)(self_c0 + r) * Dp + kcol);
+            if (!SIDE_B) n = *reinterpret_cast<const float4*>(p.nt + (size_t)(self_c0 + r) * Dp + kcol);
+        }
+        sv[i][0] = v.x; sv[i][1] = v.y; sv[i][2] = v.z; sv[i][3] = v.w;
+        sn[i][0] = n.x; sn[i][1] = n.y; sn[i][2] = n.z; sn[i][3] = n.w;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { acc[i][k] = 0.f; accn[i][k] = 0.f; }
+    }
+
+    for (int j0 = 0; j0 < n_other; j0 += BJ) {
+        for (int idx = tid; idx < BJ * kScoreTile; idx += 256) {
+            int i, j;
+            size_t at;
+            bool live;
+            if (!SIDE_B) {  // G[i0 + i][j0 + j], contiguous over j
+                j = idx & (BJ - 1); i = idx / BJ;
+                live = i0 + i < B && j0 + j < T;
+                at = (size_t)(i0 + i) * T + j0 + j;
+            } else {        // G[j0 + j][i0 + i], contiguous over i
+                i = idx & (kScoreTile - 1); j = idx / kScoreTile;
+                live = j0 + j < B && i0 + i < T;
+                at = (size_t)(j0 + j) * T + i0 + i;
+            }
+            Cs[j][i] = live ? coef[at] : 0.f;
+            Ms[j][i] = live ? cmat[at] : 0.f;
+        }
+        {
+            const int lj = tid >> 4, kk4 = (tid & 15) * 4;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int j = lj + 16 * h, gj = j0 + j, gk = kt0 + kk4;
+                float4 t = make_float4(0, 0, 0, 0), n = t;
+                if (gj < n_other && gk < Dp) {
+                    t = *reinterpret_cast<const float4*>(p.pt + (size_t)(other_c0 + gj) * Dp + gk);
+                    if (SIDE_B) n = *reinterpret_cast<const float4*>(p.nt + (size_t)(other_c0 + gj) * Dp + gk);
+                }
+                *reinterpret_cast<float4*>(&Os[j][kk4]) = t;
+                if (SIDE_B) *reinterpret_cast<float4*>(&Qs[j][kk4]) = n;
+            }
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int jj = 0; jj < BJ; ++jj) {
+            const float4 c4 = *reinterpret_cast<const float4*>(&Cs[jj][ty * 4]);
+            const float4 m4 = *reinterpret_cast<const float4*>(&Ms[jj][ty * 4]);
+            const float4 o4 = *reinterpret_cast<const float4*>(&Os[jj][tx * 4]);
+            float4 q4 = make_float4(0, 0, 0, 0);
+            if (SIDE_B) q4 = *reinterpret_cast<const float4*>(&Qs[jj][tx * 4]);
+            const float cv[4] = {c4.x, c4.y, c4.z, c4.w};
+            const float mv[4] = {m4.x, m4.y, m4.z, m4.w};
+            const float ov[4] = {o4.x, o4.y, o4.z, o4.w};
+            const float qv[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (!SIDE_B) {
+                        const float g = cv[i] * sign0(sv[i][k] - (ov[k] - sn[i][k] * mv[i]));
+                        acc[i][k] += g;
+                        accn[i][k] = fmaf(g, mv[i], accn[i][k]);
+                    } else {
+                        acc[i][k] -= cv[i] * sign0(ov[k] - (sv[i][k] - qv[k] * mv[i]));
+                    }
+                }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i0 + ty * 4 + i;
+        if (r >= n_self || kcol >= Dp) continue;
+        float* mrow = p.mm + (size_t)(self_c0 + r) * Dp + kcol;
+        const float4 add = *reinterpret_cast<const float4*>(mrow);
+        float4 out = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+        if (SIDE_B) {
+            out = f4add(out, add);
+        } else {
+            *reinterpret_cast<float4*>(mrow) =
+                make_float4(add.x + accn[i][0], add.y + accn[i][1], add.z + accn[i][2], add.w + accn[i][3]);
+        }
+        *reinterpret_cast<float4*>(p.grad + (size_t)(self_c0 + r) * Dp + kcol) = out;
+    }
+}
+void launch_transh_bwd(const TranshBwd& p, hipStream_t stream) {
+    const int gk = (p.Dp + kScoreTile - 1) / kScoreTile;
+    hipLaunchKernelGGL(k_transh_bwd<false>, tile_grid(gk, (p.B + kScoreTile - 1) / kScoreTile, p.S), dim3(256), 0,
+                       stream, p);
+    hipLaunchKernelGGL(k_transh_bwd<true>, tile_grid(gk, (p.T + kScoreTile - 1) / kScoreTile, p.S), dim3(256), 0,
+                       stream, p);
+}
+
+// Backward through transHPredict, one wave per positive c: from gp = grad[c] (d loss / d p) and
+// gn = mm[c] (d loss / d n from the score) to
+//   grad[c]            = gp - n (gp . n)                              the head's gradient
+//   relgrad[c]         = gp                                           relation embedding row
+//   relgrad[n_head+c]  = (g - n (n . g)) / |w|,  g = gn - (n . h) gp - h (gp . n)   normal row
+__global__ __launch_bounds__(256) void k_transh_back(RowSource ent, const float* __restrict__ rel,
+                                                     const uint32_t* __restrict__ crel, int n_rel, int n_head,
+                                                     int Dp, float* __restrict__ grad,
+                                                     const float* __restrict__ mm, float* __restrict__ relgrad) {
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (c >= n_head) return;
+    const float* w = rel + (size_t)(n_rel + crel[c]) * Dp;
+    const char* hrow = row_ptr(ent, c);
+    float* gp = grad + (size_t)c * Dp;
+    const float* gn = mm + (size_t)c * Dp;
+    float ss = 0.f;
+    for (int k = lane * 4; k < Dp; k += 256) {
+        const float4 w4 = *reinterpret_cast<const float4*>(w + k);
+        ss += w4.x * w4.x + w4.y * w4.y + w4.z * w4.z + w4.w * w4.w;
+    }
+    const float nrm = sqrtf(wave_sum(ss));
+    float a = 0.f, sgn = 0.f;
+    for (int k = lane * 4; k < Dp; k += 256) {
+        const float4 w4 = *reinterpret_cast<const float4*>(w + k);
+        const float4 h4 = load4(hrow, k, ent);
+        const float4 g4 = *reinterpret_cast<const float4*>(gp + k);
+        const float n[4] = {w4.x / nrm, w4.y / nrm, w4.z / nrm, w4.w / nrm};
+        a += n[0] * h4.x + n[1] * h4.y + n[2] * h4.z + n[3] * h4.w;
+        sgn += n[0] * g4.x + n[1] * g4.y + n[2] * g4.z + n[3] * g4.w;
+    }
+    a = wave_sum(a);
+    sgn = wave_sum(sgn);
+    float ngn = 0.f;
+    for (int k = lane * 4; k < Dp; k += 256) {
+        const float4 w4 = *reinterpret_cast<const float4*>(w + k);
+        const float4 h4 = load4(hrow, k, ent);
+        const float4 g4 = *reinterpret_cast<const float4*>(gp + k);
+        const float4 q4 = *reinterpret_cast<const float4*>(gn + k);
+        ngn += (w4.x / nrm) * (q4.x - a * g4.x - h4.x * sgn) + (w4.y / nrm) * (q4.y - a * g4.y - h4.y * sgn) +
+               (w4.z / nrm) * (q4.z - a * g4.z - h4.z * sgn) + (w4.w / nrm) * (q4.w - a * g4.w - h4.w * sgn);
+    }
+    ngn = wave_sum(ngn);
+    for (int k = lane * 4; k < Dp; k += 256) {
+        const float4 w4 = *reinterpret_cast<const float4*>(w + k);
+        const float4 h4 = load4(hrow, k, ent);
+        const float4 g4 = *reinterpret_cast<const float4*>(gp + k);
+        const float4 q4 = *reinterpret_cast<const float4*>(gn + k);
+        const float n[4] = {w4.x / nrm, w4.y / nrm, w4.z / nrm, w4.w / nrm};
+        const float g[4] = {g4.x, g4.y, g4.z, g4.w}, h[4] = {h4.x, h4.y, h4.z, h4.w}, qq[4] = {q4.x, q4.y, q4.z, q4.w};
+        float gh[4], gw[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            gh[x] = g[x] - n[x] * sgn;
+            gw[x] = ((qq[x] - a * g[x] - h[x] * sgn) - n[x] * ngn) / nrm;
+        }
+        *reinterpret_cast<float4*>(relgrad + (size_t)c * Dp + k) = g4;
+        *reinterpret_cast<float4*>(relgrad + (size_t)(n_head + c) * Dp + k) = make_float4(gw[0], gw[1], gw[2], gw[3]);
+        *reinterpret_cast<float4*>(gp + k) = make_float4(gh[0], gh[1], gh[2], gh[3]);
+    }
+}
+void launch_transh_back(const RowSource& ent, const float* rel, const uint32_t* crel, int n_rel, int n_head,
+                        int Dp, float* grad, const float* mm, float* relgrad, hipStream_t stream) {
+    hipLaunchKernelGGL(k_transh_back, dim3((n_head + 3) / 4), dim3(256), 0, stream, ent, rel, crel, n_rel, n_head,
+                       Dp, grad, mm, relgrad);
 }
 
 }  // namespace kge

@@ -384,7 +384,8 @@ class Engine:
     # ---- initialisation ------------------------------------------------------
     def initialise_variables(self) -> None:
         """step = 0, zero moments, scaled-normal parameters (reference :624-688):
-        relation_embedding ~ (init_scale / D) N(0, 1) (RotatE: uniform phases); feature_projection
+        relation_embedding ~ (init_scale / D) N(0, 1) (RotatE: uniform phases; TransH: relation_normal
+        drawn the same way after it); feature_projection
         ~ N(0, 1) scaled the same way and divided by sqrt(F)."""
         m = self.settings.model
         self.write_variable("step", np.zeros(m.n_shard, np.uint32))
@@ -397,6 +398,8 @@ class Engine:
         else:
             relation = self.random_normal(relation_shape)
         self.write_variable("relation_embedding", self.init_scale * relation)
+        if m.score_fn == "TransH":   # the hyperplane normals (reference :643-651)
+            self.write_variable("relation_normal", self.init_scale * self.random_normal(relation_shape))
         self.write_variable(
             "feature_projection",
             (self.init_scale / np.sqrt(max(m.entity_feature_size, 1)))

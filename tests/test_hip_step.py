@@ -85,6 +85,19 @@ CASES = {
     "aligned_complex": dict(score_fn="ComplEx", distance_fn="MatMul", loss_fn="softmax",
                             softmax_correction_weight=1.0, n_shard=2, batch=128, a2a=64, dim=64,
                             feature=0, n_entity=3000, n_relation=8),
+    # TransH (src/poplar_kge.cpp:539-565): unit hyperplane normals from relation_normal, heads
+    # and tails projected, L1 distance whatever distance_fn says
+    "transh": dict(score_fn="TransH", feature=0),
+    "transh_feat_softmax": dict(score_fn="TransH", distance_fn="L2", loss_fn="softmax",
+                                softmax_correction_weight=1.0),
+    "transh_shared": dict(score_fn="TransH", shared_table=True, n_shard=4, batch=8, a2a=4, feature=0,
+                          n_entity=60, gamma=3.0),
+    "transh_odd_adversarial": dict(score_fn="TransH", dim=10, feature=6, n_entity=41, batch=5, a2a=3,
+                                   negative_adversarial_scale=1.5),
+    "transh_aligned": dict(score_fn="TransH", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
+                           n_entity=3000, n_relation=8, gamma=6.0),
+    "transh_mid": dict(score_fn="TransH", n_shard=2, batch=70, a2a=45, dim=64, feature=0,
+                       n_entity=2000, n_relation=10, gamma=6.0),
     "aligned_complex_l2_shared": dict(score_fn="ComplEx", distance_fn="L2", n_shard=4, batch=128, a2a=32,
                                       dim=128, feature=0, n_entity=2000, n_relation=8, shared_table=True),
 }
