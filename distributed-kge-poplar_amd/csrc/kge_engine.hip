@@ -229,7 +229,7 @@ struct kge_engine {
     // step
     // predict scratch (allocated by the first predict call)
     DevBuf<uint32_t> p_idx, p_rel, p_count, p_best_i;
-    DevBuf<float> p_opnd, p_scores, p_best_s, p_hidden, p_featd;
+    DevBuf<float> p_opnd, p_scores, p_best_s, p_hidden, p_featd, p_opnd_n, p_cmat;
     DevBuf<uint16_t> opnd16, opndT16, coef16, coefT16, feat16, featT16, projT16, gT16;  // bfloat16 scoring operands
     // norm regularisers (src/poplar_kge.cpp:430-437): per distinct row gradients and loss shares
     float reg_p[3] = {3.f, 3.f, 3.f}, reg_w[3] = {0.f, 0.f, 0.f};
@@ -1188,6 +1188,10 @@ void run_predict(kge_engine& E, const Items& in) {
         E.p_count.alloc(1);
         E.p_opnd.alloc((size_t)(Qp + chunk) * Dp);
         E.p_scores.alloc((size_t)Qp * chunk);
+        if (E.score_fn == SCORE_TRANSH) {
+            E.p_opnd_n.alloc((size_t)(Qp + chunk) * Dp);
+            E.p_cmat.alloc((size_t)Qp * chunk);
+        }
         E.p_best_s.alloc((size_t)Q * nb);
         E.p_best_i.alloc((size_t)Q * nb);
         if (E.F) {
@@ -1222,6 +1226,12 @@ void run_predict(kge_engine& E, const Items& in) {
     launch_gather_operands(rows_of(E.p_idx.p, Qp), E.rel.p, E.p_rel.p, rel_mode_of(E), E.D / 2, Qp,
                            Qp, Dp, E.p_opnd.p, nullptr, st);
 
+    const bool transh = E.score_fn == SCORE_TRANSH;
+    if (transh) {  // unit normals beside the predicted tails (transHPredict, :539-549)
+        HIP_CHECK(hipMemcpyAsync(E.p_opnd_n.p, E.p_opnd.p, (size_t)Qp * Dp * 4, hipMemcpyDeviceToDevice, st));
+        launch_transh_predict(E.rel.p, E.p_rel.p, E.n_rel, Qp, Dp, E.p_opnd.p, E.p_opnd_n.p, st);
+    }
+
     ScoreShape sh = {};
     sh.S = 1; sh.B = Qp; sh.T = chunk; sh.Dp = Dp;
     sh.score_fn = E.score_fn; sh.dist_fn = E.dist_fn; sh.loss_fn = E.loss_fn;
@@ -1229,6 +1239,10 @@ void run_predict(kge_engine& E, const Items& in) {
     RowSource dense;
     dense.base = (const char*)E.p_opnd.p; dense.pitch = (int64_t)Dp * 4; dense.etype = ET_F32;
     dense.index = nullptr; dense.count = Dp; dense.vec = 1;
+    RowSource dense_n = dense;
+    dense_n.base = (const char*)E.p_opnd_n.p;
+    ScoreShape dot = sh;
+    dot.score_fn = SCORE_DISTMULT; dot.dist_fn = DIST_DOT;
 
     std::vector<float> init_s((size_t)Q * nb, -1e6f), got_s((size_t)Q * nb);
     std::vector<uint32_t> init_i((size_t)Q * nb, 0u), got_i((size_t)Q * nb);
@@ -1250,6 +1264,16 @@ void run_predict(kge_engine& E, const Items& in) {
             launch_row_range((uint32_t)(table_off + r0), live, chunk, tail_idx, st);
             launch_gather_operands(rows_of(tail_idx, chunk), E.rel.p, nullptr, 0, 0, 0, chunk, Dp,
                                    E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
+            if (transh) {  // transHScore (:551-565): c = n . tail, then the L1 part
+                HIP_CHECK(hipMemcpyAsync(E.p_opnd_n.p + (size_t)Qp * Dp, E.p_opnd.p + (size_t)Qp * Dp,
+                                         (size_t)chunk * Dp * 4, hipMemcpyDeviceToDevice, st));
+                launch_score_fwd(dot, dense_n, E.rel.p, nullptr, nullptr, E.p_cmat.p, nullptr, nullptr, nullptr,
+                                 false, st);
+                TranshFwd tf;
+                tf.sh = sh; tf.pt = E.p_opnd.p; tf.nt = E.p_opnd_n.p; tf.cmat = E.p_cmat.p; tf.clabel = nullptr;
+                tf.coef = E.p_scores.p; tf.dcm = nullptr; tf.loss_part = nullptr;
+                launch_transh_fwd(tf, false, st);
+            } else
             launch_score_fwd(sh, dense, E.rel.p, nullptr, nullptr, E.p_scores.p, nullptr, nullptr, nullptr,
                              false, st);
             launch_topk_merge(E.p_scores.p, chunk, Q, live, (uint32_t)r0, (int)nb, E.p_best_s.p, E.p_best_i.p, st);

@@ -329,7 +329,7 @@ struct TranshFwd {
     const float* cmat;       // [S, B, T] c = n . tail (the dot-product forward on `nt`)
     const uint32_t* clabel;
     float* coef;             // [S, B, T] coefficient d loss / d distance (fused loss) or raw score
-    float* dcm;              // [S, B, T] d loss / d c (fused loss) or q = sum_k sign(e) n
+    float* dcm;              // [S, B, T] d loss / d c (fused loss) or q = sum_k sign(e) n; or null
     float* loss_part;        // as launch_score_fwd's, one part per 64 x 64 tile
 };
 void launch_transh_fwd(const TranshFwd& p, bool fused_loss, hipStream_t stream);

@@ -3301,7 +3301,7 @@ __global__ __launch_bounds__(256) void k_transh_fwd(TranshFwd p) {
                 dcv = outv * q[i][j];
             }
             p.coef[((size_t)d * B + m) * T + n] = outv;
-            p.dcm[((size_t)d * B + m) * T + n] = dcv;
+            if (p.dcm) p.dcm[((size_t)d * B + m) * T + n] = dcv;
         }
     }
     if (OM == 0) {

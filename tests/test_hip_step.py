@@ -476,3 +476,42 @@ def test_engine_errors():
     bad["head"][0, 0, 0] = 10**6
     with pytest.raises(ValueError, match="out of range"):
         engine.run("train_step_loop", dict(learning_rate=lr, loss=loss, **bad))
+
+
+def test_transh_relation_normal_step_size_modifier(oracle64):
+    # training.learning_rate_modifiers is keyed by parameter name (src/poplar_kge.cpp:321-327):
+    # relation_normal takes its own factor, with private tables (per-shard step sizes) and a
+    # shared one.  One step, so that each parameter's update depends on its own step size only;
+    # the oracle has one factor for the whole relation array, so it runs once per factor.
+    import libpoplar_kge
+
+    mods = {"relation_normal": 0.25, "relation_embedding": 2.0}
+    for shared in (False, True):
+        c = K.cfg_dict(score_fn="TransH", feature=0, shared_table=shared, n_shard=2, n_entity=90)
+        rng = np.random.default_rng(31)
+        st0 = K.make_state(c, rng)
+        batch = K.random_batch(c, 1, rng)
+        lr = np.array([0.1, 0.1 if shared else 0.04], np.float32)
+        engine = libpoplar_kge.Engine(H.engine_settings(c, 1, **{"training.learning_rate_modifiers": mods}), "")
+        H.load_state(engine, c, st0)
+        H.train(engine, c, lr, batch)
+        st_h = H.read_state(engine, c)
+        for name, mod in mods.items():
+            st_o = K.copy_state(st0)
+            oracle64.train_step_loop(make_cfg(**c, lr_mod_relation=mod), st_o, lr, batch)
+            assert K.rel_l2(st_h[name] - st0[name], st_o[name] - st0[name]) < 1e-4, (shared, name)
+            for suffix in ("/adam_m", "/adam_v"):
+                assert K.rel_l2(st_h[name + suffix], st_o[name + suffix]) < 1e-5, (shared, name, suffix)
+        # and the two factors really differ in effect
+        st_o = K.copy_state(st0)
+        oracle64.train_step_loop(make_cfg(**c), st_o, lr, batch)
+        assert K.rel_l2(st_h["relation_normal"] - st0["relation_normal"],
+                        st_o["relation_normal"] - st0["relation_normal"]) > 0.5
+
+
+def test_transh_zipf_duplicates(oracle64):
+    # heavy duplicates among heads, tails and relations: hot entity rows and hot relation rows
+    # (both copies) go through the chunked reduction
+    kw = dict(score_fn="TransH", n_shard=4, batch=64, a2a=16, dim=32, feature=0, n_entity=500, n_relation=4,
+              shared_table=True, gamma=4.0)
+    run_case(oracle64, kw, n_step=2, batch_fn=K.raw_batch)

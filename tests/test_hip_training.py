@@ -164,7 +164,8 @@ def _random_queries(engine, n):
                      engine.random_integers(s.model.n_relation_type, (n,))], axis=-1)
 
 
-@pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "complex", "rotate", "no_features_big"])
+@pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "complex", "rotate", "transh", "transh_big",
+                                     "no_features_big"])
 def test_predict_vs_brute_force(variant):
     """Engine.predict against a float64 brute force over every row of every shard
     (the reference checks shapes, ranges and ordering, tests/python/test_poplar_kge.py:155-175,
@@ -183,11 +184,15 @@ def test_predict_vs_brute_force(variant):
         m.score_fn, m.distance_fn = "ComplEx", "MatMul"
     elif variant == "rotate":
         m.score_fn = "RotatE"
-    elif variant == "no_features_big":
+    elif variant == "transh":
+        m.score_fn = "TransH"
+    elif variant in ("no_features_big", "transh_big"):
         # several chunks of tails per shard, several query chunks, ragged counts
         m.n_entity, m.entity_feature_size, m.embedding_size, m.n_shard = 20000, 0, 32, 3
         settings.data.batch_size, ex.rw_batch_size, ex.predict_n_best = 6, 4096, 20
         m.distance_fn = "L2"
+        if variant == "transh_big":
+            m.score_fn = "TransH"
     settings.prepare()
     S = m.n_shard
     counts = np.array([m.n_entity - 1 - 7 * s for s in range(S)])
