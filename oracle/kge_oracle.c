@@ -58,6 +58,10 @@ typedef struct {
     int32_t loss_fn;        /* LOSS_*                                           */
     int32_t shared_table;   /* 1: every shard addresses the same n_entity rows  */
     int32_t storage;        /* STORE_*: rounding applied on row write-back      */
+    int32_t mlp_size;       /* M > 0: feature MLP (poplar_kge.cpp:453-458), the feature part of
+                             * hidden is relu([embedding | feature . W] . Up) . Down with
+                             * Up [2D, M], Down [M, D]; `proj` and its moments then hold
+                             * W, Up and Down back to back                               */
     int32_t scoring_bf16;   /* 1: predicted tails and tails rounded to bfloat16
                              * before the dot product, features and projection
                              * before theirs (products exact, sums in REAL);
@@ -457,23 +461,41 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
     /* TransH (poplar_kge.cpp:252-255): `rel` and its moments hold 2 * NREL rows, the
      * relation embeddings followed by the hyperplane normals (relation_normal)       */
     const int transh = c->score_fn == SCORE_TRANSH;
+    const int64_t M = F > 0 ? c->mlp_size : 0;
+    const float* up = proj + F * D;           /* [2D, M] */
+    const float* down = up + 2 * D * M;       /* [M, D]  */
     const int64_t NRELT = transh ? 2 * NREL : NREL;
 #define KEY(s, slot) ((c->shared_table ? 0 : (int64_t)(s) * NE) + (int64_t)remote[(s) * NR + (slot)])
 
     /* 1. gather + hidden = emb + feature * W  (:405-410, :439-467) */
     REAL* hidden = (REAL*)malloc(sizeof(REAL) * (size_t)(S * NR * D));
     REAL* ghid = (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL));
+    /* feature MLP: per slot, the projected features (the second half of the MLP's input) and
+     * the pre-activations, kept for the backward pass */
+    REAL* fproj = M ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
+    REAL* pre = M ? (REAL*)calloc((size_t)(S * NR * M), sizeof(REAL)) : NULL;
     for (int64_t s = 0; s < S; ++s)
         for (int64_t j = 0; j < NR; ++j) {
             const float* row = table + KEY(s, j) * ROW;
             REAL* h = hidden + (s * NR + j) * D;
+            REAL* fh = M ? fproj + (s * NR + j) * D : h;
             for (int64_t k = 0; k < D; ++k) h[k] = row[k];
             for (int64_t f = 0; f < F; ++f) {
                 /* bfloat16 scoring also takes the projection's operands in bfloat16 */
                 const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
                 if (x != 0)
                     for (int64_t k = 0; k < D; ++k)
-                        h[k] += x * (REAL)(c->scoring_bf16 ? round_bf16(proj[f * D + k]) : proj[f * D + k]);
+                        fh[k] += x * (REAL)(c->scoring_bf16 ? round_bf16(proj[f * D + k]) : proj[f * D + k]);
+            }
+            if (M) { /* :453-458: boom = relu(concat(value, featureHidden) . Up); featureHidden = boom . Down */
+                REAL* a = pre + (s * NR + j) * M;
+                for (int64_t i = 0; i < 2 * D; ++i) {
+                    const REAL x = i < D ? (REAL)row[i] : fh[i - D];
+                    for (int64_t m = 0; m < M; ++m) a[m] += x * (REAL)up[i * M + m];
+                }
+                for (int64_t m = 0; m < M; ++m)
+                    if (a[m] > 0)
+                        for (int64_t k = 0; k < D; ++k) h[k] += a[m] * (REAL)down[m * D + k];
             }
         }
 
@@ -760,19 +782,52 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
      * when the networks are shared, so the two uses' gradients add up to
      * the per-slot ghid already accumulated above)                          */
     REAL* gproj = NULL;
+    REAL* gmlp_val = NULL; /* feature MLP: what reaches the embedding through the MLP's input */
     if (F > 0) {
-        gproj = (REAL*)calloc((size_t)(F * D), sizeof(REAL));
+        gproj = (REAL*)calloc((size_t)(F * D + 3 * D * M), sizeof(REAL));
+        REAL* gup = gproj + F * D;
+        REAL* gdown = gup + 2 * D * M;
+        REAL* gfh = (REAL*)malloc(sizeof(REAL) * (size_t)D);
+        REAL* gpre = M ? (REAL*)malloc(sizeof(REAL) * (size_t)M) : NULL;
+        if (M) gmlp_val = (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL));
         for (int64_t s = 0; s < S; ++s)
             for (int64_t j = 0; j < NR; ++j) {
                 const float* row = table + KEY(s, j) * ROW;
                 const REAL* gh = ghid + (s * NR + j) * D;
                 const REAL* gr = greg_fh ? greg_fh + (s * NR + j) * D : NULL;
+                for (int64_t k = 0; k < D; ++k) gfh[k] = gh[k] + (gr ? gr[k] : 0);
+                if (M) {
+                    /* matMul, max(., 0) (its gradient passes where input == output, i.e. also at
+                     * exactly 0: pag.cpp:650-658), matMul, concat backward in turn */
+                    const REAL* a = pre + (s * NR + j) * M;
+                    const REAL* fh = fproj + (s * NR + j) * D;
+                    REAL* gv = gmlp_val + (s * NR + j) * D;
+                    for (int64_t m = 0; m < M; ++m) {
+                        const REAL boom = a[m] > 0 ? a[m] : 0;
+                        REAL acc = 0;
+                        for (int64_t k = 0; k < D; ++k) {
+                            gdown[m * D + k] += boom * gfh[k];
+                            acc += gfh[k] * (REAL)down[m * D + k];
+                        }
+                        gpre[m] = a[m] >= 0 ? acc : 0;
+                    }
+                    for (int64_t i = 0; i < 2 * D; ++i) {
+                        const REAL x = i < D ? (REAL)row[i] : fh[i - D];
+                        REAL acc = 0;
+                        for (int64_t m = 0; m < M; ++m) {
+                            gup[i * M + m] += x * gpre[m];
+                            acc += gpre[m] * (REAL)up[i * M + m];
+                        }
+                        if (i < D) gv[i] = acc; else gfh[i - D] = acc;
+                    }
+                }
                 for (int64_t f = 0; f < F; ++f) {
                     const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
                     if (x != 0)
-                        for (int64_t k = 0; k < D; ++k) gproj[f * D + k] += x * (gh[k] + (gr ? gr[k] : 0));
+                        for (int64_t k = 0; k < D; ++k) gproj[f * D + k] += x * gfh[k];
                 }
             }
+        free(gfh); free(gpre);
     }
 
     /* 7. entity Adam on every gathered row, one update per distinct row
@@ -793,7 +848,8 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
             for (; j < n && (int64_t)(ks[j] >> 24) == key; ++j) {
                 const REAL* gh = ghid + (int64_t)(ks[j] & 0xffffff) * D;
                 const REAL* gr = greg_val ? greg_val + (int64_t)(ks[j] & 0xffffff) * D : NULL;
-                for (int64_t k = 0; k < D; ++k) g[k] += gh[k] + (gr ? gr[k] : 0);
+                const REAL* gm = gmlp_val ? gmlp_val + (int64_t)(ks[j] & 0xffffff) * D : NULL;
+                for (int64_t k = 0; k < D; ++k) g[k] += gh[k] + (gr ? gr[k] : 0) + (gm ? gm[k] : 0);
             }
             for (int64_t k = 0; k < D; ++k) gf[k] = (float)g[k];
             float* row = table + key * ROW;
@@ -830,12 +886,27 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                             c->weight_decay, 0);
         }
         free(gf);
+        if (M) { /* the MLP's two matrices, rows split over the shards like every parameter; no
+                  * step-size modifier of their own here */
+            const int64_t off[2] = {F * D, F * D + 2 * D * M}, rows[2] = {2 * D, M}, width[2] = {M, D};
+            for (int q = 0; q < 2; ++q) {
+                float* gw = (float*)malloc(sizeof(float) * (size_t)width[q]);
+                for (int64_t r = 0; r < rows[q]; ++r) {
+                    const int64_t o = off[q] + r * width[q];
+                    for (int64_t k = 0; k < width[q]; ++k) gw[k] = (float)gproj[o + k];
+                    const int64_t shard = c->shared_table ? 0 : r / (rows[q] / S);
+                    kge_oracle_adam(proj + o, proj_m + o, proj_v + o, gw, width[q], alpha[shard], c->beta_m,
+                                    c->beta_v, c->epsilon, c->weight_decay, 0);
+                }
+                free(gw);
+            }
+        }
     }
 #undef KEY
     free(greg_val); free(greg_fh); free(reg_loss);
     free(hidden); free(ghid); free(grel); free(p); free(tl); free(score); free(dist);
     free(dscore); free(dp); free(dtl); free(alpha); free(gproj);
-    free(nv); free(dnv); free(nrm);
+    free(nv); free(dnv); free(nrm); free(fproj); free(pre); free(gmlp_val);
     return 0;
 }
 

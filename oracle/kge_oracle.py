@@ -23,7 +23,7 @@ STORE = {"float32": 0, "float16": 1, "bfloat16_embedding": 2}
 class Cfg(C.Structure):
     _fields_ = [(n, C.c_int32) for n in (
         "n_shard", "n_entity", "n_relation", "dim", "feature", "batch", "a2a", "score_fn",
-        "distance_fn", "loss_fn", "shared_table", "storage", "scoring_bf16")] + [(n, C.c_float) for n in (
+        "distance_fn", "loss_fn", "shared_table", "storage", "mlp_size", "scoring_bf16")] + [(n, C.c_float) for n in (
             "gamma", "beta_m", "beta_v", "epsilon", "weight_decay", "loss_scale",
             "softmax_correction_weight", "negative_adversarial_scale", "lr_mod_entity",
             "lr_mod_relation", "lr_mod_projection", "reg_emb_power", "reg_emb_weight", "reg_feat_power",
@@ -36,12 +36,13 @@ def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score
              loss_scale=None, softmax_correction_weight=0.0, negative_adversarial_scale=0.0,
              lr_mod_entity=1.0, lr_mod_relation=1.0, lr_mod_projection=1.0,
              embedding_regularisation=(3.0, 0.0), feature_regularisation=(3.0, 0.0),
-             hidden_regularisation=(3.0, 0.0)):
+             hidden_regularisation=(3.0, 0.0), feature_mlp_size=0):
     """The three regularisers are (power, weight) pairs (src/python/poplar_kge.py:104-108)."""
     if loss_scale is None:  # src/python/poplar_kge.py:259-262
         loss_scale = float(batch * n_shard * a2a)
     return Cfg(n_shard, n_entity, n_relation, dim, feature, batch, a2a, SCORE[score_fn],
-               DIST[distance_fn], LOSS[loss_fn], int(shared_table), STORE[storage], int(scoring_bf16),
+               DIST[distance_fn], LOSS[loss_fn], int(shared_table), STORE[storage], int(feature_mlp_size) if feature else 0,
+               int(scoring_bf16),
                gamma, beta_m,
                beta_v, epsilon, weight_decay, loss_scale, softmax_correction_weight,
                negative_adversarial_scale, lr_mod_entity, lr_mod_relation, lr_mod_projection,
@@ -235,12 +236,14 @@ class Oracle:
         for k in ("entity_data", "relation_embedding", "relation_embedding/adam_m",
                   "relation_embedding/adam_v"):
             assert state[k].dtype == np.float32 and state[k].flags.c_contiguous, k
+        mlp = ("mlp_up_projection", "mlp_down_projection") if cfg.feature and cfg.mlp_size else ()
         if cfg.feature:
-            proj = [state["feature_projection"], state["feature_projection/adam_m"],
-                    state["feature_projection/adam_v"]]
-            for a in proj:
+            # with a feature MLP the C side takes W, Up and Down back to back
+            proj_arrays = [np.concatenate([_f32(state[n + x]).reshape(-1) for n in ("feature_projection",) + mlp])
+                           if mlp else state["feature_projection" + x] for x in ("", "/adam_m", "/adam_v")]
+            for a in proj_arrays:
                 assert a.dtype == np.float32 and a.flags.c_contiguous
-            proj = [_p(a) for a in proj]
+            proj = [_p(a) for a in proj_arrays]
         else:
             proj = [None, None, None]
         step = C.c_uint32(int(state["step"]))
@@ -263,6 +266,12 @@ class Oracle:
             for x, a in zip(suffixes, rel):
                 state["relation_embedding" + x][...] = a[:n]
                 state["relation_normal" + x][...] = a[n:]
+        if mlp:
+            for x, a in zip(("", "/adam_m", "/adam_v"), proj_arrays):
+                o = 0
+                for n in ("feature_projection",) + mlp:
+                    state[n + x][...] = a[o:o + state[n + x].size].reshape(state[n + x].shape)
+                    o += state[n + x].size
         state["step"] = step.value
         return loss
 
@@ -279,7 +288,11 @@ def predict_reference(cfg, state, queries, shard_to_count, n_best):
     rows = np.asarray(state["entity_data"], np.float64).reshape(S * NE, -1)
     hidden = rows[:, :D].copy()
     if F:
-        hidden += rows[:, 3 * D:3 * D + F] @ np.asarray(state["feature_projection"], np.float64)
+        fh = rows[:, 3 * D:3 * D + F] @ np.asarray(state["feature_projection"], np.float64)
+        if cfg.mlp_size:  # src/poplar_kge.cpp:453-458
+            boom = np.maximum(np.concatenate([hidden, fh], 1) @ np.asarray(state["mlp_up_projection"], np.float64), 0)
+            fh = boom @ np.asarray(state["mlp_down_projection"], np.float64)
+        hidden += fh
     rel = np.asarray(state["relation_embedding"], np.float64)
     q = np.asarray(queries, np.int64)
     h = hidden[q[:, 0] * NE + q[:, 1]]

@@ -9,7 +9,7 @@ def cfg_dict(**kw):
              storage="float32", scoring_bf16=False, gamma=2.0, beta_m=0.9, beta_v=0.999, epsilon=1e-8,
              weight_decay=0.0, loss_scale=None, softmax_correction_weight=0.0,
              negative_adversarial_scale=0.0, embedding_regularisation=(3.0, 0.0),
-             feature_regularisation=(3.0, 0.0), hidden_regularisation=(3.0, 0.0))
+             feature_regularisation=(3.0, 0.0), hidden_regularisation=(3.0, 0.0), feature_mlp_size=0)
     d.update(kw)
     if d["loss_scale"] is None:
         d["loss_scale"] = float(d["batch"] * d["n_shard"] * d["a2a"])
@@ -49,6 +49,12 @@ def make_state(c, rng, warm=True, scale=None):
         st["feature_projection"] = rng.normal(0, scale / np.sqrt(F), (F, D)).astype(np.float32)
         st["feature_projection/adam_m"] = (rng.normal(0, 0.1, (F, D)) * warm).astype(np.float32)
         st["feature_projection/adam_v"] = ((0.05 + np.abs(rng.normal(0, 0.3, (F, D))))**2 * warm).astype(np.float32)
+        M = c.get("feature_mlp_size", 0)
+        if M:  # shapes and scales of src/python/poplar_kge.py:665-686
+            for name, shape in (("mlp_up_projection", (2 * D, M)), ("mlp_down_projection", (M, D))):
+                st[name] = rng.normal(0, 1 / np.sqrt(shape[0]), shape).astype(np.float32)
+                st[name + "/adam_m"] = (rng.normal(0, 0.1, shape) * warm).astype(np.float32)
+                st[name + "/adam_v"] = ((0.05 + np.abs(rng.normal(0, 0.3, shape)))**2 * warm).astype(np.float32)
     return st
 
 

@@ -310,6 +310,13 @@ STEP_CASES = {
                                 softmax_correction_weight=1.0),
     "transh_shared_table": dict(score_fn="TransH", shared_table=True, n_shard=4, batch=8, a2a=4,
                                 feature=0, n_entity=60, gamma=3.0),
+    # feature MLP (src/poplar_kge.cpp:453-458): relu([embedding | feature . W] . Up) . Down
+    "feature_mlp": dict(feature_mlp_size=10),
+    "feature_mlp_l2_softmax_reg": dict(feature_mlp_size=6, distance_fn="L2", loss_fn="softmax",
+                                       softmax_correction_weight=1.0, feature_regularisation=(3.0, 2e-2),
+                                       hidden_regularisation=(2.0, 1e-2)),
+    "feature_mlp_shared_distmult": dict(feature_mlp_size=8, score_fn="DistMult", distance_fn="MatMul",
+                                        shared_table=True, n_shard=4, batch=8, a2a=4, feature=4, n_entity=60),
     # norm regularisers (src/poplar_kge.cpp:430-437, 463-465), the WikiKG preset's among them
     "feature_regularisation_p3": dict(feature_regularisation=(3.0, 1e-2), loss_fn="softmax",
                                       softmax_correction_weight=1.0),

@@ -98,6 +98,14 @@ def step(cfg, state, lr, batch_step):
         params.append(proj)
         if cfg.get("scoring_bf16"):
             hidden_u = emb + round_bf16_ste(feat) @ round_bf16_ste(proj)
+        elif cfg.get("feature_mlp_size"):
+            # src/poplar_kge.cpp:453-458; max(x, 0) whose gradient passes where input == output,
+            # so also at exactly 0 (src/pag/pag.cpp:650-658), which `where` reproduces
+            up = T.tensor(state["mlp_up_projection"].astype(np.float64), requires_grad=True)
+            down = T.tensor(state["mlp_down_projection"].astype(np.float64), requires_grad=True)
+            params += [up, down]
+            pre = T.cat([emb, feat @ proj], 1) @ up
+            hidden_u = emb + T.where(pre >= 0, pre, T.zeros_like(pre)) @ down
         else:
             hidden_u = emb + feat @ proj
     else:
@@ -216,4 +224,7 @@ def step(cfg, state, lr, batch_step):
         dense("relation_normal", normal.grad.numpy())
     if F:
         dense("feature_projection", proj.grad.numpy())
+        if cfg.get("feature_mlp_size"):
+            dense("mlp_up_projection", up.grad.numpy())
+            dense("mlp_down_projection", down.grad.numpy())
     return per_shard.detach().numpy().astype(np.float32)
