@@ -188,10 +188,11 @@ struct kge_engine {
     // TransH keeps a second row per relation, the hyperplane normal (relation_normal), as rows
     // [n_rel, 2 n_rel) of the relation table: rel_copies = 2, n_rel_rows = 2 n_rel
     int rel_copies = 1, n_rel_rows = 0;
+    int mlp = 0;  // model.feature_mlp_size: hidden = value + relu([value | feature . W] . Up) . Down
     int score_fn, dist_fn, loss_fn;
     bool shared_table;
     float gamma, init_scale, beta_m, beta_v, epsilon, weight_decay, loss_scale, softmax_cw, neg_adv;
-    float lr_mod_entity = 1.f, lr_mod_rel = 1.f, lr_mod_proj = 1.f, lr_mod_normal = 1.f;
+    float lr_mod_entity = 1.f, lr_mod_rel = 1.f, lr_mod_proj = 1.f, lr_mod_normal = 1.f, lr_mod_up = 1.f, lr_mod_down = 1.f;
     uint32_t seed;
     int n_step, rw_batch;
     int predict_hr_batch = 0, predict_n_best = 0;
@@ -235,9 +236,14 @@ struct kge_engine {
     float reg_p[3] = {3.f, 3.f, 3.f}, reg_w[3] = {0.f, 0.f, 0.f};
     bool reg_on = false;
     DevBuf<float> reg_val, reg_fh, reg_loss_row, reg_loss_part;
+    // feature MLP: Up [2 Dp, M] and Down [M, Dp] with their moments and gradients; per distinct
+    // row the projected features, the MLP's input, the pre-activations, their gradient, the
+    // projected features' gradient and what the embedding's update must add
+    DevBuf<float> up, up_m, up_v, down, down_m, down_v, g_up, g_down;
+    DevBuf<float> mlp_fproj, mlp_concat, mlp_pre, mlp_gpre, mlp_gfp, mlp_gval, p_fproj, p_concat, p_pre;
     DevBuf<float> opnd_n, cmat, dcm, transh_mm, relgrad;  // TransH: [n | tails], c, d loss / d c, its products, relation contributions
     DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, d_loss, d_alpha;
-    // [n_step][entity, relation, normal, projection][S]; the relation update indexes its two
+    // [n_step][entity, relation, normal, projection, mlp up, mlp down][S]; the relation update indexes its two
     // groups as one array (key / rows_per_alpha), a shared table's [relation, normal] pair
     // sits in the first two entries of the relation group
     std::vector<float> h_alpha;
@@ -389,7 +395,13 @@ void parse_settings(kge_engine& E, const Items& s) {
     else
         throw std::invalid_argument("'training.loss.type' must be one of 'logsigmoid' or 'softmax', not '" +
                                     loss + "'");
-    if (mlp > 0) throw std::invalid_argument("'model.feature_mlp_size' > 0 is not implemented on the HIP device");
+    if (mlp > 0 && E.F == 0)
+        throw std::invalid_argument("'model.feature_mlp_size' > 0 is implemented with entity features only "
+                                    "('model.entity_feature_size' > 0)");
+    if (mlp > 0 && E.score_bf16)
+        throw std::invalid_argument("'model.feature_mlp_size' > 0 is not implemented together with "
+                                    "'execution.scoring_dtype' = 'bfloat16'");
+    E.mlp = (int)mlp;
     if (dropout > 0) throw std::invalid_argument("'model.feature_dropout' > 0 is not implemented on the HIP device");
     if (!share && E.F > 0)
         throw std::invalid_argument("'model.share_feature_networks' = false is not implemented on the HIP device");
@@ -413,6 +425,10 @@ void parse_settings(kge_engine& E, const Items& s) {
         };
         check("relation_embedding", E.n_rel, E.score_fn == SCORE_ROTATE ? E.D / 2 : E.D);
         check("feature_projection", E.F, E.D);
+        if (E.mlp) {
+            check("mlp_up_projection", 2 * E.D, E.mlp);
+            check("mlp_down_projection", E.mlp, E.D);
+        }
     }
     E.n_rel_rows = E.n_rel * E.rel_copies;
     for (size_t i = 0; i < mods.map_len; ++i) {
@@ -421,6 +437,8 @@ void parse_settings(kge_engine& E, const Items& s) {
         else if (k == "relation_embedding") E.lr_mod_rel = mods.map_vals[i];
         else if (k == "feature_projection") E.lr_mod_proj = mods.map_vals[i];
         else if (k == "relation_normal" && E.score_fn == SCORE_TRANSH) E.lr_mod_normal = mods.map_vals[i];
+        else if (k == "mlp_up_projection" && E.mlp) E.lr_mod_up = mods.map_vals[i];
+        else if (k == "mlp_down_projection" && E.mlp) E.lr_mod_down = mods.map_vals[i];
         else
             throw std::invalid_argument("Bad training.learning_rate_modifier: unknown parameter '" + k + "'");
     }
@@ -453,6 +471,10 @@ void parse_settings(kge_engine& E, const Items& s) {
         if (E.score_fn == SCORE_TRANSH)  // :252-255
             var(std::string("relation_normal") + suffix, {(size_t)E.n_rel, (size_t)E.D});
         var(std::string("feature_projection") + suffix, {(size_t)E.F, (size_t)E.D});
+        if (E.mlp) {  // :260-265
+            var(std::string("mlp_up_projection") + suffix, {(size_t)(2 * E.D), (size_t)E.mlp});
+            var(std::string("mlp_down_projection") + suffix, {(size_t)E.mlp, (size_t)E.D});
+        }
     }
 }
 
@@ -549,6 +571,19 @@ void allocate(kge_engine& E) {
             E.projR.alloc((size_t)E.Fp * E.Dp);
         }
         E.gproj.alloc(proj_n);
+        if (E.mlp) {
+            const size_t M = E.mlp, up_n = 2 * (size_t)E.Dp * M, down_n = M * E.Dp;
+            for (DevBuf<float>* b : {&E.up, &E.up_m, &E.up_v, &E.g_up}) { b->alloc(up_n); b->zero(st); }
+            for (DevBuf<float>* b : {&E.down, &E.down_m, &E.down_v, &E.g_down}) { b->alloc(down_n); b->zero(st); }
+            E.mlp_fproj.alloc(R * E.Dp);
+            E.mlp_concat.alloc(R * 2 * E.Dp);
+            E.mlp_pre.alloc(R * M);
+            E.mlp_gpre.alloc(R * M);
+            E.mlp_gfp.alloc(R * E.Dp);
+            E.mlp_gval.alloc(R * E.Dp);
+            // rows past a step's distinct count are read by the projection gradient (times zero)
+            E.mlp_gfp.zero(st);
+        }
     }
     ScoreShape sh = {};
     sh.S = E.S; sh.B = E.B; sh.T = E.T;
@@ -566,7 +601,7 @@ void allocate(kge_engine& E) {
     }
     E.loss_part.alloc(ns * S * E.n_part);
     E.d_loss.alloc(S);
-    E.d_alpha.alloc(ns * 4 * S);
+    E.d_alpha.alloc(ns * 6 * S);
 
     const size_t io_n = (size_t)E.S * E.rw_batch;
     E.io_rows.alloc(io_n);
@@ -603,6 +638,23 @@ void run_read_write(kge_engine& E, bool write, const Items& in) {
     const size_t rows = var->shape[0], cols = var->shape[1];
     if (rows == 0 || cols == 0) return;
     HIP_CHECK(hipStreamSynchronize(E.stream));
+    if (name.rfind("mlp_", 0) == 0) {
+        const bool is_up = name.rfind("mlp_up_projection", 0) == 0;
+        const bool m = name.size() > 7 && name.compare(name.size() - 7, 7, "/adam_m") == 0;
+        const bool v = name.size() > 7 && name.compare(name.size() - 7, 7, "/adam_v") == 0;
+        float* dev = is_up ? (m ? E.up_m.p : v ? E.up_v.p : E.up.p) : (m ? E.down_m.p : v ? E.down_v.p : E.down.p);
+        // Up: host rows [0, D) and [D, 2 D) are device rows [0, D) and [Dp, Dp + D), pitch M;
+        // Down: host [M, D] in device rows of pitch Dp
+        const size_t D = E.D, Dp = E.Dp, M = E.mlp;
+        for (int half = 0; half < (is_up ? 2 : 1); ++half) {
+            float* d = dev + (is_up ? (size_t)half * Dp * M : 0);
+            float* h = host + (is_up ? (size_t)half * D * M : 0);
+            const size_t dpitch = (is_up ? M : Dp) * 4, hpitch = cols * 4, n = is_up ? D : M;
+            if (write) HIP_CHECK(hipMemcpy2D(d, dpitch, h, hpitch, cols * 4, n, hipMemcpyHostToDevice));
+            else HIP_CHECK(hipMemcpy2D(h, hpitch, d, dpitch, cols * 4, n, hipMemcpyDeviceToHost));
+        }
+        return;
+    }
     if (write)
         HIP_CHECK(hipMemcpy2D(buf->p + row0 * E.Dp, (size_t)E.Dp * 4, host, cols * 4, cols * 4, rows, hipMemcpyHostToDevice));
     else
@@ -833,6 +885,7 @@ void run_step(kge_engine& E, int i) {
     RowSource ent = table_rows;
 
     FeatureArgs fa = {};
+    MlpArgs ma = {};
     if (E.F) {
         fa.uniq_key = e_uniq; fa.counts = e_counts; fa.max_rows = (int)R;
         fa.emb_base = E.table.p; fa.feat_base = E.table.p + E.L.off_f; fa.pitch = E.L.pitch;
@@ -841,6 +894,17 @@ void run_step(kge_engine& E, int i) {
         fa.featd = E.featd.p; fa.gproj_part = E.gproj_part.p; fa.use_mfma = E.use_mfma;
         fa.round_bf16 = E.score_bf16 ? 1 : 0; fa.projR = E.projR.p;
         fa.feat16 = E.feat16.p; fa.featT16 = E.featT16.p; fa.projT16 = E.projT16.p; fa.gT16 = E.gT16.p;
+        if (E.mlp) {  // feature . W alone, then the MLP on [embedding | feature . W]
+            KernelTimer t(E, K_HIDDEN);
+            FeatureArgs fp = fa;
+            fp.emb_base = nullptr;
+            launch_hidden_fwd(fp, E.mlp_fproj.p, st);
+            ma.uniq_key = e_uniq; ma.counts = e_counts; ma.max_rows = (int)R;
+            ma.emb_base = E.table.p; ma.pitch = E.L.pitch; ma.emb_etype = E.L.emb_etype;
+            ma.Dp = E.Dp; ma.M = E.mlp; ma.up = E.up.p; ma.down = E.down.p;
+            ma.concat = E.mlp_concat.p; ma.pre = E.mlp_pre.p;
+            launch_mlp_fwd(ma, E.mlp_fproj.p, E.hidden.p, st);
+        } else
         { KernelTimer t(E, K_HIDDEN); launch_hidden_fwd(fa, E.hidden.p, st); }
         ent.base = (const char*)E.hidden.p; ent.pitch = (int64_t)E.Dp * 4; ent.etype = ET_F32;
         ent.index = E.e_item_row.p + i * R;
@@ -946,7 +1010,7 @@ void run_step(kge_engine& E, int i) {
                         E.reg_loss_part.p + (size_t)i * E.S, st);
     }
 
-    const float* alpha = E.d_alpha.p + (size_t)i * 4 * E.S;
+    const float* alpha = E.d_alpha.p + (size_t)i * 6 * E.S;
     AdamArgs aa = {};
     aa.Dp = E.Dp;
     aa.beta_m = E.beta_m; aa.beta_v = E.beta_v;
@@ -1014,6 +1078,21 @@ void run_step(kge_engine& E, int i) {
     ae.alpha = alpha;
     ae.rows_per_alpha = E.shared_table ? 0u : (uint32_t)E.n_entity;
 
+    // The feature MLP's input holds the embedding, so part of the embedding's gradient comes
+    // back through the MLP: the rows' summed gradient first (a pass without update), the MLP's
+    // backward per row, then the update with what that adds.
+    auto entity_update = [&]() {
+        KernelTimer t(E, K_ADAM_ENT);
+        if (!E.mlp) { launch_adam_rows(ae, st); return; }
+        AdamArgs sum = ae;
+        sum.no_update = 1;
+        launch_adam_rows(sum, st);
+        launch_mlp_bwd_rows(ma, E.gsum.p, E.reg_on ? E.reg_val.p : nullptr, E.mlp_gpre.p, E.mlp_gval.p,
+                            E.mlp_gfp.p, st);
+        AdamArgs upd = ae;
+        upd.grad_out = nullptr; upd.grad_out_add = nullptr; upd.grad_add = E.mlp_gval.p;
+        launch_adam_rows(upd, st);
+    };
     if (contributions_read_tables(E)) {
         // entity update first (reads pre-update relation rows), writing its summed
         // gradient is not needed; then the relation update reads POST-update entity
@@ -1021,17 +1100,63 @@ void run_step(kge_engine& E, int i) {
         ar.grad_out = E.rel_gsum.p;
         ar.no_update = 1;
         { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
-        { KernelTimer t(E, K_ADAM_ENT); launch_adam_rows(ae, st); }
+        entity_update();
         ar.grad_out = nullptr; ar.no_update = 0;
         ar.grad_direct = E.rel_gsum.p;
         { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
+    } else if (E.mlp) {
+        entity_update();
+        KernelTimer t(E, K_ADAM_REL);
+        launch_adam_rows(ar, st);
     } else {
         KernelTimer t(E, K_ADAM_ENT);
         launch_adam_rows2(ae, ar, st);
     }
 
+    // dense Adam on rows [0, rows) of a parameter whose row r sits at device element
+    // offset(r); shard s owns rows [s*rows/S, (s+1)*rows/S) and its step size
+    auto dense_adam = [&](float* p, float* m, float* v, const float* g, int rows, int64_t width, int group) {
+        const int n_slices = E.shared_table ? 1 : E.S;
+        for (int s = 0; s < n_slices; ++s) {
+            const int r0 = E.shared_table ? 0 : s * (rows / E.S);
+            const int r1 = (E.shared_table || s == E.S - 1) ? rows : (s + 1) * (rows / E.S);
+            if (r1 <= r0) continue;
+            const size_t o = (size_t)r0 * width;
+            launch_adam_flat(p + o, m + o, v + o, g + o, (int64_t)(r1 - r0) * width,
+                             E.h_alpha[((size_t)i * 6 + group) * E.S + s], E.beta_m, E.beta_v, E.epsilon,
+                             E.weight_decay, 0, st);
+        }
+    };
+    if (E.mlp) {
+        KernelTimer t(E, K_PROJ_GRAD);
+        // d Down = relu(pre)^T . g, d Up = concat^T . gpre, summed over the distinct rows in order
+        launch_rows_atb(E.mlp_pre.p, E.mlp, E.mlp, true, E.gsum.p, E.Dp, E.Dp, e_counts, E.g_down.p, st);
+        launch_rows_atb(E.mlp_concat.p, 2 * E.Dp, 2 * E.Dp, false, E.mlp_gpre.p, E.mlp, E.mlp, e_counts,
+                        E.g_up.p, st);
+    }
+    if (E.mlp) {
+        KernelTimer t(E, K_ADAM_PROJ);
+        // Up's host rows [0, D) and [D, 2 D) are device rows [0, D) and [Dp, Dp + D): a shard's
+        // slice of host rows is updated half by half
+        const int n_slices = E.shared_table ? 1 : E.S, rows = 2 * E.D;
+        for (int s = 0; s < n_slices; ++s) {
+            const int r0 = E.shared_table ? 0 : s * (rows / E.S);
+            const int r1 = (E.shared_table || s == E.S - 1) ? rows : (s + 1) * (rows / E.S);
+            for (int half = 0; half < 2; ++half) {
+                const int lo = std::max(r0, half * E.D), hi = std::min(r1, (half + 1) * E.D);
+                if (hi <= lo) continue;
+                const size_t o = (size_t)(lo + half * (E.Dp - E.D)) * E.mlp;
+                launch_adam_flat(E.up.p + o, E.up_m.p + o, E.up_v.p + o, E.g_up.p + o, (int64_t)(hi - lo) * E.mlp,
+                                 E.h_alpha[((size_t)i * 6 + 4) * E.S + s], E.beta_m, E.beta_v, E.epsilon,
+                                 E.weight_decay, 0, st);
+            }
+        }
+        dense_adam(E.down.p, E.down_m.p, E.down_v.p, E.g_down.p, E.mlp, E.Dp, 5);
+    }
+
     if (E.F) {
-        { KernelTimer t(E, K_PROJ_GRAD); launch_proj_grad(fa, E.gsum.p, E.gproj.p, st); }
+        { KernelTimer t(E, K_PROJ_GRAD);
+          launch_proj_grad(fa, E.mlp ? E.mlp_gfp.p : E.gsum.p, E.gproj.p, st); }
         // dense Adam on the projection; shard s owns rows [s*F/S, (s+1)*F/S) and its step size
         KernelTimer t(E, K_ADAM_PROJ);
         const int n_slices = E.shared_table ? 1 : E.S;
@@ -1041,7 +1166,7 @@ void run_step(kge_engine& E, int i) {
             if (r1 <= r0) continue;
             const size_t o = (size_t)r0 * E.Dp;
             launch_adam_flat(E.proj.p + o, E.proj_m.p + o, E.proj_v.p + o, E.gproj.p + o,
-                             (int64_t)(r1 - r0) * E.Dp, E.h_alpha[((size_t)i * 4 + 3) * E.S + s],
+                             (int64_t)(r1 - r0) * E.Dp, E.h_alpha[((size_t)i * 6 + 3) * E.S + s],
                              E.beta_m, E.beta_v, E.epsilon, E.weight_decay, 0, st);
         }
     }
@@ -1076,21 +1201,23 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
         throw std::invalid_argument("train_step_loop with staged=true needs a preceding stage_batch");
     }
     // step sizes of every step of this call (adamStepSizeAutoIncrement, frnn.cpp:42-59)
-    E.h_alpha.resize((size_t)E.n_step * 4 * S);
+    E.h_alpha.resize((size_t)E.n_step * 6 * S);
     for (int i = s0; i < s0 + sn; ++i) {
         const double t = (double)(E.step + (uint32_t)(i - s0) + 1u);
         const double factor = std::sqrt(1.0 - std::pow((double)E.beta_v, t)) / (1.0 - std::pow((double)E.beta_m, t));
         for (size_t s = 0; s < S; ++s) {
             const float a = (float)(factor * (double)lr[s]);
-            E.h_alpha[((size_t)i * 4 + 0) * S + s] = a * E.lr_mod_entity;
-            E.h_alpha[((size_t)i * 4 + 1) * S + s] = a * E.lr_mod_rel;
-            E.h_alpha[((size_t)i * 4 + 2) * S + s] = a * E.lr_mod_normal;
-            E.h_alpha[((size_t)i * 4 + 3) * S + s] = a * E.lr_mod_proj;
+            E.h_alpha[((size_t)i * 6 + 0) * S + s] = a * E.lr_mod_entity;
+            E.h_alpha[((size_t)i * 6 + 1) * S + s] = a * E.lr_mod_rel;
+            E.h_alpha[((size_t)i * 6 + 2) * S + s] = a * E.lr_mod_normal;
+            E.h_alpha[((size_t)i * 6 + 3) * S + s] = a * E.lr_mod_proj;
+            E.h_alpha[((size_t)i * 6 + 4) * S + s] = a * E.lr_mod_up;
+            E.h_alpha[((size_t)i * 6 + 5) * S + s] = a * E.lr_mod_down;
         }
         // a shared table has one step size per parameter: the relation update finds the
         // normal rows' at index 1 of its array
         if (E.shared_table && E.score_fn == SCORE_TRANSH)
-            E.h_alpha[((size_t)i * 4 + 1) * S + 1] = (float)(factor * (double)lr[0]) * E.lr_mod_normal;
+            E.h_alpha[((size_t)i * 6 + 1) * S + 1] = (float)(factor * (double)lr[0]) * E.lr_mod_normal;
     }
     HIP_CHECK(hipMemcpyAsync(E.d_alpha.p, E.h_alpha.data(), E.h_alpha.size() * 4, hipMemcpyHostToDevice, st));
     HIP_CHECK(hipEventRecord(E.ev[1], st));
@@ -1197,6 +1324,11 @@ void run_predict(kge_engine& E, const Items& in) {
         if (E.F) {
             E.p_hidden.alloc((size_t)std::max(Qp, chunk) * Dp);
             E.p_featd.alloc((size_t)std::max(Qp, chunk) * E.Fp);
+            if (E.mlp) {
+                E.p_fproj.alloc((size_t)std::max(Qp, chunk) * Dp);
+                E.p_concat.alloc((size_t)std::max(Qp, chunk) * 2 * Dp);
+                E.p_pre.alloc((size_t)std::max(Qp, chunk) * E.mlp);
+            }
         }
     }
     HIP_CHECK(hipMemcpyAsync(E.p_idx.p, rows.data(), (size_t)Qp * 4, hipMemcpyHostToDevice, st));
@@ -1217,6 +1349,17 @@ void run_predict(kge_engine& E, const Items& in) {
             fa.emb_etype = E.L.emb_etype; fa.feat_etype = E.L.feat_etype;
             fa.Dp = Dp; fa.Fp = E.Fp; fa.proj = E.proj.p;
             fa.featd = E.p_featd.p; fa.use_mfma = E.use_mfma;
+            if (E.mlp) {
+                FeatureArgs fp = fa;
+                fp.emb_base = nullptr;
+                launch_hidden_fwd(fp, E.p_fproj.p, st);
+                MlpArgs ma = {};
+                ma.uniq_key = idx; ma.counts = E.p_count.p; ma.max_rows = n;
+                ma.emb_base = E.table.p; ma.pitch = E.L.pitch; ma.emb_etype = E.L.emb_etype;
+                ma.Dp = Dp; ma.M = E.mlp; ma.up = E.up.p; ma.down = E.down.p;
+                ma.concat = E.p_concat.p; ma.pre = E.p_pre.p;
+                launch_mlp_fwd(ma, E.p_fproj.p, E.p_hidden.p, st);
+            } else
             launch_hidden_fwd(fa, E.p_hidden.p, st);
             r.base = (const char*)E.p_hidden.p; r.pitch = (int64_t)Dp * 4; r.etype = ET_F32; r.index = nullptr;
         }

@@ -254,7 +254,7 @@ struct FeatureArgs {
     const uint32_t* uniq_key;
     const uint32_t* counts;
     int max_rows;
-    const char* emb_base;   // table + emb offset
+    const char* emb_base;   // table + emb offset; null: launch_hidden_fwd leaves the embedding out
     const char* feat_base;  // table + feature offset
     int64_t pitch;
     int emb_etype, feat_etype;
@@ -347,5 +347,24 @@ void launch_transh_bwd(const TranshBwd& p, hipStream_t stream);
 // embedding rows' contributions, rows [n_head, 2 n_head) the normal rows'
 void launch_transh_back(const RowSource& ent, const float* rel, const uint32_t* crel, int n_rel, int n_head,
                         int Dp, float* grad, const float* mm, float* relgrad, hipStream_t stream);
+
+// ---- feature MLP (src/poplar_kge.cpp:453-458) ----
+// hidden = value + relu([value | feature . W] . Up) . Down per distinct row
+struct MlpArgs {
+    const uint32_t* uniq_key; const uint32_t* counts; int max_rows;
+    const char* emb_base; int64_t pitch; int emb_etype;
+    int Dp, M;
+    const float* up;    // [2 Dp, M]: rows [0, Dp) the embedding's, [Dp, 2 Dp) the projected features'
+    const float* down;  // [M, Dp]
+    float* concat;      // [max_rows, 2 Dp] the MLP's input (written by the forward)
+    float* pre;         // [max_rows, M] pre-activations (written by the forward)
+};
+// fproj [max_rows, Dp] = feature . W (launch_hidden_fwd with a null emb_base)
+void launch_mlp_fwd(const MlpArgs& a, const float* fproj, float* hidden, hipStream_t stream);
+void launch_mlp_bwd_rows(const MlpArgs& a, const float* g, const float* val_add, float* gpre, float* gval,
+                         float* gfproj, hipStream_t stream);
+// C [Ka, N] = f(A [rows, Ka])^T . B [rows, N] over the first *count rows, summed in row order
+void launch_rows_atb(const float* A, int lda, int Ka, bool relu, const float* B, int ldb, int N,
+                     const uint32_t* count, float* C, hipStream_t stream);
 
 }  // namespace kge

@@ -2715,7 +2715,7 @@ __global__ __launch_bounds__(256) void k_hidden_fwd(FeatureArgs a, float* __rest
     const char* erow = a.emb_base + (int64_t)key * a.pitch;
     const char* frow = a.feat_base + (int64_t)key * a.pitch;
     for (int k = lane * 4; k < a.Dp; k += 256) {
-        float4 h = load4(erow, k, a.emb_etype);
+        float4 h = a.emb_base ? load4(erow, k, a.emb_etype) : make_float4(0, 0, 0, 0);
         for (int f = 0; f < a.Fp; f += 4) {
             float4 x = load4(frow, f, a.feat_etype);
             if (a.round_bf16) x = round4_bf16(x);
@@ -3515,6 +3515,106 @@ void launch_transh_back(const RowSource& ent, const float* rel, const uint32_t* 
                         int Dp, float* grad, const float* mm, float* relgrad, hipStream_t stream) {
     hipLaunchKernelGGL(k_transh_back, dim3((n_head + 3) / 4), dim3(256), 0, stream, ent, rel, crel, n_rel, n_head,
                        Dp, grad, mm, relgrad);
+}
+
+// --------------------------------------------------------------------------
+// Feature MLP (src/poplar_kge.cpp:453-458): per distinct row,
+//   hidden = value + relu([value | feature . W] . Up) . Down,   Up [2 Dp, M], Down [M, Dp]
+// (device rows of Up: [0, Dp) the embedding's, [Dp, 2 Dp) the projected features').  Plain
+// vector kernels, one workgroup per row: written for correctness, no benchmark workload uses it.
+
+// concat[u] = [embedding | fproj[u]], pre[u] = concat . Up, hidden[u] = embedding + relu(pre) . Down
+__global__ __launch_bounds__(256) void k_mlp_fwd(MlpArgs a, const float* __restrict__ fproj,
+                                                 float* __restrict__ hidden) {
+    extern __shared__ float mlp_sm[];
+    float* cc = mlp_sm;
+    float* boom = mlp_sm + 2 * a.Dp;
+    const int u = blockIdx.x, tid = threadIdx.x, Dp = a.Dp, M = a.M;
+    if (u >= (int)a.counts[0]) return;
+    const char* erow = a.emb_base + (int64_t)a.uniq_key[u] * a.pitch;
+    for (int i = tid; i < Dp; i += 256) {
+        const float e = load1(erow, i, a.emb_etype), f = fproj[(size_t)u * Dp + i];
+        cc[i] = e; cc[Dp + i] = f;
+        a.concat[(size_t)u * 2 * Dp + i] = e;
+        a.concat[(size_t)u * 2 * Dp + Dp + i] = f;
+    }
+    __syncthreads();
+    for (int m = tid; m < M; m += 256) {
+        float acc = 0.f;
+        for (int i = 0; i < 2 * Dp; ++i) acc = fmaf(cc[i], a.up[(size_t)i * M + m], acc);
+        a.pre[(size_t)u * M + m] = acc;
+        boom[m] = fmaxf(acc, 0.f);
+    }
+    __syncthreads();
+    for (int k = tid; k < Dp; k += 256) {
+        float acc = 0.f;
+        for (int m = 0; m < M; ++m) acc = fmaf(boom[m], a.down[(size_t)m * Dp + k], acc);
+        hidden[(size_t)u * Dp + k] = cc[k] + acc;
+    }
+}
+void launch_mlp_fwd(const MlpArgs& a, const float* fproj, float* hidden, hipStream_t stream) {
+    hipLaunchKernelGGL(k_mlp_fwd, dim3(a.max_rows), dim3(256), (size_t)(2 * a.Dp + a.M) * 4, stream, a, fproj,
+                       hidden);
+}
+
+// From g[u] = d loss / d (MLP output): gpre[u] = (g . Down^T) where pre >= 0 (the reference's max
+// passes the gradient where input == output, so also at exactly 0: src/pag/pag.cpp:650-658);
+// d concat = gpre . Up^T, whose first half (+ val_add[u], or null) is what the embedding's update
+// must add (-> gval) and whose second half is the projected features' gradient (-> gfproj)
+__global__ __launch_bounds__(256) void k_mlp_bwd_rows(MlpArgs a, const float* __restrict__ g,
+                                                      const float* __restrict__ val_add,
+                                                      float* __restrict__ gpre, float* __restrict__ gval,
+                                                      float* __restrict__ gfproj) {
+    extern __shared__ float mlp_sm[];
+    float* gs = mlp_sm;
+    float* gp = mlp_sm + a.Dp;
+    const int u = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, Dp = a.Dp, M = a.M;
+    if (u >= (int)a.counts[0]) return;
+    for (int k = tid; k < Dp; k += 256) gs[k] = g[(size_t)u * Dp + k];
+    __syncthreads();
+    for (int m = wave; m < M; m += 4) {
+        float part = 0.f;
+        for (int k = lane; k < Dp; k += 64) part = fmaf(gs[k], a.down[(size_t)m * Dp + k], part);
+        part = wave_sum(part);
+        const float v = a.pre[(size_t)u * M + m] >= 0.f ? part : 0.f;
+        if (lane == 0) { gpre[(size_t)u * M + m] = v; gp[m] = v; }
+    }
+    __syncthreads();
+    for (int i = wave; i < 2 * Dp; i += 4) {
+        float part = 0.f;
+        for (int m = lane; m < M; m += 64) part = fmaf(gp[m], a.up[(size_t)i * M + m], part);
+        part = wave_sum(part);
+        if (lane == 0) {
+            if (i < Dp) gval[(size_t)u * Dp + i] = part + (val_add ? val_add[(size_t)u * Dp + i] : 0.f);
+            else gfproj[(size_t)u * Dp + i - Dp] = part;
+        }
+    }
+}
+void launch_mlp_bwd_rows(const MlpArgs& a, const float* g, const float* val_add, float* gpre, float* gval,
+                         float* gfproj, hipStream_t stream) {
+    hipLaunchKernelGGL(k_mlp_bwd_rows, dim3(a.max_rows), dim3(256), (size_t)(a.Dp + a.M) * 4, stream, a, g,
+                       val_add, gpre, gval, gfproj);
+}
+
+// C[i, n] = sum over rows u < *count, in order, of f(A[u, i]) * B[u, n]; f = max(., 0) with `relu`
+__global__ __launch_bounds__(256) void k_rows_atb(const float* __restrict__ A, int lda, int relu,
+                                                  const float* __restrict__ B, int ldb, int N,
+                                                  const uint32_t* __restrict__ count, float* __restrict__ C) {
+    const int i = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
+    if (n >= N) return;
+    const int U = (int)count[0];
+    float acc = 0.f;
+    for (int u = 0; u < U; ++u) {
+        float x = A[(size_t)u * lda + i];
+        if (relu) x = fmaxf(x, 0.f);
+        acc = fmaf(x, B[(size_t)u * ldb + n], acc);
+    }
+    C[(size_t)i * N + n] = acc;
+}
+void launch_rows_atb(const float* A, int lda, int Ka, bool relu, const float* B, int ldb, int N,
+                     const uint32_t* count, float* C, hipStream_t stream) {
+    hipLaunchKernelGGL(k_rows_atb, dim3((N + 255) / 256, Ka), dim3(256), 0, stream, A, lda, relu ? 1 : 0, B, ldb,
+                       N, count, C);
 }
 
 }  // namespace kge

@@ -404,6 +404,10 @@ class Engine:
             "feature_projection",
             (self.init_scale / np.sqrt(max(m.entity_feature_size, 1)))
             * self.random_normal((m.entity_feature_size, m.embedding_size)))
+        if m.feature_mlp_size > 0:   # reference :665-686
+            for name, shape in (("mlp_up_projection", (2 * m.embedding_size, m.feature_mlp_size)),
+                                ("mlp_down_projection", (m.feature_mlp_size, m.embedding_size))):
+                self.write_variable(name, (self.init_scale / np.sqrt(shape[0])) * self.random_normal(shape))
 
     def initialise_all(self, entity_features: np.ndarray) -> None:
         """Variables, then every table row in rw_batch_size chunks."""

@@ -98,6 +98,17 @@ CASES = {
                            n_entity=3000, n_relation=8, gamma=6.0),
     "transh_mid": dict(score_fn="TransH", n_shard=2, batch=70, a2a=45, dim=64, feature=0,
                        n_entity=2000, n_relation=10, gamma=6.0),
+    # feature MLP (src/poplar_kge.cpp:453-458): hidden = value + relu([value | feature . W] . Up) . Down
+    "feature_mlp": dict(feature_mlp_size=10),
+    "feature_mlp_l2_softmax_reg": dict(feature_mlp_size=6, distance_fn="L2", loss_fn="softmax",
+                                       softmax_correction_weight=1.0, feature_regularisation=(3.0, 2e-2),
+                                       hidden_regularisation=(2.0, 1e-2)),
+    "feature_mlp_shared_distmult": dict(feature_mlp_size=8, score_fn="DistMult", distance_fn="MatMul",
+                                        shared_table=True, n_shard=4, batch=8, a2a=4, feature=4, n_entity=60),
+    "feature_mlp_odd_dim": dict(feature_mlp_size=9, dim=10, feature=6, n_entity=41, batch=5, a2a=3,
+                                distance_fn="L2", n_shard=1),
+    "feature_mlp_aligned_transh": dict(feature_mlp_size=96, score_fn="TransH", n_shard=2, batch=128, a2a=64,
+                                       dim=64, feature=32, n_entity=3000, n_relation=8, gamma=6.0),
     "aligned_complex_l2_shared": dict(score_fn="ComplEx", distance_fn="L2", n_shard=4, batch=128, a2a=32,
                                       dim=128, feature=0, n_entity=2000, n_relation=8, shared_table=True),
 }

@@ -43,7 +43,7 @@ def _oracle_cfg(settings):
                     a2a=d.a2a_size, score_fn=m.score_fn, distance_fn=m.distance_fn,
                     loss_fn=t.loss.type, gamma=m.gamma, beta_m=t.adam_beta_m, beta_v=t.adam_beta_v,
                     epsilon=t.adam_epsilon, weight_decay=t.weight_decay, loss_scale=t.loss_scale,
-                    storage=storage)
+                    storage=storage, feature_mlp_size=m.feature_mlp_size)
 
 
 def _oracle_state(state):
@@ -165,7 +165,7 @@ def _random_queries(engine, n):
 
 
 @pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "complex", "rotate", "transh", "transh_big",
-                                     "no_features_big"])
+                                     "feature_mlp", "no_features_big"])
 def test_predict_vs_brute_force(variant):
     """Engine.predict against a float64 brute force over every row of every shard
     (the reference checks shapes, ranges and ordering, tests/python/test_poplar_kge.py:155-175,
@@ -186,6 +186,8 @@ def test_predict_vs_brute_force(variant):
         m.score_fn = "RotatE"
     elif variant == "transh":
         m.score_fn = "TransH"
+    elif variant == "feature_mlp":
+        m.feature_mlp_size = 24
     elif variant in ("no_features_big", "transh_big"):
         # several chunks of tails per shard, several query chunks, ragged counts
         m.n_entity, m.entity_feature_size, m.embedding_size, m.n_shard = 20000, 0, 32, 3
