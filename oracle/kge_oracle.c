@@ -76,7 +76,21 @@ typedef struct {
      * rows of (sum_k |x_k^power|)^(1/power), of the embedding, of feature . W and of
      * their sum; weight 0 = off                                                          */
     float reg_emb_power, reg_emb_weight, reg_feat_power, reg_feat_weight, reg_hid_power, reg_hid_weight;
+    /* feature dropout (poplar_kge.cpp:459-461; pag.cpp:596-617): the feature part of hidden times
+     * a keep mask / (1 - p), drawn separately for the rows' use as heads and as tails.  The
+     * reference's device random stream cannot be matched; the mask here is kge_dropout_keep, a
+     * hash of (seed, step, role, table row, column) that the HIP kernels evaluate identically. */
+    float dropout;
+    uint32_t dropout_seed;
 } kge_oracle_cfg;
+
+/* keep (1) or drop (0) element k of table row `key` in `role` (0 head, 1 tail) at optimiser step
+ * `step`: a 32-bit integer hash compared with p * 2^32 */
+API int kge_dropout_keep(uint32_t seed, uint32_t step, uint32_t role, uint32_t key, uint32_t k, float p) {
+    uint32_t x = key * 0x9E3779B1u + k * 0x85EBCA77u + role * 0xC2B2AE3Du + step * 0x27D4EB2Fu + seed * 0x165667B1u;
+    x ^= x >> 16; x *= 0x7FEB352Du; x ^= x >> 15; x *= 0x846CA68Bu; x ^= x >> 16;
+    return x >= (uint32_t)((double)p * 4294967296.0);
+}
 
 /* ------------------------------------------------------------------------ */
 /* lpnorm (poplar_kge.cpp:389-391): pow(sum(abs(pow(a, p))), 1/p) of one row, and its
@@ -474,12 +488,23 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
      * the pre-activations, kept for the backward pass */
     REAL* fproj = M ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
     REAL* pre = M ? (REAL*)calloc((size_t)(S * NR * M), sizeof(REAL)) : NULL;
+    /* feature dropout: a slot's hidden row differs between its use as a head (`hidden`) and as
+     * a tail (`hidden_t`), and so do the gradients that come back (`ghid`, `ghid_t`); without
+     * dropout the two are the same arrays */
+    const int drop = F > 0 && c->dropout > 0;
+    const REAL keep_scale = drop ? 1 / (1 - (REAL)c->dropout) : 1;
+    REAL* hidden_t = drop ? (REAL*)malloc(sizeof(REAL) * (size_t)(S * NR * D)) : hidden;
+    REAL* ghid_t = drop ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : ghid;
+    /* whether the dropout's output is non-zero (what its backward tests), per use */
+    uint8_t* live_h = drop ? (uint8_t*)malloc((size_t)(S * NR * D)) : NULL;
+    uint8_t* live_t = drop ? (uint8_t*)malloc((size_t)(S * NR * D)) : NULL;
+    REAL* fhv = (REAL*)malloc(sizeof(REAL) * (size_t)D); /* one slot's feature part of hidden */
     for (int64_t s = 0; s < S; ++s)
         for (int64_t j = 0; j < NR; ++j) {
             const float* row = table + KEY(s, j) * ROW;
             REAL* h = hidden + (s * NR + j) * D;
-            REAL* fh = M ? fproj + (s * NR + j) * D : h;
-            for (int64_t k = 0; k < D; ++k) h[k] = row[k];
+            REAL* fh = M ? fproj + (s * NR + j) * D : fhv; /* feature . W */
+            for (int64_t k = 0; k < D; ++k) fhv[k] = 0;
             for (int64_t f = 0; f < F; ++f) {
                 /* bfloat16 scoring also takes the projection's operands in bfloat16 */
                 const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
@@ -495,15 +520,36 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                 }
                 for (int64_t m = 0; m < M; ++m)
                     if (a[m] > 0)
-                        for (int64_t k = 0; k < D; ++k) h[k] += a[m] * (REAL)down[m * D + k];
+                        for (int64_t k = 0; k < D; ++k) fhv[k] += a[m] * (REAL)down[m * D + k];
+            }
+            if (drop) { /* :459-461, once per entityHidden call: heads' and tails' masks differ */
+                REAL* ht = hidden_t + (s * NR + j) * D;
+                const uint32_t key = (uint32_t)KEY(s, j);
+                for (int64_t k = 0; k < D; ++k) {
+                    const int kh = kge_dropout_keep(c->dropout_seed, *step, 0, key, (uint32_t)k, c->dropout);
+                    const int kt = kge_dropout_keep(c->dropout_seed, *step, 1, key, (uint32_t)k, c->dropout);
+                    const REAL oh = kh ? fhv[k] * keep_scale : 0, ot = kt ? fhv[k] * keep_scale : 0;
+                    h[k] = (REAL)row[k] + oh;
+                    ht[k] = (REAL)row[k] + ot;
+                    live_h[(s * NR + j) * D + k] = oh != 0;
+                    live_t[(s * NR + j) * D + k] = ot != 0;
+                }
+            } else {
+                for (int64_t k = 0; k < D; ++k) h[k] = (REAL)row[k] + fhv[k]; /* :462 */
             }
         }
+    free(fhv);
 
     /* 1b. norm regularisers over every gathered slot (:463-465).  entityHidden runs once for
      * the heads and once for the tails on the same gathered rows and (shared networks) the
      * same projection, so every term counts twice (:676-678).  The embedding's gradient and
      * the feature product's gradient differ from here on: greg_val / greg_fh.              */
     const int reg_on = c->reg_emb_weight > 0 || c->reg_feat_weight > 0 || c->reg_hid_weight > 0;
+    if (reg_on && drop) { /* the regularised tensors would differ per use: not restated */
+        free(hidden); free(ghid); free(fproj); free(pre);
+        free(hidden_t); free(ghid_t); free(live_h); free(live_t);
+        return 2;
+    }
     REAL* greg_val = reg_on ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
     REAL* greg_fh = reg_on ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
     REAL* reg_loss = (REAL*)calloc((size_t)S, sizeof(REAL));
@@ -593,7 +639,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
          * is what shard j gathered with a2a[j][d][:]                        */
         for (int64_t j = 0; j < S; ++j)
             for (int64_t i = 0; i < A; ++i)
-                memcpy(tl + (j * A + i) * D, hidden + (j * NR + a2a[(j * S + d) * A + i]) * D,
+                memcpy(tl + (j * A + i) * D, hidden_t + (j * NR + a2a[(j * S + d) * A + i]) * D,
                        sizeof(REAL) * (size_t)D);
 
         if (c->scoring_bf16) {
@@ -761,7 +807,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
         }
         for (int64_t j = 0; j < S; ++j)
             for (int64_t i = 0; i < A; ++i) {
-                REAL* gh = ghid + (j * NR + a2a[(j * S + d) * A + i]) * D;
+                REAL* gh = ghid_t + (j * NR + a2a[(j * S + d) * A + i]) * D;
                 for (int64_t k = 0; k < D; ++k) gh[k] += dtl[(j * A + i) * D + k];
             }
     }
@@ -796,6 +842,13 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                 const REAL* gh = ghid + (s * NR + j) * D;
                 const REAL* gr = greg_fh ? greg_fh + (s * NR + j) * D : NULL;
                 for (int64_t k = 0; k < D; ++k) gfh[k] = gh[k] + (gr ? gr[k] : 0);
+                if (drop) { /* grad * (output != 0) / (1 - p) per use (pag.cpp:606-614) */
+                    const REAL* gt = ghid_t + (s * NR + j) * D;
+                    const uint8_t* lh = live_h + (s * NR + j) * D;
+                    const uint8_t* lt = live_t + (s * NR + j) * D;
+                    for (int64_t k = 0; k < D; ++k)
+                        gfh[k] = keep_scale * ((lh[k] ? gh[k] : 0) + (lt[k] ? gt[k] : 0));
+                }
                 if (M) {
                     /* matMul, max(., 0) (its gradient passes where input == output, i.e. also at
                      * exactly 0: pag.cpp:650-658), matMul, concat backward in turn */
@@ -849,7 +902,9 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                 const REAL* gh = ghid + (int64_t)(ks[j] & 0xffffff) * D;
                 const REAL* gr = greg_val ? greg_val + (int64_t)(ks[j] & 0xffffff) * D : NULL;
                 const REAL* gm = gmlp_val ? gmlp_val + (int64_t)(ks[j] & 0xffffff) * D : NULL;
-                for (int64_t k = 0; k < D; ++k) g[k] += gh[k] + (gr ? gr[k] : 0) + (gm ? gm[k] : 0);
+                const REAL* gt = drop ? ghid_t + (int64_t)(ks[j] & 0xffffff) * D : NULL;
+                for (int64_t k = 0; k < D; ++k)
+                    g[k] += gh[k] + (gt ? gt[k] : 0) + (gr ? gr[k] : 0) + (gm ? gm[k] : 0);
             }
             for (int64_t k = 0; k < D; ++k) gf[k] = (float)g[k];
             float* row = table + key * ROW;
@@ -907,6 +962,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
     free(hidden); free(ghid); free(grel); free(p); free(tl); free(score); free(dist);
     free(dscore); free(dp); free(dtl); free(alpha); free(gproj);
     free(nv); free(dnv); free(nrm); free(fproj); free(pre); free(gmlp_val);
+    if (drop) { free(hidden_t); free(ghid_t); free(live_h); free(live_t); }
     return 0;
 }
 

@@ -27,7 +27,7 @@ class Cfg(C.Structure):
             "gamma", "beta_m", "beta_v", "epsilon", "weight_decay", "loss_scale",
             "softmax_correction_weight", "negative_adversarial_scale", "lr_mod_entity",
             "lr_mod_relation", "lr_mod_projection", "reg_emb_power", "reg_emb_weight", "reg_feat_power",
-            "reg_feat_weight", "reg_hid_power", "reg_hid_weight")]
+            "reg_feat_weight", "reg_hid_power", "reg_hid_weight", "dropout")] + [("dropout_seed", C.c_uint32)]
 
 
 def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score_fn="TransE",
@@ -36,7 +36,7 @@ def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score
              loss_scale=None, softmax_correction_weight=0.0, negative_adversarial_scale=0.0,
              lr_mod_entity=1.0, lr_mod_relation=1.0, lr_mod_projection=1.0,
              embedding_regularisation=(3.0, 0.0), feature_regularisation=(3.0, 0.0),
-             hidden_regularisation=(3.0, 0.0), feature_mlp_size=0):
+             hidden_regularisation=(3.0, 0.0), feature_mlp_size=0, feature_dropout=0.0, dropout_seed=0):
     """The three regularisers are (power, weight) pairs (src/python/poplar_kge.py:104-108)."""
     if loss_scale is None:  # src/python/poplar_kge.py:259-262
         loss_scale = float(batch * n_shard * a2a)
@@ -46,7 +46,8 @@ def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score
                gamma, beta_m,
                beta_v, epsilon, weight_decay, loss_scale, softmax_correction_weight,
                negative_adversarial_scale, lr_mod_entity, lr_mod_relation, lr_mod_projection,
-               *embedding_regularisation, *feature_regularisation, *hidden_regularisation)
+               *embedding_regularisation, *feature_regularisation, *hidden_regularisation,
+               float(feature_dropout), int(dropout_seed))
 
 
 def build(force=False):
@@ -331,3 +332,16 @@ def predict_reference(cfg, state, queries, shard_to_count, n_best):
     order = np.argsort(-score, axis=1, kind="stable")[:, :n_best]
     best = np.take_along_axis(score, order, axis=1)
     return np.stack(np.divmod(order, NE), axis=-1), best
+
+
+def dropout_keep(seed, step, role, key, k, p):
+    """The oracle's dropout mask (kge_dropout_keep in kge_oracle.c) on NumPy arrays: True = keep."""
+    u = lambda v: np.asarray(v, np.uint64)
+    x = (u(key) * 0x9E3779B1 + u(k) * 0x85EBCA77 + u(role) * 0xC2B2AE3D + u(step) * 0x27D4EB2F
+         + u(seed) * 0x165667B1) & 0xFFFFFFFF
+    x ^= x >> 16
+    x = (x * 0x7FEB352D) & 0xFFFFFFFF
+    x ^= x >> 15
+    x = (x * 0x846CA68B) & 0xFFFFFFFF
+    x ^= x >> 16
+    return x >= np.uint64(int(np.float64(np.float32(p)) * 4294967296.0))

@@ -9,7 +9,8 @@ def cfg_dict(**kw):
              storage="float32", scoring_bf16=False, gamma=2.0, beta_m=0.9, beta_v=0.999, epsilon=1e-8,
              weight_decay=0.0, loss_scale=None, softmax_correction_weight=0.0,
              negative_adversarial_scale=0.0, embedding_regularisation=(3.0, 0.0),
-             feature_regularisation=(3.0, 0.0), hidden_regularisation=(3.0, 0.0), feature_mlp_size=0)
+             feature_regularisation=(3.0, 0.0), hidden_regularisation=(3.0, 0.0), feature_mlp_size=0,
+             feature_dropout=0.0, dropout_seed=0)
     d.update(kw)
     if d["loss_scale"] is None:
         d["loss_scale"] = float(d["batch"] * d["n_shard"] * d["a2a"])

@@ -317,6 +317,13 @@ STEP_CASES = {
                                        hidden_regularisation=(2.0, 1e-2)),
     "feature_mlp_shared_distmult": dict(feature_mlp_size=8, score_fn="DistMult", distance_fn="MatMul",
                                         shared_table=True, n_shard=4, batch=8, a2a=4, feature=4, n_entity=60),
+    # feature dropout (src/poplar_kge.cpp:459-461): separate masks for the head and the tail use
+    "feature_dropout": dict(feature_dropout=0.3, dropout_seed=7),
+    "feature_dropout_mlp_l2": dict(feature_dropout=0.5, dropout_seed=3, feature_mlp_size=6, distance_fn="L2",
+                                   loss_fn="softmax", softmax_correction_weight=1.0),
+    "feature_dropout_shared_distmult": dict(feature_dropout=0.2, dropout_seed=11, score_fn="DistMult",
+                                            distance_fn="MatMul", shared_table=True, n_shard=4, batch=8, a2a=4,
+                                            feature=4, n_entity=60),
     # norm regularisers (src/poplar_kge.cpp:430-437, 463-465), the WikiKG preset's among them
     "feature_regularisation_p3": dict(feature_regularisation=(3.0, 1e-2), loss_fn="softmax",
                                       softmax_correction_weight=1.0),
@@ -535,3 +542,22 @@ def test_predict_reference_transh_by_hand_and_invariances():
     st2["entity_data"][1:, :D] += rng.normal(size=(NE - 1, 1)).astype(np.float32) * st["relation_normal"][2]
     idx1, score1 = predict_reference(cfg, st2, q, [NE - 1], NE - 1)
     np.testing.assert_allclose(score1, score0, rtol=0, atol=2e-5)
+
+
+def test_dropout_mask_is_the_same_in_c_and_numpy_and_keeps_the_right_share(orc):
+    import ctypes as C
+    from oracle.kge_oracle import dropout_keep
+
+    orc.lib.kge_dropout_keep.restype = C.c_int
+    orc.lib.kge_dropout_keep.argtypes = [C.c_uint32] * 5 + [C.c_float]
+    rng = np.random.default_rng(0)
+    keys = rng.integers(0, 2**32, 200, dtype=np.uint64)
+    for p in (0.1, 0.5, 0.9):
+        want = [orc.lib.kge_dropout_keep(9, 12345, 1, int(k), 17, p) for k in keys]
+        np.testing.assert_array_equal(dropout_keep(9, 12345, 1, keys, 17, p), np.array(want, bool))
+        share = dropout_keep(9, 3, 0, np.arange(1, 4001)[:, None], np.arange(64)[None, :], p).mean()
+        assert abs(share - (1 - p)) < 0.01, (p, share)
+    # heads' and tails' masks, and successive steps', are different draws
+    a = dropout_keep(9, 3, 0, np.arange(4000), 5, 0.5)
+    assert 0.4 < (a != dropout_keep(9, 3, 1, np.arange(4000), 5, 0.5)).mean() < 0.6
+    assert 0.4 < (a != dropout_keep(9, 4, 0, np.arange(4000), 5, 0.5)).mean() < 0.6

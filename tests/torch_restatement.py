@@ -110,7 +110,26 @@ def step(cfg, state, lr, batch_step):
             hidden_u = emb + feat @ proj
     else:
         hidden_u = emb
+    hidden_tail_u = hidden_u
+    drop = cfg.get("feature_dropout", 0.0)
+    if F and drop > 0:
+        # src/poplar_kge.cpp:459-461, src/pag/pag.cpp:596-617: keep mask / (1 - p) on the feature part,
+        # drawn once for the rows' use as heads and once for their use as tails (the oracle's hash
+        # stands in for the device's random stream); the backward passes where the OUTPUT is
+        # non-zero, which differs from the mask where a kept input is exactly 0
+        from oracle.kge_oracle import dropout_keep
+        fh = hidden_u - emb
+        cols = np.arange(D)[None, :]
+
+        def dropped(role):
+            keep = dropout_keep(cfg.get("dropout_seed", 0), int(state["step"]), role, uniq.numpy()[:, None], cols,
+                                drop)
+            live = T.tensor(keep) & (fh.detach() != 0)
+            return emb + fh * live.to(T.float64) / (1 - float(np.float32(drop)))
+
+        hidden_u, hidden_tail_u = dropped(0), dropped(1)
     hidden = hidden_u[inverse].reshape(S, -1, D)  # [S, NR, D]
+    hidden_tail = hidden_tail_u[inverse].reshape(S, -1, D)
     # norm regularisers over every gathered slot, once for the heads' and once for the tails'
     # entityHidden call (src/poplar_kge.cpp:463-465, 676-678)
     reg = T.zeros(S, dtype=T.float64)
@@ -122,7 +141,7 @@ def step(cfg, state, lr, batch_step):
             reg = reg + 2 * weight * lpnorm(tensor, float(power)).sum(-1)
 
     heads = hidden[shards[:, None], head]  # [S, B, D]
-    tails = hidden[shards[:, None, None], a2a]  # [S(src), S(dst), A, D]
+    tails = hidden_tail[shards[:, None, None], a2a]  # [S(src), S(dst), A, D]
     tails = tails.transpose(0, 1).reshape(S, Tn, D)  # all-to-all
     r = rel[relation]
     if cfg["score_fn"] == "TransH":
