@@ -188,6 +188,10 @@ struct kge_engine {
     // TransH keeps a second row per relation, the hyperplane normal (relation_normal), as rows
     // [n_rel, 2 n_rel) of the relation table: rel_copies = 2, n_rel_rows = 2 n_rel
     int rel_copies = 1, n_rel_rows = 0;
+    float dropout = 0.f;  // model.feature_dropout (training only): two hidden rows per distinct row
+    DevBuf<float> fh;          // the feature part of hidden, before dropout
+    DevBuf<uint32_t> role_idx;  // the hidden row of every contribution
+    int step_of_first = 0;     // optimiser step of the first step of the running call
     int mlp = 0;  // model.feature_mlp_size: hidden = value + relu([value | feature . W] . Up) . Down
     int score_fn, dist_fn, loss_fn;
     bool shared_table;
@@ -402,7 +406,14 @@ void parse_settings(kge_engine& E, const Items& s) {
         throw std::invalid_argument("'model.feature_mlp_size' > 0 is not implemented together with "
                                     "'execution.scoring_dtype' = 'bfloat16'");
     E.mlp = (int)mlp;
-    if (dropout > 0) throw std::invalid_argument("'model.feature_dropout' > 0 is not implemented on the HIP device");
+    if (!(dropout >= 0.f && dropout < 1.f)) throw std::invalid_argument("'model.feature_dropout' must be in [0, 1)");
+    E.dropout = E.F > 0 ? dropout : 0.f;  // without features the dropped tensor is all zeros
+    if (E.dropout > 0 && E.score_bf16)
+        throw std::invalid_argument("'model.feature_dropout' > 0 is not implemented together with "
+                                    "'execution.scoring_dtype' = 'bfloat16'");
+    if (E.dropout > 0 && E.reg_on)
+        throw std::invalid_argument("'model.feature_dropout' > 0 is not implemented together with the norm "
+                                    "regularisers (weight > 0)");
     if (!share && E.F > 0)
         throw std::invalid_argument("'model.share_feature_networks' = false is not implemented on the HIP device");
     for (int i = 0; i < 3; ++i)
@@ -558,7 +569,11 @@ void allocate(kge_engine& E) {
         E.relgrad.alloc(2 * SB * E.Dp);
     }
     if (E.F) {
-        E.hidden.alloc(R * E.Dp);
+        E.hidden.alloc((E.dropout > 0 ? 2 : 1) * R * E.Dp);
+        if (E.dropout > 0) {
+            E.fh.alloc(R * E.Dp);
+            E.role_idx.alloc(R);
+        }
         E.gsum.alloc(R * E.Dp);
         E.gsum.zero(E.stream);  // rows past a step's distinct count are read (times zero): keep them finite
         E.featd.alloc(R * E.Fp);
@@ -886,6 +901,7 @@ void run_step(kge_engine& E, int i) {
 
     FeatureArgs fa = {};
     MlpArgs ma = {};
+    DropoutArgs da = {};
     if (E.F) {
         fa.uniq_key = e_uniq; fa.counts = e_counts; fa.max_rows = (int)R;
         fa.emb_base = E.table.p; fa.feat_base = E.table.p + E.L.off_f; fa.pitch = E.L.pitch;
@@ -894,6 +910,7 @@ void run_step(kge_engine& E, int i) {
         fa.featd = E.featd.p; fa.gproj_part = E.gproj_part.p; fa.use_mfma = E.use_mfma;
         fa.round_bf16 = E.score_bf16 ? 1 : 0; fa.projR = E.projR.p;
         fa.feat16 = E.feat16.p; fa.featT16 = E.featT16.p; fa.projT16 = E.projT16.p; fa.gT16 = E.gT16.p;
+        const bool drop = E.dropout > 0;
         if (E.mlp) {  // feature . W alone, then the MLP on [embedding | feature . W]
             KernelTimer t(E, K_HIDDEN);
             FeatureArgs fp = fa;
@@ -903,11 +920,30 @@ void run_step(kge_engine& E, int i) {
             ma.emb_base = E.table.p; ma.pitch = E.L.pitch; ma.emb_etype = E.L.emb_etype;
             ma.Dp = E.Dp; ma.M = E.mlp; ma.up = E.up.p; ma.down = E.down.p;
             ma.concat = E.mlp_concat.p; ma.pre = E.mlp_pre.p;
-            launch_mlp_fwd(ma, E.mlp_fproj.p, E.hidden.p, st);
+            ma.add_value = drop ? 0 : 1;
+            launch_mlp_fwd(ma, E.mlp_fproj.p, drop ? E.fh.p : E.hidden.p, st);
+        } else if (drop) {
+            KernelTimer t(E, K_HIDDEN);
+            FeatureArgs fp = fa;
+            fp.emb_base = nullptr;
+            launch_hidden_fwd(fp, E.fh.p, st);
         } else
         { KernelTimer t(E, K_HIDDEN); launch_hidden_fwd(fa, E.hidden.p, st); }
         ent.base = (const char*)E.hidden.p; ent.pitch = (int64_t)E.Dp * 4; ent.etype = ET_F32;
         ent.index = E.e_item_row.p + i * R;
+        if (drop) {
+            // a head row and a tail row per distinct row (src/poplar_kge.cpp:459-461, once per
+            // entityHidden call); every contribution reads the one of its role
+            KernelTimer t(E, K_HIDDEN);
+            da.uniq_key = e_uniq; da.counts = e_counts; da.max_rows = (int)R;
+            da.emb_base = E.table.p; da.pitch = E.L.pitch; da.emb_etype = E.L.emb_etype; da.Dp = E.Dp;
+            da.seed = E.seed; da.step = (uint32_t)(E.step_of_first + i);
+            da.threshold = (uint32_t)((double)E.dropout * 4294967296.0);
+            da.scale = 1.f / (1.f - E.dropout);
+            launch_dropout_hidden(da, E.fh.p, E.hidden.p, st);
+            launch_role_index(E.e_item_row.p + i * R, (int)SB, (int)R, E.role_idx.p, st);
+            ent.index = E.role_idx.p;
+        }
     }
 
     // dense operands: every contribution's row, float32, relation applied to the heads
@@ -1071,7 +1107,8 @@ void run_step(kge_engine& E, int i) {
     ae.chunk_off = E.e_coff.p + (size_t)i * (E.e_ustride + 1);
     ae.counts = e_counts; ae.max_rows = (int)R;
     ae.partial = E.partial.p;
-    ae.grad_out = E.F ? E.gsum.p : nullptr;
+    // (with dropout the feature part's gradient is formed per role by launch_role_sums)
+    ae.grad_out = (E.F && !(E.dropout > 0)) ? E.gsum.p : nullptr;
     if (E.reg_on) { ae.grad_add = E.reg_val.p; ae.grad_out_add = E.reg_fh.p; }
     ae.p_base = E.table.p; ae.m_base = E.table.p + E.L.off_m; ae.v_base = E.table.p + E.L.off_s;
     ae.pitch = E.L.pitch; ae.p_etype = E.L.emb_etype; ae.m_etype = E.L.mom_etype; ae.v_is_sqrt = 1;
@@ -1083,10 +1120,14 @@ void run_step(kge_engine& E, int i) {
     // backward per row, then the update with what that adds.
     auto entity_update = [&]() {
         KernelTimer t(E, K_ADAM_ENT);
+        if (E.dropout > 0)
+            launch_role_sums(da, esrc, ae.seg_start, ae.seg_real, E.fh.p, E.gsum.p, st);
         if (!E.mlp) { launch_adam_rows(ae, st); return; }
-        AdamArgs sum = ae;
-        sum.no_update = 1;
-        launch_adam_rows(sum, st);
+        if (!(E.dropout > 0)) {
+            AdamArgs sum = ae;
+            sum.no_update = 1;
+            launch_adam_rows(sum, st);
+        }
         launch_mlp_bwd_rows(ma, E.gsum.p, E.reg_on ? E.reg_val.p : nullptr, E.mlp_gpre.p, E.mlp_gval.p,
                             E.mlp_gfp.p, st);
         AdamArgs upd = ae;
@@ -1104,7 +1145,7 @@ void run_step(kge_engine& E, int i) {
         ar.grad_out = nullptr; ar.no_update = 0;
         ar.grad_direct = E.rel_gsum.p;
         { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
-    } else if (E.mlp) {
+    } else if (E.mlp || E.dropout > 0) {
         entity_update();
         KernelTimer t(E, K_ADAM_REL);
         launch_adam_rows(ar, st);
@@ -1222,6 +1263,7 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     HIP_CHECK(hipMemcpyAsync(E.d_alpha.p, E.h_alpha.data(), E.h_alpha.size() * 4, hipMemcpyHostToDevice, st));
     HIP_CHECK(hipEventRecord(E.ev[1], st));
     run_plan(E, s0, sn);
+    E.step_of_first = (int)E.step - s0;  // step i of the batch is optimiser step E.step + (i - s0)
     HIP_CHECK(hipEventRecord(E.ev[2], st));
     for (int i = s0; i < s0 + sn; ++i) run_step(E, i);
     launch_loss_finalize(E.loss_part.p + (size_t)s0 * E.S * E.n_part, sn, E.S, E.n_part, 1.f / (float)sn,
@@ -1357,7 +1399,7 @@ void run_predict(kge_engine& E, const Items& in) {
                 ma.uniq_key = idx; ma.counts = E.p_count.p; ma.max_rows = n;
                 ma.emb_base = E.table.p; ma.pitch = E.L.pitch; ma.emb_etype = E.L.emb_etype;
                 ma.Dp = Dp; ma.M = E.mlp; ma.up = E.up.p; ma.down = E.down.p;
-                ma.concat = E.p_concat.p; ma.pre = E.p_pre.p;
+                ma.concat = E.p_concat.p; ma.pre = E.p_pre.p; ma.add_value = 1;
                 launch_mlp_fwd(ma, E.p_fproj.p, E.p_hidden.p, st);
             } else
             launch_hidden_fwd(fa, E.p_hidden.p, st);

@@ -358,6 +358,7 @@ struct MlpArgs {
     const float* down;  // [M, Dp]
     float* concat;      // [max_rows, 2 Dp] the MLP's input (written by the forward)
     float* pre;         // [max_rows, M] pre-activations (written by the forward)
+    int add_value;      // the forward's output: 1 value + MLP output (hidden), 0 the MLP output alone
 };
 // fproj [max_rows, Dp] = feature . W (launch_hidden_fwd with a null emb_base)
 void launch_mlp_fwd(const MlpArgs& a, const float* fproj, float* hidden, hipStream_t stream);
@@ -366,5 +367,23 @@ void launch_mlp_bwd_rows(const MlpArgs& a, const float* g, const float* val_add,
 // C [Ka, N] = f(A [rows, Ka])^T . B [rows, N] over the first *count rows, summed in row order
 void launch_rows_atb(const float* A, int lda, int Ka, bool relu, const float* B, int ldb, int N,
                      const uint32_t* count, float* C, hipStream_t stream);
+
+// ---- feature dropout (src/poplar_kge.cpp:459-461; src/pag/pag.cpp:596-617) ----
+struct DropoutArgs {
+    const uint32_t* uniq_key; const uint32_t* counts; int max_rows;
+    const char* emb_base; int64_t pitch; int emb_etype;
+    int Dp;
+    uint32_t seed, step;   // model.seed, the optimiser step the mask belongs to
+    uint32_t threshold;    // p * 2^32: an element is kept where its hash is at least this
+    float scale;           // 1 / (1 - p)
+};
+// hidden [2 max_rows, Dp]: row u = value + dropped feature part for the head use, row
+// max_rows + u for the tail use; fh [max_rows, Dp] = the feature part
+void launch_dropout_hidden(const DropoutArgs& a, const float* fh, float* hidden, hipStream_t stream);
+// out[c] = item_row[c] (+ n for c >= n_head): the hidden row contribution c reads
+void launch_role_index(const uint32_t* item_row, int n_head, int n, uint32_t* out, hipStream_t stream);
+// out [max_rows, Dp]: the feature part's gradient of every distinct row from its contributions
+void launch_role_sums(const DropoutArgs& a, const ContribSrc& cs, const uint32_t* seg_start, const uint32_t* seg_real,
+                      const float* fh, float* out, hipStream_t stream);
 
 }  // namespace kge

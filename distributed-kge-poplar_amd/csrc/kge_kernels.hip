@@ -3549,7 +3549,7 @@ __global__ __launch_bounds__(256) void k_mlp_fwd(MlpArgs a, const float* __restr
     for (int k = tid; k < Dp; k += 256) {
         float acc = 0.f;
         for (int m = 0; m < M; ++m) acc = fmaf(boom[m], a.down[(size_t)m * Dp + k], acc);
-        hidden[(size_t)u * Dp + k] = cc[k] + acc;
+        hidden[(size_t)u * Dp + k] = a.add_value ? cc[k] + acc : acc;
     }
 }
 void launch_mlp_fwd(const MlpArgs& a, const float* fproj, float* hidden, hipStream_t stream) {
@@ -3615,6 +3615,92 @@ void launch_rows_atb(const float* A, int lda, int Ka, bool relu, const float* B,
                      const uint32_t* count, float* C, hipStream_t stream) {
     hipLaunchKernelGGL(k_rows_atb, dim3((N + 255) / 256, Ka), dim3(256), 0, stream, A, lda, relu ? 1 : 0, B, ldb,
                        N, count, C);
+}
+
+// --------------------------------------------------------------------------
+// Feature dropout (src/poplar_kge.cpp:459-461; src/pag/pag.cpp:596-617): the feature part of
+// hidden times keep / (1 - p), drawn once for a row's use as a head and once for its use as a
+// tail, so a distinct row has two hidden rows: hidden[u] (head use) and hidden[rows + u].
+// The keep mask is a hash of (seed, optimiser step, role, table row, column) compared with
+// p * 2^32; the reference's device random stream cannot be reproduced, the CPU oracle uses
+// this same hash.
+DEVINL bool dropout_keep(uint32_t seed, uint32_t step, uint32_t role, uint32_t key, uint32_t k, uint32_t threshold) {
+    uint32_t x = key * 0x9E3779B1u + k * 0x85EBCA77u + role * 0xC2B2AE3Du + step * 0x27D4EB2Fu + seed * 0x165667B1u;
+    x ^= x >> 16; x *= 0x7FEB352Du; x ^= x >> 15; x *= 0x846CA68Bu; x ^= x >> 16;
+    return x >= threshold;
+}
+
+// one wave per distinct row: fh [max_rows, Dp] = the feature part, hidden [2 max_rows, Dp]
+__global__ __launch_bounds__(256) void k_dropout_hidden(DropoutArgs a, const float* __restrict__ fh,
+                                                        float* __restrict__ hidden) {
+    const int lane = threadIdx.x & 63;
+    const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (u >= (int)a.counts[0]) return;
+    const uint32_t key = a.uniq_key[u];
+    const char* erow = a.emb_base + (int64_t)key * a.pitch;
+    for (int k = lane * 4; k < a.Dp; k += 256) {
+        const float4 v4 = load4(erow, k, a.emb_etype);
+        const float4 f4 = *reinterpret_cast<const float4*>(fh + (size_t)u * a.Dp + k);
+        const float v[4] = {v4.x, v4.y, v4.z, v4.w}, f[4] = {f4.x, f4.y, f4.z, f4.w};
+        float oh[4], ot[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            oh[x] = v[x] + (dropout_keep(a.seed, a.step, 0u, key, (uint32_t)(k + x), a.threshold) ? f[x] * a.scale : 0.f);
+            ot[x] = v[x] + (dropout_keep(a.seed, a.step, 1u, key, (uint32_t)(k + x), a.threshold) ? f[x] * a.scale : 0.f);
+        }
+        *reinterpret_cast<float4*>(hidden + (size_t)u * a.Dp + k) = make_float4(oh[0], oh[1], oh[2], oh[3]);
+        *reinterpret_cast<float4*>(hidden + (size_t)(a.max_rows + u) * a.Dp + k) = make_float4(ot[0], ot[1], ot[2], ot[3]);
+    }
+}
+void launch_dropout_hidden(const DropoutArgs& a, const float* fh, float* hidden, hipStream_t stream) {
+    hipLaunchKernelGGL(k_dropout_hidden, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, fh, hidden);
+}
+
+// which hidden row contribution c reads: its distinct row, in the tail half for a tail
+__global__ __launch_bounds__(256) void k_role_index(const uint32_t* __restrict__ item_row, int n_head, int n,
+                                                    uint32_t* __restrict__ out) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c < n) out[c] = item_row[c] + (c >= n_head ? (uint32_t)n : 0u);
+}
+void launch_role_index(const uint32_t* item_row, int n_head, int n, uint32_t* out, hipStream_t stream) {
+    hipLaunchKernelGGL(k_role_index, dim3((n + 255) / 256), dim3(256), 0, stream, item_row, n_head, n, out);
+}
+
+// The feature part's gradient per distinct row, one wave per row: its head contributions and its
+// tail contributions summed apart (in sorted order), each passed where that use's dropout output
+// is non-zero (the reference's backward tests the output, pag.cpp:610), times 1 / (1 - p).
+__global__ __launch_bounds__(256) void k_role_sums(DropoutArgs a, ContribSrc cs, const uint32_t* __restrict__ seg_start,
+                                                   const uint32_t* __restrict__ seg_real,
+                                                   const float* __restrict__ fh, float* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (u >= (int)a.counts[0]) return;
+    const uint32_t key = a.uniq_key[u], pos = seg_start[u], n = seg_real[u];
+    for (int k0 = 0; k0 < a.Dp; k0 += 256) {
+        const int k = k0 + lane * 4;
+        if (k >= a.Dp) continue;
+        float4 gh = make_float4(0, 0, 0, 0), gt = gh;
+        for (uint32_t j = 0; j < n; ++j) {
+            const uint32_t c = cs.sorted_item[pos + j];
+            const float4 v = load_contrib<true>(cs, c, k, a.Dp);
+            if (c < (uint32_t)cs.n_head) gh = f4add(gh, v); else gt = f4add(gt, v);
+        }
+        const float4 f4 = *reinterpret_cast<const float4*>(fh + (size_t)u * a.Dp + k);
+        const float f[4] = {f4.x, f4.y, f4.z, f4.w}, h[4] = {gh.x, gh.y, gh.z, gh.w}, t[4] = {gt.x, gt.y, gt.z, gt.w};
+        float o[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const bool live = f[x] * a.scale != 0.f;
+            const bool kh = live && dropout_keep(a.seed, a.step, 0u, key, (uint32_t)(k + x), a.threshold);
+            const bool kt = live && dropout_keep(a.seed, a.step, 1u, key, (uint32_t)(k + x), a.threshold);
+            o[x] = a.scale * ((kh ? h[x] : 0.f) + (kt ? t[x] : 0.f));
+        }
+        *reinterpret_cast<float4*>(out + (size_t)u * a.Dp + k) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+}
+void launch_role_sums(const DropoutArgs& a, const ContribSrc& cs, const uint32_t* seg_start, const uint32_t* seg_real,
+                      const float* fh, float* out, hipStream_t stream) {
+    hipLaunchKernelGGL(k_role_sums, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, cs, seg_start, seg_real, fh, out);
 }
 
 }  // namespace kge

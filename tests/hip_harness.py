@@ -36,12 +36,12 @@ def engine_settings(c, n_step, rw_batch=64, **extra):
     if c["loss_fn"] == "softmax":
         loss["training.loss.correction_weight"] = float(c["softmax_correction_weight"])
     s = {
-        "seed": 1, "model.seed": 1234,
+        "seed": 1, "model.seed": int(c.get("dropout_seed") or 1234),
         "model.score_fn": c["score_fn"], "model.distance_fn": c["distance_fn"],
         "model.n_shard": c["n_shard"], "model.n_entity": c["n_entity"],
         "model.n_relation_type": c["n_relation"], "model.embedding_size": c["dim"],
         "model.entity_feature_size": c["feature"], "model.feature_mlp_size": int(c.get("feature_mlp_size", 0)),
-        "model.feature_dropout": 0.0,
+        "model.feature_dropout": float(c.get("feature_dropout", 0.0)),
         "model.negative_adversarial_scale": float(c["negative_adversarial_scale"]),
         "model.share_feature_networks": True, "model.gamma": float(c["gamma"]),
         "model.init_scale": 1.0,

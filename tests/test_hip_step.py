@@ -109,6 +109,16 @@ CASES = {
                                 distance_fn="L2", n_shard=1),
     "feature_mlp_aligned_transh": dict(feature_mlp_size=96, score_fn="TransH", n_shard=2, batch=128, a2a=64,
                                        dim=64, feature=32, n_entity=3000, n_relation=8, gamma=6.0),
+    # feature dropout (src/poplar_kge.cpp:459-461): a row's head use and tail use are dropped apart
+    "feature_dropout": dict(feature_dropout=0.3, dropout_seed=7),
+    "feature_dropout_mlp_l2": dict(feature_dropout=0.5, dropout_seed=3, feature_mlp_size=6, distance_fn="L2",
+                                   loss_fn="softmax", softmax_correction_weight=1.0),
+    "feature_dropout_shared_distmult": dict(feature_dropout=0.2, dropout_seed=11, score_fn="DistMult",
+                                            distance_fn="MatMul", shared_table=True, n_shard=4, batch=8, a2a=4,
+                                            feature=4, n_entity=60),
+    "feature_dropout_aligned_l2": dict(feature_dropout=0.4, dropout_seed=5, distance_fn="L2", n_shard=2,
+                                       batch=128, a2a=64, dim=64, feature=32, n_entity=3000, n_relation=8,
+                                       gamma=6.0),
     "aligned_complex_l2_shared": dict(score_fn="ComplEx", distance_fn="L2", n_shard=4, batch=128, a2a=32,
                                       dim=128, feature=0, n_entity=2000, n_relation=8, shared_table=True),
 }
@@ -526,3 +536,27 @@ def test_transh_zipf_duplicates(oracle64):
     kw = dict(score_fn="TransH", n_shard=4, batch=64, a2a=16, dim=32, feature=0, n_entity=500, n_relation=4,
               shared_table=True, gamma=4.0)
     run_case(oracle64, kw, n_step=2, batch_fn=K.raw_batch)
+
+
+def test_dropout_masks_follow_the_optimiser_step(oracle64):
+    # two calls of two steps each: the masks of the second call are those of steps 2 and 3 after
+    # the state's own step count, on the device as in the oracle; and dropout really acts (the
+    # same run without it ends elsewhere)
+    kw = dict(feature_dropout=0.5, dropout_seed=21)
+    c, st0, st_h, _ = run_case(oracle64, kw, n_step=2, n_loop=2)
+    st_plain = K.copy_state(st0)
+    rng = np.random.default_rng(11)
+    K.make_state(c, rng)  # advance the generator as run_case did
+    plain = dict(c, feature_dropout=0.0)
+    for _ in range(2):
+        oracle64.train_step_loop(make_cfg(**plain), st_plain, np.array([0.1, 0.07], np.float32), K.random_batch(c, 2, rng))
+    k = "feature_projection"
+    assert K.rel_l2(st_h[k] - st0[k], st_plain[k] - st0[k]) > 0.05
+
+
+def test_dropout_rejected_with_regularisers():
+    import libpoplar_kge
+
+    c = K.cfg_dict(feature_dropout=0.1, feature_regularisation=(3.0, 1e-3))
+    with pytest.raises(ValueError, match="feature_dropout"):
+        libpoplar_kge.Engine(H.engine_settings(c, 1), "")

@@ -165,7 +165,7 @@ def _random_queries(engine, n):
 
 
 @pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "complex", "rotate", "transh", "transh_big",
-                                     "feature_mlp", "no_features_big"])
+                                     "feature_mlp", "feature_dropout", "no_features_big"])
 def test_predict_vs_brute_force(variant):
     """Engine.predict against a float64 brute force over every row of every shard
     (the reference checks shapes, ranges and ordering, tests/python/test_poplar_kge.py:155-175,
@@ -188,6 +188,8 @@ def test_predict_vs_brute_force(variant):
         m.score_fn = "TransH"
     elif variant == "feature_mlp":
         m.feature_mlp_size = 24
+    elif variant == "feature_dropout":
+        m.feature_dropout = 0.4   # training only (entityHidden(..., training=false), src/poplar_kge.cpp:419-422)
     elif variant in ("no_features_big", "transh_big"):
         # several chunks of tails per shard, several query chunks, ragged counts
         m.n_entity, m.entity_feature_size, m.embedding_size, m.n_shard = 20000, 0, 32, 3
