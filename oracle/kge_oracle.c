@@ -82,6 +82,10 @@ typedef struct {
      * hash of (seed, step, role, table row, column) that the HIP kernels evaluate identically. */
     float dropout;
     uint32_t dropout_seed;
+    /* 1: separate feature networks for a row's use as a head and as a tail
+     * (share_feature_networks = false, poplar_kge.cpp:268-273): `proj` and its moments hold the
+     * head network's parameters, then the tail network's                                      */
+    int32_t separate_networks;
 } kge_oracle_cfg;
 
 /* keep (1) or drop (0) element k of table row `key` in `role` (0 head, 1 tail) at optimiser step
@@ -476,68 +480,77 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
      * relation embeddings followed by the hyperplane normals (relation_normal)       */
     const int transh = c->score_fn == SCORE_TRANSH;
     const int64_t M = F > 0 ? c->mlp_size : 0;
-    const float* up = proj + F * D;           /* [2D, M] */
-    const float* down = up + 2 * D * M;       /* [M, D]  */
+    /* one feature network = W [F, D], Up [2D, M], Down [M, D] back to back */
+    const int64_t NETSIZE = F * D + 3 * D * M;
+    const int nets = (F > 0 && c->separate_networks) ? 2 : 1;
     const int64_t NRELT = transh ? 2 * NREL : NREL;
 #define KEY(s, slot) ((c->shared_table ? 0 : (int64_t)(s) * NE) + (int64_t)remote[(s) * NR + (slot)])
 
-    /* 1. gather + hidden = emb + feature * W  (:405-410, :439-467) */
+    /* 1. gather + hidden = emb + feature part (:405-410, :439-467).  entityHidden runs once for
+     * the rows' use as heads and once for their use as tails (:676-678).  The two differ when
+     * the feature networks are separate or with dropout (masks drawn per call): then a slot has
+     * two hidden rows (`hidden`, `hidden_t`) and two gradients (`ghid`, `ghid_t`); otherwise
+     * these are the same arrays.                                                              */
+    const int drop = F > 0 && c->dropout > 0;
+    const int n_role = (drop || nets == 2) ? 2 : 1;
+    const REAL keep_scale = drop ? 1 / (1 - (REAL)c->dropout) : 1;
     REAL* hidden = (REAL*)malloc(sizeof(REAL) * (size_t)(S * NR * D));
     REAL* ghid = (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL));
-    /* feature MLP: per slot, the projected features (the second half of the MLP's input) and
-     * the pre-activations, kept for the backward pass */
-    REAL* fproj = M ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
-    REAL* pre = M ? (REAL*)calloc((size_t)(S * NR * M), sizeof(REAL)) : NULL;
-    /* feature dropout: a slot's hidden row differs between its use as a head (`hidden`) and as
-     * a tail (`hidden_t`), and so do the gradients that come back (`ghid`, `ghid_t`); without
-     * dropout the two are the same arrays */
-    const int drop = F > 0 && c->dropout > 0;
-    const REAL keep_scale = drop ? 1 / (1 - (REAL)c->dropout) : 1;
-    REAL* hidden_t = drop ? (REAL*)malloc(sizeof(REAL) * (size_t)(S * NR * D)) : hidden;
-    REAL* ghid_t = drop ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : ghid;
-    /* whether the dropout's output is non-zero (what its backward tests), per use */
-    uint8_t* live_h = drop ? (uint8_t*)malloc((size_t)(S * NR * D)) : NULL;
-    uint8_t* live_t = drop ? (uint8_t*)malloc((size_t)(S * NR * D)) : NULL;
+    REAL* hidden_t = n_role == 2 ? (REAL*)malloc(sizeof(REAL) * (size_t)(S * NR * D)) : hidden;
+    REAL* ghid_t = n_role == 2 ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : ghid;
+    /* per role: the projected features (second half of the MLP's input) and the MLP's
+     * pre-activations, kept for the backward pass; whether the dropout's output is non-zero
+     * (what its backward tests)                                                               */
+    REAL *fproj_r[2] = {NULL, NULL}, *pre_r[2] = {NULL, NULL};
+    uint8_t* live_r[2] = {NULL, NULL};
     REAL* fhv = (REAL*)malloc(sizeof(REAL) * (size_t)D); /* one slot's feature part of hidden */
-    for (int64_t s = 0; s < S; ++s)
-        for (int64_t j = 0; j < NR; ++j) {
-            const float* row = table + KEY(s, j) * ROW;
-            REAL* h = hidden + (s * NR + j) * D;
-            REAL* fh = M ? fproj + (s * NR + j) * D : fhv; /* feature . W */
-            for (int64_t k = 0; k < D; ++k) fhv[k] = 0;
-            for (int64_t f = 0; f < F; ++f) {
-                /* bfloat16 scoring also takes the projection's operands in bfloat16 */
-                const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
-                if (x != 0)
-                    for (int64_t k = 0; k < D; ++k)
-                        fh[k] += x * (REAL)(c->scoring_bf16 ? round_bf16(proj[f * D + k]) : proj[f * D + k]);
-            }
-            if (M) { /* :453-458: boom = relu(concat(value, featureHidden) . Up); featureHidden = boom . Down */
-                REAL* a = pre + (s * NR + j) * M;
-                for (int64_t i = 0; i < 2 * D; ++i) {
-                    const REAL x = i < D ? (REAL)row[i] : fh[i - D];
-                    for (int64_t m = 0; m < M; ++m) a[m] += x * (REAL)up[i * M + m];
-                }
-                for (int64_t m = 0; m < M; ++m)
-                    if (a[m] > 0)
-                        for (int64_t k = 0; k < D; ++k) fhv[k] += a[m] * (REAL)down[m * D + k];
-            }
-            if (drop) { /* :459-461, once per entityHidden call: heads' and tails' masks differ */
-                REAL* ht = hidden_t + (s * NR + j) * D;
-                const uint32_t key = (uint32_t)KEY(s, j);
-                for (int64_t k = 0; k < D; ++k) {
-                    const int kh = kge_dropout_keep(c->dropout_seed, *step, 0, key, (uint32_t)k, c->dropout);
-                    const int kt = kge_dropout_keep(c->dropout_seed, *step, 1, key, (uint32_t)k, c->dropout);
-                    const REAL oh = kh ? fhv[k] * keep_scale : 0, ot = kt ? fhv[k] * keep_scale : 0;
-                    h[k] = (REAL)row[k] + oh;
-                    ht[k] = (REAL)row[k] + ot;
-                    live_h[(s * NR + j) * D + k] = oh != 0;
-                    live_t[(s * NR + j) * D + k] = ot != 0;
-                }
-            } else {
-                for (int64_t k = 0; k < D; ++k) h[k] = (REAL)row[k] + fhv[k]; /* :462 */
-            }
+    for (int role = 0; role < n_role; ++role) {
+        const float* W = proj + (nets == 2 ? role : 0) * NETSIZE;
+        const float* up = W + F * D;          /* [2D, M] */
+        const float* down = up + 2 * D * M;   /* [M, D]  */
+        REAL* hid = role ? hidden_t : hidden;
+        if (M) {
+            fproj_r[role] = (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL));
+            pre_r[role] = (REAL*)calloc((size_t)(S * NR * M), sizeof(REAL));
         }
+        if (drop) live_r[role] = (uint8_t*)malloc((size_t)(S * NR * D));
+        for (int64_t s = 0; s < S; ++s)
+            for (int64_t j = 0; j < NR; ++j) {
+                const float* row = table + KEY(s, j) * ROW;
+                REAL* h = hid + (s * NR + j) * D;
+                REAL* fh = M ? fproj_r[role] + (s * NR + j) * D : fhv; /* feature . W */
+                for (int64_t k = 0; k < D; ++k) fhv[k] = 0;
+                for (int64_t f = 0; f < F; ++f) {
+                    /* bfloat16 scoring also takes the projection's operands in bfloat16 */
+                    const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
+                    if (x != 0)
+                        for (int64_t k = 0; k < D; ++k)
+                            fh[k] += x * (REAL)(c->scoring_bf16 ? round_bf16(W[f * D + k]) : W[f * D + k]);
+                }
+                if (M) { /* :453-458: boom = relu(concat(value, featureHidden) . Up); featureHidden = boom . Down */
+                    REAL* a = pre_r[role] + (s * NR + j) * M;
+                    for (int64_t i = 0; i < 2 * D; ++i) {
+                        const REAL x = i < D ? (REAL)row[i] : fh[i - D];
+                        for (int64_t m = 0; m < M; ++m) a[m] += x * (REAL)up[i * M + m];
+                    }
+                    for (int64_t m = 0; m < M; ++m)
+                        if (a[m] > 0)
+                            for (int64_t k = 0; k < D; ++k) fhv[k] += a[m] * (REAL)down[m * D + k];
+                }
+                if (drop) { /* :459-461: keep mask / (1 - p), a draw of its own for every call */
+                    const uint32_t key = (uint32_t)KEY(s, j);
+                    for (int64_t k = 0; k < D; ++k) {
+                        const int keep = kge_dropout_keep(c->dropout_seed, *step, (uint32_t)role, key, (uint32_t)k,
+                                                          c->dropout);
+                        const REAL o = keep ? fhv[k] * keep_scale : 0;
+                        h[k] = (REAL)row[k] + o;
+                        live_r[role][(s * NR + j) * D + k] = o != 0;
+                    }
+                } else {
+                    for (int64_t k = 0; k < D; ++k) h[k] = (REAL)row[k] + fhv[k]; /* :462 */
+                }
+            }
+    }
     free(fhv);
 
     /* 1b. norm regularisers over every gathered slot (:463-465).  entityHidden runs once for
@@ -545,9 +558,9 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
      * same projection, so every term counts twice (:676-678).  The embedding's gradient and
      * the feature product's gradient differ from here on: greg_val / greg_fh.              */
     const int reg_on = c->reg_emb_weight > 0 || c->reg_feat_weight > 0 || c->reg_hid_weight > 0;
-    if (reg_on && drop) { /* the regularised tensors would differ per use: not restated */
-        free(hidden); free(ghid); free(fproj); free(pre);
-        free(hidden_t); free(ghid_t); free(live_h); free(live_t);
+    if (reg_on && n_role == 2) { /* the regularised tensors would differ per use: not restated */
+        free(hidden); free(ghid); free(hidden_t); free(ghid_t);
+        for (int role = 0; role < 2; ++role) { free(fproj_r[role]); free(pre_r[role]); free(live_r[role]); }
         return 2;
     }
     REAL* greg_val = reg_on ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
@@ -830,56 +843,61 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
     REAL* gproj = NULL;
     REAL* gmlp_val = NULL; /* feature MLP: what reaches the embedding through the MLP's input */
     if (F > 0) {
-        gproj = (REAL*)calloc((size_t)(F * D + 3 * D * M), sizeof(REAL));
-        REAL* gup = gproj + F * D;
-        REAL* gdown = gup + 2 * D * M;
+        gproj = (REAL*)calloc((size_t)(nets * NETSIZE), sizeof(REAL));
         REAL* gfh = (REAL*)malloc(sizeof(REAL) * (size_t)D);
         REAL* gpre = M ? (REAL*)malloc(sizeof(REAL) * (size_t)M) : NULL;
         if (M) gmlp_val = (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL));
-        for (int64_t s = 0; s < S; ++s)
-            for (int64_t j = 0; j < NR; ++j) {
-                const float* row = table + KEY(s, j) * ROW;
-                const REAL* gh = ghid + (s * NR + j) * D;
-                const REAL* gr = greg_fh ? greg_fh + (s * NR + j) * D : NULL;
-                for (int64_t k = 0; k < D; ++k) gfh[k] = gh[k] + (gr ? gr[k] : 0);
-                if (drop) { /* grad * (output != 0) / (1 - p) per use (pag.cpp:606-614) */
-                    const REAL* gt = ghid_t + (s * NR + j) * D;
-                    const uint8_t* lh = live_h + (s * NR + j) * D;
-                    const uint8_t* lt = live_t + (s * NR + j) * D;
-                    for (int64_t k = 0; k < D; ++k)
-                        gfh[k] = keep_scale * ((lh[k] ? gh[k] : 0) + (lt[k] ? gt[k] : 0));
-                }
-                if (M) {
-                    /* matMul, max(., 0) (its gradient passes where input == output, i.e. also at
-                     * exactly 0: pag.cpp:650-658), matMul, concat backward in turn */
-                    const REAL* a = pre + (s * NR + j) * M;
-                    const REAL* fh = fproj + (s * NR + j) * D;
-                    REAL* gv = gmlp_val + (s * NR + j) * D;
-                    for (int64_t m = 0; m < M; ++m) {
-                        const REAL boom = a[m] > 0 ? a[m] : 0;
-                        REAL acc = 0;
-                        for (int64_t k = 0; k < D; ++k) {
-                            gdown[m * D + k] += boom * gfh[k];
-                            acc += gfh[k] * (REAL)down[m * D + k];
-                        }
-                        gpre[m] = a[m] >= 0 ? acc : 0;
+        for (int role = 0; role < n_role; ++role) {
+            const int net = nets == 2 ? role : 0;
+            const float* W = proj + net * NETSIZE;
+            const float* up = W + F * D;
+            const float* down = up + 2 * D * M;
+            REAL* gW = gproj + net * NETSIZE;
+            REAL* gup = gW + F * D;
+            REAL* gdown = gup + 2 * D * M;
+            const REAL* gsrc = role ? ghid_t : ghid;
+            for (int64_t s = 0; s < S; ++s)
+                for (int64_t j = 0; j < NR; ++j) {
+                    const float* row = table + KEY(s, j) * ROW;
+                    const REAL* gh = gsrc + (s * NR + j) * D;
+                    const REAL* gr = greg_fh ? greg_fh + (s * NR + j) * D : NULL;
+                    for (int64_t k = 0; k < D; ++k) gfh[k] = gh[k] + (gr ? gr[k] : 0);
+                    if (drop) { /* grad * (output != 0) / (1 - p) (pag.cpp:606-614) */
+                        const uint8_t* lv = live_r[role] + (s * NR + j) * D;
+                        for (int64_t k = 0; k < D; ++k) gfh[k] = lv[k] ? keep_scale * gh[k] : 0;
                     }
-                    for (int64_t i = 0; i < 2 * D; ++i) {
-                        const REAL x = i < D ? (REAL)row[i] : fh[i - D];
-                        REAL acc = 0;
+                    if (M) {
+                        /* matMul, max(., 0) (its gradient passes where input == output, i.e. also at
+                         * exactly 0: pag.cpp:650-658), matMul, concat backward in turn */
+                        const REAL* a = pre_r[role] + (s * NR + j) * M;
+                        const REAL* fh = fproj_r[role] + (s * NR + j) * D;
+                        REAL* gv = gmlp_val + (s * NR + j) * D;
                         for (int64_t m = 0; m < M; ++m) {
-                            gup[i * M + m] += x * gpre[m];
-                            acc += gpre[m] * (REAL)up[i * M + m];
+                            const REAL boom = a[m] > 0 ? a[m] : 0;
+                            REAL acc = 0;
+                            for (int64_t k = 0; k < D; ++k) {
+                                gdown[m * D + k] += boom * gfh[k];
+                                acc += gfh[k] * (REAL)down[m * D + k];
+                            }
+                            gpre[m] = a[m] >= 0 ? acc : 0;
                         }
-                        if (i < D) gv[i] = acc; else gfh[i - D] = acc;
+                        for (int64_t i = 0; i < 2 * D; ++i) {
+                            const REAL x = i < D ? (REAL)row[i] : fh[i - D];
+                            REAL acc = 0;
+                            for (int64_t m = 0; m < M; ++m) {
+                                gup[i * M + m] += x * gpre[m];
+                                acc += gpre[m] * (REAL)up[i * M + m];
+                            }
+                            if (i < D) gv[i] += acc; else gfh[i - D] = acc;
+                        }
+                    }
+                    for (int64_t f = 0; f < F; ++f) {
+                        const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
+                        if (x != 0)
+                            for (int64_t k = 0; k < D; ++k) gW[f * D + k] += x * gfh[k];
                     }
                 }
-                for (int64_t f = 0; f < F; ++f) {
-                    const REAL x = c->scoring_bf16 ? round_bf16(row[3 * D + f]) : row[3 * D + f];
-                    if (x != 0)
-                        for (int64_t k = 0; k < D; ++k) gproj[f * D + k] += x * gfh[k];
-                }
-            }
+        }
         free(gfh); free(gpre);
     }
 
@@ -902,7 +920,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                 const REAL* gh = ghid + (int64_t)(ks[j] & 0xffffff) * D;
                 const REAL* gr = greg_val ? greg_val + (int64_t)(ks[j] & 0xffffff) * D : NULL;
                 const REAL* gm = gmlp_val ? gmlp_val + (int64_t)(ks[j] & 0xffffff) * D : NULL;
-                const REAL* gt = drop ? ghid_t + (int64_t)(ks[j] & 0xffffff) * D : NULL;
+                const REAL* gt = n_role == 2 ? ghid_t + (int64_t)(ks[j] & 0xffffff) * D : NULL;
                 for (int64_t k = 0; k < D; ++k)
                     g[k] += gh[k] + (gt ? gt[k] : 0) + (gr ? gr[k] : 0) + (gm ? gm[k] : 0);
             }
@@ -933,25 +951,23 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                             alpha[shard] * c->lr_mod_relation, c->beta_m, c->beta_v, c->epsilon,
                             c->weight_decay, 0);
         }
-        for (int64_t f = 0; f < F; ++f) {
-            for (int64_t k = 0; k < D; ++k) gf[k] = (float)gproj[f * D + k];
-            const int64_t shard = c->shared_table ? 0 : f / (F / S);
-            kge_oracle_adam(proj + f * D, proj_m + f * D, proj_v + f * D, gf, D,
-                            alpha[shard] * c->lr_mod_projection, c->beta_m, c->beta_v, c->epsilon,
-                            c->weight_decay, 0);
-        }
         free(gf);
-        if (M) { /* the MLP's two matrices, rows split over the shards like every parameter; no
-                  * step-size modifier of their own here */
-            const int64_t off[2] = {F * D, F * D + 2 * D * M}, rows[2] = {2 * D, M}, width[2] = {M, D};
-            for (int q = 0; q < 2; ++q) {
+        /* the feature networks' matrices, rows split over the shards like every parameter; the
+         * MLP's have no step-size modifier of their own here */
+        for (int net = 0; net < nets && F > 0; ++net) {
+            const int64_t base = net * NETSIZE;
+            const int64_t off[3] = {base, base + F * D, base + F * D + 2 * D * M};
+            const int64_t rows[3] = {F, M ? 2 * D : 0, M}, width[3] = {D, M, D};
+            for (int q = 0; q < 3; ++q) {
+                if (rows[q] == 0) continue;
                 float* gw = (float*)malloc(sizeof(float) * (size_t)width[q]);
                 for (int64_t r = 0; r < rows[q]; ++r) {
                     const int64_t o = off[q] + r * width[q];
                     for (int64_t k = 0; k < width[q]; ++k) gw[k] = (float)gproj[o + k];
                     const int64_t shard = c->shared_table ? 0 : r / (rows[q] / S);
-                    kge_oracle_adam(proj + o, proj_m + o, proj_v + o, gw, width[q], alpha[shard], c->beta_m,
-                                    c->beta_v, c->epsilon, c->weight_decay, 0);
+                    kge_oracle_adam(proj + o, proj_m + o, proj_v + o, gw, width[q],
+                                    alpha[shard] * (q == 0 ? c->lr_mod_projection : 1.0f), c->beta_m, c->beta_v,
+                                    c->epsilon, c->weight_decay, 0);
                 }
                 free(gw);
             }
@@ -961,8 +977,9 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
     free(greg_val); free(greg_fh); free(reg_loss);
     free(hidden); free(ghid); free(grel); free(p); free(tl); free(score); free(dist);
     free(dscore); free(dp); free(dtl); free(alpha); free(gproj);
-    free(nv); free(dnv); free(nrm); free(fproj); free(pre); free(gmlp_val);
-    if (drop) { free(hidden_t); free(ghid_t); free(live_h); free(live_t); }
+    free(nv); free(dnv); free(nrm); free(gmlp_val);
+    for (int role = 0; role < 2; ++role) { free(fproj_r[role]); free(pre_r[role]); free(live_r[role]); }
+    if (n_role == 2) { free(hidden_t); free(ghid_t); }
     return 0;
 }
 

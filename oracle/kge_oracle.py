@@ -27,7 +27,8 @@ class Cfg(C.Structure):
             "gamma", "beta_m", "beta_v", "epsilon", "weight_decay", "loss_scale",
             "softmax_correction_weight", "negative_adversarial_scale", "lr_mod_entity",
             "lr_mod_relation", "lr_mod_projection", "reg_emb_power", "reg_emb_weight", "reg_feat_power",
-            "reg_feat_weight", "reg_hid_power", "reg_hid_weight", "dropout")] + [("dropout_seed", C.c_uint32)]
+            "reg_feat_weight", "reg_hid_power", "reg_hid_weight", "dropout")] + [
+                ("dropout_seed", C.c_uint32), ("separate_networks", C.c_int32)]
 
 
 def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score_fn="TransE",
@@ -36,7 +37,8 @@ def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score
              loss_scale=None, softmax_correction_weight=0.0, negative_adversarial_scale=0.0,
              lr_mod_entity=1.0, lr_mod_relation=1.0, lr_mod_projection=1.0,
              embedding_regularisation=(3.0, 0.0), feature_regularisation=(3.0, 0.0),
-             hidden_regularisation=(3.0, 0.0), feature_mlp_size=0, feature_dropout=0.0, dropout_seed=0):
+             hidden_regularisation=(3.0, 0.0), feature_mlp_size=0, feature_dropout=0.0, dropout_seed=0,
+             share_feature_networks=True):
     """The three regularisers are (power, weight) pairs (src/python/poplar_kge.py:104-108)."""
     if loss_scale is None:  # src/python/poplar_kge.py:259-262
         loss_scale = float(batch * n_shard * a2a)
@@ -47,7 +49,7 @@ def make_cfg(*, n_shard, n_entity, n_relation, dim, feature=0, batch, a2a, score
                beta_v, epsilon, weight_decay, loss_scale, softmax_correction_weight,
                negative_adversarial_scale, lr_mod_entity, lr_mod_relation, lr_mod_projection,
                *embedding_regularisation, *feature_regularisation, *hidden_regularisation,
-               float(feature_dropout), int(dropout_seed))
+               float(feature_dropout), int(dropout_seed), int(bool(feature) and not share_feature_networks))
 
 
 def build(force=False):
@@ -238,10 +240,15 @@ class Oracle:
                   "relation_embedding/adam_v"):
             assert state[k].dtype == np.float32 and state[k].flags.c_contiguous, k
         mlp = ("mlp_up_projection", "mlp_down_projection") if cfg.feature and cfg.mlp_size else ()
+        # the feature networks' parameters: one network, or the head's then the tail's
+        # (src/poplar_kge.cpp:268-273), each W then the MLP's Up and Down
+        net_names = [pre + n for pre in (("head_", "tail_") if cfg.separate_networks else ("",))
+                     for n in ("feature_projection",) + mlp]
         if cfg.feature:
-            # with a feature MLP the C side takes W, Up and Down back to back
-            proj_arrays = [np.concatenate([_f32(state[n + x]).reshape(-1) for n in ("feature_projection",) + mlp])
-                           if mlp else state["feature_projection" + x] for x in ("", "/adam_m", "/adam_v")]
+            # the C side takes them back to back
+            proj_arrays = [np.concatenate([_f32(state[n + x]).reshape(-1) for n in net_names])
+                           if len(net_names) > 1 else state["feature_projection" + x]
+                           for x in ("", "/adam_m", "/adam_v")]
             for a in proj_arrays:
                 assert a.dtype == np.float32 and a.flags.c_contiguous
             proj = [_p(a) for a in proj_arrays]
@@ -267,10 +274,10 @@ class Oracle:
             for x, a in zip(suffixes, rel):
                 state["relation_embedding" + x][...] = a[:n]
                 state["relation_normal" + x][...] = a[n:]
-        if mlp:
+        if cfg.feature and len(net_names) > 1:
             for x, a in zip(("", "/adam_m", "/adam_v"), proj_arrays):
                 o = 0
-                for n in ("feature_projection",) + mlp:
+                for n in net_names:
                     state[n + x][...] = a[o:o + state[n + x].size].reshape(state[n + x].shape)
                     o += state[n + x].size
         state["step"] = step.value
@@ -287,16 +294,23 @@ def predict_reference(cfg, state, queries, shard_to_count, n_best):
     [n_shard * n_entity, 3D+F]); queries int[n, 3]."""
     S, NE, D, F = cfg.n_shard, cfg.n_entity, cfg.dim, cfg.feature
     rows = np.asarray(state["entity_data"], np.float64).reshape(S * NE, -1)
-    hidden = rows[:, :D].copy()
-    if F:
-        fh = rows[:, 3 * D:3 * D + F] @ np.asarray(state["feature_projection"], np.float64)
-        if cfg.mlp_size:  # src/poplar_kge.cpp:453-458
-            boom = np.maximum(np.concatenate([hidden, fh], 1) @ np.asarray(state["mlp_up_projection"], np.float64), 0)
-            fh = boom @ np.asarray(state["mlp_down_projection"], np.float64)
-        hidden += fh
+    value = rows[:, :D]
+
+    def hidden_of(prefix):  # entityHidden for the part whose network has this prefix (:439-467)
+        if not F:
+            return value.copy()
+        fh = rows[:, 3 * D:3 * D + F] @ np.asarray(state[prefix + "feature_projection"], np.float64)
+        if cfg.mlp_size:  # :453-458
+            boom = np.maximum(np.concatenate([value, fh], 1)
+                              @ np.asarray(state[prefix + "mlp_up_projection"], np.float64), 0)
+            fh = boom @ np.asarray(state[prefix + "mlp_down_projection"], np.float64)
+        return value + fh
+
+    # the candidates are tails, the queries heads (:811-855)
+    hidden = hidden_of("tail_" if cfg.separate_networks else "")
     rel = np.asarray(state["relation_embedding"], np.float64)
     q = np.asarray(queries, np.int64)
-    h = hidden[q[:, 0] * NE + q[:, 1]]
+    h = (hidden_of("head_") if cfg.separate_networks else hidden)[q[:, 0] * NE + q[:, 1]]
     dot = cfg.score_fn == SCORE["DistMult"] or cfg.distance_fn == DIST["MatMul"]
     r = rel[q[:, 2]]
     if cfg.score_fn == SCORE["RotatE"]:  # src/poplar_kge.cpp:516-530: phases, sine, cosine in float16

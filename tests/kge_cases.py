@@ -10,7 +10,7 @@ def cfg_dict(**kw):
              weight_decay=0.0, loss_scale=None, softmax_correction_weight=0.0,
              negative_adversarial_scale=0.0, embedding_regularisation=(3.0, 0.0),
              feature_regularisation=(3.0, 0.0), hidden_regularisation=(3.0, 0.0), feature_mlp_size=0,
-             feature_dropout=0.0, dropout_seed=0)
+             feature_dropout=0.0, dropout_seed=0, share_feature_networks=True)
     d.update(kw)
     if d["loss_scale"] is None:
         d["loss_scale"] = float(d["batch"] * d["n_shard"] * d["a2a"])
@@ -46,16 +46,16 @@ def make_state(c, rng, warm=True, scale=None):
         st["relation_normal"] = rng.normal(0, scale, (NR, D)).astype(np.float32)
         st["relation_normal/adam_m"] = (rng.normal(0, 0.1, (NR, D)) * warm).astype(np.float32)
         st["relation_normal/adam_v"] = ((0.05 + np.abs(rng.normal(0, 0.3, (NR, D))))**2 * warm).astype(np.float32)
-    if F:
-        st["feature_projection"] = rng.normal(0, scale / np.sqrt(F), (F, D)).astype(np.float32)
-        st["feature_projection/adam_m"] = (rng.normal(0, 0.1, (F, D)) * warm).astype(np.float32)
-        st["feature_projection/adam_v"] = ((0.05 + np.abs(rng.normal(0, 0.3, (F, D))))**2 * warm).astype(np.float32)
+    # one feature network, or a head and a tail one (src/python/poplar_kge.py:652-686)
+    for pre in (("",) if c.get("share_feature_networks", True) else ("head_", "tail_")) if F else ():
+        shapes = [("feature_projection", (F, D), scale / np.sqrt(F))]
         M = c.get("feature_mlp_size", 0)
-        if M:  # shapes and scales of src/python/poplar_kge.py:665-686
-            for name, shape in (("mlp_up_projection", (2 * D, M)), ("mlp_down_projection", (M, D))):
-                st[name] = rng.normal(0, 1 / np.sqrt(shape[0]), shape).astype(np.float32)
-                st[name + "/adam_m"] = (rng.normal(0, 0.1, shape) * warm).astype(np.float32)
-                st[name + "/adam_v"] = ((0.05 + np.abs(rng.normal(0, 0.3, shape)))**2 * warm).astype(np.float32)
+        if M:
+            shapes += [("mlp_up_projection", (2 * D, M), 1 / np.sqrt(2 * D)), ("mlp_down_projection", (M, D), 1 / np.sqrt(M))]
+        for name, shape, sigma in shapes:
+            st[pre + name] = rng.normal(0, sigma, shape).astype(np.float32)
+            st[pre + name + "/adam_m"] = (rng.normal(0, 0.1, shape) * warm).astype(np.float32)
+            st[pre + name + "/adam_v"] = ((0.05 + np.abs(rng.normal(0, 0.3, shape)))**2 * warm).astype(np.float32)
     return st
 
 

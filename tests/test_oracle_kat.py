@@ -324,6 +324,13 @@ STEP_CASES = {
     "feature_dropout_shared_distmult": dict(feature_dropout=0.2, dropout_seed=11, score_fn="DistMult",
                                             distance_fn="MatMul", shared_table=True, n_shard=4, batch=8, a2a=4,
                                             feature=4, n_entity=60),
+    # separate feature networks for the head and the tail use (src/poplar_kge.cpp:268-273)
+    "separate_networks": dict(share_feature_networks=False),
+    "separate_networks_mlp_dropout_l2": dict(share_feature_networks=False, feature_mlp_size=6, feature_dropout=0.3,
+                                             dropout_seed=5, distance_fn="L2", loss_fn="softmax",
+                                             softmax_correction_weight=1.0),
+    "separate_networks_shared_distmult": dict(share_feature_networks=False, score_fn="DistMult", distance_fn="MatMul",
+                                              shared_table=True, n_shard=4, batch=8, a2a=4, feature=4, n_entity=60),
     # norm regularisers (src/poplar_kge.cpp:430-437, 463-465), the WikiKG preset's among them
     "feature_regularisation_p3": dict(feature_regularisation=(3.0, 1e-2), loss_fn="softmax",
                                       softmax_correction_weight=1.0),

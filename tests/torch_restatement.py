@@ -93,24 +93,27 @@ def step(cfg, state, lr, batch_step):
     if cfg["score_fn"] == "TransH":
         normal = T.tensor(state["relation_normal"].astype(np.float64), requires_grad=True)
         params.append(normal)
-    if F:
-        proj = T.tensor(state["feature_projection"].astype(np.float64), requires_grad=True)
-        params.append(proj)
+    # feature networks (src/poplar_kge.cpp:256-273, 439-458): one, or one for a row's use as a
+    # head and one for its use as a tail
+    prefixes = ("",) if cfg.get("share_feature_networks", True) or not F else ("head_", "tail_")
+    nets = {}
+
+    def feature_hidden(prefix):
+        if not F:
+            return emb
+        leaf = lambda n: nets.setdefault(prefix + n, T.tensor(state[prefix + n].astype(np.float64), requires_grad=True))
+        proj = leaf("feature_projection")
         if cfg.get("scoring_bf16"):
-            hidden_u = emb + round_bf16_ste(feat) @ round_bf16_ste(proj)
-        elif cfg.get("feature_mlp_size"):
-            # src/poplar_kge.cpp:453-458; max(x, 0) whose gradient passes where input == output,
-            # so also at exactly 0 (src/pag/pag.cpp:650-658), which `where` reproduces
-            up = T.tensor(state["mlp_up_projection"].astype(np.float64), requires_grad=True)
-            down = T.tensor(state["mlp_down_projection"].astype(np.float64), requires_grad=True)
-            params += [up, down]
-            pre = T.cat([emb, feat @ proj], 1) @ up
-            hidden_u = emb + T.where(pre >= 0, pre, T.zeros_like(pre)) @ down
-        else:
-            hidden_u = emb + feat @ proj
-    else:
-        hidden_u = emb
-    hidden_tail_u = hidden_u
+            return emb + round_bf16_ste(feat) @ round_bf16_ste(proj)
+        if cfg.get("feature_mlp_size"):
+            # :453-458; max(x, 0) whose gradient passes where input == output, so also at exactly 0
+            # (src/pag/pag.cpp:650-658), which `where` reproduces
+            pre = T.cat([emb, feat @ proj], 1) @ leaf("mlp_up_projection")
+            return emb + T.where(pre >= 0, pre, T.zeros_like(pre)) @ leaf("mlp_down_projection")
+        return emb + feat @ proj
+
+    hidden_u = feature_hidden(prefixes[0])
+    hidden_tail_u = feature_hidden(prefixes[-1]) if len(prefixes) == 2 else hidden_u
     drop = cfg.get("feature_dropout", 0.0)
     if F and drop > 0:
         # src/poplar_kge.cpp:459-461, src/pag/pag.cpp:596-617: keep mask / (1 - p) on the feature part,
@@ -118,16 +121,16 @@ def step(cfg, state, lr, batch_step):
         # stands in for the device's random stream); the backward passes where the OUTPUT is
         # non-zero, which differs from the mask where a kept input is exactly 0
         from oracle.kge_oracle import dropout_keep
-        fh = hidden_u - emb
         cols = np.arange(D)[None, :]
 
-        def dropped(role):
+        def dropped(role, hid):
+            fh = hid - emb
             keep = dropout_keep(cfg.get("dropout_seed", 0), int(state["step"]), role, uniq.numpy()[:, None], cols,
                                 drop)
             live = T.tensor(keep) & (fh.detach() != 0)
             return emb + fh * live.to(T.float64) / (1 - float(np.float32(drop)))
 
-        hidden_u, hidden_tail_u = dropped(0), dropped(1)
+        hidden_u, hidden_tail_u = dropped(0, hidden_u), dropped(1, hidden_tail_u)
     hidden = hidden_u[inverse].reshape(S, -1, D)  # [S, NR, D]
     hidden_tail = hidden_tail_u[inverse].reshape(S, -1, D)
     # norm regularisers over every gathered slot, once for the heads' and once for the tails'
@@ -241,9 +244,6 @@ def step(cfg, state, lr, batch_step):
     dense("relation_embedding", rel.grad.numpy())
     if cfg["score_fn"] == "TransH":
         dense("relation_normal", normal.grad.numpy())
-    if F:
-        dense("feature_projection", proj.grad.numpy())
-        if cfg.get("feature_mlp_size"):
-            dense("mlp_up_projection", up.grad.numpy())
-            dense("mlp_down_projection", down.grad.numpy())
+    for name, leaf in nets.items():
+        dense(name, leaf.grad.numpy())
     return per_shard.detach().numpy().astype(np.float32)
