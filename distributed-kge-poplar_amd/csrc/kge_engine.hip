@@ -188,6 +188,10 @@ struct kge_engine {
     // TransH keeps a second row per relation, the hyperplane normal (relation_normal), as rows
     // [n_rel, 2 n_rel) of the relation table: rel_copies = 2, n_rel_rows = 2 n_rel
     int rel_copies = 1, n_rel_rows = 0;
+    // model.share_feature_networks = false: a head and a tail feature network (src/poplar_kge.cpp:268-273);
+    // every parameter / gradient buffer of the feature path then holds the head's part and
+    // the tail's part one after the other, and a distinct row has a hidden row per role
+    int nets = 1;
     float dropout = 0.f;  // model.feature_dropout (training only): two hidden rows per distinct row
     DevBuf<float> fh;          // the feature part of hidden, before dropout
     DevBuf<uint32_t> role_idx;  // the hidden row of every contribution
@@ -196,7 +200,8 @@ struct kge_engine {
     int score_fn, dist_fn, loss_fn;
     bool shared_table;
     float gamma, init_scale, beta_m, beta_v, epsilon, weight_decay, loss_scale, softmax_cw, neg_adv;
-    float lr_mod_entity = 1.f, lr_mod_rel = 1.f, lr_mod_proj = 1.f, lr_mod_normal = 1.f, lr_mod_up = 1.f, lr_mod_down = 1.f;
+    float lr_mod_entity = 1.f, lr_mod_rel = 1.f, lr_mod_normal = 1.f;
+    float lr_mod_proj[2] = {1.f, 1.f}, lr_mod_up[2] = {1.f, 1.f}, lr_mod_down[2] = {1.f, 1.f};  // per network
     uint32_t seed;
     int n_step, rw_batch;
     int predict_hr_batch = 0, predict_n_best = 0;
@@ -247,7 +252,7 @@ struct kge_engine {
     DevBuf<float> mlp_fproj, mlp_concat, mlp_pre, mlp_gpre, mlp_gfp, mlp_gval, p_fproj, p_concat, p_pre;
     DevBuf<float> opnd_n, cmat, dcm, transh_mm, relgrad;  // TransH: [n | tails], c, d loss / d c, its products, relation contributions
     DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, d_loss, d_alpha;
-    // [n_step][entity, relation, normal, projection, mlp up, mlp down][S]; the relation update indexes its two
+    // [n_step][entity, relation, normal, then per feature network projection, mlp up, mlp down][S]; the relation update indexes its two
     // groups as one array (key / rows_per_alpha), a shared table's [relation, normal] pair
     // sits in the first two entries of the relation group
     std::vector<float> h_alpha;
@@ -276,6 +281,23 @@ namespace {
 
 // DistMult, ComplEx and RotatE form a row's gradient contributions from rows of the other
 // table when they are summed (TransE's and TransH's are materialised before that)
+// a step-size modifier of a feature network's parameter, by the variable's name
+// (src/poplar_kge.cpp:321-327): [head_ | tail_]{feature_projection, mlp_up_projection, mlp_down_projection}
+bool feature_modifier(kge_engine& E, const std::string& key, float value) {
+    std::string name = key;
+    int net = 0;
+    if (E.nets == 2) {
+        if (name.rfind("head_", 0) == 0) name = name.substr(5);
+        else if (name.rfind("tail_", 0) == 0) { name = name.substr(5); net = 1; }
+        else return false;
+    }
+    if (name == "feature_projection") E.lr_mod_proj[net] = value;
+    else if (name == "mlp_up_projection" && E.mlp) E.lr_mod_up[net] = value;
+    else if (name == "mlp_down_projection" && E.mlp) E.lr_mod_down[net] = value;
+    else return false;
+    return true;
+}
+
 bool contributions_read_tables(const kge_engine& E) {
     return E.score_fn == SCORE_DISTMULT || E.score_fn == SCORE_COMPLEX || E.score_fn == SCORE_ROTATE;
 }
@@ -414,8 +436,10 @@ void parse_settings(kge_engine& E, const Items& s) {
     if (E.dropout > 0 && E.reg_on)
         throw std::invalid_argument("'model.feature_dropout' > 0 is not implemented together with the norm "
                                     "regularisers (weight > 0)");
-    if (!share && E.F > 0)
-        throw std::invalid_argument("'model.share_feature_networks' = false is not implemented on the HIP device");
+    E.nets = (!share && E.F > 0) ? 2 : 1;
+    if (E.nets == 2 && (E.reg_on || E.score_bf16))
+        throw std::invalid_argument("'model.share_feature_networks' = false is not implemented together with "
+                                    "the norm regularisers (weight > 0) or 'execution.scoring_dtype' = 'bfloat16'");
     for (int i = 0; i < 3; ++i)
         if (E.reg_w[i] > 0 && !(E.reg_p[i] > 0))
             throw std::invalid_argument(std::string("'") + reg_names[i] + ".power' must be positive");
@@ -435,10 +459,10 @@ void parse_settings(kge_engine& E, const Items& s) {
             }
         };
         check("relation_embedding", E.n_rel, E.score_fn == SCORE_ROTATE ? E.D / 2 : E.D);
-        check("feature_projection", E.F, E.D);
+        check(E.nets == 2 ? "head_feature_projection" : "feature_projection", E.F, E.D);
         if (E.mlp) {
-            check("mlp_up_projection", 2 * E.D, E.mlp);
-            check("mlp_down_projection", E.mlp, E.D);
+            check(E.nets == 2 ? "head_mlp_up_projection" : "mlp_up_projection", 2 * E.D, E.mlp);
+            check(E.nets == 2 ? "head_mlp_down_projection" : "mlp_down_projection", E.mlp, E.D);
         }
     }
     E.n_rel_rows = E.n_rel * E.rel_copies;
@@ -446,10 +470,8 @@ void parse_settings(kge_engine& E, const Items& s) {
         const std::string k = mods.map_keys[i];
         if (k == "entity_embedding") E.lr_mod_entity = mods.map_vals[i];
         else if (k == "relation_embedding") E.lr_mod_rel = mods.map_vals[i];
-        else if (k == "feature_projection") E.lr_mod_proj = mods.map_vals[i];
         else if (k == "relation_normal" && E.score_fn == SCORE_TRANSH) E.lr_mod_normal = mods.map_vals[i];
-        else if (k == "mlp_up_projection" && E.mlp) E.lr_mod_up = mods.map_vals[i];
-        else if (k == "mlp_down_projection" && E.mlp) E.lr_mod_down = mods.map_vals[i];
+        else if (feature_modifier(E, k, mods.map_vals[i])) {}
         else
             throw std::invalid_argument("Bad training.learning_rate_modifier: unknown parameter '" + k + "'");
     }
@@ -481,10 +503,13 @@ void parse_settings(kge_engine& E, const Items& s) {
             {(size_t)E.n_rel, (size_t)(E.score_fn == SCORE_ROTATE ? E.D / 2 : E.D)});
         if (E.score_fn == SCORE_TRANSH)  // :252-255
             var(std::string("relation_normal") + suffix, {(size_t)E.n_rel, (size_t)E.D});
-        var(std::string("feature_projection") + suffix, {(size_t)E.F, (size_t)E.D});
-        if (E.mlp) {  // :260-265
-            var(std::string("mlp_up_projection") + suffix, {(size_t)(2 * E.D), (size_t)E.mlp});
-            var(std::string("mlp_down_projection") + suffix, {(size_t)E.mlp, (size_t)E.D});
+        for (int net = 0; net < E.nets; ++net) {  // :256-273
+            const std::string pre = E.nets == 2 ? (net ? "tail_" : "head_") : "";
+            var(pre + "feature_projection" + suffix, {(size_t)E.F, (size_t)E.D});
+            if (E.mlp) {
+                var(pre + "mlp_up_projection" + suffix, {(size_t)(2 * E.D), (size_t)E.mlp});
+                var(pre + "mlp_down_projection" + suffix, {(size_t)E.mlp, (size_t)E.D});
+            }
         }
     }
 }
@@ -505,7 +530,7 @@ void allocate(kge_engine& E) {
     E.table.zero(st);
     const size_t rel_n = (size_t)E.n_rel_rows * E.Dp, proj_n = (size_t)E.Fp * E.Dp;
     for (DevBuf<float>* b : {&E.rel, &E.rel_m, &E.rel_v}) { b->alloc(rel_n); b->zero(st); }
-    for (DevBuf<float>* b : {&E.proj, &E.proj_m, &E.proj_v}) { b->alloc(proj_n); b->zero(st); }
+    for (DevBuf<float>* b : {&E.proj, &E.proj_m, &E.proj_v}) { b->alloc(E.nets * proj_n); b->zero(st); }
 
     const size_t ns = E.n_step, S = E.S, B = E.B, A = E.A, R = E.R, SB = S * B;
     E.d_remote.alloc(ns * R);
@@ -569,12 +594,11 @@ void allocate(kge_engine& E) {
         E.relgrad.alloc(2 * SB * E.Dp);
     }
     if (E.F) {
-        E.hidden.alloc((E.dropout > 0 ? 2 : 1) * R * E.Dp);
-        if (E.dropout > 0) {
-            E.fh.alloc(R * E.Dp);
-            E.role_idx.alloc(R);
-        }
-        E.gsum.alloc(R * E.Dp);
+        const bool roles = E.dropout > 0 || E.nets == 2;
+        E.hidden.alloc((roles ? 2 : 1) * R * E.Dp);
+        if (E.dropout > 0) E.fh.alloc(E.nets * R * E.Dp);
+        if (roles) E.role_idx.alloc(R);
+        E.gsum.alloc(E.nets * R * E.Dp);
         E.gsum.zero(E.stream);  // rows past a step's distinct count are read (times zero): keep them finite
         E.featd.alloc(R * E.Fp);
         E.gproj_part.alloc((size_t)16 * E.Fp * E.Dp);
@@ -585,16 +609,16 @@ void allocate(kge_engine& E) {
             E.gT16.alloc(R * E.Dp);
             E.projR.alloc((size_t)E.Fp * E.Dp);
         }
-        E.gproj.alloc(proj_n);
+        E.gproj.alloc(E.nets * proj_n);
         if (E.mlp) {
-            const size_t M = E.mlp, up_n = 2 * (size_t)E.Dp * M, down_n = M * E.Dp;
-            for (DevBuf<float>* b : {&E.up, &E.up_m, &E.up_v, &E.g_up}) { b->alloc(up_n); b->zero(st); }
-            for (DevBuf<float>* b : {&E.down, &E.down_m, &E.down_v, &E.g_down}) { b->alloc(down_n); b->zero(st); }
-            E.mlp_fproj.alloc(R * E.Dp);
-            E.mlp_concat.alloc(R * 2 * E.Dp);
-            E.mlp_pre.alloc(R * M);
-            E.mlp_gpre.alloc(R * M);
-            E.mlp_gfp.alloc(R * E.Dp);
+            const size_t M = E.mlp, up_n = 2 * (size_t)E.Dp * M, down_n = M * E.Dp, N = E.nets;
+            for (DevBuf<float>* b : {&E.up, &E.up_m, &E.up_v, &E.g_up}) { b->alloc(N * up_n); b->zero(st); }
+            for (DevBuf<float>* b : {&E.down, &E.down_m, &E.down_v, &E.g_down}) { b->alloc(N * down_n); b->zero(st); }
+            E.mlp_fproj.alloc(N * R * E.Dp);
+            E.mlp_concat.alloc(N * R * 2 * E.Dp);
+            E.mlp_pre.alloc(N * R * M);
+            E.mlp_gpre.alloc(N * R * M);
+            E.mlp_gfp.alloc(N * R * E.Dp);
             E.mlp_gval.alloc(R * E.Dp);
             // rows past a step's distinct count are read by the projection gradient (times zero)
             E.mlp_gfp.zero(st);
@@ -616,7 +640,7 @@ void allocate(kge_engine& E) {
     }
     E.loss_part.alloc(ns * S * E.n_part);
     E.d_loss.alloc(S);
-    E.d_alpha.alloc(ns * 6 * S);
+    E.d_alpha.alloc(ns * 9 * S);
 
     const size_t io_n = (size_t)E.S * E.rw_batch;
     E.io_rows.alloc(io_n);
@@ -628,11 +652,11 @@ void allocate(kge_engine& E) {
 // ---- variables: "read" / "write" (src/poplar_kge.cpp:977-991) ----------------
 
 void run_read_write(kge_engine& E, bool write, const Items& in) {
-    const std::string name = in.str("name");
+    const std::string full_name = in.str("name");
     const Variable* var = nullptr;
-    for (auto& v : E.variables) if (v.name == name) var = &v;
-    if (!var) throw std::invalid_argument("Key not found '" + name + "'");
-    if (name == "step") {
+    for (auto& v : E.variables) if (v.name == full_name) var = &v;
+    if (!var) throw std::invalid_argument("Key not found '" + full_name + "'");
+    if (full_name == "step") {
         uint32_t* v = (uint32_t*)in.array("value", KGE_U32, var->shape);
         if (write) E.step = v[0];
         else for (int s = 0; s < E.S; ++s) v[s] = E.step;
@@ -641,15 +665,22 @@ void run_read_write(kge_engine& E, bool write, const Items& in) {
     float* host = (float*)in.array("value", KGE_F32, var->shape);
     DevBuf<float>* buf = nullptr;
     size_t row0 = 0;  // first device row of the variable
+    // the feature networks' variables: head_ / tail_ name the network when there are two
+    std::string name = full_name;
+    size_t net = 0;
+    if (E.nets == 2 && (name.rfind("head_", 0) == 0 || name.rfind("tail_", 0) == 0)) {
+        net = name[0] == 't';
+        name = name.substr(5);
+    }
     if (name == "relation_embedding") buf = &E.rel;
     else if (name == "relation_embedding/adam_m") buf = &E.rel_m;
     else if (name == "relation_embedding/adam_v") buf = &E.rel_v;
     else if (name == "relation_normal") { buf = &E.rel; row0 = E.n_rel; }
     else if (name == "relation_normal/adam_m") { buf = &E.rel_m; row0 = E.n_rel; }
     else if (name == "relation_normal/adam_v") { buf = &E.rel_v; row0 = E.n_rel; }
-    else if (name == "feature_projection") buf = &E.proj;
-    else if (name == "feature_projection/adam_m") buf = &E.proj_m;
-    else if (name == "feature_projection/adam_v") buf = &E.proj_v;
+    else if (name == "feature_projection") { buf = &E.proj; row0 = net * E.Fp; }
+    else if (name == "feature_projection/adam_m") { buf = &E.proj_m; row0 = net * E.Fp; }
+    else if (name == "feature_projection/adam_v") { buf = &E.proj_v; row0 = net * E.Fp; }
     const size_t rows = var->shape[0], cols = var->shape[1];
     if (rows == 0 || cols == 0) return;
     HIP_CHECK(hipStreamSynchronize(E.stream));
@@ -658,6 +689,7 @@ void run_read_write(kge_engine& E, bool write, const Items& in) {
         const bool m = name.size() > 7 && name.compare(name.size() - 7, 7, "/adam_m") == 0;
         const bool v = name.size() > 7 && name.compare(name.size() - 7, 7, "/adam_v") == 0;
         float* dev = is_up ? (m ? E.up_m.p : v ? E.up_v.p : E.up.p) : (m ? E.down_m.p : v ? E.down_v.p : E.down.p);
+        dev += net * (is_up ? 2 * (size_t)E.Dp * E.mlp : (size_t)E.mlp * E.Dp);
         // Up: host rows [0, D) and [D, 2 D) are device rows [0, D) and [Dp, Dp + D), pitch M;
         // Down: host [M, D] in device rows of pitch Dp
         const size_t D = E.D, Dp = E.Dp, M = E.mlp;
@@ -899,48 +931,57 @@ void run_step(kge_engine& E, int i) {
     table_rows.index = ckey; table_rows.count = E.Dp; table_rows.vec = 1;
     RowSource ent = table_rows;
 
-    FeatureArgs fa = {};
-    MlpArgs ma = {};
+    // Feature path.  One feature network, or a head and a tail one (index 0 / 1 of fa, ma and
+    // of every per-network buffer).  A distinct row has one hidden row, or two (its use as a head,
+    // its use as a tail) when the networks are separate or with dropout.
+    FeatureArgs fa[2] = {};
+    MlpArgs ma[2] = {};
     DropoutArgs da = {};
+    const int nets = E.nets;
+    const bool drop = E.dropout > 0, roles = E.F && (drop || nets == 2);
+    const size_t rows_n = R * (size_t)E.Dp;  // elements of one per-row buffer
     if (E.F) {
-        fa.uniq_key = e_uniq; fa.counts = e_counts; fa.max_rows = (int)R;
-        fa.emb_base = E.table.p; fa.feat_base = E.table.p + E.L.off_f; fa.pitch = E.L.pitch;
-        fa.emb_etype = E.L.emb_etype; fa.feat_etype = E.L.feat_etype;
-        fa.Dp = E.Dp; fa.Fp = E.Fp; fa.proj = E.proj.p;
-        fa.featd = E.featd.p; fa.gproj_part = E.gproj_part.p; fa.use_mfma = E.use_mfma;
-        fa.round_bf16 = E.score_bf16 ? 1 : 0; fa.projR = E.projR.p;
-        fa.feat16 = E.feat16.p; fa.featT16 = E.featT16.p; fa.projT16 = E.projT16.p; fa.gT16 = E.gT16.p;
-        const bool drop = E.dropout > 0;
-        if (E.mlp) {  // feature . W alone, then the MLP on [embedding | feature . W]
-            KernelTimer t(E, K_HIDDEN);
-            FeatureArgs fp = fa;
+        KernelTimer t(E, K_HIDDEN);
+        for (int net = 0; net < nets; ++net) {
+            FeatureArgs& f = fa[net];
+            f.uniq_key = e_uniq; f.counts = e_counts; f.max_rows = (int)R;
+            f.emb_base = E.table.p; f.feat_base = E.table.p + E.L.off_f; f.pitch = E.L.pitch;
+            f.emb_etype = E.L.emb_etype; f.feat_etype = E.L.feat_etype;
+            f.Dp = E.Dp; f.Fp = E.Fp; f.proj = E.proj.p + (size_t)net * E.Fp * E.Dp;
+            f.featd = E.featd.p; f.gproj_part = E.gproj_part.p; f.use_mfma = E.use_mfma;
+            f.round_bf16 = E.score_bf16 ? 1 : 0; f.projR = E.projR.p;
+            f.feat16 = E.feat16.p; f.featT16 = E.featT16.p; f.projT16 = E.projT16.p; f.gT16 = E.gT16.p;
+            FeatureArgs fp = f;  // the feature part alone, without the embedding
             fp.emb_base = nullptr;
-            launch_hidden_fwd(fp, E.mlp_fproj.p, st);
-            ma.uniq_key = e_uniq; ma.counts = e_counts; ma.max_rows = (int)R;
-            ma.emb_base = E.table.p; ma.pitch = E.L.pitch; ma.emb_etype = E.L.emb_etype;
-            ma.Dp = E.Dp; ma.M = E.mlp; ma.up = E.up.p; ma.down = E.down.p;
-            ma.concat = E.mlp_concat.p; ma.pre = E.mlp_pre.p;
-            ma.add_value = drop ? 0 : 1;
-            launch_mlp_fwd(ma, E.mlp_fproj.p, drop ? E.fh.p : E.hidden.p, st);
-        } else if (drop) {
-            KernelTimer t(E, K_HIDDEN);
-            FeatureArgs fp = fa;
-            fp.emb_base = nullptr;
-            launch_hidden_fwd(fp, E.fh.p, st);
-        } else
-        { KernelTimer t(E, K_HIDDEN); launch_hidden_fwd(fa, E.hidden.p, st); }
+            float* hid = E.hidden.p + net * rows_n;          // value + feature part
+            float* part = drop ? E.fh.p + net * rows_n : hid;  // what this network's kernels write
+            if (E.mlp) {  // feature . W alone, then the MLP on [embedding | feature . W]
+                MlpArgs& m = ma[net];
+                float* fproj = E.mlp_fproj.p + net * rows_n;
+                launch_hidden_fwd(fp, fproj, st);
+                m.uniq_key = e_uniq; m.counts = e_counts; m.max_rows = (int)R;
+                m.emb_base = E.table.p; m.pitch = E.L.pitch; m.emb_etype = E.L.emb_etype;
+                m.Dp = E.Dp; m.M = E.mlp;
+                m.up = E.up.p + (size_t)net * 2 * E.Dp * E.mlp; m.down = E.down.p + (size_t)net * E.mlp * E.Dp;
+                m.concat = E.mlp_concat.p + 2 * net * rows_n; m.pre = E.mlp_pre.p + (size_t)net * R * E.mlp;
+                m.add_value = drop ? 0 : 1;
+                launch_mlp_fwd(m, fproj, part, st);
+            } else {
+                launch_hidden_fwd(drop ? fp : f, part, st);
+            }
+        }
         ent.base = (const char*)E.hidden.p; ent.pitch = (int64_t)E.Dp * 4; ent.etype = ET_F32;
         ent.index = E.e_item_row.p + i * R;
-        if (drop) {
-            // a head row and a tail row per distinct row (src/poplar_kge.cpp:459-461, once per
-            // entityHidden call); every contribution reads the one of its role
-            KernelTimer t(E, K_HIDDEN);
+        if (roles) {
             da.uniq_key = e_uniq; da.counts = e_counts; da.max_rows = (int)R;
             da.emb_base = E.table.p; da.pitch = E.L.pitch; da.emb_etype = E.L.emb_etype; da.Dp = E.Dp;
             da.seed = E.seed; da.step = (uint32_t)(E.step_of_first + i);
             da.threshold = (uint32_t)((double)E.dropout * 4294967296.0);
-            da.scale = 1.f / (1.f - E.dropout);
-            launch_dropout_hidden(da, E.fh.p, E.hidden.p, st);
+            da.scale = drop ? 1.f / (1.f - E.dropout) : 1.f;
+            da.enabled = drop ? 1 : 0;
+            // with dropout (src/poplar_kge.cpp:459-461, once per entityHidden call) the two hidden
+            // rows are formed here; every contribution reads the one of its role
+            if (drop) launch_dropout_hidden(da, E.fh.p, E.fh.p + (nets - 1) * rows_n, E.hidden.p, st);
             launch_role_index(E.e_item_row.p + i * R, (int)SB, (int)R, E.role_idx.p, st);
             ent.index = E.role_idx.p;
         }
@@ -1046,7 +1087,7 @@ void run_step(kge_engine& E, int i) {
                         E.reg_loss_part.p + (size_t)i * E.S, st);
     }
 
-    const float* alpha = E.d_alpha.p + (size_t)i * 6 * E.S;
+    const float* alpha = E.d_alpha.p + (size_t)i * 9 * E.S;
     AdamArgs aa = {};
     aa.Dp = E.Dp;
     aa.beta_m = E.beta_m; aa.beta_v = E.beta_v;
@@ -1108,7 +1149,7 @@ void run_step(kge_engine& E, int i) {
     ae.counts = e_counts; ae.max_rows = (int)R;
     ae.partial = E.partial.p;
     // (with dropout the feature part's gradient is formed per role by launch_role_sums)
-    ae.grad_out = (E.F && !(E.dropout > 0)) ? E.gsum.p : nullptr;
+    ae.grad_out = (E.F && !roles) ? E.gsum.p : nullptr;
     if (E.reg_on) { ae.grad_add = E.reg_val.p; ae.grad_out_add = E.reg_fh.p; }
     ae.p_base = E.table.p; ae.m_base = E.table.p + E.L.off_m; ae.v_base = E.table.p + E.L.off_s;
     ae.pitch = E.L.pitch; ae.p_etype = E.L.emb_etype; ae.m_etype = E.L.mom_etype; ae.v_is_sqrt = 1;
@@ -1120,16 +1161,19 @@ void run_step(kge_engine& E, int i) {
     // backward per row, then the update with what that adds.
     auto entity_update = [&]() {
         KernelTimer t(E, K_ADAM_ENT);
-        if (E.dropout > 0)
-            launch_role_sums(da, esrc, ae.seg_start, ae.seg_real, E.fh.p, E.gsum.p, st);
+        if (roles)  // the feature part's gradient per use: one array (added up) or one per network
+            launch_role_sums(da, esrc, ae.seg_start, ae.seg_real, E.fh.p, E.fh.p + (nets - 1) * rows_n, E.gsum.p,
+                             nets == 2 ? E.gsum.p + rows_n : nullptr, st);
         if (!E.mlp) { launch_adam_rows(ae, st); return; }
-        if (!(E.dropout > 0)) {
+        if (!roles) {
             AdamArgs sum = ae;
             sum.no_update = 1;
             launch_adam_rows(sum, st);
         }
-        launch_mlp_bwd_rows(ma, E.gsum.p, E.reg_on ? E.reg_val.p : nullptr, E.mlp_gpre.p, E.mlp_gval.p,
-                            E.mlp_gfp.p, st);
+        for (int net = 0; net < nets; ++net)  // what reaches the embedding adds up over the networks
+            launch_mlp_bwd_rows(ma[net], E.gsum.p + net * rows_n,
+                                net ? E.mlp_gval.p : (E.reg_on ? E.reg_val.p : nullptr),
+                                E.mlp_gpre.p + (size_t)net * R * E.mlp, E.mlp_gval.p, E.mlp_gfp.p + net * rows_n, st);
         AdamArgs upd = ae;
         upd.grad_out = nullptr; upd.grad_out_add = nullptr; upd.grad_add = E.mlp_gval.p;
         launch_adam_rows(upd, st);
@@ -1145,7 +1189,7 @@ void run_step(kge_engine& E, int i) {
         ar.grad_out = nullptr; ar.no_update = 0;
         ar.grad_direct = E.rel_gsum.p;
         { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
-    } else if (E.mlp || E.dropout > 0) {
+    } else if (E.mlp || roles) {
         entity_update();
         KernelTimer t(E, K_ADAM_REL);
         launch_adam_rows(ar, st);
@@ -1154,62 +1198,55 @@ void run_step(kge_engine& E, int i) {
         launch_adam_rows2(ae, ar, st);
     }
 
-    // dense Adam on rows [0, rows) of a parameter whose row r sits at device element
-    // offset(r); shard s owns rows [s*rows/S, (s+1)*rows/S) and its step size
-    auto dense_adam = [&](float* p, float* m, float* v, const float* g, int rows, int64_t width, int group) {
+    // dense Adam on rows [0, rows) of a parameter of row pitch `width`; shard s owns rows
+    // [s*rows/S, (s+1)*rows/S) and its step size (group `group` of this step's step sizes)
+    auto dense_adam = [&](float* p, float* m, float* v, const float* g, int rows, int last_row, int64_t width,
+                          int group) {
         const int n_slices = E.shared_table ? 1 : E.S;
         for (int s = 0; s < n_slices; ++s) {
             const int r0 = E.shared_table ? 0 : s * (rows / E.S);
-            const int r1 = (E.shared_table || s == E.S - 1) ? rows : (s + 1) * (rows / E.S);
+            const int r1 = (E.shared_table || s == E.S - 1) ? last_row : (s + 1) * (rows / E.S);
             if (r1 <= r0) continue;
             const size_t o = (size_t)r0 * width;
             launch_adam_flat(p + o, m + o, v + o, g + o, (int64_t)(r1 - r0) * width,
-                             E.h_alpha[((size_t)i * 6 + group) * E.S + s], E.beta_m, E.beta_v, E.epsilon,
+                             E.h_alpha[((size_t)i * 9 + group) * E.S + s], E.beta_m, E.beta_v, E.epsilon,
                              E.weight_decay, 0, st);
         }
     };
-    if (E.mlp) {
-        KernelTimer t(E, K_PROJ_GRAD);
-        // d Down = relu(pre)^T . g, d Up = concat^T . gpre, summed over the distinct rows in order
-        launch_rows_atb(E.mlp_pre.p, E.mlp, E.mlp, true, E.gsum.p, E.Dp, E.Dp, e_counts, E.g_down.p, st);
-        launch_rows_atb(E.mlp_concat.p, 2 * E.Dp, 2 * E.Dp, false, E.mlp_gpre.p, E.mlp, E.mlp, e_counts,
-                        E.g_up.p, st);
-    }
-    if (E.mlp) {
-        KernelTimer t(E, K_ADAM_PROJ);
-        // Up's host rows [0, D) and [D, 2 D) are device rows [0, D) and [Dp, Dp + D): a shard's
-        // slice of host rows is updated half by half
-        const int n_slices = E.shared_table ? 1 : E.S, rows = 2 * E.D;
-        for (int s = 0; s < n_slices; ++s) {
-            const int r0 = E.shared_table ? 0 : s * (rows / E.S);
-            const int r1 = (E.shared_table || s == E.S - 1) ? rows : (s + 1) * (rows / E.S);
-            for (int half = 0; half < 2; ++half) {
-                const int lo = std::max(r0, half * E.D), hi = std::min(r1, (half + 1) * E.D);
-                if (hi <= lo) continue;
-                const size_t o = (size_t)(lo + half * (E.Dp - E.D)) * E.mlp;
-                launch_adam_flat(E.up.p + o, E.up_m.p + o, E.up_v.p + o, E.g_up.p + o, (int64_t)(hi - lo) * E.mlp,
-                                 E.h_alpha[((size_t)i * 6 + 4) * E.S + s], E.beta_m, E.beta_v, E.epsilon,
-                                 E.weight_decay, 0, st);
+    for (int net = 0; net < nets && E.F; ++net) {
+        const float* g_rows = E.gsum.p + net * rows_n;  // d loss / d (feature part) per distinct row
+        if (E.mlp) {
+            const size_t up_o = (size_t)net * 2 * E.Dp * E.mlp, down_o = (size_t)net * E.mlp * E.Dp;
+            { KernelTimer t(E, K_PROJ_GRAD);
+              // d Down = relu(pre)^T . g, d Up = concat^T . gpre, summed over the distinct rows in order
+              launch_rows_atb(ma[net].pre, E.mlp, E.mlp, true, g_rows, E.Dp, E.Dp, e_counts, E.g_down.p + down_o, st);
+              launch_rows_atb(ma[net].concat, 2 * E.Dp, 2 * E.Dp, false, E.mlp_gpre.p + (size_t)net * R * E.mlp,
+                              E.mlp, E.mlp, e_counts, E.g_up.p + up_o, st); }
+            KernelTimer t(E, K_ADAM_PROJ);
+            // Up's host rows [0, D) and [D, 2 D) are device rows [0, D) and [Dp, Dp + D): a shard's
+            // slice of host rows is updated half by half
+            const int n_slices = E.shared_table ? 1 : E.S, rows = 2 * E.D;
+            for (int s = 0; s < n_slices; ++s) {
+                const int r0 = E.shared_table ? 0 : s * (rows / E.S);
+                const int r1 = (E.shared_table || s == E.S - 1) ? rows : (s + 1) * (rows / E.S);
+                for (int half = 0; half < 2; ++half) {
+                    const int lo = std::max(r0, half * E.D), hi = std::min(r1, (half + 1) * E.D);
+                    if (hi <= lo) continue;
+                    const size_t o = up_o + (size_t)(lo + half * (E.Dp - E.D)) * E.mlp;
+                    launch_adam_flat(E.up.p + o, E.up_m.p + o, E.up_v.p + o, E.g_up.p + o, (int64_t)(hi - lo) * E.mlp,
+                                     E.h_alpha[((size_t)i * 9 + 4 + 3 * net) * E.S + s], E.beta_m, E.beta_v,
+                                     E.epsilon, E.weight_decay, 0, st);
+                }
             }
+            dense_adam(E.down.p + down_o, E.down_m.p + down_o, E.down_v.p + down_o, E.g_down.p + down_o, E.mlp, E.mlp,
+                       E.Dp, 5 + 3 * net);
+            g_rows = E.mlp_gfp.p + net * rows_n;  // the projected features' gradient
         }
-        dense_adam(E.down.p, E.down_m.p, E.down_v.p, E.g_down.p, E.mlp, E.Dp, 5);
-    }
-
-    if (E.F) {
-        { KernelTimer t(E, K_PROJ_GRAD);
-          launch_proj_grad(fa, E.mlp ? E.mlp_gfp.p : E.gsum.p, E.gproj.p, st); }
-        // dense Adam on the projection; shard s owns rows [s*F/S, (s+1)*F/S) and its step size
+        const size_t proj_o = (size_t)net * E.Fp * E.Dp;
+        { KernelTimer t(E, K_PROJ_GRAD); launch_proj_grad(fa[net], g_rows, E.gproj.p + proj_o, st); }
         KernelTimer t(E, K_ADAM_PROJ);
-        const int n_slices = E.shared_table ? 1 : E.S;
-        for (int s = 0; s < n_slices; ++s) {
-            const int r0 = E.shared_table ? 0 : s * (E.F / E.S);
-            const int r1 = (E.shared_table || s == E.S - 1) ? E.Fp : (s + 1) * (E.F / E.S);
-            if (r1 <= r0) continue;
-            const size_t o = (size_t)r0 * E.Dp;
-            launch_adam_flat(E.proj.p + o, E.proj_m.p + o, E.proj_v.p + o, E.gproj.p + o,
-                             (int64_t)(r1 - r0) * E.Dp, E.h_alpha[((size_t)i * 6 + 3) * E.S + s],
-                             E.beta_m, E.beta_v, E.epsilon, E.weight_decay, 0, st);
-        }
+        dense_adam(E.proj.p + proj_o, E.proj_m.p + proj_o, E.proj_v.p + proj_o, E.gproj.p + proj_o, E.F, E.Fp, E.Dp,
+                   3 + 3 * net);
     }
     HIP_CHECK(hipGetLastError());
 }
@@ -1242,23 +1279,25 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
         throw std::invalid_argument("train_step_loop with staged=true needs a preceding stage_batch");
     }
     // step sizes of every step of this call (adamStepSizeAutoIncrement, frnn.cpp:42-59)
-    E.h_alpha.resize((size_t)E.n_step * 6 * S);
+    E.h_alpha.resize((size_t)E.n_step * 9 * S);
     for (int i = s0; i < s0 + sn; ++i) {
         const double t = (double)(E.step + (uint32_t)(i - s0) + 1u);
         const double factor = std::sqrt(1.0 - std::pow((double)E.beta_v, t)) / (1.0 - std::pow((double)E.beta_m, t));
         for (size_t s = 0; s < S; ++s) {
             const float a = (float)(factor * (double)lr[s]);
-            E.h_alpha[((size_t)i * 6 + 0) * S + s] = a * E.lr_mod_entity;
-            E.h_alpha[((size_t)i * 6 + 1) * S + s] = a * E.lr_mod_rel;
-            E.h_alpha[((size_t)i * 6 + 2) * S + s] = a * E.lr_mod_normal;
-            E.h_alpha[((size_t)i * 6 + 3) * S + s] = a * E.lr_mod_proj;
-            E.h_alpha[((size_t)i * 6 + 4) * S + s] = a * E.lr_mod_up;
-            E.h_alpha[((size_t)i * 6 + 5) * S + s] = a * E.lr_mod_down;
+            E.h_alpha[((size_t)i * 9 + 0) * S + s] = a * E.lr_mod_entity;
+            E.h_alpha[((size_t)i * 9 + 1) * S + s] = a * E.lr_mod_rel;
+            E.h_alpha[((size_t)i * 9 + 2) * S + s] = a * E.lr_mod_normal;
+            for (int net = 0; net < 2; ++net) {
+                E.h_alpha[((size_t)i * 9 + 3 + 3 * net) * S + s] = a * E.lr_mod_proj[net];
+                E.h_alpha[((size_t)i * 9 + 4 + 3 * net) * S + s] = a * E.lr_mod_up[net];
+                E.h_alpha[((size_t)i * 9 + 5 + 3 * net) * S + s] = a * E.lr_mod_down[net];
+            }
         }
         // a shared table has one step size per parameter: the relation update finds the
         // normal rows' at index 1 of its array
         if (E.shared_table && E.score_fn == SCORE_TRANSH)
-            E.h_alpha[((size_t)i * 6 + 1) * S + 1] = (float)(factor * (double)lr[0]) * E.lr_mod_normal;
+            E.h_alpha[((size_t)i * 9 + 1) * S + 1] = (float)(factor * (double)lr[0]) * E.lr_mod_normal;
     }
     HIP_CHECK(hipMemcpyAsync(E.d_alpha.p, E.h_alpha.data(), E.h_alpha.size() * 4, hipMemcpyHostToDevice, st));
     HIP_CHECK(hipEventRecord(E.ev[1], st));
@@ -1377,7 +1416,8 @@ void run_predict(kge_engine& E, const Items& in) {
     HIP_CHECK(hipMemcpyAsync(E.p_rel.p, rels.data(), (size_t)Qp * 4, hipMemcpyHostToDevice, st));
 
     // rows `idx[0..n)` of the table as a row source: the embeddings, or hidden = emb + feature . W
-    auto rows_of = [&](const uint32_t* idx, int n) {
+    // (`net`: the head's feature network for the queries, the tail's for the candidates)
+    auto rows_of = [&](const uint32_t* idx, int n, int net) {
         RowSource r;
         r.base = E.table.p; r.pitch = E.L.pitch; r.etype = E.L.emb_etype;
         r.index = idx; r.count = Dp; r.vec = 1;
@@ -1389,7 +1429,7 @@ void run_predict(kge_engine& E, const Items& in) {
             fa.uniq_key = idx; fa.counts = E.p_count.p; fa.max_rows = n;
             fa.emb_base = E.table.p; fa.feat_base = E.table.p + E.L.off_f; fa.pitch = E.L.pitch;
             fa.emb_etype = E.L.emb_etype; fa.feat_etype = E.L.feat_etype;
-            fa.Dp = Dp; fa.Fp = E.Fp; fa.proj = E.proj.p;
+            fa.Dp = Dp; fa.Fp = E.Fp; fa.proj = E.proj.p + (size_t)net * E.Fp * Dp;
             fa.featd = E.p_featd.p; fa.use_mfma = E.use_mfma;
             if (E.mlp) {
                 FeatureArgs fp = fa;
@@ -1398,7 +1438,8 @@ void run_predict(kge_engine& E, const Items& in) {
                 MlpArgs ma = {};
                 ma.uniq_key = idx; ma.counts = E.p_count.p; ma.max_rows = n;
                 ma.emb_base = E.table.p; ma.pitch = E.L.pitch; ma.emb_etype = E.L.emb_etype;
-                ma.Dp = Dp; ma.M = E.mlp; ma.up = E.up.p; ma.down = E.down.p;
+                ma.Dp = Dp; ma.M = E.mlp;
+                ma.up = E.up.p + (size_t)net * 2 * Dp * E.mlp; ma.down = E.down.p + (size_t)net * E.mlp * Dp;
                 ma.concat = E.p_concat.p; ma.pre = E.p_pre.p; ma.add_value = 1;
                 launch_mlp_fwd(ma, E.p_fproj.p, E.p_hidden.p, st);
             } else
@@ -1408,7 +1449,7 @@ void run_predict(kge_engine& E, const Items& in) {
         return r;
     };
     // predicted tails of all queries: dense rows [0, Qp)
-    launch_gather_operands(rows_of(E.p_idx.p, Qp), E.rel.p, E.p_rel.p, rel_mode_of(E), E.D / 2, Qp,
+    launch_gather_operands(rows_of(E.p_idx.p, Qp, 0), E.rel.p, E.p_rel.p, rel_mode_of(E), E.D / 2, Qp,
                            Qp, Dp, E.p_opnd.p, nullptr, st);
 
     const bool transh = E.score_fn == SCORE_TRANSH;
@@ -1447,7 +1488,7 @@ void run_predict(kge_engine& E, const Items& in) {
             const int live = (int)std::min<int64_t>(chunk, hi - r0);
             uint32_t* tail_idx = E.p_idx.p + Qp;
             launch_row_range((uint32_t)(table_off + r0), live, chunk, tail_idx, st);
-            launch_gather_operands(rows_of(tail_idx, chunk), E.rel.p, nullptr, 0, 0, 0, chunk, Dp,
+            launch_gather_operands(rows_of(tail_idx, chunk, E.nets - 1), E.rel.p, nullptr, 0, 0, 0, chunk, Dp,
                                    E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
             if (transh) {  // transHScore (:551-565): c = n . tail, then the L1 part
                 HIP_CHECK(hipMemcpyAsync(E.p_opnd_n.p + (size_t)Qp * Dp, E.p_opnd.p + (size_t)Qp * Dp,

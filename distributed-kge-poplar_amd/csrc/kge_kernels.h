@@ -376,14 +376,19 @@ struct DropoutArgs {
     uint32_t seed, step;   // model.seed, the optimiser step the mask belongs to
     uint32_t threshold;    // p * 2^32: an element is kept where its hash is at least this
     float scale;           // 1 / (1 - p)
+    int enabled;           // 0: no dropout (separate feature networks alone): keep everything, scale 1
 };
 // hidden [2 max_rows, Dp]: row u = value + dropped feature part for the head use, row
-// max_rows + u for the tail use; fh [max_rows, Dp] = the feature part
-void launch_dropout_hidden(const DropoutArgs& a, const float* fh, float* hidden, hipStream_t stream);
+// max_rows + u for the tail use; fh_head / fh_tail [max_rows, Dp] = the feature part for either
+// use (one array unless the feature networks are separate)
+void launch_dropout_hidden(const DropoutArgs& a, const float* fh_head, const float* fh_tail, float* hidden,
+                           hipStream_t stream);
 // out[c] = item_row[c] (+ n for c >= n_head): the hidden row contribution c reads
 void launch_role_index(const uint32_t* item_row, int n_head, int n, uint32_t* out, hipStream_t stream);
-// out [max_rows, Dp]: the feature part's gradient of every distinct row from its contributions
+// The feature part's gradient of every distinct row [max_rows, Dp] from its contributions:
+// out_head alone (the head and tail uses added up) or one array per use
 void launch_role_sums(const DropoutArgs& a, const ContribSrc& cs, const uint32_t* seg_start, const uint32_t* seg_real,
-                      const float* fh, float* out, hipStream_t stream);
+                      const float* fh_head, const float* fh_tail, float* out_head, float* out_tail,
+                      hipStream_t stream);
 
 }  // namespace kge

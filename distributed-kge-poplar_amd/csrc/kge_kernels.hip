@@ -3630,8 +3630,10 @@ DEVINL bool dropout_keep(uint32_t seed, uint32_t step, uint32_t role, uint32_t k
     return x >= threshold;
 }
 
-// one wave per distinct row: fh [max_rows, Dp] = the feature part, hidden [2 max_rows, Dp]
-__global__ __launch_bounds__(256) void k_dropout_hidden(DropoutArgs a, const float* __restrict__ fh,
+// one wave per distinct row: fh_head / fh_tail [max_rows, Dp] = the feature part for either use
+// (the same array unless the feature networks are separate), hidden [2 max_rows, Dp]
+__global__ __launch_bounds__(256) void k_dropout_hidden(DropoutArgs a, const float* __restrict__ fh_head,
+                                                        const float* __restrict__ fh_tail,
                                                         float* __restrict__ hidden) {
     const int lane = threadIdx.x & 63;
     const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -3640,20 +3642,23 @@ __global__ __launch_bounds__(256) void k_dropout_hidden(DropoutArgs a, const flo
     const char* erow = a.emb_base + (int64_t)key * a.pitch;
     for (int k = lane * 4; k < a.Dp; k += 256) {
         const float4 v4 = load4(erow, k, a.emb_etype);
-        const float4 f4 = *reinterpret_cast<const float4*>(fh + (size_t)u * a.Dp + k);
-        const float v[4] = {v4.x, v4.y, v4.z, v4.w}, f[4] = {f4.x, f4.y, f4.z, f4.w};
+        const float4 f4 = *reinterpret_cast<const float4*>(fh_head + (size_t)u * a.Dp + k);
+        const float4 t4 = *reinterpret_cast<const float4*>(fh_tail + (size_t)u * a.Dp + k);
+        const float v[4] = {v4.x, v4.y, v4.z, v4.w}, f[4] = {f4.x, f4.y, f4.z, f4.w}, ft[4] = {t4.x, t4.y, t4.z, t4.w};
         float oh[4], ot[4];
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
             oh[x] = v[x] + (dropout_keep(a.seed, a.step, 0u, key, (uint32_t)(k + x), a.threshold) ? f[x] * a.scale : 0.f);
-            ot[x] = v[x] + (dropout_keep(a.seed, a.step, 1u, key, (uint32_t)(k + x), a.threshold) ? f[x] * a.scale : 0.f);
+            ot[x] = v[x] + (dropout_keep(a.seed, a.step, 1u, key, (uint32_t)(k + x), a.threshold) ? ft[x] * a.scale : 0.f);
         }
         *reinterpret_cast<float4*>(hidden + (size_t)u * a.Dp + k) = make_float4(oh[0], oh[1], oh[2], oh[3]);
         *reinterpret_cast<float4*>(hidden + (size_t)(a.max_rows + u) * a.Dp + k) = make_float4(ot[0], ot[1], ot[2], ot[3]);
     }
 }
-void launch_dropout_hidden(const DropoutArgs& a, const float* fh, float* hidden, hipStream_t stream) {
-    hipLaunchKernelGGL(k_dropout_hidden, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, fh, hidden);
+void launch_dropout_hidden(const DropoutArgs& a, const float* fh_head, const float* fh_tail, float* hidden,
+                           hipStream_t stream) {
+    hipLaunchKernelGGL(k_dropout_hidden, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, fh_head, fh_tail,
+                       hidden);
 }
 
 // which hidden row contribution c reads: its distinct row, in the tail half for a tail
@@ -3667,11 +3672,15 @@ void launch_role_index(const uint32_t* item_row, int n_head, int n, uint32_t* ou
 }
 
 // The feature part's gradient per distinct row, one wave per row: its head contributions and its
-// tail contributions summed apart (in sorted order), each passed where that use's dropout output
-// is non-zero (the reference's backward tests the output, pag.cpp:610), times 1 / (1 - p).
+// tail contributions summed apart (in sorted order).  With dropout (a.enabled) each sum passes
+// where that use's dropout output is non-zero (the reference's backward tests the output,
+// pag.cpp:610), times 1 / (1 - p).  out_tail null: the two sums go to out_head added up (one
+// feature network); else each to its own array (separate networks).
 __global__ __launch_bounds__(256) void k_role_sums(DropoutArgs a, ContribSrc cs, const uint32_t* __restrict__ seg_start,
                                                    const uint32_t* __restrict__ seg_real,
-                                                   const float* __restrict__ fh, float* __restrict__ out) {
+                                                   const float* __restrict__ fh_head,
+                                                   const float* __restrict__ fh_tail,
+                                                   float* __restrict__ out_head, float* __restrict__ out_tail) {
     const int lane = threadIdx.x & 63;
     const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (u >= (int)a.counts[0]) return;
@@ -3685,22 +3694,33 @@ __global__ __launch_bounds__(256) void k_role_sums(DropoutArgs a, ContribSrc cs,
             const float4 v = load_contrib<true>(cs, c, k, a.Dp);
             if (c < (uint32_t)cs.n_head) gh = f4add(gh, v); else gt = f4add(gt, v);
         }
-        const float4 f4 = *reinterpret_cast<const float4*>(fh + (size_t)u * a.Dp + k);
-        const float f[4] = {f4.x, f4.y, f4.z, f4.w}, h[4] = {gh.x, gh.y, gh.z, gh.w}, t[4] = {gt.x, gt.y, gt.z, gt.w};
-        float o[4];
+        float h[4] = {gh.x, gh.y, gh.z, gh.w}, t[4] = {gt.x, gt.y, gt.z, gt.w};
+        if (a.enabled) {
+            const float4 f4 = *reinterpret_cast<const float4*>(fh_head + (size_t)u * a.Dp + k);
+            const float4 t4 = *reinterpret_cast<const float4*>(fh_tail + (size_t)u * a.Dp + k);
+            const float f[4] = {f4.x, f4.y, f4.z, f4.w}, ft[4] = {t4.x, t4.y, t4.z, t4.w};
 #pragma unroll
-        for (int x = 0; x < 4; ++x) {
-            const bool live = f[x] * a.scale != 0.f;
-            const bool kh = live && dropout_keep(a.seed, a.step, 0u, key, (uint32_t)(k + x), a.threshold);
-            const bool kt = live && dropout_keep(a.seed, a.step, 1u, key, (uint32_t)(k + x), a.threshold);
-            o[x] = a.scale * ((kh ? h[x] : 0.f) + (kt ? t[x] : 0.f));
+            for (int x = 0; x < 4; ++x) {
+                const bool kh = f[x] * a.scale != 0.f && dropout_keep(a.seed, a.step, 0u, key, (uint32_t)(k + x), a.threshold);
+                const bool kt = ft[x] * a.scale != 0.f && dropout_keep(a.seed, a.step, 1u, key, (uint32_t)(k + x), a.threshold);
+                h[x] = kh ? a.scale * h[x] : 0.f;
+                t[x] = kt ? a.scale * t[x] : 0.f;
+            }
         }
-        *reinterpret_cast<float4*>(out + (size_t)u * a.Dp + k) = make_float4(o[0], o[1], o[2], o[3]);
+        if (out_tail) {
+            *reinterpret_cast<float4*>(out_head + (size_t)u * a.Dp + k) = make_float4(h[0], h[1], h[2], h[3]);
+            *reinterpret_cast<float4*>(out_tail + (size_t)u * a.Dp + k) = make_float4(t[0], t[1], t[2], t[3]);
+        } else {
+            *reinterpret_cast<float4*>(out_head + (size_t)u * a.Dp + k) =
+                make_float4(h[0] + t[0], h[1] + t[1], h[2] + t[2], h[3] + t[3]);
+        }
     }
 }
 void launch_role_sums(const DropoutArgs& a, const ContribSrc& cs, const uint32_t* seg_start, const uint32_t* seg_real,
-                      const float* fh, float* out, hipStream_t stream) {
-    hipLaunchKernelGGL(k_role_sums, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, cs, seg_start, seg_real, fh, out);
+                      const float* fh_head, const float* fh_tail, float* out_head, float* out_tail,
+                      hipStream_t stream) {
+    hipLaunchKernelGGL(k_role_sums, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, cs, seg_start, seg_real,
+                       fh_head, fh_tail, out_head, out_tail);
 }
 
 }  // namespace kge

@@ -400,14 +400,18 @@ class Engine:
         self.write_variable("relation_embedding", self.init_scale * relation)
         if m.score_fn == "TransH":   # the hyperplane normals (reference :643-651)
             self.write_variable("relation_normal", self.init_scale * self.random_normal(relation_shape))
-        self.write_variable(
-            "feature_projection",
-            (self.init_scale / np.sqrt(max(m.entity_feature_size, 1)))
-            * self.random_normal((m.entity_feature_size, m.embedding_size)))
-        if m.feature_mlp_size > 0:   # reference :665-686
-            for name, shape in (("mlp_up_projection", (2 * m.embedding_size, m.feature_mlp_size)),
-                                ("mlp_down_projection", (m.feature_mlp_size, m.embedding_size))):
-                self.write_variable(name, (self.init_scale / np.sqrt(shape[0])) * self.random_normal(shape))
+        # one feature network, or one for the heads and one for the tails (reference :652-686)
+        separate = not m.share_feature_networks and m.entity_feature_size > 0
+        for prefix in (("head_", "tail_") if separate else ("",)):
+            self.write_variable(
+                prefix + "feature_projection",
+                (self.init_scale / np.sqrt(max(m.entity_feature_size, 1)))
+                * self.random_normal((m.entity_feature_size, m.embedding_size)))
+            if m.feature_mlp_size > 0:
+                for name, shape in (("mlp_up_projection", (2 * m.embedding_size, m.feature_mlp_size)),
+                                    ("mlp_down_projection", (m.feature_mlp_size, m.embedding_size))):
+                    self.write_variable(prefix + name,
+                                        (self.init_scale / np.sqrt(shape[0])) * self.random_normal(shape))
 
     def initialise_all(self, entity_features: np.ndarray) -> None:
         """Variables, then every table row in rw_batch_size chunks."""

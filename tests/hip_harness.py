@@ -43,7 +43,7 @@ def engine_settings(c, n_step, rw_batch=64, **extra):
         "model.entity_feature_size": c["feature"], "model.feature_mlp_size": int(c.get("feature_mlp_size", 0)),
         "model.feature_dropout": float(c.get("feature_dropout", 0.0)),
         "model.negative_adversarial_scale": float(c["negative_adversarial_scale"]),
-        "model.share_feature_networks": True, "model.gamma": float(c["gamma"]),
+        "model.share_feature_networks": bool(c.get("share_feature_networks", True)), "model.gamma": float(c["gamma"]),
         "model.init_scale": 1.0,
         "data.seed": 5, "data.batch_size": c["batch"], "data.a2a_size": c["a2a"],
         "data.entity_feature_mapping": "full",

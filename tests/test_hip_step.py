@@ -119,6 +119,16 @@ CASES = {
     "feature_dropout_aligned_l2": dict(feature_dropout=0.4, dropout_seed=5, distance_fn="L2", n_shard=2,
                                        batch=128, a2a=64, dim=64, feature=32, n_entity=3000, n_relation=8,
                                        gamma=6.0),
+    # separate feature networks for the head and the tail use (src/poplar_kge.cpp:268-273)
+    "separate_networks": dict(share_feature_networks=False),
+    "separate_networks_mlp_dropout_l2": dict(share_feature_networks=False, feature_mlp_size=6, feature_dropout=0.3,
+                                             dropout_seed=5, distance_fn="L2", loss_fn="softmax",
+                                             softmax_correction_weight=1.0),
+    "separate_networks_shared_distmult": dict(share_feature_networks=False, score_fn="DistMult", distance_fn="MatMul",
+                                              shared_table=True, n_shard=4, batch=8, a2a=4, feature=4, n_entity=60),
+    "separate_networks_mlp_aligned": dict(share_feature_networks=False, feature_mlp_size=48, distance_fn="L2",
+                                          n_shard=2, batch=128, a2a=64, dim=64, feature=32, n_entity=3000,
+                                          n_relation=8, gamma=6.0),
     "aligned_complex_l2_shared": dict(score_fn="ComplEx", distance_fn="L2", n_shard=4, batch=128, a2a=32,
                                       dim=128, feature=0, n_entity=2000, n_relation=8, shared_table=True),
 }

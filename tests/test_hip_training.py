@@ -43,7 +43,8 @@ def _oracle_cfg(settings):
                     a2a=d.a2a_size, score_fn=m.score_fn, distance_fn=m.distance_fn,
                     loss_fn=t.loss.type, gamma=m.gamma, beta_m=t.adam_beta_m, beta_v=t.adam_beta_v,
                     epsilon=t.adam_epsilon, weight_decay=t.weight_decay, loss_scale=t.loss_scale,
-                    storage=storage, feature_mlp_size=m.feature_mlp_size)
+                    storage=storage, feature_mlp_size=m.feature_mlp_size,
+                    share_feature_networks=m.share_feature_networks)
 
 
 def _oracle_state(state):
@@ -165,7 +166,8 @@ def _random_queries(engine, n):
 
 
 @pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "complex", "rotate", "transh", "transh_big",
-                                     "feature_mlp", "feature_dropout", "no_features_big"])
+                                     "feature_mlp", "feature_dropout", "separate_networks_mlp",
+                                     "no_features_big"])
 def test_predict_vs_brute_force(variant):
     """Engine.predict against a float64 brute force over every row of every shard
     (the reference checks shapes, ranges and ordering, tests/python/test_poplar_kge.py:155-175,
@@ -188,6 +190,8 @@ def test_predict_vs_brute_force(variant):
         m.score_fn = "TransH"
     elif variant == "feature_mlp":
         m.feature_mlp_size = 24
+    elif variant == "separate_networks_mlp":
+        m.share_feature_networks, m.feature_mlp_size = False, 16
     elif variant == "feature_dropout":
         m.feature_dropout = 0.4   # training only (entityHidden(..., training=false), src/poplar_kge.cpp:419-422)
     elif variant in ("no_features_big", "transh_big"):
