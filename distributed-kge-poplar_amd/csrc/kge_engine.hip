@@ -433,13 +433,11 @@ void parse_settings(kge_engine& E, const Items& s) {
     if (E.dropout > 0 && E.score_bf16)
         throw std::invalid_argument("'model.feature_dropout' > 0 is not implemented together with "
                                     "'execution.scoring_dtype' = 'bfloat16'");
-    if (E.dropout > 0 && E.reg_on)
-        throw std::invalid_argument("'model.feature_dropout' > 0 is not implemented together with the norm "
-                                    "regularisers (weight > 0)");
+
     E.nets = (!share && E.F > 0) ? 2 : 1;
-    if (E.nets == 2 && (E.reg_on || E.score_bf16))
+    if (E.nets == 2 && E.score_bf16)
         throw std::invalid_argument("'model.share_feature_networks' = false is not implemented together with "
-                                    "the norm regularisers (weight > 0) or 'execution.scoring_dtype' = 'bfloat16'");
+                                    "'execution.scoring_dtype' = 'bfloat16'");
     for (int i = 0; i < 3; ++i)
         if (E.reg_w[i] > 0 && !(E.reg_p[i] > 0))
             throw std::invalid_argument(std::string("'") + reg_names[i] + ".power' must be positive");
@@ -634,7 +632,7 @@ void allocate(kge_engine& E) {
     }
     if (E.reg_on) {
         E.reg_val.alloc(R * E.Dp);
-        if (E.F) E.reg_fh.alloc(R * E.Dp);
+        if (E.F) E.reg_fh.alloc(((E.dropout > 0 || E.nets == 2) ? 2 : 1) * R * E.Dp);
         E.reg_loss_row.alloc(R);
         E.reg_loss_part.alloc(ns * S);
     }
@@ -1082,6 +1080,12 @@ void run_step(kge_engine& E, int i) {
         for (int q = 0; q < 3; ++q) { ra.power[q] = E.reg_p[q]; ra.weight[q] = E.reg_w[q]; }
         ra.loss_scale = E.loss_scale;
         ra.add_val = E.reg_val.p; ra.add_fh = E.reg_fh.p; ra.loss_row = E.reg_loss_row.p;
+        ra.uses = 2.f; ra.accumulate = 0;
+        if (roles) {  // the two entityHidden calls see different rows: one launch for each
+            ra.uses = 1.f;
+            launch_reg_rows(ra, st);
+            ra.hidden = E.hidden.p + rows_n; ra.add_fh = E.reg_fh.p + rows_n; ra.accumulate = 1;
+        }
         launch_reg_rows(ra, st);
         launch_reg_loss(e_uniq, e_counts, E.reg_loss_row.p, (uint32_t)E.n_entity, E.S,
                         E.reg_loss_part.p + (size_t)i * E.S, st);
@@ -1162,7 +1166,8 @@ void run_step(kge_engine& E, int i) {
     auto entity_update = [&]() {
         KernelTimer t(E, K_ADAM_ENT);
         if (roles)  // the feature part's gradient per use: one array (added up) or one per network
-            launch_role_sums(da, esrc, ae.seg_start, ae.seg_real, E.fh.p, E.fh.p + (nets - 1) * rows_n, E.gsum.p,
+            launch_role_sums(da, esrc, ae.seg_start, ae.seg_real, E.fh.p, E.fh.p + (nets - 1) * rows_n,
+                             E.reg_on ? E.reg_fh.p : nullptr, E.reg_on ? E.reg_fh.p + rows_n : nullptr, E.gsum.p,
                              nets == 2 ? E.gsum.p + rows_n : nullptr, st);
         if (!E.mlp) { launch_adam_rows(ae, st); return; }
         if (!roles) {

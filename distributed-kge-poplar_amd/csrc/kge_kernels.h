@@ -243,6 +243,9 @@ struct RegArgs {
     float* add_val;             // [rows, Dp] gradient for the embedding
     float* add_fh;              // [rows, Dp] gradient for the feature product (or null)
     float* loss_row;            // [rows] the row's share of the loss
+    float uses;                 // entityHidden calls this launch stands for: 2 (heads' and tails' calls
+                                // see the same tensors) or 1 (one launch per call, with its hidden rows)
+    int accumulate;             // add to add_val and loss_row instead of overwriting them
 };
 void launch_reg_rows(const RegArgs& a, hipStream_t stream);
 // out[s] = sum of loss_row over the distinct rows owned by shard s (key / rows_per_shard), fixed order
@@ -388,7 +391,7 @@ void launch_role_index(const uint32_t* item_row, int n_head, int n, uint32_t* ou
 // The feature part's gradient of every distinct row [max_rows, Dp] from its contributions:
 // out_head alone (the head and tail uses added up) or one array per use
 void launch_role_sums(const DropoutArgs& a, const ContribSrc& cs, const uint32_t* seg_start, const uint32_t* seg_real,
-                      const float* fh_head, const float* fh_tail, float* out_head, float* out_tail,
-                      hipStream_t stream);
+                      const float* fh_head, const float* fh_tail, const float* add_head, const float* add_tail,
+                      float* out_head, float* out_tail, hipStream_t stream);  // add_*: null, or rows added per use
 
 }  // namespace kge

@@ -2663,11 +2663,11 @@ __global__ __launch_bounds__(256) void k_reg_rows(RegArgs a) {
     for (int q = 0; q < 3; ++q) {
         sum[q] = wave_sum(sum[q]);
         norm[q] = a.weight[q] > 0.f ? powf(sum[q], 1.f / a.power[q]) : 0.f;
-        // d loss / d x_k = seed * (norm / sum) * |x_k^p| / x_k, seed = 2 * mult * weight * loss_scale
-        coef[q] = sum[q] != 0.f ? 2.f * mult * a.weight[q] * a.loss_scale * norm[q] / sum[q] : 0.f;
-        loss += 2.f * mult * a.weight[q] * norm[q];
+        // d loss / d x_k = seed * (norm / sum) * |x_k^p| / x_k, seed = uses * mult * weight * loss_scale
+        coef[q] = sum[q] != 0.f ? a.uses * mult * a.weight[q] * a.loss_scale * norm[q] / sum[q] : 0.f;
+        loss += a.uses * mult * a.weight[q] * norm[q];
     }
-    if (lane == 0) a.loss_row[u] = loss;
+    if (lane == 0) a.loss_row[u] = a.accumulate ? a.loss_row[u] + loss : loss;
     for (int k = lane; k < a.Dp; k += 64) {
         float gv = 0.f, gf = 0.f;
         if (k < a.D) {
@@ -2679,7 +2679,7 @@ __global__ __launch_bounds__(256) void k_reg_rows(RegArgs a) {
                 gv += gh; gf += gh;
             }
         }
-        a.add_val[(size_t)u * a.Dp + k] = gv;
+        a.add_val[(size_t)u * a.Dp + k] = a.accumulate ? a.add_val[(size_t)u * a.Dp + k] + gv : gv;
         if (a.add_fh) a.add_fh[(size_t)u * a.Dp + k] = gf;
     }
 }
@@ -3680,6 +3680,8 @@ __global__ __launch_bounds__(256) void k_role_sums(DropoutArgs a, ContribSrc cs,
                                                    const uint32_t* __restrict__ seg_real,
                                                    const float* __restrict__ fh_head,
                                                    const float* __restrict__ fh_tail,
+                                                   const float* __restrict__ add_head,
+                                                   const float* __restrict__ add_tail,
                                                    float* __restrict__ out_head, float* __restrict__ out_tail) {
     const int lane = threadIdx.x & 63;
     const int u = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -3693,6 +3695,10 @@ __global__ __launch_bounds__(256) void k_role_sums(DropoutArgs a, ContribSrc cs,
             const uint32_t c = cs.sorted_item[pos + j];
             const float4 v = load_contrib<true>(cs, c, k, a.Dp);
             if (c < (uint32_t)cs.n_head) gh = f4add(gh, v); else gt = f4add(gt, v);
+        }
+        if (add_head) {  // the regularisers' share (of the tensors after dropout)
+            gh = f4add(gh, *reinterpret_cast<const float4*>(add_head + (size_t)u * a.Dp + k));
+            gt = f4add(gt, *reinterpret_cast<const float4*>(add_tail + (size_t)u * a.Dp + k));
         }
         float h[4] = {gh.x, gh.y, gh.z, gh.w}, t[4] = {gt.x, gt.y, gt.z, gt.w};
         if (a.enabled) {
@@ -3717,10 +3723,10 @@ __global__ __launch_bounds__(256) void k_role_sums(DropoutArgs a, ContribSrc cs,
     }
 }
 void launch_role_sums(const DropoutArgs& a, const ContribSrc& cs, const uint32_t* seg_start, const uint32_t* seg_real,
-                      const float* fh_head, const float* fh_tail, float* out_head, float* out_tail,
-                      hipStream_t stream) {
+                      const float* fh_head, const float* fh_tail, const float* add_head, const float* add_tail,
+                      float* out_head, float* out_tail, hipStream_t stream) {
     hipLaunchKernelGGL(k_role_sums, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a, cs, seg_start, seg_real,
-                       fh_head, fh_tail, out_head, out_tail);
+                       fh_head, fh_tail, add_head, add_tail, out_head, out_tail);
 }
 
 }  // namespace kge

@@ -554,44 +554,50 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
     free(fhv);
 
     /* 1b. norm regularisers over every gathered slot (:463-465).  entityHidden runs once for
-     * the heads and once for the tails on the same gathered rows and (shared networks) the
-     * same projection, so every term counts twice (:676-678).  The embedding's gradient and
-     * the feature product's gradient differ from here on: greg_val / greg_fh.              */
+     * the heads and once for the tails on the same gathered rows (:676-678), so every term
+     * counts twice; when the two runs differ (separate networks, dropout) each run's feature
+     * part and hidden row are regularised once.  The embedding's gradient (greg_val) and the
+     * feature part's gradient per run (greg_fh_r) differ from here on.                        */
     const int reg_on = c->reg_emb_weight > 0 || c->reg_feat_weight > 0 || c->reg_hid_weight > 0;
-    if (reg_on && n_role == 2) { /* the regularised tensors would differ per use: not restated */
-        free(hidden); free(ghid); free(hidden_t); free(ghid_t);
-        for (int role = 0; role < 2; ++role) { free(fproj_r[role]); free(pre_r[role]); free(live_r[role]); }
-        return 2;
-    }
     REAL* greg_val = reg_on ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
-    REAL* greg_fh = reg_on ? (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL)) : NULL;
+    REAL* greg_fh_r[2] = {NULL, NULL};
     REAL* reg_loss = (REAL*)calloc((size_t)S, sizeof(REAL));
     if (reg_on) {
         REAL* fh = (REAL*)malloc(sizeof(REAL) * (size_t)D);
         REAL* val = (REAL*)malloc(sizeof(REAL) * (size_t)D);
-        for (int64_t s = 0; s < S; ++s)
-            for (int64_t j = 0; j < NR; ++j) {
-                const float* row = table + KEY(s, j) * ROW;
-                const REAL* h = hidden + (s * NR + j) * D;
-                REAL* gv = greg_val + (s * NR + j) * D;
-                REAL* gf = greg_fh + (s * NR + j) * D;
-                for (int64_t k = 0; k < D; ++k) { val[k] = row[k]; fh[k] = h[k] - val[k]; }
-                const REAL seed = 2 * (REAL)c->loss_scale;
-                if (c->reg_emb_weight > 0)
-                    reg_loss[s] += 2 * c->reg_emb_weight *
-                                   lpnorm_row(val, D, c->reg_emb_power, seed * c->reg_emb_weight, gv);
-                if (c->reg_feat_weight > 0)
-                    reg_loss[s] += 2 * c->reg_feat_weight *
-                                   lpnorm_row(fh, D, c->reg_feat_power, seed * c->reg_feat_weight, gf);
-                if (c->reg_hid_weight > 0) {
-                    REAL* tmp = (REAL*)calloc((size_t)D, sizeof(REAL));
-                    reg_loss[s] += 2 * c->reg_hid_weight *
-                                   lpnorm_row(h, D, c->reg_hid_power, seed * c->reg_hid_weight, tmp);
-                    for (int64_t k = 0; k < D; ++k) { gv[k] += tmp[k]; gf[k] += tmp[k]; }
-                    free(tmp);
+        REAL* tmp = (REAL*)malloc(sizeof(REAL) * (size_t)D);
+        const REAL uses = n_role == 2 ? 1 : 2; /* runs of entityHidden one pass of this loop stands for */
+        for (int role = 0; role < n_role; ++role) {
+            greg_fh_r[role] = (REAL*)calloc((size_t)(S * NR * D), sizeof(REAL));
+            for (int64_t s = 0; s < S; ++s)
+                for (int64_t j = 0; j < NR; ++j) {
+                    const float* row = table + KEY(s, j) * ROW;
+                    const REAL* h = (role ? hidden_t : hidden) + (s * NR + j) * D;
+                    REAL* gv = greg_val + (s * NR + j) * D;
+                    REAL* gf = greg_fh_r[role] + (s * NR + j) * D;
+                    for (int64_t k = 0; k < D; ++k) { val[k] = row[k]; fh[k] = h[k] - val[k]; }
+                    const REAL seed = uses * (REAL)c->loss_scale;
+                    if (c->reg_emb_weight > 0) {
+                        for (int64_t k = 0; k < D; ++k) tmp[k] = 0;
+                        reg_loss[s] += uses * c->reg_emb_weight *
+                                       lpnorm_row(val, D, c->reg_emb_power, seed * c->reg_emb_weight, tmp);
+                        for (int64_t k = 0; k < D; ++k) gv[k] += tmp[k];
+                    }
+                    if (c->reg_feat_weight > 0) {
+                        for (int64_t k = 0; k < D; ++k) tmp[k] = 0;
+                        reg_loss[s] += uses * c->reg_feat_weight *
+                                       lpnorm_row(fh, D, c->reg_feat_power, seed * c->reg_feat_weight, tmp);
+                        for (int64_t k = 0; k < D; ++k) gf[k] += tmp[k];
+                    }
+                    if (c->reg_hid_weight > 0) {
+                        for (int64_t k = 0; k < D; ++k) tmp[k] = 0;
+                        reg_loss[s] += uses * c->reg_hid_weight *
+                                       lpnorm_row(h, D, c->reg_hid_power, seed * c->reg_hid_weight, tmp);
+                        for (int64_t k = 0; k < D; ++k) { gv[k] += tmp[k]; gf[k] += tmp[k]; }
+                    }
                 }
-            }
-        free(fh); free(val);
+        }
+        free(fh); free(val); free(tmp);
     }
 
     REAL* grel = (REAL*)calloc((size_t)(NRELT * RD), sizeof(REAL));
@@ -860,11 +866,11 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                 for (int64_t j = 0; j < NR; ++j) {
                     const float* row = table + KEY(s, j) * ROW;
                     const REAL* gh = gsrc + (s * NR + j) * D;
-                    const REAL* gr = greg_fh ? greg_fh + (s * NR + j) * D : NULL;
+                    const REAL* gr = greg_fh_r[role] ? greg_fh_r[role] + (s * NR + j) * D : NULL;
                     for (int64_t k = 0; k < D; ++k) gfh[k] = gh[k] + (gr ? gr[k] : 0);
                     if (drop) { /* grad * (output != 0) / (1 - p) (pag.cpp:606-614) */
                         const uint8_t* lv = live_r[role] + (s * NR + j) * D;
-                        for (int64_t k = 0; k < D; ++k) gfh[k] = lv[k] ? keep_scale * gh[k] : 0;
+                        for (int64_t k = 0; k < D; ++k) gfh[k] = lv[k] ? keep_scale * gfh[k] : 0;
                     }
                     if (M) {
                         /* matMul, max(., 0) (its gradient passes where input == output, i.e. also at
@@ -974,7 +980,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
         }
     }
 #undef KEY
-    free(greg_val); free(greg_fh); free(reg_loss);
+    free(greg_val); free(greg_fh_r[0]); free(greg_fh_r[1]); free(reg_loss);
     free(hidden); free(ghid); free(grel); free(p); free(tl); free(score); free(dist);
     free(dscore); free(dp); free(dtl); free(alpha); free(gproj);
     free(nv); free(dnv); free(nrm); free(gmlp_val);

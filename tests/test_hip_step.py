@@ -129,6 +129,16 @@ CASES = {
     "separate_networks_mlp_aligned": dict(share_feature_networks=False, feature_mlp_size=48, distance_fn="L2",
                                           n_shard=2, batch=128, a2a=64, dim=64, feature=32, n_entity=3000,
                                           n_relation=8, gamma=6.0),
+    # regularisers where the two entityHidden calls differ: each call's tensors once
+    "regularisers_dropout": dict(feature_dropout=0.3, dropout_seed=9, embedding_regularisation=(2.0, 3e-2),
+                                 feature_regularisation=(3.0, 2e-2), hidden_regularisation=(4.0, 1e-2)),
+    "regularisers_separate_mlp": dict(share_feature_networks=False, feature_mlp_size=6,
+                                      feature_regularisation=(3.0, 2e-2), hidden_regularisation=(2.0, 1e-2),
+                                      distance_fn="L2"),
+    "regularisers_separate_dropout_softmax": dict(share_feature_networks=False, feature_dropout=0.25, dropout_seed=2,
+                                                  embedding_regularisation=(3.0, 1e-2),
+                                                  feature_regularisation=(2.0, 3e-2), loss_fn="softmax",
+                                                  softmax_correction_weight=1.0),
     "aligned_complex_l2_shared": dict(score_fn="ComplEx", distance_fn="L2", n_shard=4, batch=128, a2a=32,
                                       dim=128, feature=0, n_entity=2000, n_relation=8, shared_table=True),
 }
@@ -562,11 +572,3 @@ def test_dropout_masks_follow_the_optimiser_step(oracle64):
         oracle64.train_step_loop(make_cfg(**plain), st_plain, np.array([0.1, 0.07], np.float32), K.random_batch(c, 2, rng))
     k = "feature_projection"
     assert K.rel_l2(st_h[k] - st0[k], st_plain[k] - st0[k]) > 0.05
-
-
-def test_dropout_rejected_with_regularisers():
-    import libpoplar_kge
-
-    c = K.cfg_dict(feature_dropout=0.1, feature_regularisation=(3.0, 1e-3))
-    with pytest.raises(ValueError, match="feature_dropout"):
-        libpoplar_kge.Engine(H.engine_settings(c, 1), "")

@@ -331,6 +331,12 @@ STEP_CASES = {
                                              softmax_correction_weight=1.0),
     "separate_networks_shared_distmult": dict(share_feature_networks=False, score_fn="DistMult", distance_fn="MatMul",
                                               shared_table=True, n_shard=4, batch=8, a2a=4, feature=4, n_entity=60),
+    # regularisers where the two entityHidden calls differ: each call's tensors once
+    "regularisers_dropout": dict(feature_dropout=0.3, dropout_seed=9, embedding_regularisation=(2.0, 3e-2),
+                                 feature_regularisation=(3.0, 2e-2), hidden_regularisation=(4.0, 1e-2)),
+    "regularisers_separate_mlp": dict(share_feature_networks=False, feature_mlp_size=6,
+                                      feature_regularisation=(3.0, 2e-2), hidden_regularisation=(2.0, 1e-2),
+                                      distance_fn="L2"),
     # norm regularisers (src/poplar_kge.cpp:430-437, 463-465), the WikiKG preset's among them
     "feature_regularisation_p3": dict(feature_regularisation=(3.0, 1e-2), loss_fn="softmax",
                                       softmax_correction_weight=1.0),

@@ -137,11 +137,12 @@ def step(cfg, state, lr, batch_step):
     # entityHidden call (src/poplar_kge.cpp:463-465, 676-678)
     reg = T.zeros(S, dtype=T.float64)
     value = emb[inverse].reshape(S, -1, D)
-    for key, tensor in (("embedding_regularisation", value), ("feature_regularisation", hidden - value),
-                        ("hidden_regularisation", hidden)):
-        power, weight = cfg.get(key, (3.0, 0.0))
-        if weight > 0:
-            reg = reg + 2 * weight * lpnorm(tensor, float(power)).sum(-1)
+    for hid in (hidden, hidden_tail):  # the two calls (the same tensors unless dropout / separate networks)
+        for key, tensor in (("embedding_regularisation", value), ("feature_regularisation", hid - value),
+                            ("hidden_regularisation", hid)):
+            power, weight = cfg.get(key, (3.0, 0.0))
+            if weight > 0:
+                reg = reg + weight * lpnorm(tensor, float(power)).sum(-1)
 
     heads = hidden[shards[:, None], head]  # [S, B, D]
     tails = hidden_tail[shards[:, None, None], a2a]  # [S(src), S(dst), A, D]
