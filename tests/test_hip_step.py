@@ -96,6 +96,8 @@ CASES = {
                                    negative_adversarial_scale=1.5),
     "transh_aligned": dict(score_fn="TransH", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
                            n_entity=3000, n_relation=8, gamma=6.0),
+    "transh_bf16_embedding": dict(score_fn="TransH", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
+                                  n_entity=3000, n_relation=8, gamma=6.0, storage="bfloat16_embedding"),
     "transh_mid": dict(score_fn="TransH", n_shard=2, batch=70, a2a=45, dim=64, feature=0,
                        n_entity=2000, n_relation=10, gamma=6.0),
     # feature MLP (src/poplar_kge.cpp:453-458): hidden = value + relu([value | feature . W] . Up) . Down
@@ -192,7 +194,7 @@ def test_step_bf16_scoring(oracle64, name):
     assert K.rel_l2(st_f[k] - st0[k], st_o[k] - st0[k]) > 1e-4
 
 
-@pytest.mark.parametrize("name", ["demo", "l2_aligned"])
+@pytest.mark.parametrize("name", ["demo", "l2_aligned", "transh_mlp_dropout"])
 def test_step_float16_table(oracle64, name):
     """execution.dtype = "float16" (src/poplar_kge.cpp:237-246): embedding, both
     moments and features stored as float16, read / write streams in float16.  The
@@ -204,6 +206,9 @@ def test_step_float16_table(oracle64, name):
     kw = dict(storage="float16", feature=6) if name == "demo" else dict(
         storage="float16", distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
         n_entity=3000, n_relation=8, gamma=6.0)
+    if name == "transh_mlp_dropout":  # the later model options on float16 rows
+        kw = dict(storage="float16", feature=6, score_fn="TransH", feature_mlp_size=8, feature_dropout=0.25,
+                  dropout_seed=4, share_feature_networks=False)
     c = K.cfg_dict(**kw)
     rng = np.random.default_rng(13)
     st0 = K.make_state(c, rng)
