@@ -196,6 +196,12 @@ struct kge_engine {
     DevBuf<float> fh;          // the feature part of hidden, before dropout
     DevBuf<uint32_t> role_idx;  // the hidden row of every contribution
     int step_of_first = 0;     // optimiser step of the first step of the running call
+    // {distinct rows, chunks} of the entity plan and of the relation plan for every step of the
+    // resident batch, read back once after the plan phase of a call with enough steps to pay
+    // for the wait: the per-row and per-chunk launches then start no workgroup that only finds
+    // out it has nothing to do (two thirds of them under power-law sampling)
+    std::vector<uint32_t> h_e_counts, h_r_counts;
+    bool counts_known = false;
     int mlp = 0;  // model.feature_mlp_size: hidden = value + relu([value | feature . W] . Up) . Down
     int score_fn, dist_fn, loss_fn;
     bool shared_table;
@@ -1116,6 +1122,7 @@ void run_step(kge_engine& E, int i) {
     rr.chunk_pos = E.r_cpos.p + (size_t)i * E.r_cstride;
     rr.chunk_len = E.r_clen.p + (size_t)i * E.r_cstride;
     rr.counts = r_counts; rr.max_chunks = E.r_cstride; rr.chunk = E.chunk;
+    if (E.counts_known) rr.max_chunks = (int)E.h_r_counts[2 * (size_t)i + 1];
     rr.partial = E.rel_partial.p; rr.Dp = E.Dp;
 
     ReduceArgs re = {};
@@ -1123,6 +1130,7 @@ void run_step(kge_engine& E, int i) {
     re.chunk_pos = E.e_cpos.p + (size_t)i * E.e_cstride;
     re.chunk_len = E.e_clen.p + (size_t)i * E.e_cstride;
     re.counts = e_counts; re.max_chunks = E.e_cstride; re.chunk = E.chunk;
+    if (E.counts_known) re.max_chunks = (int)E.h_e_counts[2 * (size_t)i + 1];
     re.partial = E.partial.p; re.Dp = E.Dp;
     { KernelTimer t(E, K_REDUCE_ENT); launch_reduce_chunks2(re, rr, st); }
 
@@ -1150,7 +1158,7 @@ void run_step(kge_engine& E, int i) {
     ae.seg_start = E.e_seg.p + (size_t)i * (E.e_ustride + 1);
     ae.seg_real = E.e_real.p + (size_t)i * E.e_ustride;
     ae.chunk_off = E.e_coff.p + (size_t)i * (E.e_ustride + 1);
-    ae.counts = e_counts; ae.max_rows = (int)R;
+    ae.counts = e_counts; ae.max_rows = E.counts_known ? (int)E.h_e_counts[2 * (size_t)i] : (int)R;
     ae.partial = E.partial.p;
     // (with dropout the feature part's gradient is formed per role by launch_role_sums)
     ae.grad_out = (E.F && !roles) ? E.gsum.p : nullptr;
@@ -1199,8 +1207,10 @@ void run_step(kge_engine& E, int i) {
         KernelTimer t(E, K_ADAM_REL);
         launch_adam_rows(ar, st);
     } else {
+        // the relation rows first: they are few and slow (a dozen contributions each, two rounds
+        // of loads), and at the end of the grid they ran on alone after the entity rows were done
         KernelTimer t(E, K_ADAM_ENT);
-        launch_adam_rows2(ae, ar, st);
+        launch_adam_rows2(ar, ae, st);
     }
 
     // dense Adam on rows [0, rows) of a parameter of row pitch `width`; shard s owns rows
@@ -1308,6 +1318,16 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     HIP_CHECK(hipEventRecord(E.ev[1], st));
     run_plan(E, s0, sn);
     E.step_of_first = (int)E.step - s0;  // step i of the batch is optimiser step E.step + (i - s0)
+    E.counts_known = sn >= 8;
+    if (E.counts_known) {
+        E.h_e_counts.resize(2 * (size_t)E.n_step);
+        E.h_r_counts.resize(2 * (size_t)E.n_step);
+        HIP_CHECK(hipMemcpyAsync(E.h_e_counts.data() + 2 * s0, E.e_counts.p + 2 * s0, 2 * (size_t)sn * 4,
+                                 hipMemcpyDeviceToHost, st));
+        HIP_CHECK(hipMemcpyAsync(E.h_r_counts.data() + 2 * s0, E.r_counts.p + 2 * s0, 2 * (size_t)sn * 4,
+                                 hipMemcpyDeviceToHost, st));
+        HIP_CHECK(hipStreamSynchronize(st));
+    }
     HIP_CHECK(hipEventRecord(E.ev[2], st));
     for (int i = s0; i < s0 + sn; ++i) run_step(E, i);
     launch_loss_finalize(E.loss_part.p + (size_t)s0 * E.S * E.n_part, sn, E.S, E.n_part, 1.f / (float)sn,

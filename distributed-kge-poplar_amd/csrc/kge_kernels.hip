@@ -2459,8 +2459,10 @@ __global__ __launch_bounds__(NW * 64) void k_reduce_chunks(ReduceArgs a0, Reduce
     const bool second = (int)blockIdx.x >= a0.max_chunks;
     const ReduceArgs& a = second ? a1 : a0;
     const int q = second ? blockIdx.x - a0.max_chunks : blockIdx.x;
-    if (q >= (int)a.counts[1]) return;
+    // fetched together with the chunk count (entries past it are stale but inside the arrays):
+    // one round trip less in front of every chunk
     const uint32_t pos = a.chunk_pos[q], len = a.chunk_len[q];
+    if (q >= (int)a.counts[1]) return;
     const int Dp = a.Dp;
     if (Dp & 3) {  // unaligned rows (stand-alone scatter-add on arbitrary widths): wave 0 only
         if (wave == 0)
@@ -2476,7 +2478,9 @@ __global__ __launch_bounds__(NW * 64) void k_reduce_chunks(ReduceArgs a0, Reduce
     const uint32_t w0 = min(len, wave * share), w1 = min(len, w0 + share);
     for (int k0 = 0; k0 < Dp; k0 += 256) {
         const int k = k0 + lane * 4;
-        float4 acc = sum_contribs<8, XF>(a.src, pos + w0, w1 - w0, k, Dp, lane, k < Dp);
+        // sixteen loads in flight: a wave's share of a 64-item chunk in one round (same order of
+        // additions as any other round size)
+        float4 acc = sum_contribs<16, XF>(a.src, pos + w0, w1 - w0, k, Dp, lane, k < Dp);
         if (wave > 0) *reinterpret_cast<float4*>(&part[wave - 1][lane * 4]) = acc;
         __syncthreads();
         if (wave == 0 && k < Dp) {
@@ -2535,15 +2539,18 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
     const bool second = (int)blockIdx.x >= blocks0;
     const AdamArgs& a = second ? a1 : a0;
     const int u = (second ? blockIdx.x - blocks0 : blockIdx.x) * 4 + (threadIdx.x >> 6);
-    if (u >= (int)a.counts[0]) return;
-    const uint32_t key = a.uniq_key[u];
-    const float alpha = a.alpha[a.rows_per_alpha ? key / a.rows_per_alpha : 0u];
-    const int Dp = a.Dp;
+    // the row's plan entries are fetched together with the row count (entries past it are stale
+    // but inside the arrays): one round trip less in front of every row
+    const int uc = min(u, a.max_rows - 1);
+    const uint32_t key = a.uniq_key[uc];
     uint32_t q0 = 0, q1 = 0, pos = 0, n_real = 0;
     if (!a.grad_direct) {
-        q0 = a.chunk_off[u]; q1 = a.chunk_off[u + 1];
-        pos = a.seg_start[u]; n_real = a.seg_real[u];
+        q0 = a.chunk_off[uc]; q1 = a.chunk_off[uc + 1];
+        pos = a.seg_start[uc]; n_real = a.seg_real[uc];
     }
+    if (u >= (int)a.counts[0]) return;
+    const float alpha = a.alpha[a.rows_per_alpha ? key / a.rows_per_alpha : 0u];
+    const int Dp = a.Dp;
     char* prow = a.p_base + (int64_t)key * a.pitch;
     char* mrow = a.m_base + (int64_t)key * a.pitch;
     char* vrow = a.v_base + (int64_t)key * a.pitch;
