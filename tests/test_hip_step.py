@@ -141,6 +141,12 @@ CASES = {
                                                   embedding_regularisation=(3.0, 1e-2),
                                                   feature_regularisation=(2.0, 3e-2), loss_fn="softmax",
                                                   softmax_correction_weight=1.0),
+    # 8192 contributions and more: the gather's two-rows-per-wave kernel, multiply mode and rows
+    # through the feature path's index; an odd row count
+    "distmult_many_rows_feat": dict(score_fn="DistMult", distance_fn="MatMul", n_shard=32, batch=128, a2a=4, dim=32,
+                                    feature=8, n_entity=3000, n_relation=8, shared_table=True),
+    "l1_many_rows_odd": dict(distance_fn="L1", n_shard=31, batch=129, a2a=5, dim=20, feature=0, n_entity=3000,
+                             n_relation=8, shared_table=True, gamma=4.0),
     "aligned_complex_l2_shared": dict(score_fn="ComplEx", distance_fn="L2", n_shard=4, batch=128, a2a=32,
                                       dim=128, feature=0, n_entity=2000, n_relation=8, shared_table=True),
 }
