@@ -200,8 +200,9 @@ struct kge_engine {
     // resident batch, read back once after the plan phase of a call with enough steps to pay
     // for the wait: the per-row and per-chunk launches then start no workgroup that only finds
     // out it has nothing to do (two thirds of them under power-law sampling)
-    std::vector<uint32_t> h_e_counts, h_r_counts;
+    std::vector<uint32_t> h_e_counts, h_r_counts, h_e_hot, h_r_hot;
     bool counts_known = false;
+    int plan_readback_steps = 8;  // additive setting execution.plan_readback_steps: calls of at least this many steps
     int mlp = 0;  // model.feature_mlp_size: hidden = value + relu([value | feature . W] . Up) . Down
     int score_fn, dist_fn, loss_fn;
     bool shared_table;
@@ -239,6 +240,7 @@ struct kge_engine {
     DevBuf<uint32_t> ckey, crel, clabel, ek_a, ev_a, ek_b, ev_b, rk_a, rv_a, rk_b, rv_b, hist;
     DevBuf<uint32_t> e_uniq, e_seg, e_coff, e_cpos, e_clen, e_counts, e_item_row, e_real;
     DevBuf<uint32_t> r_uniq, r_seg, r_coff, r_cpos, r_clen, r_counts, r_real;
+    DevBuf<uint32_t> e_hot, e_hot_count, r_hot, r_hot_count;  // the rows with chunks, per step
     DevBuf<uint32_t> nearflag;
     int e_ustride, e_cstride, r_ustride, r_cstride, n_rel_items;
     uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
@@ -285,8 +287,9 @@ struct kge_engine {
 
 namespace {
 
-// DistMult, ComplEx and RotatE form a row's gradient contributions from rows of the other
-// table when they are summed (TransE's and TransH's are materialised before that)
+// the most contributions a row may have for the update's launch to sum it (launch_adam_rows_hot2)
+constexpr uint32_t kHotInUpdateMax = 4096;
+
 // a step-size modifier of a feature network's parameter, by the variable's name
 // (src/poplar_kge.cpp:321-327): [head_ | tail_]{feature_projection, mlp_up_projection, mlp_down_projection}
 bool feature_modifier(kge_engine& E, const std::string& key, float value) {
@@ -304,6 +307,8 @@ bool feature_modifier(kge_engine& E, const std::string& key, float value) {
     return true;
 }
 
+// DistMult, ComplEx and RotatE form a row's gradient contributions from rows of the other
+// table when they are summed (TransE's and TransH's are materialised before that)
 bool contributions_read_tables(const kge_engine& E) {
     return E.score_fn == SCORE_DISTMULT || E.score_fn == SCORE_COMPLEX || E.score_fn == SCORE_ROTATE;
 }
@@ -377,6 +382,7 @@ void parse_settings(kge_engine& E, const Items& s) {
                                     "'execution.shared_table' a row's loss share has no owning shard");
     E.profile_kernels = s.find("execution.profile_kernels") ? s.boolean("execution.profile_kernels") : false;
     if (s.find("execution.reduce_chunk")) E.chunk = (int)s.uint("execution.reduce_chunk");
+    if (s.find("execution.plan_readback_steps")) E.plan_readback_steps = std::max(1, (int)s.uint("execution.plan_readback_steps"));
     if (s.find("execution.scoring")) {
         const std::string v = s.str("execution.scoring");
         if (v == "mfma") E.use_mfma = 1;
@@ -561,6 +567,8 @@ void allocate(kge_engine& E) {
     E.e_cpos.alloc(ns * E.e_cstride);
     E.e_clen.alloc(ns * E.e_cstride);
     E.e_counts.alloc(ns * 2);
+    E.e_hot.alloc(ns * E.e_cstride);
+    E.e_hot_count.alloc(ns * 2);
     if (E.F) E.e_item_row.alloc(ns * R);
     E.r_ustride = E.n_rel_rows;
     E.r_cstride = (int)(SB * E.rel_copies / std::min(E.chunk, E.direct_max + 1) + 2);
@@ -571,6 +579,8 @@ void allocate(kge_engine& E) {
     E.r_cpos.alloc(ns * E.r_cstride);
     E.r_clen.alloc(ns * E.r_cstride);
     E.r_counts.alloc(ns * 2);
+    E.r_hot.alloc(ns * E.r_cstride);
+    E.r_hot_count.alloc(ns * 2);
 
     E.coef.alloc(SB * E.T);
     const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f && !E.score_bf16;
@@ -878,6 +888,7 @@ void run_plan(kge_engine& E, int s0, int sn) {
     ep.counts = E.e_counts.p + 2 * (size_t)s0;
     ep.item_row = E.F ? E.e_item_row.p + s0 * R : nullptr;
     ep.seg_real = E.e_real.p + (size_t)s0 * ep.u_stride;
+    ep.hot_rows = E.e_hot.p + (size_t)s0 * ep.c_stride; ep.hot_count = E.e_hot_count.p + 2 * s0;
     launch_find_segments(ek + s0 * N, E.e_sorted_vals + s0 * N, (int)N, (int)R, E.chunk, E.direct_max, sn, ep, st);
 
     which = launch_radix_sort(E.rk_a.p + s0 * NRI, E.rv_a.p + s0 * NRI, E.rk_b.p + s0 * NRI,
@@ -894,6 +905,7 @@ void run_plan(kge_engine& E, int s0, int sn) {
     rp.counts = E.r_counts.p + 2 * (size_t)s0;
     rp.item_row = nullptr;
     rp.seg_real = E.r_real.p + (size_t)s0 * rp.u_stride;
+    rp.hot_rows = E.r_hot.p + (size_t)s0 * rp.c_stride; rp.hot_count = E.r_hot_count.p + 2 * s0;
     launch_find_segments(rk + s0 * NRI, E.r_sorted_vals + s0 * NRI, (int)NRI, (int)SB * E.rel_copies, E.chunk, E.direct_max, sn, rp, st);
     HIP_CHECK(hipGetLastError());
 }
@@ -1132,7 +1144,16 @@ void run_step(kge_engine& E, int i) {
     re.counts = e_counts; re.max_chunks = E.e_cstride; re.chunk = E.chunk;
     if (E.counts_known) re.max_chunks = (int)E.h_e_counts[2 * (size_t)i + 1];
     re.partial = E.partial.p; re.Dp = E.Dp;
-    { KernelTimer t(E, K_REDUCE_ENT); launch_reduce_chunks2(re, rr, st); }
+    // Contributions used as stored, nothing between the sums and the updates, and no row with
+    // more contributions than a handful of workgroups sum in the time the other rows take (known
+    // from the plan's read-back): the rows with chunks are summed and updated by workgroups of
+    // their own inside the update's launch, and the first-level reduction (a launch whose time
+    // is all latency) is not needed.  A row of 5 600 contributions (the 22.8M-row workload's
+    // hottest) takes its eight workgroups longer than the whole update takes otherwise; one of
+    // 2 200 (the 1M-row workload's) fits under it.
+    const bool hot_in_update = !contributions_read_tables(E) && !E.mlp && !roles && E.counts_known &&
+                               std::max(E.h_e_hot[2 * (size_t)i + 1], E.h_r_hot[2 * (size_t)i + 1]) <= kHotInUpdateMax;
+    if (!hot_in_update) { KernelTimer t(E, K_REDUCE_ENT); launch_reduce_chunks2(re, rr, st); }
 
     // With DistMult / ComplEx the relation rows' direct contributions read entity rows and
     // the entity rows' read relation rows, so neither table may be updated before
@@ -1206,6 +1227,14 @@ void run_step(kge_engine& E, int i) {
         entity_update();
         KernelTimer t(E, K_ADAM_REL);
         launch_adam_rows(ar, st);
+    } else if (hot_in_update) {
+        KernelTimer t(E, K_ADAM_ENT);
+        HotRows he, hr;
+        he.hot_rows = E.e_hot.p + (size_t)i * E.e_cstride; he.hot_count = E.e_hot_count.p + 2 * i;
+        he.max_hot = (int)E.h_e_hot[2 * (size_t)i];
+        hr.hot_rows = E.r_hot.p + (size_t)i * E.r_cstride; hr.hot_count = E.r_hot_count.p + 2 * i;
+        hr.max_hot = (int)E.h_r_hot[2 * (size_t)i];
+        launch_adam_rows_hot2(ar, hr, ae, he, st);
     } else {
         // the relation rows first: they are few and slow (a dozen contributions each, two rounds
         // of loads), and at the end of the grid they ran on alone after the entity rows were done
@@ -1318,13 +1347,19 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     HIP_CHECK(hipEventRecord(E.ev[1], st));
     run_plan(E, s0, sn);
     E.step_of_first = (int)E.step - s0;  // step i of the batch is optimiser step E.step + (i - s0)
-    E.counts_known = sn >= 8;
+    E.counts_known = sn >= E.plan_readback_steps;
     if (E.counts_known) {
         E.h_e_counts.resize(2 * (size_t)E.n_step);
         E.h_r_counts.resize(2 * (size_t)E.n_step);
         HIP_CHECK(hipMemcpyAsync(E.h_e_counts.data() + 2 * s0, E.e_counts.p + 2 * s0, 2 * (size_t)sn * 4,
                                  hipMemcpyDeviceToHost, st));
         HIP_CHECK(hipMemcpyAsync(E.h_r_counts.data() + 2 * s0, E.r_counts.p + 2 * s0, 2 * (size_t)sn * 4,
+                                 hipMemcpyDeviceToHost, st));
+        E.h_e_hot.resize(2 * (size_t)E.n_step);
+        E.h_r_hot.resize(2 * (size_t)E.n_step);
+        HIP_CHECK(hipMemcpyAsync(E.h_e_hot.data() + 2 * s0, E.e_hot_count.p + 2 * s0, 2 * (size_t)sn * 4,
+                                 hipMemcpyDeviceToHost, st));
+        HIP_CHECK(hipMemcpyAsync(E.h_r_hot.data() + 2 * s0, E.r_hot_count.p + 2 * s0, 2 * (size_t)sn * 4,
                                  hipMemcpyDeviceToHost, st));
         HIP_CHECK(hipStreamSynchronize(st));
     }
@@ -1750,7 +1785,7 @@ int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* i
     sp.item_row = nullptr; sp.u_stride = (int)rows; sp.c_stride = (int)L.cmax;
     const uint32_t* sk = which ? u32(L.off_keys_b) : u32(L.off_keys_a);
     const uint32_t* sv = which ? u32(L.off_vals_b) : u32(L.off_vals_a);
-    sp.seg_real = nullptr;
+    sp.seg_real = nullptr; sp.hot_rows = nullptr; sp.hot_count = nullptr;
     launch_find_segments(sk, sv, (int)L.N, (int)n, 32, 0, 1, sp, st);
     ReduceArgs ra = {};
     ra.src.sorted_item = sv; ra.src.grad = grad_out; ra.src.transform = 0;

@@ -76,6 +76,11 @@ struct SegPlan {
     uint32_t* counts;     // [n_seg, 2]             {distinct rows, chunks}
     uint32_t* item_row;   // [n_seg, n_real] or null: distinct-row index of each real item
     uint32_t* seg_real;   // [n_seg, u_stride] or null: real items of each row
+    // or null: the rows that get chunks (more than direct_max real items), as distinct-row
+    // indices in ascending order [n_seg, c_stride], and [n_seg, 2] {how many, real items of the
+    // row with the most} (needs seg_real)
+    uint32_t* hot_rows;
+    uint32_t* hot_count;
     int u_stride, c_stride;
 };
 
@@ -221,6 +226,17 @@ struct AdamArgs {
 };
 void launch_adam_rows(const AdamArgs& a, hipStream_t stream);
 void launch_adam_rows2(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream);  // one launch
+// The same two updates without the first-level reduction (launch_reduce_chunks) before them:
+// a row with chunks ("hot", SegPlan::hot_rows) is summed and updated by workgroups of its own,
+// one per 32 columns, the other rows by one wave each as in launch_adam_rows.  Contributions
+// as stored (ContribSrc::transform 0) only.  max_hot: upper bound of *hot_count.
+struct HotRows {
+    const uint32_t* hot_rows;
+    const uint32_t* hot_count;
+    int max_hot;
+};
+void launch_adam_rows_hot2(const AdamArgs& a0, const HotRows& h0, const AdamArgs& a1, const HotRows& h1,
+                           hipStream_t stream);
 
 // loss[s] = sum over steps and parts of loss_part / n_step, in a fixed order; `extra`
 // (or null) holds one more term per (step, shard).

@@ -409,6 +409,26 @@ __global__ __launch_bounds__(1024) void k_find_segments(const uint32_t* __restri
         plan.counts[2 * seg] = U;
         plan.counts[2 * seg + 1] = NC;
     }
+    if (plan.hot_rows) {  // the rows with chunks, in ascending order
+        uint32_t nh = 0;
+        for (int u = ulo; u < uhi; ++u) nh += seg_real[u] > (uint32_t)direct_max ? 1u : 0u;
+        __syncthreads();  // lds is reused
+        uint32_t H;
+        uint32_t hb = block_scan_1024(nh, lds, &H);
+        uint32_t* hot = plan.hot_rows + (size_t)seg * plan.c_stride;
+        uint32_t biggest = 0;
+        for (int u = ulo; u < uhi; ++u) {
+            biggest = max(biggest, seg_real[u]);
+            if (seg_real[u] > (uint32_t)direct_max) hot[hb++] = (uint32_t)u;
+        }
+        // {rows with chunks, real items of the biggest row}
+        __syncthreads();
+        if (tid == 0) lds[0] = 0u;
+        __syncthreads();
+        atomicMax(&lds[0], biggest);
+        __syncthreads();
+        if (tid == 0) { plan.hot_count[2 * seg] = H; plan.hot_count[2 * seg + 1] = lds[0]; }
+    }
 }
 
 void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sorted, int N,
@@ -2644,6 +2664,148 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
             store4(vrow, k, a.m_etype, v);
         }
     }
+}
+
+// One launch for both tables without a first-level reduction before it.
+//   blocks [0, NS0 * max_hot0), [.., + NS1 * max_hot1): hot rows, one workgroup per (row, 16 columns).
+//     Lane = (slot, column group): sixteen contributions per load instruction (64 bytes of each),
+//     eight such loads in flight; a lane adds
+//     its slot's contributions in sorted order, the sixteen slots meet by butterfly shuffles (both
+//     operand orders give the same float), the four waves' sums in LDS in wave order; four lanes
+//     of wave 0 then update the 16 columns.
+//   the remaining blocks: every other row, one wave per row, as k_adam_rows.
+// columns per hot-row workgroup: 32 (128 bytes of every contribution per load; 16 and 8 columns
+// measured slower: the same rows are then fetched by two and four times as many workgroups)
+constexpr int kHotColumns = 32;
+template <bool MF32>
+__global__ __launch_bounds__(256) void k_adam_rows_hot(AdamArgs a0, HotRows h0, AdamArgs a1, HotRows h1) {
+    constexpr int HC = kHotColumns, HS = 64 / (HC / 4);  // columns per workgroup, slots per wave
+    __shared__ __attribute__((aligned(16))) float part[3][HC];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ns0 = (a0.Dp + HC - 1) / HC, ns1 = (a1.Dp + HC - 1) / HC;
+    const int hot0 = ns0 * h0.max_hot, hot1 = ns1 * h1.max_hot;
+    int b = blockIdx.x;
+    if (b < hot0 + hot1) {
+        const bool second = b >= hot0;
+        const AdamArgs& a = second ? a1 : a0;
+        const HotRows& h = second ? h1 : h0;
+        if (second) b -= hot0;
+        const int ns = second ? ns1 : ns0, hb = b / ns, cb = b - hb * ns;
+        if (hb >= (int)h.hot_count[0]) return;
+        const int u = (int)h.hot_rows[hb], Dp = a.Dp;
+        const uint32_t key = a.uniq_key[u], pos = a.seg_start[u], n = a.seg_real[u];
+        const float alpha = a.alpha[a.rows_per_alpha ? key / a.rows_per_alpha : 0u];
+        const int cg = lane & (HC / 4 - 1), slot = lane / (HC / 4), col = cb * HC + cg * 4;
+        const bool active = col < Dp;
+        // this wave's quarter of the contributions, in whole groups of HS
+        const uint32_t groups = (n + HS - 1) / HS, gshare = (groups + 3) / 4;
+        const uint32_t w0 = min(n, wave * gshare * HS), w1 = min(n, w0 + gshare * HS);
+        const uint32_t* __restrict__ items = a.src.sorted_item + pos;
+        const float* __restrict__ grad = a.src.grad;
+        float4 acc = make_float4(0, 0, 0, 0);
+        for (uint32_t j = w0; j < w1; j += 8 * HS) {
+            uint32_t c[8];
+            float4 v[8];
+#pragma unroll
+            for (int x = 0; x < 8; ++x) {
+                const uint32_t idx = j + x * HS + slot;
+                c[x] = idx < w1 ? items[idx] : 0xffffffffu;
+            }
+#pragma unroll
+            for (int x = 0; x < 8; ++x)
+                v[x] = (active && c[x] != 0xffffffffu) ? *reinterpret_cast<const float4*>(grad + (size_t)c[x] * Dp + col)
+                                                      : make_float4(0, 0, 0, 0);
+#pragma unroll
+            for (int x = 0; x < 8; ++x) acc = f4add(acc, v[x]);
+        }
+#pragma unroll
+        for (int off = HC / 4; off < 64; off <<= 1) {
+            acc.x += __shfl_xor(acc.x, off, 64); acc.y += __shfl_xor(acc.y, off, 64);
+            acc.z += __shfl_xor(acc.z, off, 64); acc.w += __shfl_xor(acc.w, off, 64);
+        }
+        if (wave > 0 && slot == 0) *reinterpret_cast<float4*>(&part[wave - 1][cg * 4]) = acc;
+        __syncthreads();
+        if (wave != 0 || slot != 0 || !active) return;
+        float4 g = acc;
+#pragma unroll
+        for (int w = 0; w < 3; ++w) g = f4add(g, *reinterpret_cast<const float4*>(&part[w][cg * 4]));
+        char* prow = a.p_base + (int64_t)key * a.pitch;
+        char* mrow = a.m_base + (int64_t)key * a.pitch;
+        char* vrow = a.v_base + (int64_t)key * a.pitch;
+        if (a.grad_out) {
+            float4 go = g;
+            if (a.grad_out_add) go = f4add(go, *reinterpret_cast<const float4*>(a.grad_out_add + (size_t)u * Dp + col));
+            *reinterpret_cast<float4*>(a.grad_out + (size_t)u * Dp + col) = go;
+        }
+        if (a.no_update) return;
+        if (a.grad_add) g = f4add(g, *reinterpret_cast<const float4*>(a.grad_add + (size_t)u * Dp + col));
+        float4 p = load4(prow, col, a.p_etype);
+        float4 m = load4(mrow, col, a.m_etype), v = load4(vrow, col, a.m_etype);
+        adam4(p, m, v, g, a, alpha);
+        store4(prow, col, a.p_etype, p);
+        store4(mrow, col, a.m_etype, m);
+        store4(vrow, col, a.m_etype, v);
+        return;
+    }
+    b -= hot0 + hot1;
+    const int blocks0 = (a0.max_rows + 3) / 4;
+    const bool second = b >= blocks0;
+    const AdamArgs& a = second ? a1 : a0;
+    const int u = (second ? b - blocks0 : b) * 4 + wave;
+    const int uc = min(u, a.max_rows - 1);
+    const uint32_t key = a.uniq_key[uc];
+    const uint32_t q0 = a.chunk_off[uc], q1 = a.chunk_off[uc + 1];
+    const uint32_t pos = a.seg_start[uc], n_real = a.seg_real[uc];
+    if (u >= (int)a.counts[0] || q1 > q0) return;  // a row with chunks belongs to the hot blocks
+    const float alpha = a.alpha[a.rows_per_alpha ? key / a.rows_per_alpha : 0u];
+    const int Dp = a.Dp;
+    char* prow = a.p_base + (int64_t)key * a.pitch;
+    char* mrow = a.m_base + (int64_t)key * a.pitch;
+    char* vrow = a.v_base + (int64_t)key * a.pitch;
+    for (int k0 = 0; k0 < Dp; k0 += 256) {
+        const int k = k0 + lane * 4;
+        const bool active = k < Dp;
+        float4 g = make_float4(0, 0, 0, 0);
+        if (n_real)  // wave-uniform: all lanes take part in the shuffles
+            g = sum_contribs<8, false>(a.src, pos, n_real, k, Dp, lane, active);
+        if (!active) continue;
+        float4 p = load4(prow, k, a.p_etype);
+        float4 m, v;
+        if constexpr (MF32) {
+            m = *reinterpret_cast<const float4*>(mrow + (size_t)k * 4);
+            v = *reinterpret_cast<const float4*>(vrow + (size_t)k * 4);
+        } else {
+            m = load4(mrow, k, a.m_etype);
+            v = load4(vrow, k, a.m_etype);
+        }
+        if (a.grad_out) {
+            float4 go = g;
+            if (a.grad_out_add) go = f4add(go, *reinterpret_cast<const float4*>(a.grad_out_add + (size_t)u * Dp + k));
+            *reinterpret_cast<float4*>(a.grad_out + (size_t)u * Dp + k) = go;
+        }
+        if (a.no_update) continue;
+        if (a.grad_add) g = f4add(g, *reinterpret_cast<const float4*>(a.grad_add + (size_t)u * Dp + k));
+        adam4(p, m, v, g, a, alpha);
+        store4(prow, k, a.p_etype, p);
+        if constexpr (MF32) {
+            *reinterpret_cast<float4*>(mrow + (size_t)k * 4) = m;
+            *reinterpret_cast<float4*>(vrow + (size_t)k * 4) = v;
+        } else {
+            store4(mrow, k, a.m_etype, m);
+            store4(vrow, k, a.m_etype, v);
+        }
+    }
+}
+
+void launch_adam_rows_hot2(const AdamArgs& a0, const HotRows& h0, const AdamArgs& a1, const HotRows& h1,
+                           hipStream_t stream) {
+    const int hot = ((a0.Dp + kHotColumns - 1) / kHotColumns) * h0.max_hot +
+                    ((a1.Dp + kHotColumns - 1) / kHotColumns) * h1.max_hot;
+    const dim3 grid(hot + (a0.max_rows + 3) / 4 + (a1.max_rows + 3) / 4);
+    if (grid.x == 0) return;
+    const bool f32 = (a0.max_rows == 0 || a0.m_etype == ET_F32) && (a1.max_rows == 0 || a1.m_etype == ET_F32);
+    if (f32) hipLaunchKernelGGL((k_adam_rows_hot<true>), grid, dim3(256), 0, stream, a0, h0, a1, h1);
+    else hipLaunchKernelGGL((k_adam_rows_hot<false>), grid, dim3(256), 0, stream, a0, h0, a1, h1);
 }
 
 static void launch_adam_kernel(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream) {

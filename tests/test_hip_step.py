@@ -472,6 +472,36 @@ def test_step_raw_zipf_duplicates(oracle64):
              batch_fn=K.raw_batch, n_loop=2)
 
 
+READBACK = {"execution.plan_readback_steps": 1}
+
+
+@pytest.mark.parametrize("name", ["l2_logsigmoid", "shared_l2", "paired_l1_t256", "transh_shared", "bf16_embedding_l2",
+                                  "l2_feat", "mid_l1", "feature_mlp", "distmult_logsigmoid"])
+def test_step_vs_oracle_plan_readback(oracle64, name):
+    # the plan's counts read back after the plan phase (what calls of eight steps and more do):
+    # launches sized to the step's distinct rows and chunks, and, where the contributions are used
+    # as stored, the rows with chunks summed inside the update's launch
+    run_case(oracle64, CASES[name], **READBACK)
+
+
+@pytest.mark.parametrize("shape", [dict(n_shard=8, batch=64, a2a=8, n_entity=500), dict(n_shard=16, batch=128, a2a=8, n_entity=40),
+                                   dict(n_shard=4, batch=256, a2a=64, n_entity=3, dim=40)])
+def test_step_raw_zipf_duplicates_plan_readback(oracle64, shape):
+    # hot rows of a few dozen up to 2 000 contributions summed by the update's own workgroups
+    # (n_entity = 3: two real rows share every contribution)
+    kw = dict(distance_fn="L2", shared_table=True, dim=64, feature=0, n_relation=20, gamma=5.0)
+    kw.update(shape)
+    run_case(oracle64, kw, batch_fn=K.raw_batch, n_loop=2, **READBACK)
+
+
+def test_step_hottest_row_above_the_in_launch_limit(oracle64):
+    # 4 096 contributions for two rows: past the limit, the two-level reduction runs as without
+    # the read-back
+    kw = dict(distance_fn="L2", shared_table=True, n_shard=8, batch=256, a2a=32, n_entity=3, dim=32, feature=0,
+              n_relation=4, gamma=5.0)
+    run_case(oracle64, kw, n_step=2, batch_fn=K.raw_batch, **READBACK)
+
+
 def test_step_cold_start(oracle64):
     # zero moments and step 0: the first Adam step is sign-like and the most sensitive
     run_case(oracle64, dict(distance_fn="L2", feature=0, gamma=4.0), warm=False)
@@ -485,15 +515,16 @@ def test_step_deterministic():
     rng = np.random.default_rng(5)
     st0 = K.make_state(c, rng)
     batch = K.raw_batch(c, 2, rng)
-    outs = []
-    for _ in range(2):
-        engine = libpoplar_kge.Engine(H.engine_settings(c, 2), "")
-        H.load_state(engine, c, st0)
-        loss = H.train(engine, c, 0.05, batch)
-        outs.append((loss, H.read_state(engine, c)))
-    np.testing.assert_array_equal(outs[0][0], outs[1][0])
-    for k in ("entity_data", "relation_embedding"):
-        np.testing.assert_array_equal(outs[0][1][k], outs[1][1][k])
+    for extra in ({}, READBACK):  # the two-level reduction; hot rows inside the update's launch
+        outs = []
+        for _ in range(2):
+            engine = libpoplar_kge.Engine(H.engine_settings(c, 2, **extra), "")
+            H.load_state(engine, c, st0)
+            loss = H.train(engine, c, 0.05, batch)
+            outs.append((loss, H.read_state(engine, c)))
+        np.testing.assert_array_equal(outs[0][0], outs[1][0])
+        for k in ("entity_data", "relation_embedding"):
+            np.testing.assert_array_equal(outs[0][1][k], outs[1][1][k])
 
 
 def test_engine_errors():
