@@ -495,9 +495,9 @@ def test_step_raw_zipf_duplicates_plan_readback(oracle64, shape):
 
 
 def test_step_hottest_row_above_the_in_launch_limit(oracle64):
-    # 4 096 contributions for two rows: past the limit, the two-level reduction runs as without
-    # the read-back
-    kw = dict(distance_fn="L2", shared_table=True, n_shard=8, batch=256, a2a=32, n_entity=3, dim=32, feature=0,
+    # 8 192 contributions for two rows, about 5 600 of them for the first: past the limit, the
+    # two-level reduction runs as without the read-back
+    kw = dict(distance_fn="L2", shared_table=True, n_shard=16, batch=256, a2a=16, n_entity=3, dim=32, feature=0,
               n_relation=4, gamma=5.0)
     run_case(oracle64, kw, n_step=2, batch_fn=K.raw_batch, **READBACK)
 
