@@ -74,7 +74,7 @@ PEAK_BF16_TFLOPS = 2500.0
 # here and refreshed together with the committed profiler summaries.
 MEASURED_TRAFFIC_BYTES = {
     ("c2", "score_bwd"): 41.9e6,     # 25.1 MB fetched + 16.8 MB written
-    ("c3l2", "score_bwd"): 148.4e6,  # 98.0 MB fetched + 50.3 MB written
+    ("c3l2", "score_bwd"): 215.5e6,  # 165.1 MB fetched + 50.3 MB written
 }
 
 

@@ -567,8 +567,8 @@ void launch_gather_operands(const RowSource& ent, const float* rel, const uint32
 // tiles on one XCD (block z on XCD z % 8), in consecutive slots of that XCD.
 struct TileId { int x, y, z, gx, gy; };
 constexpr int kXcdGroup = 2;
-DEVINL TileId xcd_tile(int gx, int gy, int gz) {
-    const int L = blockIdx.x, n = gx * gy;
+DEVINL TileId xcd_tile(int gx, int gy, int gz, int L) {
+    const int n = gx * gy;
     int z, t;
     if ((gz & 7) == 0) {
         // kXcdGroup blocks of an XCD are interleaved tile by tile, so that the CUs of
@@ -586,6 +586,7 @@ DEVINL TileId xcd_tile(int gx, int gy, int gz) {
     id.y = t / gx; id.x = t - id.y * gx; id.z = z; id.gx = gx; id.gy = gy;
     return id;
 }
+DEVINL TileId xcd_tile(int gx, int gy, int gz) { return xcd_tile(gx, gy, gz, (int)blockIdx.x); }
 static dim3 tile_grid(int gx, int gy, int gz) { return dim3((unsigned)(gx * gy * gz)); }
 
 // --------------------------------------------------------------------------
@@ -2157,13 +2158,24 @@ __global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma(BwdParams p) {
 }
 template <int DIST, int BJT, bool ALIGNED, int NW>
 __global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma_both(BwdParams p) {
-    // a block's head-side tiles and then its tail-side tiles, back to back on one XCD:
-    // both sides read the same operand rows and coefficient matrix
     __shared__ __attribute__((aligned(16))) char smem[kBwdSmemBytes];  // one allocation serves either side
-    const int gy = (p.B > p.T ? p.B : p.T) / BM_TI;
-    const TileId tile = xcd_tile(p.Dp / BM_TK, 2 * gy, p.S);
-    if (tile.y < gy) bwd_mfma_body<DIST, 0, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y, smem);
-    else bwd_mfma_body<DIST, 1, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y - gy, smem);
+    // One launch for both sides. The side whose tiles loop over more rows of the other side comes
+    // first, for every block, then the other side: the long tiles do not start last (at the end of
+    // the launch the CUs run dry while the longest tiles finish), and no workgroup is started for
+    // a tile that does not exist. A block's tiles of one side stay together on one XCD; its two
+    // sides no longer run close enough in time to share the L2's copy of the operand rows and the
+    // coefficient matrix, which was measured to cost less than the late long tiles did.
+    const int gx = p.Dp / BM_TK, ga = p.B / BM_TI, gb = p.T / BM_TI;
+    const bool heads_first = p.T >= p.B;  // a head tile loops over T rows, a tail tile over B
+    const int n_first = gx * (heads_first ? ga : gb) * p.S;
+    const int L = blockIdx.x;
+    if ((L < n_first) == heads_first) {
+        const TileId tile = xcd_tile(gx, ga, p.S, heads_first ? L : L - n_first);
+        bwd_mfma_body<DIST, 0, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y, smem);
+    } else {
+        const TileId tile = xcd_tile(gx, gb, p.S, heads_first ? L - n_first : L);
+        bwd_mfma_body<DIST, 1, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y, smem);
+    }
 }
 
 static void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
@@ -2287,7 +2299,7 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
     const bool both = sh.use_mfma && plain && sh.B % BM_TI == 0 && sh.T % BM_TI == 0 && sh.Dp % BM_TK == 0 &&
                       (dist_fn == DIST_DOT || (dist_fn == DIST_L2 && nearflag));
     if (both) {
-        const dim3 grid = tile_grid(sh.Dp / BM_TK, 2 * (std::max(sh.B, sh.T) / BM_TI), sh.S);
+        const dim3 grid = tile_grid(sh.Dp / BM_TK, sh.B / BM_TI + sh.T / BM_TI, sh.S);
         // eight waves per workgroup (two per SIMD): measured faster than four at
         // every benchmark shape, few workgroups (1M-row workload) or many (22.8M-row workload)
         if (dist_fn == DIST_L2)
