@@ -2679,20 +2679,23 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
 }
 
 // One launch for both tables without a first-level reduction before it.
-//   blocks [0, NS0 * max_hot0), [.., + NS1 * max_hot1): hot rows, one workgroup per (row, 16 columns).
-//     Lane = (slot, column group): sixteen contributions per load instruction (64 bytes of each),
-//     eight such loads in flight; a lane adds
-//     its slot's contributions in sorted order, the sixteen slots meet by butterfly shuffles (both
-//     operand orders give the same float), the four waves' sums in LDS in wave order; four lanes
-//     of wave 0 then update the 16 columns.
+//   blocks [0, NS0 * max_hot0), [.., + NS1 * max_hot1): hot rows, one workgroup per (row, 32 columns).
+//     Lane = (slot, column group): eight contributions per load instruction (128 bytes of each),
+//     sixteen such loads in flight; a lane adds its slot's contributions in sorted order, the
+//     eight slots meet by butterfly shuffles (both operand orders give the same float), the four
+//     waves' sums in LDS in wave order; eight lanes of wave 0 then update the 32 columns.
 //   the remaining blocks: every other row, one wave per row, as k_adam_rows.
 // columns per hot-row workgroup: 32 (128 bytes of every contribution per load; 16 and 8 columns
 // measured slower: the same rows are then fetched by two and four times as many workgroups)
 constexpr int kHotColumns = 32;
+// loads in flight per lane: 16 (the update of a 1M-row table's step measured 22.4 / 20.5 / 20.8 /
+// 23.6 us with 8 / 16 / 24 / 32; the registers of the larger ones cost the other rows' waves
+// their residency); four waves per workgroup (2, 8 and 16 measured slower)
+constexpr int kHotLoads = 16, kHotWaves = 4;
 template <bool MF32>
-__global__ __launch_bounds__(256) void k_adam_rows_hot(AdamArgs a0, HotRows h0, AdamArgs a1, HotRows h1) {
+__global__ __launch_bounds__(kHotWaves * 64) void k_adam_rows_hot(AdamArgs a0, HotRows h0, AdamArgs a1, HotRows h1) {
     constexpr int HC = kHotColumns, HS = 64 / (HC / 4);  // columns per workgroup, slots per wave
-    __shared__ __attribute__((aligned(16))) float part[3][HC];
+    __shared__ __attribute__((aligned(16))) float part[kHotWaves - 1][HC];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ns0 = (a0.Dp + HC - 1) / HC, ns1 = (a1.Dp + HC - 1) / HC;
     const int hot0 = ns0 * h0.max_hot, hot1 = ns1 * h1.max_hot;
@@ -2710,25 +2713,25 @@ __global__ __launch_bounds__(256) void k_adam_rows_hot(AdamArgs a0, HotRows h0, 
         const int cg = lane & (HC / 4 - 1), slot = lane / (HC / 4), col = cb * HC + cg * 4;
         const bool active = col < Dp;
         // this wave's quarter of the contributions, in whole groups of HS
-        const uint32_t groups = (n + HS - 1) / HS, gshare = (groups + 3) / 4;
+        const uint32_t groups = (n + HS - 1) / HS, gshare = (groups + kHotWaves - 1) / kHotWaves;
         const uint32_t w0 = min(n, wave * gshare * HS), w1 = min(n, w0 + gshare * HS);
         const uint32_t* __restrict__ items = a.src.sorted_item + pos;
         const float* __restrict__ grad = a.src.grad;
         float4 acc = make_float4(0, 0, 0, 0);
-        for (uint32_t j = w0; j < w1; j += 8 * HS) {
-            uint32_t c[8];
-            float4 v[8];
+        for (uint32_t j = w0; j < w1; j += kHotLoads * HS) {
+            uint32_t c[kHotLoads];
+            float4 v[kHotLoads];
 #pragma unroll
-            for (int x = 0; x < 8; ++x) {
+            for (int x = 0; x < kHotLoads; ++x) {
                 const uint32_t idx = j + x * HS + slot;
                 c[x] = idx < w1 ? items[idx] : 0xffffffffu;
             }
 #pragma unroll
-            for (int x = 0; x < 8; ++x)
+            for (int x = 0; x < kHotLoads; ++x)
                 v[x] = (active && c[x] != 0xffffffffu) ? *reinterpret_cast<const float4*>(grad + (size_t)c[x] * Dp + col)
                                                       : make_float4(0, 0, 0, 0);
 #pragma unroll
-            for (int x = 0; x < 8; ++x) acc = f4add(acc, v[x]);
+            for (int x = 0; x < kHotLoads; ++x) acc = f4add(acc, v[x]);
         }
 #pragma unroll
         for (int off = HC / 4; off < 64; off <<= 1) {
@@ -2740,7 +2743,7 @@ __global__ __launch_bounds__(256) void k_adam_rows_hot(AdamArgs a0, HotRows h0, 
         if (wave != 0 || slot != 0 || !active) return;
         float4 g = acc;
 #pragma unroll
-        for (int w = 0; w < 3; ++w) g = f4add(g, *reinterpret_cast<const float4*>(&part[w][cg * 4]));
+        for (int w = 0; w < kHotWaves - 1; ++w) g = f4add(g, *reinterpret_cast<const float4*>(&part[w][cg * 4]));
         char* prow = a.p_base + (int64_t)key * a.pitch;
         char* mrow = a.m_base + (int64_t)key * a.pitch;
         char* vrow = a.v_base + (int64_t)key * a.pitch;
@@ -2760,10 +2763,10 @@ __global__ __launch_bounds__(256) void k_adam_rows_hot(AdamArgs a0, HotRows h0, 
         return;
     }
     b -= hot0 + hot1;
-    const int blocks0 = (a0.max_rows + 3) / 4;
+    const int blocks0 = (a0.max_rows + kHotWaves - 1) / kHotWaves;
     const bool second = b >= blocks0;
     const AdamArgs& a = second ? a1 : a0;
-    const int u = (second ? b - blocks0 : b) * 4 + wave;
+    const int u = (second ? b - blocks0 : b) * kHotWaves + wave;
     const int uc = min(u, a.max_rows - 1);
     const uint32_t key = a.uniq_key[uc];
     const uint32_t q0 = a.chunk_off[uc], q1 = a.chunk_off[uc + 1];
@@ -2813,11 +2816,11 @@ void launch_adam_rows_hot2(const AdamArgs& a0, const HotRows& h0, const AdamArgs
                            hipStream_t stream) {
     const int hot = ((a0.Dp + kHotColumns - 1) / kHotColumns) * h0.max_hot +
                     ((a1.Dp + kHotColumns - 1) / kHotColumns) * h1.max_hot;
-    const dim3 grid(hot + (a0.max_rows + 3) / 4 + (a1.max_rows + 3) / 4);
+    const dim3 grid(hot + (a0.max_rows + kHotWaves - 1) / kHotWaves + (a1.max_rows + kHotWaves - 1) / kHotWaves);
     if (grid.x == 0) return;
     const bool f32 = (a0.max_rows == 0 || a0.m_etype == ET_F32) && (a1.max_rows == 0 || a1.m_etype == ET_F32);
-    if (f32) hipLaunchKernelGGL((k_adam_rows_hot<true>), grid, dim3(256), 0, stream, a0, h0, a1, h1);
-    else hipLaunchKernelGGL((k_adam_rows_hot<false>), grid, dim3(256), 0, stream, a0, h0, a1, h1);
+    if (f32) hipLaunchKernelGGL((k_adam_rows_hot<true>), grid, dim3(kHotWaves * 64), 0, stream, a0, h0, a1, h1);
+    else hipLaunchKernelGGL((k_adam_rows_hot<false>), grid, dim3(kHotWaves * 64), 0, stream, a0, h0, a1, h1);
 }
 
 static void launch_adam_kernel(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream) {
