@@ -299,8 +299,103 @@ def kernel_table(w, timing, n_steps, uniq_rows):
     return out
 
 
+def predict_bench(args, w, kge, torch):
+    """`--mode predict`: the all-entity scoring sweep with the running n_best
+    (reference src/poplar_kge.cpp:743-855 behind Engine.predict,
+    src/python/poplar_kge.py:781-861).  One "step" is one `predict` program
+    run: predict_hr_batch_size queries against every row of one shard's table,
+    query batch and n_best as in the reference's large configuration
+    (src/python/poplar_kge.py:395-397).  Prints one JSON line of its own."""
+    Q, n_best = 128, 100
+    s = kge.Settings.create_demo()
+    s.seed = 20240611
+    m, d, e = s.model, s.data, s.execution
+    m.score_fn, m.distance_fn = w.get("score_fn", "TransE"), w["distance_fn"]
+    m.n_shard, m.n_entity, m.n_relation_type = 1, w["n_entity"], w["n_relation"]
+    m.embedding_size, m.entity_feature_size, m.gamma = w["dim"], 0, 10.0
+    m.init_scale = float(np.sqrt(w["dim"]))
+    d.batch_size, d.a2a_size = 256, 256
+    e.device, e.dtype, e.shared_table = "hip", "float32", False
+    e.embedding_dtype = w.get("embedding_dtype")
+    e.train_steps_per_program_run, e.rw_batch_size = 1, 8192
+    e.predict_hr_batch_size, e.predict_n_best = Q, n_best
+    settings = s.prepare()
+    engine = kge.Engine(settings, np.full(1, m.n_entity - 1))
+    init_tables(engine, settings)
+    rng = np.random.default_rng(7)
+    head = rng.integers(1, m.n_entity, (1, Q)).astype(np.uint32)
+    relation = rng.integers(0, m.n_relation_type, (1, Q)).astype(np.uint32)
+    scores = np.zeros((1, 1, Q, n_best), np.float32)
+    rows = np.zeros(scores.shape, np.uint32)
+    call = dict(predict_head=head, predict_relation=relation,
+                predict_entity_count=np.full(1, m.n_entity - 1, np.uint32),
+                predict_scores=scores, predict_indices=rows)
+    for _ in range(args.warmup):
+        engine.engine.run("predict", call)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        engine.engine.run("predict", call)   # synchronous: the n_best are on the host when it returns
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+
+    # check: ranks sorted, rows valid, and every returned score recomputed in float64 from the
+    # returned row, the head's row and the relation's (TransE: gamma - |h + r - t|)
+    sc, ix = scores[0, 0], rows[0, 0]
+    assert np.all(sc[:, :-1] >= sc[:, 1:]) and ix.min() >= 1 and ix.max() < m.n_entity
+    D = m.embedding_size
+    rel = engine.read_variable("relation_embedding").reshape(-1, D).astype(np.float64)
+    nq = 8
+    t_rows = read_rows(engine, settings, ix[:nq].reshape(-1))[:, :D].astype(np.float64).reshape(nq, n_best, D)
+    h_rows = read_rows(engine, settings, head[0, :nq])[:, :D].astype(np.float64)
+    diff = (h_rows + rel[relation[0, :nq]])[:, None, :] - t_rows
+    dist = np.sqrt((diff ** 2).sum(-1)) if m.distance_fn == "L2" else np.abs(diff).sum(-1)
+    err = float(np.max(np.abs((m.gamma - dist) - sc[:nq]) / np.maximum(1.0, np.abs(sc[:nq]))))
+    assert err < 1e-5, err
+
+    # CPU baseline: the same sweep in NumPy float32 over a bounded sample of the table
+    # (the product form for L2, |a - b| summed in slabs for L1), one thread
+    n_cpu = min(m.n_entity - 1, 200_000 if m.distance_fn == "L2" else 20_000)
+    cand = read_rows(engine, settings, np.arange(1, n_cpu + 1, dtype=np.uint32))[:, :D]
+    q32 = (read_rows(engine, settings, head[0])[:, :D] + rel[relation[0]].astype(np.float32)).astype(np.float32)
+    torch.set_num_threads(1)
+    t1 = time.perf_counter()
+    if m.distance_fn == "L2":
+        d2 = (q32 ** 2).sum(1)[:, None] + (cand ** 2).sum(1)[None, :] - 2.0 * (q32 @ cand.T)
+        sc_cpu = m.gamma - np.sqrt(np.maximum(d2, 0.0))
+    else:
+        sc_cpu = np.stack([m.gamma - np.abs(q[None, :] - cand).sum(1) for q in q32])
+    top = np.argpartition(-sc_cpu, n_best, axis=1)[:, :n_best]
+    cpu_dt = time.perf_counter() - t1
+    del top
+
+    pairs = float(Q) * (m.n_entity - 1)
+    flop = 3.0 * pairs * D
+    emb_bytes = 2 if w.get("embedding_dtype") == "bfloat16" else 4
+    table_bytes = float(m.n_entity - 1) * D * emb_bytes
+    frac_flop, frac_hbm = flop / dt / 1e12 / PEAK_FP32_TFLOPS, table_bytes / dt / 1e9 / PEAK_HBM_GBPS
+    roof = (dict(bound="mfma", achieved=flop / dt / 1e12, peak=PEAK_FP32_TFLOPS, unit="TFLOP/s", frac=frac_flop)
+            if frac_flop >= frac_hbm else
+            dict(bound="hbm", achieved=table_bytes / dt / 1e9, peak=PEAK_HBM_GBPS, unit="GB/s", frac=frac_hbm))
+    roof.update(traffic=None, kernel="predict sweep (gather + score + n_best merge), whole program run",
+                launch_ms=dt * 1e3)
+    print(json.dumps(dict(
+        metric="predict_candidate_scores_per_s", value=pairs / dt, unit="scores/s", n_gpus=1,
+        steps=args.steps, warmup=args.warmup, ms_per_step=dt * 1e3, higher_is_better=True,
+        scaling="weak", vs_baseline=None, dtype="f32", data="synthetic",
+        config=dict(workload=f"predict over {w['desc'].split(',')[0]}, {m.n_entity} rows of one shard, "
+                             f"{Q} queries per run, n_best {n_best}"),
+        roofline=roof,
+        cpu_baseline=dict(value=float(Q) * n_cpu / cpu_dt, unit="scores/s", cores=1, kind="port",
+                          sample=f"{Q} queries against the first {n_cpu} rows, NumPy float32, "
+                                 f"scores and n_best selection, {cpu_dt:.2f} s"),
+        check=dict(recomputed_score_rel_err=err, queries_checked=nq))))
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--mode", default="train", choices=["train", "predict"],
+                    help="train: the training step (the headline metric); predict: the all-entity scoring sweep")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
@@ -328,6 +423,10 @@ def main():
     if args.n_entity:
         w["n_entity"] = args.n_entity
         w["desc"] += f" [table size overridden: {args.n_entity}]"
+    if args.mode == "predict":
+        if w.get("feature") or w.get("score_fn", "TransE") != "TransE":
+            sys.exit("--mode predict covers the TransE workloads without features")
+        return predict_bench(args, w, kge, torch)
     n_total = args.warmup + args.steps
     settings = make_settings(w, n_total, kge)
     if args.scoring:

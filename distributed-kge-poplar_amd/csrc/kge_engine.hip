@@ -212,6 +212,7 @@ struct kge_engine {
     uint32_t seed;
     int n_step, rw_batch;
     int predict_hr_batch = 0, predict_n_best = 0;
+    int predict_chunk_rows = 32768;  // additive setting execution.predict_chunk_rows: tails scored per launch
     int stream_kind;  // KGE_F32 or KGE_F16: dtype of the entity read/write streams
     bool profile_kernels = false;
     // additive setting execution.scoring: "mfma_bf16x3" (2, the default: matrix cores, the forward
@@ -382,6 +383,11 @@ void parse_settings(kge_engine& E, const Items& s) {
                                     "'execution.shared_table' a row's loss share has no owning shard");
     E.profile_kernels = s.find("execution.profile_kernels") ? s.boolean("execution.profile_kernels") : false;
     if (s.find("execution.reduce_chunk")) E.chunk = (int)s.uint("execution.reduce_chunk");
+    if (s.find("execution.predict_chunk_rows")) {
+        const unsigned v = s.uint("execution.predict_chunk_rows");
+        if (v < 64 || v > (1u << 20)) throw std::invalid_argument("'execution.predict_chunk_rows' must be in [64, 1048576]");
+        E.predict_chunk_rows = (int)v;
+    }
     if (s.find("execution.plan_readback_steps")) E.plan_readback_steps = std::max(1, (int)s.uint("execution.plan_readback_steps"));
     if (s.find("execution.scoring")) {
         const std::string v = s.str("execution.scoring");
@@ -1436,7 +1442,7 @@ void run_predict(kge_engine& E, const Items& in) {
     uint32_t* out_i = (uint32_t*)in.array("predict_indices", KGE_U32, {S, S, Hb, nb});
     const hipStream_t st = E.stream;
     const int Q = (int)(S * Hb), Qp = round_up(Q, 128), Dp = E.Dp;
-    const int chunk = round_up((int)std::min<int64_t>(E.n_entity, 8192), 64);
+    const int chunk = round_up((int)std::min<int64_t>(E.n_entity, E.predict_chunk_rows), 64);
 
     std::vector<uint32_t> rows(Qp, 0u), rels(Qp, 0u);
     for (size_t s = 0; s < S; ++s) {

@@ -2331,11 +2331,19 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
 // predict: running top-k over a stream of score chunks
 // (TopKCollector, src/poplar_kge.cpp:743-809).  One workgroup per query keeps
 // its n_best (score, index) pairs sorted by (score descending, index
-// ascending); a block of 1024 new scores is merged only if one of them beats
-// the current n_best-th score, by a bitonic sort of the 2048-entry union in LDS.
-// Ties therefore resolve to the lower index, whatever the chunking.
+// ascending).  New scores are compared with the current n_best-th score a span
+// of 8192 at a time (32 per thread, loads back to back); the few that beat it
+// are collected in LDS (in any order) and merged by rank: every element of
+// (current best, candidates) counts the candidates that come before it, a
+// candidate also finds its place among the sorted best by binary search, and
+// the elements whose rank is below n_best are written to that place.  The
+// order is total on distinct rows, so the result does not depend on the order
+// of collection, and ties resolve to the lower index whatever the chunking.
+// A span with more than 1024 candidates (the first rows of a sweep) is redone
+// 1024 scores at a time.
 
-constexpr int TK_BLOCK = 1024, TK_SORT = 2048;
+constexpr int TK_BLOCK = 1024;  // most n_best, and the candidate list's capacity
+constexpr int TK_SPAN = 8192;
 
 DEVINL bool topk_before(float sa, uint32_t ia, float sb, uint32_t ib) {
     return sa > sb || (sa == sb && ia < ib);
@@ -2345,74 +2353,118 @@ __global__ __launch_bounds__(256) void k_topk_merge(const float* __restrict__ sc
                                                     int n_valid, uint32_t first_index, int n_best,
                                                     float* __restrict__ best_score,
                                                     uint32_t* __restrict__ best_index) {
-    __shared__ float ks[TK_SORT];
-    __shared__ uint32_t vs[TK_SORT];
+    __shared__ __attribute__((aligned(16))) float cand_s[TK_BLOCK];
+    __shared__ __attribute__((aligned(16))) uint32_t cand_i[TK_BLOCK];
+    __shared__ float cur_s[TK_BLOCK], next_s[TK_BLOCK];
+    __shared__ uint32_t cur_i[TK_BLOCK], next_i[TK_BLOCK];
+    // candidate counters of three consecutive passes: the one of the pass after this one is cleared
+    // before this pass's barrier, when every thread has read its previous value (a pass ago)
+    __shared__ int n_cand[3];
     const int q = blockIdx.x, tid = threadIdx.x;
     const float* row = scores + (size_t)q * ld;
     float* bs = best_score + (size_t)q * n_best;
     uint32_t* bi = best_index + (size_t)q * n_best;
-    // the current best live in ks / vs [TK_BLOCK, TK_BLOCK + n_best)
-    for (int i = tid; i < TK_BLOCK; i += 256) {
-        ks[TK_BLOCK + i] = i < n_best ? bs[i] : -INFINITY;
-        vs[TK_BLOCK + i] = i < n_best ? bi[i] : 0xffffffffu;
+    for (int i = tid; i < n_best; i += 256) {
+        cur_s[i] = bs[i];
+        cur_i[i] = bi[i];
     }
+    if (tid == 0) n_cand[0] = n_cand[1] = 0;
     __syncthreads();
     bool changed = false;
-    for (int base = 0; base < n_valid; base += TK_BLOCK) {
-        const float kth = ks[TK_BLOCK + n_best - 1];
-        float v[4];
-        bool beats = false;
+    int pass = 0;
+    for (int span0 = 0; span0 < n_valid; span0 += TK_SPAN) {
+        const int span1 = min(n_valid, span0 + TK_SPAN);
+        int piece = TK_SPAN;
+        for (int base = span0; base < span1;) {
+            const int end = min(span1, base + piece);
+            const float kth = cur_s[n_best - 1];
+            int* counter = &n_cand[pass % 3];
+            if (tid == 0) n_cand[(pass + 1) % 3] = 0;
+            ++pass;
+            for (int i0 = base; i0 < end; i0 += 256 * 8) {
+                float v[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int i = base + tid + 256 * j;
-            v[j] = i < n_valid ? row[i] : -INFINITY;
-            beats = beats || v[j] > kth;
-        }
-        if (!__syncthreads_or(beats)) continue;
-        changed = true;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            ks[tid + 256 * j] = v[j];
-            vs[tid + 256 * j] = first_index + (uint32_t)(base + tid + 256 * j);
-        }
-        __syncthreads();
-        // bitonic sort of all TK_SORT entries, best first
-        for (int size = 2; size <= TK_SORT; size <<= 1)
-            for (int stride = size >> 1; stride > 0; stride >>= 1) {
-                for (int t = tid; t < TK_SORT / 2; t += 256) {
-                    const int lo = 2 * t - (t & (stride - 1)), hi = lo + stride;
-                    const bool up = (lo & size) == 0;  // this run sorts best-first
-                    const float sa = ks[lo], sb = ks[hi];
-                    const uint32_t ia = vs[lo], ib = vs[hi];
-                    const bool ordered = topk_before(sa, ia, sb, ib) || (sa == sb && ia == ib);
-                    if (ordered != up) {
-                        ks[lo] = sb; ks[hi] = sa;
-                        vs[lo] = ib; vs[hi] = ia;
-                    }
+                for (int j = 0; j < 8; ++j) {
+                    const int i = i0 + tid + 256 * j;
+                    v[j] = i < end ? row[i] : -INFINITY;
                 }
-                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (v[j] > kth) {  // false for NaN, and for -inf padding
+                        const int slot = atomicAdd(counter, 1);
+                        if (slot < TK_BLOCK) {
+                            cand_s[slot] = v[j];
+                            cand_i[slot] = first_index + (uint32_t)(i0 + tid + 256 * j);
+                        }
+                    }
             }
-        // the n_best winners move back to their place, the rest is dropped
-        float ws[4];
-        uint32_t wi[4];
+            __syncthreads();
+            const int c = *counter;  // the same for every thread: all branches below are uniform
+            if (c > TK_BLOCK) {  // only a whole span can overflow: a piece of TK_BLOCK scores cannot
+                piece = TK_BLOCK;
+                continue;
+            }
+            base = end;
+            if (c == 0) continue;
+            changed = true;
+            // candidates padded to whole groups of four with entries that come before nothing
+            for (int x = c + tid; x < ((c + 3) & ~3); x += 256) {
+                cand_s[x] = -INFINITY;
+                cand_i[x] = 0xffffffffu;
+            }
+            __syncthreads();
+            // a thread's elements: candidates tid + 256 m (m < 4), current best tid + 256 (m - 4)
+            constexpr int PER = TK_BLOCK / 256;
+            float es[2 * PER];
+            uint32_t ei[2 * PER];
+            int r[2 * PER];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int i = tid + 256 * j;
-            ws[j] = i < n_best ? ks[i] : -INFINITY;
-            wi[j] = i < n_best ? vs[i] : 0xffffffffu;
-        }
-        __syncthreads();
+            for (int m = 0; m < PER; ++m) {
+                const int e = tid + 256 * m;
+                es[m] = e < c ? cand_s[e] : -INFINITY;
+                ei[m] = e < c ? cand_i[e] : 0xffffffffu;
+                int lo = 0, hi = e < c ? n_best : 0;
+                while (lo < hi) {  // entries of the sorted best that come before this candidate
+                    const int mid = (lo + hi) >> 1;
+                    if (topk_before(cur_s[mid], cur_i[mid], es[m], ei[m])) lo = mid + 1;
+                    else hi = mid;
+                }
+                r[m] = e < c ? lo : n_best;
+                es[PER + m] = e < n_best ? cur_s[e] : -INFINITY;
+                ei[PER + m] = e < n_best ? cur_i[e] : 0xffffffffu;
+                r[PER + m] = e < n_best ? e : n_best;
+            }
+            // every element counts the candidates before it: four candidates per LDS read (the same
+            // address for all lanes), up to eight elements per lane against them
+            for (int x = 0; x < c; x += 4) {
+                const float4 s4 = *reinterpret_cast<const float4*>(&cand_s[x]);
+                const uint4 i4 = *reinterpret_cast<const uint4*>(&cand_i[x]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            ks[TK_BLOCK + tid + 256 * j] = ws[j];
-            vs[TK_BLOCK + tid + 256 * j] = wi[j];
+                for (int m = 0; m < 2 * PER; ++m) {
+                    const bool live = m < PER ? 256 * m < c : 256 * (m - PER) < n_best;  // uniform
+                    if (!live) continue;
+                    r[m] += (topk_before(s4.x, i4.x, es[m], ei[m]) ? 1 : 0) + (topk_before(s4.y, i4.y, es[m], ei[m]) ? 1 : 0) +
+                            (topk_before(s4.z, i4.z, es[m], ei[m]) ? 1 : 0) + (topk_before(s4.w, i4.w, es[m], ei[m]) ? 1 : 0);
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < 2 * PER; ++m)
+                if (r[m] < n_best) {
+                    next_s[r[m]] = es[m];
+                    next_i[r[m]] = ei[m];
+                }
+            __syncthreads();
+            for (int i = tid; i < n_best; i += 256) {
+                cur_s[i] = next_s[i];
+                cur_i[i] = next_i[i];
+            }
+            __syncthreads();
         }
-        __syncthreads();
     }
     if (changed)
         for (int i = tid; i < n_best; i += 256) {
-            bs[i] = ks[TK_BLOCK + i];
-            bi[i] = vs[TK_BLOCK + i];
+            bs[i] = cur_s[i];
+            bi[i] = cur_i[i];
         }
 }
 

@@ -167,7 +167,7 @@ def _random_queries(engine, n):
 
 @pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "complex", "rotate", "transh", "transh_big",
                                      "feature_mlp", "feature_dropout", "separate_networks_mlp",
-                                     "no_features_big"])
+                                     "no_features_big", "n_best_max", "one_chunk"])
 def test_predict_vs_brute_force(variant):
     """Engine.predict against a float64 brute force over every row of every shard
     (the reference checks shapes, ranges and ordering, tests/python/test_poplar_kge.py:155-175,
@@ -194,10 +194,18 @@ def test_predict_vs_brute_force(variant):
         m.share_feature_networks, m.feature_mlp_size = False, 16
     elif variant == "feature_dropout":
         m.feature_dropout = 0.4   # training only (entityHidden(..., training=false), src/poplar_kge.cpp:419-422)
+    elif variant in ("n_best_max", "one_chunk"):
+        # the whole shard in one chunk of tails (several spans of the merge, the first ones with more
+        # candidates than its list holds); the largest n_best the device keeps
+        m.n_entity, m.entity_feature_size, m.embedding_size, m.n_shard = 20000, 0, 32, 2
+        settings.data.batch_size, ex.rw_batch_size = 6, 4096
+        ex.predict_n_best = 1024 if variant == "n_best_max" else 100
+        m.distance_fn = "L2"
     elif variant in ("no_features_big", "transh_big"):
         # several chunks of tails per shard, several query chunks, ragged counts
         m.n_entity, m.entity_feature_size, m.embedding_size, m.n_shard = 20000, 0, 32, 3
         settings.data.batch_size, ex.rw_batch_size, ex.predict_n_best = 6, 4096, 20
+        ex.predict_chunk_rows = 8192
         m.distance_fn = "L2"
         if variant == "transh_big":
             m.score_fn = "TransH"
@@ -225,6 +233,34 @@ def test_predict_vs_brute_force(variant):
     close = np.abs(found.score - want_score) <= 1e-5 * np.maximum(1.0, np.abs(want_score))
     assert np.all(agree | close)
     assert agree.mean() > 0.99
+
+
+@pytest.mark.parametrize("chunk_rows", [None, 4096])
+def test_predict_ties_go_to_the_lower_row(chunk_rows):
+    """All embeddings zero: every tail scores the same, so each tail shard's n_best are its
+    first rows in order, however the sweep is cut into chunks (the reference leaves ties to
+    the host's argsort, src/python/poplar_kge.py:806-817; this build fixes them)."""
+    import poplar_kge as kge
+
+    settings = kge.Settings.create_demo()
+    m, ex = settings.model, settings.execution
+    m.n_entity, m.entity_feature_size, m.embedding_size, m.n_shard = 20000, 0, 32, 2
+    m.distance_fn, m.init_scale = "L2", 0.0
+    settings.data.batch_size, ex.rw_batch_size, ex.predict_n_best = 6, 4096, 100
+    ex.predict_chunk_rows = chunk_rows
+    settings.prepare()
+    S, Hb, nb = m.n_shard, ex.predict_hr_batch_size, ex.predict_n_best
+    counts = np.array([m.n_entity - 1, m.n_entity - 50])
+    engine = kge.Engine(settings, counts)
+    engine.initialise_all(np.zeros((S, m.n_entity, 0), np.float16))
+    scores = np.full((S, S, Hb, nb), np.nan, np.float32)
+    rows = np.zeros(scores.shape, np.uint32)
+    engine.engine.run("predict", dict(
+        predict_head=engine.random_integers(m.n_entity - 60, (S, Hb)) + 1,
+        predict_relation=engine.random_integers(m.n_relation_type, (S, Hb)),
+        predict_entity_count=counts.astype(np.uint32), predict_scores=scores, predict_indices=rows))
+    np.testing.assert_array_equal(rows, np.broadcast_to(np.arange(1, nb + 1, dtype=np.uint32), rows.shape))
+    np.testing.assert_array_equal(scores, np.full(scores.shape, m.gamma, np.float32))
 
 
 def test_training_mrr_matches_brute_force():
