@@ -319,6 +319,7 @@ def predict_bench(args, w, kge, torch):
     e.embedding_dtype = w.get("embedding_dtype")
     e.train_steps_per_program_run, e.rw_batch_size = 1, 8192
     e.predict_hr_batch_size, e.predict_n_best = Q, n_best
+    e.predict_chunk_rows = args.predict_chunk_rows
     settings = s.prepare()
     engine = kge.Engine(settings, np.full(1, m.n_entity - 1))
     init_tables(engine, settings)
@@ -404,6 +405,8 @@ def main():
                     help="steps the CPU baseline times (default: sized for ~10-30 s)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--n-entity", type=int, default=None, help="override the table size (experiments)")
+    ap.add_argument("--predict-chunk-rows", type=int, default=None,
+                    help="--mode predict: tails scored per launch (experiments; default: the engine's)")
     ap.add_argument("--scoring", default=None, choices=["mfma", "mfma_bf16x3", "valu"], help="scoring kernels (default mfma_bf16x3)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -212,7 +212,7 @@ struct kge_engine {
     uint32_t seed;
     int n_step, rw_batch;
     int predict_hr_batch = 0, predict_n_best = 0;
-    int predict_chunk_rows = 32768;  // additive setting execution.predict_chunk_rows: tails scored per launch
+    int predict_chunk_rows = 65536;  // additive setting execution.predict_chunk_rows: tails scored per launch
     int stream_kind;  // KGE_F32 or KGE_F16: dtype of the entity read/write streams
     bool profile_kernels = false;
     // additive setting execution.scoring: "mfma_bf16x3" (2, the default: matrix cores, the forward
@@ -230,6 +230,10 @@ struct kge_engine {
 
     // ---- device state ----
     hipStream_t stream = nullptr;
+    // predict: the n_best merge of one chunk of tails runs here while the next chunk is gathered
+    // and scored on `stream` (the merge occupies one workgroup per query, a fraction of the chip)
+    hipStream_t merge_stream = nullptr;
+    hipEvent_t scored[2] = {nullptr, nullptr}, merged[2] = {nullptr, nullptr};
     DevBuf<char> table;
     DevBuf<float> rel, rel_m, rel_v, proj, proj_m, proj_v;
     uint32_t step = 0;
@@ -282,6 +286,9 @@ struct kge_engine {
     ~kge_engine() {
         for (auto& e : ev) if (e) (void)hipEventDestroy(e);
         for (auto& e : kev) (void)hipEventDestroy(e);
+        for (auto& e : scored) if (e) (void)hipEventDestroy(e);
+        for (auto& e : merged) if (e) (void)hipEventDestroy(e);
+        if (merge_stream) (void)hipStreamDestroy(merge_stream);
         if (stream) (void)hipStreamDestroy(stream);
     }
 };
@@ -539,7 +546,10 @@ void allocate(kge_engine& E) {
                                  (dev_err != hipSuccess ? hipGetErrorString(dev_err) : "no device") + ")");
     }
     HIP_CHECK(hipStreamCreate(&E.stream));
+    HIP_CHECK(hipStreamCreate(&E.merge_stream));
     for (auto& e : E.ev) HIP_CHECK(hipEventCreate(&e));
+    for (auto& e : E.scored) HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    for (auto& e : E.merged) HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
     const hipStream_t st = E.stream;
 
     E.table.alloc((size_t)E.n_rows * E.L.pitch);
@@ -1461,7 +1471,7 @@ void run_predict(kge_engine& E, const Items& in) {
         E.p_rel.alloc(Qp);
         E.p_count.alloc(1);
         E.p_opnd.alloc((size_t)(Qp + chunk) * Dp);
-        E.p_scores.alloc((size_t)Qp * chunk);
+        E.p_scores.alloc((size_t)2 * Qp * chunk);  // two chunks: one being merged, one being scored
         if (E.score_fn == SCORE_TRANSH) {
             E.p_opnd_n.alloc((size_t)(Qp + chunk) * Dp);
             E.p_cmat.alloc((size_t)Qp * chunk);
@@ -1539,9 +1549,12 @@ void run_predict(kge_engine& E, const Items& in) {
     std::vector<float> init_s((size_t)Q * nb, -1e6f), got_s((size_t)Q * nb);
     std::vector<uint32_t> init_i((size_t)Q * nb, 0u), got_i((size_t)Q * nb);
     const int64_t per_range = ((int64_t)E.n_entity - 1 + (int64_t)S - 1) / (int64_t)S;
+    const hipStream_t mst = E.merge_stream;
+    const size_t score_elems = (size_t)Qp * chunk;
     for (size_t ts = 0; ts < S; ++ts) {
-        HIP_CHECK(hipMemcpyAsync(E.p_best_s.p, init_s.data(), init_s.size() * 4, hipMemcpyHostToDevice, st));
-        HIP_CHECK(hipMemcpyAsync(E.p_best_i.p, init_i.data(), init_i.size() * 4, hipMemcpyHostToDevice, st));
+        // the n_best lists belong to the merge stream (the previous tail shard's read-back waited for it)
+        HIP_CHECK(hipMemcpyAsync(E.p_best_s.p, init_s.data(), init_s.size() * 4, hipMemcpyHostToDevice, mst));
+        HIP_CHECK(hipMemcpyAsync(E.p_best_i.p, init_i.data(), init_i.size() * 4, hipMemcpyHostToDevice, mst));
         int64_t lo, hi, table_off;
         if (E.shared_table) {
             lo = 1 + (int64_t)ts * per_range;
@@ -1550,12 +1563,24 @@ void run_predict(kge_engine& E, const Items& in) {
         } else {
             lo = 1; hi = 1 + (int64_t)count[ts]; table_off = (int64_t)ts * E.n_entity;
         }
-        for (int64_t r0 = lo; r0 < hi; r0 += chunk) {
+        int64_t n_chunk = 0;
+        for (int64_t r0 = lo; r0 < hi; r0 += chunk, ++n_chunk) {
             const int live = (int)std::min<int64_t>(chunk, hi - r0);
+            const int buf = (int)(n_chunk & 1);
+            float* scores = E.p_scores.p + (size_t)buf * score_elems;
             uint32_t* tail_idx = E.p_idx.p + Qp;
-            launch_row_range((uint32_t)(table_off + r0), live, chunk, tail_idx, st);
-            launch_gather_operands(rows_of(tail_idx, chunk, E.nets - 1), E.rel.p, nullptr, 0, 0, 0, chunk, Dp,
-                                   E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
+            RowSource tails;
+            if (!E.F && live == chunk) {
+                // a whole chunk of consecutive table rows needs no row list
+                tails.base = E.table.p + (table_off + r0) * E.L.pitch; tails.pitch = E.L.pitch;
+                tails.etype = E.L.emb_etype; tails.index = nullptr; tails.count = Dp; tails.vec = 1;
+            } else {
+                launch_row_range((uint32_t)(table_off + r0), live, chunk, tail_idx, st);
+                tails = rows_of(tail_idx, chunk, E.nets - 1);
+            }
+            launch_gather_operands(tails, E.rel.p, nullptr, 0, 0, 0, chunk, Dp, E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
+            // this buffer's previous scores (two chunks ago) must have been merged
+            if (n_chunk >= 2) HIP_CHECK(hipStreamWaitEvent(st, E.merged[buf], 0));
             if (transh) {  // transHScore (:551-565): c = n . tail, then the L1 part
                 HIP_CHECK(hipMemcpyAsync(E.p_opnd_n.p + (size_t)Qp * Dp, E.p_opnd.p + (size_t)Qp * Dp,
                                          (size_t)chunk * Dp * 4, hipMemcpyDeviceToDevice, st));
@@ -1563,16 +1588,20 @@ void run_predict(kge_engine& E, const Items& in) {
                                  false, st);
                 TranshFwd tf;
                 tf.sh = sh; tf.pt = E.p_opnd.p; tf.nt = E.p_opnd_n.p; tf.cmat = E.p_cmat.p; tf.clabel = nullptr;
-                tf.coef = E.p_scores.p; tf.dcm = nullptr; tf.loss_part = nullptr;
+                tf.coef = scores; tf.dcm = nullptr; tf.loss_part = nullptr;
                 launch_transh_fwd(tf, false, st);
             } else
-            launch_score_fwd(sh, dense, E.rel.p, nullptr, nullptr, E.p_scores.p, nullptr, nullptr, nullptr,
+            launch_score_fwd(sh, dense, E.rel.p, nullptr, nullptr, scores, nullptr, nullptr, nullptr,
                              false, st);
-            launch_topk_merge(E.p_scores.p, chunk, Q, live, (uint32_t)r0, (int)nb, E.p_best_s.p, E.p_best_i.p, st);
+            HIP_CHECK(hipEventRecord(E.scored[buf], st));
+            HIP_CHECK(hipStreamWaitEvent(mst, E.scored[buf], 0));
+            launch_topk_merge(scores, chunk, Q, live, (uint32_t)r0, (int)nb, E.p_best_s.p, E.p_best_i.p, mst);
+            HIP_CHECK(hipEventRecord(E.merged[buf], mst));
         }
         HIP_CHECK(hipGetLastError());
-        HIP_CHECK(hipMemcpyAsync(got_s.data(), E.p_best_s.p, got_s.size() * 4, hipMemcpyDeviceToHost, st));
-        HIP_CHECK(hipMemcpyAsync(got_i.data(), E.p_best_i.p, got_i.size() * 4, hipMemcpyDeviceToHost, st));
+        HIP_CHECK(hipMemcpyAsync(got_s.data(), E.p_best_s.p, got_s.size() * 4, hipMemcpyDeviceToHost, mst));
+        HIP_CHECK(hipMemcpyAsync(got_i.data(), E.p_best_i.p, got_i.size() * 4, hipMemcpyDeviceToHost, mst));
+        HIP_CHECK(hipStreamSynchronize(mst));
         HIP_CHECK(hipStreamSynchronize(st));
         for (size_t hs = 0; hs < S; ++hs) {
             std::memcpy(out_s + (hs * S + ts) * Hb * nb, got_s.data() + hs * Hb * nb, Hb * nb * 4);

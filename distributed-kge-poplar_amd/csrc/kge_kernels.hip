@@ -12,6 +12,8 @@
 #include "kge_kernels.h"
 
 #include <algorithm>
+#include <cstdint>
+#include <stdexcept>
 #include <type_traits>
 
 namespace kge {
@@ -2331,19 +2333,18 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
 // predict: running top-k over a stream of score chunks
 // (TopKCollector, src/poplar_kge.cpp:743-809).  One workgroup per query keeps
 // its n_best (score, index) pairs sorted by (score descending, index
-// ascending).  New scores are compared with the current n_best-th score a span
-// of 8192 at a time (32 per thread, loads back to back); the few that beat it
+// ascending).  New scores are compared with the current n_best-th score 16384
+// at a time (64 per thread, all loads in flight together); the few that beat it
 // are collected in LDS (in any order) and merged by rank: every element of
 // (current best, candidates) counts the candidates that come before it, a
 // candidate also finds its place among the sorted best by binary search, and
 // the elements whose rank is below n_best are written to that place.  The
 // order is total on distinct rows, so the result does not depend on the order
 // of collection, and ties resolve to the lower index whatever the chunking.
-// A span with more than 1024 candidates (the first rows of a sweep) is redone
-// 1024 scores at a time.
+// A pass with more than 1024 candidates is redone 1024 scores at a time.
 
 constexpr int TK_BLOCK = 1024;  // most n_best, and the candidate list's capacity
-constexpr int TK_SPAN = 8192;
+constexpr int TK_SPAN = 16384;
 
 DEVINL bool topk_before(float sa, uint32_t ia, float sb, uint32_t ib) {
     return sa > sb || (sa == sb && ia < ib);
@@ -2372,39 +2373,47 @@ __global__ __launch_bounds__(256) void k_topk_merge(const float* __restrict__ sc
     __syncthreads();
     bool changed = false;
     int pass = 0;
-    for (int span0 = 0; span0 < n_valid; span0 += TK_SPAN) {
-        const int span1 = min(n_valid, span0 + TK_SPAN);
-        int piece = TK_SPAN;
-        for (int base = span0; base < span1;) {
-            const int end = min(span1, base + piece);
+    // Scores per pass: TK_SPAN, all loads of a pass in flight together.  While the list still holds
+    // its initial entries (row 0, which never competes) every score is a candidate, so a sweep
+    // starts with 256 and doubles: each pass then brings about n_best * ln 2 candidates.
+    int piece = cur_i[n_best - 1] == 0u ? 256 : TK_SPAN;
+    {
+        for (int base = 0; base < n_valid;) {
+            const int end = min(n_valid, base + piece);
             const float kth = cur_s[n_best - 1];
             int* counter = &n_cand[pass % 3];
             if (tid == 0) n_cand[(pass + 1) % 3] = 0;
             ++pass;
-            for (int i0 = base; i0 < end; i0 += 256 * 8) {
-                float v[8];
+            constexpr int NV = TK_SPAN / 1024;
+            float4 v[NV];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int i = i0 + tid + 256 * j;
-                    v[j] = i < end ? row[i] : -INFINITY;
-                }
+            for (int j = 0; j < NV; ++j) {  // rows are 16-byte aligned and hold a multiple of 4 scores
+                const int i = base + 1024 * j + tid * 4;
+                v[j] = i < end ? *reinterpret_cast<const float4*>(row + i) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+            }
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (v[j] > kth) {  // false for NaN, and for -inf padding
+            for (int j = 0; j < NV; ++j) {
+                const float* vv = &v[j].x;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int i = base + 1024 * j + tid * 4 + e;
+                    if (i < end && vv[e] > kth) {  // false for NaN
                         const int slot = atomicAdd(counter, 1);
                         if (slot < TK_BLOCK) {
-                            cand_s[slot] = v[j];
-                            cand_i[slot] = first_index + (uint32_t)(i0 + tid + 256 * j);
+                            cand_s[slot] = vv[e];
+                            cand_i[slot] = first_index + (uint32_t)i;
                         }
                     }
+                }
             }
             __syncthreads();
             const int c = *counter;  // the same for every thread: all branches below are uniform
-            if (c > TK_BLOCK) {  // only a whole span can overflow: a piece of TK_BLOCK scores cannot
+            if (c > TK_BLOCK) {  // more than the list holds: the same scores again, TK_BLOCK at a time
                 piece = TK_BLOCK;
                 continue;
             }
             base = end;
+            piece = min(2 * piece, TK_SPAN);
             if (c == 0) continue;
             changed = true;
             // candidates padded to whole groups of four with entries that come before nothing
@@ -2470,6 +2479,7 @@ __global__ __launch_bounds__(256) void k_topk_merge(const float* __restrict__ sc
 
 void launch_topk_merge(const float* scores, int64_t ld, int n_queries, int n_valid, uint32_t first_index,
                        int n_best, float* best_score, uint32_t* best_index, hipStream_t stream) {
+    if ((ld & 3) || n_valid > ld || ((uintptr_t)scores & 15)) throw std::invalid_argument("top-k merge: score rows must be 16-byte aligned");
     hipLaunchKernelGGL(k_topk_merge, dim3(n_queries), dim3(256), 0, stream, scores, ld, n_valid, first_index,
                        n_best, best_score, best_index);
 }
