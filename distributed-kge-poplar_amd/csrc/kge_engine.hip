@@ -233,7 +233,8 @@ struct kge_engine {
     // predict: the n_best merge of one chunk of tails runs here while the next chunk is gathered
     // and scored on `stream` (the merge occupies one workgroup per query, a fraction of the chip)
     hipStream_t merge_stream = nullptr;
-    hipEvent_t scored[2] = {nullptr, nullptr}, merged[2] = {nullptr, nullptr};
+    static constexpr int kScoreBuffers = 3;  // a sweep's first merge (list still filling) takes three chunks' time
+    hipEvent_t scored[kScoreBuffers] = {}, merged[kScoreBuffers] = {};
     DevBuf<char> table;
     DevBuf<float> rel, rel_m, rel_v, proj, proj_m, proj_v;
     uint32_t step = 0;
@@ -1471,7 +1472,7 @@ void run_predict(kge_engine& E, const Items& in) {
         E.p_rel.alloc(Qp);
         E.p_count.alloc(1);
         E.p_opnd.alloc((size_t)(Qp + chunk) * Dp);
-        E.p_scores.alloc((size_t)2 * Qp * chunk);  // two chunks: one being merged, one being scored
+        E.p_scores.alloc((size_t)kge_engine::kScoreBuffers * Qp * chunk);  // chunks being merged and being scored
         if (E.score_fn == SCORE_TRANSH) {
             E.p_opnd_n.alloc((size_t)(Qp + chunk) * Dp);
             E.p_cmat.alloc((size_t)Qp * chunk);
@@ -1566,11 +1567,12 @@ void run_predict(kge_engine& E, const Items& in) {
         int64_t n_chunk = 0;
         for (int64_t r0 = lo; r0 < hi; r0 += chunk, ++n_chunk) {
             const int live = (int)std::min<int64_t>(chunk, hi - r0);
-            const int buf = (int)(n_chunk & 1);
+            const int buf = (int)(n_chunk % kge_engine::kScoreBuffers);
             float* scores = E.p_scores.p + (size_t)buf * score_elems;
             uint32_t* tail_idx = E.p_idx.p + Qp;
             RowSource tails;
-            if (!E.F && live == chunk) {
+            const bool whole = !E.F && live == chunk;
+            if (whole) {
                 // a whole chunk of consecutive table rows needs no row list
                 tails.base = E.table.p + (table_off + r0) * E.L.pitch; tails.pitch = E.L.pitch;
                 tails.etype = E.L.emb_etype; tails.index = nullptr; tails.count = Dp; tails.vec = 1;
@@ -1578,9 +1580,16 @@ void run_predict(kge_engine& E, const Items& in) {
                 launch_row_range((uint32_t)(table_off + r0), live, chunk, tail_idx, st);
                 tails = rows_of(tail_idx, chunk, E.nets - 1);
             }
-            launch_gather_operands(tails, E.rel.p, nullptr, 0, 0, 0, chunk, Dp, E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
-            // this buffer's previous scores (two chunks ago) must have been merged
-            if (n_chunk >= 2) HIP_CHECK(hipStreamWaitEvent(st, E.merged[buf], 0));
+            // such a chunk is scored where it lies (the tails take no relation); the others, and
+            // TransH's two operand matrices, go through the dense copy
+            const bool in_place = whole && !transh;
+            if (!in_place)
+                launch_gather_operands(tails, E.rel.p, nullptr, 0, 0, 0, chunk, Dp, E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
+            // this buffer's previous scores must have been merged
+            if (n_chunk >= kge_engine::kScoreBuffers) HIP_CHECK(hipStreamWaitEvent(st, E.merged[buf], 0));
+            if (in_place)
+                launch_score_fwd_rows(sh, dense, tails, scores, st);
+            else
             if (transh) {  // transHScore (:551-565): c = n . tail, then the L1 part
                 HIP_CHECK(hipMemcpyAsync(E.p_opnd_n.p + (size_t)Qp * Dp, E.p_opnd.p + (size_t)Qp * Dp,
                                          (size_t)chunk * Dp * 4, hipMemcpyDeviceToDevice, st));

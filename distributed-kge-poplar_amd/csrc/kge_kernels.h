@@ -145,6 +145,9 @@ void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, i
 void launch_score_fwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
                       const uint32_t* crel, const uint32_t* clabel, float* coef, float* dist,
                       uint32_t* nearflag, float* loss_part, bool fused_loss, hipStream_t stream);
+// raw scores of rows `a` against rows `b` of a second source (no relation, no loss): out [S, B, T]
+void launch_score_fwd_rows(const ScoreShape& sh, const RowSource& a, const RowSource& b, float* scores,
+                           hipStream_t stream);
 // words of the near-identical-pair flag matrix the L2 matrix-core path needs
 inline size_t nearflag_words(const ScoreShape& sh) {
     return (size_t)sh.S * ((sh.B + 31) / 32) * ((sh.T + 31) / 32);

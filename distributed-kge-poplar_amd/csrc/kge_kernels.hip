@@ -1275,6 +1275,21 @@ void launch_score_fwd(const ScoreShape& sh, const RowSource& ent, const float* r
     launch_fwd(p, stream);
 }
 
+// Raw scores of prepared rows `a` (rows 0 .. S*B) against rows `b` (rows 0 .. S*T) of another
+// source, e.g. consecutive rows of the table itself: no copy of the b side is made.
+void launch_score_fwd_rows(const ScoreShape& sh, const RowSource& a, const RowSource& b, float* scores,
+                           hipStream_t stream) {
+    FwdParams p;
+    p.nearflag = nullptr;
+    p.sh = sh;
+    if (sh.score_fn == SCORE_DISTMULT) p.sh.dist_fn = DIST_DOT;
+    p.ent_a = a; p.ent_b = b; p.rel = nullptr; p.crel = nullptr; p.clabel = nullptr;
+    p.coef = scores; p.dist = nullptr; p.loss_part = nullptr;
+    p.a_rel_mode = 0; p.out_mode = 1;
+    p.a_c0 = 0; p.b_c0 = 0;
+    launch_fwd(p, stream);
+}
+
 
 // --------------------------------------------------------------------------
 // bfloat16 matrix-core products (execution.scoring_dtype = "bfloat16"):
