@@ -167,7 +167,8 @@ def _random_queries(engine, n):
 
 @pytest.mark.parametrize("variant", ["demo_l1", "l2", "distmult", "complex", "rotate", "transh", "transh_big",
                                      "feature_mlp", "feature_dropout", "separate_networks_mlp",
-                                     "no_features_big", "n_best_max", "one_chunk"])
+                                     "no_features_big", "n_best_max", "one_chunk",
+                                     "l1_big", "distmult_big", "bf16_rows_big"])
 def test_predict_vs_brute_force(variant):
     """Engine.predict against a float64 brute force over every row of every shard
     (the reference checks shapes, ranges and ordering, tests/python/test_poplar_kge.py:155-175,
@@ -201,7 +202,7 @@ def test_predict_vs_brute_force(variant):
         settings.data.batch_size, ex.rw_batch_size = 6, 4096
         ex.predict_n_best = 1024 if variant == "n_best_max" else 100
         m.distance_fn = "L2"
-    elif variant in ("no_features_big", "transh_big"):
+    elif variant in ("no_features_big", "transh_big", "l1_big", "distmult_big", "bf16_rows_big"):
         # several chunks of tails per shard, several query chunks, ragged counts
         m.n_entity, m.entity_feature_size, m.embedding_size, m.n_shard = 20000, 0, 32, 3
         settings.data.batch_size, ex.rw_batch_size, ex.predict_n_best = 6, 4096, 20
@@ -209,6 +210,12 @@ def test_predict_vs_brute_force(variant):
         m.distance_fn = "L2"
         if variant == "transh_big":
             m.score_fn = "TransH"
+        elif variant == "l1_big":      # whole chunks are scored where they lie in the table: every
+            m.distance_fn = "L1"       # forward kernel family reads table rows as its tail operand
+        elif variant == "distmult_big":
+            m.score_fn, m.distance_fn = "DistMult", "MatMul"
+        elif variant == "bf16_rows_big":
+            ex.embedding_dtype = "bfloat16"
     settings.prepare()
     S = m.n_shard
     counts = np.array([m.n_entity - 1 - 7 * s for s in range(S)])
