@@ -146,3 +146,48 @@ def test_c4_float32_scoring_full_size_vs_oracle():
 
 def test_c5_full_size_vs_oracle():
     _run("c5", n_step=2)
+
+
+@pytest.mark.parametrize("distance_fn", ["L2", "L1"])
+def test_predict_full_size_vs_brute_force(distance_fn):
+    """Engine.predict over one shard's 1M-row table (fifteen whole chunks of tails scored
+    where they lie in the table, one partial chunk through the dense copy, the merge on its
+    own stream) against a float64 brute force over every row, for 128 queries and the
+    reference's n_best (src/python/poplar_kge.py:395-397; oracle tests/python/reference_model.py:169-206)."""
+    import gc
+
+    import poplar_kge as kge
+
+    gc.collect()
+    s = kge.Settings.create_demo()
+    s.seed = 4242
+    m, d, e = s.model, s.data, s.execution
+    m.score_fn, m.distance_fn, m.n_shard = "TransE", distance_fn, 1
+    m.n_entity, m.n_relation_type, m.embedding_size, m.entity_feature_size = 1_000_000, 1000, 256, 0
+    m.gamma, m.init_scale = 10.0, 16.0
+    d.batch_size, d.a2a_size = 256, 256
+    e.device, e.dtype, e.shared_table, e.rw_batch_size = "hip", "float32", False, 8192
+    e.train_steps_per_program_run, e.predict_hr_batch_size, e.predict_n_best = 1, 128, 100
+    settings = s.prepare()
+    count = m.n_entity - 12345   # the last rows of the table do not take part
+    engine = kge.Engine(settings, np.full(1, count))
+    bench.init_tables(engine, settings)
+    n = 128 + 7                  # a second, mostly empty program run
+    rng = np.random.default_rng(5)
+    queries = np.stack([np.zeros(n, np.uint32), rng.integers(1, count + 1, n).astype(np.uint32),
+                        rng.integers(0, m.n_relation_type, n).astype(np.uint32)], axis=-1)
+    found = engine.predict(queries)
+
+    D = m.embedding_size
+    table = bench.read_rows(engine, settings, np.arange(0, count + 1, dtype=np.uint32))[:, :D].astype(np.float64)
+    rel = engine.read_variable("relation_embedding").reshape(-1, D).astype(np.float64)
+    for q in range(0, n, 9):   # fifteen of the queries, both program runs
+        diff = (table[queries[q, 1]] + rel[queries[q, 2]])[None, :] - table[1:]
+        dist = np.sqrt(np.einsum("nd,nd->n", diff, diff)) if distance_fn == "L2" else np.abs(diff).sum(-1)
+        score = m.gamma - dist
+        order = np.lexsort((np.arange(count), -score))[:e.predict_n_best]
+        np.testing.assert_allclose(found.score[q], score[order], rtol=1e-5, atol=1e-5)
+        agree = found.shard_idx[q, :, 1] == order + 1
+        close = np.abs(found.score[q] - score[order]) <= 1e-5 * np.maximum(1.0, np.abs(score[order]))
+        assert np.all(agree | close) and agree.mean() > 0.97
+        assert np.all(found.shard_idx[q, :, 0] == 0)
