@@ -1582,7 +1582,10 @@ void run_predict(kge_engine& E, const Items& in) {
             }
             // such a chunk is scored where it lies (the tails take no relation); the others, and
             // TransH's two operand matrices, go through the dense copy
-            const bool in_place = whole && !transh;
+            // (16-bit rows on the matrix-core kernels too: their fast staging path takes float32 rows,
+            // and converting while copying costs less than the slower path does)
+            const bool in_place = whole && !transh &&
+                                  (E.L.emb_etype == ET_F32 || !E.use_mfma || (E.dist_fn == DIST_L1 && E.score_fn != SCORE_DISTMULT));
             if (!in_place)
                 launch_gather_operands(tails, E.rel.p, nullptr, 0, 0, 0, chunk, Dp, E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
             // this buffer's previous scores must have been merged
