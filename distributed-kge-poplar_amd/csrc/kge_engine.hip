@@ -300,6 +300,8 @@ struct kge_engine {
 
 namespace {
 
+// zeroed rows behind the table's last: predict scores whole tiles of 64 consecutive rows in place
+constexpr int64_t kSpareRows = 64;
 // the most contributions a row may have for the update's launch to sum it (launch_adam_rows_hot2)
 constexpr uint32_t kHotInUpdateMax = 4096;
 
@@ -557,7 +559,7 @@ void allocate(kge_engine& E) {
     for (auto& e : E.merged) HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
     const hipStream_t st = E.stream;
 
-    E.table.alloc((size_t)E.n_rows * E.L.pitch);
+    E.table.alloc((size_t)(E.n_rows + kSpareRows) * E.L.pitch);
     E.table.zero(st);
     const size_t rel_n = (size_t)E.n_rel_rows * E.Dp, proj_n = (size_t)E.Fp * E.Dp;
     for (DevBuf<float>* b : {&E.rel, &E.rel_m, &E.rel_v}) { b->alloc(rel_n); b->zero(st); }
@@ -1592,28 +1594,34 @@ void run_predict(kge_engine& E, const Items& in) {
             const int buf = (int)(n_chunk % kge_engine::kScoreBuffers);
             float* scores = E.p_scores.p + (size_t)buf * score_elems;
             uint32_t* tail_idx = E.p_idx.p + Qp;
+            // Consecutive table rows need no row list, and most are scored where they lie (the tails
+            // take no relation): the kernels take whole tiles of 64 rows, so a chunk's last tile may
+            // read up to 63 rows past the shard's count - rows of the table all the same (it ends in
+            // kSpareRows rows that belong to nobody), whose scores the merge never looks at.
+            // TransH's two operand matrices go through the dense copy, and so do 16-bit rows on the
+            // matrix-core kernels (their fast staging path takes float32 rows, and converting while
+            // copying costs less than the slower path does).
+            const int live_tiles = round_up(live, 64);
+            const bool in_place = !E.F && !transh &&
+                                  (E.L.emb_etype == ET_F32 || !E.use_mfma || (E.dist_fn == DIST_L1 && E.score_fn != SCORE_DISTMULT));
+            const int n_tail = in_place ? live_tiles : chunk;  // rows the scoring launch covers = the scores' row pitch
             RowSource tails;
-            const bool whole = !E.F && live == chunk;
-            if (whole) {
-                // a whole chunk of consecutive table rows needs no row list
+            if (!E.F && (in_place || live == chunk)) {
                 tails.base = E.table.p + (table_off + r0) * E.L.pitch; tails.pitch = E.L.pitch;
                 tails.etype = E.L.emb_etype; tails.index = nullptr; tails.count = Dp; tails.vec = 1;
             } else {
                 launch_row_range((uint32_t)(table_off + r0), live, chunk, tail_idx, st);
                 tails = rows_of(tail_idx, chunk, E.nets - 1);
             }
-            // such a chunk is scored where it lies (the tails take no relation); the others, and
-            // TransH's two operand matrices, go through the dense copy
-            // (16-bit rows on the matrix-core kernels too: their fast staging path takes float32 rows,
-            // and converting while copying costs less than the slower path does)
-            const bool in_place = whole && !transh &&
-                                  (E.L.emb_etype == ET_F32 || !E.use_mfma || (E.dist_fn == DIST_L1 && E.score_fn != SCORE_DISTMULT));
             if (!in_place)
                 launch_gather_operands(tails, E.rel.p, nullptr, 0, 0, 0, chunk, Dp, E.p_opnd.p + (size_t)Qp * Dp, nullptr, st);
             // this buffer's previous scores must have been merged
             if (n_chunk >= kge_engine::kScoreBuffers) HIP_CHECK(hipStreamWaitEvent(st, E.merged[buf], 0));
-            if (in_place)
-                launch_score_fwd_rows(sh, dense, tails, scores, st);
+            if (in_place) {
+                ScoreShape shp = sh;
+                shp.T = n_tail;
+                launch_score_fwd_rows(shp, dense, tails, scores, st);
+            }
             else
             if (transh) {  // transHScore (:551-565): c = n . tail, then the L1 part
                 HIP_CHECK(hipMemcpyAsync(E.p_opnd_n.p + (size_t)Qp * Dp, E.p_opnd.p + (size_t)Qp * Dp,
@@ -1629,7 +1637,7 @@ void run_predict(kge_engine& E, const Items& in) {
                              false, st);
             HIP_CHECK(hipEventRecord(E.scored[buf], st));
             HIP_CHECK(hipStreamWaitEvent(mst, E.scored[buf], 0));
-            launch_topk_merge(scores, chunk, Q, live, (uint32_t)r0, (int)nb, E.p_best_s.p, E.p_best_i.p, mst);
+            launch_topk_merge(scores, n_tail, Q, live, (uint32_t)r0, (int)nb, E.p_best_s.p, E.p_best_i.p, mst);
             HIP_CHECK(hipEventRecord(E.merged[buf], mst));
         }
         HIP_CHECK(hipGetLastError());
