@@ -540,6 +540,8 @@ def test_engine_errors():
         libpoplar_kge.Engine({**s, "model.gamma": "two"}, "")
     with pytest.raises(ValueError, match="not divisible by n_shard"):
         libpoplar_kge.Engine({**s, "model.n_relation_type": 13}, "")
+    with pytest.raises(ValueError, match="predict_chunk_rows"):
+        libpoplar_kge.Engine({**s, "execution.predict_chunk_rows": 10}, "")
     engine = libpoplar_kge.Engine(s, "")
     with pytest.raises(ValueError, match="Unknown command"):
         engine.run("fly", {})
