@@ -191,3 +191,43 @@ def test_predict_full_size_vs_brute_force(distance_fn):
         close = np.abs(found.score[q] - score[order]) <= 1e-5 * np.maximum(1.0, np.abs(score[order]))
         assert np.all(agree | close) and agree.mean() > 0.97
         assert np.all(found.shard_idx[q, :, 0] == 0)
+
+
+def test_predict_shared_table_vs_brute_force():
+    """`predict` with one table shared by the blocks (this build's layout for the benchmark
+    shapes): the table is swept in n_shard contiguous row ranges, the returned rows are table
+    rows, and the ranges' n_best pooled give the overall n_best of a float64 brute force."""
+    import gc
+
+    import poplar_kge as kge
+
+    gc.collect()
+    w = dict(bench.WORKLOADS["c2"], n_entity=50_000, blocks=4, n_relation=40, dim=64, batch=32, tails=32)
+    settings = bench.make_settings(w, 1, kge)
+    m, e = settings.model, settings.execution
+    e.predict_hr_batch_size, e.predict_n_best, e.predict_chunk_rows = 16, 50, 4096
+    S, Hb, nb, D = m.n_shard, 16, 50, m.embedding_size
+    count = m.n_entity - 77
+    engine = kge.Engine(settings, np.full(S, count))
+    bench.init_tables(engine, settings)
+    rng = np.random.default_rng(11)
+    head = rng.integers(1, count + 1, (S, Hb)).astype(np.uint32)
+    relation = rng.integers(0, m.n_relation_type, (S, Hb)).astype(np.uint32)
+    scores = np.full((S, S, Hb, nb), np.nan, np.float32)
+    rows = np.zeros(scores.shape, np.uint32)
+    engine.engine.run("predict", dict(predict_head=head, predict_relation=relation,
+                                      predict_entity_count=np.full(S, count, np.uint32),
+                                      predict_scores=scores, predict_indices=rows))
+    table = bench.read_rows(engine, settings, np.arange(0, count + 1, dtype=np.uint32))[:, :D].astype(np.float64)
+    rel = engine.read_variable("relation_embedding").reshape(-1, D).astype(np.float64)
+    per_range = -(-(m.n_entity - 1) // S)
+    for s in range(S):
+        for q in range(0, Hb, 5):
+            diff = (table[head[s, q]] + rel[relation[s, q]])[None, :] - table[1:]
+            score = m.gamma - np.sqrt(np.einsum("nd,nd->n", diff, diff))
+            for ts in range(S):   # each range's own n_best, rows inside the range
+                lo, hi = 1 + ts * per_range, min(1 + (ts + 1) * per_range, count + 1)
+                assert np.all((rows[s, ts, q] >= lo) & (rows[s, ts, q] < hi))
+                order = lo + np.lexsort((np.arange(hi - lo), -score[lo - 1:hi - 1]))[:nb]
+                np.testing.assert_allclose(scores[s, ts, q], score[order - 1], rtol=1e-5, atol=1e-5)
+                assert np.mean(rows[s, ts, q] == order) > 0.95
