@@ -651,18 +651,15 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
     const int B = sh.B, T = sh.T, Dp = sh.Dp;
     if (OM == 0 && tid < kScoreTile) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
 
-    // staging assignment: row lr (+32) of each operand, float4 column k4
-    const int lr = tid >> 3, k4 = (tid & 7) * 4;
-    const char* arow[2];
-    const char* brow[2];
-    const float* rrow[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int m = m0 + lr + 32 * h, n = n0 + lr + 32 * h;
-        arow[h] = m < B ? row_ptr(p.ent_a, p.a_c0 + d * B + m) : nullptr;
-        rrow[h] = (m < B && p.a_rel_mode) ? p.rel + (size_t)p.crel[d * B + m] * Dp : nullptr;
-        brow[h] = n < T ? row_ptr(p.ent_b, p.b_c0 + d * T + n) : nullptr;
-    }
+    // staging assignment: row lr of each operand, float4 columns k4 and k4 + 16.  Sixteen
+    // consecutive rows per wave and four column groups: a store instruction's 64 lanes fall on
+    // every LDS bank exactly twice (with eight column groups per row they met four to a bank).
+    static_assert(BK == 32 && kScoreTile == 64, "the staging assignment covers 64 rows x 32 columns");
+    const int lr = tid >> 2, k4 = (tid & 3) * 4;
+    const int sm = m0 + lr, sn = n0 + lr;
+    const char* arow = sm < B ? row_ptr(p.ent_a, p.a_c0 + d * B + sm) : nullptr;
+    const float* rrow = (sm < B && p.a_rel_mode) ? p.rel + (size_t)p.crel[d * B + sm] * Dp : nullptr;
+    const char* brow = sn < T ? row_ptr(p.ent_b, p.b_c0 + d * T + sn) : nullptr;
 
     float acc[4][4];
 #pragma unroll
@@ -671,17 +668,16 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
         for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
 
     for (int k0 = 0; k0 < Dp; k0 += BK) {
-        const int k = k0 + k4;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
+            const int kc = 16 * h + k4, k = k0 + kc;
             float4 a = make_float4(0, 0, 0, 0), b = a;
             if (k < Dp) {
-                if (arow[h]) a = combine_rel(load4(arow[h], k, p.ent_a), rrow[h], k, p.a_rel_mode);
-                if (brow[h]) b = load4(brow[h], k, p.ent_b);
+                if (arow) a = combine_rel(load4(arow, k, p.ent_a), rrow, k, p.a_rel_mode);
+                if (brow) b = load4(brow, k, p.ent_b);
             }
-            const int r = lr + 32 * h;
-            As[k4 + 0][r] = a.x; As[k4 + 1][r] = a.y; As[k4 + 2][r] = a.z; As[k4 + 3][r] = a.w;
-            Bs[k4 + 0][r] = b.x; Bs[k4 + 1][r] = b.y; Bs[k4 + 2][r] = b.z; Bs[k4 + 3][r] = b.w;
+            As[kc + 0][lr] = a.x; As[kc + 1][lr] = a.y; As[kc + 2][lr] = a.z; As[kc + 3][lr] = a.w;
+            Bs[kc + 0][lr] = b.x; Bs[kc + 1][lr] = b.y; Bs[kc + 2][lr] = b.z; Bs[kc + 3][lr] = b.w;
         }
         __syncthreads();
 #pragma unroll
