@@ -13,10 +13,15 @@ back and the stream synchronised.  Prints ONE JSON line.
 Extra objects in that line:
   roofline      the kernel with the largest share of the step time: algorithmic
                 bytes or flops per launch over its mean launch duration, measured
-                with HIP events on the engine's stream in a second (untimed) pass
+                with HIP events on the engine's stream in a second (untimed) pass;
+                `traffic` = its HBM-side bytes per launch from the committed counter
+                summary named in `traffic_source` (null without one)
   kernels       the same figures for every kernel of the step
-  cpu_baseline  the sequential float32 CPU oracle on the first steps of the same
-                workload, on this host's cores (1 thread)
+  cpu_baseline  the reference's CPU path (its PyTorch demo step: fancy-index gather,
+                torch.cdist, autograd, Adam on the gathered rows) on the first steps of
+                the same workload, all of this host's threads, a bounded sample
+  cpu_baseline_port  the sequential float32 C port of the step (1 thread), ~15 s
+  workloads     the same measurement on the 22.8M-row (L2 and L1) and 91.2M-row tables
   host_batches  the same steps with the index arrays handed over as host buffers
                 every call (PCIe-inclusive; never the headline value)
   copy_calibration  one plain row copy much larger than the caches, whose known
@@ -33,114 +38,42 @@ from pathlib import Path
 import numpy as np
 
 ROOT = Path(__file__).resolve().parent
-for p in (ROOT, ROOT / "distributed-kge-poplar_amd", ROOT / "tests"):
+for p in (ROOT, ROOT / "distributed-kge-poplar_amd"):
     sys.path.insert(0, os.fspath(p))
 
-# Synthetic workloads (ids Zipf s=1.1 over 1..N-1, relations uniform, one shared
-# table addressed by K blocks = K virtual shards).  c2 is the configuration the
-# headline metric is quoted on.
-WORKLOADS = {
-    "c1": dict(desc="TransE-L2 D=64 fp32, 10k entities, 1 block x (256 positives, 64 shared tails)",
-               n_entity=10_000, n_relation=50, dim=64, blocks=1, batch=256, tails=64,
-               distance_fn="L2", uniform=True),
-    "c2": dict(desc="TransE-L2 D=256 fp32, 1M entities, 32 blocks x (256 positives, 256 shared tails)",
-               n_entity=1_000_000, n_relation=1000, dim=256, blocks=32, batch=256, tails=256,
-               distance_fn="L2"),
-    "c3": dict(desc="TransE-L1 D=256 fp32, 22.8M entities, 64 blocks x (256 positives, 512 shared tails)",
-               n_entity=22_800_000, n_relation=1387, dim=256, blocks=64, batch=256, tails=512,
-               distance_fn="L1"),
-    "c3l2": dict(desc="TransE-L2 D=256 fp32, 22.8M entities, 64 blocks x (256 positives, 512 shared tails)",
-                 n_entity=22_800_000, n_relation=1387, dim=256, blocks=64, batch=256, tails=512,
-                 distance_fn="L2"),
-    "c4": dict(desc="DistMult D=512 + 768-dim fp16 feature projected 768->512, 4M entities, "
-                    "1 block x (8192 positives, 2048 shared tails), softmax CE",
-               n_entity=4_000_000, n_relation=1387, dim=512, blocks=1, batch=8192, tails=2048,
-               score_fn="DistMult", distance_fn="MatMul", loss="softmax", feature=768,
-               feature_dtype="float16", scoring_dtype="bfloat16"),
-    "c5": dict(desc="TransE-L2 D=256 bf16 embedding + fp32 moments, 91.2M entities, "
-                    "32 blocks x (512 positives, 512 shared tails)",
-               n_entity=91_200_000, n_relation=1387, dim=256, blocks=32, batch=512, tails=512,
-               distance_fn="L2", embedding_dtype="bfloat16"),
-}
+from kge_synthetic import WORKLOADS, init_tables, make_batch, make_settings, read_rows, row_bytes  # noqa: E402
 
 PEAK_HBM_GBPS = 8000.0
 PEAK_FP32_TFLOPS = 157.3
 PEAK_BF16_TFLOPS = 2500.0
 
-# HBM bytes per launch (fetched + written) of the dominant kernel, from two
-# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each
-# scaled by what the same counter reads for the calibration copy below.
-# Counters cannot be read from inside this process, so the figures are carried
-# here and refreshed together with the committed profiler summaries.
-MEASURED_TRAFFIC_BYTES = {
-    ("c2", "score_bwd"): 41.9e6,     # 25.1 MB fetched + 16.8 MB written
-    ("c3l2", "score_bwd"): 215.5e6,  # 165.1 MB fetched + 50.3 MB written
-}
+# kernels of the step by the names the profiler summaries list them under
+KERNEL_SYMBOLS = {"gather_operands": "k_gather_operands", "score_fwd": "k_score_fwd", "score_bwd": "k_score_bwd",
+                  "reduce_entity": "k_reduce_chunks", "adam_entity": "k_adam_rows", "loss_rows": "k_loss_rows"}
 
 
-def make_settings(w, n_step, kge):
-    s = kge.Settings.create_demo()
-    s.seed = 20240611
-    m, d, t, e = s.model, s.data, s.training, s.execution
-    m.score_fn, m.distance_fn = w.get("score_fn", "TransE"), w["distance_fn"]
-    m.n_shard, m.n_entity, m.n_relation_type = w["blocks"], w["n_entity"], w["n_relation"]
-    m.embedding_size, m.entity_feature_size, m.gamma = w["dim"], w.get("feature", 0), 10.0
-    m.init_scale = float(np.sqrt(w["dim"]))  # embeddings ~ N(0, 1/sqrt(D)): sigma = init_scale / D
-    d.batch_size, d.a2a_size = w["batch"], w["tails"] // w["blocks"]
-    t.learning_rate = 1e-3
-    t.loss = kge.SoftmaxLoss(correction_weight=1.0) if w.get("loss") == "softmax" else kge.LogSigmoidLoss()
-    e.device, e.dtype, e.shared_table = "hip", "float32", True
-    e.embedding_dtype, e.feature_dtype = w.get("embedding_dtype"), w.get("feature_dtype")
-    e.scoring_dtype = w.get("scoring_dtype")
-    e.train_steps_per_program_run = n_step
-    e.rw_batch_size = 8192
-    return s.prepare()
-
-
-def make_batch(w, n_step, kge, K):
-    """Raw ids with identity slot maps: every block lists its heads then the
-    tails it contributes; the device does all the de-duplication."""
-    c = dict(n_shard=w["blocks"], n_entity=w["n_entity"], batch=w["batch"],
-             a2a=w["tails"] // w["blocks"], n_relation=w["n_relation"])
-    rng = np.random.Generator(np.random.PCG64(20240611 + 1))
-    return kge.Batch(**K.raw_batch(c, n_step, rng, zipf=not w.get("uniform", False)))
-
-
-def init_tables(engine, settings):
-    """write_entity over the whole table (random-normal embeddings drawn on the
-    device).  The table is shared, so each of the n_shard index rows of one call
-    covers a different range of table rows."""
-    engine.initialise_variables()
-    m, e = settings.model, settings.execution
-    per_call = m.n_shard * e.rw_batch_size
-    feat = np.zeros(settings.entity_data_w_shape, np.float32)
-    if m.entity_feature_size:
-        # N(0, 1) features; one block of them serves every call (rows per_call apart share features)
-        feat = np.random.default_rng(settings.seed + 5).normal(size=feat.shape).astype(np.float32)
-    for off in range(0, m.n_entity, per_call):
-        idx = np.arange(off, off + per_call, dtype=np.int64)
-        idx[idx >= m.n_entity] = 0
-        engine.engine.run("write_entity", dict(
-            write_indices=idx.astype(np.uint32).reshape(m.n_shard, -1), write_features=feat))
-    # row 0 last, so that the overflow of the final chunk does not decide its content
-    idx = np.zeros(per_call, np.uint32)
-    engine.engine.run("write_entity", dict(write_indices=idx.reshape(m.n_shard, -1), write_features=feat))
-    engine.uninitialized_entity_data[:] = False
-
-
-def read_rows(engine, settings, ids):
-    """Rows `ids` of the shared table as float32 [len(ids), 3D+F] (read_entity)."""
-    m, e = settings.model, settings.execution
-    per_call = m.n_shard * e.rw_batch_size
-    out = np.zeros((len(ids), settings.entity_data_r_size), np.float32)
-    for off in range(0, len(ids), per_call):
-        chunk = ids[off:off + per_call]
-        idx = np.zeros(per_call, np.uint32)
-        idx[:len(chunk)] = chunk
-        data = np.zeros(settings.entity_data_r_shape, np.float32)
-        engine.engine.run("read_entity", dict(read_indices=idx.reshape(m.n_shard, -1), read_data=data))
-        out[off:off + len(chunk)] = data.reshape(per_call, -1)[:len(chunk)]
-    return out
+def measured_traffic(workload):
+    """HBM-side bytes per launch (fetched + written) of every step kernel, read from the committed
+    summary of two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, each scaled
+    by what the same counter reads for the calibration copy).  Counters cannot be read from inside
+    this process; the summary names the command it came from.  None when there is no summary."""
+    path = ROOT / "profiles" / f"{workload}_step_hbm_traffic.md"
+    if not path.exists():
+        return None, None
+    table = {}
+    for line in path.read_text().splitlines():
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) == 5 and cells[0].startswith("`"):
+            try:
+                table[cells[0].strip("`")] = (float(cells[3]) + float(cells[4])) * 1e6
+            except ValueError:
+                pass
+    out = {}
+    for name, symbol in KERNEL_SYMBOLS.items():
+        hits = [v for k, v in table.items() if symbol in k]
+        if hits:
+            out[name] = max(hits)  # variants of one kernel (e.g. with and without hot rows): the one that ran most
+    return out, f"profiles/{path.name}"
 
 
 def cpu_start_state(engine, settings, w, sub):
@@ -212,28 +145,29 @@ def cpu_torch_prepare(engine, settings, w, batch, n_max, threads):
 
 
 def cpu_torch_run(prepared, settings, n_check, budget_s=10.0):
-    """One untimed step to start the thread pool, then steps until `budget_s` seconds have gone
-    (at most the prepared ones).  Returns (json object, mean loss of the first n_check steps)."""
+    """One untimed step to start the thread pool, then steps until `budget_s` seconds have gone,
+    going round the prepared steps as often as that takes (the state keeps evolving; only the
+    first pass's losses are compared).  Returns (json object, mean loss of the first n_check steps)."""
     path, sub, threads = prepared
     m, d = settings.model, settings.data
     lr = settings.training.learning_rate
-    losses, dt, n = [], 0.0, 0
-    for i in range(sub["remote"].shape[1]):
+    n_prepared = sub["remote"].shape[1]
+    losses, dt, n, i = [], 0.0, 0, 0
+    while dt <= budget_s and n < 100000:
         t0 = time.perf_counter()
-        losses.append(path.step(lr, {k: v[:, i] for k, v in sub.items()}))
+        loss = path.step(lr, {k: v[:, i % n_prepared] for k, v in sub.items()})
         if i > 0:
             dt += time.perf_counter() - t0
             n += 1
-        if dt > budget_s:
-            break
-    if n == 0:
-        return None, None
+        if i < n_prepared:
+            losses.append(loss)
+        i += 1
     triples = n * m.n_shard * d.batch_size
     loss = np.mean(losses[:n_check], axis=0) if len(losses) >= n_check else None
     return dict(value=triples / dt, unit="triples/s", cores=threads, kind="port",
-                sample=f"{n} step(s) of the same workload ({triples} triples) in {dt:.1f} s after one "
-                       f"untimed step, float32 PyTorch demo path, {threads} threads of "
-                       f"{os.cpu_count()} host cpus"), loss
+                sample=f"{n} step(s) of the same workload ({triples} triples; the first {n_prepared} steps' "
+                       f"index arrays, repeated) in {dt:.1f} s after one untimed step, float32 PyTorch demo "
+                       f"path, {threads} threads of {os.cpu_count()} host cpus"), loss
 
 
 def split_forward(w):
@@ -402,74 +336,49 @@ def predict_bench(args, w, kge, torch):
         check=dict(recomputed_score_rel_err=err, queries_checked=nq))))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--mode", default="train", choices=["train", "predict"],
-                    help="train: the training step (the headline metric); predict: the all-entity scoring sweep")
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-steps", type=int, default=None,
-                    help="steps the CPU baseline times (default: sized for ~10-30 s)")
-    ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--n-entity", type=int, default=None, help="override the table size (experiments)")
-    ap.add_argument("--predict-chunk-rows", type=int, default=None,
-                    help="--mode predict: tails scored per launch (experiments; default: the engine's)")
-    ap.add_argument("--scoring", default=None, choices=["mfma", "mfma_bf16x3", "valu"], help="scoring kernels (default mfma_bf16x3)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py measures one GPU holding one shard's whole table: --gpus must be 1 "
-                 "(the step has no collectives; nothing here uses a second GPU)")
-    if args.steps < 1 or args.warmup < 0:
-        sys.exit("--steps must be >= 1 and --warmup >= 0")
-
-    import torch  # device discovery only; all device memory is the engine's own
-
-    if not torch.cuda.is_available():
-        sys.exit("no HIP device visible")
-    import kge_cases as K
-    import poplar_kge as kge
-
-    w = dict(WORKLOADS[args.workload])
-    if args.n_entity:
+def measure(name, args, kge, torch, full):
+    """One workload: W untimed warm-up steps, exactly K timed steps (one `train_step_loop` call over
+    index arrays resident in HBM, plan phase included, device idle on both sides), then the same K
+    steps once more with an event pair around every kernel.  With `full` also the CPU baselines,
+    the stand-alone gather, the calibration copy and the host-buffer variant."""
+    w = dict(WORKLOADS[name])
+    if args.n_entity and full:
         w["n_entity"] = args.n_entity
         w["desc"] += f" [table size overridden: {args.n_entity}]"
-    if args.mode == "predict":
-        if w.get("feature") or w.get("score_fn", "TransE") != "TransE":
-            sys.exit("--mode predict covers the TransE workloads without features")
-        return predict_bench(args, w, kge, torch)
+    if args.scoring:
+        w["scoring"] = args.scoring
     n_total = args.warmup + args.steps
     settings = make_settings(w, n_total, kge)
-    if args.scoring:
-        settings.execution.scoring = w["scoring"] = args.scoring
     m, d = settings.model, settings.data
     engine = kge.Engine(settings, np.full(m.n_shard, m.n_entity - 1))
     init_tables(engine, settings)
-    batch = make_batch(w, n_total, kge, K)
+    batch = make_batch(w, n_total, kge)
     engine.stage_batch(batch)
 
-    # CPU baseline on the first steps, from the same initial state the GPU starts from
-    # (about 15 s of CPU work: ~2e9 pair-dims per second for the whole step on one core)
+    # CPU baselines on the first steps, from the same initial state the GPU starts from.  The C
+    # port: about 15 s of work on one core (~2e9 pair-dims per second for the whole step).
     pair_dims = m.n_shard * d.batch_size * settings.n_tail * m.embedding_size
     n_cpu = args.cpu_steps or int(np.clip(round(15 * 2e9 / pair_dims), 1, n_total))
     n_cpu = min(n_cpu, n_total)
     n_check = max(1, min(n_cpu, args.warmup))
-    cpu, cpu_loss = (None, None) if args.no_cpu else cpu_baseline(engine, settings, w, batch, n_check, n_cpu)
+    with_cpu = not args.no_cpu and (full or name in args.cpu_workloads)
+    port, port_loss = cpu_baseline(engine, settings, w, batch, n_check, n_cpu) if with_cpu and full else (None, None)
     # the worker threads this process may use: the host's share for one GPU, not the node's core count
     threads = int(os.environ.get("OMP_NUM_THREADS") or min(16, os.cpu_count()))
-    torch_path = None if args.no_cpu else cpu_torch_prepare(engine, settings, w, batch, n_total, threads)
+    torch_path = cpu_torch_prepare(engine, settings, w, batch, n_total, threads) if with_cpu else None
 
-    # warm-up: W untimed steps; the first n_cpu of them double as the parity check
+    # warm-up: W untimed steps; the first n_check of them double as the parity check
     check = None
     done = 0
     if args.warmup > 0:
-        first = n_check if cpu is not None else args.warmup
+        first = n_check if with_cpu else args.warmup
         loss, _ = engine.train_step_loop(None, step_begin=0, step_count=first)
         done = first
-        if cpu is not None:
-            check = dict(gpu_loss=loss, cpu_loss=float(np.sum(cpu_loss)),
-                         rel_err=abs(loss - float(np.sum(cpu_loss))) / abs(float(np.sum(cpu_loss))))
+        if with_cpu:
+            check = dict(gpu_loss=loss)
+            if port is not None:
+                check.update(cpu_port_loss=float(np.sum(port_loss)),
+                             cpu_port_rel_err=abs(loss - float(np.sum(port_loss))) / abs(float(np.sum(port_loss))))
         if args.warmup > done:
             engine.train_step_loop(None, step_begin=done, step_count=args.warmup - done)
 
@@ -486,86 +395,170 @@ def main():
     engine.train_step_loop(None, step_begin=args.warmup, step_count=args.steps, profile_kernels=True)
     prof = engine.timing()
     kernels = kernel_table(w, prof, args.steps, uniq_rows)
+    traffic, traffic_source = measured_traffic(name)
+    for k, v in kernels.items():
+        v["traffic"] = traffic.get(k) if traffic else None
     step_kernels = {k: v for k, v in kernels.items() if k != "plan"}
     dominant = max(step_kernels, key=lambda k: step_kernels[k]["ms_per_step"])
     dom = kernels[dominant]
     roofline = dict(kernel=dominant, bound=dom["bound"], achieved=dom["achieved"], peak=dom["peak"],
-                    unit=dom["unit"], frac=dom["frac"], traffic=None,
+                    unit=dom["unit"], frac=dom["frac"], traffic=dom["traffic"], traffic_source=traffic_source,
                     launch_ms=dom["ms_per_step"] / dom["launches_per_step"])
 
-    # stand-alone row gather (fr::Buffer::read) over one step's distinct rows
-    ids = np.unique(batch.remote[:, args.warmup]).astype(np.uint32)
-    gms = np.zeros(1, np.float32)
-    engine.engine.run("gather_benchmark", dict(indices=ids, ms=gms, repeats=20))
-    row_bytes = ((2 if w.get("embedding_dtype") == "bfloat16" else 4) * m.embedding_size + 8 * m.embedding_size
-                 + (2 if w.get("feature_dtype") == "float16" else 4) * m.entity_feature_size)
-    gather = dict(rows=int(ids.size), ms=float(gms[0]),
-                  achieved=2 * ids.size * row_bytes / (gms[0] * 1e-3) / 1e9, unit="GB/s (read + write)")
-
-    # one large plain copy (distinct rows, > 1 GB each way): scales the profiler's byte counters
-    n_cal = min(m.n_entity - 1, 400_000)
-    cal_ids = (1 + np.random.default_rng(5).permutation(m.n_entity - 1)[:n_cal]).astype(np.uint32)
-    engine.engine.run("gather_benchmark", dict(indices=cal_ids, ms=gms, repeats=1))
-    calibration = dict(kernel="k_rows_copy", rows=int(n_cal), bytes_read=int(n_cal * row_bytes),
-                       bytes_written=int(n_cal * row_bytes), ms=float(gms[0]),
-                       achieved=2 * n_cal * row_bytes / (gms[0] * 1e-3) / 1e9, unit="GB/s (read + write)")
-
-    # one call over all W + K steps with the index arrays passed as host buffers
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    engine.train_step_loop(batch)
-    torch.cuda.synchronize()
-    dt_host = (time.perf_counter() - t1) / n_total
-
-    # the multi-threaded CPU path last: nothing of the device is timed after it
-    cpu_torch, cpu_torch_loss = cpu_torch_run(torch_path, settings, n_check) if torch_path else (None, None)
-    if check is not None and cpu_torch_loss is not None:
-        check["cpu_torch_loss"] = float(np.sum(cpu_torch_loss))
-        check["cpu_torch_rel_err"] = (abs(check["gpu_loss"] - check["cpu_torch_loss"])
-                                      / abs(check["cpu_torch_loss"]))
-
     triples = args.steps * m.n_shard * d.batch_size
-    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get((args.workload, dominant))
     U = float(np.mean(uniq_rows))
     R = m.n_shard * settings.n_remote
-    step_bytes = (U * 2 * row_bytes + 4 * (R + 2 * m.n_shard * d.batch_size) + 4 * U
+    rb = row_bytes(w)
+    step_bytes = (U * 2 * rb + 4 * (R + 2 * m.n_shard * d.batch_size) + 4 * U
                   + 2 * 3 * m.n_relation_type * m.embedding_size * 4)
+    step_traffic = sum(v for k, v in traffic.items() if k in step_kernels) if traffic else None
     out = {
-        "metric": "train triples/sec (fwd+bwd+sparse Adam) at dim 256; achieved HBM GB/s",
         "value": triples / dt,
         "unit": "triples/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
         "ms_per_step": dt / args.steps * 1e3,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
         "dtype": ("bf16 scoring operands / f32 accumulate" if w.get("scoring_dtype") == "bfloat16" else
                   "bf16 rows / f32 math" if w.get("embedding_dtype") == "bfloat16" else "f32"),
-        "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {w['desc']}; Zipf s=1.1 ids, "
+        "config": {"workload": f"{name}: {w['desc']}; {'uniform' if w.get('uniform') else 'Zipf s=1.1'} ids, "
                                f"{w.get('loss', 'logsigmoid')} loss, "
                                f"Adam lr 1e-3, raw ids de-duplicated on the device",
                    "positives_per_step": m.n_shard * d.batch_size, "row_refs_per_step": R,
                    "unique_rows_per_step": U},
         "step_hbm": {"algorithmic_bytes_per_step": step_bytes,
-                     "achieved": step_bytes / (dt / args.steps) / 1e9, "unit": "GB/s"},
+                     "achieved": step_bytes / (dt / args.steps) / 1e9, "unit": "GB/s",
+                     "traffic_per_step": step_traffic,
+                     "traffic_over_algorithmic": step_traffic / step_bytes if step_traffic else None,
+                     "traffic_source": traffic_source},
         "device_ms": {"plan_per_step": timing["plan_ms"] / args.steps,
                       "kernels_per_step": timing["steps_ms"] / args.steps},
         "loss": loss,
         "roofline": roofline,
         "kernels": kernels,
-        "row_gather": gather,
-        "copy_calibration": calibration,
-        "host_batches": {"value": m.n_shard * d.batch_size / dt_host, "unit": "triples/s",
-                         "ms_per_step": dt_host * 1e3,
-                         "note": f"one call over {n_total} steps, index arrays uploaded from host "
-                                 "memory inside the timed call"},
-        "cpu_baseline": cpu,
-        "cpu_baseline_torch": cpu_torch,
-        "check": check,
     }
+    if full:
+        # stand-alone row gather (fr::Buffer::read) over one step's distinct rows
+        ids = np.unique(batch.remote[:, args.warmup]).astype(np.uint32)
+        gms = np.zeros(1, np.float32)
+        engine.engine.run("gather_benchmark", dict(indices=ids, ms=gms, repeats=20))
+        out["row_gather"] = dict(rows=int(ids.size), ms=float(gms[0]),
+                                 achieved=2 * ids.size * rb / (gms[0] * 1e-3) / 1e9, unit="GB/s (read + write)",
+                                 note="working set of a few tens of MB: served by the caches, not an HBM figure")
+        # one large plain copy (distinct rows, > 1 GB each way): scales the profiler's byte counters,
+        # and is the HBM bandwidth a plain streaming kernel reaches on this device
+        n_cal = min(m.n_entity - 1, 400_000)
+        cal_ids = (1 + np.random.default_rng(5).permutation(m.n_entity - 1)[:n_cal]).astype(np.uint32)
+        engine.engine.run("gather_benchmark", dict(indices=cal_ids, ms=gms, repeats=1))
+        out["copy_calibration"] = dict(kernel="k_rows_copy", rows=int(n_cal), bytes_read=int(n_cal * rb),
+                                       bytes_written=int(n_cal * rb), ms=float(gms[0]),
+                                       achieved=2 * n_cal * rb / (gms[0] * 1e-3) / 1e9, unit="GB/s (read + write)")
+        # one call over all W + K steps with the index arrays passed as host buffers
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        engine.train_step_loop(batch)
+        torch.cuda.synchronize()
+        dt_host = (time.perf_counter() - t1) / n_total
+        out["host_batches"] = {"value": m.n_shard * d.batch_size / dt_host, "unit": "triples/s",
+                               "ms_per_step": dt_host * 1e3,
+                               "note": f"one call over {n_total} steps, index arrays validated and uploaded "
+                                       "from host memory inside the timed call"}
+
+    # the multi-threaded CPU path last: nothing of this workload's device work is timed after it
+    cpu_torch, cpu_torch_loss = (cpu_torch_run(torch_path, settings, n_check, args.cpu_torch_seconds)
+                                 if torch_path else (None, None))
+    if check is not None and cpu_torch_loss is not None:
+        check["cpu_loss"] = float(np.sum(cpu_torch_loss))
+        check["cpu_rel_err"] = abs(check["gpu_loss"] - check["cpu_loss"]) / abs(check["cpu_loss"])
+    # the reference's own CPU path (PyTorch, all host threads) where it covers the workload; the
+    # sequential C port beside it
+    out["cpu_baseline"] = cpu_torch if cpu_torch is not None else port
+    if with_cpu and full:
+        out["cpu_baseline_port"] = port
+    if out["cpu_baseline"]:
+        out["speedup_over_cpu_baseline"] = out["value"] / out["cpu_baseline"]["value"]
+    out["check"] = check
+    del engine
+    import gc
+    gc.collect()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--mode", default="train", choices=["train", "predict"],
+                    help="train: the training step (the headline metric); predict: the all-entity scoring sweep")
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--also", default=None,
+                    help="comma-separated workloads measured after the headline one and reported under "
+                         "`workloads` (default with --workload c2: c3l2,c3,c5 - the 22.8M- and 91.2M-row tables; "
+                         "'none' to skip)")
+    ap.add_argument("--cpu-steps", type=int, default=None,
+                    help="steps the sequential CPU port times (default: sized for ~15 s)")
+    ap.add_argument("--cpu-torch-seconds", type=float, default=8.0, help="time budget of the PyTorch CPU path")
+    ap.add_argument("--cpu-workloads", default="c3l2",
+                    help="workloads of --also that also time the PyTorch CPU path (comma-separated)")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--n-entity", type=int, default=None, help="override the table size (experiments)")
+    ap.add_argument("--predict-chunk-rows", type=int, default=None,
+                    help="--mode predict: tails scored per launch (experiments; default: the engine's)")
+    ap.add_argument("--scoring", default=None, choices=["mfma", "mfma_bf16x3", "valu"], help="scoring kernels (default mfma_bf16x3)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU holding one shard's whole table: --gpus must be 1 "
+                 "(the step has no collectives; nothing here uses a second GPU)")
+    if args.steps < 1 or args.warmup < 0:
+        sys.exit("--steps must be >= 1 and --warmup >= 0")
+    args.cpu_workloads = [x for x in args.cpu_workloads.split(",") if x]
+
+    import torch  # device discovery only; all device memory is the engine's own
+
+    if not torch.cuda.is_available():
+        sys.exit("no HIP device visible")
+    import poplar_kge as kge
+
+    if args.mode == "predict":
+        w = dict(WORKLOADS[args.workload])
+        if args.n_entity:
+            w["n_entity"] = args.n_entity
+            w["desc"] += f" [table size overridden: {args.n_entity}]"
+        if w.get("feature") or w.get("score_fn", "TransE") != "TransE":
+            sys.exit("--mode predict covers the TransE workloads without features")
+        return predict_bench(args, w, kge, torch)
+
+    also = args.also if args.also is not None else ("c3l2,c3,c5" if args.workload == "c2" and not args.n_entity else "none")
+    also = [x for x in also.split(",") if x and x != "none"]
+    for x in also:
+        if x not in WORKLOADS:
+            sys.exit(f"unknown workload '{x}' in --also")
+
+    head = measure(args.workload, args, kge, torch, full=True)
+    out = {
+        "metric": "train triples/sec (fwd+bwd+sparse Adam) at dim 256; achieved HBM GB/s",
+        "value": head.pop("value"),
+        "unit": head.pop("unit"),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head.pop("ms_per_step"),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": head.pop("dtype"),
+        "data": "synthetic",
+    }
+    out.update(head)
+    # the other table sizes, same protocol (W warm-up, K timed steps, kernel pass), one after the other
+    extra = {}
+    for x in also:
+        need = WORKLOADS[x]["n_entity"] * row_bytes(WORKLOADS[x]) + (6 << 30)
+        if torch.cuda.mem_get_info()[0] < need:
+            extra[x] = {"skipped": f"needs {need >> 30} GiB of free HBM"}
+            continue
+        extra[x] = measure(x, args, kge, torch, full=False)
+    if extra:
+        out["workloads"] = extra
+
     def plain(o):  # numpy scalars -> Python numbers
         if isinstance(o, np.generic):
             return o.item()

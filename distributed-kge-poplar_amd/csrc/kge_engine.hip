@@ -396,7 +396,13 @@ void parse_settings(kge_engine& E, const Items& s) {
         throw std::invalid_argument("norm regularisers (weight > 0) need private shard tables: with "
                                     "'execution.shared_table' a row's loss share has no owning shard");
     E.profile_kernels = s.find("execution.profile_kernels") ? s.boolean("execution.profile_kernels") : false;
-    if (s.find("execution.reduce_chunk")) E.chunk = (int)s.uint("execution.reduce_chunk");
+    if (s.find("execution.reduce_chunk")) {
+        // the chunk tables are sized for chunks of at least 64 contributions (allocate: one chunk
+        // per `chunk` contributions plus one per row that has more than direct_max)
+        const unsigned v = s.uint("execution.reduce_chunk");
+        if (v < 64 || v > 4096) throw std::invalid_argument("'execution.reduce_chunk' must be in [64, 4096]");
+        E.chunk = (int)v;
+    }
     if (s.find("execution.predict_chunk_rows")) {
         const unsigned v = s.uint("execution.predict_chunk_rows");
         if (v < 64 || v > (1u << 20)) throw std::invalid_argument("'execution.predict_chunk_rows' must be in [64, 1048576]");
@@ -582,7 +588,9 @@ void allocate(kge_engine& E) {
     E.hist.alloc(ns * 256 * tiles);
 
     E.e_ustride = (int)R;
-    E.e_cstride = (int)(R / std::min(E.chunk, E.direct_max + 1) + 2);
+    // a row gets chunks only with more than direct_max contributions and then ceil(n / chunk) of
+    // them: at most n / chunk + 1 per such row, of which there are at most R / (direct_max + 1)
+    E.e_cstride = (int)(R / E.chunk + R / (E.direct_max + 1) + 2);
     E.e_real.alloc(ns * E.e_ustride);
     E.e_uniq.alloc(ns * E.e_ustride);
     E.e_seg.alloc(ns * (E.e_ustride + 1));
@@ -594,7 +602,7 @@ void allocate(kge_engine& E) {
     E.e_hot_count.alloc(ns * 2);
     if (E.F) E.e_item_row.alloc(ns * R);
     E.r_ustride = E.n_rel_rows;
-    E.r_cstride = (int)(SB * E.rel_copies / std::min(E.chunk, E.direct_max + 1) + 2);
+    E.r_cstride = (int)(SB * E.rel_copies / E.chunk + SB * E.rel_copies / (E.direct_max + 1) + 2);
     E.r_real.alloc(ns * E.r_ustride);
     E.r_uniq.alloc(ns * E.r_ustride);
     E.r_seg.alloc(ns * (E.r_ustride + 1));
@@ -1439,6 +1447,43 @@ void run_timing(kge_engine& E, const Items& in) {
     }
 }
 
+// "plan_dump": the index work of one step of the last train_step_loop call, as the device
+// left it.  The plan phase is the device-side counterpart of the host's unique_pad
+// (src/python/poplar_kge_dataset.py:161-164: distinct rows, inverse indices) and of the grouping
+// multiUpdateAdd does for duplicate indices (src/pag/pag.cpp:721-743), so every array here has
+// an exact integer answer.  Items: step (scalar, index into the call's batch) and outputs
+//   contribution_row u32[R]      table row of every head / tail contribution
+//   unique_rows u32[R], segment_start u32[R + 1], segment_contributions u32[R]
+//                                distinct rows ascending, their first sorted position, how many
+//                                of their members are gradient contributions (the others are the
+//                                zero-gradient `remote` slots)
+//   sorted_items u32[2 R]        item numbers in (row, item) order: item < R is contribution
+//                                `item`, item >= R is slot `item - R` of `remote`
+//   counts u32[2]                {distinct rows, chunks}
+// and the same for the relation plan under relation_* (N = S B + n_relation items per copy).
+void run_plan_dump(kge_engine& E, const Items& in) {
+    const size_t i = in.uint("step");
+    if (i >= (size_t)E.n_step || !E.e_sorted_vals) throw std::invalid_argument("'plan_dump' needs a planned step of the last train_step_loop");
+    const size_t R = E.R, NRI = E.n_rel_items, RU = E.r_ustride;
+    HIP_CHECK(hipStreamSynchronize(E.stream));
+    auto out = [&](const char* name, const uint32_t* dev, size_t n) {
+        if (!in.find(name)) return;
+        uint32_t* host = (uint32_t*)in.array(name, KGE_U32, {n});
+        HIP_CHECK(hipMemcpy(host, dev, n * 4, hipMemcpyDeviceToHost));
+    };
+    out("contribution_row", E.ckey.p + i * R, R);
+    out("unique_rows", E.e_uniq.p + i * E.e_ustride, R);
+    out("segment_start", E.e_seg.p + i * (E.e_ustride + 1), R + 1);
+    out("segment_contributions", E.e_real.p + i * E.e_ustride, R);
+    out("sorted_items", E.e_sorted_vals + i * 2 * R, 2 * R);
+    out("counts", E.e_counts.p + 2 * i, 2);
+    out("relation_unique_rows", E.r_uniq.p + i * RU, RU);
+    out("relation_segment_start", E.r_seg.p + i * (RU + 1), RU + 1);
+    out("relation_segment_contributions", E.r_real.p + i * RU, RU);
+    out("relation_sorted_items", E.r_sorted_vals + i * NRI, NRI);
+    out("relation_counts", E.r_counts.p + 2 * i, 2);
+}
+
 // "predict" (Model::predict, src/poplar_kge.cpp:811-855): for every (head row,
 // relation) of every shard the n_best best-scoring tails of every shard's table.
 //   predict_head, predict_relation  u32[S, Hb]   rows inside the query's own shard
@@ -1735,6 +1780,7 @@ int kge_engine_run(kge_engine* engine, const char* command, kge_item* items, siz
         else if (cmd == "write") run_read_write(E, true, in);
         else if (cmd == "stage_batch") run_stage_batch(E, in);
         else if (cmd == "timing") run_timing(E, in);
+        else if (cmd == "plan_dump") run_plan_dump(E, in);
         else if (cmd == "gather_benchmark") run_gather_benchmark(E, in);
         else if (cmd == "variables") { /* served by kge_engine_variable_info */ }
         else if (cmd == "predict") run_predict(E, in);
@@ -1813,6 +1859,42 @@ int kge_buffer_write(void* buf, const uint32_t* idx, const void* data, int64_t n
     if (n < 0 || row_bytes < 4 || row_bytes % 4) return KGE_INVALID_ARGUMENT;
     launch_rows_scatter(buf, idx, data, n, row_bytes, (hipStream_t)stream);
     return op_status("buffer_write");
+}
+
+int kge_log_sigmoid(const float* x, const float* dy, float* y, float* dx, int64_t n, int form, void* stream) {
+    if (n < 0 || (form != 0 && form != 1) || (n > 0 && !x)) return KGE_INVALID_ARGUMENT;
+    launch_log_sigmoid(x, dy, y, dx, n, form, (hipStream_t)stream);
+    return op_status("log_sigmoid");
+}
+int kge_log_softmax(const float* x, float* y, int64_t rows, int64_t cols, void* stream) {
+    if (rows < 0 || cols < 1 || (rows > 0 && (!x || !y))) return KGE_INVALID_ARGUMENT;
+    launch_log_softmax(x, nullptr, y, rows, cols, (hipStream_t)stream);
+    return op_status("log_softmax");
+}
+int kge_log_softmax_grad(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols, void* stream) {
+    if (rows < 0 || cols < 1 || (rows > 0 && (!y || !dy || !dx))) return KGE_INVALID_ARGUMENT;
+    launch_log_softmax(y, dy, dx, rows, cols, (hipStream_t)stream);
+    return op_status("log_softmax_grad");
+}
+int kge_loss(int loss_fn, const float* score, const uint32_t* label, int S, int B, int T,
+             float softmax_correction, float negative_adversarial_scale, float loss_scale,
+             float* loss, float* row_loss, float* dscore, void* stream) {
+    if ((loss_fn != LOSS_LOGSIGMOID && loss_fn != LOSS_SOFTMAX) || S < 1 || B < 1 || T < 2) return KGE_INVALID_ARGUMENT;
+    if (!score || !label || !loss || !row_loss || !dscore) return KGE_INVALID_ARGUMENT;
+    const hipStream_t st = (hipStream_t)stream;
+    ScoreShape sh = {};
+    sh.S = S; sh.B = B; sh.T = T; sh.Dp = 0;
+    // a score that is the distance function's value itself: the coefficient launch_loss_rows
+    // leaves is d loss / d score (times the loss scale), without the sign of gamma - distance
+    sh.score_fn = SCORE_DISTMULT; sh.dist_fn = DIST_DOT; sh.loss_fn = loss_fn;
+    sh.loss_scale = loss_scale; sh.softmax_correction = softmax_correction;
+    sh.negative_adversarial_scale = negative_adversarial_scale;
+    if (dscore != score &&
+        hipMemcpyAsync(dscore, score, (size_t)S * B * T * 4, hipMemcpyDeviceToDevice, st) != hipSuccess)
+        return KGE_RUNTIME_ERROR;
+    launch_loss_rows(sh, label, dscore, nullptr, row_loss, nullptr, st);
+    launch_loss_finalize(row_loss, 1, S, B, 1.f, loss, st);
+    return op_status("loss");
 }
 
 namespace {

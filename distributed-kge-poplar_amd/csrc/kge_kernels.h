@@ -160,6 +160,15 @@ int score_fwd_parts(const ScoreShape& sh);
 void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef, const float* dist,
                       float* loss_part, uint16_t* coef16, hipStream_t stream);
 
+// Stand-alone loss ops.  log_sigmoid: y = logsigmoid(x), dx = dy * its derivative (dy null: 1);
+// form 0 evaluates them as launch_loss_rows does, form 1 as the fused scoring epilogue does.
+// log_softmax: rows of `cols`; with dy null out = log_softmax(x), otherwise `x` holds the
+// forward's output and out = dy - exp(x) * sum(dy).
+void launch_log_sigmoid(const float* x, const float* dy, float* y, float* dx, int64_t n, int form,
+                        hipStream_t stream);
+void launch_log_softmax(const float* x, const float* dy, float* out, int64_t rows, int64_t cols,
+                        hipStream_t stream);
+
 // Gradient rows of every contribution: grad[c, :] for head contributions
 // (w.r.t. the predicted tail / the head-times-relation product) and tail
 // contributions, from the coefficient matrix.

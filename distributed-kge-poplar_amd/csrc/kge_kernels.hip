@@ -1638,6 +1638,62 @@ void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef,
 }
 
 // --------------------------------------------------------------------------
+// The loss functions as stand-alone device ops (pag::ops::logSigmoid, src/pag/pag.cpp:888-910;
+// pag::ops::logSoftmax, :841-864), evaluated by the same device functions the step's kernels call.
+
+// form 0: log_sigmoid / log_sigmoid_grad as k_loss_rows calls them; form 1: log_sigmoid_both,
+// the one-exponential form of the scoring epilogues
+__global__ __launch_bounds__(256) void k_log_sigmoid(const float* __restrict__ x, const float* __restrict__ dy,
+                                                     float* __restrict__ y, float* __restrict__ dx, int64_t n,
+                                                     int form) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float v, g;
+    if (form) log_sigmoid_both(x[i], v, g);
+    else { v = log_sigmoid(x[i]); g = log_sigmoid_grad(x[i]); }
+    if (y) y[i] = v;
+    if (dx) dx[i] = (dy ? dy[i] : 1.f) * g;
+}
+void launch_log_sigmoid(const float* x, const float* dy, float* y, float* dx, int64_t n, int form,
+                        hipStream_t stream) {
+    if (n <= 0) return;
+    hipLaunchKernelGGL(k_log_sigmoid, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, dy, y, dx, n, form);
+}
+
+// One wave per row.  Forward: y = x - max - log(sum exp(x - max)) (the reduction k_loss_rows makes
+// for the softmax loss).  Backward (dy given, `x` holds y): dx = dy - exp(y) * sum(dy)
+// (src/pag/pag.cpp:853-859).
+__global__ __launch_bounds__(256) void k_log_softmax(const float* __restrict__ x, const float* __restrict__ dy,
+                                                     float* __restrict__ out, int64_t rows, int64_t cols) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* xr = x + row * cols;
+    float* o = out + row * cols;
+    if (!dy) {
+        float mx = -INFINITY;
+        for (int64_t t = lane; t < cols; t += 64) mx = fmaxf(mx, xr[t]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int64_t t = lane; t < cols; t += 64) sum += expf(xr[t] - mx);
+        sum = wave_sum(sum);
+        const float lse = mx + logf(sum);
+        for (int64_t t = lane; t < cols; t += 64) o[t] = xr[t] - lse;
+    } else {
+        const float* dr = dy + row * cols;
+        float sum = 0.f;
+        for (int64_t t = lane; t < cols; t += 64) sum += dr[t];
+        sum = wave_sum(sum);
+        for (int64_t t = lane; t < cols; t += 64) o[t] = dr[t] - expf(xr[t]) * sum;
+    }
+}
+void launch_log_softmax(const float* x, const float* dy, float* out, int64_t rows, int64_t cols,
+                        hipStream_t stream) {
+    if (rows <= 0 || cols <= 0) return;
+    hipLaunchKernelGGL(k_log_softmax, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, x, dy, out, rows, cols);
+}
+
+// --------------------------------------------------------------------------
 // scoring: backward.  out[i, k] = sum_j c[i, j] * phi(self[i, k], other[j, k])
 //   L1   phi = signum(self - other)
 //   L2   phi = self - other              (c already holds g / dist)

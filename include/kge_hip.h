@@ -7,9 +7,9 @@
  *      (src/lib.cpp:46-51 -> poplar_kge::Engine, src/poplar_kge.hpp:57-75),
  *      i.e. Engine(settings, gp_folder) and Engine::run(command, data);
  *   2. the device ops: what the reference's PAG layer calls for this path
- *      (src/poplar_extensions/distance.hpp:11-36, src/pag/pag.hpp multiSlice /
- *      logSigmoid / logSoftmax, src/fructose/frnn.hpp adam), taking plain
- *      device pointers and sizes.
+ *      (src/poplar_extensions/distance.hpp:11-36, src/pag/pag.hpp multiSlice,
+ *      logSigmoid, logSoftmax, Model::getLoss, src/fructose/frnn.hpp adam),
+ *      taking plain device pointers and sizes.
  *
  * Plain C types only.  All functions return a kge_status; on failure `err`
  * (if non-NULL) receives a NUL-terminated message.  The status maps back to
@@ -75,12 +75,23 @@ int kge_engine_create(const kge_item* settings, size_t n_settings, const char* g
                       kge_engine** out, char* err, size_t err_len);
 
 /* Replaces poplar_kge::Engine::run(const std::string& command, Batch& data)
- * (src/poplar_kge.cpp:950-965, 1004-1006).  Commands: "train_step_loop",
- * "read_entity", "write_entity", "read", "write" (and "variables", served by
- * the two functions below because its result is not an array).  Additive
- * commands, not in the reference: "write_entity_raw" (full rows from the
- * host), "stage_batch" + "train_step_loop" with {"staged": true} (keeps the
- * index arrays resident in HBM), "gather_benchmark", "timing". */
+ * (src/poplar_kge.cpp:950-965, 1004-1006).  Commands, with the reference's item
+ * names, dtypes and shapes (every array has the leading n_shard axis S):
+ *   "train_step_loop"  learning_rate f32[S], loss f32[S] (out), remote
+ *                      u32[S, n_step, B + S*A], a2a u32[S, n_step, S, A], head /
+ *                      relation / tail u32[S, n_step, B]      (:713-720, 740)
+ *   "predict"          predict_head, predict_relation u32[S, Hb],
+ *                      predict_entity_count u32[S]; out predict_scores f32 and
+ *                      predict_indices u32 [S, S, Hb, n_best]  (:812-855)
+ *   "read_entity"      read_indices u32[S, rw], read_data [S, rw, 3D+F] (out)
+ *   "write_entity"     write_indices u32[S, rw], write_features [S, rw, F]
+ *   "read" / "write"   name (string), value (the variable's shape)  (:977-991)
+ *   "variables"        served by the two functions below, because its result is
+ *                      a list and not an array                      (:993-998)
+ * Additive commands, not in the reference: "write_entity_raw" (full rows from
+ * the host), "stage_batch" + "train_step_loop" with {"staged": true} (keeps the
+ * index arrays resident in HBM), "gather_benchmark", "timing", "plan_dump" (the
+ * distinct rows, segments and sorted items the device derived for one step). */
 int kge_engine_run(kge_engine* engine, const char* command, kge_item* items, size_t n_items,
                    char* err, size_t err_len);
 
@@ -125,8 +136,10 @@ int kge_buffer_write(void* buf, const uint32_t* idx, const void* data, int64_t n
                      int64_t row_bytes, void* stream);
 
 /* pag::ops::multiSlice backward = popops::multiUpdateAdd into a zeroed table
- * (src/pag/pag.cpp:721-743): grad_t[idx[i],:] += grad_out[i,:], duplicates
- * summed, deterministically (sort by index + segmented reduce).  `workspace`
+ * (src/pag/pag.cpp:721-743): grad_t[r,:] = sum over i with idx[i] == r of
+ * grad_out[i,:] -- every row of grad_t is overwritten (rows nobody indexes
+ * become zero, as the reference's zeroed table leaves them), duplicates are
+ * summed deterministically (sort by index + segmented reduce).  `workspace`
  * must hold kge_scatter_add_workspace_bytes(n, rows, cols) bytes (16-byte aligned). */
 size_t kge_scatter_add_workspace_bytes(int64_t n, int64_t rows, int64_t cols);
 int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* idx, int64_t n,
@@ -137,6 +150,33 @@ int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* i
  * (src/poplar_kge.cpp:695-703). */
 int kge_adam(float* p, float* m, float* v, const float* g, int64_t n, float alpha, float beta_m,
              float beta_v, float epsilon, float weight_decay, int v_is_sqrt, void* stream);
+
+/* pag::ops::logSigmoid forward and backward (src/pag/pag.cpp:888-910, with its
+ * clamps at -11 / +11): y[i] = logsigmoid(x[i]), dx[i] = dy[i] * d logsigmoid /
+ * dx (dy NULL: 1; y or dx NULL: not stored).  form 0 evaluates the two
+ * functions as the row-wise loss kernel does, form 1 as the scoring kernels'
+ * fused epilogue does (one hardware exponential for both). */
+int kge_log_sigmoid(const float* x, const float* dy, float* y, float* dx, int64_t n, int form,
+                    void* stream);
+
+/* pag::ops::logSoftmax over the last axis (src/pag/pag.cpp:841-852) and its
+ * backward dx = dy - exp(y) * sum(dy) (:853-859); [rows, cols] row-major. */
+int kge_log_softmax(const float* x, float* y, int64_t rows, int64_t cols, void* stream);
+int kge_log_softmax_grad(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols,
+                         void* stream);
+
+/* Model::getLoss (src/poplar_kge.cpp:615-660) on the score matrices of S shards,
+ * by the kernel the training step runs for the softmax and the adversarial
+ * loss: score f32[S, B, T] (T = S * a2a_size), label u32[S, B] (position of the
+ * true tail in the row).  loss_fn 0 logsigmoid (weights :617-622, self-
+ * adversarial weighting :623-633 when negative_adversarial_scale > 0), 1 softmax
+ * (softmax_correction = correction_weight * (log(n_entity*S - 1) - log(T - 1)),
+ * :640-650).  Outputs: loss f32[S] per shard, row_loss f32[S, B] its per-positive
+ * terms, dscore f32[S, B, T] = loss_scale * d loss / d score (dscore may alias
+ * score). */
+int kge_loss(int loss_fn, const float* score, const uint32_t* label, int S, int B, int T,
+             float softmax_correction, float negative_adversarial_scale, float loss_scale,
+             float* loss, float* row_loss, float* dscore, void* stream);
 
 #ifdef __cplusplus
 }

@@ -83,30 +83,8 @@ def random_batch(c, n_step, rng, pad=0):
     )
 
 
-def zipf_ids(rng, n_rows, size, s=1.1):
-    """Bounded power law P(k) ~ k^-s over ids 1..n_rows-1, inverse-CDF sampled."""
-    k = np.arange(1, n_rows, dtype=np.float64)
-    cdf = np.cumsum(k**-s)
-    cdf /= cdf[-1]
-    return (1 + np.searchsorted(cdf, rng.random(size))).astype(np.uint32)
-
-
-def raw_batch(c, n_step, rng, zipf=True):
-    """Raw (non-deduplicated) ids with identity slot maps: ``remote`` holds
-    every head id then every tail id the shard sends; duplicates allowed."""
-    S, NE, B, A = c["n_shard"], c["n_entity"], c["batch"], c["a2a"]
-    T = S * A
-    NR = B + T
-    shape = (S, n_step, NR)
-    remote = zipf_ids(rng, NE, shape) if zipf else rng.integers(1, NE, shape).astype(np.uint32)
-    head = np.broadcast_to(np.arange(B, dtype=np.uint32), (S, n_step, B)).copy()
-    a2a = np.broadcast_to((B + np.arange(T, dtype=np.uint32)).reshape(S, A),
-                          (S, n_step, S, A)).copy()
-    return dict(
-        remote=remote, a2a=a2a, head=head,
-        relation=rng.integers(0, c["n_relation"], (S, n_step, B)).astype(np.uint32),
-        tail=rng.integers(0, T, (S, n_step, B)).astype(np.uint32),
-    )
+# the raw-id batches and the power-law id sampler are the measurement workloads' own
+from kge_synthetic import raw_batch, zipf_ids  # noqa: E402,F401
 
 
 def step_slice(batch, i):

@@ -10,8 +10,8 @@ first bit for bit."""
 import numpy as np
 import pytest
 
-import bench
 import kge_cases as K
+import kge_synthetic as W
 from oracle.kge_oracle import Oracle, make_cfg
 
 pytestmark = pytest.mark.gpu
@@ -38,23 +38,21 @@ def _close_but_for_sign_flips(got, ref, what, max_flip_fraction=5e-4, tol=1e-5):
 def _run(workload, n_step, rng_rows=2000, **override):
     import poplar_kge as kge
 
-    w = dict(bench.WORKLOADS[workload], **override)
-    row_bytes = ((2 if w.get("embedding_dtype") else 4) * w["dim"] + 8 * w["dim"]
-                 + (2 if w.get("feature_dtype") else 4) * w.get("feature", 0))
-    need = w["n_entity"] * row_bytes + (4 << 30)
+    w = dict(W.WORKLOADS[workload], **override)
+    need = w["n_entity"] * W.row_bytes(w) + (4 << 30)
     if _free_gpu_bytes() < need:
         pytest.skip(f"needs {need >> 30} GiB of free HBM")
-    settings = bench.make_settings(w, n_step, kge)
+    settings = W.make_settings(w, n_step, kge)
     m, d = settings.model, settings.data
     engine = kge.Engine(settings, np.full(m.n_shard, m.n_entity - 1))
-    bench.init_tables(engine, settings)
-    batch = bench.make_batch(w, n_step, kge, K)
+    W.init_tables(engine, settings)
+    batch = W.make_batch(w, n_step, kge)
 
     ids = np.unique(batch.remote)                       # every row the steps touch
     rng = np.random.default_rng(1)
     others = np.setdiff1d(rng.integers(1, m.n_entity, rng_rows).astype(np.uint32), ids)
-    before = bench.read_rows(engine, settings, ids)
-    before_others = bench.read_rows(engine, settings, others)
+    before = W.read_rows(engine, settings, ids)
+    before_others = W.read_rows(engine, settings, others)
     # the generator gives N(0, init_scale / D) embeddings and zero moments
     D = m.embedding_size
     assert abs(before[:, :D].std() * np.sqrt(D) - 1.0) < 0.02 and abs(before[:, :D].mean()) < 1e-3
@@ -63,8 +61,8 @@ def _run(workload, n_step, rng_rows=2000, **override):
     dense = ["relation_embedding"] + (["feature_projection"] if m.entity_feature_size else [])
     dense_before = {k + sfx: engine.read_variable(k + sfx) for k in dense for sfx in ("", "/adam_m", "/adam_v")}
     loss, _ = engine.train_step_loop(batch)
-    after = bench.read_rows(engine, settings, ids)
-    after_others = bench.read_rows(engine, settings, others)
+    after = W.read_rows(engine, settings, ids)
+    after_others = W.read_rows(engine, settings, others)
     np.testing.assert_array_equal(after_others, before_others)
 
     # the oracle on a compact table: row k+1 of the copy is table row ids[k]
@@ -110,6 +108,14 @@ def _run(workload, n_step, rng_rows=2000, **override):
     return settings, batch, ids, after, loss
 
 
+@pytest.mark.parametrize("scoring", ["mfma_bf16x3", "mfma", "valu"])
+def test_c1_full_size_vs_oracle(scoring):
+    """The smallest listed configuration (TransE-L2 D=64, 10k entities, 256 positives x 64 shared
+    tails, uniform ids): one block, the smallest shape the aligned scoring tiles take, under
+    every scoring path."""
+    _run("c1", n_step=3, scoring=scoring)
+
+
 def test_c2_full_size_vs_oracle_and_deterministic():
     import poplar_kge as kge
 
@@ -120,10 +126,10 @@ def test_c2_full_size_vs_oracle_and_deterministic():
     # a second engine, same seeds, same batch: bit-identical rows and loss
     m = settings.model
     engine = kge.Engine(settings, np.full(m.n_shard, m.n_entity - 1))
-    bench.init_tables(engine, settings)
+    W.init_tables(engine, settings)
     loss2, _ = engine.train_step_loop(batch)
     assert loss2 == loss
-    np.testing.assert_array_equal(bench.read_rows(engine, settings, ids), after)
+    np.testing.assert_array_equal(W.read_rows(engine, settings, ids), after)
 
 
 def test_c3_full_size_vs_oracle():
@@ -171,7 +177,7 @@ def test_predict_full_size_vs_brute_force(distance_fn):
     settings = s.prepare()
     count = m.n_entity - 12345   # the last rows of the table do not take part
     engine = kge.Engine(settings, np.full(1, count))
-    bench.init_tables(engine, settings)
+    W.init_tables(engine, settings)
     n = 128 + 7                  # a second, mostly empty program run
     rng = np.random.default_rng(5)
     queries = np.stack([np.zeros(n, np.uint32), rng.integers(1, count + 1, n).astype(np.uint32),
@@ -179,7 +185,7 @@ def test_predict_full_size_vs_brute_force(distance_fn):
     found = engine.predict(queries)
 
     D = m.embedding_size
-    table = bench.read_rows(engine, settings, np.arange(0, count + 1, dtype=np.uint32))[:, :D].astype(np.float64)
+    table = W.read_rows(engine, settings, np.arange(0, count + 1, dtype=np.uint32))[:, :D].astype(np.float64)
     rel = engine.read_variable("relation_embedding").reshape(-1, D).astype(np.float64)
     for q in range(0, n, 9):   # fifteen of the queries, both program runs
         diff = (table[queries[q, 1]] + rel[queries[q, 2]])[None, :] - table[1:]
@@ -202,14 +208,14 @@ def test_predict_shared_table_vs_brute_force():
     import poplar_kge as kge
 
     gc.collect()
-    w = dict(bench.WORKLOADS["c2"], n_entity=50_000, blocks=4, n_relation=40, dim=64, batch=32, tails=32)
-    settings = bench.make_settings(w, 1, kge)
+    w = dict(W.WORKLOADS["c2"], n_entity=50_000, blocks=4, n_relation=40, dim=64, batch=32, tails=32)
+    settings = W.make_settings(w, 1, kge)
     m, e = settings.model, settings.execution
     e.predict_hr_batch_size, e.predict_n_best, e.predict_chunk_rows = 16, 50, 4096
     S, Hb, nb, D = m.n_shard, 16, 50, m.embedding_size
     count = m.n_entity - 77
     engine = kge.Engine(settings, np.full(S, count))
-    bench.init_tables(engine, settings)
+    W.init_tables(engine, settings)
     rng = np.random.default_rng(11)
     head = rng.integers(1, count + 1, (S, Hb)).astype(np.uint32)
     relation = rng.integers(0, m.n_relation_type, (S, Hb)).astype(np.uint32)
@@ -218,7 +224,7 @@ def test_predict_shared_table_vs_brute_force():
     engine.engine.run("predict", dict(predict_head=head, predict_relation=relation,
                                       predict_entity_count=np.full(S, count, np.uint32),
                                       predict_scores=scores, predict_indices=rows))
-    table = bench.read_rows(engine, settings, np.arange(0, count + 1, dtype=np.uint32))[:, :D].astype(np.float64)
+    table = W.read_rows(engine, settings, np.arange(0, count + 1, dtype=np.uint32))[:, :D].astype(np.float64)
     rel = engine.read_variable("relation_embedding").reshape(-1, D).astype(np.float64)
     per_range = -(-(m.n_entity - 1) // S)
     for s in range(S):

@@ -242,3 +242,131 @@ def test_adam_vs_oracle(oracle64, v_is_sqrt):
     np.testing.assert_allclose(tm.cpu().numpy(), m, rtol=1e-5, atol=1e-7)
     np.testing.assert_allclose(tv.cpu().numpy(), v, rtol=1e-5, atol=1e-7)
     assert K.rel_l2(tp.cpu().numpy() - p0, p - p0) < 1e-5
+
+
+# ---- loss functions as device ops ---------------------------------------------
+
+def _log_sigmoid(x, dy=None, form=0):
+    tx = dev(np.asarray(x, np.float32))
+    ty, tdx = torch.empty_like(tx), torch.empty_like(tx)
+    tdy = dev(np.asarray(dy, np.float32)) if dy is not None else None
+    rc = H.lib().kge_log_sigmoid(H.dptr(tx), H.dptr(tdy) if tdy is not None else None, H.dptr(ty),
+                                 H.dptr(tdx), C.c_int64(tx.numel()), form, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    return ty.cpu().numpy(), tdx.cpu().numpy()
+
+
+@pytest.mark.parametrize("form", [0, 1])
+def test_logsigmoid_kat(form):
+    # tests/pag/testPag.cpp:817-845 (margin 1e-2 as there, which tolerates the clamp)
+    x = np.array([-100, -12, -1, 0, 1, 12, 100], np.float32)
+    y, dx = _log_sigmoid(x, np.full(7, 10, np.float32), form)
+    np.testing.assert_allclose(y, -np.log1p(np.exp(-x.astype(np.float64))), atol=1e-2)
+    np.testing.assert_allclose(dx, 10.0 / (1 + np.exp(x.astype(np.float64))), atol=1e-2)
+
+
+@pytest.mark.parametrize("form", [0, 1])
+def test_logsigmoid_clamps_and_oracle(oracle64, form):
+    """src/pag/pag.cpp:894-903: the value is x itself at x <= -11, the derivative stays at
+    1 / (1 + e^11) from x = 11 on; everywhere the device agrees with the oracle to 1e-5
+    relative (the bar on scores and gradients), both forms of the device function."""
+    rng = np.random.default_rng(4)
+    x = np.concatenate([np.array([-30, -11.5, -11, -10.9, -3, -0.0, 0.0, 0.5, 10.9, 11, 11.5, 30, 88, -88]),
+                        rng.normal(0, 6, 5000), rng.uniform(-12, 12, 5000)]).astype(np.float32)
+    y, dx = _log_sigmoid(x, None, form)
+    np.testing.assert_array_equal(y[x <= -11], x[x <= -11])
+    np.testing.assert_allclose(dx[x >= 11], 1 / (1 + np.exp(11.0)), rtol=2e-6)
+    np.testing.assert_allclose(y, oracle64.log_sigmoid(x), rtol=1e-5, atol=1e-9)
+    np.testing.assert_allclose(dx, oracle64.log_sigmoid_grad(x, np.ones_like(x)), rtol=1e-5)
+
+
+def _log_softmax(x, dy=None):
+    tx = dev(np.asarray(x, np.float32))
+    rows, cols = tx.reshape(-1, tx.shape[-1]).shape
+    ty = torch.empty_like(tx)
+    assert H.lib().kge_log_softmax(H.dptr(tx), H.dptr(ty), C.c_int64(rows), C.c_int64(cols), None) == 0
+    if dy is None:
+        torch.cuda.synchronize()
+        return ty.cpu().numpy()
+    tdy, tdx = dev(np.asarray(dy, np.float32)), torch.empty_like(tx)
+    assert H.lib().kge_log_softmax_grad(H.dptr(ty), H.dptr(tdy), H.dptr(tdx), C.c_int64(rows),
+                                        C.c_int64(cols), None) == 0
+    torch.cuda.synchronize()
+    return ty.cpu().numpy(), tdx.cpu().numpy()
+
+
+def test_logsoftmax_kat(oracle64):
+    # tests/pag/testPag.cpp:775-794
+    a = np.array([1, 1, 2], np.float32)
+    norm = np.log(np.exp(1.0) + np.exp(1.0) + np.exp(2.0))
+    y, dx = _log_softmax(a, np.array([10, 15, 5], np.float32))
+    np.testing.assert_allclose(y, [1 - norm, 1 - norm, 2 - norm], rtol=1e-6)
+    np.testing.assert_allclose(dx, [10 - 30 * np.exp(1 - norm), 15 - 30 * np.exp(1 - norm),
+                                    5 - 30 * np.exp(2 - norm)], rtol=1e-5)
+    rng = np.random.default_rng(5)
+    x, dy = rng.normal(0, 4, (37, 300)).astype(np.float32), rng.normal(size=(37, 300)).astype(np.float32)
+    y, dx = _log_softmax(x, dy)
+    ref = oracle64.log_softmax(x)
+    np.testing.assert_allclose(y, ref, rtol=1e-5, atol=1e-6)
+    assert K.rel_l2(dx, oracle64.log_softmax_grad(ref, dy)) < 1e-6
+
+
+def _loss(loss_fn, score, label, correction=0.0, adversarial=0.0, loss_scale=1.0):
+    S, B, T = score.shape
+    ts, tl = dev(score.astype(np.float32)), dev(label.astype(np.uint32).view(np.int32))
+    loss, rows = torch.empty(S, device="cuda"), torch.empty(S, B, device="cuda")
+    ds = torch.empty_like(ts)
+    rc = H.lib().kge_loss({"logsigmoid": 0, "softmax": 1}[loss_fn], H.dptr(ts), H.dptr(tl), S, B, T,
+                          C.c_float(correction), C.c_float(adversarial), C.c_float(loss_scale),
+                          H.dptr(loss), H.dptr(rows), H.dptr(ds), None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    return loss.cpu().numpy(), rows.cpu().numpy(), ds.cpu().numpy()
+
+
+def test_softmax_xent_kat():
+    # tests/fructose/testFructose.cpp:57-67: softmaxCrossEntropy([-100, 2, 2, 2, 2], 1) = log 4
+    loss, rows, ds = _loss("softmax", np.array([[[-100, 2, 2, 2, 2]]], np.float32), np.array([[1]]))
+    np.testing.assert_allclose(loss, [np.log(4)], rtol=1e-6)
+    np.testing.assert_allclose(ds.ravel(), [0, 0.25 - 1, 0.25, 0.25, 0.25], atol=1e-7)
+    # tests/pag/testPag.cpp:775-794 through the loss kernel: with label i the row's loss is
+    # -logsoftmax(a)[i] and dscore = softmax(a) - onehot(i)
+    a = np.broadcast_to(np.array([1, 1, 2], np.float32), (1, 3, 3)).copy()
+    norm = np.log(np.exp(1.0) + np.exp(1.0) + np.exp(2.0))
+    loss, rows, ds = _loss("softmax", a, np.array([[0, 1, 2]]))
+    np.testing.assert_allclose(rows.ravel() * 3, [norm - 1, norm - 1, norm - 2], rtol=1e-6)
+    soft = np.exp(np.array([1, 1, 2]) - norm)
+    np.testing.assert_allclose(ds[0] * 3, soft[None, :] - np.eye(3), rtol=1e-5, atol=1e-7)
+    grad_b = np.array([10, 15, 5])
+    np.testing.assert_allclose(-(grad_b[:, None] * ds[0] * 3).sum(0), grad_b - 30 * soft, rtol=1e-5)
+
+
+@pytest.mark.parametrize("variant", ["logsigmoid", "logsigmoid_saturated", "adversarial", "softmax",
+                                     "softmax_corrected", "softmax_wide"])
+def test_loss_vs_oracle(oracle64, variant):
+    """Model::getLoss on the device (the kernel the step runs for the softmax and adversarial
+    losses) against the oracle's shard_loss: per-shard loss 1e-5, d loss / d score 1e-5."""
+    from oracle.kge_oracle import make_cfg
+
+    rng = np.random.default_rng(len(variant))
+    S, B, A = (2, 37, 50) if variant != "softmax_wide" else (2, 12, 1200)
+    T = S * A
+    loss_fn = "softmax" if variant.startswith("softmax") else "logsigmoid"
+    cw = 1.0 if variant == "softmax_corrected" else 0.0
+    adv = 1.5 if variant == "adversarial" else 0.0
+    spread = 14.0 if variant == "logsigmoid_saturated" else 3.0   # |score| beyond the +-11 clamps
+    score = rng.normal(0, spread, (S, B, T)).astype(np.float32)
+    label = rng.integers(0, T, (S, B)).astype(np.uint32)
+    n_entity = 5000
+    cfg = make_cfg(n_shard=S, n_entity=n_entity, n_relation=4, dim=8, batch=B, a2a=A, loss_fn=loss_fn,
+                   softmax_correction_weight=cw, negative_adversarial_scale=adv)
+    corr = cw * float(np.float32(np.log(n_entity * S - 1) - np.log(T - 1)))
+    loss_scale = 64.0
+    loss, rows, ds = _loss(loss_fn, score, label, corr, adv, loss_scale)
+    for s in range(S):
+        ref_loss, ref_ds = oracle64.loss(cfg, score[s], label[s])
+        np.testing.assert_allclose(loss[s], ref_loss, rtol=1e-5)
+        np.testing.assert_allclose(rows[s].sum(dtype=np.float64), ref_loss, rtol=1e-5)
+        assert K.rel_l2(ds[s], loss_scale * ref_ds) < 1e-5
+        np.testing.assert_allclose(ds[s], loss_scale * ref_ds, rtol=2e-5, atol=1e-9 * loss_scale)

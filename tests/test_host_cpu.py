@@ -49,6 +49,12 @@ def test_engine_settings_validation_precedes_device_attach():
         libpoplar_kge.Engine({**s, "training.learning_rate_modifiers": {"nope": 2.0}}, "")
     with pytest.raises(ValueError, match="holds value of unexpected type"):
         libpoplar_kge.Engine({**s, "model.gamma": 2}, "")
+    # additive settings that size device tables are range-checked before anything is allocated
+    for bad in (0, 16, 63, 4097):
+        with pytest.raises(ValueError, match=r"'execution.reduce_chunk' must be in \[64, 4096\]"):
+            libpoplar_kge.Engine({**s, "execution.reduce_chunk": bad}, "")
+    with pytest.raises(ValueError, match="predict_chunk_rows"):
+        libpoplar_kge.Engine({**s, "execution.predict_chunk_rows": 10}, "")
 
 
 def test_settings_tree():
