@@ -12,6 +12,7 @@
 #include <cmath>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <sstream>
 #include <stdexcept>
 #include <string>
@@ -1954,6 +1955,78 @@ int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* i
     launch_reduce_chunks(ra, st);
     launch_sum_partials_rows(sp.chunk_off, ra.partial, rows, cols, grad_t, st);
     return op_status("scatter_add");
+}
+
+// ---- the scatter-add without a workspace argument and without allocation ----
+// Callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+// forbid hipMalloc) get the workspace from a fixed array in device memory.  Each GPU holds its own
+// copy of the array at its own address, which hipGetSymbolAddress reports with that GPU current:
+// the address is looked up once per device and every later use goes through it (the array's name
+// is a host-side stand-in in host code, not a device address).
+}  // extern "C"
+
+namespace {
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// the current device's copy of `scratch`, or null with `what` set
+void* static_scratch(std::string& what) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        what = std::string("no current HIP device (") + (e != hipSuccess ? hipGetErrorString(e) : "index out of range") + ")";
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            what = std::string("hipGetSymbolAddress(scratch) failed: ") + hipGetErrorString(e);
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" {
+
+size_t kge_scatter_add_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int kge_scatter_add_static(float* grad_t, int64_t rows, int64_t cols, const uint32_t* idx, int64_t n,
+                           const float* grad_out, void* stream, char* err, size_t err_len) {
+    if (n < 0 || rows < 1 || cols < 1 || n + rows >= ((int64_t)1 << 31)) {
+        set_error(err, err_len, "kge_scatter_add_static: sizes out of range (n >= 0, rows >= 1, cols >= 1, n + rows < 2^31)");
+        return KGE_INVALID_ARGUMENT;
+    }
+    const size_t need = scatter_layout(n, rows, cols).total;
+    if (need > kStaticScratchBytes) {
+        std::ostringstream msg;
+        msg << "kge_scatter_add_static: n = " << n << ", rows = " << rows << ", cols = " << cols << " need " << need
+            << " bytes of workspace, more than the " << kStaticScratchBytes
+            << " bytes of the static scratch array; use kge_scatter_add with a workspace of your own";
+        set_error(err, err_len, msg.str().c_str());
+        return KGE_INVALID_ARGUMENT;
+    }
+    std::string what;
+    void* ptr = static_scratch(what);
+    if (!ptr) {
+        set_error(err, err_len, what.c_str());
+        return KGE_RUNTIME_ERROR;
+    }
+    // nothing in the workspace has to start at zero: every word a kernel reads, an earlier kernel
+    // of the same call wrote (histograms, keys, segment tables, partial sums)
+    const int rc = kge_scatter_add(grad_t, rows, cols, idx, n, grad_out, ptr, stream);
+    if (rc != KGE_OK) set_error(err, err_len, "kge_scatter_add_static: kernel launch failed");
+    return rc;
 }
 
 int kge_adam(float* p, float* m, float* v, const float* g, int64_t n, float alpha, float beta_m,

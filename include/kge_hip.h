@@ -145,6 +145,21 @@ size_t kge_scatter_add_workspace_bytes(int64_t n, int64_t rows, int64_t cols);
 int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* idx, int64_t n,
                     const float* grad_out, void* workspace, void* stream);
 
+/* kge_scatter_add for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same arguments and results as kge_scatter_add,
+ * without the workspace: it lives in a fixed array of
+ * kge_scatter_add_static_max_bytes() bytes (16 MiB) that every GPU the library
+ * runs on holds until the process ends.  Sizes whose workspace
+ * (kge_scatter_add_workspace_bytes) exceeds that are rejected with
+ * KGE_INVALID_ARGUMENT and a message in `err`.  The call allocates and frees
+ * nothing.  All calls on one GPU share that GPU's array: calls that overlap in
+ * time on one GPU (different streams, or host threads) race; issue them in
+ * order on one stream. */
+size_t kge_scatter_add_static_max_bytes(void);
+int kge_scatter_add_static(float* grad_t, int64_t rows, int64_t cols, const uint32_t* idx, int64_t n,
+                           const float* grad_out, void* stream, char* err, size_t err_len);
+
 /* fr::nn::adam (src/fructose/frnn.cpp:61-90), fused, in place.  With
  * v_is_sqrt != 0 the third array holds sqrt(v) as the entity rows do
  * (src/poplar_kge.cpp:695-703). */
