@@ -201,7 +201,17 @@ struct kge_engine {
     // resident batch, read back once after the plan phase of a call with enough steps to pay
     // for the wait: the per-row and per-chunk launches then start no workgroup that only finds
     // out it has nothing to do (two thirds of them under power-law sampling)
-    std::vector<uint32_t> h_e_counts, h_r_counts, h_e_hot, h_r_hot;
+    // (pinned host memory: the copies are asynchronous and waited for only when the first launch
+    // that needs them is due, behind the first step's gather and scoring launches)
+    // per step {distinct rows, chunks, rows with chunks, contributions of the biggest row}, which
+    // the segment kernel writes straight into this (device-visible) host memory
+    uint32_t *h_e_counts = nullptr, *h_r_counts = nullptr;  // [n_step][4] each
+    uint32_t *d_e_counts = nullptr, *d_r_counts = nullptr;  // the same memory as the device addresses it
+    void* h_pin = nullptr;          // the two arrays above, the step sizes and the loss
+    float* h_alpha_pin = nullptr;
+    float* h_loss_pin = nullptr;
+    hipEvent_t counts_ready = nullptr;
+    bool counts_pending = false;
     bool counts_known = false;
     int plan_readback_steps = 8;  // additive setting execution.plan_readback_steps: calls of at least this many steps
     int mlp = 0;  // model.feature_mlp_size: hidden = value + relu([value | feature . W] . Up) . Down
@@ -247,7 +257,7 @@ struct kge_engine {
     DevBuf<uint32_t> d_remote, d_a2a, d_head, d_relation, d_tail;
     bool staged = false;
     // plan
-    DevBuf<uint32_t> ckey, crel, clabel, ek_a, ev_a, ek_b, ev_b, rk_a, rv_a, rk_b, rv_b, hist;
+    DevBuf<uint32_t> ckey, crel, clabel, ek_a, ev_a, ek_b, ev_b, rk_a, rv_a, rk_b, rv_b, hist, seg_scratch;
     DevBuf<uint32_t> e_uniq, e_seg, e_coff, e_cpos, e_clen, e_counts, e_item_row, e_real;
     DevBuf<uint32_t> r_uniq, r_seg, r_coff, r_cpos, r_clen, r_counts, r_real;
     DevBuf<uint32_t> e_hot, e_hot_count, r_hot, r_hot_count;  // the rows with chunks, per step
@@ -292,6 +302,8 @@ struct kge_engine {
         for (auto& e : ev) if (e) (void)hipEventDestroy(e);
         for (auto& e : kev) (void)hipEventDestroy(e);
         if (p_pin) (void)hipHostFree(p_pin);
+        if (h_pin) (void)hipHostFree(h_pin);
+        if (counts_ready) (void)hipEventDestroy(counts_ready);
         for (auto& e : scored) if (e) (void)hipEventDestroy(e);
         for (auto& e : merged) if (e) (void)hipEventDestroy(e);
         if (merge_stream) (void)hipStreamDestroy(merge_stream);
@@ -585,8 +597,21 @@ void allocate(kge_engine& E) {
     for (DevBuf<uint32_t>* b : {&E.ek_a, &E.ev_a, &E.ek_b, &E.ev_b}) b->alloc(ns * 2 * R);
     E.n_rel_items = (int)((SB + E.n_rel) * E.rel_copies);
     for (DevBuf<uint32_t>* b : {&E.rk_a, &E.rv_a, &E.rk_b, &E.rv_b}) b->alloc(ns * E.n_rel_items);
-    const size_t tiles = (std::max<size_t>(2 * R, E.n_rel_items) + kSortTile - 1) / kSortTile;
-    E.hist.alloc(ns * 256 * tiles);
+    E.hist.alloc(std::max(radix_sort_hist_words((int)(2 * R), (int)ns, std::max(1, bit_length((uint64_t)E.n_rows - 1))),
+                          radix_sort_hist_words(E.n_rel_items, (int)ns, std::max(1, bit_length((uint64_t)E.n_rel_rows - 1)))));
+    E.seg_scratch.alloc(find_segments_scratch_words((int)(2 * R), E.n_rel_items, (int)ns));
+    {   // pinned host staging: plan counts [4][2 ns], step sizes [ns 9 S], loss [S]
+        const size_t words = 8 * ns + ns * 9 * S + S;  // counts [2][ns][4]
+        HIP_CHECK(hipHostMalloc(&E.h_pin, words * 4, hipHostMallocDefault));
+        std::memset(E.h_pin, 0, words * 4);
+        E.h_e_counts = (uint32_t*)E.h_pin; E.h_r_counts = E.h_e_counts + 4 * ns;
+        E.h_alpha_pin = (float*)(E.h_r_counts + 4 * ns);
+        void* dev_view = nullptr;
+        HIP_CHECK(hipHostGetDevicePointer(&dev_view, E.h_pin, 0));
+        E.d_e_counts = (uint32_t*)dev_view; E.d_r_counts = E.d_e_counts + 4 * ns;
+        E.h_loss_pin = E.h_alpha_pin + ns * 9 * S;
+        HIP_CHECK(hipEventCreateWithFlags(&E.counts_ready, hipEventDisableTiming));
+    }
 
     E.e_ustride = (int)R;
     // a row gets chunks only with more than direct_max contributions and then ceil(n / chunk) of
@@ -910,7 +935,10 @@ void run_plan(kge_engine& E, int s0, int sn) {
                                   E.hist.p, (int)N, sn, ebits, st);
     const uint32_t* ek = which ? E.ek_b.p : E.ek_a.p;
     E.e_sorted_vals = which ? E.ev_b.p : E.ev_a.p;
-    SegPlan ep;
+    SegJob ej = {};
+    ej.keys = ek + s0 * N; ej.vals = E.e_sorted_vals + s0 * N;
+    ej.N = (int)N; ej.n_real = (int)R; ej.chunk = E.chunk; ej.direct_max = E.direct_max;
+    SegPlan& ep = ej.plan;
     ep.u_stride = E.e_ustride; ep.c_stride = E.e_cstride;
     ep.uniq_key = E.e_uniq.p + (size_t)s0 * ep.u_stride;
     ep.seg_start = E.e_seg.p + (size_t)s0 * (ep.u_stride + 1);
@@ -921,13 +949,16 @@ void run_plan(kge_engine& E, int s0, int sn) {
     ep.item_row = E.F ? E.e_item_row.p + s0 * R : nullptr;
     ep.seg_real = E.e_real.p + (size_t)s0 * ep.u_stride;
     ep.hot_rows = E.e_hot.p + (size_t)s0 * ep.c_stride; ep.hot_count = E.e_hot_count.p + 2 * s0;
-    launch_find_segments(ek + s0 * N, E.e_sorted_vals + s0 * N, (int)N, (int)R, E.chunk, E.direct_max, sn, ep, st);
+    ep.host_counts = E.d_e_counts + 4 * (size_t)s0;
 
     which = launch_radix_sort(E.rk_a.p + s0 * NRI, E.rv_a.p + s0 * NRI, E.rk_b.p + s0 * NRI,
                               E.rv_b.p + s0 * NRI, E.hist.p, (int)NRI, sn, rbits, st);
     const uint32_t* rk = which ? E.rk_b.p : E.rk_a.p;
     E.r_sorted_vals = which ? E.rv_b.p : E.rv_a.p;
-    SegPlan rp;
+    SegJob rj = {};
+    rj.keys = rk + s0 * NRI; rj.vals = E.r_sorted_vals + s0 * NRI;
+    rj.N = (int)NRI; rj.n_real = (int)SB * E.rel_copies; rj.chunk = E.chunk; rj.direct_max = E.direct_max;
+    SegPlan& rp = rj.plan;
     rp.u_stride = E.r_ustride; rp.c_stride = E.r_cstride;
     rp.uniq_key = E.r_uniq.p + (size_t)s0 * rp.u_stride;
     rp.seg_start = E.r_seg.p + (size_t)s0 * (rp.u_stride + 1);
@@ -938,7 +969,8 @@ void run_plan(kge_engine& E, int s0, int sn) {
     rp.item_row = nullptr;
     rp.seg_real = E.r_real.p + (size_t)s0 * rp.u_stride;
     rp.hot_rows = E.r_hot.p + (size_t)s0 * rp.c_stride; rp.hot_count = E.r_hot_count.p + 2 * s0;
-    launch_find_segments(rk + s0 * NRI, E.r_sorted_vals + s0 * NRI, (int)NRI, (int)SB * E.rel_copies, E.chunk, E.direct_max, sn, rp, st);
+    rp.host_counts = E.d_r_counts + 4 * (size_t)s0;
+    launch_find_segments2(ej, &rj, sn, E.seg_scratch.p, st);  // both plans' segments in one launch
     HIP_CHECK(hipGetLastError());
 }
 
@@ -1141,6 +1173,10 @@ void run_step(kge_engine& E, int i) {
                         E.reg_loss_part.p + (size_t)i * E.S, st);
     }
 
+    if (E.counts_pending) {  // the plan's counts size the launches from here on
+        HIP_CHECK(hipEventSynchronize(E.counts_ready));
+        E.counts_pending = false;
+    }
     const float* alpha = E.d_alpha.p + (size_t)i * 9 * E.S;
     AdamArgs aa = {};
     aa.Dp = E.Dp;
@@ -1166,7 +1202,7 @@ void run_step(kge_engine& E, int i) {
     rr.chunk_pos = E.r_cpos.p + (size_t)i * E.r_cstride;
     rr.chunk_len = E.r_clen.p + (size_t)i * E.r_cstride;
     rr.counts = r_counts; rr.max_chunks = E.r_cstride; rr.chunk = E.chunk;
-    if (E.counts_known) rr.max_chunks = (int)E.h_r_counts[2 * (size_t)i + 1];
+    if (E.counts_known) rr.max_chunks = (int)E.h_r_counts[4 * (size_t)i + 1];
     rr.partial = E.rel_partial.p; rr.Dp = E.Dp;
 
     ReduceArgs re = {};
@@ -1174,7 +1210,7 @@ void run_step(kge_engine& E, int i) {
     re.chunk_pos = E.e_cpos.p + (size_t)i * E.e_cstride;
     re.chunk_len = E.e_clen.p + (size_t)i * E.e_cstride;
     re.counts = e_counts; re.max_chunks = E.e_cstride; re.chunk = E.chunk;
-    if (E.counts_known) re.max_chunks = (int)E.h_e_counts[2 * (size_t)i + 1];
+    if (E.counts_known) re.max_chunks = (int)E.h_e_counts[4 * (size_t)i + 1];
     re.partial = E.partial.p; re.Dp = E.Dp;
     // Contributions used as stored, nothing between the sums and the updates, and no row with
     // more contributions than a handful of workgroups sum in the time the other rows take (known
@@ -1184,7 +1220,7 @@ void run_step(kge_engine& E, int i) {
     // hottest) takes its eight workgroups longer than the whole update takes otherwise; one of
     // 2 200 (the 1M-row workload's) fits under it.
     const bool hot_in_update = !contributions_read_tables(E) && !E.mlp && !roles && E.counts_known &&
-                               std::max(E.h_e_hot[2 * (size_t)i + 1], E.h_r_hot[2 * (size_t)i + 1]) <= kHotInUpdateMax;
+                               std::max(E.h_e_counts[4 * (size_t)i + 3], E.h_r_counts[4 * (size_t)i + 3]) <= kHotInUpdateMax;
     if (!hot_in_update) { KernelTimer t(E, K_REDUCE_ENT); launch_reduce_chunks2(re, rr, st); }
 
     // With DistMult / ComplEx the relation rows' direct contributions read entity rows and
@@ -1211,7 +1247,7 @@ void run_step(kge_engine& E, int i) {
     ae.seg_start = E.e_seg.p + (size_t)i * (E.e_ustride + 1);
     ae.seg_real = E.e_real.p + (size_t)i * E.e_ustride;
     ae.chunk_off = E.e_coff.p + (size_t)i * (E.e_ustride + 1);
-    ae.counts = e_counts; ae.max_rows = E.counts_known ? (int)E.h_e_counts[2 * (size_t)i] : (int)R;
+    ae.counts = e_counts; ae.max_rows = E.counts_known ? (int)E.h_e_counts[4 * (size_t)i] : (int)R;
     ae.partial = E.partial.p;
     // (with dropout the feature part's gradient is formed per role by launch_role_sums)
     ae.grad_out = (E.F && !roles) ? E.gsum.p : nullptr;
@@ -1263,9 +1299,9 @@ void run_step(kge_engine& E, int i) {
         KernelTimer t(E, K_ADAM_ENT);
         HotRows he, hr;
         he.hot_rows = E.e_hot.p + (size_t)i * E.e_cstride; he.hot_count = E.e_hot_count.p + 2 * i;
-        he.max_hot = (int)E.h_e_hot[2 * (size_t)i];
+        he.max_hot = (int)E.h_e_counts[4 * (size_t)i + 2];
         hr.hot_rows = E.r_hot.p + (size_t)i * E.r_cstride; hr.hot_count = E.r_hot_count.p + 2 * i;
-        hr.max_hot = (int)E.h_r_hot[2 * (size_t)i];
+        hr.max_hot = (int)E.h_r_counts[4 * (size_t)i + 2];
         launch_adam_rows_hot2(ar, hr, ae, he, st);
     } else {
         // the relation rows first: they are few and slow (a dozen contributions each, two rounds
@@ -1375,25 +1411,19 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
         if (E.shared_table && E.score_fn == SCORE_TRANSH)
             E.h_alpha[((size_t)i * 9 + 1) * S + 1] = (float)(factor * (double)lr[0]) * E.lr_mod_normal;
     }
-    HIP_CHECK(hipMemcpyAsync(E.d_alpha.p, E.h_alpha.data(), E.h_alpha.size() * 4, hipMemcpyHostToDevice, st));
+    std::memcpy(E.h_alpha_pin, E.h_alpha.data(), E.h_alpha.size() * 4);
+    HIP_CHECK(hipMemcpyAsync(E.d_alpha.p, E.h_alpha_pin, E.h_alpha.size() * 4, hipMemcpyHostToDevice, st));
     HIP_CHECK(hipEventRecord(E.ev[1], st));
     run_plan(E, s0, sn);
     E.step_of_first = (int)E.step - s0;  // step i of the batch is optimiser step E.step + (i - s0)
     E.counts_known = sn >= E.plan_readback_steps;
+    E.counts_pending = false;
     if (E.counts_known) {
-        E.h_e_counts.resize(2 * (size_t)E.n_step);
-        E.h_r_counts.resize(2 * (size_t)E.n_step);
-        HIP_CHECK(hipMemcpyAsync(E.h_e_counts.data() + 2 * s0, E.e_counts.p + 2 * s0, 2 * (size_t)sn * 4,
-                                 hipMemcpyDeviceToHost, st));
-        HIP_CHECK(hipMemcpyAsync(E.h_r_counts.data() + 2 * s0, E.r_counts.p + 2 * s0, 2 * (size_t)sn * 4,
-                                 hipMemcpyDeviceToHost, st));
-        E.h_e_hot.resize(2 * (size_t)E.n_step);
-        E.h_r_hot.resize(2 * (size_t)E.n_step);
-        HIP_CHECK(hipMemcpyAsync(E.h_e_hot.data() + 2 * s0, E.e_hot_count.p + 2 * s0, 2 * (size_t)sn * 4,
-                                 hipMemcpyDeviceToHost, st));
-        HIP_CHECK(hipMemcpyAsync(E.h_r_hot.data() + 2 * s0, E.r_hot_count.p + 2 * s0, 2 * (size_t)sn * 4,
-                                 hipMemcpyDeviceToHost, st));
-        HIP_CHECK(hipStreamSynchronize(st));
+        // the segment kernel has written the counts into pinned host memory; the host waits for
+        // that kernel when the first launch sized by them is due, with the first step's scoring
+        // launches already queued behind it
+        HIP_CHECK(hipEventRecord(E.counts_ready, st));
+        E.counts_pending = true;
     }
     HIP_CHECK(hipEventRecord(E.ev[2], st));
     for (int i = s0; i < s0 + sn; ++i) run_step(E, i);
@@ -1401,8 +1431,9 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
                          E.d_loss.p, st, E.reg_on ? E.reg_loss_part.p + (size_t)s0 * E.S : nullptr);
     HIP_CHECK(hipGetLastError());
     HIP_CHECK(hipEventRecord(E.ev[3], st));
-    HIP_CHECK(hipMemcpyAsync(loss, E.d_loss.p, S * 4, hipMemcpyDeviceToHost, st));
+    HIP_CHECK(hipMemcpyAsync(E.h_loss_pin, E.d_loss.p, S * 4, hipMemcpyDeviceToHost, st));
     HIP_CHECK(hipStreamSynchronize(st));
+    std::memcpy(loss, E.h_loss_pin, S * 4);
     E.step += (uint32_t)sn;
     for (int k = 0; k < 3; ++k) HIP_CHECK(hipEventElapsedTime(&E.phase_ms[k], E.ev[k], E.ev[k + 1]));
     HIP_CHECK(hipEventElapsedTime(&E.phase_ms[3], E.ev[0], E.ev[3]));
@@ -1902,7 +1933,7 @@ namespace {
 struct ScatterLayout {
     size_t N, tiles, cmax;
     size_t off_keys_a, off_vals_a, off_keys_b, off_vals_b, off_hist, off_uniq, off_seg, off_coff,
-        off_cpos, off_clen, off_counts, off_partial, total;
+        off_cpos, off_clen, off_counts, off_real, off_scratch, off_partial, total;
 };
 ScatterLayout scatter_layout(int64_t n, int64_t rows, int64_t cols) {
     ScatterLayout L;
@@ -1913,9 +1944,10 @@ ScatterLayout scatter_layout(int64_t n, int64_t rows, int64_t cols) {
     auto take = [&](size_t words) { size_t at = o; o += (words * 4 + 15) / 16 * 16; return at; };
     L.off_keys_a = take(L.N); L.off_vals_a = take(L.N);
     L.off_keys_b = take(L.N); L.off_vals_b = take(L.N);
-    L.off_hist = take(256 * L.tiles);
+    L.off_hist = take(radix_sort_hist_words((int)L.N, 1, std::max(1, bit_length((uint64_t)rows - 1))));
     L.off_uniq = take(rows); L.off_seg = take(rows + 1); L.off_coff = take(rows + 1);
     L.off_cpos = take(L.cmax); L.off_clen = take(L.cmax); L.off_counts = take(2);
+    L.off_real = take(rows); L.off_scratch = take(find_segments_scratch_words((int)L.N, 0, 1));
     L.off_partial = take(L.cmax * (size_t)cols);
     L.total = o;
     return L;
@@ -1939,14 +1971,16 @@ int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* i
     const int bits = std::max(1, bit_length((uint64_t)rows - 1));
     const int which = launch_radix_sort(u32(L.off_keys_a), u32(L.off_vals_a), u32(L.off_keys_b),
                                         u32(L.off_vals_b), u32(L.off_hist), (int)L.N, 1, bits, st);
-    SegPlan sp;
+    const uint32_t* sv = which ? u32(L.off_vals_b) : u32(L.off_vals_a);
+    SegJob job = {};
+    job.keys = which ? u32(L.off_keys_b) : u32(L.off_keys_a); job.vals = sv;
+    job.N = (int)L.N; job.n_real = (int)n; job.chunk = 32; job.direct_max = 0;
+    SegPlan& sp = job.plan;
     sp.uniq_key = u32(L.off_uniq); sp.seg_start = u32(L.off_seg); sp.chunk_off = u32(L.off_coff);
     sp.chunk_pos = u32(L.off_cpos); sp.chunk_len = u32(L.off_clen); sp.counts = u32(L.off_counts);
     sp.item_row = nullptr; sp.u_stride = (int)rows; sp.c_stride = (int)L.cmax;
-    const uint32_t* sk = which ? u32(L.off_keys_b) : u32(L.off_keys_a);
-    const uint32_t* sv = which ? u32(L.off_vals_b) : u32(L.off_vals_a);
-    sp.seg_real = nullptr; sp.hot_rows = nullptr; sp.hot_count = nullptr;
-    launch_find_segments(sk, sv, (int)L.N, (int)n, 32, 0, 1, sp, st);
+    sp.seg_real = u32(L.off_real); sp.hot_rows = nullptr; sp.hot_count = nullptr; sp.host_counts = nullptr;
+    launch_find_segments2(job, nullptr, 1, u32(L.off_scratch), st);
     ReduceArgs ra = {};
     ra.src.sorted_item = sv; ra.src.grad = grad_out; ra.src.transform = 0;
     ra.chunk_pos = sp.chunk_pos; ra.chunk_len = sp.chunk_len; ra.counts = sp.counts;

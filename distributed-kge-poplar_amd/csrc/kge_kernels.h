@@ -57,12 +57,16 @@ struct PlanShape {
 void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
                         const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
                         uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
-                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals,
-                        hipStream_t stream);
+                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals, hipStream_t stream);
 
 // Stable LSD radix sort of n_seg independent arrays of N (key, value) pairs on
-// the low `key_bits` bits.  Result is in keys_a/vals_a if the return value is
-// 0, in keys_b/vals_b if it is 1.  hist must hold n_seg * 256 * ceil(N/kSortTile) words.
+// the low `key_bits` bits, in sort_passes(key_bits).n passes of at most kSortMaxBits bits.
+// Result is in keys_a/vals_a if the return value is 0, in keys_b/vals_b if it is 1.
+// hist must hold radix_sort_hist_words(N, n_seg, key_bits) words.
+constexpr int kSortMaxBits = 11;
+struct SortPasses { int n; int bits[4]; int shift[4]; };
+SortPasses sort_passes(int key_bits);
+size_t radix_sort_hist_words(int N, int n_seg, int key_bits);
 int launch_radix_sort(uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
                       uint32_t* hist, int N, int n_seg, int key_bits, hipStream_t stream);
 
@@ -75,20 +79,33 @@ struct SegPlan {
     uint32_t* chunk_len;  // [n_seg, c_stride]      real items in the chunk (<= chunk size)
     uint32_t* counts;     // [n_seg, 2]             {distinct rows, chunks}
     uint32_t* item_row;   // [n_seg, n_real] or null: distinct-row index of each real item
-    uint32_t* seg_real;   // [n_seg, u_stride] or null: real items of each row
+    uint32_t* seg_real;   // [n_seg, u_stride]      real items of each row
     // or null: the rows that get chunks (more than direct_max real items), as distinct-row
     // indices in ascending order [n_seg, c_stride], and [n_seg, 2] {how many, real items of the
-    // row with the most} (needs seg_real)
+    // row with the most}
     uint32_t* hot_rows;
     uint32_t* hot_count;
+    // or null: [n_seg, 4] {distinct rows, chunks, rows with chunks, real items of the biggest row}
+    // once more, in device-visible host memory (the host sizes its launches from them)
+    uint32_t* host_counts;
     int u_stride, c_stride;
 };
 
+// One sorted array per step and what to derive from it.  Real items (value < n_real) are the
+// gradient contributions; every distinct key must also hold at least one other item (its
+// zero-gradient member of the update set), which the stable sort leaves behind the real ones.
 // Rows with at most `direct_max` real items get no chunks (their consumer sums
 // the items itself); longer rows are cut into chunks of `chunk` items.
-void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sorted, int N,
-                          int n_real, int chunk, int direct_max, int n_seg, const SegPlan& plan,
-                          hipStream_t stream);
+struct SegJob {
+    const uint32_t* keys;  // [n_seg, N] sorted
+    const uint32_t* vals;
+    int N, n_real, chunk, direct_max;
+    SegPlan plan;
+};
+// j1 (or null): a second job with the same number of segments, served by the same launches.
+// scratch: find_segments_scratch_words(j0.N, j1 ? j1->N : 0, n_seg) words, no initial content needed.
+size_t find_segments_scratch_words(int N0, int N1, int n_seg);
+void launch_find_segments2(const SegJob& j0, const SegJob* j1, int n_seg, uint32_t* scratch, hipStream_t stream);
 
 // ---- step phase ----------------------------------------------------------
 

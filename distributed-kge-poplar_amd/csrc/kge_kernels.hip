@@ -109,338 +109,6 @@ DEVINL float wave_max(float v) {
 }
 
 // --------------------------------------------------------------------------
-// plan phase
-
-__global__ __launch_bounds__(256) void k_build_items(PlanShape ps, const uint32_t* __restrict__ remote,
-                                                     const uint32_t* __restrict__ a2a,
-                                                     const uint32_t* __restrict__ head,
-                                                     const uint32_t* __restrict__ relation,
-                                                     const uint32_t* __restrict__ tail,
-                                                     uint32_t* __restrict__ ckey,
-                                                     uint32_t* __restrict__ crel,
-                                                     uint32_t* __restrict__ clabel,
-                                                     uint32_t* __restrict__ ent_keys,
-                                                     uint32_t* __restrict__ ent_vals,
-                                                     uint32_t* __restrict__ rel_keys,
-                                                     uint32_t* __restrict__ rel_vals) {
-    const int step = ps.step0 + blockIdx.y;
-    const int S = ps.S, B = ps.B, A = ps.A, NR = ps.NR, T = S * A, nst = ps.n_step;
-    const int R = S * NR, SB = S * B;
-    const int item = blockIdx.x * 256 + threadIdx.x;
-    const int SBr = SB * ps.rel_copies;
-    const int n_rel_items = SBr + ps.n_relation * ps.rel_copies;
-    if (item < 2 * R) {
-        int src, slot;
-        if (item < SB) {
-            const int d = item / B, b = item - d * B;
-            src = d;
-            slot = head[((size_t)d * nst + step) * B + b];
-        } else if (item < R) {
-            const int cc = item - SB;
-            const int d = cc / T, t = cc - d * T;
-            const int j = t / A, i = t - j * A;
-            src = j;
-            slot = a2a[(((size_t)j * nst + step) * S + d) * A + i];
-        } else {
-            const int sl = item - R;
-            src = sl / NR;
-            slot = sl - src * NR;
-        }
-        const uint32_t base = ps.shared_table ? 0u : (uint32_t)src * (uint32_t)ps.n_entity;
-        const uint32_t key = base + remote[((size_t)src * nst + step) * NR + slot];
-        if (item < R) ckey[(size_t)step * R + item] = key;
-        ent_keys[(size_t)step * 2 * R + item] = key;
-        ent_vals[(size_t)step * 2 * R + item] = item;
-    }
-    if (item < n_rel_items) {
-        uint32_t key;
-        if (item < SBr) {
-            const int copy = item / SB, c = item - copy * SB;
-            const int d = c / B, b = c - d * B;
-            key = relation[((size_t)d * nst + step) * B + b];
-            if (copy == 0) {
-                crel[(size_t)step * SB + c] = key;
-                clabel[(size_t)step * SB + c] = tail[((size_t)d * nst + step) * B + b];
-            }
-            key += (uint32_t)(copy * ps.n_relation);
-        } else {
-            key = item - SBr;
-        }
-        rel_keys[(size_t)step * n_rel_items + item] = key;
-        rel_vals[(size_t)step * n_rel_items + item] = item;
-    }
-}
-
-void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
-                        const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
-                        uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
-                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals,
-                        hipStream_t stream) {
-    const int R = ps.S * ps.NR;
-    const int n = std::max(2 * R, (ps.S * ps.B + ps.n_relation) * ps.rel_copies);
-    dim3 grid((n + 255) / 256, ps.step_count);
-    hipLaunchKernelGGL(k_build_items, grid, dim3(256), 0, stream, ps, remote, a2a, head, relation,
-                       tail, ckey, crel, clabel, ent_keys, ent_vals, rel_keys, rel_vals);
-}
-
-// ---- stable LSD radix sort, 8 bits per pass --------------------------------
-// hist layout: [seg][digit][tile]
-
-__global__ __launch_bounds__(256) void k_sort_hist(const uint32_t* __restrict__ keys, int N,
-                                                   int n_tiles, int shift,
-                                                   uint32_t* __restrict__ hist) {
-    __shared__ uint32_t h[256];
-    const int seg = blockIdx.y, tile = blockIdx.x;
-    h[threadIdx.x] = 0;
-    __syncthreads();
-    const uint32_t* k = keys + (size_t)seg * N;
-    const int base = tile * kSortTile;
-#pragma unroll
-    for (int r = 0; r < kSortTile / 256; ++r) {
-        const int i = base + r * 256 + threadIdx.x;
-        if (i < N) atomicAdd(&h[(k[i] >> shift) & 255u], 1u);
-    }
-    __syncthreads();
-    hist[((size_t)seg * 256 + threadIdx.x) * n_tiles + tile] = h[threadIdx.x];
-}
-
-// exclusive scan over (digit-major, tile-minor) for one segment per block
-__global__ __launch_bounds__(256) void k_sort_scan(uint32_t* __restrict__ hist, int n_tiles) {
-    __shared__ uint32_t tot[256];
-    const int seg = blockIdx.x, d = threadIdx.x;
-    uint32_t* h = hist + ((size_t)seg * 256 + d) * n_tiles;
-    uint32_t sum = 0;
-    for (int t = 0; t < n_tiles; ++t) sum += h[t];
-    tot[d] = sum;
-    __syncthreads();
-    // Hillis-Steele inclusive scan over the 256 digit totals
-    for (int off = 1; off < 256; off <<= 1) {
-        uint32_t v = d >= off ? tot[d - off] : 0;
-        __syncthreads();
-        tot[d] += v;
-        __syncthreads();
-    }
-    uint32_t run = tot[d] - sum;  // exclusive base of digit d
-    for (int t = 0; t < n_tiles; ++t) {
-        const uint32_t c = h[t];
-        h[t] = run;
-        run += c;
-    }
-}
-
-__global__ __launch_bounds__(256) void k_sort_scatter(const uint32_t* __restrict__ keys_in,
-                                                      const uint32_t* __restrict__ vals_in,
-                                                      uint32_t* __restrict__ keys_out,
-                                                      uint32_t* __restrict__ vals_out, int N,
-                                                      int n_tiles, int shift,
-                                                      const uint32_t* __restrict__ hist) {
-    // run[w][digit]: next output position for wave w's items with that digit
-    __shared__ uint32_t run[4][256];
-    const int seg = blockIdx.y, tile = blockIdx.x;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const uint32_t* kin = keys_in + (size_t)seg * N;
-    const uint32_t* vin = vals_in + (size_t)seg * N;
-    constexpr int ROUNDS = kSortTile / 256;  // rounds of 64 items per wave
-    const int wbase = tile * kSortTile + wave * (kSortTile / 4);
-
-    for (int i = tid; i < 4 * 256; i += 256) (&run[0][0])[i] = 0;
-    __syncthreads();
-    uint32_t key[ROUNDS], val[ROUNDS];
-#pragma unroll
-    for (int r = 0; r < ROUNDS; ++r) {
-        const int i = wbase + r * 64 + lane;
-        key[r] = i < N ? kin[i] : 0xffffffffu;
-        val[r] = i < N ? vin[i] : 0u;
-        if (i < N) atomicAdd(&run[wave][(key[r] >> shift) & 255u], 1u);
-    }
-    __syncthreads();
-    {   // per digit: exclusive prefix over the four waves + the tile's global base
-        const int d = tid;
-        uint32_t base = hist[((size_t)seg * 256 + d) * n_tiles + tile];
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const uint32_t c = run[w][d];
-            run[w][d] = base;
-            base += c;
-        }
-    }
-    __syncthreads();
-    uint32_t* kout = keys_out + (size_t)seg * N;
-    uint32_t* vout = vals_out + (size_t)seg * N;
-#pragma unroll
-    for (int r = 0; r < ROUNDS; ++r) {
-        const int i = wbase + r * 64 + lane;
-        const bool valid = i < N;
-        const uint32_t digit = (key[r] >> shift) & 255u;
-        // lanes of this wave holding the same digit (match-any by 8 ballots)
-        uint64_t peers = __ballot(valid);
-#pragma unroll
-        for (int bit = 0; bit < 8; ++bit) {
-            const uint64_t m = __ballot((digit >> bit) & 1u);
-            peers &= ((digit >> bit) & 1u) ? m : ~m;
-        }
-        const uint64_t lt = (1ull << lane) - 1ull;
-        const uint32_t rank = __popcll(peers & lt);
-        uint32_t off = 0;
-        if (valid) off = run[wave][digit];
-        __syncthreads();
-        if (valid && rank == 0) run[wave][digit] = off + (uint32_t)__popcll(peers);
-        __syncthreads();
-        if (valid) {
-            kout[off + rank] = key[r];
-            vout[off + rank] = val[r];
-        }
-    }
-}
-
-int launch_radix_sort(uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
-                      uint32_t* hist, int N, int n_seg, int key_bits, hipStream_t stream) {
-    const int n_tiles = (N + kSortTile - 1) / kSortTile;
-    int passes = (key_bits + 7) / 8;
-    if (passes < 1) passes = 1;
-    uint32_t *kin = keys_a, *vin = vals_a, *kout = keys_b, *vout = vals_b;
-    for (int p = 0; p < passes; ++p) {
-        const int shift = 8 * p;
-        hipLaunchKernelGGL(k_sort_hist, dim3(n_tiles, n_seg), dim3(256), 0, stream, kin, N, n_tiles,
-                           shift, hist);
-        hipLaunchKernelGGL(k_sort_scan, dim3(n_seg), dim3(256), 0, stream, hist, n_tiles);
-        hipLaunchKernelGGL(k_sort_scatter, dim3(n_tiles, n_seg), dim3(256), 0, stream, kin, vin,
-                           kout, vout, N, n_tiles, shift, hist);
-        uint32_t* t = kin; kin = kout; kout = t;
-        t = vin; vin = vout; vout = t;
-    }
-    return (passes & 1);  // odd number of passes: result is in the b buffers
-}
-
-// ---- segments and chunks ---------------------------------------------------
-
-// exclusive scan of one value per thread over a 1024-thread block
-DEVINL uint32_t block_scan_1024(uint32_t v, uint32_t* lds /*[16]*/, uint32_t* total) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    uint32_t inc = v;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const uint32_t t = __shfl_up(inc, off, 64);
-        if (lane >= off) inc += t;
-    }
-    __syncthreads();
-    if (lane == 63) lds[wave] = inc;
-    __syncthreads();
-    uint32_t wbase = 0, tot = 0;
-#pragma unroll
-    for (int w = 0; w < 16; ++w) {
-        const uint32_t c = lds[w];
-        if (w < wave) wbase += c;
-        tot += c;
-    }
-    *total = tot;
-    return wbase + inc - v;
-}
-
-__global__ __launch_bounds__(1024) void k_find_segments(const uint32_t* __restrict__ keys,
-                                                        const uint32_t* __restrict__ vals, int N,
-                                                        int n_real, int chunk, int direct_max,
-                                                        SegPlan plan) {
-    __shared__ uint32_t lds[16];
-    const int seg = blockIdx.x, tid = threadIdx.x;
-    keys += (size_t)seg * N;
-    vals += (size_t)seg * N;
-    uint32_t* uniq_key = plan.uniq_key + (size_t)seg * plan.u_stride;
-    uint32_t* seg_start = plan.seg_start + (size_t)seg * (plan.u_stride + 1);
-    uint32_t* chunk_off = plan.chunk_off + (size_t)seg * (plan.u_stride + 1);
-    uint32_t* chunk_pos = plan.chunk_pos + (size_t)seg * plan.c_stride;
-    uint32_t* chunk_len = plan.chunk_len + (size_t)seg * plan.c_stride;
-    uint32_t* item_row = plan.item_row ? plan.item_row + (size_t)seg * n_real : nullptr;
-    uint32_t* seg_real = plan.seg_real ? plan.seg_real + (size_t)seg * plan.u_stride : nullptr;
-
-    const int per = (N + 1023) / 1024;
-    const int lo = min(N, tid * per), hi = min(N, lo + per);
-    uint32_t cnt = 0;
-    for (int i = lo; i < hi; ++i) cnt += (i == 0 || keys[i] != keys[i - 1]) ? 1u : 0u;
-    uint32_t U;
-    const uint32_t ubase = block_scan_1024(cnt, lds, &U);
-    {
-        uint32_t u = ubase;  // index of the next distinct row to start
-        for (int i = lo; i < hi; ++i) {
-            if (i == 0 || keys[i] != keys[i - 1]) {
-                uniq_key[u] = keys[i];
-                seg_start[u] = i;
-                ++u;
-            }
-            if (item_row && vals[i] < (uint32_t)n_real) item_row[vals[i]] = u - 1;
-        }
-    }
-    if (tid == 0) seg_start[U] = N;
-    __syncthreads();
-
-    const int uper = ((int)U + 1023) / 1024;
-    const int ulo = min((int)U, tid * uper), uhi = min((int)U, ulo + uper);
-    uint32_t nch = 0;
-    for (int u = ulo; u < uhi; ++u) {
-        const uint32_t s = seg_start[u], e = seg_start[u + 1];
-        // real items (value < n_real) precede the others within a segment
-        uint32_t a = s, b = e;
-        while (a < b) {
-            const uint32_t mid = (a + b) >> 1;
-            if (vals[mid] < (uint32_t)n_real) a = mid + 1; else b = mid;
-        }
-        const uint32_t real = a - s;
-        if (seg_real) seg_real[u] = real;
-        if (real > (uint32_t)direct_max) nch += (real + chunk - 1) / chunk;
-    }
-    uint32_t NC;
-    uint32_t cb = block_scan_1024(nch, lds, &NC);
-    for (int u = ulo; u < uhi; ++u) {
-        const uint32_t s = seg_start[u], e = seg_start[u + 1];
-        uint32_t a = s, b = e;
-        while (a < b) {
-            const uint32_t mid = (a + b) >> 1;
-            if (vals[mid] < (uint32_t)n_real) a = mid + 1; else b = mid;
-        }
-        const uint32_t real = a - s;
-        chunk_off[u] = cb;
-        if (real <= (uint32_t)direct_max) continue;
-        for (uint32_t l = 0; l * chunk < real; ++l) {
-            chunk_pos[cb] = s + l * chunk;
-            chunk_len[cb] = min((uint32_t)chunk, real - l * chunk);
-            ++cb;
-        }
-    }
-    if (tid == 0) {
-        chunk_off[U] = NC;
-        plan.counts[2 * seg] = U;
-        plan.counts[2 * seg + 1] = NC;
-    }
-    if (plan.hot_rows) {  // the rows with chunks, in ascending order
-        uint32_t nh = 0;
-        for (int u = ulo; u < uhi; ++u) nh += seg_real[u] > (uint32_t)direct_max ? 1u : 0u;
-        __syncthreads();  // lds is reused
-        uint32_t H;
-        uint32_t hb = block_scan_1024(nh, lds, &H);
-        uint32_t* hot = plan.hot_rows + (size_t)seg * plan.c_stride;
-        uint32_t biggest = 0;
-        for (int u = ulo; u < uhi; ++u) {
-            biggest = max(biggest, seg_real[u]);
-            if (seg_real[u] > (uint32_t)direct_max) hot[hb++] = (uint32_t)u;
-        }
-        // {rows with chunks, real items of the biggest row}
-        __syncthreads();
-        if (tid == 0) lds[0] = 0u;
-        __syncthreads();
-        atomicMax(&lds[0], biggest);
-        __syncthreads();
-        if (tid == 0) { plan.hot_count[2 * seg] = H; plan.hot_count[2 * seg + 1] = lds[0]; }
-    }
-}
-
-void launch_find_segments(const uint32_t* keys_sorted, const uint32_t* vals_sorted, int N,
-                          int n_real, int chunk, int direct_max, int n_seg, const SegPlan& plan,
-                          hipStream_t stream) {
-    hipLaunchKernelGGL(k_find_segments, dim3(n_seg), dim3(1024), 0, stream, keys_sorted,
-                       vals_sorted, N, n_real, chunk, direct_max, plan);
-}
-
-// --------------------------------------------------------------------------
 // operand gather: one wave per contribution copies its entity (or hidden) row,
 // converted to float32 and with the relation already applied for the heads
 // (predicted tail h + r, or h * r), into the dense operand matrix the scoring
@@ -2971,25 +2639,31 @@ void launch_adam_rows2(const AdamArgs& a0, const AdamArgs& a1, hipStream_t strea
     launch_adam_kernel(a0, a1, stream);
 }
 
-__global__ __launch_bounds__(64) void k_loss_finalize(const float* __restrict__ loss_part, int n_step,
-                                                      int S, int n_part, float scale,
-                                                      float* __restrict__ loss,
-                                                      const float* __restrict__ extra) {
-    const int s = blockIdx.x, lane = threadIdx.x;
+// One workgroup per shard; a fixed order of additions whatever the launch: thread t takes entries
+// t, t + 256, ... of the shard's (step, part) pairs, lanes meet by butterfly, waves in wave order.
+__global__ __launch_bounds__(256) void k_loss_finalize(const float* __restrict__ loss_part, int n_step,
+                                                       int S, int n_part, float scale,
+                                                       float* __restrict__ loss,
+                                                       const float* __restrict__ extra) {
+    __shared__ float red[4];
+    const int s = blockIdx.x, tid = threadIdx.x;
+    const int n = n_step * n_part;
     float acc = 0.f;
-    for (int i = 0; i < n_step; ++i) {
-        const float* p = loss_part + ((size_t)i * S + s) * n_part;
-        float part = 0.f;
-        for (int t = lane; t < n_part; t += 64) part += p[t];
-        acc += wave_sum(part);
-        if (extra) acc += extra[(size_t)i * S + s];
+    for (int e = tid; e < n; e += 256) {
+        const int i = e / n_part, t = e - i * n_part;
+        acc += loss_part[((size_t)i * S + s) * n_part + t];
     }
-    if (lane == 0) loss[s] = acc * scale;
+    if (extra)
+        for (int i = tid; i < n_step; i += 256) acc += extra[(size_t)i * S + s];
+    acc = wave_sum(acc);
+    if ((tid & 63) == 0) red[tid >> 6] = acc;
+    __syncthreads();
+    if (tid == 0) loss[s] = (red[0] + red[1] + red[2] + red[3]) * scale;
 }
 
 void launch_loss_finalize(const float* loss_part, int n_step, int S, int n_part, float scale,
                           float* loss, hipStream_t stream, const float* extra) {
-    hipLaunchKernelGGL(k_loss_finalize, dim3(S), dim3(64), 0, stream, loss_part, n_step, S, n_part,
+    hipLaunchKernelGGL(k_loss_finalize, dim3(S), dim3(256), 0, stream, loss_part, n_step, S, n_part,
                        scale, loss, extra);
 }
 
@@ -3458,23 +3132,6 @@ __global__ __launch_bounds__(256) void k_fill_u32(uint32_t* p, uint32_t value, i
 void launch_fill_u32(uint32_t* p, uint32_t value, int64_t n, hipStream_t stream) {
     if (n == 0) return;
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, value, n);
-}
-
-// items for a plain scatter-add: n real items keyed by idx, then one
-// zero-gradient item per table row so that every row forms a segment
-__global__ __launch_bounds__(256) void k_iota_keys(const uint32_t* __restrict__ idx,
-                                                   uint32_t* __restrict__ keys,
-                                                   uint32_t* __restrict__ vals, int64_t n,
-                                                   int64_t rows) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n + rows) return;
-    keys[i] = i < n ? idx[i] : (uint32_t)(i - n);
-    vals[i] = (uint32_t)i;
-}
-void launch_iota_keys(const uint32_t* idx, uint32_t* keys, uint32_t* vals, int64_t n, int64_t rows,
-                      hipStream_t stream) {
-    hipLaunchKernelGGL(k_iota_keys, dim3((unsigned)((n + rows + 255) / 256)), dim3(256), 0, stream,
-                       idx, keys, vals, n, rows);
 }
 
 // out[r, :] = sum of the partial rows of table row r's chunks (second level

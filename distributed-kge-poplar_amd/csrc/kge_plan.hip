@@ -1,0 +1,602 @@
+// gfx950 kernels of the plan phase: the index-only work of a training step, batched over the
+// steps of one call.
+//
+//   build_items     every head / tail contribution resolved to its table row
+//                   (remote[src][slot], the all-to-all folded into the index arithmetic,
+//                   tests/python/reference_model.py:132-138)
+//   radix sort      (row, item) order: equal rows adjacent, ordered by item number
+//   find_segments   distinct rows, their members, the chunks of rows with many contributions
+//
+// Together the device-side counterpart of the host's np.unique (unique_pad,
+// src/python/poplar_kge_dataset.py:161-164) and of the grouping multiUpdateAdd does for
+// duplicate indices (src/pag/pag.cpp:721-743).  Integer work throughout: every result is exact
+// and independent of scheduling (the only atomics are integer counters).
+#include "kge_kernels.h"
+
+#include <algorithm>
+#include <cstdint>
+
+namespace kge {
+
+#define DEVINL __device__ __forceinline__
+
+__global__ __launch_bounds__(256) void k_build_items(PlanShape ps, const uint32_t* __restrict__ remote,
+                                                     const uint32_t* __restrict__ a2a,
+                                                     const uint32_t* __restrict__ head,
+                                                     const uint32_t* __restrict__ relation,
+                                                     const uint32_t* __restrict__ tail,
+                                                     uint32_t* __restrict__ ckey,
+                                                     uint32_t* __restrict__ crel,
+                                                     uint32_t* __restrict__ clabel,
+                                                     uint32_t* __restrict__ ent_keys,
+                                                     uint32_t* __restrict__ ent_vals,
+                                                     uint32_t* __restrict__ rel_keys,
+                                                     uint32_t* __restrict__ rel_vals) {
+    const int step = ps.step0 + blockIdx.y;
+    const int S = ps.S, B = ps.B, A = ps.A, NR = ps.NR, T = S * A, nst = ps.n_step;
+    const int R = S * NR, SB = S * B;
+    const int item = blockIdx.x * 256 + threadIdx.x;
+    const int SBr = SB * ps.rel_copies;
+    const int n_rel_items = SBr + ps.n_relation * ps.rel_copies;
+    if (item < 2 * R) {
+        int src, slot;
+        if (item < SB) {
+            const int d = item / B, b = item - d * B;
+            src = d;
+            slot = head[((size_t)d * nst + step) * B + b];
+        } else if (item < R) {
+            const int cc = item - SB;
+            const int d = cc / T, t = cc - d * T;
+            const int j = t / A, i = t - j * A;
+            src = j;
+            slot = a2a[(((size_t)j * nst + step) * S + d) * A + i];
+        } else {
+            const int sl = item - R;
+            src = sl / NR;
+            slot = sl - src * NR;
+        }
+        const uint32_t base = ps.shared_table ? 0u : (uint32_t)src * (uint32_t)ps.n_entity;
+        const uint32_t key = base + remote[((size_t)src * nst + step) * NR + slot];
+        if (item < R) ckey[(size_t)step * R + item] = key;
+        ent_keys[(size_t)step * 2 * R + item] = key;
+        ent_vals[(size_t)step * 2 * R + item] = item;
+    }
+    if (item < n_rel_items) {
+        uint32_t key;
+        if (item < SBr) {
+            const int copy = item / SB, c = item - copy * SB;
+            const int d = c / B, b = c - d * B;
+            key = relation[((size_t)d * nst + step) * B + b];
+            if (copy == 0) {
+                crel[(size_t)step * SB + c] = key;
+                clabel[(size_t)step * SB + c] = tail[((size_t)d * nst + step) * B + b];
+            }
+            key += (uint32_t)(copy * ps.n_relation);
+        } else {
+            key = item - SBr;
+        }
+        rel_keys[(size_t)step * n_rel_items + item] = key;
+        rel_vals[(size_t)step * n_rel_items + item] = item;
+    }
+}
+
+void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
+                        const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
+                        uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
+                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals, hipStream_t stream) {
+    const int R = ps.S * ps.NR;
+    const int n = std::max(2 * R, (ps.S * ps.B + ps.n_relation) * ps.rel_copies);
+    dim3 grid((n + 255) / 256, ps.step_count);
+    hipLaunchKernelGGL(k_build_items, grid, dim3(256), 0, stream, ps, remote, a2a, head, relation,
+                       tail, ckey, crel, clabel, ent_keys, ent_vals, rel_keys, rel_vals);
+}
+
+// items for a plain scatter-add: n real items keyed by idx, then one
+// zero-gradient item per table row so that every row forms a segment
+__global__ __launch_bounds__(256) void k_iota_keys(const uint32_t* __restrict__ idx,
+                                                   uint32_t* __restrict__ keys,
+                                                   uint32_t* __restrict__ vals, int64_t n,
+                                                   int64_t rows) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n + rows) return;
+    keys[i] = i < n ? idx[i] : (uint32_t)(i - n);
+    vals[i] = (uint32_t)i;
+}
+void launch_iota_keys(const uint32_t* idx, uint32_t* keys, uint32_t* vals, int64_t n, int64_t rows,
+                      hipStream_t stream) {
+    hipLaunchKernelGGL(k_iota_keys, dim3((unsigned)((n + rows + 255) / 256)), dim3(256), 0, stream, idx, keys, vals,
+                       n, rows);
+}
+
+// ---- stable LSD radix sort -------------------------------------------------------------------
+// As few passes as the key width allows with digits of at most 11 bits (20-bit row numbers: two
+// passes of 10; 25 bits: 9 + 8 + 8; a relation table's 11 bits: one pass).  Two launches per
+// pass: tile histograms, then the stable scatter, whose workgroups each derive their output
+// positions from the histograms of all tiles (one round of loads; a separate scan launch, or
+// workgroups that hand results to each other through fences, both cost more than the reads).
+// hist layout: [seg][tile][digit] (digits contiguous: every access below is coalesced).
+
+SortPasses sort_passes(int key_bits) {
+    SortPasses p = {};
+    key_bits = std::max(1, key_bits);
+    p.n = (key_bits + kSortMaxBits - 1) / kSortMaxBits;
+    const int base = key_bits / p.n, extra = key_bits % p.n;
+    int shift = 0;
+    for (int i = 0; i < p.n; ++i) {
+        p.bits[i] = base + (i < extra ? 1 : 0);
+        p.shift[i] = shift;
+        shift += p.bits[i];
+    }
+    return p;
+}
+
+size_t radix_sort_hist_words(int N, int n_seg, int key_bits) {
+    const SortPasses p = sort_passes(key_bits);
+    const size_t n_tiles = ((size_t)N + kSortTile - 1) / kSortTile;
+    return (size_t)n_seg * ((size_t)1 << p.bits[0]) * n_tiles;  // the first pass has the widest digit
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void k_sort_hist(const uint32_t* __restrict__ keys, int N,
+                                                   int n_tiles, int shift,
+                                                   uint32_t* __restrict__ hist) {
+    constexpr int DIG = 1 << BITS;
+    __shared__ uint32_t h[DIG];
+    const int seg = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+    const uint32_t* k = keys + (size_t)seg * N;
+    const int base = tile * kSortTile;
+    uint32_t key[kSortTile / 256];
+#pragma unroll
+    for (int r = 0; r < kSortTile / 256; ++r) {
+        const int i = base + r * 256 + tid;
+        key[r] = i < N ? k[i] : 0u;
+    }
+    for (int d = tid; d < DIG; d += 256) h[d] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSortTile / 256; ++r)
+        if (base + r * 256 + tid < N) atomicAdd(&h[(key[r] >> shift) & (DIG - 1)], 1u);
+    __syncthreads();
+    uint32_t* hrow = hist + ((size_t)seg * n_tiles + tile) * DIG;
+    for (int d = tid; d < DIG; d += 256) hrow[d] = h[d];
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void k_sort_scatter(const uint32_t* __restrict__ keys_in,
+                                                      const uint32_t* __restrict__ vals_in,
+                                                      uint32_t* __restrict__ keys_out,
+                                                      uint32_t* __restrict__ vals_out, int N,
+                                                      int n_tiles, int shift,
+                                                      const uint32_t* __restrict__ hist) {
+    constexpr int DIG = 1 << BITS;
+    constexpr int DPT = (DIG + 255) / 256;  // digits per thread
+    // run[w][digit]: next output position for wave w's items with that digit
+    __shared__ uint32_t run[4][DIG];
+    __shared__ uint32_t s_tot[DPT * 256];   // items of each digit in all tiles, then their exclusive prefix
+    __shared__ uint32_t wtot[4];
+    const int seg = blockIdx.y, tile = blockIdx.x;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const uint32_t* kin = keys_in + (size_t)seg * N;
+    const uint32_t* vin = vals_in + (size_t)seg * N;
+    constexpr int ROUNDS = kSortTile / 256;  // rounds of 64 items per wave
+    const int wbase = tile * kSortTile + wave * (kSortTile / 4);
+
+    uint32_t key[ROUNDS], val[ROUNDS];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        const int i = wbase + r * 64 + lane;
+        key[r] = i < N ? kin[i] : 0xffffffffu;
+        val[r] = i < N ? vin[i] : 0u;
+    }
+    // This tile's first output position of every digit, from the histograms of all tiles: items
+    // of smaller digits anywhere, then items of the same digit in earlier tiles.
+    // Step 1: thread t sums digits t, t + 256, ... over the tiles (lanes read consecutive words).
+    uint32_t pre[DPT];
+    {
+        const uint32_t* hseg = hist + (size_t)seg * n_tiles * DIG;
+        uint32_t tot[DPT];
+#pragma unroll
+        for (int q = 0; q < DPT; ++q) { tot[q] = 0; pre[q] = 0; }
+        for (int t = 0; t < n_tiles; ++t) {
+#pragma unroll
+            for (int q = 0; q < DPT; ++q) {
+                const int d = q * 256 + tid;
+                const uint32_t c = d < DIG ? hseg[(size_t)t * DIG + d] : 0u;
+                tot[q] += c;
+                pre[q] += t < tile ? c : 0u;
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < DPT; ++q) s_tot[q * 256 + tid] = tot[q];
+    }
+    for (int i = tid; i < 4 * DIG; i += 256) (&run[0][0])[i] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r)
+        if (wbase + r * 64 + lane < N) atomicAdd(&run[wave][(key[r] >> shift) & (DIG - 1)], 1u);
+    {   // step 2: exclusive scan of the digit totals; thread t owns digits [t * DPT, (t + 1) * DPT)
+        uint32_t mine[DPT], sum = 0;
+#pragma unroll
+        for (int q = 0; q < DPT; ++q) { mine[q] = s_tot[tid * DPT + q]; sum += mine[q]; }
+        uint32_t inc = sum;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t t = __shfl_up(inc, off, 64);
+            if (lane >= off) inc += t;
+        }
+        if (lane == 63) wtot[wave] = inc;
+        __syncthreads();  // also: every thread has read its s_tot entries, every wave's counts are in run[][]
+        uint32_t base = inc - sum;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) base += w < wave ? wtot[w] : 0u;
+#pragma unroll
+        for (int q = 0; q < DPT; ++q) {
+            s_tot[tid * DPT + q] = base;
+            base += mine[q];
+        }
+    }
+    __syncthreads();
+    // step 3: per digit the exclusive prefix over the four waves on top of the tile's base
+#pragma unroll
+    for (int q = 0; q < DPT; ++q) {
+        const int d = q * 256 + tid;
+        if (d < DIG) {
+            uint32_t b = s_tot[d] + pre[q];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t c = run[w][d];
+                run[w][d] = b;
+                b += c;
+            }
+        }
+    }
+    __syncthreads();
+    uint32_t* kout = keys_out + (size_t)seg * N;
+    uint32_t* vout = vals_out + (size_t)seg * N;
+    // a wave's counters are its own: the rounds need no workgroup barrier, only the order of
+    // the wave's own LDS accesses
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        const int i = wbase + r * 64 + lane;
+        const bool valid = i < N;
+        const uint32_t digit = (key[r] >> shift) & (DIG - 1);
+        // lanes of this wave holding the same digit (match-any by BITS ballots)
+        uint64_t peers = __ballot(valid);
+#pragma unroll
+        for (int bit = 0; bit < BITS; ++bit) {
+            const uint64_t m = __ballot((digit >> bit) & 1u);
+            peers &= ((digit >> bit) & 1u) ? m : ~m;
+        }
+        const uint64_t lt = (1ull << lane) - 1ull;
+        const uint32_t rank = __popcll(peers & lt);
+        uint32_t off = 0;
+        if (valid) off = run[wave][digit];
+        __builtin_amdgcn_wave_barrier();
+        if (valid && rank == 0) run[wave][digit] = off + (uint32_t)__popcll(peers);
+        __builtin_amdgcn_wave_barrier();
+        if (valid) {
+            kout[off + rank] = key[r];
+            vout[off + rank] = val[r];
+        }
+    }
+}
+
+int launch_radix_sort(uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
+                      uint32_t* hist, int N, int n_seg, int key_bits, hipStream_t stream) {
+    const int n_tiles = (N + kSortTile - 1) / kSortTile;
+    const SortPasses sp = sort_passes(key_bits);
+    uint32_t *kin = keys_a, *vin = vals_a, *kout = keys_b, *vout = vals_b;
+    for (int p = 0; p < sp.n; ++p) {
+        const int shift = sp.shift[p];
+        const dim3 grid(n_tiles, n_seg);
+#define KGE_SORT_PASS(B_)                                                                                     \
+    case B_:                                                                                                  \
+        hipLaunchKernelGGL(k_sort_hist<B_>, grid, dim3(256), 0, stream, kin, N, n_tiles, shift, hist);        \
+        hipLaunchKernelGGL(k_sort_scatter<B_>, grid, dim3(256), 0, stream, kin, vin, kout, vout, N, n_tiles,  \
+                           shift, hist);                                                                      \
+        break;
+        switch (sp.bits[p]) {
+            KGE_SORT_PASS(1) KGE_SORT_PASS(2) KGE_SORT_PASS(3) KGE_SORT_PASS(4) KGE_SORT_PASS(5) KGE_SORT_PASS(6)
+            KGE_SORT_PASS(7) KGE_SORT_PASS(8) KGE_SORT_PASS(9) KGE_SORT_PASS(10) KGE_SORT_PASS(11)
+        }
+#undef KGE_SORT_PASS
+        uint32_t* t = kin; kin = kout; kout = t;
+        t = vin; vin = vout; vout = t;
+    }
+    return (sp.n & 1);  // odd number of passes: result is in the b buffers
+}
+
+// ---- segments and chunks ---------------------------------------------------------------------
+// Three launches over tiles of 2048 sorted items (256 threads x 8 consecutive items), both
+// plans of every step in each launch, nothing handed between workgroups inside a launch:
+//   1. count: row starts per tile (a row starts where the key changes) and the tile's last one
+//   2. rows:  with the earlier tiles' counts in front, every item knows its distinct-row index
+//      and its row's first position.  Within a row the gradient contributions (value < n_real)
+//      come first (the sort is stable and they have the smaller item numbers), and every row
+//      holds at least one other member (its `remote` slot / the scatter-add's one item per table
+//      row): the first of those knows the row's number of contributions and "owns" the row.
+//      The rows a tile owns are consecutive; their chunk counts are summed per tile.
+//   3. chunks: with the earlier tiles' chunk counts in front, the chunk tables of rows with more
+//      than direct_max contributions and the list of those rows.
+
+constexpr int kSegTile = 2048, kSegPer = 8;
+static_assert(kSegTile == 256 * kSegPer, "256 threads x kSegPer items");
+
+// per (array, tile): words of SegScratch::tile_info
+//   0 row starts in the tile   1 (position of the tile's last row start) + 1, 0 if none
+//   2 chunks of the rows the tile owns   3 how many of them have chunks   4 the most contributions among them
+//   5 rows the tile owns   6 the first of them
+constexpr int kSegInfo = 8;
+
+// kSegPer consecutive words from p + i0 (words past n read as zero); 16-byte loads when `vec`
+DEVINL void load_run(const uint32_t* __restrict__ p, int i0, int n, bool vec, uint32_t out[kSegPer]) {
+    if (vec && i0 + kSegPer <= n) {
+#pragma unroll
+        for (int x = 0; x < kSegPer; x += 4) {
+            const uint4 v = *reinterpret_cast<const uint4*>(p + i0 + x);
+            out[x] = v.x; out[x + 1] = v.y; out[x + 2] = v.z; out[x + 3] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int x = 0; x < kSegPer; ++x) out[x] = i0 + x < n ? p[i0 + x] : 0u;
+    }
+}
+
+struct SegWg {  // what every segment kernel derives from its block index
+    const SegJob* job;
+    int seg, tile, n_tiles, slot;  // slot: index of (job, seg) in the scratch arrays
+};
+DEVINL bool seg_workgroup(const SegJob& j0, const SegJob& j1, int n_seg, SegWg& w) {
+    const int y = blockIdx.y;
+    w.job = y >= n_seg ? &j1 : &j0;
+    w.seg = y >= n_seg ? y - n_seg : y;
+    w.slot = y;
+    w.tile = blockIdx.x;
+    w.n_tiles = (w.job->N + kSegTile - 1) / kSegTile;
+    return w.tile < w.n_tiles;
+}
+
+// (sum, max) over the workgroup's 256 threads, to every thread
+DEVINL void block_sum_max(uint32_t& a, uint32_t& b, uint32_t (*lds)[2]) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        a += __shfl_xor(a, off, 64);
+        b = max(b, __shfl_xor(b, off, 64));
+    }
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { lds[wave][0] = a; lds[wave][1] = b; }
+    __syncthreads();
+    a = lds[0][0] + lds[1][0] + lds[2][0] + lds[3][0];
+    b = max(max(lds[0][1], lds[1][1]), max(lds[2][1], lds[3][1]));
+    __syncthreads();
+}
+
+// exclusive scan of (a: sum, b: sum or maximum) over the workgroup's 256 threads in thread
+// order; total: the whole workgroup's
+template <bool MAX_B>
+DEVINL void block_scan_256(uint32_t a, uint32_t b, uint32_t (*lds)[2], uint32_t& ea, uint32_t& eb,
+                           uint32_t& ta, uint32_t& tb) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t ia = a, ib = b;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t xa = __shfl_up(ia, off, 64), xb = __shfl_up(ib, off, 64);
+        if (lane >= off) { ia += xa; ib = MAX_B ? max(ib, xb) : ib + xb; }
+    }
+    if (lane == 63) { lds[wave][0] = ia; lds[wave][1] = ib; }
+    ea = __shfl_up(ia, 1, 64); eb = __shfl_up(ib, 1, 64);
+    if (lane == 0) { ea = 0u; eb = 0u; }
+    __syncthreads();
+    ta = 0u; tb = 0u;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t ca = lds[w][0], cb = lds[w][1];
+        if (w < wave) { ea += ca; eb = MAX_B ? max(eb, cb) : eb + cb; }
+        ta += ca; tb = MAX_B ? max(tb, cb) : tb + cb;
+    }
+    __syncthreads();
+}
+
+// the row-start flags of this thread's items (bit x: item i0 + x starts a row)
+DEVINL uint32_t start_flags(const uint32_t k[kSegPer], uint32_t k_prev, int i0, int N) {
+    uint32_t flags = 0;
+#pragma unroll
+    for (int x = 0; x < kSegPer; ++x) {
+        const int i = i0 + x;
+        if (i < N && (i == 0 || k[x] != (x ? k[x - 1] : k_prev))) flags |= 1u << x;
+    }
+    return flags;
+}
+
+__global__ __launch_bounds__(256) void k_seg_count(SegJob j0, SegJob j1, int n_seg, int max_tiles,
+                                                   uint32_t* __restrict__ tile_info) {
+    __shared__ uint32_t lds[4][2];
+    SegWg w;
+    if (!seg_workgroup(j0, j1, n_seg, w)) return;
+    const int N = w.job->N, tid = threadIdx.x;
+    const uint32_t* __restrict__ keys = w.job->keys + (size_t)w.seg * N;
+    const bool vec = (reinterpret_cast<uintptr_t>(keys) & 15) == 0;
+    const int i0 = w.tile * kSegTile + kSegPer * tid;
+    uint32_t k[kSegPer];
+    load_run(keys, i0, N, vec, k);
+    const uint32_t k_prev = (i0 > 0 && i0 < N) ? keys[i0 - 1] : 0u;
+    const uint32_t flags = start_flags(k, k_prev, i0, N);
+    uint32_t cnt = __popc(flags), mx = flags ? (uint32_t)(i0 + 31 - __clz(flags)) + 1u : 0u;
+    block_sum_max(cnt, mx, lds);
+    if (tid == 0) {
+        uint32_t* info = tile_info + ((size_t)w.slot * max_tiles + w.tile) * kSegInfo;
+        info[0] = cnt; info[1] = mx;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_seg_rows(SegJob j0, SegJob j1, int n_seg, int max_tiles,
+                                                  uint32_t* __restrict__ tile_info) {
+    __shared__ uint32_t lds[4][2];
+    SegWg w;
+    if (!seg_workgroup(j0, j1, n_seg, w)) return;
+    const SegJob& job = *w.job;
+    const int N = job.N, tid = threadIdx.x, seg = w.seg;
+    const uint32_t n_real = (uint32_t)job.n_real, chunk = (uint32_t)job.chunk, direct_max = (uint32_t)job.direct_max;
+    const SegPlan& plan = job.plan;
+    const uint32_t* __restrict__ keys = job.keys + (size_t)seg * N;
+    const uint32_t* __restrict__ vals = job.vals + (size_t)seg * N;
+    uint32_t* __restrict__ uniq_key = plan.uniq_key + (size_t)seg * plan.u_stride;
+    uint32_t* __restrict__ seg_start = plan.seg_start + (size_t)seg * (plan.u_stride + 1);
+    uint32_t* __restrict__ item_row = plan.item_row ? plan.item_row + (size_t)seg * n_real : nullptr;
+    uint32_t* __restrict__ seg_real = plan.seg_real + (size_t)seg * plan.u_stride;
+    uint32_t* info_seg = tile_info + (size_t)w.slot * max_tiles * kSegInfo;
+
+    const bool vec = ((reinterpret_cast<uintptr_t>(keys) | reinterpret_cast<uintptr_t>(vals)) & 15) == 0;
+    const int i0 = w.tile * kSegTile + kSegPer * tid;
+    uint32_t k[kSegPer], v[kSegPer];
+    load_run(keys, i0, N, vec, k);
+    load_run(vals, i0, N, vec, v);
+    const bool has_prev = i0 > 0 && i0 < N;
+    const uint32_t k_prev = has_prev ? keys[i0 - 1] : 0u, v_prev = has_prev ? vals[i0 - 1] : 0u;
+    // the earlier tiles: rows started in them, and the last start among them
+    uint32_t rows_before = 0, start1_before = 0;
+    for (int t = tid; t < w.tile; t += 256) {
+        rows_before += info_seg[(size_t)t * kSegInfo];
+        start1_before = max(start1_before, info_seg[(size_t)t * kSegInfo + 1]);
+    }
+    block_sum_max(rows_before, start1_before, lds);
+
+    const uint32_t flags = start_flags(k, k_prev, i0, N);
+    const uint32_t cnt = __popc(flags), mx = flags ? (uint32_t)(i0 + 31 - __clz(flags)) + 1u : 0u;
+    uint32_t ea, eb, total_rows, total_mx;
+    block_scan_256<true>(cnt, mx, lds, ea, eb, total_rows, total_mx);
+    uint32_t u = rows_before + ea;                 // rows started in front of this thread's items
+    uint32_t start1 = max(start1_before, eb);      // (first position of the row open there) + 1
+    uint32_t own_chunks = 0, own_hot = 0, own_big = 0, own_rows = 0, own_first = 0xffffffffu;
+#pragma unroll
+    for (int x = 0; x < kSegPer; ++x) {
+        const int i = i0 + x;
+        if (i < N) {
+            const bool f = (flags >> x) & 1u;
+            if (f) {
+                uniq_key[u] = k[x];
+                seg_start[u] = (uint32_t)i;
+                start1 = (uint32_t)i + 1u;
+                ++u;
+            }
+            // u - 1 is this item's row, start1 - 1 that row's first position
+            if (v[x] < n_real) {
+                if (item_row) item_row[v[x]] = u - 1;
+            } else if (f || (x ? v[x - 1] : v_prev) < n_real) {
+                const uint32_t real = (uint32_t)i - (start1 - 1u);  // the row's contributions lie in front of it
+                seg_real[u - 1] = real;
+                const uint32_t nch = real > direct_max ? (real + chunk - 1) / chunk : 0u;
+                own_chunks += nch; own_hot += nch ? 1u : 0u; own_big = max(own_big, real);
+                own_first = min(own_first, u - 1); ++own_rows;
+            }
+        }
+    }
+    block_sum_max(own_chunks, own_big, lds);
+    uint32_t not_first = ~own_first;   // minimum through the maximum
+    block_sum_max(own_hot, not_first, lds);
+    uint32_t zero = 0;
+    block_sum_max(own_rows, zero, lds);
+    if (tid == 0) {
+        uint32_t* info = info_seg + (size_t)w.tile * kSegInfo;
+        info[2] = own_chunks; info[3] = own_hot; info[4] = own_big; info[5] = own_rows; info[6] = ~not_first;
+        if (w.tile == w.n_tiles - 1) {
+            const uint32_t U = rows_before + total_rows;
+            seg_start[U] = (uint32_t)N;
+            plan.counts[2 * seg] = U;
+            if (plan.host_counts) plan.host_counts[4 * (size_t)seg] = U;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void k_seg_chunks(SegJob j0, SegJob j1, int n_seg, int max_tiles,
+                                                    const uint32_t* __restrict__ tile_info) {
+    __shared__ uint32_t lds[4][2];
+    SegWg w;
+    if (!seg_workgroup(j0, j1, n_seg, w)) return;
+    const SegJob& job = *w.job;
+    const int tid = threadIdx.x, seg = w.seg;
+    const uint32_t chunk = (uint32_t)job.chunk, direct_max = (uint32_t)job.direct_max;
+    const SegPlan& plan = job.plan;
+    const uint32_t* __restrict__ seg_start = plan.seg_start + (size_t)seg * (plan.u_stride + 1);
+    const uint32_t* __restrict__ seg_real = plan.seg_real + (size_t)seg * plan.u_stride;
+    uint32_t* __restrict__ chunk_off = plan.chunk_off + (size_t)seg * (plan.u_stride + 1);
+    uint32_t* __restrict__ chunk_pos = plan.chunk_pos + (size_t)seg * plan.c_stride;
+    uint32_t* __restrict__ chunk_len = plan.chunk_len + (size_t)seg * plan.c_stride;
+    uint32_t* __restrict__ hot = plan.hot_rows ? plan.hot_rows + (size_t)seg * plan.c_stride : nullptr;
+    const uint32_t* info_seg = tile_info + (size_t)w.slot * max_tiles * kSegInfo;
+
+    // chunks and rows with chunks that the earlier tiles own
+    uint32_t chunks_before = 0, hot_before = 0;
+    for (int t = tid; t < w.tile; t += 256) {
+        chunks_before += info_seg[(size_t)t * kSegInfo + 2];
+        hot_before += info_seg[(size_t)t * kSegInfo + 3];
+    }
+    {
+        uint32_t z0 = 0, z1 = 0;
+        block_sum_max(chunks_before, z0, lds);
+        block_sum_max(hot_before, z1, lds);
+    }
+    const uint32_t* info = info_seg + (size_t)w.tile * kSegInfo;
+    const uint32_t own_rows = info[5], own_first = info[6];
+    // the rows this tile owns are consecutive: kSegPer of them per thread, in order
+    uint32_t real[kSegPer], nch[kSegPer], mine = 0, hot_mine = 0;
+    const uint32_t r0 = (uint32_t)(kSegPer * tid);
+#pragma unroll
+    for (int x = 0; x < kSegPer; ++x) {
+        real[x] = r0 + x < own_rows ? seg_real[own_first + r0 + x] : 0u;
+        nch[x] = real[x] > direct_max ? (real[x] + chunk - 1) / chunk : 0u;
+        mine += nch[x];
+        hot_mine += nch[x] ? 1u : 0u;
+    }
+    uint32_t ea, eb, ta, tb;
+    block_scan_256<false>(mine, hot_mine, lds, ea, eb, ta, tb);
+    uint32_t cb = chunks_before + ea, hb = hot_before + eb;
+#pragma unroll
+    for (int x = 0; x < kSegPer; ++x) {
+        if (r0 + x < own_rows) {
+            const uint32_t u = own_first + r0 + x;
+            chunk_off[u] = cb;
+            if (nch[x]) {
+                const uint32_t s = seg_start[u];
+                for (uint32_t l = 0; l < nch[x]; ++l) {
+                    chunk_pos[cb + l] = s + l * chunk;
+                    chunk_len[cb + l] = min(chunk, real[x] - l * chunk);
+                }
+                cb += nch[x];
+                if (hot) hot[hb] = u;
+                ++hb;
+            }
+        }
+    }
+    if (w.tile == w.n_tiles - 1) {  // the totals, by the workgroup that has every tile in front of it
+        uint32_t biggest = 0, z = 0;
+        for (int t = tid; t < w.n_tiles; t += 256) biggest = max(biggest, info_seg[(size_t)t * kSegInfo + 4]);
+        block_sum_max(z, biggest, lds);
+        if (tid == 0) {
+            const uint32_t U = plan.counts[2 * seg], NC = chunks_before + ta, H = hot_before + tb;
+            chunk_off[U] = NC;
+            plan.counts[2 * seg + 1] = NC;
+            if (plan.hot_count) { plan.hot_count[2 * seg] = H; plan.hot_count[2 * seg + 1] = biggest; }
+            if (plan.host_counts) {
+                uint32_t* h = plan.host_counts + 4 * (size_t)seg;
+                h[1] = NC; h[2] = H; h[3] = biggest;
+            }
+        }
+    }
+}
+
+size_t find_segments_scratch_words(int N0, int N1, int n_seg) {
+    const size_t max_tiles = ((size_t)std::max(N0, N1) + kSegTile - 1) / kSegTile;
+    return 2 * (size_t)n_seg * max_tiles * kSegInfo;
+}
+
+void launch_find_segments2(const SegJob& j0, const SegJob* j1, int n_seg, uint32_t* scratch, hipStream_t stream) {
+    const SegJob& second = j1 ? *j1 : j0;
+    const int max_tiles = (std::max(j0.N, j1 ? j1->N : 0) + kSegTile - 1) / kSegTile;
+    const dim3 grid(max_tiles, j1 ? 2 * n_seg : n_seg);
+    hipLaunchKernelGGL(k_seg_count, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
+    hipLaunchKernelGGL(k_seg_rows, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
+    hipLaunchKernelGGL(k_seg_chunks, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
+}
+
+}  // namespace kge
