@@ -1,0 +1,712 @@
+// gfx950 kernels of the scoring backward pass: l1 / l2distancegrad and the matMul backward
+// (src/pag/pag.cpp:685-700, 777-836; the distance codelets of src/poplar_extensions).
+#include "kge_device.h"
+
+#include <algorithm>
+#include <cstdint>
+
+namespace kge {
+
+// --------------------------------------------------------------------------
+// scoring: backward.  out[i, k] = sum_j c[i, j] * phi(self[i, k], other[j, k])
+//   L1   phi = signum(self - other)
+//   L2   phi = self - other              (c already holds g / dist)
+//   DOT  phi = other
+
+
+
+template <int DIST>
+__global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
+    __shared__ __attribute__((aligned(16))) float Cs[BJ][LDP];  // Cs[j][i]
+    __shared__ __attribute__((aligned(16))) float Os[BJ][LDP];  // Os[j][k]
+    const int B = p.B, T = p.T, Dp = p.Dp;
+    const int n_self = p.side_b ? T : B, n_other = p.side_b ? B : T;
+    const TileId tile = xcd_tile((Dp + kScoreTile - 1) / kScoreTile, (n_self + kScoreTile - 1) / kScoreTile, p.S);
+    const int d = tile.z, i0 = tile.y * kScoreTile, kt0 = tile.x * kScoreTile;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int self_c0 = (p.side_b ? p.b_c0 + d * T : p.a_c0 + d * B);
+    const int other_c0 = (p.side_b ? p.a_c0 + d * B : p.b_c0 + d * T);
+    const int self_rel = p.side_b ? 0 : p.a_rel_mode, other_rel = p.side_b ? p.a_rel_mode : 0;
+    const RowSource& self_src = p.side_b ? p.ent_b : p.ent_a;
+    const RowSource& other_src = p.side_b ? p.ent_a : p.ent_b;
+    const float* coef = p.coef + (size_t)d * B * T;
+    const float* cdiv = p.coef_div ? p.coef_div + (size_t)d * B * T : nullptr;
+
+    // this thread's 4x4 block of `self` (needed by L1 in the loop, by L2 at the end)
+    float sv[4][4];
+    const int kcol = kt0 + tx * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i0 + ty * 4 + i;
+        float4 v = make_float4(0, 0, 0, 0);
+        if (DIST != DIST_DOT && r < n_self && kcol < Dp) {
+            v = load4(row_ptr(self_src, self_c0 + r), kcol, self_src);
+            if (self_rel) v = combine_rel(v, p.rel + (size_t)p.crel[d * B + r] * Dp, kcol, self_rel);
+        }
+        sv[i][0] = v.x; sv[i][1] = v.y; sv[i][2] = v.z; sv[i][3] = v.w;
+    }
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[i][k] = 0.f;
+
+    for (int j0 = 0; j0 < n_other; j0 += BJ) {
+        // coefficient tile -> Cs[j][i]
+        if (!p.side_b) {
+            // c[i][j] = coef[i0+i][j0+j], contiguous over j: transposing store
+            const int li = tid >> 3, j4 = (tid & 7) * 4;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int i = li + 32 * h, gi = i0 + i, gj = j0 + j4;
+                float v[4] = {0.f, 0.f, 0.f, 0.f};
+                if (gi < B) {
+                    const float* src = coef + (size_t)gi * T + gj;
+                    if (cdiv) {
+                        const float* dv = cdiv + (size_t)gi * T + gj;
+#pragma unroll
+                        for (int x = 0; x < 4; ++x)
+                            if (gj + x < T) v[x] = dv[x] != 0.f ? src[x] / dv[x] : 0.f;
+                    } else if (gj + 3 < T && (T & 3) == 0) {
+                        const float4 t = *reinterpret_cast<const float4*>(src);
+                        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+                    } else {
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) if (gj + x < T) v[x] = src[x];
+                    }
+                }
+#pragma unroll
+                for (int x = 0; x < 4; ++x) Cs[j4 + x][i] = v[x];
+            }
+        } else {
+            // c[i][j] = coef[j0+j][i0+i], contiguous over i: direct store
+            const int lj = tid >> 4, i4 = (tid & 15) * 4;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int j = lj + 16 * h, gj = j0 + j, gi = i0 + i4;
+                float4 t = make_float4(0, 0, 0, 0);
+                if (gj < B) {
+                    const float* src = coef + (size_t)gj * T + gi;
+                    if (cdiv) {
+                        const float* dv = cdiv + (size_t)gj * T + gi;
+                        if (gi + 0 < T) t.x = dv[0] != 0.f ? src[0] / dv[0] : 0.f;
+                        if (gi + 1 < T) t.y = dv[1] != 0.f ? src[1] / dv[1] : 0.f;
+                        if (gi + 2 < T) t.z = dv[2] != 0.f ? src[2] / dv[2] : 0.f;
+                        if (gi + 3 < T) t.w = dv[3] != 0.f ? src[3] / dv[3] : 0.f;
+                    } else if (gi + 3 < T && (T & 3) == 0) {
+                        t = *reinterpret_cast<const float4*>(src);
+                    } else {
+                        if (gi + 0 < T) t.x = src[0];
+                        if (gi + 1 < T) t.y = src[1];
+                        if (gi + 2 < T) t.z = src[2];
+                        if (gi + 3 < T) t.w = src[3];
+                    }
+                }
+                *reinterpret_cast<float4*>(&Cs[j][i4]) = t;
+            }
+        }
+        // other rows -> Os[j][k]
+        {
+            const int lj = tid >> 4, kk4 = (tid & 15) * 4;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int j = lj + 16 * h, gj = j0 + j, gk = kt0 + kk4;
+                float4 t = make_float4(0, 0, 0, 0);
+                if (gj < n_other && gk < Dp) {
+                    t = load4(row_ptr(other_src, other_c0 + gj), gk, other_src);
+                    if (other_rel)
+                        t = combine_rel(t, p.rel + (size_t)p.crel[d * B + gj] * Dp, gk, other_rel);
+                }
+                *reinterpret_cast<float4*>(&Os[j][kk4]) = t;
+            }
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int jj = 0; jj < BJ; ++jj) {
+            const float4 c4 = *reinterpret_cast<const float4*>(&Cs[jj][ty * 4]);
+            const float4 o4 = *reinterpret_cast<const float4*>(&Os[jj][tx * 4]);
+            const float cv[4] = {c4.x, c4.y, c4.z, c4.w};
+            const float ov[4] = {o4.x, o4.y, o4.z, o4.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (DIST == DIST_L1) {
+                        const float t = sv[i][k] - ov[k];
+                        const float sg = (t > 0.f ? 1.f : 0.f) - (t < 0.f ? 1.f : 0.f);
+                        acc[i][k] = fmaf(cv[i], sg, acc[i][k]);
+                    } else if (DIST == DIST_L2) {
+                        acc[i][k] = fmaf(cv[i], sv[i][k] - ov[k], acc[i][k]);
+                    } else {
+                        acc[i][k] = fmaf(cv[i], ov[k], acc[i][k]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i0 + ty * 4 + i;
+        if (r >= n_self || kcol >= Dp) continue;
+        float o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            o[k] = acc[i][k];
+        }
+        float* dst = p.grad + (size_t)(p.grad_c0 + d * n_self + r) * Dp + kcol;
+        if (p.vec_out) {
+            *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) if (kcol + k < Dp) dst[k] = o[k];
+        }
+    }
+}
+
+// --------------------------------------------------------------------------
+// scoring backward on the matrix cores (L2 and dot):
+//   out[i,k] = sum_j c[i,j] other[j,k]          (a [I x J] . [J x Dp] product)
+//   L2: out[i,k] = self[i,k] * sum_j c[i,j] - that product
+// Workgroup tile 128 (self rows) x 64 (embedding columns), waves 2 x 2, each
+// wave two 32x32 accumulators; the next chunk of c and `other` is fetched into
+// registers while the matrix cores work on the current one.
+
+constexpr int BM_TI = 128, BM_TK = 64, BM_LDK = BM_TK + 4;
+// LDS of a backward workgroup: two coefficient tiles (the larger layout: 128 x 36 floats),
+// two `other` tiles (32 x 68 floats) and the 128 coefficient row sums
+constexpr int kBwdSmemBytes = 2 * (BM_TI * 36 * 4) + 2 * (32 * BM_LDK * 4) + BM_TI * 4;
+
+// BJT = rows of `other` staged per iteration (32 or 128) and NW = waves per
+// workgroup (4 or 8), chosen as in the forward kernel.
+// ALIGNED: n_self % 128 == 0, n_other % BJT == 0, Dp % 64 == 0, T % 4 == 0,
+// dense float32 operands without a relation to apply: branch-free staging loads.
+template <int DIST, int SIDE_B, int BJT, bool ALIGNED, int NW>
+DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, const int tile_y, char* smem) {
+    // Both tiles are float4 copies of global memory.  Head side: Cs[i][j] (the
+    // coefficient rows as stored), a lane reads four consecutive j of its row i
+    // in one 16-byte LDS read.  Tail side: Cs[j][i] (coefficient rows are the
+    // other operand's rows), a lane reads its column i of four rows j.
+    constexpr int NT = NW * 64;
+    constexpr int AT = 8 / NW;        // 32-row accumulator tiles per wave
+    constexpr int NCH = BJT / 32;     // 32-row sub-chunks per iteration
+    constexpr int HC = 1024 / NT;     // float4 of a 32 x 128 coefficient sub-tile per thread
+    constexpr int HO = 512 / NT;      // float4 of a 32 x 64 `other` sub-tile per thread
+    constexpr int CS_ROWS = SIDE_B ? BJT : BM_TI, CS_LD = SIDE_B ? BM_TI + 4 : BJT + 4;
+    // two copies of each tile: while the matrix cores work on one slab the next is
+    // staged into the other copy, with a single barrier per slab
+    typedef float CsTile[CS_ROWS][CS_LD];
+    typedef float OsTile[BJT][BM_LDK];
+    static_assert(2 * sizeof(CsTile) + 2 * sizeof(OsTile) + BM_TI * 4 <= kBwdSmemBytes, "LDS carve-up");
+    CsTile* Cs2 = reinterpret_cast<CsTile*>(smem);
+    OsTile* Os2 = reinterpret_cast<OsTile*>(smem + 2 * sizeof(CsTile));
+    float* csum_s = reinterpret_cast<float*>(smem + 2 * sizeof(CsTile) + 2 * sizeof(OsTile));
+    const int i0 = tile_y * BM_TI, kt0 = tile_x * BM_TK;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wi = (wave >> 1) * (32 * AT), wk = (wave & 1) * 32;
+    const int B = p.B, T = p.T, Dp = p.Dp;
+    const int n_self = SIDE_B ? T : B, n_other = SIDE_B ? B : T;
+    if (i0 >= n_self) return;  // the grid is sized for the longer side
+    const int grad_c0 = SIDE_B ? p.b_c0 : p.a_c0;
+    const int self_c0 = SIDE_B ? p.b_c0 + d * T : p.a_c0 + d * B;
+    const int other_c0 = SIDE_B ? p.a_c0 + d * B : p.b_c0 + d * T;
+    const int self_rel = SIDE_B ? 0 : p.a_rel_mode, other_rel = SIDE_B ? p.a_rel_mode : 0;
+    const RowSource& self_src = SIDE_B ? p.ent_b : p.ent_a;
+    const RowSource& other_src = SIDE_B ? p.ent_a : p.ent_b;
+    const float* coef = p.coef + (size_t)d * B * T;
+
+    floatx16 acc[AT];
+#pragma unroll
+    for (int t = 0; t < AT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+    float cs_acc = 0.f;
+    constexpr int NQ = NT / BM_TI, QL = 32 / NQ;  // threads per coefficient row, coefficients per thread and slab
+    const int crow = tid & (BM_TI - 1), cq = tid / BM_TI;
+    const int kcol = kt0 + wk + (lane & 31);
+
+    // L2: this lane's `self` values, in accumulator layout
+    float sv[AT][16];
+    if (DIST == DIST_L2) {
+#pragma unroll
+        for (int t = 0; t < AT; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = i0 + wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (ALIGNED) {
+                    sv[t][r] = reinterpret_cast<const float*>(
+                        self_src.base + (int64_t)(self_c0 + i) * self_src.pitch)[kcol];
+                    continue;
+                }
+                float v = 0.f;
+                if (i < n_self && kcol < Dp) {
+                    v = load1(row_ptr(self_src, self_c0 + i), kcol, self_src.etype);
+                    if (self_rel) {
+                        const float rv = p.rel[(size_t)p.crel[d * B + i] * Dp + kcol];
+                        v = self_rel == 1 ? v + rv : v * rv;
+                    }
+                }
+                sv[t][r] = v;
+            }
+    }
+    // near-identical-pair flags of the (self sub-tile, other chunk) blocks
+    const int MT = (B + 31) >> 5, NTL = (T + 31) >> 5;
+    const uint32_t* nflag = (DIST == DIST_L2 && p.nearflag) ? p.nearflag + (size_t)d * MT * NTL : nullptr;
+    auto flag_of = [&](int i_tile, int j_tile) -> uint32_t {
+        if (!nflag) return 0u;
+        const int mt = SIDE_B ? j_tile : i_tile, nt = SIDE_B ? i_tile : j_tile;
+        if (ALIGNED) return nflag[(size_t)mt * NTL + nt];
+        return (mt < MT && nt < NTL) ? nflag[(size_t)mt * NTL + nt] : 0u;
+    };
+    uint32_t nf_next[NCH][AT], nf_row_next[NCH];
+    floatx4 creg[NCH][HC], oreg[NCH][HO];
+    auto prefetch = [&](int jbase) __attribute__((always_inline)) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int j0 = jbase + 32 * c;
+#pragma unroll
+            for (int t = 0; t < AT; ++t) nf_next[c][t] = flag_of((i0 + wi + 32 * t) >> 5, j0 >> 5);
+            nf_row_next[c] = flag_of((i0 + (tid & (BM_TI - 1))) >> 5, j0 >> 5);
+            if constexpr (ALIGNED) {
+#pragma unroll
+                for (int h = 0; h < HC; ++h) {
+                    const int idx = tid + NT * h;
+                    const float* src = SIDE_B ? coef + (size_t)(j0 + (idx >> 5)) * T + i0 + (idx & 31) * 4
+                                              : coef + (size_t)(i0 + (idx >> 3)) * T + j0 + (idx & 7) * 4;
+                    creg[c][h] = *reinterpret_cast<const floatx4*>(src);
+                }
+#pragma unroll
+                for (int h = 0; h < HO; ++h) {
+                    const int idx = tid + NT * h;
+                    oreg[c][h] = *reinterpret_cast<const floatx4*>(
+                        other_src.base + (int64_t)(other_c0 + j0 + (idx >> 4)) * other_src.pitch +
+                        (size_t)(kt0 + (idx & 15) * 4) * 4);
+                }
+            } else {
+#pragma unroll
+            for (int h = 0; h < HC; ++h) {
+                const int idx = tid + NT * h;
+                creg[c][h] = floatx4{0.f, 0.f, 0.f, 0.f};
+                if (!SIDE_B) {  // c[i][j] = coef[i0+i][j0+j]: float4 along j
+                    const int gi = i0 + (idx >> 3), gj = j0 + (idx & 7) * 4;
+                    if (gi < B && gj < T) {
+                        const float* src = coef + (size_t)gi * T + gj;
+                        if (gj + 3 < T && (T & 3) == 0) creg[c][h] = *reinterpret_cast<const floatx4*>(src);
+                        else {
+                            creg[c][h].x = src[0];
+                            if (gj + 1 < T) creg[c][h].y = src[1];
+                            if (gj + 2 < T) creg[c][h].z = src[2];
+                            if (gj + 3 < T) creg[c][h].w = src[3];
+                        }
+                    }
+                } else {        // c[i][j] = coef[j0+j][i0+i]: float4 along i
+                    const int gj = j0 + (idx >> 5), gi = i0 + (idx & 31) * 4;
+                    if (gj < B && gi < T) {
+                        const float* src = coef + (size_t)gj * T + gi;
+                        if (gi + 3 < T && (T & 3) == 0) creg[c][h] = *reinterpret_cast<const floatx4*>(src);
+                        else {
+                            creg[c][h].x = src[0];
+                            if (gi + 1 < T) creg[c][h].y = src[1];
+                            if (gi + 2 < T) creg[c][h].z = src[2];
+                            if (gi + 3 < T) creg[c][h].w = src[3];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < HO; ++h) {
+                const int idx = tid + NT * h;
+                const int gj = j0 + (idx >> 4), gk = kt0 + (idx & 15) * 4;
+                oreg[c][h] = floatx4{0.f, 0.f, 0.f, 0.f};
+                if (gj < n_other && gk < Dp) {
+                    oreg[c][h] = as_x4(load4(row_ptr(other_src, other_c0 + gj), gk, other_src));
+                    if (other_rel)
+                        oreg[c][h] = as_x4(combine_rel(as_f4(oreg[c][h]), p.rel + (size_t)p.crel[d * B + gj] * Dp, gk, other_rel));
+                }
+            }
+            }
+        }
+    };
+    bool direct_next[NCH][AT], direct_row_next[NCH], any_direct_next[NCH];
+    // writes the prefetched slab into tile copy `nb` and latches its near-pair flags
+    auto stage = [&](int nb) __attribute__((always_inline)) {
+        CsTile& Cn = Cs2[nb];
+        OsTile& On = Os2[nb];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            any_direct_next[c] = false;
+#pragma unroll
+            for (int t = 0; t < AT; ++t) {
+                direct_next[c][t] = nf_next[c][t] != 0u;
+                any_direct_next[c] = any_direct_next[c] || direct_next[c][t];
+            }
+            direct_row_next[c] = nf_row_next[c] != 0u;
+#pragma unroll
+            for (int h = 0; h < HC; ++h) {
+                const int idx = tid + NT * h;
+                if (!SIDE_B) {
+                    *reinterpret_cast<floatx4*>(&Cn[idx >> 3][32 * c + (idx & 7) * 4]) = creg[c][h];
+                } else {
+                    *reinterpret_cast<floatx4*>(&Cn[32 * c + (idx >> 5)][(idx & 31) * 4]) = creg[c][h];
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < HO; ++h) {
+                const int idx = tid + NT * h;
+                *reinterpret_cast<floatx4*>(&On[32 * c + (idx >> 4)][(idx & 15) * 4]) = oreg[c][h];
+            }
+        }
+    };
+    prefetch(0);
+    stage(0);
+    __syncthreads();
+    if (BJT < n_other) prefetch(BJT);
+    for (int jbase = 0, buf = 0; jbase < n_other; jbase += BJT, buf ^= 1) {
+        bool direct[NCH][AT], direct_row[NCH], any_direct[NCH];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            any_direct[c] = any_direct_next[c];
+            direct_row[c] = direct_row_next[c];
+#pragma unroll
+            for (int t = 0; t < AT; ++t) direct[c][t] = direct_next[c][t];
+        }
+        if (jbase + BJT < n_other) {
+            stage(buf ^ 1);  // the other copy: last read one slab ago, before the barrier
+            if (jbase + 2 * BJT < n_other) prefetch(jbase + 2 * BJT);
+        }
+        const CsTile& Cc = Cs2[buf];
+        const OsTile& Oc = Os2[buf];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int jo = 32 * c;
+            // coefficient row sums (L2): NQ threads share a row, each adds its QL of the slab's
+            // 32 coefficients, so that every wave carries the same small load
+            if (DIST == DIST_L2 && !direct_row[c]) {
+                if (SIDE_B) {
+#pragma unroll
+                    for (int jj = 0; jj < QL; ++jj) cs_acc += Cc[jo + cq * QL + jj][crow];
+                } else {
+#pragma unroll
+                    for (int jj = 0; jj < QL; jj += 4) {
+                        const float4 v = *reinterpret_cast<const float4*>(&Cc[crow][jo + cq * QL + jj]);
+                        cs_acc += v.x; cs_acc += v.y; cs_acc += v.z; cs_acc += v.w;
+                    }
+                }
+            }
+            if (!any_direct[c]) {
+                // group g covers rows j = jo + 8g .. 8g+7 of `other`: instruction x
+                // takes row 8g + x (lower half-wave) and 8g + 4 + x (upper)
+                float ra[2][AT][4], rb[2][4];
+                const int hl = lane >> 5, cl = lane & 31;
+                auto fetch = [&](int buf, int g) {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) rb[buf][x] = Oc[jo + 8 * g + 4 * hl + x][wk + cl];
+#pragma unroll
+                    for (int t = 0; t < AT; ++t) {
+                        if (SIDE_B) {
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) ra[buf][t][x] = Cc[jo + 8 * g + 4 * hl + x][wi + 32 * t + cl];
+                        } else {
+                            const float4 v = *reinterpret_cast<const float4*>(&Cc[wi + 32 * t + cl][jo + 8 * g + 4 * hl]);
+                            ra[buf][t][0] = v.x; ra[buf][t][1] = v.y; ra[buf][t][2] = v.z; ra[buf][t][3] = v.w;
+                        }
+                    }
+                };
+                fetch(0, 0);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    if (g + 1 < 4) fetch((g + 1) & 1, g + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+#pragma unroll
+                        for (int t = 0; t < AT; ++t)
+                            acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[g & 1][t][x], rb[g & 1][x], acc[t], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                // some pair of this block is nearly identical: c * (self - other) directly,
+                // as the reference codelet does (acc holds the negated sum, see the epilogue)
+#pragma unroll
+                for (int t = 0; t < AT; ++t) {
+                    if (direct[c][t]) {
+                        for (int jj = jo; jj < jo + 32; ++jj) {
+                            const float o = Oc[jj][wk + (lane & 31)];
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                const int il = wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                                const float cc = SIDE_B ? Cc[jj][il] : Cc[il][jj];
+                                acc[t][r] = fmaf(-cc, sv[t][r] - o, acc[t][r]);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 16; ++q) {
+                            const int jj = jo + 2 * q + (lane >> 5);
+                            const float b = Oc[jj][wk + (lane & 31)];
+                            const float a = SIDE_B ? Cc[jj][wi + 32 * t + (lane & 31)] : Cc[wi + 32 * t + (lane & 31)][jj];
+                            acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[t], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (DIST == DIST_L2) {
+        // the NQ partial sums of a row, added in a fixed order (the tiles are no longer read)
+        float* part = reinterpret_cast<float*>(smem);
+        part[cq * BM_TI + crow] = cs_acc;
+        __syncthreads();
+        if (tid < BM_TI) {
+            float sum = part[tid];
+#pragma unroll
+            for (int q = 1; q < NQ; ++q) sum += part[q * BM_TI + tid];
+            csum_s[tid] = sum;
+        }
+        __syncthreads();
+    }
+    float* __restrict__ const gout = p.grad;
+    if (DIST == DIST_DOT && p.add_base) {
+        // added rows: all row ids, then all values, then the stores, so that a tile's loads are
+        // in flight together instead of sixteen dependent round trips one after the other
+        const char* __restrict__ const ab = p.add_base;
+        const uint32_t* __restrict__ const ai = p.add_index;
+        const uint32_t cnt = *p.add_count;
+#pragma unroll
+        for (int t = 0; t < AT; ++t) {
+            uint32_t row[16];
+            float addv[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = i0 + wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                row[r] = ((ALIGNED || i < n_self) && (uint32_t)i < cnt) ? ai[i] : 0u;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                addv[r] = (ALIGNED || kcol < Dp) ? load1(ab + (int64_t)row[r] * p.add_pitch, kcol, p.add_etype) : 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = i0 + wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (!ALIGNED && (i >= n_self || kcol >= Dp)) continue;
+                gout[(size_t)(grad_c0 + d * n_self + i) * Dp + kcol] = acc[t][r] + addv[r];
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int t = 0; t < AT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i_loc = wi + 32 * t + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int i = i0 + i_loc;
+            if (!ALIGNED && (i >= n_self || kcol >= Dp)) continue;
+            float o = acc[t][r];
+            if (DIST == DIST_L2) o = sv[t][r] * csum_s[i_loc] - o;
+            gout[(size_t)(grad_c0 + d * n_self + i) * Dp + kcol] = o;
+        }
+}
+
+// one side per launch (p.side_b), or both sides in one launch
+template <int DIST, int SIDE_B, int BJT, bool ALIGNED, int NW>
+__global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma(BwdParams p) {
+    __shared__ __attribute__((aligned(16))) char smem[kBwdSmemBytes];
+    const int n_self = SIDE_B ? p.T : p.B;
+    const TileId tile = xcd_tile((p.Dp + BM_TK - 1) / BM_TK, (n_self + BM_TI - 1) / BM_TI, p.S);
+    bwd_mfma_body<DIST, SIDE_B, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y, smem);
+}
+template <int DIST, int BJT, bool ALIGNED, int NW>
+__global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma_both(BwdParams p) {
+    __shared__ __attribute__((aligned(16))) char smem[kBwdSmemBytes];  // one allocation serves either side
+    // One launch for both sides. The side whose tiles loop over more rows of the other side comes
+    // first, for every block, then the other side: the long tiles do not start last (at the end of
+    // the launch the CUs run dry while the longest tiles finish), and no workgroup is started for
+    // a tile that does not exist. A block's tiles of one side stay together on one XCD; its two
+    // sides no longer run close enough in time to share the L2's copy of the operand rows and the
+    // coefficient matrix, which was measured to cost less than the late long tiles did.
+    const int gx = p.Dp / BM_TK, ga = p.B / BM_TI, gb = p.T / BM_TI;
+    const bool heads_first = p.T >= p.B;  // a head tile loops over T rows, a tail tile over B
+    const int n_first = gx * (heads_first ? ga : gb) * p.S;
+    const int L = blockIdx.x;
+    if ((L < n_first) == heads_first) {
+        const TileId tile = xcd_tile(gx, ga, p.S, heads_first ? L : L - n_first);
+        bwd_mfma_body<DIST, 0, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y, smem);
+    } else {
+        const TileId tile = xcd_tile(gx, gb, p.S, heads_first ? L - n_first : L);
+        bwd_mfma_body<DIST, 1, BJT, ALIGNED, NW>(p, tile.z, tile.x, tile.y, smem);
+    }
+}
+
+void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
+    const int n_self = p.side_b ? p.T : p.B;
+    const bool mfma_ok = p.use_mfma && !p.coef_div && p.ent_a.vec && p.ent_b.vec && (p.Dp & 3) == 0 &&
+                         (dist_fn == DIST_DOT || (dist_fn == DIST_L2 && p.nearflag));
+    if (mfma_ok) {
+        const dim3 grid = tile_grid((p.Dp + BM_TK - 1) / BM_TK, (n_self + BM_TI - 1) / BM_TI, p.S);
+        const int n_other = p.side_b ? p.B : p.T;
+        const bool plain = p.ent_a.etype == ET_F32 && p.ent_b.etype == ET_F32 && !p.ent_a.index &&
+                           !p.ent_b.index && p.a_rel_mode == 0;
+        const bool aligned = plain && n_self % BM_TI == 0 && p.Dp % BM_TK == 0 && p.T % 4 == 0 && n_other % 32 == 0;
+#define KGE_BWD(D_, S_)                                                                                     \
+    do {                                                                                                    \
+        if (aligned) hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 32, true, 8>), grid, dim3(512), 0, stream, p); \
+        else hipLaunchKernelGGL((k_score_bwd_mfma<D_, S_, 32, false, 4>), grid, dim3(256), 0, stream, p);    \
+    } while (0)
+        if (dist_fn == DIST_L2) {
+            if (p.side_b) KGE_BWD(DIST_L2, 1); else KGE_BWD(DIST_L2, 0);
+        } else {
+            if (p.side_b) KGE_BWD(DIST_DOT, 1); else KGE_BWD(DIST_DOT, 0);
+        }
+#undef KGE_BWD
+        return;
+    }
+    const dim3 grid = tile_grid((p.Dp + kScoreTile - 1) / kScoreTile, (n_self + kScoreTile - 1) / kScoreTile, p.S);
+    if (dist_fn == DIST_L1)
+        hipLaunchKernelGGL(k_score_bwd<DIST_L1>, grid, dim3(256), 0, stream, p);
+    else if (dist_fn == DIST_L2)
+        hipLaunchKernelGGL(k_score_bwd<DIST_L2>, grid, dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL(k_score_bwd<DIST_DOT>, grid, dim3(256), 0, stream, p);
+}
+
+
+// --------------------------------------------------------------------------
+// L1 backward, both sides in one pass over the pairs.  c * signum(a - b) has no
+// contraction form, so this is vector-ALU work; computing the term once and
+// adding it to the head's sum and (negated) to the tail's sum halves it.
+// One workgroup of 16 waves per (block, 64-column slice); a lane owns one
+// column.  Wave w keeps tails [w*TW, (w+1)*TW) and their gradient sums in
+// registers and walks over all heads; a head's sum over one wave's tails is a
+// partial, the 16 partials of a head meet in LDS and are added in wave order
+// (deterministic).  The coefficients of a (head, tail range) are wave-uniform
+// and come in through scalar loads.
+constexpr int L1P_CB = 16;     // heads per chunk (one per wave in the reduction)
+constexpr int L1P_WAVES = 16;
+
+template <int TW>
+__global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restrict__ operands,
+                                                            const float* __restrict__ coef,
+                                                            float* __restrict__ grad, int B, int T,
+                                                            int Dp, int a_c0, int b_c0) {
+    __shared__ float part[2][L1P_WAVES][L1P_CB][64];
+    const TileId tile = xcd_tile(Dp / 64, 1, (int)gridDim.x / (Dp / 64));
+    const int d = tile.z, k = tile.x * 64 + (threadIdx.x & 63);
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int t0 = w * TW;
+    const float* a_rows = operands + (size_t)(a_c0 + d * B) * Dp + k;
+    const float* b_rows = operands + (size_t)(b_c0 + d * T + t0) * Dp + k;
+    const float* crow = coef + (size_t)d * B * T + t0;
+
+    float bt[TW], gt[TW];
+#pragma unroll
+    for (int j = 0; j < TW; ++j) {
+        bt[j] = b_rows[(size_t)j * Dp];
+        gt[j] = 0.f;
+    }
+    for (int b0 = 0, buf = 0; b0 < B; b0 += L1P_CB, buf ^= 1) {
+        float a_next = a_rows[(size_t)b0 * Dp];
+        for (int bi = 0; bi < L1P_CB; ++bi) {
+            const float a = a_next;
+            if (bi + 1 < L1P_CB) a_next = a_rows[(size_t)(b0 + bi + 1) * Dp];
+            const float* c = crow + (size_t)(b0 + bi) * T;
+            float gp = 0.f;
+#pragma unroll
+            for (int j = 0; j < TW; ++j) {
+                // signum(a - b) with signum(0) = 0 (poplar_extensions l1distance.codelet.cpp:76-79):
+                // the difference's bit pattern read as an integer has its sign and is zero
+                // only for +0; converted to float (magnitude >= 1 unless zero) and clamped
+                // to [-1, 1].  (-0 never appears: the dense operands are stored with +0 added.)
+                const float sg = __builtin_amdgcn_fmed3f((float)__float_as_int(a - bt[j]), -1.f, 1.f);
+                gp = fmaf(c[j], sg, gp);
+                gt[j] = fmaf(-c[j], sg, gt[j]);
+            }
+            part[buf][w][bi][lane] = gp;
+        }
+        __syncthreads();
+        // wave w adds the 16 partials of head b0 + w
+        float sum = 0.f;
+#pragma unroll
+        for (int v = 0; v < L1P_WAVES; ++v) sum += part[buf][v][w][lane];
+        grad[(size_t)(a_c0 + d * B + b0 + w) * Dp + k] = sum;
+    }
+#pragma unroll
+    for (int j = 0; j < TW; ++j) grad[(size_t)(b_c0 + d * T + t0 + j) * Dp + k] = gt[j];
+}
+
+// shapes the paired L1 kernel takes: tails split evenly over 16 waves, whole
+// chunks of heads, whole 64-column slices, and enough workgroups for the chip
+static bool l1_pair_ok(const ScoreShape& sh) {
+    const int tw = sh.T / L1P_WAVES;
+    return sh.T % L1P_WAVES == 0 && (tw == 8 || tw == 16 || tw == 32) && sh.B % L1P_CB == 0 &&
+           sh.Dp % 64 == 0 && sh.S * (sh.Dp / 64) >= 128;
+}
+
+void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
+                      const uint32_t* crel, const float* coef, const uint32_t* nearflag, float* grad,
+                      hipStream_t stream) {
+    BwdParams p;
+    p.ent_a = ent; p.ent_b = ent; p.rel = rel; p.crel = crel; p.coef = coef; p.grad = grad;
+    p.coef_div = nullptr; p.add_base = nullptr;
+    p.S = sh.S; p.B = sh.B; p.T = sh.T; p.Dp = sh.Dp; p.vec_out = 1; p.use_mfma = sh.use_mfma;
+    p.nearflag = nearflag;
+    p.a_rel_mode = sh.operands_dense ? 0 : (sh.score_fn == SCORE_DISTMULT ? 2 : 1);
+    p.a_c0 = 0; p.b_c0 = sh.S * sh.B;
+    const int dist_fn = sh.score_fn == SCORE_DISTMULT ? DIST_DOT : sh.dist_fn;
+    // matrix-core path: both sides in one launch (tile-aligned shapes)
+    const bool plain = ent.etype == ET_F32 && !ent.index && p.a_rel_mode == 0 && ent.vec;
+    const bool both = sh.use_mfma && plain && sh.B % BM_TI == 0 && sh.T % BM_TI == 0 && sh.Dp % BM_TK == 0 &&
+                      (dist_fn == DIST_DOT || (dist_fn == DIST_L2 && nearflag));
+    if (both) {
+        const dim3 grid = tile_grid(sh.Dp / BM_TK, sh.B / BM_TI + sh.T / BM_TI, sh.S);
+        // eight waves per workgroup (two per SIMD): measured faster than four at
+        // every benchmark shape, few workgroups (1M-row workload) or many (22.8M-row workload)
+        if (dist_fn == DIST_L2)
+            hipLaunchKernelGGL((k_score_bwd_mfma_both<DIST_L2, 32, true, 8>), grid, dim3(512), 0, stream, p);
+        else
+            hipLaunchKernelGGL((k_score_bwd_mfma_both<DIST_DOT, 32, true, 8>), grid, dim3(512), 0, stream, p);
+        return;
+    }
+    if (dist_fn == DIST_L1 && sh.use_mfma && sh.operands_dense && plain && ent.pitch == (int64_t)sh.Dp * 4 && l1_pair_ok(sh)) {
+        const float* ops = reinterpret_cast<const float*>(ent.base);
+        const dim3 grid = tile_grid(sh.Dp / 64, 1, sh.S);
+        const int tw = sh.T / L1P_WAVES;
+        if (tw == 32)
+            hipLaunchKernelGGL(k_score_bwd_l1_pair<32>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
+        else if (tw == 16)
+            hipLaunchKernelGGL(k_score_bwd_l1_pair<16>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
+        else
+            hipLaunchKernelGGL(k_score_bwd_l1_pair<8>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
+        return;
+    }
+    p.side_b = 0; p.grad_c0 = p.a_c0;
+    launch_bwd(p, dist_fn, stream);
+    p.side_b = 1; p.grad_c0 = p.b_c0;
+    launch_bwd(p, dist_fn, stream);
+}
+
+
+static RowSource plain_rows_bwd(const float* ptr, int D) {
+    RowSource s;
+    s.base = reinterpret_cast<const char*>(ptr); s.pitch = (int64_t)D * 4; s.etype = ET_F32; s.index = nullptr;
+    s.count = D; s.vec = (D % 4 == 0) && ((uintptr_t)ptr % 16 == 0);
+    return s;
+}
+
+// g [M, N]; dist [M, N] (L2 only, else null): gradient of the first operand
+void launch_distance_grad(int dist_fn, const float* a, const float* b, const float* dist,
+                          const float* g, float* grad, int M, int N, int D, hipStream_t stream) {
+    BwdParams p;
+    p.ent_a = plain_rows_bwd(a, D); p.ent_b = plain_rows_bwd(b, D);
+    p.rel = nullptr; p.crel = nullptr;
+    p.coef = g;
+    p.coef_div = dist_fn == DIST_L2 ? dist : nullptr;
+    p.grad = grad;
+    p.S = 1; p.B = M; p.T = N; p.Dp = D;
+    p.side_b = 0; p.a_rel_mode = 0;
+    p.a_c0 = 0; p.b_c0 = 0; p.grad_c0 = 0; p.use_mfma = 1; p.nearflag = nullptr;
+    p.vec_out = (D % 4 == 0) && ((uintptr_t)grad % 16 == 0);
+    launch_bwd(p, dist_fn, stream);
+}
+
+}  // namespace kge
