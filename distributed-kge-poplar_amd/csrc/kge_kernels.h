@@ -20,7 +20,7 @@ enum { DIST_L1 = 0, DIST_L2 = 1, DIST_DOT = 2 };
 enum { LOSS_LOGSIGMOID = 0, LOSS_SOFTMAX = 1 };
 enum { ET_F32 = 0, ET_BF16 = 1, ET_F16 = 2 };
 
-constexpr int kSortTile = 2048;  // items per workgroup in one radix pass
+constexpr int kSortTile = 4096;  // items per workgroup in one radix pass
 constexpr int kScoreTile = 64;   // score tile edge (rows of either operand)
 
 // Indexed rows: logical row r is `count` elements of type `etype` starting at
