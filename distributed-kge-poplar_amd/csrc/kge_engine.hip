@@ -279,7 +279,7 @@ struct kge_engine {
     DevBuf<float> up, up_m, up_v, down, down_m, down_v, g_up, g_down;
     DevBuf<float> mlp_fproj, mlp_concat, mlp_pre, mlp_gpre, mlp_gfp, mlp_gval, p_fproj, p_concat, p_pre;
     DevBuf<float> opnd_n, cmat, dcm, transh_mm, relgrad;  // TransH: [n | tails], c, d loss / d c, its products, relation contributions
-    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, d_loss, d_alpha;
+    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, loss_step, d_loss, d_alpha;
     // [n_step][entity, relation, normal, then per feature network projection, mlp up, mlp down][S]; the relation update indexes its two
     // groups as one array (key / rows_per_alpha), a shared table's [relation, normal] pair
     // sits in the first two entries of the relation group
@@ -710,6 +710,7 @@ void allocate(kge_engine& E) {
         E.reg_loss_part.alloc(ns * S);
     }
     E.loss_part.alloc(ns * S * E.n_part);
+    E.loss_step.alloc(ns * S);
     E.d_loss.alloc(S);
     E.d_alpha.alloc(ns * 9 * S);
 
@@ -1428,7 +1429,7 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     HIP_CHECK(hipEventRecord(E.ev[2], st));
     for (int i = s0; i < s0 + sn; ++i) run_step(E, i);
     launch_loss_finalize(E.loss_part.p + (size_t)s0 * E.S * E.n_part, sn, E.S, E.n_part, 1.f / (float)sn,
-                         E.d_loss.p, st, E.reg_on ? E.reg_loss_part.p + (size_t)s0 * E.S : nullptr);
+                         E.d_loss.p, st, E.reg_on ? E.reg_loss_part.p + (size_t)s0 * E.S : nullptr, E.loss_step.p);
     HIP_CHECK(hipGetLastError());
     HIP_CHECK(hipEventRecord(E.ev[3], st));
     HIP_CHECK(hipMemcpyAsync(E.h_loss_pin, E.d_loss.p, S * 4, hipMemcpyDeviceToHost, st));

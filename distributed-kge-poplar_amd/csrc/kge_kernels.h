@@ -270,7 +270,8 @@ void launch_adam_rows_hot2(const AdamArgs& a0, const HotRows& h0, const AdamArgs
 // loss[s] = sum over steps and parts of loss_part / n_step, in a fixed order; `extra`
 // (or null) holds one more term per (step, shard).
 void launch_loss_finalize(const float* loss_part, int n_step, int S, int n_part, float scale,
-                          float* loss, hipStream_t stream, const float* extra = nullptr);
+                          float* loss, hipStream_t stream, const float* extra = nullptr,
+                          float* step_sums = nullptr);
 
 // Norm regularisers (src/poplar_kge.cpp:430-437, 463-465) on the distinct rows of one step:
 // weight * (sum_k |x_k^power|)^(1/power) of the embedding, of feature . W (hidden - embedding)

@@ -1823,8 +1823,28 @@ __global__ __launch_bounds__(256) void k_loss_finalize(const float* __restrict__
     if (tid == 0) loss[s] = (red[0] + red[1] + red[2] + red[3]) * scale;
 }
 
+// One workgroup per (step, shard): the sum of that step's parts, in the same fixed order.
+__global__ __launch_bounds__(256) void k_loss_step_sums(const float* __restrict__ loss_part, int n_part,
+                                                        float* __restrict__ step_sums) {
+    __shared__ float red[4];
+    const float* part = loss_part + (size_t)blockIdx.x * n_part;
+    const int tid = threadIdx.x;
+    float acc = 0.f;
+    for (int t = tid; t < n_part; t += 256) acc += part[t];
+    acc = wave_sum(acc);
+    if ((tid & 63) == 0) red[tid >> 6] = acc;
+    __syncthreads();
+    if (tid == 0) step_sums[blockIdx.x] = red[0] + red[1] + red[2] + red[3];
+}
+
+// `step_sums` (n_step * S floats, may be null): scratch for the two-level sum that long part lists take.
 void launch_loss_finalize(const float* loss_part, int n_step, int S, int n_part, float scale,
-                          float* loss, hipStream_t stream, const float* extra) {
+                          float* loss, hipStream_t stream, const float* extra, float* step_sums) {
+    if (step_sums && n_part > 256 && n_step > 1) {
+        hipLaunchKernelGGL(k_loss_step_sums, dim3(n_step * S), dim3(256), 0, stream, loss_part, n_part, step_sums);
+        loss_part = step_sums;
+        n_part = 1;
+    }
     hipLaunchKernelGGL(k_loss_finalize, dim3(S), dim3(256), 0, stream, loss_part, n_step, S, n_part,
                        scale, loss, extra);
 }
