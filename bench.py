@@ -103,17 +103,27 @@ def cpu_start_state(engine, settings, w, sub):
     return cfg, state
 
 
-def cpu_baseline(engine, settings, w, batch, n_check, n_cpu_steps):
-    """Times the sequential float32 oracle on the first `n_cpu_steps` steps of
-    the workload, starting from the device's own initial rows.  The first
-    `n_check` of them are run as a separate call so that their mean loss can be
-    compared with the GPU's.  Returns (json object, loss of the first call)."""
-    from oracle.kge_oracle import Oracle, make_cfg
+def cpu_port_prepare(engine, settings, w, batch, n_cpu_steps):
+    """The sequential float32 oracle's configuration and start state (the device's own initial
+    rows) for the first `n_cpu_steps` steps.  Called before the device runs a step; timed by
+    cpu_port_run after the device's timed regions, so that the device is not left idle for the
+    oracle's ~15 s right before them."""
+    from oracle.kge_oracle import make_cfg
 
-    m, d = settings.model, settings.data
     sub = {k: np.ascontiguousarray(v[:, :n_cpu_steps]) for k, v in vars(batch).items()}
     cfg, state = cpu_start_state(engine, settings, w, sub)
-    cfg = make_cfg(**cfg)
+    return make_cfg(**cfg), state, sub
+
+
+def cpu_port_run(prepared, settings, n_check):
+    """Times the oracle on the prepared steps.  The first `n_check` of them are run as a separate
+    call so that their mean loss can be compared with the GPU's.  Returns (json object, loss of
+    the first call)."""
+    from oracle.kge_oracle import Oracle
+
+    cfg, state, sub = prepared
+    m, d = settings.model, settings.data
+    n_cpu_steps = sub["remote"].shape[1]
     oracle = Oracle("f32")
     lr = settings.training.learning_rate
     t0 = time.perf_counter()
@@ -348,12 +358,14 @@ def measure(name, args, kge, torch, full):
         w["desc"] += f" [table size overridden: {args.n_entity}]"
     if args.scoring:
         w["scoring"] = args.scoring
+    if args.execution:
+        w["execution"] = {k: json.loads(v) for k, v in (kv.split("=", 1) for kv in args.execution)}
     n_total = args.warmup + args.steps
     settings = make_settings(w, n_total, kge)
     m, d = settings.model, settings.data
+    batch = make_batch(w, n_total, kge)  # host work first: the device goes from initialisation straight to the steps
     engine = kge.Engine(settings, np.full(m.n_shard, m.n_entity - 1))
     init_tables(engine, settings)
-    batch = make_batch(w, n_total, kge)
     engine.stage_batch(batch)
 
     # CPU baselines on the first steps, from the same initial state the GPU starts from.  The C
@@ -363,7 +375,7 @@ def measure(name, args, kge, torch, full):
     n_cpu = min(n_cpu, n_total)
     n_check = max(1, min(n_cpu, args.warmup))
     with_cpu = not args.no_cpu and (full or name in args.cpu_workloads)
-    port, port_loss = cpu_baseline(engine, settings, w, batch, n_check, n_cpu) if with_cpu and full else (None, None)
+    port_prepared = cpu_port_prepare(engine, settings, w, batch, n_cpu) if with_cpu and full else None
     # the worker threads this process may use: the host's share for one GPU, not the node's core count
     threads = int(os.environ.get("OMP_NUM_THREADS") or min(16, os.cpu_count()))
     torch_path = cpu_torch_prepare(engine, settings, w, batch, n_total, threads) if with_cpu else None
@@ -377,9 +389,6 @@ def measure(name, args, kge, torch, full):
         done = first
         if with_cpu:
             check = dict(gpu_loss=loss)
-            if port is not None:
-                check.update(cpu_port_loss=float(np.sum(port_loss)),
-                             cpu_port_rel_err=abs(loss - float(np.sum(port_loss))) / abs(float(np.sum(port_loss))))
         if args.warmup > done:
             engine.train_step_loop(None, step_begin=done, step_count=args.warmup - done)
 
@@ -462,7 +471,13 @@ def measure(name, args, kge, torch, full):
                                "note": f"one call over {n_total} steps, index arrays validated and uploaded "
                                        "from host memory inside the timed call"}
 
-    # the multi-threaded CPU path last: nothing of this workload's device work is timed after it
+    # the CPU paths last: nothing of this workload's device work is timed after them
+    port = None
+    if port_prepared is not None:
+        port, port_loss = cpu_port_run(port_prepared, settings, n_check)
+        if check is not None:
+            check.update(cpu_port_loss=float(np.sum(port_loss)),
+                         cpu_port_rel_err=abs(check["gpu_loss"] - float(np.sum(port_loss))) / abs(float(np.sum(port_loss))))
     cpu_torch, cpu_torch_loss = (cpu_torch_run(torch_path, settings, n_check, args.cpu_torch_seconds)
                                  if torch_path else (None, None))
     if check is not None and cpu_torch_loss is not None:
@@ -503,6 +518,8 @@ def main():
     ap.add_argument("--n-entity", type=int, default=None, help="override the table size (experiments)")
     ap.add_argument("--predict-chunk-rows", type=int, default=None,
                     help="--mode predict: tails scored per launch (experiments; default: the engine's)")
+    ap.add_argument("--execution", action="append", default=[], metavar="KEY=JSON",
+                    help="further execution.* settings, e.g. plan_side_stream=false (experiments)")
     ap.add_argument("--scoring", default=None, choices=["mfma", "mfma_bf16x3", "valu"], help="scoring kernels (default mfma_bf16x3)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -210,6 +210,7 @@ struct kge_engine {
     void* h_pin = nullptr;          // the two arrays above, the step sizes and the loss
     float* h_alpha_pin = nullptr;
     float* h_loss_pin = nullptr;
+    float* d_loss_pin = nullptr;  // the device's view of h_loss_pin: the loss kernel stores there, no copy follows
     hipEvent_t counts_ready = nullptr;
     bool counts_pending = false;
     bool counts_known = false;
@@ -279,7 +280,7 @@ struct kge_engine {
     DevBuf<float> up, up_m, up_v, down, down_m, down_v, g_up, g_down;
     DevBuf<float> mlp_fproj, mlp_concat, mlp_pre, mlp_gpre, mlp_gfp, mlp_gval, p_fproj, p_concat, p_pre;
     DevBuf<float> opnd_n, cmat, dcm, transh_mm, relgrad;  // TransH: [n | tails], c, d loss / d c, its products, relation contributions
-    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, loss_step, d_loss, d_alpha;
+    DevBuf<float> coef, dist, grad, opnd, partial, rel_partial, rel_gsum, hidden, gsum, gproj, featd, gproj_part, gemm_part, projR, loss_part, loss_step, d_alpha;
     // [n_step][entity, relation, normal, then per feature network projection, mlp up, mlp down][S]; the relation update indexes its two
     // groups as one array (key / rows_per_alpha), a shared table's [relation, normal] pair
     // sits in the first two entries of the relation group
@@ -610,6 +611,7 @@ void allocate(kge_engine& E) {
         HIP_CHECK(hipHostGetDevicePointer(&dev_view, E.h_pin, 0));
         E.d_e_counts = (uint32_t*)dev_view; E.d_r_counts = E.d_e_counts + 4 * ns;
         E.h_loss_pin = E.h_alpha_pin + ns * 9 * S;
+        E.d_loss_pin = (float*)dev_view + (E.h_loss_pin - (float*)E.h_pin);
         HIP_CHECK(hipEventCreateWithFlags(&E.counts_ready, hipEventDisableTiming));
     }
 
@@ -711,7 +713,6 @@ void allocate(kge_engine& E) {
     }
     E.loss_part.alloc(ns * S * E.n_part);
     E.loss_step.alloc(ns * S);
-    E.d_loss.alloc(S);
     E.d_alpha.alloc(ns * 9 * S);
 
     const size_t io_n = (size_t)E.S * E.rw_batch;
@@ -1429,10 +1430,9 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     HIP_CHECK(hipEventRecord(E.ev[2], st));
     for (int i = s0; i < s0 + sn; ++i) run_step(E, i);
     launch_loss_finalize(E.loss_part.p + (size_t)s0 * E.S * E.n_part, sn, E.S, E.n_part, 1.f / (float)sn,
-                         E.d_loss.p, st, E.reg_on ? E.reg_loss_part.p + (size_t)s0 * E.S : nullptr, E.loss_step.p);
+                         E.d_loss_pin, st, E.reg_on ? E.reg_loss_part.p + (size_t)s0 * E.S : nullptr, E.loss_step.p);
     HIP_CHECK(hipGetLastError());
     HIP_CHECK(hipEventRecord(E.ev[3], st));
-    HIP_CHECK(hipMemcpyAsync(E.h_loss_pin, E.d_loss.p, S * 4, hipMemcpyDeviceToHost, st));
     HIP_CHECK(hipStreamSynchronize(st));
     std::memcpy(loss, E.h_loss_pin, S * 4);
     E.step += (uint32_t)sn;
@@ -1558,7 +1558,7 @@ void run_predict(kge_engine& E, const Items& in) {
     if (E.p_idx.n < (size_t)(Qp + chunk)) {
         E.p_idx.alloc(Qp + chunk);
         E.p_rel.alloc(Qp);
-        E.p_count.alloc(1);
+        E.p_count.alloc(2);
         E.p_opnd.alloc((size_t)(Qp + chunk) * Dp);
         E.p_scores.alloc((size_t)kge_engine::kScoreBuffers * Qp * chunk);  // chunks being merged and being scored
         if (E.score_fn == SCORE_TRANSH) {
@@ -1593,6 +1593,10 @@ void run_predict(kge_engine& E, const Items& in) {
     HIP_CHECK(hipMemcpyAsync(E.p_idx.p, pin_rows, (size_t)Qp * 4, hipMemcpyHostToDevice, st));
     HIP_CHECK(hipMemcpyAsync(E.p_rel.p, pin_rels, (size_t)Qp * 4, hipMemcpyHostToDevice, st));
 
+    if (E.F) {  // the two row counts of this call's feature products (queries, a chunk of tails), uploaded once
+        const uint32_t counts[2] = {(uint32_t)Qp, (uint32_t)chunk};
+        HIP_CHECK(hipMemcpy(E.p_count.p, counts, sizeof(counts), hipMemcpyHostToDevice));
+    }
     // rows `idx[0..n)` of the table as a row source: the embeddings, or hidden = emb + feature . W
     // (`net`: the head's feature network for the queries, the tail's for the candidates)
     auto rows_of = [&](const uint32_t* idx, int n, int net) {
@@ -1600,11 +1604,10 @@ void run_predict(kge_engine& E, const Items& in) {
         r.base = E.table.p; r.pitch = E.L.pitch; r.etype = E.L.emb_etype;
         r.index = idx; r.count = Dp; r.vec = 1;
         if (E.F) {
-            const uint32_t n_u = (uint32_t)n;
-            HIP_CHECK(hipMemcpyAsync(E.p_count.p, &n_u, 4, hipMemcpyHostToDevice, st));
-            HIP_CHECK(hipStreamSynchronize(st));  // n_u leaves scope
+            // the row count as the feature kernels read it: one of the call's two constants
+            const uint32_t* count = E.p_count.p + (n == Qp ? 0 : 1);
             FeatureArgs fa = {};
-            fa.uniq_key = idx; fa.counts = E.p_count.p; fa.max_rows = n;
+            fa.uniq_key = idx; fa.counts = count; fa.max_rows = n;
             fa.emb_base = E.table.p; fa.feat_base = E.table.p + E.L.off_f; fa.pitch = E.L.pitch;
             fa.emb_etype = E.L.emb_etype; fa.feat_etype = E.L.feat_etype;
             fa.Dp = Dp; fa.Fp = E.Fp; fa.proj = E.proj.p + (size_t)net * E.Fp * Dp;
@@ -1614,7 +1617,7 @@ void run_predict(kge_engine& E, const Items& in) {
                 fp.emb_base = nullptr;
                 launch_hidden_fwd(fp, E.p_fproj.p, st);
                 MlpArgs ma = {};
-                ma.uniq_key = idx; ma.counts = E.p_count.p; ma.max_rows = n;
+                ma.uniq_key = idx; ma.counts = count; ma.max_rows = n;
                 ma.emb_base = E.table.p; ma.pitch = E.L.pitch; ma.emb_etype = E.L.emb_etype;
                 ma.Dp = Dp; ma.M = E.mlp;
                 ma.up = E.up.p + (size_t)net * 2 * Dp * E.mlp; ma.down = E.down.p + (size_t)net * E.mlp * Dp;

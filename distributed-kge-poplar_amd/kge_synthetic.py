@@ -89,6 +89,8 @@ def make_settings(w, n_step, kge):
     e.scoring_dtype = w.get("scoring_dtype")
     if w.get("scoring"):
         e.scoring = w["scoring"]
+    for key, value in w.get("execution", {}).items():  # further execution.* settings (experiments)
+        setattr(e, key, value)
     e.train_steps_per_program_run = n_step
     e.rw_batch_size = 8192
     return s.prepare()
