@@ -598,8 +598,10 @@ void allocate(kge_engine& E) {
     for (DevBuf<uint32_t>* b : {&E.ek_a, &E.ev_a, &E.ek_b, &E.ev_b}) b->alloc(ns * 2 * R);
     E.n_rel_items = (int)((SB + E.n_rel) * E.rel_copies);
     for (DevBuf<uint32_t>* b : {&E.rk_a, &E.rv_a, &E.rk_b, &E.rv_b}) b->alloc(ns * E.n_rel_items);
-    E.hist.alloc(std::max(radix_sort_hist_words((int)(2 * R), (int)ns, std::max(1, bit_length((uint64_t)E.n_rows - 1))),
-                          radix_sort_hist_words(E.n_rel_items, (int)ns, std::max(1, bit_length((uint64_t)E.n_rel_rows - 1)))));
+    {   // the two sorts of a call run in shared launches: a histogram region each, both at the wider key's digit width
+        const int bits = std::max(std::max(1, bit_length((uint64_t)E.n_rows - 1)), std::max(1, bit_length((uint64_t)E.n_rel_rows - 1)));
+        E.hist.alloc(radix_sort_hist_words((int)(2 * R), (int)ns, bits) + radix_sort_hist_words(E.n_rel_items, (int)ns, bits));
+    }
     E.seg_scratch.alloc(find_segments_scratch_words((int)(2 * R), E.n_rel_items, (int)ns));
     {   // pinned host staging: plan counts [4][2 ns], step sizes [ns 9 S], loss [S]
         const size_t words = 8 * ns + ns * 9 * S + S;  // counts [2][ns][4]
@@ -929,14 +931,22 @@ void run_plan(kge_engine& E, int s0, int sn) {
     ps.n_entity = E.n_entity; ps.shared_table = E.shared_table; ps.n_relation = E.n_rel;
     ps.rel_copies = E.rel_copies;
     ps.step0 = s0; ps.step_count = sn;
-    launch_build_items(ps, E.d_remote.p, E.d_a2a.p, E.d_head.p, E.d_relation.p, E.d_tail.p, E.ckey.p,
-                       E.crel.p, E.clabel.p, E.ek_a.p, E.ev_a.p, E.rk_a.p, E.rv_a.p, st);
     const int ebits = std::max(1, bit_length((uint64_t)E.n_rows - 1));
     const int rbits = std::max(1, bit_length((uint64_t)E.n_rel_rows - 1));
-    int which = launch_radix_sort(E.ek_a.p + s0 * N, E.ev_a.p + s0 * N, E.ek_b.p + s0 * N, E.ev_b.p + s0 * N,
-                                  E.hist.p, (int)N, sn, ebits, st);
-    const uint32_t* ek = which ? E.ek_b.p : E.ek_a.p;
-    E.e_sorted_vals = which ? E.ev_b.p : E.ev_a.p;
+    // both sorts in shared launches, the first pass's histograms from the item kernel
+    uint32_t* const e_hist = E.hist.p;
+    uint32_t* const r_hist = E.hist.p + radix_sort_hist_words((int)N, E.n_step, std::max(ebits, rbits));
+    launch_build_items(ps, E.d_remote.p, E.d_a2a.p, E.d_head.p, E.d_relation.p, E.d_tail.p, E.ckey.p,
+                       E.crel.p, E.clabel.p, E.ek_a.p, E.ev_a.p, E.rk_a.p, E.rv_a.p,
+                       sort_passes(std::max(ebits, rbits)).bits[0], e_hist, r_hist, st);
+    SortBuffers es = {}, rs = {};
+    es.keys_a = E.ek_a.p + s0 * N; es.vals_a = E.ev_a.p + s0 * N; es.keys_b = E.ek_b.p + s0 * N; es.vals_b = E.ev_b.p + s0 * N;
+    es.hist = e_hist; es.N = (int)N; es.key_bits = ebits;
+    rs.keys_a = E.rk_a.p + s0 * NRI; rs.vals_a = E.rv_a.p + s0 * NRI; rs.keys_b = E.rk_b.p + s0 * NRI; rs.vals_b = E.rv_b.p + s0 * NRI;
+    rs.hist = r_hist; rs.N = (int)NRI; rs.key_bits = rbits;
+    launch_radix_sort2(&es, &rs, sn, true, st);
+    const uint32_t* ek = es.result_in_b ? E.ek_b.p : E.ek_a.p;
+    E.e_sorted_vals = es.result_in_b ? E.ev_b.p : E.ev_a.p;
     SegJob ej = {};
     ej.keys = ek + s0 * N; ej.vals = E.e_sorted_vals + s0 * N;
     ej.N = (int)N; ej.n_real = (int)R; ej.chunk = E.chunk; ej.direct_max = E.direct_max;
@@ -953,10 +963,8 @@ void run_plan(kge_engine& E, int s0, int sn) {
     ep.hot_rows = E.e_hot.p + (size_t)s0 * ep.c_stride; ep.hot_count = E.e_hot_count.p + 2 * s0;
     ep.host_counts = E.d_e_counts + 4 * (size_t)s0;
 
-    which = launch_radix_sort(E.rk_a.p + s0 * NRI, E.rv_a.p + s0 * NRI, E.rk_b.p + s0 * NRI,
-                              E.rv_b.p + s0 * NRI, E.hist.p, (int)NRI, sn, rbits, st);
-    const uint32_t* rk = which ? E.rk_b.p : E.rk_a.p;
-    E.r_sorted_vals = which ? E.rv_b.p : E.rv_a.p;
+    const uint32_t* rk = rs.result_in_b ? E.rk_b.p : E.rk_a.p;
+    E.r_sorted_vals = rs.result_in_b ? E.rv_b.p : E.rv_a.p;
     SegJob rj = {};
     rj.keys = rk + s0 * NRI; rj.vals = E.r_sorted_vals + s0 * NRI;
     rj.N = (int)NRI; rj.n_real = (int)SB * E.rel_copies; rj.chunk = E.chunk; rj.direct_max = E.direct_max;
@@ -1103,7 +1111,8 @@ void run_step(kge_engine& E, int i) {
           g.C = E.coef.p; g.ldc = Tn; g.c_batch = (int64_t)Bn * Tn;
           g.M = Bn; g.N = Tn; g.K = Dp;
           launch_gemm_nt_bf16(g, st); }
-        { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, nullptr, loss_part, E.coef16.p, st); }
+        // only the bfloat16 coefficients are read from here on
+        { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, nullptr, loss_part, E.coef16.p, st, false); }
         { KernelTimer t(E, K_BWD);
           launch_transpose_bf16(E.opnd16.p, false, E.S, Bn, Dp, Dp, (int64_t)Bn * Dp, E.opndT16.p, nullptr, st);
           launch_transpose_bf16(E.opnd16.p + head_n, false, E.S, Tn, Dp, Dp, (int64_t)Tn * Dp,

@@ -54,10 +54,13 @@ struct PlanShape {
 // relation plan (S*B + n_relation items): head contributions, then every relation id; with
 // rel_copies = 2 both parts twice, the second copies keyed n_relation + r (item S*B + c is the
 // normal row's contribution of positive c).
+// `digit_bits`: the width of the first radix pass (sort_passes of the wider of the two key
+// widths); ent_hist / rel_hist receive every tile's digit histogram for that pass.
 void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
                         const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
                         uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
-                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals, hipStream_t stream);
+                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals, int digit_bits,
+                        uint32_t* ent_hist, uint32_t* rel_hist, hipStream_t stream);
 
 // Stable LSD radix sort of n_seg independent arrays of N (key, value) pairs on
 // the low `key_bits` bits, in sort_passes(key_bits).n passes of at most kSortMaxBits bits.
@@ -69,6 +72,19 @@ SortPasses sort_passes(int key_bits);
 size_t radix_sort_hist_words(int N, int n_seg, int key_bits);
 int launch_radix_sort(uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
                       uint32_t* hist, int N, int n_seg, int key_bits, hipStream_t stream);
+
+// Two such sorts in shared launches (the wider key's pass schedule; `schedule_bits` in the
+// histogram size: radix_sort_hist_words(N, n_seg, max of the two key widths) words per job).
+struct SortBuffers {
+    uint32_t *keys_a, *vals_a, *keys_b, *vals_b, *hist;
+    int N, key_bits;
+    int result_in_b;   // out: 1 if the sorted pairs are in keys_b / vals_b
+};
+struct SortJob {       // one job of one pass, as the kernels see it
+    uint32_t *keys_in, *vals_in, *keys_out, *vals_out, *hist;
+    int N, n_tiles;
+};
+void launch_radix_sort2(SortBuffers* j0, SortBuffers* j1, int n_seg, bool first_hist_done, hipStream_t stream);
 
 // Per-segment outputs of the segment finder, all with a per-step stride.
 struct SegPlan {
@@ -173,9 +189,10 @@ int score_fwd_parts(const ScoreShape& sh);
 
 // Row-wise losses (softmax; logsigmoid with adversarial weighting): converts
 // the raw scores in `coef` to backward coefficients in place; loss_part gets
-// S * B partial sums.
+// S * B partial sums.  `coef16` (may be null): a bfloat16 copy of the coefficients; with
+// `keep_f32` false and the softmax row held in registers only that copy is written.
 void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef, const float* dist,
-                      float* loss_part, uint16_t* coef16, hipStream_t stream);
+                      float* loss_part, uint16_t* coef16, hipStream_t stream, bool keep_f32 = true);
 
 // Stand-alone loss ops.  log_sigmoid: y = logsigmoid(x), dx = dy * its derivative (dy null: 1);
 // form 0 evaluates them as launch_loss_rows does, form 1 as the fused scoring epilogue does.

@@ -1041,7 +1041,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
                                                    float* __restrict__ coef,
                                                    const float* __restrict__ dist,
                                                    float* __restrict__ loss_part,
-                                                   uint16_t* __restrict__ coef16) {
+                                                   uint16_t* __restrict__ coef16, int keep_f32) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // d*B + b
     if (row >= sh.S * sh.B) return;
@@ -1097,7 +1097,7 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
 #pragma unroll
                     for (int x = 0; x < 4; ++x) c[x] = dv[x] != 0.f ? c[x] / dv[x] : 0.f;
                 }
-                *reinterpret_cast<floatx4*>(s + t) = c;
+                if (keep_f32) *reinterpret_cast<floatx4*>(s + t) = c;
                 if (s16) {
                     uint2 raw;
                     raw.x = (uint32_t)f32_to_bf16(c.x) | ((uint32_t)f32_to_bf16(c.y) << 16);
@@ -1163,11 +1163,11 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
 }
 
 void launch_loss_rows(const ScoreShape& sh, const uint32_t* clabel, float* coef, const float* dist,
-                      float* loss_part, uint16_t* coef16, hipStream_t stream) {
+                      float* loss_part, uint16_t* coef16, hipStream_t stream, bool keep_f32) {
     const int rows = sh.S * sh.B;
     const bool l2 = sh.score_fn != SCORE_DISTMULT && sh.dist_fn == DIST_L2;
     hipLaunchKernelGGL(k_loss_rows, dim3((rows + 3) / 4), dim3(256), 0, stream, sh, clabel, coef,
-                       l2 ? dist : nullptr, loss_part, coef16);
+                       l2 ? dist : nullptr, loss_part, coef16, (coef16 && !keep_f32) ? 0 : 1);
 }
 
 // --------------------------------------------------------------------------

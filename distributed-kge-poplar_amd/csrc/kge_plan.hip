@@ -20,7 +20,11 @@ namespace kge {
 
 #define DEVINL __device__ __forceinline__
 
-__global__ __launch_bounds__(256) void k_build_items(PlanShape ps, const uint32_t* __restrict__ remote,
+// One workgroup per sort tile (kSortTile items) of the entity items or of the relation items of
+// one step: the items' keys and values, the per-contribution arrays the step kernels read, and
+// the tile's digit histogram for the first radix pass (hist layout as k_sort_hist writes it).
+constexpr int kBuildThreads = 1024;
+__global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, const uint32_t* __restrict__ remote,
                                                      const uint32_t* __restrict__ a2a,
                                                      const uint32_t* __restrict__ head,
                                                      const uint32_t* __restrict__ relation,
@@ -31,64 +35,110 @@ __global__ __launch_bounds__(256) void k_build_items(PlanShape ps, const uint32_
                                                      uint32_t* __restrict__ ent_keys,
                                                      uint32_t* __restrict__ ent_vals,
                                                      uint32_t* __restrict__ rel_keys,
-                                                     uint32_t* __restrict__ rel_vals) {
-    const int step = ps.step0 + blockIdx.y;
+                                                     uint32_t* __restrict__ rel_vals,
+                                                     int digit_bits, uint32_t* __restrict__ ent_hist,
+                                                     uint32_t* __restrict__ rel_hist) {
+    __shared__ uint32_t h[1 << kSortMaxBits];
+    const int seg = blockIdx.y, step = ps.step0 + seg, tid = threadIdx.x;
     const int S = ps.S, B = ps.B, A = ps.A, NR = ps.NR, T = S * A, nst = ps.n_step;
     const int R = S * NR, SB = S * B;
-    const int item = blockIdx.x * 256 + threadIdx.x;
     const int SBr = SB * ps.rel_copies;
     const int n_rel_items = SBr + ps.n_relation * ps.rel_copies;
-    if (item < 2 * R) {
-        int src, slot;
-        if (item < SB) {
-            const int d = item / B, b = item - d * B;
-            src = d;
-            slot = head[((size_t)d * nst + step) * B + b];
-        } else if (item < R) {
-            const int cc = item - SB;
-            const int d = cc / T, t = cc - d * T;
-            const int j = t / A, i = t - j * A;
-            src = j;
-            slot = a2a[(((size_t)j * nst + step) * S + d) * A + i];
-        } else {
-            const int sl = item - R;
-            src = sl / NR;
-            slot = sl - src * NR;
-        }
-        const uint32_t base = ps.shared_table ? 0u : (uint32_t)src * (uint32_t)ps.n_entity;
-        const uint32_t key = base + remote[((size_t)src * nst + step) * NR + slot];
-        if (item < R) ckey[(size_t)step * R + item] = key;
-        ent_keys[(size_t)step * 2 * R + item] = key;
-        ent_vals[(size_t)step * 2 * R + item] = item;
-    }
-    if (item < n_rel_items) {
-        uint32_t key;
-        if (item < SBr) {
-            const int copy = item / SB, c = item - copy * SB;
-            const int d = c / B, b = c - d * B;
-            key = relation[((size_t)d * nst + step) * B + b];
-            if (copy == 0) {
-                crel[(size_t)step * SB + c] = key;
-                clabel[(size_t)step * SB + c] = tail[((size_t)d * nst + step) * B + b];
+    const int e_tiles = (2 * R + kSortTile - 1) / kSortTile, r_tiles = (n_rel_items + kSortTile - 1) / kSortTile;
+    const int DIG = 1 << digit_bits;
+    const bool entity = (int)blockIdx.x < e_tiles;
+    const int tile = entity ? blockIdx.x : blockIdx.x - e_tiles;
+    for (int d = tid; d < DIG; d += kBuildThreads) h[d] = 0;
+    __syncthreads();
+    constexpr int PER = kSortTile / kBuildThreads;  // items per thread; their loads go out together
+    if (entity) {
+        int item[PER], src[PER];
+        uint32_t slot[PER], key[PER];
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            item[r] = tile * kSortTile + r * kBuildThreads + tid;
+            const int it = item[r];
+            slot[r] = 0; src[r] = 0;
+            if (it < SB) {
+                const int d = it / B, b = it - d * B;
+                src[r] = d;
+                slot[r] = head[((size_t)d * nst + step) * B + b];
+            } else if (it < R) {
+                const int cc = it - SB;
+                const int d = cc / T, t = cc - d * T;
+                const int j = t / A, i = t - j * A;
+                src[r] = j;
+                slot[r] = a2a[(((size_t)j * nst + step) * S + d) * A + i];
+            } else if (it < 2 * R) {
+                const int sl = it - R;
+                src[r] = sl / NR;
+                slot[r] = sl - src[r] * NR;
             }
-            key += (uint32_t)(copy * ps.n_relation);
-        } else {
-            key = item - SBr;
         }
-        rel_keys[(size_t)step * n_rel_items + item] = key;
-        rel_vals[(size_t)step * n_rel_items + item] = item;
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const uint32_t base = ps.shared_table ? 0u : (uint32_t)src[r] * (uint32_t)ps.n_entity;
+            key[r] = item[r] < 2 * R ? base + remote[((size_t)src[r] * nst + step) * NR + slot[r]] : 0u;
+        }
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            if (item[r] >= 2 * R) continue;
+            if (item[r] < R) ckey[(size_t)step * R + item[r]] = key[r];
+            ent_keys[(size_t)step * 2 * R + item[r]] = key[r];
+            ent_vals[(size_t)step * 2 * R + item[r]] = item[r];
+            atomicAdd(&h[key[r] & (uint32_t)(DIG - 1)], 1u);
+        }
+    } else {
+        int item[PER];
+        uint32_t key[PER], label[PER];
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            item[r] = tile * kSortTile + r * kBuildThreads + tid;
+            const int it = item[r];
+            key[r] = 0; label[r] = 0;
+            if (it < SBr) {
+                const int copy = it / SB, c = it - copy * SB;
+                const int d = c / B, b = c - d * B;
+                key[r] = relation[((size_t)d * nst + step) * B + b];
+                if (copy == 0) label[r] = tail[((size_t)d * nst + step) * B + b];
+            } else if (it < n_rel_items) {
+                key[r] = it - SBr;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int it = item[r];
+            if (it >= n_rel_items) continue;
+            uint32_t k = key[r];
+            if (it < SBr) {
+                const int copy = it / SB, c = it - copy * SB;
+                if (copy == 0) {
+                    crel[(size_t)step * SB + c] = k;
+                    clabel[(size_t)step * SB + c] = label[r];
+                }
+                k += (uint32_t)(copy * ps.n_relation);
+            }
+            rel_keys[(size_t)step * n_rel_items + it] = k;
+            rel_vals[(size_t)step * n_rel_items + it] = it;
+            atomicAdd(&h[k & (uint32_t)(DIG - 1)], 1u);
+        }
     }
+    __syncthreads();
+    uint32_t* hrow = (entity ? ent_hist : rel_hist) + ((size_t)seg * (entity ? e_tiles : r_tiles) + tile) * DIG;
+    for (int d = tid; d < DIG; d += kBuildThreads) hrow[d] = h[d];
 }
 
 void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
                         const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
                         uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
-                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals, hipStream_t stream) {
-    const int R = ps.S * ps.NR;
-    const int n = std::max(2 * R, (ps.S * ps.B + ps.n_relation) * ps.rel_copies);
-    dim3 grid((n + 255) / 256, ps.step_count);
-    hipLaunchKernelGGL(k_build_items, grid, dim3(256), 0, stream, ps, remote, a2a, head, relation,
-                       tail, ckey, crel, clabel, ent_keys, ent_vals, rel_keys, rel_vals);
+                        uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals, int digit_bits,
+                        uint32_t* ent_hist, uint32_t* rel_hist, hipStream_t stream) {
+    const int R = ps.S * ps.NR, n_rel_items = (ps.S * ps.B + ps.n_relation) * ps.rel_copies;
+    const int e_tiles = (2 * R + kSortTile - 1) / kSortTile, r_tiles = (n_rel_items + kSortTile - 1) / kSortTile;
+    dim3 grid(e_tiles + r_tiles, ps.step_count);
+    hipLaunchKernelGGL(k_build_items, grid, dim3(kBuildThreads), 0, stream, ps, remote, a2a, head, relation,
+                       tail, ckey, crel, clabel, ent_keys, ent_vals, rel_keys, rel_vals, digit_bits, ent_hist,
+                       rel_hist);
 }
 
 // items for a plain scatter-add: n real items keyed by idx, then one
@@ -111,7 +161,8 @@ void launch_iota_keys(const uint32_t* idx, uint32_t* keys, uint32_t* vals, int64
 // ---- stable LSD radix sort -------------------------------------------------------------------
 // As few passes as the key width allows with digits of at most 11 bits (20-bit row numbers: two
 // passes of 10; 25 bits: 9 + 8 + 8; a relation table's 11 bits: one pass).  Two launches per
-// pass: tile histograms, then the stable scatter, whose workgroups each derive their output
+// pass (the first pass's histograms come from k_build_items; the entity and the relation sort
+// of a training call share their launches): tile histograms, then the stable scatter, whose workgroups each derive their output
 // positions from the histograms of all tiles (one round of loads; a separate scan launch, or
 // workgroups that hand results to each other through fences, both cost more than the reads).
 // hist layout: [seg][tile][digit] (digits contiguous: every access below is coalesced).
@@ -136,14 +187,22 @@ size_t radix_sort_hist_words(int N, int n_seg, int key_bits) {
     return (size_t)n_seg * ((size_t)1 << p.bits[0]) * n_tiles;  // the first pass has the widest digit
 }
 
+// Which of a launch's two jobs a workgroup serves: blockIdx.x counts job 0's tiles, then job 1's.
+DEVINL const SortJob& sort_job(const SortJob& j0, const SortJob& j1, int& tile) {
+    tile = blockIdx.x;
+    if (tile < j0.n_tiles) return j0;
+    tile -= j0.n_tiles;
+    return j1;
+}
+
 template <int BITS>
-__global__ __launch_bounds__(256) void k_sort_hist(const uint32_t* __restrict__ keys, int N,
-                                                   int n_tiles, int shift,
-                                                   uint32_t* __restrict__ hist) {
+__global__ __launch_bounds__(256) void k_sort_hist(SortJob j0, SortJob j1, int shift) {
     constexpr int DIG = 1 << BITS;
     __shared__ uint32_t h[DIG];
-    const int seg = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
-    const uint32_t* k = keys + (size_t)seg * N;
+    int tile;
+    const SortJob& job = sort_job(j0, j1, tile);
+    const int seg = blockIdx.y, tid = threadIdx.x, N = job.N;
+    const uint32_t* __restrict__ k = job.keys_in + (size_t)seg * N;
     const int base = tile * kSortTile;
     uint32_t key[kSortTile / 256];
 #pragma unroll
@@ -157,27 +216,25 @@ __global__ __launch_bounds__(256) void k_sort_hist(const uint32_t* __restrict__ 
     for (int r = 0; r < kSortTile / 256; ++r)
         if (base + r * 256 + tid < N) atomicAdd(&h[(key[r] >> shift) & (DIG - 1)], 1u);
     __syncthreads();
-    uint32_t* hrow = hist + ((size_t)seg * n_tiles + tile) * DIG;
+    uint32_t* hrow = job.hist + ((size_t)seg * job.n_tiles + tile) * DIG;
     for (int d = tid; d < DIG; d += 256) hrow[d] = h[d];
 }
 
 template <int BITS>
-__global__ __launch_bounds__(256) void k_sort_scatter(const uint32_t* __restrict__ keys_in,
-                                                      const uint32_t* __restrict__ vals_in,
-                                                      uint32_t* __restrict__ keys_out,
-                                                      uint32_t* __restrict__ vals_out, int N,
-                                                      int n_tiles, int shift,
-                                                      const uint32_t* __restrict__ hist) {
+__global__ __launch_bounds__(256) void k_sort_scatter(SortJob j0, SortJob j1, int shift) {
     constexpr int DIG = 1 << BITS;
     constexpr int DPT = (DIG + 255) / 256;  // digits per thread
     // run[w][digit]: next output position for wave w's items with that digit
     __shared__ uint32_t run[4][DIG];
     __shared__ uint32_t s_tot[DPT * 256];   // items of each digit in all tiles, then their exclusive prefix
     __shared__ uint32_t wtot[4];
-    const int seg = blockIdx.y, tile = blockIdx.x;
+    int tile;
+    const SortJob& job = sort_job(j0, j1, tile);
+    const int seg = blockIdx.y, N = job.N, n_tiles = job.n_tiles;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const uint32_t* kin = keys_in + (size_t)seg * N;
-    const uint32_t* vin = vals_in + (size_t)seg * N;
+    const uint32_t* __restrict__ kin = job.keys_in + (size_t)seg * N;
+    const uint32_t* __restrict__ vin = job.vals_in + (size_t)seg * N;
+    const uint32_t* __restrict__ hist = job.hist;
     constexpr int ROUNDS = kSortTile / 256;  // rounds of 64 items per wave
     const int wbase = tile * kSortTile + wave * (kSortTile / 4);
 
@@ -251,8 +308,8 @@ __global__ __launch_bounds__(256) void k_sort_scatter(const uint32_t* __restrict
         }
     }
     __syncthreads();
-    uint32_t* kout = keys_out + (size_t)seg * N;
-    uint32_t* vout = vals_out + (size_t)seg * N;
+    uint32_t* __restrict__ kout = job.keys_out + (size_t)seg * N;
+    uint32_t* __restrict__ vout = job.vals_out + (size_t)seg * N;
     // a wave's counters are its own: the rounds need no workgroup barrier, only the order of
     // the wave's own LDS accesses
 #pragma unroll
@@ -281,35 +338,65 @@ __global__ __launch_bounds__(256) void k_sort_scatter(const uint32_t* __restrict
     }
 }
 
-int launch_radix_sort(uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
-                      uint32_t* hist, int N, int n_seg, int key_bits, hipStream_t stream) {
-    const int n_tiles = (N + kSortTile - 1) / kSortTile;
-    const SortPasses sp = sort_passes(key_bits);
-    uint32_t *kin = keys_a, *vin = vals_a, *kout = keys_b, *vout = vals_b;
+// Two sorts in shared launches.  The pass schedule is that of the wider key; a job takes part in
+// the passes that still cover bits of its own keys (a prefix of them) and ends in its b buffers
+// after an odd number of passes.  `first_hist_done`: the caller has already written both jobs'
+// histograms of pass 0 (k_build_items).  j1 may be null.
+void launch_radix_sort2(SortBuffers* j0, SortBuffers* j1, int n_seg, bool first_hist_done, hipStream_t stream) {
+    const SortPasses sp = sort_passes(std::max(j0->key_bits, j1 ? j1->key_bits : 1));
+    SortBuffers* jobs[2] = {j0, j1};
+    SortJob cur[2] = {};
+    for (int q = 0; q < 2; ++q) {
+        if (!jobs[q]) continue;
+        cur[q].keys_in = jobs[q]->keys_a; cur[q].vals_in = jobs[q]->vals_a;
+        cur[q].keys_out = jobs[q]->keys_b; cur[q].vals_out = jobs[q]->vals_b;
+        cur[q].hist = jobs[q]->hist; cur[q].N = jobs[q]->N;
+        cur[q].n_tiles = (jobs[q]->N + kSortTile - 1) / kSortTile;
+        jobs[q]->result_in_b = 0;
+    }
     for (int p = 0; p < sp.n; ++p) {
         const int shift = sp.shift[p];
-        const dim3 grid(n_tiles, n_seg);
+        SortJob a[2] = {};
+        int n = 0;
+        for (int q = 0; q < 2; ++q)
+            if (jobs[q] && (p == 0 || shift < jobs[q]->key_bits)) a[n++] = cur[q];
+        if (n == 0) break;
+        if (n == 1) a[1].n_tiles = 0;
+        const dim3 grid(a[0].n_tiles + a[1].n_tiles, n_seg);
+        const bool hist_done = p == 0 && first_hist_done;
 #define KGE_SORT_PASS(B_)                                                                                     \
     case B_:                                                                                                  \
-        hipLaunchKernelGGL(k_sort_hist<B_>, grid, dim3(256), 0, stream, kin, N, n_tiles, shift, hist);        \
-        hipLaunchKernelGGL(k_sort_scatter<B_>, grid, dim3(256), 0, stream, kin, vin, kout, vout, N, n_tiles,  \
-                           shift, hist);                                                                      \
+        if (!hist_done) hipLaunchKernelGGL(k_sort_hist<B_>, grid, dim3(256), 0, stream, a[0], a[1], shift);   \
+        hipLaunchKernelGGL(k_sort_scatter<B_>, grid, dim3(256), 0, stream, a[0], a[1], shift);                \
         break;
         switch (sp.bits[p]) {
             KGE_SORT_PASS(1) KGE_SORT_PASS(2) KGE_SORT_PASS(3) KGE_SORT_PASS(4) KGE_SORT_PASS(5) KGE_SORT_PASS(6)
             KGE_SORT_PASS(7) KGE_SORT_PASS(8) KGE_SORT_PASS(9) KGE_SORT_PASS(10) KGE_SORT_PASS(11)
         }
 #undef KGE_SORT_PASS
-        uint32_t* t = kin; kin = kout; kout = t;
-        t = vin; vin = vout; vout = t;
+        for (int q = 0; q < 2; ++q)
+            if (jobs[q] && (p == 0 || shift < jobs[q]->key_bits)) {
+                std::swap(cur[q].keys_in, cur[q].keys_out);
+                std::swap(cur[q].vals_in, cur[q].vals_out);
+                jobs[q]->result_in_b ^= 1;
+            }
     }
-    return (sp.n & 1);  // odd number of passes: result is in the b buffers
+}
+
+int launch_radix_sort(uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
+                      uint32_t* hist, int N, int n_seg, int key_bits, hipStream_t stream) {
+    SortBuffers j = {};
+    j.keys_a = keys_a; j.vals_a = vals_a; j.keys_b = keys_b; j.vals_b = vals_b; j.hist = hist;
+    j.N = N; j.key_bits = key_bits;
+    launch_radix_sort2(&j, nullptr, n_seg, false, stream);
+    return j.result_in_b;
 }
 
 // ---- segments and chunks ---------------------------------------------------------------------
 // Three launches over tiles of 2048 sorted items (256 threads x 8 consecutive items), both
 // plans of every step in each launch, nothing handed between workgroups inside a launch:
 //   1. count: row starts per tile (a row starts where the key changes) and the tile's last one
+//      (short arrays skip this launch: the workgroups of 2. read the keys in front of their tile)
 //   2. rows:  with the earlier tiles' counts in front, every item knows its distinct-row index
 //      and its row's first position.  Within a row the gradient contributions (value < n_real)
 //      come first (the sort is stable and they have the smaller item numbers), and every row
@@ -327,6 +414,7 @@ static_assert(kSegTile == 256 * kSegPer, "256 threads x kSegPer items");
 //   2 chunks of the rows the tile owns   3 how many of them have chunks   4 the most contributions among them
 //   5 rows the tile owns   6 the first of them
 constexpr int kSegInfo = 8;
+constexpr int kSegInlineTiles = 0;   // (0: the count launch always runs)
 
 // kSegPer consecutive words from p + i0 (words past n read as zero); 16-byte loads when `vec`
 DEVINL void load_run(const uint32_t* __restrict__ p, int i0, int n, bool vec, uint32_t out[kSegPer]) {
@@ -429,6 +517,10 @@ __global__ __launch_bounds__(256) void k_seg_count(SegJob j0, SegJob j1, int n_s
     }
 }
 
+// COUNT_INLINE: no k_seg_count launch went before; every workgroup counts the row starts of the
+// tiles in front of it itself (one pass over their keys: cheaper than a launch while the
+// arrays are short).
+template <bool COUNT_INLINE>
 __global__ __launch_bounds__(256) void k_seg_rows(SegJob j0, SegJob j1, int n_seg, int max_tiles,
                                                   uint32_t* __restrict__ tile_info) {
     __shared__ uint32_t lds[4][2];
@@ -455,9 +547,28 @@ __global__ __launch_bounds__(256) void k_seg_rows(SegJob j0, SegJob j1, int n_se
     const uint32_t k_prev = has_prev ? keys[i0 - 1] : 0u, v_prev = has_prev ? vals[i0 - 1] : 0u;
     // the earlier tiles: rows started in them, and the last start among them
     uint32_t rows_before = 0, start1_before = 0;
-    for (int t = tid; t < w.tile; t += 256) {
-        rows_before += info_seg[(size_t)t * kSegInfo];
-        start1_before = max(start1_before, info_seg[(size_t)t * kSegInfo + 1]);
+    if (COUNT_INLINE) {
+        const int n_prev = w.tile * kSegTile;  // a multiple of 4, at most N
+        for (int p = 4 * tid; p < n_prev; p += 4 * 256) {
+            uint32_t q[4];
+            if (vec) {
+                const uint4 v4 = *reinterpret_cast<const uint4*>(keys + p);
+                q[0] = v4.x; q[1] = v4.y; q[2] = v4.z; q[3] = v4.w;
+            } else {
+#pragma unroll
+                for (int x = 0; x < 4; ++x) q[x] = keys[p + x];
+            }
+            const uint32_t before = p ? keys[p - 1] : ~q[0];  // position 0 starts a row
+            uint32_t f = (q[0] != before ? 1u : 0u) | (q[1] != q[0] ? 2u : 0u) | (q[2] != q[1] ? 4u : 0u) |
+                         (q[3] != q[2] ? 8u : 0u);
+            rows_before += __popc(f);
+            if (f) start1_before = (uint32_t)(p + 31 - __clz(f)) + 1u;  // positions grow with the loop
+        }
+    } else {
+        for (int t = tid; t < w.tile; t += 256) {
+            rows_before += info_seg[(size_t)t * kSegInfo];
+            start1_before = max(start1_before, info_seg[(size_t)t * kSegInfo + 1]);
+        }
     }
     block_sum_max(rows_before, start1_before, lds);
 
@@ -594,8 +705,13 @@ void launch_find_segments2(const SegJob& j0, const SegJob* j1, int n_seg, uint32
     const SegJob& second = j1 ? *j1 : j0;
     const int max_tiles = (std::max(j0.N, j1 ? j1->N : 0) + kSegTile - 1) / kSegTile;
     const dim3 grid(max_tiles, j1 ? 2 * n_seg : n_seg);
-    hipLaunchKernelGGL(k_seg_count, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
-    hipLaunchKernelGGL(k_seg_rows, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
+    // up to kSegInlineTiles tiles per array the row kernel counts the tiles in front of it itself
+    if (max_tiles <= kSegInlineTiles) {
+        hipLaunchKernelGGL(k_seg_rows<true>, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
+    } else {
+        hipLaunchKernelGGL(k_seg_count, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
+        hipLaunchKernelGGL(k_seg_rows<false>, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
+    }
     hipLaunchKernelGGL(k_seg_chunks, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
 }
 
