@@ -114,3 +114,14 @@ def test_plan_unique_pad_layout_bit_exact(shared):
                  relation=rng.integers(0, 52, (S, n_step, B)).astype(np.uint32),
                  tail=rng.integers(0, S * A, (S, n_step, B)).astype(np.uint32))
     _check_plan(c, batch, n_step)
+
+
+@pytest.mark.parametrize("n_entity,n_relation", [(50, 5000), (3000, 300), (70_000, 3)])
+def test_plan_shared_sort_launches_key_widths(n_entity, n_relation):
+    """The entity and the relation sort share their launches on the wider key's pass schedule:
+    relation keys wider than entity keys (13 bits against 6: the entity sort takes part in the
+    first of two passes only), about equal, and much narrower (2 bits against 17)."""
+    c = K.cfg_dict(n_shard=2, batch=160, a2a=40, n_entity=n_entity, n_relation=n_relation, dim=8, feature=0,
+                   shared_table=True)
+    rng = np.random.default_rng(21)
+    _check_plan(c, K.raw_batch(c, 3, rng), 3)
