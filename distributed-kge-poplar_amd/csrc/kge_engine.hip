@@ -1113,20 +1113,28 @@ void run_step(kge_engine& E, int i) {
           launch_gemm_nt_bf16(g, st); }
         // only the bfloat16 coefficients are read from here on
         { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, nullptr, loss_part, E.coef16.p, st, false); }
+        // q^T and tails^T: one launch over all operand rows when there is a single block
+        // (rows [0, B) heads, [B, B + T) tails: the transposed matrix [Dp, B + T] holds both)
+        const bool one_block = E.S == 1;
+        const int64_t ldT = one_block ? Bn + Tn : 0;
         { KernelTimer t(E, K_BWD);
-          launch_transpose_bf16(E.opnd16.p, false, E.S, Bn, Dp, Dp, (int64_t)Bn * Dp, E.opndT16.p, nullptr, st);
-          launch_transpose_bf16(E.opnd16.p + head_n, false, E.S, Tn, Dp, Dp, (int64_t)Tn * Dp,
-                                E.opndT16.p + head_n, nullptr, st);
+          if (one_block) {
+              launch_transpose_bf16(E.opnd16.p, false, 1, Bn + Tn, Dp, Dp, 0, E.opndT16.p, nullptr, st);
+          } else {
+              launch_transpose_bf16(E.opnd16.p, false, E.S, Bn, Dp, Dp, (int64_t)Bn * Dp, E.opndT16.p, nullptr, st);
+              launch_transpose_bf16(E.opnd16.p + head_n, false, E.S, Tn, Dp, Dp, (int64_t)Tn * Dp,
+                                    E.opndT16.p + head_n, nullptr, st);
+          }
           launch_transpose_bf16(E.coef16.p, false, E.S, Bn, Tn, Tn, (int64_t)Bn * Tn, E.coefT16.p, nullptr, st);
           // d q [B, Dp] = c [B, T] . tails [T, Dp]
           g.A = E.coef16.p; g.lda = Tn; g.a_batch = (int64_t)Bn * Tn;
-          g.Bt = E.opndT16.p + head_n; g.ldb = Tn; g.b_batch = (int64_t)Dp * Tn;
+          g.Bt = one_block ? E.opndT16.p + Bn : E.opndT16.p + head_n; g.ldb = one_block ? (int)ldT : Tn; g.b_batch = (int64_t)Dp * Tn;
           g.C = E.grad.p; g.ldc = Dp; g.c_batch = (int64_t)Bn * Dp;
           g.M = Bn; g.N = Dp; g.K = Tn; g.part = E.gemm_part.p;
           launch_gemm_nt_bf16(g, st);
           // d tails [T, Dp] = c^T [T, B] . q [B, Dp]
           g.A = E.coefT16.p; g.lda = Bn; g.a_batch = (int64_t)Tn * Bn;
-          g.Bt = E.opndT16.p; g.ldb = Bn; g.b_batch = (int64_t)Dp * Bn;
+          g.Bt = E.opndT16.p; g.ldb = one_block ? (int)ldT : Bn; g.b_batch = (int64_t)Dp * Bn;
           g.C = E.grad.p + head_n; g.ldc = Dp; g.c_batch = (int64_t)Tn * Dp;
           g.M = Tn; g.N = Dp; g.K = Bn;
           launch_gemm_nt_bf16(g, st); }
@@ -1297,8 +1305,15 @@ void run_step(kge_engine& E, int i) {
         // rows unless its gradient was materialised: do that with a zero-step pass
         ar.grad_out = E.rel_gsum.p;
         ar.no_update = 1;
-        { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
-        entity_update();
+        if (E.F && !E.mlp && !roles) {
+            // with entity features the relation rows' contributions read the hidden rows formed
+            // at the start of the step, not the table: their sum can share the entity update's launch
+            KernelTimer t(E, K_ADAM_ENT);
+            launch_adam_rows2(ar, ae, st);
+        } else {
+            { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
+            entity_update();
+        }
         ar.grad_out = nullptr; ar.no_update = 0;
         ar.grad_direct = E.rel_gsum.p;
         { KernelTimer t(E, K_ADAM_REL); launch_adam_rows(ar, st); }
