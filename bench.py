@@ -507,7 +507,8 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--also", default=None,
                     help="comma-separated workloads measured after the headline one and reported under "
-                         "`workloads` (default with --workload c2: c3l2,c3,c5 - the 22.8M- and 91.2M-row tables; "
+                         "`workloads` (default with --workload c2: c3l2,c3,c5,c4 - the 22.8M- and 91.2M-row tables and the "
+                         "DistMult + feature configuration; "
                          "'none' to skip)")
     ap.add_argument("--cpu-steps", type=int, default=None,
                     help="steps the sequential CPU port times (default: sized for ~15 s)")
@@ -544,7 +545,7 @@ def main():
             sys.exit("--mode predict covers the TransE workloads without features")
         return predict_bench(args, w, kge, torch)
 
-    also = args.also if args.also is not None else ("c3l2,c3,c5" if args.workload == "c2" and not args.n_entity else "none")
+    also = args.also if args.also is not None else ("c3l2,c3,c5,c4" if args.workload == "c2" and not args.n_entity else "none")
     also = [x for x in also.split(",") if x and x != "none"]
     for x in also:
         if x not in WORKLOADS:

@@ -130,3 +130,31 @@ def test_predictions_topk():
     assert multi.shard_idx.shape == (2, 1, 3, 2) and multi.score.shape == (2, 1, 3)
     np.testing.assert_equal(multi.shard_idx[:, 0], post.shard_idx)
     np.testing.assert_equal(multi.score[:, 0], post.score)
+
+
+def test_bench_reads_traffic_of_the_most_launched_kernel_variant():
+    """bench.py takes `roofline.traffic` from the committed rocprofv3 summaries: every step kernel
+    of a profiled workload has a figure, and where two variants of a kernel ran (the sparse update
+    with and without hot rows inside) the one launched more often is taken."""
+    import re
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    sys.path.insert(0, str(root))
+    from bench import measured_traffic
+
+    for workload in ("c2", "c3l2", "c3", "c5"):
+        traffic, source = measured_traffic(workload)
+        assert source == f"profiles/{workload}_step_hbm_traffic.md"
+        for kernel in ("gather_operands", "score_fwd", "score_bwd", "adam_entity"):
+            assert traffic[kernel] > 1e6, (workload, kernel)
+    rows = {}
+    for line in (root / "profiles" / "c2_step_hbm_traffic.md").read_text().splitlines():
+        m = re.match(r"\| `(kge::k_adam_rows[^`]*)` \|[^|]*\|[^|]*\| ([0-9.]+) \| ([0-9.]+) \| (\d+) \|", line)
+        if m:
+            rows[m.group(1)] = ((float(m.group(2)) + float(m.group(3))) * 1e6, int(m.group(4)))
+    assert len(rows) == 2
+    most = max(rows.values(), key=lambda r: r[1])
+    assert measured_traffic("c2")[0]["adam_entity"] == pytest.approx(most[0])
+    assert measured_traffic("no_such_workload") == (None, None)
