@@ -164,6 +164,9 @@ struct BwdParams {
     int a_c0, b_c0;
     int use_mfma;
     const uint32_t* nearflag;  // from the forward pass (L2 on the matrix cores), or null
+    // merged tails (ScoreShape::tcount, tpad), or null: a block's b-operand rows end at tail_limit
+    const uint32_t* tcount = nullptr;
+    int tpad = 64;
     // optional rows added to the output (the feature projection's `embedding + ...`):
     // output row i gets row add_index[i] of add_base, row 0 for i >= *add_count
     const char* add_base;

@@ -263,6 +263,12 @@ struct kge_engine {
     DevBuf<uint32_t> r_uniq, r_seg, r_coff, r_cpos, r_clen, r_counts, r_real;
     DevBuf<uint32_t> e_hot, e_hot_count, r_hot, r_hot_count;  // the rows with chunks, per step
     DevBuf<uint32_t> nearflag;
+    // additive setting execution.merge_tails (default true): a block scores one column per distinct
+    // tail row, weighted by how many of its tail positions hold that row
+    bool merge_tails = true;
+    int tpad = 64;  // live tail columns come in whole groups of this many (the scoring kernels' tile)
+    DevBuf<uint32_t> tkey, tcol, tcount;
+    DevBuf<float> tmult;
     int e_ustride, e_cstride, r_ustride, r_cstride, n_rel_items;
     uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
     // step
@@ -529,6 +535,11 @@ void parse_settings(kge_engine& E, const Items& s) {
     E.T = E.S * E.A;
     E.NR = E.B + E.T;
     E.R = E.S * E.NR;
+    // additive: merged tails.  Not with TransH (its L1 part has kernels of its own), the norm
+    // regularisers (they count a row's members that carry no gradient as its gathered slots) or
+    // bfloat16 scoring, and for tail lists that fit one workgroup's sort.
+    E.merge_tails = s.find("execution.merge_tails") ? s.boolean("execution.merge_tails") : true;
+    if (E.score_fn == SCORE_TRANSH || E.reg_on || E.score_bf16 || E.T > kMergeMaxT) E.merge_tails = false;
     E.Dp = round_up(E.D, (emb_et == ET_F32 && mom_et == ET_F32) ? 4 : 8);
     E.Fp = E.F ? round_up(E.F, feat_et == ET_F32 ? 4 : 8) : 0;
     RowLayout& L = E.L;
@@ -539,6 +550,8 @@ void parse_settings(kge_engine& E, const Items& s) {
     L.off_f = L.off_s + (int64_t)E.Dp * elem_size(mom_et);
     L.pitch = L.off_f + (int64_t)E.Fp * elem_size(feat_et);
     E.n_rows = E.shared_table ? (int64_t)E.n_entity : (int64_t)E.S * E.n_entity;
+    if (E.n_rows >= ((int64_t)1 << (32 - kKeyFlagBits)))
+        throw std::invalid_argument("the entity table must have fewer than 2^31 rows (32-bit sort keys: row number and one flag bit)");
     if (E.n_rows >= (int64_t)1 << 32) throw std::invalid_argument("more than 2^32 table rows");
     if ((int64_t)2 * E.R >= (int64_t)1 << 31) throw std::invalid_argument("batch too large");
 
@@ -599,10 +612,16 @@ void allocate(kge_engine& E) {
     E.n_rel_items = (int)((SB + E.n_rel) * E.rel_copies);
     for (DevBuf<uint32_t>* b : {&E.rk_a, &E.rv_a, &E.rk_b, &E.rv_b}) b->alloc(ns * E.n_rel_items);
     {   // the two sorts of a call run in shared launches: a histogram region each, both at the wider key's digit width
-        const int bits = std::max(std::max(1, bit_length((uint64_t)E.n_rows - 1)), std::max(1, bit_length((uint64_t)E.n_rel_rows - 1)));
+        const int bits = kKeyFlagBits + std::max(std::max(1, bit_length((uint64_t)E.n_rows - 1)), std::max(1, bit_length((uint64_t)E.n_rel_rows - 1)));
         E.hist.alloc(radix_sort_hist_words((int)(2 * R), (int)ns, bits) + radix_sort_hist_words(E.n_rel_items, (int)ns, bits));
     }
     E.seg_scratch.alloc(find_segments_scratch_words((int)(2 * R), E.n_rel_items, (int)ns));
+    if (E.merge_tails) {
+        E.tkey.alloc(ns * S * E.T);
+        E.tcol.alloc(ns * S * E.T);
+        E.tmult.alloc(ns * S * E.T);
+        E.tcount.alloc(ns * S);
+    }
     {   // pinned host staging: plan counts [4][2 ns], step sizes [ns 9 S], loss [S]
         const size_t words = 8 * ns + ns * 9 * S + S;  // counts [2][ns][4]
         HIP_CHECK(hipHostMalloc(&E.h_pin, words * 4, hipHostMallocDefault));
@@ -658,6 +677,13 @@ void allocate(kge_engine& E) {
     }
     E.grad.alloc(R * E.Dp);
     E.opnd.alloc(R * E.Dp);
+    if (E.merge_tails) {
+        // columns past a block's distinct tails are never written; the kernels that read whole
+        // tiles of them (and drop the results) must find finite values there
+        E.opnd.zero(st);
+        E.coef.zero(st);
+        if (E.score_bf16) { E.opnd16.zero(st); E.coef16.zero(st); }
+    }
     E.partial.alloc((size_t)E.e_cstride * E.Dp);
     E.rel_partial.alloc((size_t)E.r_cstride * E.Dp);
     if (contributions_read_tables(E)) E.rel_gsum.alloc((size_t)E.n_rel * E.Dp);
@@ -931,12 +957,15 @@ void run_plan(kge_engine& E, int s0, int sn) {
     ps.n_entity = E.n_entity; ps.shared_table = E.shared_table; ps.n_relation = E.n_rel;
     ps.rel_copies = E.rel_copies;
     ps.step0 = s0; ps.step_count = sn;
-    const int ebits = std::max(1, bit_length((uint64_t)E.n_rows - 1));
-    const int rbits = std::max(1, bit_length((uint64_t)E.n_rel_rows - 1));
+    ps.merge_tails = E.merge_tails ? 1 : 0;
+    const int ebits = std::max(1, bit_length((uint64_t)E.n_rows - 1)) + kKeyFlagBits;
+    const int rbits = std::max(1, bit_length((uint64_t)E.n_rel_rows - 1)) + kKeyFlagBits;
     // both sorts in shared launches, the first pass's histograms from the item kernel
     uint32_t* const e_hist = E.hist.p;
     uint32_t* const r_hist = E.hist.p + radix_sort_hist_words((int)N, E.n_step, std::max(ebits, rbits));
-    launch_build_items(ps, E.d_remote.p, E.d_a2a.p, E.d_head.p, E.d_relation.p, E.d_tail.p, E.ckey.p,
+    if (E.merge_tails)
+        launch_merge_tails(ps, E.d_remote.p, E.d_a2a.p, E.tkey.p, E.tmult.p, E.tcol.p, E.tcount.p, st);
+    launch_build_items(ps, E.d_remote.p, E.d_a2a.p, E.d_head.p, E.d_relation.p, E.d_tail.p, E.tkey.p, E.tcol.p, E.ckey.p,
                        E.crel.p, E.clabel.p, E.ek_a.p, E.ev_a.p, E.rk_a.p, E.rv_a.p,
                        sort_passes(std::max(ebits, rbits)).bits[0], e_hist, r_hist, st);
     SortBuffers es = {}, rs = {};
@@ -1007,6 +1036,9 @@ void run_step(kge_engine& E, int i) {
     sh.negative_adversarial_scale = E.neg_adv;
     sh.use_mfma = E.use_mfma;
     sh.operands_dense = 0;
+    sh.tcount = E.merge_tails ? E.tcount.p + (size_t)i * E.S : nullptr;
+    sh.tmult = E.merge_tails ? E.tmult.p + (size_t)i * E.S * E.T : nullptr;
+    sh.tpad = E.tpad;
     const bool fused = E.loss_fn == LOSS_LOGSIGMOID && E.neg_adv <= 0.f && !E.score_bf16;
 
     const uint32_t* ckey = E.ckey.p + i * R;
@@ -1079,8 +1111,9 @@ void run_step(kge_engine& E, int i) {
 
     // dense operands: every contribution's row, float32, relation applied to the heads
     { KernelTimer t(E, K_GATHER);
+      TailCols tc = {sh.tcount, E.T, E.tpad};
       launch_gather_operands(ent, E.rel.p, crel, rel_mode_of(E), E.D / 2, (int)SB, (int)R, E.Dp,
-                             E.opnd.p, E.score_bf16 ? E.opnd16.p : nullptr, st); }
+                             E.opnd.p, E.score_bf16 ? E.opnd16.p : nullptr, st, &tc); }
     RowSource dense;
     dense.base = (const char*)E.opnd.p; dense.pitch = (int64_t)E.Dp * 4; dense.etype = ET_F32;
     dense.index = nullptr; dense.count = E.Dp; dense.vec = 1;
@@ -1517,7 +1550,11 @@ void run_timing(kge_engine& E, const Items& in) {
 //   sorted_items u32[2 R]        item numbers in (row, item) order: item < R is contribution
 //                                `item`, item >= R is slot `item - R` of `remote`
 //   counts u32[2]                {distinct rows, chunks}
-// and the same for the relation plan under relation_* (N = S B + n_relation items per copy).
+// and the same for the relation plan under relation_* (N = S B + n_relation items per copy);
+//   label_column u32[S B]        the score column that holds every positive's label
+//   tail_count u32[S], tail_column u32[S T], tail_multiplicity f32[S T]
+//                                (merged tails) distinct tail rows per block, the column of every
+//                                tail position, the positions every column stands for
 void run_plan_dump(kge_engine& E, const Items& in) {
     const size_t i = in.uint("step");
     if (i >= (size_t)E.n_step || !E.e_sorted_vals) throw std::invalid_argument("'plan_dump' needs a planned step of the last train_step_loop");
@@ -1539,6 +1576,19 @@ void run_plan_dump(kge_engine& E, const Items& in) {
     out("relation_segment_contributions", E.r_real.p + i * RU, RU);
     out("relation_sorted_items", E.r_sorted_vals + i * NRI, NRI);
     out("relation_counts", E.r_counts.p + 2 * i, 2);
+    out("label_column", E.clabel.p + i * (size_t)E.S * E.B, (size_t)E.S * E.B);
+    // merged tails: distinct rows per block, the column of every tail position, and how many
+    // positions every column stands for (float32, as the kernels read it)
+    const size_t ST = (size_t)E.S * E.T;
+    if (in.find("tail_count") || in.find("tail_column") || in.find("tail_multiplicity")) {
+        if (!E.merge_tails) throw std::invalid_argument("'plan_dump': the tail lists were not merged (execution.merge_tails)");
+        out("tail_count", E.tcount.p + i * E.S, E.S);
+        out("tail_column", E.tcol.p + i * ST, ST);
+        if (in.find("tail_multiplicity")) {
+            float* host = (float*)in.array("tail_multiplicity", KGE_F32, {ST});
+            HIP_CHECK(hipMemcpy(host, E.tmult.p + i * ST, ST * 4, hipMemcpyDeviceToHost));
+        }
+    }
 }
 
 // "predict" (Model::predict, src/poplar_kge.cpp:811-855): for every (head row,
@@ -1972,7 +2022,7 @@ ScatterLayout scatter_layout(int64_t n, int64_t rows, int64_t cols) {
     auto take = [&](size_t words) { size_t at = o; o += (words * 4 + 15) / 16 * 16; return at; };
     L.off_keys_a = take(L.N); L.off_vals_a = take(L.N);
     L.off_keys_b = take(L.N); L.off_vals_b = take(L.N);
-    L.off_hist = take(radix_sort_hist_words((int)L.N, 1, std::max(1, bit_length((uint64_t)rows - 1))));
+    L.off_hist = take(radix_sort_hist_words((int)L.N, 1, std::max(1, bit_length((uint64_t)rows - 1)) + kKeyFlagBits));
     L.off_uniq = take(rows); L.off_seg = take(rows + 1); L.off_coff = take(rows + 1);
     L.off_cpos = take(L.cmax); L.off_clen = take(L.cmax); L.off_counts = take(2);
     L.off_real = take(rows); L.off_scratch = take(find_segments_scratch_words((int)L.N, 0, 1));
@@ -1996,7 +2046,7 @@ int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* i
     char* w = (char*)workspace;
     auto u32 = [&](size_t off) { return (uint32_t*)(w + off); };
     launch_iota_keys(idx, u32(L.off_keys_a), u32(L.off_vals_a), n, rows, st);
-    const int bits = std::max(1, bit_length((uint64_t)rows - 1));
+    const int bits = std::max(1, bit_length((uint64_t)rows - 1)) + kKeyFlagBits;
     const int which = launch_radix_sort(u32(L.off_keys_a), u32(L.off_vals_a), u32(L.off_keys_b),
                                         u32(L.off_vals_b), u32(L.off_hist), (int)L.N, 1, bits, st);
     const uint32_t* sv = which ? u32(L.off_vals_b) : u32(L.off_vals_a);

@@ -44,7 +44,28 @@ struct PlanShape {
     int rel_copies;           // 1; 2 for TransH, whose relation table holds a second row (the
                               // hyperplane normal, row n_relation + r) per relation
     int step0, step_count;    // the steps of the resident batch to plan
+    int merge_tails;          // the blocks' tail lists have been merged (launch_merge_tails)
 };
+
+// Sort keys carry one flag bit under the row number: key = row << 1 | (0: the item is a
+// gradient contribution, 1: a zero-gradient member of the update set).  Within a row the
+// contributions therefore sort in front, whatever their item numbers.
+constexpr int kKeyFlagBits = 1;
+
+// A block's T shared tails repeat rows under power-law sampling (a third of them on the
+// benchmark workloads), and equal rows give equal score columns.  One workgroup per (step,
+// block) sorts the block's tail rows and keeps one column per distinct row:
+//   tkey   [n_step, S*T]  sort key of tail column j of block d (row << 1; columns from the
+//                         block's distinct count on repeat column 0's row with the flag bit set:
+//                         they are scored in whole tiles but carry no gradient)
+//   tmult  [n_step, S*T]  how many of the block's tail positions hold column j's row (0 from the
+//                         distinct count on)
+//   tcol   [n_step, S*T]  the column of every original tail position (labels are positions)
+//   tcount [n_step, S]    distinct rows per block
+// T <= kMergeMaxT.  Integer work: exact, independent of scheduling.
+constexpr int kMergeMaxT = 4096;
+void launch_merge_tails(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a, uint32_t* tkey,
+                        float* tmult, uint32_t* tcol, uint32_t* tcount, hipStream_t stream);
 
 // Compact per-step arrays + the items to sort for the entity plan and the
 // relation plan.  Item layout, entity plan (2R items, R = S*NR):
@@ -56,8 +77,10 @@ struct PlanShape {
 // normal row's contribution of positive c).
 // `digit_bits`: the width of the first radix pass (sort_passes of the wider of the two key
 // widths); ent_hist / rel_hist receive every tile's digit histogram for that pass.
+// With ps.merge_tails the tail items take their keys from `tkey` and the labels go through `tcol`.
 void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
                         const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
+                        const uint32_t* tkey, const uint32_t* tcol,
                         uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
                         uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals, int digit_bits,
                         uint32_t* ent_hist, uint32_t* rel_hist, hipStream_t stream);
@@ -133,16 +156,42 @@ struct ScoreShape {
     float negative_adversarial_scale;
     int use_mfma;                  // L2 / dot scoring on the matrix cores (else the VALU kernels)
     int operands_dense;            // a-operand rows already hold the predicted tails (launch_gather_operands)
+    // merged tails (launch_merge_tails), or null: block d scores its first tcount[d] tail columns
+    // only (in whole groups of `tpad` columns, never more than T), column j standing for
+    // tmult[d * T + j] tail positions: one of them the label's if the positive's label names the
+    // column, the others negatives
+    // (default member initialisers: a shape built field by field scores every column)
+    const uint32_t* tcount = nullptr;
+    const float* tmult = nullptr;
+    int tpad = 64;
 };
+// the tail columns block d scores and differentiates
+__host__ __device__ inline int tail_limit(const uint32_t* tcount, int d, int T, int tpad) {
+    if (!tcount) return T;
+    const int t = ((int)tcount[d] + tpad - 1) / tpad * tpad;
+    return t < T ? t : T;
+}
 
 // Dense float32 operand matrix [n_rows, Dp] from indexed rows: rows [0, n_head)
 // combined with their relation row (rel_mode 1 add, 2 multiply, 3 complex product on the
 // halves [0, half) | [half, 2 half) of the row, 4 rotation by the row's `half` phases).
 // With `out16` the values are rounded to bfloat16, stored there, and the float32
 // copy holds the same rounded values.
+// `tail_cols` (or null): rows from n_head on are the blocks' tail columns [S, T]; the columns past a
+// block's limit (tail_limit) are left alone.
+struct TailCols {
+    const uint32_t* tcount = nullptr;
+    int T = 1, tpad = 1;
+    // whether the row `t` places behind the heads is to be gathered
+    __device__ bool live(int t) const {
+        if (!tcount || t < 0) return true;
+        const int d = t / T;
+        return t - d * T < tail_limit(tcount, d, T, tpad);
+    }
+};
 void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
                             int half, int n_head, int n_rows, int Dp, float* out, uint16_t* out16,
-                            hipStream_t stream);
+                            hipStream_t stream, const TailCols* tail_cols = nullptr);
 
 // Batched bfloat16 product on the matrix cores: C[z] = A[z] . Bt[z]^T, float32 out.
 // Strides in elements.  Optional rows added to the output: output row m gets row

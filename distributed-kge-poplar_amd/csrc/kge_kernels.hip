@@ -30,10 +30,10 @@ __global__ __launch_bounds__(256) void k_gather_operands(RowSource ent, const fl
                                                          const uint32_t* __restrict__ crel,
                                                          int rel_mode, int half, int n_head, int n_rows,
                                                          int Dp, float* __restrict__ out,
-                                                         uint16_t* __restrict__ out16) {
+                                                         uint16_t* __restrict__ out16, TailCols tc) {
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (c >= n_rows) return;
+    if (c >= n_rows || !tc.live(c - n_head)) return;
     const char* row = row_ptr(ent, c);
     const float* rrow = (c < n_head && rel_mode) ? rel + (size_t)crel[c] * Dp : nullptr;
     for (int k = lane * 4; k < Dp; k += 256) {
@@ -90,10 +90,11 @@ template <int RPW>
 __global__ __launch_bounds__(256) void k_gather_operands_multi(RowSource ent, const float* __restrict__ rel,
                                                                const uint32_t* __restrict__ crel, int rel_mode,
                                                                int n_head, int n_rows, int Dp,
-                                                               float* __restrict__ out) {
+                                                               float* __restrict__ out, TailCols tc) {
     const int lane = threadIdx.x & 63;
     const int c0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW;
-    if (c0 >= n_rows) return;
+    // (limits are multiples of RPW: the rows of a wave are live or not together)
+    if (c0 >= n_rows || !tc.live(c0 - n_head)) return;
     const char* row[RPW];
     const float* rrow[RPW];
 #pragma unroll
@@ -125,17 +126,21 @@ __global__ __launch_bounds__(256) void k_gather_operands_multi(RowSource ent, co
 constexpr int kGatherRowsPerWave = 2;
 void launch_gather_operands(const RowSource& ent, const float* rel, const uint32_t* crel, int rel_mode,
                             int half, int n_head, int n_rows, int Dp, float* out, uint16_t* out16,
-                            hipStream_t stream) {
+                            hipStream_t stream, const TailCols* tail_cols) {
+    TailCols tc = {};
+    if (tail_cols) tc = *tail_cols;
+    const bool pairs_ok = !tc.tcount || (n_head % kGatherRowsPerWave == 0 && tc.T % kGatherRowsPerWave == 0 &&
+                                         tc.tpad % kGatherRowsPerWave == 0);
     if (rel_mode >= 3)
         hipLaunchKernelGGL(k_gather_operands<true>, dim3((n_rows + 3) / 4), dim3(256), 0, stream, ent, rel, crel,
-                           rel_mode, half, n_head, n_rows, Dp, out, out16);
-    else if (!out16 && n_rows >= 8192)
+                           rel_mode, half, n_head, n_rows, Dp, out, out16, tc);
+    else if (!out16 && n_rows >= 8192 && pairs_ok)
         hipLaunchKernelGGL(k_gather_operands_multi<kGatherRowsPerWave>,
                            dim3((n_rows + 4 * kGatherRowsPerWave - 1) / (4 * kGatherRowsPerWave)),
-                           dim3(256), 0, stream, ent, rel, crel, rel_mode, n_head, n_rows, Dp, out);
+                           dim3(256), 0, stream, ent, rel, crel, rel_mode, n_head, n_rows, Dp, out, tc);
     else
         hipLaunchKernelGGL(k_gather_operands<false>, dim3((n_rows + 3) / 4), dim3(256), 0, stream, ent, rel, crel,
-                           rel_mode, half, n_head, n_rows, Dp, out, out16);
+                           rel_mode, half, n_head, n_rows, Dp, out, out16, tc);
 }
 
 // --------------------------------------------------------------------------
@@ -167,6 +172,31 @@ DEVINL void log_sigmoid_both(float z, float& value, float& grad) {
     grad = z >= 0.f ? g_pos : rw;
 }
 
+// The same for both signs of one score: exp(-|z|) serves z = s and z = -s alike.
+DEVINL void log_sigmoid_pair(float s, float& v_pos, float& g_pos, float& v_neg, float& g_neg) {
+    const float u = __builtin_amdgcn_exp2f(-1.44269504089f * fabsf(s));
+    const float w = 1.f + u;
+    const float rw = __builtin_amdgcn_rcpf(w);
+    const float l1p = 0.69314718056f * __builtin_amdgcn_logf(w) - ((w - 1.f) - u) * rw;
+    const float g_big = fmaxf(u * rw, 1.670142184e-5f);  // e^-11 / (1 + e^-11)
+    v_pos = fminf(s, 0.f) - (s > -11.f ? l1p : 0.f);
+    v_neg = fminf(-s, 0.f) - (s < 11.f ? l1p : 0.f);
+    g_pos = s >= 0.f ? g_big : rw;
+    g_neg = s <= 0.f ? g_big : rw;
+}
+
+// The logsigmoid loss of one score column that stands for `mult` tail positions, one of them the
+// positive's label if `pos` (src/poplar_kge.cpp:615-636 summed over the positions that share the
+// row): returns the loss term (before the normalisation) and sets d loss / d score (times grad_scale).
+DEVINL float logsigmoid_column(float score, bool pos, float mult, float w_pos, float w_neg, float grad_scale,
+                               float& dscore) {
+    float v_pos, g_pos, v_neg, g_neg;
+    log_sigmoid_pair(score, v_pos, g_pos, v_neg, g_neg);
+    const float wp = pos ? w_pos : 0.f, wn = (mult - (pos ? 1.f : 0.f)) * w_neg;
+    dscore = (wn * g_neg - wp * g_pos) * grad_scale;
+    return -(wp * v_pos + wn * v_neg);
+}
+
 struct FwdParams {
     ScoreShape sh;
     RowSource ent_a, ent_b;
@@ -195,7 +225,17 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
     const int d = tile.z, m0 = tile.y * kScoreTile, n0 = tile.x * kScoreTile;
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int B = sh.B, T = sh.T, Dp = sh.Dp;
+    if (n0 >= tail_limit(sh.tcount, d, T, sh.tpad)) {  // merged tails: the block has no such column
+        if (OM == 0 && tid == 0) p.loss_part[(size_t)d * (tile.gx * tile.gy) + tile.y * tile.gx + tile.x] = 0.f;
+        return;
+    }
     if (OM == 0 && tid < kScoreTile) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
+    float mult[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = n0 + tx * 4 + j;
+        mult[j] = (OM == 0 && sh.tmult && n < T) ? sh.tmult[(size_t)d * T + n] : 1.f;
+    }
 
     // staging assignment: row lr of each operand, float4 columns k4 and k4 + 16.  Sixteen
     // consecutive rows per wave and four column groups: a store instruction's 64 lanes fall on
@@ -270,14 +310,9 @@ __global__ __launch_bounds__(256) void k_score_fwd(FwdParams p) {
             if (OM == 2) { outv[j] = dist; continue; }
             const float score = score_is_distance_value(sh.score_fn) ? dist : sh.gamma - dist;
             if (OM == 1) { outv[j] = score; continue; }
-            const bool pos = (uint32_t)n == label;
-            const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
-            const float z = sign * score;
-            float lsig, dlsig;
-            log_sigmoid_both(z, lsig, dlsig);
-            if (n < T) loss_acc -= w * lsig;
-            // d loss / d score, times the loss scale
-            const float ds = -w * sign * dlsig * grad_scale;
+            float ds;  // d loss / d score, times the loss scale
+            const float term = logsigmoid_column(score, (uint32_t)n == label, mult[j], w_pos, w_neg, grad_scale, ds);
+            if (n < T) loss_acc += term;
             float c = score_is_distance_value(sh.score_fn) ? ds : -ds;  // score = gamma - dist
             if (DIST == DIST_L2) c = dist != 0.f ? c * __builtin_amdgcn_rcpf(dist) : 0.f;
             outv[j] = c;
@@ -407,6 +442,10 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * (32 * AT), wn = (wave & 1) * 32;
     const int B = sh.B, T = sh.T, Dp = sh.Dp;
+    if (n0 >= tail_limit(sh.tcount, d, T, sh.tpad)) {  // merged tails: the block has no such column
+        if (OM == 0 && tid == 0) p.loss_part[(size_t)d * (tile.gx * tile.gy) + tile.y * tile.gx + tile.x] = 0.f;
+        return;
+    }
     if (OM == 0 && tid < FM_TM) label_s[tid] = m0 + tid < B ? p.clabel[d * B + m0 + tid] : 0u;
 
     const int srow = tid >> 3, k4 = (tid & 7) * 4;
@@ -639,6 +678,7 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
     float* const coef_blk = p.coef + (size_t)d * B * T;
     float* const dist_blk = p.dist ? p.dist + (size_t)d * B * T : nullptr;
     const float nb = DIST == DIST_L2 ? nb_s[n_loc] : 0.f;
+    const float mult = (OM == 0 && sh.tmult && n < T) ? sh.tmult[(size_t)d * T + n] : 1.f;
 #pragma unroll
     for (int t = 0; t < AT; ++t) {
         // phase 1 (straight-line): squared distances and which of them cancelled
@@ -705,13 +745,9 @@ __global__ __launch_bounds__(NW * 64) void k_score_fwd_mfma(FwdParams p) {
                     outv = score;
                     if (live && DIST == DIST_L2 && dist_blk) dist_blk[m * T + n] = dist;
                 } else {
-                    const bool pos = (uint32_t)n == label_r[r];
-                    const float sign = pos ? 1.f : -1.f, w = pos ? w_pos : w_neg;
-                    const float z = sign * score;
-                    float lsig, dlsig;
-                    log_sigmoid_both(z, lsig, dlsig);
-                    if (live) loss_acc -= w * lsig;
-                    const float ds = -w * sign * dlsig * grad_scale;
+                    float ds;
+                    const float term = logsigmoid_column(score, (uint32_t)n == label_r[r], mult, w_pos, w_neg, grad_scale, ds);
+                    if (live) loss_acc += term;
                     outv = score_is_distance_value(sh.score_fn) ? ds : -ds;
                     if (DIST == DIST_L2) outv = dist != 0.f ? outv * __builtin_amdgcn_rcpf(dist) : 0.f;
                 }
@@ -1050,22 +1086,31 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
     uint16_t* s16 = coef16 ? coef16 + (size_t)row * T : nullptr;  // bfloat16 copy for the matrix cores
     const float* dr = dist ? dist + (size_t)row * T : nullptr;
     const uint32_t label = clabel[row];
+    // merged tails: the block's live columns and how many tail positions each stands for.  Column j
+    // of multiplicity m holds m negatives, or the label's position and m - 1 negatives; the sums
+    // below run over positions, so a column enters them m times (src/poplar_kge.cpp:615-652).
+    const int blk = row / sh.B;
+    const int TL = tail_limit(sh.tcount, blk, T, sh.tpad);
+    const float* mu = sh.tmult ? sh.tmult + (size_t)blk * T : nullptr;
     float loss = 0.f;
     if (sh.loss_fn == LOSS_SOFTMAX && (T & 3) == 0 && T <= 2048) {
         // the row stays in registers (up to eight float4 per lane): one read, one write
         const float corr = sh.softmax_correction;
         constexpr int NV = 8;
-        floatx4 z[NV];
+        floatx4 z[NV], m[NV];
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int t = 4 * lane + 256 * i;
-            if (t < T) {
+            if (t < TL) {
                 z[i] = *reinterpret_cast<const floatx4*>(s + t);
+                m[i] = mu ? *reinterpret_cast<const floatx4*>(mu + t) : floatx4{1.f, 1.f, 1.f, 1.f};
 #pragma unroll
                 for (int x = 0; x < 4; ++x) {
-                    z[i][x] += (uint32_t)(t + x) == label ? 0.f : corr;
-                    mx = fmaxf(mx, z[i][x]);
+                    const bool pos = (uint32_t)(t + x) == label;
+                    if (m[i][x] == 0.f) z[i][x] = -INFINITY;  // no position holds this column
+                    if (!pos || m[i][x] > 1.f) mx = fmaxf(mx, z[i][x] + corr);
+                    if (pos) mx = fmaxf(mx, z[i][x]);
                 }
             }
         }
@@ -1073,9 +1118,14 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
         float sum = 0.f;
 #pragma unroll
         for (int i = 0; i < NV; ++i)
-            if (4 * lane + 256 * i < T)
+            if (4 * lane + 256 * i < TL)
 #pragma unroll
-                for (int x = 0; x < 4; ++x) sum += __expf(z[i][x] - mx);
+                for (int x = 0; x < 4; ++x) {
+                    const bool pos = (uint32_t)(4 * lane + 256 * i + x) == label;
+                    const float neg = m[i][x] - (pos ? 1.f : 0.f);
+                    if (neg > 0.f) sum += neg * __expf(z[i][x] + corr - mx);
+                    if (pos) sum += __expf(z[i][x] - mx);
+                }
         sum = wave_sum(sum);
         const float lse = mx + logf(sum);
         const float inv_norm = 1.f / ((float)sh.S * (float)sh.B);
@@ -1084,13 +1134,18 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int t = 4 * lane + 256 * i;
-            if (t < T) {
+            if (t < TL) {
                 floatx4 c;
 #pragma unroll
                 for (int x = 0; x < 4; ++x) {
                     const bool pos = (uint32_t)(t + x) == label;
-                    if (pos) loss = -(z[i][x] - lse) * inv_norm;
-                    c[x] = sgn * (__expf(z[i][x] - lse) - (pos ? 1.f : 0.f)) * gs;
+                    const float neg = m[i][x] - (pos ? 1.f : 0.f);
+                    float g = neg > 0.f ? neg * __expf(z[i][x] + corr - lse) : 0.f;
+                    if (pos) {
+                        loss = -(z[i][x] - lse) * inv_norm;
+                        g += __expf(z[i][x] - lse) - 1.f;
+                    }
+                    c[x] = sgn * g * gs;
                 }
                 if (dr) {
                     const floatx4 dv = *reinterpret_cast<const floatx4*>(dr + t);
@@ -1109,18 +1164,32 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
     } else if (sh.loss_fn == LOSS_SOFTMAX) {
         const float corr = sh.softmax_correction;
         float mx = -INFINITY;
-        for (int t = lane; t < T; t += 64) mx = fmaxf(mx, s[t] + ((uint32_t)t == label ? 0.f : corr));
+        for (int t = lane; t < TL; t += 64) {
+            const bool pos = (uint32_t)t == label;
+            const float m = mu ? mu[t] : 1.f;
+            if (m - (pos ? 1.f : 0.f) > 0.f) mx = fmaxf(mx, s[t] + corr);
+            if (pos) mx = fmaxf(mx, s[t]);
+        }
         mx = wave_max(mx);
         float sum = 0.f;
-        for (int t = lane; t < T; t += 64) sum += expf(s[t] + ((uint32_t)t == label ? 0.f : corr) - mx);
+        for (int t = lane; t < TL; t += 64) {
+            const bool pos = (uint32_t)t == label;
+            const float neg = (mu ? mu[t] : 1.f) - (pos ? 1.f : 0.f);
+            if (neg > 0.f) sum += neg * expf(s[t] + corr - mx);
+            if (pos) sum += expf(s[t] - mx);
+        }
         sum = wave_sum(sum);
         const float lse = mx + logf(sum);
         const float inv_norm = 1.f / ((float)sh.S * (float)sh.B);
-        for (int t = lane; t < T; t += 64) {
+        for (int t = lane; t < TL; t += 64) {
             const bool pos = (uint32_t)t == label;
-            const float z = s[t] + (pos ? 0.f : corr);
-            if (pos) loss = -(z - lse) * inv_norm;
-            const float ds = (expf(z - lse) - (pos ? 1.f : 0.f)) * inv_norm * sh.loss_scale;
+            const float neg = (mu ? mu[t] : 1.f) - (pos ? 1.f : 0.f);
+            float g = neg > 0.f ? neg * expf(s[t] + corr - lse) : 0.f;
+            if (pos) {
+                loss = -(s[t] - lse) * inv_norm;
+                g += expf(s[t] - lse) - 1.f;
+            }
+            const float ds = g * inv_norm * sh.loss_scale;
             float c = score_is_distance_value(sh.score_fn) ? ds : -ds;
             if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
             s[t] = c;
@@ -1133,25 +1202,42 @@ __global__ __launch_bounds__(256) void k_loss_rows(ScoreShape sh, const uint32_t
         const float inv_norm = 1.f / ((float)sh.S * (float)sh.B * Tn);
         float mx = -INFINITY, sum = 1.f;
         if (adv > 0.f) {
-            for (int t = lane; t < T; t += 64)
-                mx = fmaxf(mx, adv * s[t] + ((uint32_t)t == label ? -10000.f : 0.f));
+            // softmax over the positions of adv * score, the label's position pushed down by 10000
+            for (int t = lane; t < TL; t += 64) {
+                const bool pos = (uint32_t)t == label;
+                const float m = mu ? mu[t] : 1.f;
+                if (m - (pos ? 1.f : 0.f) > 0.f) mx = fmaxf(mx, adv * s[t]);
+                if (pos) mx = fmaxf(mx, adv * s[t] - 10000.f);
+            }
             mx = wave_max(mx);
             sum = 0.f;
-            for (int t = lane; t < T; t += 64)
-                sum += expf(adv * s[t] + ((uint32_t)t == label ? -10000.f : 0.f) - mx);
+            for (int t = lane; t < TL; t += 64) {
+                const bool pos = (uint32_t)t == label;
+                const float neg = (mu ? mu[t] : 1.f) - (pos ? 1.f : 0.f);
+                if (neg > 0.f) sum += neg * expf(adv * s[t] - mx);
+                if (pos) sum += expf(adv * s[t] - 10000.f - mx);
+            }
             sum = wave_sum(sum);
         }
-        for (int t = lane; t < T; t += 64) {
+        for (int t = lane; t < TL; t += 64) {
             const bool pos = (uint32_t)t == label;
+            const float neg = (mu ? mu[t] : 1.f) - (pos ? 1.f : 0.f);
             const float sc = s[t];
-            float w = pos ? w_pos : w_neg;
+            float wl = w_pos, wn = w_neg;  // weight of the label's position, of one negative position
             if (adv > 0.f) {
-                const float sm = expf(adv * sc + (pos ? -10000.f : 0.f) - mx) / sum;
-                w *= (pos ? 1.f : 0.f) + (Tn - 1.f) * sm;
+                wl *= 1.f + (Tn - 1.f) * (expf(adv * sc - 10000.f - mx) / sum);
+                wn *= (Tn - 1.f) * (expf(adv * sc - mx) / sum);
             }
-            const float sign = pos ? 1.f : -1.f, z = sign * sc;
-            loss -= w * log_sigmoid(z) * inv_norm;
-            const float ds = -w * sign * log_sigmoid_grad(z) * inv_norm * sh.loss_scale;
+            float ds = 0.f;
+            if (pos) {
+                loss -= wl * log_sigmoid(sc) * inv_norm;
+                ds -= wl * log_sigmoid_grad(sc);
+            }
+            if (neg > 0.f) {
+                loss -= neg * wn * log_sigmoid(-sc) * inv_norm;
+                ds += neg * wn * log_sigmoid_grad(-sc);
+            }
+            ds *= inv_norm * sh.loss_scale;
             float c = score_is_distance_value(sh.score_fn) ? ds : -ds;
             if (dr) c = dr[t] != 0.f ? c / dr[t] : 0.f;
             s[t] = c;

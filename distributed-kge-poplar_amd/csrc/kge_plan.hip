@@ -1,10 +1,12 @@
 // gfx950 kernels of the plan phase: the index-only work of a training step, batched over the
 // steps of one call.
 //
+//   merge_tails     a block's tail list reduced to its distinct rows, with multiplicities
 //   build_items     every head / tail contribution resolved to its table row
 //                   (remote[src][slot], the all-to-all folded into the index arithmetic,
 //                   tests/python/reference_model.py:132-138)
-//   radix sort      (row, item) order: equal rows adjacent, ordered by item number
+//   radix sort      (row, contribution or not, item) order: equal rows adjacent, a row's gradient
+//                   contributions in front of its other members, each group ordered by item number
 //   find_segments   distinct rows, their members, the chunks of rows with many contributions
 //
 // Together the device-side counterpart of the host's np.unique (unique_pad,
@@ -29,6 +31,8 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
                                                      const uint32_t* __restrict__ head,
                                                      const uint32_t* __restrict__ relation,
                                                      const uint32_t* __restrict__ tail,
+                                                     const uint32_t* __restrict__ tkey,
+                                                     const uint32_t* __restrict__ tcol,
                                                      uint32_t* __restrict__ ckey,
                                                      uint32_t* __restrict__ crel,
                                                      uint32_t* __restrict__ clabel,
@@ -54,6 +58,7 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
     if (entity) {
         int item[PER], src[PER];
         uint32_t slot[PER], key[PER];
+        const bool merged = ps.merge_tails != 0;
 #pragma unroll
         for (int r = 0; r < PER; ++r) {
             item[r] = tile * kSortTile + r * kBuildThreads + tid;
@@ -65,10 +70,14 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
                 slot[r] = head[((size_t)d * nst + step) * B + b];
             } else if (it < R) {
                 const int cc = it - SB;
-                const int d = cc / T, t = cc - d * T;
-                const int j = t / A, i = t - j * A;
-                src[r] = j;
-                slot[r] = a2a[(((size_t)j * nst + step) * S + d) * A + i];
+                if (merged) {
+                    slot[r] = tkey[(size_t)step * S * T + cc];  // the finished key of the block's column
+                } else {
+                    const int d = cc / T, t = cc - d * T;
+                    const int j = t / A, i = t - j * A;
+                    src[r] = j;
+                    slot[r] = a2a[(((size_t)j * nst + step) * S + d) * A + i];
+                }
             } else if (it < 2 * R) {
                 const int sl = it - R;
                 src[r] = sl / NR;
@@ -78,12 +87,16 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
 #pragma unroll
         for (int r = 0; r < PER; ++r) {
             const uint32_t base = ps.shared_table ? 0u : (uint32_t)src[r] * (uint32_t)ps.n_entity;
-            key[r] = item[r] < 2 * R ? base + remote[((size_t)src[r] * nst + step) * NR + slot[r]] : 0u;
+            const int it = item[r];
+            if (merged && it >= SB && it < R) key[r] = slot[r];
+            else if (it < 2 * R)
+                key[r] = ((base + remote[((size_t)src[r] * nst + step) * NR + slot[r]]) << kKeyFlagBits) | (it < R ? 0u : 1u);
+            else key[r] = 0u;
         }
 #pragma unroll
         for (int r = 0; r < PER; ++r) {
             if (item[r] >= 2 * R) continue;
-            if (item[r] < R) ckey[(size_t)step * R + item[r]] = key[r];
+            if (item[r] < R) ckey[(size_t)step * R + item[r]] = key[r] >> kKeyFlagBits;
             ent_keys[(size_t)step * 2 * R + item[r]] = key[r];
             ent_vals[(size_t)step * 2 * R + item[r]] = item[r];
             atomicAdd(&h[key[r] & (uint32_t)(DIG - 1)], 1u);
@@ -101,6 +114,7 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
                 const int d = c / B, b = c - d * B;
                 key[r] = relation[((size_t)d * nst + step) * B + b];
                 if (copy == 0) label[r] = tail[((size_t)d * nst + step) * B + b];
+                if (copy == 0 && ps.merge_tails) label[r] = tcol[((size_t)step * S + d) * T + label[r]];
             } else if (it < n_rel_items) {
                 key[r] = it - SBr;
             }
@@ -118,18 +132,20 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
                 }
                 k += (uint32_t)(copy * ps.n_relation);
             }
+            k = (k << kKeyFlagBits) | (it < SBr ? 0u : 1u);
             rel_keys[(size_t)step * n_rel_items + it] = k;
             rel_vals[(size_t)step * n_rel_items + it] = it;
             atomicAdd(&h[k & (uint32_t)(DIG - 1)], 1u);
         }
     }
     __syncthreads();
-    uint32_t* hrow = (entity ? ent_hist : rel_hist) + ((size_t)seg * (entity ? e_tiles : r_tiles) + tile) * DIG;
+    uint32_t* hrow = (entity ? ent_hist : rel_hist) + ((size_t)seg * ((entity ? e_tiles : r_tiles) + 1) + tile) * DIG;
     for (int d = tid; d < DIG; d += kBuildThreads) hrow[d] = h[d];
 }
 
 void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a,
                         const uint32_t* head, const uint32_t* relation, const uint32_t* tail,
+                        const uint32_t* tkey, const uint32_t* tcol,
                         uint32_t* ckey, uint32_t* crel, uint32_t* clabel, uint32_t* ent_keys,
                         uint32_t* ent_vals, uint32_t* rel_keys, uint32_t* rel_vals, int digit_bits,
                         uint32_t* ent_hist, uint32_t* rel_hist, hipStream_t stream) {
@@ -137,7 +153,7 @@ void launch_build_items(const PlanShape& ps, const uint32_t* remote, const uint3
     const int e_tiles = (2 * R + kSortTile - 1) / kSortTile, r_tiles = (n_rel_items + kSortTile - 1) / kSortTile;
     dim3 grid(e_tiles + r_tiles, ps.step_count);
     hipLaunchKernelGGL(k_build_items, grid, dim3(kBuildThreads), 0, stream, ps, remote, a2a, head, relation,
-                       tail, ckey, crel, clabel, ent_keys, ent_vals, rel_keys, rel_vals, digit_bits, ent_hist,
+                       tail, tkey, tcol, ckey, crel, clabel, ent_keys, ent_vals, rel_keys, rel_vals, digit_bits, ent_hist,
                        rel_hist);
 }
 
@@ -149,7 +165,10 @@ __global__ __launch_bounds__(256) void k_iota_keys(const uint32_t* __restrict__ 
                                                    int64_t rows) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n + rows) return;
-    keys[i] = i < n ? idx[i] : (uint32_t)(i - n);
+    // an index outside the table carries no gradient anywhere: it joins row 0's other members
+    const uint32_t row = i < n ? idx[i] : (uint32_t)(i - n);
+    const bool real = i < n && (int64_t)row < rows;
+    keys[i] = ((real || i >= n ? row : 0u) << kKeyFlagBits) | (real ? 0u : 1u);
     vals[i] = (uint32_t)i;
 }
 void launch_iota_keys(const uint32_t* idx, uint32_t* keys, uint32_t* vals, int64_t n, int64_t rows,
@@ -165,7 +184,11 @@ void launch_iota_keys(const uint32_t* idx, uint32_t* keys, uint32_t* vals, int64
 // of a training call share their launches): tile histograms, then the stable scatter, whose workgroups each derive their output
 // positions from the histograms of all tiles (one round of loads; a separate scan launch, or
 // workgroups that hand results to each other through fences, both cost more than the reads).
-// hist layout: [seg][tile][digit] (digits contiguous: every access below is coalesced).
+// hist layout: [seg][tile][digit] (digits contiguous: every access below is coalesced), n_tiles + 1
+// rows per segment.  Arrays of more than kSortFoldTiles tiles (the stand-alone scatter-add on
+// millions of items; a training call's arrays have a few dozen) get a scan launch between the two:
+// every tile's row then holds the counts of the tiles in front of it and row n_tiles the totals,
+// so that a scatter workgroup reads two rows instead of all of them.
 
 SortPasses sort_passes(int key_bits) {
     SortPasses p = {};
@@ -184,7 +207,8 @@ SortPasses sort_passes(int key_bits) {
 size_t radix_sort_hist_words(int N, int n_seg, int key_bits) {
     const SortPasses p = sort_passes(key_bits);
     const size_t n_tiles = ((size_t)N + kSortTile - 1) / kSortTile;
-    return (size_t)n_seg * ((size_t)1 << p.bits[0]) * n_tiles;  // the first pass has the widest digit
+    // the first pass has the widest digit; one more row per segment for the digit totals of a scanned histogram
+    return (size_t)n_seg * ((size_t)1 << p.bits[0]) * (n_tiles + 1);
 }
 
 // Which of a launch's two jobs a workgroup serves: blockIdx.x counts job 0's tiles, then job 1's.
@@ -216,8 +240,30 @@ __global__ __launch_bounds__(256) void k_sort_hist(SortJob j0, SortJob j1, int s
     for (int r = 0; r < kSortTile / 256; ++r)
         if (base + r * 256 + tid < N) atomicAdd(&h[(key[r] >> shift) & (DIG - 1)], 1u);
     __syncthreads();
-    uint32_t* hrow = job.hist + ((size_t)seg * job.n_tiles + tile) * DIG;
+    uint32_t* hrow = job.hist + ((size_t)seg * (job.n_tiles + 1) + tile) * DIG;
     for (int d = tid; d < DIG; d += 256) hrow[d] = h[d];
+}
+
+constexpr int kSortFoldTiles = 64;
+// one thread per (segment, digit): the tiles' counts become exclusive prefixes over the tiles,
+// row n_tiles the totals
+template <int BITS>
+__global__ __launch_bounds__(256) void k_sort_scan(SortJob job) {
+    constexpr int DIG = 1 << BITS;
+    const int d = blockIdx.x * 256 + threadIdx.x, seg = blockIdx.y;
+    if (d >= DIG) return;
+    uint32_t* h = job.hist + (size_t)seg * (job.n_tiles + 1) * DIG + d;
+    uint32_t run = 0;
+    int t = 0;
+    for (; t + 8 <= job.n_tiles; t += 8) {  // eight loads in flight
+        uint32_t c[8];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) c[x] = h[(size_t)(t + x) * DIG];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) { h[(size_t)(t + x) * DIG] = run; run += c[x]; }
+    }
+    for (; t < job.n_tiles; ++t) { const uint32_t c = h[(size_t)t * DIG]; h[(size_t)t * DIG] = run; run += c; }
+    h[(size_t)job.n_tiles * DIG] = run;
 }
 
 template <int BITS>
@@ -250,10 +296,18 @@ __global__ __launch_bounds__(256) void k_sort_scatter(SortJob j0, SortJob j1, in
     // Step 1: thread t sums digits t, t + 256, ... over the tiles (lanes read consecutive words).
     uint32_t pre[DPT];
     {
-        const uint32_t* hseg = hist + (size_t)seg * n_tiles * DIG;
+        const uint32_t* hseg = hist + (size_t)seg * (n_tiles + 1) * DIG;
         uint32_t tot[DPT];
 #pragma unroll
         for (int q = 0; q < DPT; ++q) { tot[q] = 0; pre[q] = 0; }
+        if (n_tiles > kSortFoldTiles) {  // scanned by k_sort_scan
+#pragma unroll
+            for (int q = 0; q < DPT; ++q) {
+                const int d = q * 256 + tid;
+                pre[q] = d < DIG ? hseg[(size_t)tile * DIG + d] : 0u;
+                tot[q] = d < DIG ? hseg[(size_t)n_tiles * DIG + d] : 0u;
+            }
+        } else
         for (int t = 0; t < n_tiles; ++t) {
 #pragma unroll
             for (int q = 0; q < DPT; ++q) {
@@ -367,6 +421,9 @@ void launch_radix_sort2(SortBuffers* j0, SortBuffers* j1, int n_seg, bool first_
 #define KGE_SORT_PASS(B_)                                                                                     \
     case B_:                                                                                                  \
         if (!hist_done) hipLaunchKernelGGL(k_sort_hist<B_>, grid, dim3(256), 0, stream, a[0], a[1], shift);   \
+        for (int q = 0; q < n; ++q)                                                                           \
+            if (a[q].n_tiles > kSortFoldTiles)                                                                \
+                hipLaunchKernelGGL(k_sort_scan<B_>, dim3(((1 << B_) + 255) / 256, n_seg), dim3(256), 0, stream, a[q]); \
         hipLaunchKernelGGL(k_sort_scatter<B_>, grid, dim3(256), 0, stream, a[0], a[1], shift);                \
         break;
         switch (sp.bits[p]) {
@@ -395,13 +452,12 @@ int launch_radix_sort(uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint
 // ---- segments and chunks ---------------------------------------------------------------------
 // Three launches over tiles of 2048 sorted items (256 threads x 8 consecutive items), both
 // plans of every step in each launch, nothing handed between workgroups inside a launch:
-//   1. count: row starts per tile (a row starts where the key changes) and the tile's last one
-//      (short arrays skip this launch: the workgroups of 2. read the keys in front of their tile)
+//   1. count: row starts per tile (a row starts where the key's row number changes) and the tile's last one
 //   2. rows:  with the earlier tiles' counts in front, every item knows its distinct-row index
-//      and its row's first position.  Within a row the gradient contributions (value < n_real)
-//      come first (the sort is stable and they have the smaller item numbers), and every row
-//      holds at least one other member (its `remote` slot / the scatter-add's one item per table
-//      row): the first of those knows the row's number of contributions and "owns" the row.
+//      and its row's first position.  Within a row the gradient contributions (key flag 0)
+//      come first, and every row holds at least one other member (its `remote` slot / the
+//      scatter-add's one item per table row): the first of those knows the row's number of
+//      contributions and "owns" the row.
 //      The rows a tile owns are consecutive; their chunk counts are summed per tile.
 //   3. chunks: with the earlier tiles' chunk counts in front, the chunk tables of rows with more
 //      than direct_max contributions and the list of those rows.
@@ -414,7 +470,6 @@ static_assert(kSegTile == 256 * kSegPer, "256 threads x kSegPer items");
 //   2 chunks of the rows the tile owns   3 how many of them have chunks   4 the most contributions among them
 //   5 rows the tile owns   6 the first of them
 constexpr int kSegInfo = 8;
-constexpr int kSegInlineTiles = 0;   // (0: the count launch always runs)
 
 // kSegPer consecutive words from p + i0 (words past n read as zero); 16-byte loads when `vec`
 DEVINL void load_run(const uint32_t* __restrict__ p, int i0, int n, bool vec, uint32_t out[kSegPer]) {
@@ -491,7 +546,7 @@ DEVINL uint32_t start_flags(const uint32_t k[kSegPer], uint32_t k_prev, int i0, 
 #pragma unroll
     for (int x = 0; x < kSegPer; ++x) {
         const int i = i0 + x;
-        if (i < N && (i == 0 || k[x] != (x ? k[x - 1] : k_prev))) flags |= 1u << x;
+        if (i < N && (i == 0 || (k[x] >> kKeyFlagBits) != ((x ? k[x - 1] : k_prev) >> kKeyFlagBits))) flags |= 1u << x;
     }
     return flags;
 }
@@ -517,10 +572,6 @@ __global__ __launch_bounds__(256) void k_seg_count(SegJob j0, SegJob j1, int n_s
     }
 }
 
-// COUNT_INLINE: no k_seg_count launch went before; every workgroup counts the row starts of the
-// tiles in front of it itself (one pass over their keys: cheaper than a launch while the
-// arrays are short).
-template <bool COUNT_INLINE>
 __global__ __launch_bounds__(256) void k_seg_rows(SegJob j0, SegJob j1, int n_seg, int max_tiles,
                                                   uint32_t* __restrict__ tile_info) {
     __shared__ uint32_t lds[4][2];
@@ -544,31 +595,12 @@ __global__ __launch_bounds__(256) void k_seg_rows(SegJob j0, SegJob j1, int n_se
     load_run(keys, i0, N, vec, k);
     load_run(vals, i0, N, vec, v);
     const bool has_prev = i0 > 0 && i0 < N;
-    const uint32_t k_prev = has_prev ? keys[i0 - 1] : 0u, v_prev = has_prev ? vals[i0 - 1] : 0u;
+    const uint32_t k_prev = has_prev ? keys[i0 - 1] : 0u;
     // the earlier tiles: rows started in them, and the last start among them
     uint32_t rows_before = 0, start1_before = 0;
-    if (COUNT_INLINE) {
-        const int n_prev = w.tile * kSegTile;  // a multiple of 4, at most N
-        for (int p = 4 * tid; p < n_prev; p += 4 * 256) {
-            uint32_t q[4];
-            if (vec) {
-                const uint4 v4 = *reinterpret_cast<const uint4*>(keys + p);
-                q[0] = v4.x; q[1] = v4.y; q[2] = v4.z; q[3] = v4.w;
-            } else {
-#pragma unroll
-                for (int x = 0; x < 4; ++x) q[x] = keys[p + x];
-            }
-            const uint32_t before = p ? keys[p - 1] : ~q[0];  // position 0 starts a row
-            uint32_t f = (q[0] != before ? 1u : 0u) | (q[1] != q[0] ? 2u : 0u) | (q[2] != q[1] ? 4u : 0u) |
-                         (q[3] != q[2] ? 8u : 0u);
-            rows_before += __popc(f);
-            if (f) start1_before = (uint32_t)(p + 31 - __clz(f)) + 1u;  // positions grow with the loop
-        }
-    } else {
-        for (int t = tid; t < w.tile; t += 256) {
-            rows_before += info_seg[(size_t)t * kSegInfo];
-            start1_before = max(start1_before, info_seg[(size_t)t * kSegInfo + 1]);
-        }
+    for (int t = tid; t < w.tile; t += 256) {
+        rows_before += info_seg[(size_t)t * kSegInfo];
+        start1_before = max(start1_before, info_seg[(size_t)t * kSegInfo + 1]);
     }
     block_sum_max(rows_before, start1_before, lds);
 
@@ -585,16 +617,16 @@ __global__ __launch_bounds__(256) void k_seg_rows(SegJob j0, SegJob j1, int n_se
         if (i < N) {
             const bool f = (flags >> x) & 1u;
             if (f) {
-                uniq_key[u] = k[x];
+                uniq_key[u] = k[x] >> kKeyFlagBits;
                 seg_start[u] = (uint32_t)i;
                 start1 = (uint32_t)i + 1u;
                 ++u;
             }
             // u - 1 is this item's row, start1 - 1 that row's first position
-            if (v[x] < n_real) {
-                if (item_row) item_row[v[x]] = u - 1;
-            } else if (f || (x ? v[x - 1] : v_prev) < n_real) {
-                const uint32_t real = (uint32_t)i - (start1 - 1u);  // the row's contributions lie in front of it
+            if (item_row && v[x] < n_real) item_row[v[x]] = u - 1;
+            // the row's first member that is no contribution: its contributions lie in front of it
+            if ((k[x] & 1u) && (f || !((x ? k[x - 1] : k_prev) & 1u))) {
+                const uint32_t real = (uint32_t)i - (start1 - 1u);
                 seg_real[u - 1] = real;
                 const uint32_t nch = real > direct_max ? (real + chunk - 1) / chunk : 0u;
                 own_chunks += nch; own_hot += nch ? 1u : 0u; own_big = max(own_big, real);
@@ -705,14 +737,89 @@ void launch_find_segments2(const SegJob& j0, const SegJob* j1, int n_seg, uint32
     const SegJob& second = j1 ? *j1 : j0;
     const int max_tiles = (std::max(j0.N, j1 ? j1->N : 0) + kSegTile - 1) / kSegTile;
     const dim3 grid(max_tiles, j1 ? 2 * n_seg : n_seg);
-    // up to kSegInlineTiles tiles per array the row kernel counts the tiles in front of it itself
-    if (max_tiles <= kSegInlineTiles) {
-        hipLaunchKernelGGL(k_seg_rows<true>, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
-    } else {
-        hipLaunchKernelGGL(k_seg_count, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
-        hipLaunchKernelGGL(k_seg_rows<false>, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
-    }
+    hipLaunchKernelGGL(k_seg_count, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
+    hipLaunchKernelGGL(k_seg_rows, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
     hipLaunchKernelGGL(k_seg_chunks, grid, dim3(256), 0, stream, j0, second, n_seg, max_tiles, scratch);
+}
+
+// ---- merged tails ----------------------------------------------------------------------------
+// One workgroup per (block, step): the block's T tail rows (resolved like the tail contributions
+// in k_build_items) are sorted together with their positions by a bitonic network in LDS; a
+// distinct row becomes a column, numbered in ascending row order.
+constexpr int kMergeThreads = 256;
+__global__ __launch_bounds__(kMergeThreads) void k_merge_tails(PlanShape ps, const uint32_t* __restrict__ remote,
+                                                               const uint32_t* __restrict__ a2a,
+                                                               uint32_t* __restrict__ tkey, float* __restrict__ tmult,
+                                                               uint32_t* __restrict__ tcol,
+                                                               uint32_t* __restrict__ tcount) {
+    __shared__ uint64_t e[kMergeMaxT];          // (row, position), ascending after the sort
+    __shared__ uint32_t first[kMergeMaxT + 1];  // sorted index of every column's first entry
+    __shared__ uint32_t lds[4][2];
+    const int d = blockIdx.x, seg = blockIdx.y, step = ps.step0 + seg, tid = threadIdx.x;
+    const int S = ps.S, A = ps.A, NR = ps.NR, T = S * A, nst = ps.n_step;
+    int N = 1;
+    while (N < T) N <<= 1;
+    for (int i = tid; i < N; i += kMergeThreads) {
+        uint64_t v = ~0ull;  // padding sorts behind every row
+        if (i < T) {
+            const int j = i / A, ii = i - j * A;
+            const uint32_t slot = a2a[(((size_t)j * nst + step) * S + d) * A + ii];
+            const uint32_t base = ps.shared_table ? 0u : (uint32_t)j * (uint32_t)ps.n_entity;
+            const uint32_t row = base + remote[((size_t)j * nst + step) * NR + slot];
+            v = ((uint64_t)row << 32) | (uint32_t)i;
+        }
+        e[i] = v;
+    }
+    __syncthreads();
+    for (int k = 2; k <= N; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = tid; i < N / 2; i += kMergeThreads) {
+                const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1)), hi = lo | j;
+                const uint64_t a = e[lo], b = e[hi];
+                if ((a > b) == ((lo & k) == 0)) { e[lo] = b; e[hi] = a; }
+            }
+            __syncthreads();
+        }
+    // thread t owns sorted entries [t * per, (t + 1) * per)
+    const int per = (N + kMergeThreads - 1) / kMergeThreads;
+    const int i0 = tid * per;
+    uint32_t mine = 0;
+    for (int x = 0; x < per; ++x) {
+        const int i = i0 + x;
+        if (i < T && (i == 0 || (uint32_t)(e[i] >> 32) != (uint32_t)(e[i - 1] >> 32))) ++mine;
+    }
+    uint32_t before, eb, total, tb;
+    block_scan_256<false>(mine, 0u, lds, before, eb, total, tb);
+    const size_t out = ((size_t)step * S + d) * T;
+    uint32_t col = before;  // columns started in front of this thread's entries
+    for (int x = 0; x < per; ++x) {
+        const int i = i0 + x;
+        if (i >= T) break;
+        const uint32_t row = (uint32_t)(e[i] >> 32), pos = (uint32_t)e[i];
+        if (i == 0 || row != (uint32_t)(e[i - 1] >> 32)) {
+            first[col] = (uint32_t)i;
+            tkey[out + col] = row << kKeyFlagBits;
+            ++col;
+        }
+        tcol[out + pos] = col - 1;
+    }
+    if (tid == 0) {
+        first[total] = (uint32_t)T;
+        tcount[(size_t)step * S + d] = total;
+    }
+    __syncthreads();
+    const uint32_t pad_key = ((uint32_t)(e[0] >> 32) << kKeyFlagBits) | 1u;
+    for (int j = tid; j < T; j += kMergeThreads) {
+        const bool live = (uint32_t)j < total;
+        tmult[out + j] = live ? (float)(first[j + 1] - first[j]) : 0.f;
+        if (!live) tkey[out + j] = pad_key;
+    }
+}
+
+void launch_merge_tails(const PlanShape& ps, const uint32_t* remote, const uint32_t* a2a, uint32_t* tkey,
+                        float* tmult, uint32_t* tcol, uint32_t* tcount, hipStream_t stream) {
+    hipLaunchKernelGGL(k_merge_tails, dim3(ps.S, ps.step_count), dim3(kMergeThreads), 0, stream, ps, remote, a2a,
+                       tkey, tmult, tcol, tcount);
 }
 
 }  // namespace kge

@@ -20,9 +20,12 @@ __global__ __launch_bounds__(256) void k_score_bwd(BwdParams p) {
     __shared__ __attribute__((aligned(16))) float Cs[BJ][LDP];  // Cs[j][i]
     __shared__ __attribute__((aligned(16))) float Os[BJ][LDP];  // Os[j][k]
     const int B = p.B, T = p.T, Dp = p.Dp;
-    const int n_self = p.side_b ? T : B, n_other = p.side_b ? B : T;
+    const int n_self = p.side_b ? T : B;
     const TileId tile = xcd_tile((Dp + kScoreTile - 1) / kScoreTile, (n_self + kScoreTile - 1) / kScoreTile, p.S);
     const int d = tile.z, i0 = tile.y * kScoreTile, kt0 = tile.x * kScoreTile;
+    const int t_live = tail_limit(p.tcount, d, T, p.tpad);  // merged tails: the block's live columns
+    const int n_other = p.side_b ? B : t_live;
+    if (p.side_b && i0 >= t_live) return;
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int self_c0 = (p.side_b ? p.b_c0 + d * T : p.a_c0 + d * B);
     const int other_c0 = (p.side_b ? p.a_c0 + d * B : p.b_c0 + d * T);
@@ -205,8 +208,9 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wi = (wave >> 1) * (32 * AT), wk = (wave & 1) * 32;
     const int B = p.B, T = p.T, Dp = p.Dp;
-    const int n_self = SIDE_B ? T : B, n_other = SIDE_B ? B : T;
-    if (i0 >= n_self) return;  // the grid is sized for the longer side
+    const int t_live = tail_limit(p.tcount, d, T, p.tpad);  // merged tails: the block's live columns
+    const int n_self = SIDE_B ? T : B, n_other = SIDE_B ? B : t_live;
+    if (i0 >= (SIDE_B ? t_live : n_self)) return;  // the grid is sized for the longer side
     const int grad_c0 = SIDE_B ? p.b_c0 : p.a_c0;
     const int self_c0 = SIDE_B ? p.b_c0 + d * T : p.a_c0 + d * B;
     const int other_c0 = SIDE_B ? p.a_c0 + d * B : p.b_c0 + d * T;
@@ -255,6 +259,7 @@ DEVINL void bwd_mfma_body(const BwdParams& p, const int d, const int tile_x, con
     auto flag_of = [&](int i_tile, int j_tile) -> uint32_t {
         if (!nflag) return 0u;
         const int mt = SIDE_B ? j_tile : i_tile, nt = SIDE_B ? i_tile : j_tile;
+        if (32 * nt >= t_live) return 0u;  // columns the forward pass did not visit
         if (ALIGNED) return nflag[(size_t)mt * NTL + nt];
         return (mt < MT && nt < NTL) ? nflag[(size_t)mt * NTL + nt] : 0u;
     };
@@ -587,13 +592,17 @@ template <int TW>
 __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restrict__ operands,
                                                             const float* __restrict__ coef,
                                                             float* __restrict__ grad, int B, int T,
-                                                            int Dp, int a_c0, int b_c0) {
+                                                            int Dp, int a_c0, int b_c0,
+                                                            const uint32_t* __restrict__ tcount, int tpad) {
     __shared__ float part[2][L1P_WAVES][L1P_CB][64];
     const TileId tile = xcd_tile(Dp / 64, 1, (int)gridDim.x / (Dp / 64));
     const int d = tile.z, k = tile.x * 64 + (threadIdx.x & 63);
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int t0 = w * TW;
+    // merged tails: the block's live columns (a multiple of 64), split evenly over the waves in
+    // groups of four; TW is the most a wave may get
+    const int tw = __builtin_amdgcn_readfirstlane(tail_limit(tcount, d, T, tpad) / L1P_WAVES);
+    const int t0 = w * tw;
     const float* a_rows = operands + (size_t)(a_c0 + d * B) * Dp + k;
     const float* b_rows = operands + (size_t)(b_c0 + d * T + t0) * Dp + k;
     const float* crow = coef + (size_t)d * B * T + t0;
@@ -601,7 +610,7 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
     float bt[TW], gt[TW];
 #pragma unroll
     for (int j = 0; j < TW; ++j) {
-        bt[j] = b_rows[(size_t)j * Dp];
+        bt[j] = j < tw ? b_rows[(size_t)j * Dp] : 0.f;
         gt[j] = 0.f;
     }
     for (int b0 = 0, buf = 0; b0 < B; b0 += L1P_CB, buf ^= 1) {
@@ -612,14 +621,18 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
             const float* c = crow + (size_t)(b0 + bi) * T;
             float gp = 0.f;
 #pragma unroll
-            for (int j = 0; j < TW; ++j) {
-                // signum(a - b) with signum(0) = 0 (poplar_extensions l1distance.codelet.cpp:76-79):
-                // the difference's bit pattern read as an integer has its sign and is zero
-                // only for +0; converted to float (magnitude >= 1 unless zero) and clamped
-                // to [-1, 1].  (-0 never appears: the dense operands are stored with +0 added.)
-                const float sg = __builtin_amdgcn_fmed3f((float)__float_as_int(a - bt[j]), -1.f, 1.f);
-                gp = fmaf(c[j], sg, gp);
-                gt[j] = fmaf(-c[j], sg, gt[j]);
+            for (int j4 = 0; j4 < TW; j4 += 4) {
+                if (j4 >= tw) break;  // wave-uniform
+#pragma unroll
+                for (int j = j4; j < j4 + 4; ++j) {
+                    // signum(a - b) with signum(0) = 0 (poplar_extensions l1distance.codelet.cpp:76-79):
+                    // the difference's bit pattern read as an integer has its sign and is zero
+                    // only for +0; converted to float (magnitude >= 1 unless zero) and clamped
+                    // to [-1, 1].  (-0 never appears: the dense operands are stored with +0 added.)
+                    const float sg = __builtin_amdgcn_fmed3f((float)__float_as_int(a - bt[j]), -1.f, 1.f);
+                    gp = fmaf(c[j], sg, gp);
+                    gt[j] = fmaf(-c[j], sg, gt[j]);
+                }
             }
             part[buf][w][bi][lane] = gp;
         }
@@ -631,7 +644,8 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
         grad[(size_t)(a_c0 + d * B + b0 + w) * Dp + k] = sum;
     }
 #pragma unroll
-    for (int j = 0; j < TW; ++j) grad[(size_t)(b_c0 + d * T + t0 + j) * Dp + k] = gt[j];
+    for (int j = 0; j < TW; ++j)
+        if (j < tw) grad[(size_t)(b_c0 + d * T + t0 + j) * Dp + k] = gt[j];
 }
 
 // shapes the paired L1 kernel takes: tails split evenly over 16 waves, whole
@@ -639,7 +653,7 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
 static bool l1_pair_ok(const ScoreShape& sh) {
     const int tw = sh.T / L1P_WAVES;
     return sh.T % L1P_WAVES == 0 && (tw == 8 || tw == 16 || tw == 32) && sh.B % L1P_CB == 0 &&
-           sh.Dp % 64 == 0 && sh.S * (sh.Dp / 64) >= 128;
+           sh.Dp % 64 == 0 && sh.S * (sh.Dp / 64) >= 128 && (!sh.tcount || sh.tpad == 64);
 }
 
 void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* rel,
@@ -650,6 +664,7 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
     p.coef_div = nullptr; p.add_base = nullptr;
     p.S = sh.S; p.B = sh.B; p.T = sh.T; p.Dp = sh.Dp; p.vec_out = 1; p.use_mfma = sh.use_mfma;
     p.nearflag = nearflag;
+    p.tcount = sh.tcount; p.tpad = sh.tpad;
     p.a_rel_mode = sh.operands_dense ? 0 : (sh.score_fn == SCORE_DISTMULT ? 2 : 1);
     p.a_c0 = 0; p.b_c0 = sh.S * sh.B;
     const int dist_fn = sh.score_fn == SCORE_DISTMULT ? DIST_DOT : sh.dist_fn;
@@ -672,11 +687,11 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
         const dim3 grid = tile_grid(sh.Dp / 64, 1, sh.S);
         const int tw = sh.T / L1P_WAVES;
         if (tw == 32)
-            hipLaunchKernelGGL(k_score_bwd_l1_pair<32>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
+            hipLaunchKernelGGL(k_score_bwd_l1_pair<32>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0, sh.tcount, sh.tpad);
         else if (tw == 16)
-            hipLaunchKernelGGL(k_score_bwd_l1_pair<16>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
+            hipLaunchKernelGGL(k_score_bwd_l1_pair<16>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0, sh.tcount, sh.tpad);
         else
-            hipLaunchKernelGGL(k_score_bwd_l1_pair<8>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0);
+            hipLaunchKernelGGL(k_score_bwd_l1_pair<8>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0, sh.tcount, sh.tpad);
         return;
     }
     p.side_b = 0; p.grad_c0 = p.a_c0;
@@ -705,6 +720,7 @@ void launch_distance_grad(int dist_fn, const float* a, const float* b, const flo
     p.S = 1; p.B = M; p.T = N; p.Dp = D;
     p.side_b = 0; p.a_rel_mode = 0;
     p.a_c0 = 0; p.b_c0 = 0; p.grad_c0 = 0; p.use_mfma = 1; p.nearflag = nullptr;
+    p.tcount = nullptr; p.tpad = 1;
     p.vec_out = (D % 4 == 0) && ((uintptr_t)grad % 16 == 0);
     launch_bwd(p, dist_fn, stream);
 }
