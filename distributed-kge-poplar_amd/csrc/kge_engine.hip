@@ -269,6 +269,11 @@ struct kge_engine {
     int tpad = 64;  // live tail columns come in whole groups of this many (the scoring kernels' tile)
     DevBuf<uint32_t> tkey, tcol, tcount;
     DevBuf<float> tmult;
+    // additive setting execution.keep_gradients: the summed gradient of every distinct entity
+    // row and of every relation row of the last step stays on the device for "grad_dump"
+    bool keep_gradients = false;
+    DevBuf<float> gkeep_e, gkeep_r;
+    int last_step = -1;  // index (in the call's batch) of the step the kept gradients belong to
     int e_ustride, e_cstride, r_ustride, r_cstride, n_rel_items;
     uint32_t *e_sorted_vals = nullptr, *r_sorted_vals = nullptr;
     // step
@@ -538,6 +543,10 @@ void parse_settings(kge_engine& E, const Items& s) {
     // additive: merged tails.  Not with TransH (its L1 part has kernels of its own), the norm
     // regularisers (they count a row's members that carry no gradient as its gathered slots) or
     // bfloat16 scoring, and for tail lists that fit one workgroup's sort.
+    E.keep_gradients = s.find("execution.keep_gradients") ? s.boolean("execution.keep_gradients") : false;
+    if (E.keep_gradients && (E.F || contributions_read_tables(E)))
+        throw std::invalid_argument("'execution.keep_gradients' is implemented for score functions whose gradient "
+                                    "contributions are used as stored (TransE, TransH) without entity features");
     E.merge_tails = s.find("execution.merge_tails") ? s.boolean("execution.merge_tails") : true;
     if (E.score_fn == SCORE_TRANSH || E.reg_on || E.score_bf16 || E.T > kMergeMaxT) E.merge_tails = false;
     E.Dp = round_up(E.D, (emb_et == ET_F32 && mom_et == ET_F32) ? 4 : 8);
@@ -616,6 +625,10 @@ void allocate(kge_engine& E) {
         E.hist.alloc(radix_sort_hist_words((int)(2 * R), (int)ns, bits) + radix_sort_hist_words(E.n_rel_items, (int)ns, bits));
     }
     E.seg_scratch.alloc(find_segments_scratch_words((int)(2 * R), E.n_rel_items, (int)ns));
+    if (E.keep_gradients) {
+        E.gkeep_e.alloc(R * E.Dp);
+        E.gkeep_r.alloc((size_t)E.n_rel_rows * E.Dp);
+    }
     if (E.merge_tails) {
         E.tkey.alloc(ns * S * E.T);
         E.tcol.alloc(ns * S * E.T);
@@ -1309,6 +1322,8 @@ void run_step(kge_engine& E, int i) {
     ae.alpha = alpha;
     ae.rows_per_alpha = E.shared_table ? 0u : (uint32_t)E.n_entity;
 
+    if (E.keep_gradients) { ae.grad_out = E.gkeep_e.p; ar.grad_out = E.gkeep_r.p; E.last_step = i; }
+
     // The feature MLP's input holds the embedding, so part of the embedding's gradient comes
     // back through the MLP: the rows' summed gradient first (a pass without update), the MLP's
     // backward per row, then the update with what that adds.
@@ -1588,6 +1603,36 @@ void run_plan_dump(kge_engine& E, const Items& in) {
             float* host = (float*)in.array("tail_multiplicity", KGE_F32, {ST});
             HIP_CHECK(hipMemcpy(host, E.tmult.p + i * ST, ST * 4, hipMemcpyDeviceToHost));
         }
+    }
+}
+
+// "grad_dump" (with execution.keep_gradients): the gradients the last step's updates were made
+// from, as the step's loss.backward(lossScale) leaves them after multiUpdateAdd
+// (src/poplar_kge.cpp:691, src/pag/pag.cpp:721-743), i.e. times the loss scale:
+//   unique_rows u32[R], counts u32[2]   the step's distinct entity rows (ascending), how many
+//   entity_gradient f32[R, D]           their summed gradients, in that order
+//   relation_gradient f32[n_relation rows, D]  every relation row's (TransH: then the normals')
+void run_grad_dump(kge_engine& E, const Items& in) {
+    if (!E.keep_gradients || E.last_step < 0)
+        throw std::invalid_argument("'grad_dump' needs execution.keep_gradients and a train_step_loop before it");
+    const size_t R = E.R, i = (size_t)E.last_step;
+    HIP_CHECK(hipStreamSynchronize(E.stream));
+    if (in.find("unique_rows")) {
+        uint32_t* host = (uint32_t*)in.array("unique_rows", KGE_U32, {R});
+        HIP_CHECK(hipMemcpy(host, E.e_uniq.p + i * E.e_ustride, R * 4, hipMemcpyDeviceToHost));
+    }
+    if (in.find("counts")) {
+        uint32_t* host = (uint32_t*)in.array("counts", KGE_U32, {2});
+        HIP_CHECK(hipMemcpy(host, E.e_counts.p + 2 * i, 8, hipMemcpyDeviceToHost));
+    }
+    if (in.find("entity_gradient")) {
+        float* host = (float*)in.array("entity_gradient", KGE_F32, {R, (size_t)E.D});
+        HIP_CHECK(hipMemcpy2D(host, (size_t)E.D * 4, E.gkeep_e.p, (size_t)E.Dp * 4, (size_t)E.D * 4, R, hipMemcpyDeviceToHost));
+    }
+    if (in.find("relation_gradient")) {
+        float* host = (float*)in.array("relation_gradient", KGE_F32, {(size_t)E.n_rel_rows, (size_t)E.D});
+        HIP_CHECK(hipMemcpy2D(host, (size_t)E.D * 4, E.gkeep_r.p, (size_t)E.Dp * 4, (size_t)E.D * 4, (size_t)E.n_rel_rows,
+                              hipMemcpyDeviceToHost));
     }
 }
 
@@ -1891,6 +1936,7 @@ int kge_engine_run(kge_engine* engine, const char* command, kge_item* items, siz
         else if (cmd == "stage_batch") run_stage_batch(E, in);
         else if (cmd == "timing") run_timing(E, in);
         else if (cmd == "plan_dump") run_plan_dump(E, in);
+        else if (cmd == "grad_dump") run_grad_dump(E, in);
         else if (cmd == "gather_benchmark") run_gather_benchmark(E, in);
         else if (cmd == "variables") { /* served by kge_engine_variable_info */ }
         else if (cmd == "predict") run_predict(E, in);

@@ -580,79 +580,120 @@ void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
 // contraction form, so this is vector-ALU work; computing the term once and
 // adding it to the head's sum and (negated) to the tail's sum halves it.
 // One workgroup of 16 waves per (block, 64-column slice); a lane owns one
-// column.  Wave w keeps tails [w*TW, (w+1)*TW) and their gradient sums in
+// column.  Wave w keeps tails [w*tw, (w+1)*tw) and their gradient sums in
 // registers and walks over all heads; a head's sum over one wave's tails is a
 // partial, the 16 partials of a head meet in LDS and are added in wave order
-// (deterministic).  The coefficients of a (head, tail range) are wave-uniform
-// and come in through scalar loads.
-constexpr int L1P_CB = 16;     // heads per chunk (one per wave in the reduction)
+// (deterministic).  The coefficients of a (head, tail range) are the same for
+// every lane: the workgroup stages the coefficient rows of eight heads at a time
+// in LDS (one 16-byte load per thread, the next chunk's in flight under the
+// current one's arithmetic) and every wave reads its four at a time with one
+// LDS instruction whose lanes all name the same address (a broadcast, no bank
+// conflict).  As scalar loads (wave-uniform operands straight from memory) the
+// same coefficients bounded the kernel: each of a block's four column slices
+// pulled the whole coefficient matrix through the scalar caches.
+constexpr int L1P_CB = 8;      // heads per chunk
 constexpr int L1P_WAVES = 16;
 
+constexpr int L1P_MAX_T = 512;  // tails per block at most (32 per wave)
+
+// the work of one wave with exactly TW tails (TW a multiple of 4): straight-line code over
+// its tails, their values and sums in registers
 template <int TW>
+DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restrict__ b_rows,
+                         const float* __restrict__ cblk, float* __restrict__ grad_a, float* __restrict__ grad_b,
+                         int B, int T, int Dp, int t0, int t4, int w, int lane,
+                         float (*part)[L1P_WAVES][L1P_CB][64], float (*cs)[L1P_CB][L1P_MAX_T]) {
+    const int tid = threadIdx.x;
+    // staging: thread -> (head, four columns) of a chunk's coefficient rows
+    const bool stager = tid < L1P_CB * t4;
+    const int s_head = tid / t4, s_col = (tid - s_head * t4) * 4;
+    float4 c_next = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (stager) {
+        c_next = *reinterpret_cast<const float4*>(cblk + (size_t)s_head * T + s_col);
+        *reinterpret_cast<float4*>(&cs[0][s_head][s_col]) = c_next;
+    }
+    float bt[TW], gt[TW];
+#pragma unroll
+    for (int j = 0; j < TW; ++j) {
+        bt[j] = b_rows[(size_t)j * Dp];
+        gt[j] = 0.f;
+    }
+    __syncthreads();
+    for (int b0 = 0, buf = 0; b0 < B; b0 += L1P_CB, buf ^= 1) {
+        const bool more = b0 + L1P_CB < B;
+        if (stager && more) c_next = *reinterpret_cast<const float4*>(cblk + (size_t)(b0 + L1P_CB + s_head) * T + s_col);
+        float a_next = a_rows[(size_t)b0 * Dp];
+#pragma unroll 1
+        for (int bi = 0; bi < L1P_CB; ++bi) {
+            const float a = a_next;
+            if (bi + 1 < L1P_CB) a_next = a_rows[(size_t)(b0 + bi + 1) * Dp];
+            const float* c = &cs[buf][bi][t0];
+            float gp = 0.f;
+#pragma unroll
+            for (int j4 = 0; j4 < TW; j4 += 4) {
+                const float4 c4 = *reinterpret_cast<const float4*>(c + j4);
+                const float cv[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    // signum(a - b) with signum(0) = 0 (poplar_extensions l1distance.codelet.cpp:76-79)
+                    // from instructions of the fast class only (subtract, fused multiply-add):
+                    // the difference times 2^126 plus one half, clamped to [0, 1] by the
+                    // instruction's own output modifier, is 1 / 0.5 / 0 for a positive / zero /
+                    // negative difference (any normal float times 2^126 is at least 1 in
+                    // magnitude); twice that minus one is the sign.
+                    const float half_step = __builtin_amdgcn_fmed3f(fmaf(a - bt[j4 + x], 0x1p126f, 0.5f), 0.f, 1.f);
+                    const float sg = fmaf(half_step, 2.f, -1.f);
+                    gp = fmaf(cv[x], sg, gp);
+                    gt[j4 + x] = fmaf(-cv[x], sg, gt[j4 + x]);
+                }
+            }
+            part[buf][w][bi][lane] = gp;
+        }
+        if (stager && more) *reinterpret_cast<float4*>(&cs[buf ^ 1][s_head][s_col]) = c_next;
+        __syncthreads();
+        // waves 0 .. 7 add the 16 partials of head b0 + w
+        if (w < L1P_CB) {
+            float sum = 0.f;
+#pragma unroll
+            for (int v = 0; v < L1P_WAVES; ++v) sum += part[buf][v][w][lane];
+            grad_a[(size_t)(b0 + w) * Dp] = sum;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < TW; ++j) grad_b[(size_t)j * Dp] = gt[j];
+}
+
 __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restrict__ operands,
                                                             const float* __restrict__ coef,
                                                             float* __restrict__ grad, int B, int T,
                                                             int Dp, int a_c0, int b_c0,
                                                             const uint32_t* __restrict__ tcount, int tpad) {
     __shared__ float part[2][L1P_WAVES][L1P_CB][64];
+    __shared__ __attribute__((aligned(16))) float cs[2][L1P_CB][L1P_MAX_T];
     const TileId tile = xcd_tile(Dp / 64, 1, (int)gridDim.x / (Dp / 64));
-    const int d = tile.z, k = tile.x * 64 + (threadIdx.x & 63);
-    const int lane = threadIdx.x & 63;
+    const int d = tile.z, lane = threadIdx.x & 63, k = tile.x * 64 + lane;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // merged tails: the block's live columns (a multiple of 64), split evenly over the waves in
-    // groups of four; TW is the most a wave may get
-    const int tw = __builtin_amdgcn_readfirstlane(tail_limit(tcount, d, T, tpad) / L1P_WAVES);
-    const int t0 = w * tw;
+    // merged tails: the block's live columns (a multiple of 64), split evenly over the waves
+    const int t_live = __builtin_amdgcn_readfirstlane(tail_limit(tcount, d, T, tpad));
+    const int tw = t_live / L1P_WAVES, t0 = w * tw;
     const float* a_rows = operands + (size_t)(a_c0 + d * B) * Dp + k;
     const float* b_rows = operands + (size_t)(b_c0 + d * T + t0) * Dp + k;
-    const float* crow = coef + (size_t)d * B * T + t0;
-
-    float bt[TW], gt[TW];
-#pragma unroll
-    for (int j = 0; j < TW; ++j) {
-        bt[j] = j < tw ? b_rows[(size_t)j * Dp] : 0.f;
-        gt[j] = 0.f;
+    const float* cblk = coef + (size_t)d * B * T;
+    float* grad_a = grad + (size_t)(a_c0 + d * B) * Dp + k;
+    float* grad_b = grad + (size_t)(b_c0 + d * T + t0) * Dp + k;
+#define KGE_L1P(TW_) \
+    case TW_: l1_pair_wave<TW_>(a_rows, b_rows, cblk, grad_a, grad_b, B, T, Dp, t0, t_live / 4, w, lane, part, cs); break;
+    switch (tw) {  // one of eight copies of the loop, chosen per block
+        KGE_L1P(4) KGE_L1P(8) KGE_L1P(12) KGE_L1P(16) KGE_L1P(20) KGE_L1P(24) KGE_L1P(28) KGE_L1P(32)
     }
-    for (int b0 = 0, buf = 0; b0 < B; b0 += L1P_CB, buf ^= 1) {
-        float a_next = a_rows[(size_t)b0 * Dp];
-        for (int bi = 0; bi < L1P_CB; ++bi) {
-            const float a = a_next;
-            if (bi + 1 < L1P_CB) a_next = a_rows[(size_t)(b0 + bi + 1) * Dp];
-            const float* c = crow + (size_t)(b0 + bi) * T;
-            float gp = 0.f;
-#pragma unroll
-            for (int j4 = 0; j4 < TW; j4 += 4) {
-                if (j4 >= tw) break;  // wave-uniform
-#pragma unroll
-                for (int j = j4; j < j4 + 4; ++j) {
-                    // signum(a - b) with signum(0) = 0 (poplar_extensions l1distance.codelet.cpp:76-79):
-                    // the difference's bit pattern read as an integer has its sign and is zero
-                    // only for +0; converted to float (magnitude >= 1 unless zero) and clamped
-                    // to [-1, 1].  (-0 never appears: the dense operands are stored with +0 added.)
-                    const float sg = __builtin_amdgcn_fmed3f((float)__float_as_int(a - bt[j]), -1.f, 1.f);
-                    gp = fmaf(c[j], sg, gp);
-                    gt[j] = fmaf(-c[j], sg, gt[j]);
-                }
-            }
-            part[buf][w][bi][lane] = gp;
-        }
-        __syncthreads();
-        // wave w adds the 16 partials of head b0 + w
-        float sum = 0.f;
-#pragma unroll
-        for (int v = 0; v < L1P_WAVES; ++v) sum += part[buf][v][w][lane];
-        grad[(size_t)(a_c0 + d * B + b0 + w) * Dp + k] = sum;
-    }
-#pragma unroll
-    for (int j = 0; j < TW; ++j)
-        if (j < tw) grad[(size_t)(b_c0 + d * T + t0 + j) * Dp + k] = gt[j];
+#undef KGE_L1P
 }
 
 // shapes the paired L1 kernel takes: tails split evenly over 16 waves, whole
 // chunks of heads, whole 64-column slices, and enough workgroups for the chip
 static bool l1_pair_ok(const ScoreShape& sh) {
-    const int tw = sh.T / L1P_WAVES;
-    return sh.T % L1P_WAVES == 0 && (tw == 8 || tw == 16 || tw == 32) && sh.B % L1P_CB == 0 &&
+    // (T % 64 == 0: every live count is a multiple of 64, 4 tails per wave at least)
+    return sh.T % 64 == 0 && sh.T >= 128 && sh.T <= L1P_MAX_T && sh.B % L1P_CB == 0 &&
            sh.Dp % 64 == 0 && sh.S * (sh.Dp / 64) >= 128 && (!sh.tcount || sh.tpad == 64);
 }
 
@@ -685,13 +726,8 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
     if (dist_fn == DIST_L1 && sh.use_mfma && sh.operands_dense && plain && ent.pitch == (int64_t)sh.Dp * 4 && l1_pair_ok(sh)) {
         const float* ops = reinterpret_cast<const float*>(ent.base);
         const dim3 grid = tile_grid(sh.Dp / 64, 1, sh.S);
-        const int tw = sh.T / L1P_WAVES;
-        if (tw == 32)
-            hipLaunchKernelGGL(k_score_bwd_l1_pair<32>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0, sh.tcount, sh.tpad);
-        else if (tw == 16)
-            hipLaunchKernelGGL(k_score_bwd_l1_pair<16>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0, sh.tcount, sh.tpad);
-        else
-            hipLaunchKernelGGL(k_score_bwd_l1_pair<8>, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0, p.b_c0, sh.tcount, sh.tpad);
+        hipLaunchKernelGGL(k_score_bwd_l1_pair, grid, dim3(1024), 0, stream, ops, coef, grad, sh.B, sh.T, sh.Dp, p.a_c0,
+                           p.b_c0, sh.tcount, sh.tpad);
         return;
     }
     p.side_b = 0; p.grad_c0 = p.a_c0;

@@ -461,6 +461,13 @@ API float kge_oracle_loss(const kge_oracle_cfg* c, const float* score, const uin
  * sum of all their slots' gradients; with unique `remote` per shard and
  * private tables this is exactly the reference.                            */
 
+/* Test hook: when set, every training step also stores the gradients its updates are made from
+ * (after the scatter-add over duplicate slots, times the loss scale; later steps overwrite):
+ * ent[key * D + k] for every gathered table row, rel[r * RD + k] for every relation row.     */
+static double* g_tap_ent = NULL;
+static double* g_tap_rel = NULL;
+API void kge_oracle_gradient_tap(double* ent, double* rel) { g_tap_ent = ent; g_tap_rel = rel; }
+
 static int cmp_u64(const void* a, const void* b) {
     uint64_t x = *(const uint64_t*)a, y = *(const uint64_t*)b;
     return (x > y) - (x < y);
@@ -931,6 +938,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
                     g[k] += gh[k] + (gt ? gt[k] : 0) + (gr ? gr[k] : 0) + (gm ? gm[k] : 0);
             }
             for (int64_t k = 0; k < D; ++k) gf[k] = (float)g[k];
+            if (g_tap_ent) for (int64_t k = 0; k < D; ++k) g_tap_ent[key * D + k] = (double)g[k];
             float* row = table + key * ROW;
             const int64_t shard = c->shared_table ? 0 : key / NE;
             kge_oracle_adam(row, row + D, row + 2 * D, gf, D, alpha[shard] * c->lr_mod_entity,
@@ -952,6 +960,7 @@ API int kge_oracle_train_step(const kge_oracle_cfg* c, float* table, float* rel,
         float* gf = (float*)malloc(sizeof(float) * (size_t)D);
         for (int64_t r = 0; r < NRELT; ++r) {
             for (int64_t k = 0; k < RD; ++k) gf[k] = (float)grel[r * RD + k];
+            if (g_tap_rel) for (int64_t k = 0; k < RD; ++k) g_tap_rel[r * RD + k] = (double)grel[r * RD + k];
             const int64_t shard = c->shared_table ? 0 : (r % NREL) / (NREL / S);
             kge_oracle_adam(rel + r * RD, rel_m + r * RD, rel_v + r * RD, gf, RD,
                             alpha[shard] * c->lr_mod_relation, c->beta_m, c->beta_v, c->epsilon,

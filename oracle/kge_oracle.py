@@ -220,6 +220,15 @@ class Oracle:
         loss = self.lib.kge_oracle_loss(C.byref(cfg), _p(score), _p(label), _p(ds))
         return loss, ds
 
+    def gradient_tap(self, ent=None, rel=None):
+        """Test hook: float64 arrays [table rows, D] and [relation rows, D] that every following
+        training step fills with the summed gradients its updates are made from (None: off)."""
+        for a in (ent, rel):
+            assert a is None or (a.dtype == np.float64 and a.flags.c_contiguous)
+        self._tap = (ent, rel)   # keeps the arrays alive while the C side writes to them
+        self.lib.kge_oracle_gradient_tap(_p(ent) if ent is not None else None,
+                                         _p(rel) if rel is not None else None)
+
     # -- whole step --------------------------------------------------------
     def train_step_loop(self, cfg, state, lr, batch):
         """Runs n_step steps in place on ``state`` and returns loss f32[S].

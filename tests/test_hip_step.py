@@ -616,3 +616,97 @@ def test_dropout_masks_follow_the_optimiser_step(oracle64):
         oracle64.train_step_loop(make_cfg(**plain), st_plain, np.array([0.1, 0.07], np.float32), K.random_batch(c, 2, rng))
     k = "feature_projection"
     assert K.rel_l2(st_h[k] - st0[k], st_plain[k] - st0[k]) > 0.05
+
+
+# ---- the step's gradients themselves -------------------------------------------------------------
+
+GRADIENT_CASES = {
+    # the 1M-row workload's block shape (256 positives x 256 shared tails, D = 256), raw power-law
+    # ids over one shared table: hot rows, repeated tails, tile-aligned fast paths
+    "c2_shaped_l2": (dict(distance_fn="L2", n_shard=4, batch=256, a2a=64, dim=256, feature=0, n_entity=20_000,
+                          n_relation=40, gamma=10.0, shared_table=True), ("mfma_bf16x3", "mfma", "valu")),
+    # the one-pass L1 backward (tails split over sixteen waves)
+    "paired_l1": (dict(distance_fn="L1", n_shard=32, batch=32, a2a=8, dim=256, feature=0, n_entity=4000,
+                       n_relation=8, gamma=6.0, shared_table=True), ("mfma_bf16x3",)),
+}
+
+
+@pytest.mark.parametrize("merge", [True, False])
+@pytest.mark.parametrize("name,scoring", [(n, s) for n, (_, ss) in GRADIENT_CASES.items() for s in ss])
+def test_step_gradients_vs_oracle(oracle64, name, scoring, merge):
+    """The summed gradient of every distinct entity row and of every relation row of one step
+    (what loss.backward(lossScale) and multiUpdateAdd leave, src/poplar_kge.cpp:691,
+    src/pag/pag.cpp:721-743) against the float64 oracle's: 1e-5 relative as a whole, and every
+    element within 1e-5 of its row's root mean square."""
+    import libpoplar_kge
+
+    c = K.cfg_dict(**GRADIENT_CASES[name][0])
+    rng = np.random.default_rng(31)
+    st0 = K.make_state(c, rng)
+    batch = K.raw_batch(c, 1, rng)
+    lr = np.full(c["n_shard"], 0.01, np.float32)
+    engine = libpoplar_kge.Engine(H.engine_settings(c, 1, **{"execution.scoring": scoring,
+                                                             "execution.keep_gradients": True,
+                                                             "execution.merge_tails": merge}), "")
+    H.load_state(engine, c, st0)
+    H.train(engine, c, lr, batch)
+    S, B, A, D = c["n_shard"], c["batch"], c["a2a"], c["dim"]
+    R = S * (B + S * A)
+    out = dict(unique_rows=np.zeros(R, np.uint32), counts=np.zeros(2, np.uint32),
+               entity_gradient=np.zeros((R, D), np.float32),
+               relation_gradient=np.zeros((c["n_relation"], D), np.float32))
+    engine.run("grad_dump", out)
+    ent = np.full((st0["entity_data"].shape[0], D), np.nan)
+    rel = np.full((c["n_relation"], D), np.nan)
+    oracle64.gradient_tap(ent, rel)
+    try:
+        oracle64.train_step_loop(make_cfg(**c), K.copy_state(st0), lr, batch)
+    finally:
+        oracle64.gradient_tap(None, None)
+    U = int(out["counts"][0])
+    rows = out["unique_rows"][:U]
+    np.testing.assert_array_equal(rows, np.flatnonzero(~np.isnan(ent[:, 0])))
+    for got, ref in ((out["entity_gradient"][:U], ent[rows]), (out["relation_gradient"], rel)):
+        assert K.rel_l2(got, ref) < 1e-5
+        rms = np.sqrt(np.mean(ref * ref, axis=1, keepdims=True))
+        assert np.all(np.abs(got - ref) <= 1e-5 * rms + 1e-30), float(np.max(np.abs(got - ref) / (rms + 1e-30)))
+    assert np.count_nonzero(np.any(ent[rows] != 0, axis=1)) > U // 2
+
+
+# ---- merged tails: blocks whose tail lists repeat rows ---------------------------------------------
+
+def _repeated_tail_batch(c, n_step, rng, kind):
+    """Batches in the reference's layout whose tail lists repeat rows: `label_repeated` points every
+    positive's label at a row that other tail positions of the block hold too; `one_row` fills a
+    whole block's tails with a single row; `few_rows` draws all tails from four rows."""
+    batch = K.random_batch(c, n_step, rng)
+    S, A = c["n_shard"], c["a2a"]
+    a2a = batch["a2a"]                      # [src shard, step, dst block, A]: slots of the source's remote
+    if kind == "one_row":
+        # block 0: every source sends its slot 0 only, which holds the same id everywhere (one
+        # table row with a shared table, one row per source's table otherwise)
+        a2a[:, :, 0, :] = 0
+        batch["remote"][:, :, 0] = batch["remote"][:1, :, 0]
+    elif kind == "few_rows":
+        a2a[...] = rng.integers(0, 4, a2a.shape)
+        batch["remote"][1:, :, :4] = batch["remote"][:1, :, :4]
+    else:
+        # tail position 0 of every block repeats at positions 1 and 2 (same source, same slot); labels name 0, 1 or 2
+        a2a[0, :, :, 1] = a2a[0, :, :, 0]
+        a2a[0, :, :, 2] = a2a[0, :, :, 0]
+        batch["tail"][...] = rng.integers(0, 3, batch["tail"].shape)
+    return batch
+
+
+@pytest.mark.parametrize("kind", ["label_repeated", "one_row", "few_rows"])
+@pytest.mark.parametrize("name", ["l2_logsigmoid", "l2_softmax", "l1_adversarial", "demo_l1_logsigmoid",
+                                  "distmult_softmax_feat", "aligned_l2", "aligned_l2_softmax", "paired_l1_t256",
+                                  "mid_l1"])
+def test_step_repeated_tails(oracle64, name, kind):
+    """One score column per distinct tail row, weighted by its multiplicity, against the oracle,
+    which scores every tail position (src/poplar_kge.cpp:615-660): the label's row repeated among
+    the negatives, a block whose tails are all one row, tails drawn from four rows."""
+    kw = dict(CASES[name])
+    run_case(oracle64, kw, n_step=2, batch_fn=lambda c, n, rng: _repeated_tail_batch(c, n, rng, kind))
+    run_case(oracle64, kw, n_step=2, batch_fn=lambda c, n, rng: _repeated_tail_batch(c, n, rng, kind),
+             **{"execution.merge_tails": False})

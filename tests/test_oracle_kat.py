@@ -379,6 +379,32 @@ def _run_case(orc, kw, batch_fn, n_step=3, pad=0, lr=(0.1, 0.07)):
     return c, st0, st_o, batch
 
 
+@pytest.mark.parametrize("name", ["l2_logsigmoid_nofeat", "transe_matmul", "shared_table_l2", "l1_adversarial"])
+def test_gradient_tap_vs_autograd(orc, name):
+    """The oracle's gradient tap (the summed gradient of every gathered row and of every relation
+    row, as the updates use them) against autograd's gradients of the independent restatement."""
+    c = K.cfg_dict(**dict(STEP_CASES[name], feature=0))
+    rng = np.random.default_rng(4)
+    st0 = K.make_state(c, rng)
+    batch = K.random_batch(c, 1, rng)
+    lr = np.full(c["n_shard"], 0.05, np.float32)
+    n_rows = st0["entity_data"].shape[0]
+    ent = np.full((n_rows, c["dim"]), np.nan)
+    rel = np.full((c["n_relation"], c["dim"]), np.nan)
+    orc.gradient_tap(ent, rel)
+    try:
+        orc.train_step_loop(make_cfg(**c), K.copy_state(st0), lr, batch)
+    finally:
+        orc.gradient_tap(None, None)
+    grads = {}
+    torch_restatement.step(c, K.copy_state(st0), lr, K.step_slice(batch, 0), grads)
+    tol = 1e-9 if orc.precision == "f64" else 2e-4
+    assert np.array_equal(np.flatnonzero(~np.isnan(ent[:, 0])), grads["rows"])   # exactly the gathered rows
+    assert K.rel_l2(ent[grads["rows"]], grads["entity"]) < tol
+    assert K.rel_l2(rel, grads["relation"]) < tol
+    assert np.any(grads["entity"] != 0) and np.any(grads["relation"] != 0)
+
+
 @pytest.mark.parametrize("name", list(STEP_CASES))
 def test_train_step_vs_autograd(orc, name):
     _run_case(orc, STEP_CASES[name], K.random_batch)

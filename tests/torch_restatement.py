@@ -62,8 +62,10 @@ def round_bf16_ste(x):
     return x + (x.detach().to(T.float32).to(T.bfloat16).to(T.float64) - x.detach())
 
 
-def step(cfg, state, lr, batch_step):
-    """One step in place on ``state`` (float32 arrays); returns loss[S].
+def step(cfg, state, lr, batch_step, grads=None):
+    """One step in place on ``state`` (float32 arrays); returns loss[S].  ``grads`` (a dict):
+    receives autograd's gradients of the step, ``rows`` (distinct table rows, ascending),
+    ``entity`` [rows, D] and ``relation`` [n_relation, D].
 
     cfg: dict(n_shard, n_entity, n_relation, dim, feature, batch, a2a,
     score_fn, distance_fn, loss_fn, shared_table, gamma, beta_m, beta_v,
@@ -221,6 +223,8 @@ def step(cfg, state, lr, batch_step):
 
     g = emb.grad.numpy()
     rows = uniq.numpy()
+    if grads is not None:
+        grads.update(rows=rows.copy(), entity=g.copy(), relation=rel.grad.numpy().copy())
     ed = state["entity_data"]
     p = ed[rows, :D].astype(np.float64)
     m = ed[rows, D:2 * D].astype(np.float64)
