@@ -12,7 +12,10 @@
 #include <cmath>
 #include <cstring>
 #include <memory>
+#include <condition_variable>
+#include <exception>
 #include <mutex>
+#include <thread>
 #include <sstream>
 #include <stdexcept>
 #include <string>
@@ -212,6 +215,7 @@ struct kge_engine {
     float* h_loss_pin = nullptr;
     float* d_loss_pin = nullptr;  // the device's view of h_loss_pin: the loss kernel stores there, no copy follows
     hipEvent_t counts_ready = nullptr;
+    hipEvent_t counts_wait = nullptr;  // the event the host waits for before it reads the counts
     bool counts_pending = false;
     bool counts_known = false;
     int plan_readback_steps = 8;  // additive setting execution.plan_readback_steps: calls of at least this many steps
@@ -255,7 +259,18 @@ struct kge_engine {
     uint32_t step = 0;
 
     // staged batch
-    DevBuf<uint32_t> d_remote, d_a2a, d_head, d_relation, d_tail;
+    // The batch on the device, step by step: step i's remote [S, NR], a2a [S, S, A], head, relation,
+    // tail [S, B] back to back (idx_words words per step), so that any range of steps is one
+    // contiguous upload.  h_idx: the same layout in pinned host memory, filled (and every index
+    // checked) by the host while it re-orders the caller's [S, n_step, ...] arrays.
+    DevBuf<uint32_t> d_idx;
+    uint32_t* h_idx = nullptr;
+    size_t idx_words = 0, off_a2a = 0, off_head = 0, off_relation = 0, off_tail = 0;
+    // Host arrays are taken in chunks of steps: while the device runs one chunk, the host checks
+    // and re-orders the next, whose upload (copy_stream) and plan (plan_stream) run beside the
+    // current chunk's kernels
+    hipStream_t copy_stream = nullptr, plan_stream = nullptr;
+    std::vector<hipEvent_t> chunk_copied, chunk_planned;
     bool staged = false;
     // plan
     DevBuf<uint32_t> ckey, crel, clabel, ek_a, ev_a, ek_b, ev_b, rk_a, rv_a, rk_b, rv_b, hist, seg_scratch;
@@ -319,6 +334,11 @@ struct kge_engine {
         for (auto& e : scored) if (e) (void)hipEventDestroy(e);
         for (auto& e : merged) if (e) (void)hipEventDestroy(e);
         if (merge_stream) (void)hipStreamDestroy(merge_stream);
+        if (copy_stream) (void)hipStreamDestroy(copy_stream);
+        if (plan_stream) (void)hipStreamDestroy(plan_stream);
+        for (auto& e : chunk_copied) (void)hipEventDestroy(e);
+        for (auto& e : chunk_planned) (void)hipEventDestroy(e);
+        if (h_idx) (void)hipHostFree(h_idx);
         if (stream) (void)hipStreamDestroy(stream);
     }
 };
@@ -608,11 +628,12 @@ void allocate(kge_engine& E) {
     for (DevBuf<float>* b : {&E.proj, &E.proj_m, &E.proj_v}) { b->alloc(E.nets * proj_n); b->zero(st); }
 
     const size_t ns = E.n_step, S = E.S, B = E.B, A = E.A, R = E.R, SB = S * B;
-    E.d_remote.alloc(ns * R);
-    E.d_a2a.alloc(ns * S * S * A);
-    E.d_head.alloc(ns * SB);
-    E.d_relation.alloc(ns * SB);
-    E.d_tail.alloc(ns * SB);
+    E.off_a2a = R; E.off_head = E.off_a2a + S * S * A; E.off_relation = E.off_head + SB;
+    E.off_tail = E.off_relation + SB; E.idx_words = E.off_tail + SB;
+    E.d_idx.alloc(ns * E.idx_words);
+    HIP_CHECK(hipHostMalloc((void**)&E.h_idx, ns * E.idx_words * 4, hipHostMallocDefault));
+    HIP_CHECK(hipStreamCreate(&E.copy_stream));
+    HIP_CHECK(hipStreamCreate(&E.plan_stream));
 
     E.ckey.alloc(ns * R);
     E.crel.alloc(ns * SB);
@@ -901,32 +922,53 @@ BatchPtrs bind_batch(kge_engine& E, const Items& in) {
     return b;
 }
 
-// Every index a kernel will dereference is checked here, on the host.
-void validate_batch(const kge_engine& E, const BatchPtrs& b) {
-    auto check = [](const char* name, const uint32_t* v, size_t n, uint32_t limit) {
-        uint32_t worst = 0;
-        for (size_t i = 0; i < n; ++i) worst = std::max(worst, v[i]);
-        if (n && worst >= limit) {
-            std::ostringstream msg;
-            msg << "'" << name << "' holds index " << worst << " out of range [0, " << limit << ")";
-            throw std::invalid_argument(msg.str());
-        }
-    };
+// Steps [s0, s0 + sn) of the caller's arrays ([S, n_step, ...] each) into the pinned staging
+// buffer in the device's step-by-step layout.  Every index a kernel will dereference is checked
+// here, on the host, while it passes through.
+void stage_steps(kge_engine& E, const BatchPtrs& b, int s0, int sn) {
     const size_t S = E.S, ns = E.n_step;
-    check("remote", b.remote, S * ns * E.NR, (uint32_t)E.n_entity);
-    check("a2a", b.a2a, S * ns * S * E.A, (uint32_t)E.NR);
-    check("head", b.head, S * ns * E.B, (uint32_t)E.NR);
-    check("relation", b.relation, S * ns * E.B, (uint32_t)E.n_rel);
-    check("tail", b.tail, S * ns * E.B, (uint32_t)E.T);
+    struct Part { const char* name; const uint32_t* src; size_t width, offset; uint32_t limit; };
+    const Part parts[5] = {
+        {"remote", b.remote, (size_t)E.NR, 0, (uint32_t)E.n_entity},
+        {"a2a", b.a2a, S * E.A, E.off_a2a, (uint32_t)E.NR},
+        {"head", b.head, (size_t)E.B, E.off_head, (uint32_t)E.NR},
+        {"relation", b.relation, (size_t)E.B, E.off_relation, (uint32_t)E.n_rel},
+        {"tail", b.tail, (size_t)E.B, E.off_tail, (uint32_t)E.T},
+    };
+    for (int i = s0; i < s0 + sn; ++i) {
+        uint32_t* step_block = E.h_idx + (size_t)i * E.idx_words;
+        for (const Part& p : parts) {
+            // v < limit for every word, without a compare per word: with limit <= 2^31 the top bit
+            // of v | (limit - 1 - v) is set exactly when v >= limit
+            const uint32_t lm1 = p.limit - 1u;
+            uint32_t acc = 0;
+            for (size_t s = 0; s < S; ++s) {
+                const uint32_t* src = p.src + (s * ns + (size_t)i) * p.width;
+                uint32_t* dst = step_block + p.offset + s * p.width;
+                for (size_t x = 0; x < p.width; ++x) {
+                    const uint32_t v = src[x];
+                    dst[x] = v;
+                    acc |= v | (lm1 - v);
+                }
+            }
+            uint32_t worst = 0;
+            if (acc >> 31)
+                for (size_t s = 0; s < S; ++s)
+                    for (size_t x = 0; x < p.width; ++x)
+                        worst = std::max(worst, p.src[(s * ns + (size_t)i) * p.width + x]);
+            if (worst >= p.limit) {
+                std::ostringstream msg;
+                msg << "'" << p.name << "' holds index " << worst << " out of range [0, " << p.limit << ") (step " << i << ")";
+                throw std::invalid_argument(msg.str());
+            }
+        }
+    }
 }
 
-void upload_batch(kge_engine& E, const BatchPtrs& b) {
-    const hipStream_t st = E.stream;
-    HIP_CHECK(hipMemcpyAsync(E.d_remote.p, b.remote, E.d_remote.n * 4, hipMemcpyHostToDevice, st));
-    HIP_CHECK(hipMemcpyAsync(E.d_a2a.p, b.a2a, E.d_a2a.n * 4, hipMemcpyHostToDevice, st));
-    HIP_CHECK(hipMemcpyAsync(E.d_head.p, b.head, E.d_head.n * 4, hipMemcpyHostToDevice, st));
-    HIP_CHECK(hipMemcpyAsync(E.d_relation.p, b.relation, E.d_relation.n * 4, hipMemcpyHostToDevice, st));
-    HIP_CHECK(hipMemcpyAsync(E.d_tail.p, b.tail, E.d_tail.n * 4, hipMemcpyHostToDevice, st));
+// the staged steps' upload
+void upload_steps(kge_engine& E, int s0, int sn, hipStream_t st) {
+    HIP_CHECK(hipMemcpyAsync(E.d_idx.p + (size_t)s0 * E.idx_words, E.h_idx + (size_t)s0 * E.idx_words,
+                             (size_t)sn * E.idx_words * 4, hipMemcpyHostToDevice, st));
 }
 
 struct KernelTimer {
@@ -961,15 +1003,15 @@ void collect_kernel_times(kge_engine& E) {
 
 // Index-only work for steps [s0, s0 + sn) of the resident batch: contribution
 // keys, the two sorts and the segment / chunk tables.
-void run_plan(kge_engine& E, int s0, int sn) {
-    KernelTimer timer(E, K_PLAN);
-    const hipStream_t st = E.stream;
+void run_plan(kge_engine& E, int s0, int sn, hipStream_t st) {
+    KernelTimer timer(E, K_PLAN);  // (events on the engine's stream: meaningful when st is that stream)
     const size_t R = E.R, SB = (size_t)E.S * E.B, N = 2 * R, NRI = E.n_rel_items;
     PlanShape ps;
     ps.n_step = E.n_step; ps.S = E.S; ps.B = E.B; ps.A = E.A; ps.NR = E.NR;
     ps.n_entity = E.n_entity; ps.shared_table = E.shared_table; ps.n_relation = E.n_rel;
     ps.rel_copies = E.rel_copies;
     ps.step0 = s0; ps.step_count = sn;
+    ps.idx_step_stride = (int64_t)E.idx_words;
     ps.merge_tails = E.merge_tails ? 1 : 0;
     const int ebits = std::max(1, bit_length((uint64_t)E.n_rows - 1)) + kKeyFlagBits;
     const int rbits = std::max(1, bit_length((uint64_t)E.n_rel_rows - 1)) + kKeyFlagBits;
@@ -977,8 +1019,9 @@ void run_plan(kge_engine& E, int s0, int sn) {
     uint32_t* const e_hist = E.hist.p;
     uint32_t* const r_hist = E.hist.p + radix_sort_hist_words((int)N, E.n_step, std::max(ebits, rbits));
     if (E.merge_tails)
-        launch_merge_tails(ps, E.d_remote.p, E.d_a2a.p, E.tkey.p, E.tmult.p, E.tcol.p, E.tcount.p, st);
-    launch_build_items(ps, E.d_remote.p, E.d_a2a.p, E.d_head.p, E.d_relation.p, E.d_tail.p, E.tkey.p, E.tcol.p, E.ckey.p,
+        launch_merge_tails(ps, E.d_idx.p, E.d_idx.p + E.off_a2a, E.tkey.p, E.tmult.p, E.tcol.p, E.tcount.p, st);
+    launch_build_items(ps, E.d_idx.p, E.d_idx.p + E.off_a2a, E.d_idx.p + E.off_head, E.d_idx.p + E.off_relation,
+                       E.d_idx.p + E.off_tail, E.tkey.p, E.tcol.p, E.ckey.p,
                        E.crel.p, E.clabel.p, E.ek_a.p, E.ev_a.p, E.rk_a.p, E.rv_a.p,
                        sort_passes(std::max(ebits, rbits)).bits[0], e_hist, r_hist, st);
     SortBuffers es = {}, rs = {};
@@ -1239,7 +1282,7 @@ void run_step(kge_engine& E, int i) {
     }
 
     if (E.counts_pending) {  // the plan's counts size the launches from here on
-        HIP_CHECK(hipEventSynchronize(E.counts_ready));
+        HIP_CHECK(hipEventSynchronize(E.counts_wait));
         E.counts_pending = false;
     }
     const float* alpha = E.d_alpha.p + (size_t)i * 9 * E.S;
@@ -1457,13 +1500,9 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     if (in.find("profile_kernels")) E.profile_kernels = in.boolean("profile_kernels");
     struct Restore { bool& ref; bool v; ~Restore() { ref = v; } } restore{E.profile_kernels, profile_saved};
     HIP_CHECK(hipEventRecord(E.ev[0], st));
-    if (!staged) {
-        const BatchPtrs b = bind_batch(E, in);
-        validate_batch(E, b);
-        upload_batch(E, b);
-    } else if (!E.staged) {
-        throw std::invalid_argument("train_step_loop with staged=true needs a preceding stage_batch");
-    }
+    if (staged && !E.staged) throw std::invalid_argument("train_step_loop with staged=true needs a preceding stage_batch");
+    BatchPtrs host = {};
+    if (!staged) host = bind_batch(E, in);
     // step sizes of every step of this call (adamStepSizeAutoIncrement, frnn.cpp:42-59)
     E.h_alpha.resize((size_t)E.n_step * 9 * S);
     for (int i = s0; i < s0 + sn; ++i) {
@@ -1488,19 +1527,129 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
     std::memcpy(E.h_alpha_pin, E.h_alpha.data(), E.h_alpha.size() * 4);
     HIP_CHECK(hipMemcpyAsync(E.d_alpha.p, E.h_alpha_pin, E.h_alpha.size() * 4, hipMemcpyHostToDevice, st));
     HIP_CHECK(hipEventRecord(E.ev[1], st));
-    run_plan(E, s0, sn);
     E.step_of_first = (int)E.step - s0;  // step i of the batch is optimiser step E.step + (i - s0)
+    // the per-step counts (distinct rows, chunks, rows with chunks, biggest row) size the launches of
+    // calls long enough to pay for the wait; the segment kernel writes them into pinned host memory
     E.counts_known = sn >= E.plan_readback_steps;
     E.counts_pending = false;
-    if (E.counts_known) {
-        // the segment kernel has written the counts into pinned host memory; the host waits for
-        // that kernel when the first launch sized by them is due, with the first step's scoring
-        // launches already queued behind it
-        HIP_CHECK(hipEventRecord(E.counts_ready, st));
-        E.counts_pending = true;
+    if (staged) {
+        run_plan(E, s0, sn, st);
+        if (E.counts_known) {
+            // the host waits for that kernel when the first launch sized by the counts is due, with
+            // the first step's scoring launches already queued behind it
+            HIP_CHECK(hipEventRecord(E.counts_ready, st));
+            E.counts_wait = E.counts_ready;
+            E.counts_pending = true;
+        }
+        HIP_CHECK(hipEventRecord(E.ev[2], st));
+        for (int i = s0; i < s0 + sn; ++i) run_step(E, i);
+    } else {
+        // Host arrays (EngineImpl::runProgram binds them on every run, src/poplar_kge.cpp:967-975):
+        // chunks of 2, 4, 8, ... steps.  A helper thread checks and re-orders chunk k + 1 (host
+        // memory only) while this thread launches chunk k's kernels; chunk k + 1's upload and
+        // plan then run beside chunk k's kernels on streams of their own.  Only the first chunk's
+        // preparation is exposed.
+        std::vector<std::pair<int, int>> chunks;
+        for (int c0 = s0, cn = 2; c0 < s0 + sn; c0 += cn, cn *= 2) {
+            cn = std::min(cn, s0 + sn - c0);
+            chunks.emplace_back(c0, cn);
+        }
+        while (E.chunk_copied.size() < chunks.size()) {
+            hipEvent_t a = nullptr, b = nullptr;
+            HIP_CHECK(hipEventCreateWithFlags(&a, hipEventDisableTiming));
+            E.chunk_copied.push_back(a);
+            HIP_CHECK(hipEventCreateWithFlags(&b, hipEventDisableTiming));
+            E.chunk_planned.push_back(b);
+        }
+        // the helper: chunks 1 .. n - 1 in order; `ready` counts the chunks staged so far
+        std::mutex mu;
+        std::condition_variable cv;
+        size_t ready = 1;
+        std::exception_ptr failed;
+        std::thread helper;
+        if (chunks.size() > 1)
+            helper = std::thread([&]() {
+                for (size_t k = 1; k < chunks.size(); ++k) {
+                    try {
+                        stage_steps(E, host, chunks[k].first, chunks[k].second);
+                    } catch (...) {
+                        std::lock_guard<std::mutex> lock(mu);
+                        failed = std::current_exception();
+                        cv.notify_all();
+                        return;
+                    }
+                    std::lock_guard<std::mutex> lock(mu);
+                    ready = k + 1;
+                    cv.notify_all();
+                }
+            });
+        int done = 0;  // steps handed to the device
+        const bool readback = E.counts_known;
+        auto enqueue = [&](size_t k) {  // chunk k is staged: its upload and its plan
+            if (k == 0) {
+                // nothing to run beside: straight onto the engine's stream, and no wait for the
+                // plan's counts (the first chunk's launches are sized for the worst case), so
+                // that this thread goes on to the next chunk at once
+                upload_steps(E, chunks[0].first, chunks[0].second, st);
+                run_plan(E, chunks[0].first, chunks[0].second, st);
+                HIP_CHECK(hipEventRecord(E.chunk_planned[0], st));
+                return;
+            }
+            upload_steps(E, chunks[k].first, chunks[k].second, E.copy_stream);
+            HIP_CHECK(hipEventRecord(E.chunk_copied[k], E.copy_stream));
+            HIP_CHECK(hipStreamWaitEvent(E.plan_stream, E.chunk_copied[k], 0));
+            // every plan works in the same histogram and segment scratch: one at a time (plans
+            // from the second chunk's on follow one another on their stream anyway)
+            if (k == 1) HIP_CHECK(hipStreamWaitEvent(E.plan_stream, E.chunk_planned[0], 0));
+            run_plan(E, chunks[k].first, chunks[k].second, E.plan_stream);
+            HIP_CHECK(hipEventRecord(E.chunk_planned[k], E.plan_stream));
+        };
+        try {
+            stage_steps(E, host, chunks[0].first, chunks[0].second);
+            enqueue(0);
+            for (size_t k = 0; k < chunks.size(); ++k) {
+                if (k > 0) HIP_CHECK(hipStreamWaitEvent(st, E.chunk_planned[k], 0));
+                if (k == 0) HIP_CHECK(hipEventRecord(E.ev[2], st));
+                E.counts_known = readback && k > 0;
+                if (E.counts_known) {  // waited for when the chunk's first update is due
+                    E.counts_wait = E.chunk_planned[k];
+                    E.counts_pending = true;
+                }
+                // the next chunk's upload and plan go out as soon as the helper has staged it, between
+                // this chunk's step launches: the plan is a chain of short launches and needs the
+                // time this chunk's kernels take
+                bool next_out = k + 1 >= chunks.size();
+                for (int i = chunks[k].first; i < chunks[k].first + chunks[k].second; ++i) {
+                    run_step(E, i);
+                    if (!next_out) {
+                        std::unique_lock<std::mutex> lock(mu);
+                        const bool staged_next = ready > k + 1;
+                        lock.unlock();
+                        if (staged_next) { enqueue(k + 1); next_out = true; }
+                    }
+                }
+                done += chunks[k].second;
+                if (!next_out) {
+                    std::unique_lock<std::mutex> lock(mu);
+                    cv.wait(lock, [&]() { return ready > k + 1 || failed; });
+                    if (ready <= k + 1) std::rethrow_exception(failed);
+                    lock.unlock();
+                    enqueue(k + 1);
+                }
+            }
+            if (helper.joinable()) helper.join();
+        } catch (...) {
+            // an index out of range in a later chunk: the chunks before it have run
+            if (helper.joinable()) helper.join();
+            (void)hipStreamSynchronize(E.copy_stream);
+            (void)hipStreamSynchronize(E.plan_stream);
+            (void)hipStreamSynchronize(st);
+            E.step += (uint32_t)done;
+            E.staged = false;
+            throw;
+        }
+        E.staged = true;  // the whole batch is resident now
     }
-    HIP_CHECK(hipEventRecord(E.ev[2], st));
-    for (int i = s0; i < s0 + sn; ++i) run_step(E, i);
     launch_loss_finalize(E.loss_part.p + (size_t)s0 * E.S * E.n_part, sn, E.S, E.n_part, 1.f / (float)sn,
                          E.d_loss_pin, st, E.reg_on ? E.reg_loss_part.p + (size_t)s0 * E.S : nullptr, E.loss_step.p);
     HIP_CHECK(hipGetLastError());
@@ -1515,8 +1664,9 @@ void run_train_step_loop(kge_engine& E, const Items& in) {
 
 void run_stage_batch(kge_engine& E, const Items& in) {
     const BatchPtrs b = bind_batch(E, in);
-    validate_batch(E, b);
-    upload_batch(E, b);
+    E.staged = false;
+    stage_steps(E, b, 0, E.n_step);
+    upload_steps(E, 0, E.n_step, E.stream);
     HIP_CHECK(hipStreamSynchronize(E.stream));
     E.staged = true;
 }

@@ -44,6 +44,10 @@ struct PlanShape {
     int rel_copies;           // 1; 2 for TransH, whose relation table holds a second row (the
                               // hyperplane normal, row n_relation + r) per relation
     int step0, step_count;    // the steps of the resident batch to plan
+    // the index arrays lie step by step: step i's remote [S, NR], a2a [S, S, A], head, relation and
+    // tail [S, B] start idx_step_stride words behind step i - 1's (the pointers handed to the
+    // launchers are step 0's)
+    int64_t idx_step_stride;
     int merge_tails;          // the blocks' tail lists have been merged (launch_merge_tails)
 };
 

@@ -44,7 +44,8 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
                                                      uint32_t* __restrict__ rel_hist) {
     __shared__ uint32_t h[1 << kSortMaxBits];
     const int seg = blockIdx.y, step = ps.step0 + seg, tid = threadIdx.x;
-    const int S = ps.S, B = ps.B, A = ps.A, NR = ps.NR, T = S * A, nst = ps.n_step;
+    const int S = ps.S, B = ps.B, A = ps.A, NR = ps.NR, T = S * A;
+    const size_t W = (size_t)ps.idx_step_stride;
     const int R = S * NR, SB = S * B;
     const int SBr = SB * ps.rel_copies;
     const int n_rel_items = SBr + ps.n_relation * ps.rel_copies;
@@ -67,7 +68,7 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
             if (it < SB) {
                 const int d = it / B, b = it - d * B;
                 src[r] = d;
-                slot[r] = head[((size_t)d * nst + step) * B + b];
+                slot[r] = head[(size_t)step * W + d * B + b];
             } else if (it < R) {
                 const int cc = it - SB;
                 if (merged) {
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
                     const int d = cc / T, t = cc - d * T;
                     const int j = t / A, i = t - j * A;
                     src[r] = j;
-                    slot[r] = a2a[(((size_t)j * nst + step) * S + d) * A + i];
+                    slot[r] = a2a[(size_t)step * W + ((size_t)j * S + d) * A + i];
                 }
             } else if (it < 2 * R) {
                 const int sl = it - R;
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
             const int it = item[r];
             if (merged && it >= SB && it < R) key[r] = slot[r];
             else if (it < 2 * R)
-                key[r] = ((base + remote[((size_t)src[r] * nst + step) * NR + slot[r]]) << kKeyFlagBits) | (it < R ? 0u : 1u);
+                key[r] = ((base + remote[(size_t)step * W + (size_t)src[r] * NR + slot[r]]) << kKeyFlagBits) | (it < R ? 0u : 1u);
             else key[r] = 0u;
         }
 #pragma unroll
@@ -112,8 +113,8 @@ __global__ __launch_bounds__(kBuildThreads) void k_build_items(PlanShape ps, con
             if (it < SBr) {
                 const int copy = it / SB, c = it - copy * SB;
                 const int d = c / B, b = c - d * B;
-                key[r] = relation[((size_t)d * nst + step) * B + b];
-                if (copy == 0) label[r] = tail[((size_t)d * nst + step) * B + b];
+                key[r] = relation[(size_t)step * W + d * B + b];
+                if (copy == 0) label[r] = tail[(size_t)step * W + d * B + b];
                 if (copy == 0 && ps.merge_tails) label[r] = tcol[((size_t)step * S + d) * T + label[r]];
             } else if (it < n_rel_items) {
                 key[r] = it - SBr;
@@ -756,16 +757,17 @@ __global__ __launch_bounds__(kMergeThreads) void k_merge_tails(PlanShape ps, con
     __shared__ uint32_t first[kMergeMaxT + 1];  // sorted index of every column's first entry
     __shared__ uint32_t lds[4][2];
     const int d = blockIdx.x, seg = blockIdx.y, step = ps.step0 + seg, tid = threadIdx.x;
-    const int S = ps.S, A = ps.A, NR = ps.NR, T = S * A, nst = ps.n_step;
+    const int S = ps.S, A = ps.A, NR = ps.NR, T = S * A;
+    const size_t W = (size_t)ps.idx_step_stride;
     int N = 1;
     while (N < T) N <<= 1;
     for (int i = tid; i < N; i += kMergeThreads) {
         uint64_t v = ~0ull;  // padding sorts behind every row
         if (i < T) {
             const int j = i / A, ii = i - j * A;
-            const uint32_t slot = a2a[(((size_t)j * nst + step) * S + d) * A + ii];
+            const uint32_t slot = a2a[(size_t)step * W + ((size_t)j * S + d) * A + ii];
             const uint32_t base = ps.shared_table ? 0u : (uint32_t)j * (uint32_t)ps.n_entity;
-            const uint32_t row = base + remote[((size_t)j * nst + step) * NR + slot];
+            const uint32_t row = base + remote[(size_t)step * W + (size_t)j * NR + slot];
             v = ((uint64_t)row << 32) | (uint32_t)i;
         }
         e[i] = v;

@@ -65,14 +65,15 @@ TrainingSettings = _record(
     "hidden_regularisation learning_rate:float learning_rate_decay learning_rate_modifiers "
     "adam_beta_m:float adam_beta_v:float adam_epsilon:float weight_decay:float loss_scale:float")
 # additive fields: shared_table, embedding_dtype, feature_dtype, profile_kernels, scoring, scoring_dtype,
-# predict_chunk_rows
+# predict_chunk_rows, merge_tails, keep_gradients
 ExecutionSettings = _record(
     "ExecutionSettings",
     "device:str dtype:str train_steps_per_program_run:int rw_batch_size:int "
     "predict_hr_batch_size:int predict_tail_batch_size:int predict_n_best:int shared_table:bool "
-    "embedding_dtype feature_dtype profile_kernels:bool scoring scoring_dtype predict_chunk_rows",
+    "embedding_dtype feature_dtype profile_kernels:bool scoring scoring_dtype predict_chunk_rows "
+    "merge_tails keep_gradients",
     shared_table=False, embedding_dtype=None, feature_dtype=None, profile_kernels=False, scoring=None,
-    scoring_dtype=None, predict_chunk_rows=None)
+    scoring_dtype=None, predict_chunk_rows=None, merge_tails=None, keep_gradients=None)
 LogSettings = _record("LogSettings", "path wandb:bool steps_per_log:int predict_at")
 
 CODE_CHANGES: Tuple[str, ...] = ("HIP-device",)

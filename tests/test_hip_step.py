@@ -710,3 +710,41 @@ def test_step_repeated_tails(oracle64, name, kind):
     run_case(oracle64, kw, n_step=2, batch_fn=lambda c, n, rng: _repeated_tail_batch(c, n, rng, kind))
     run_case(oracle64, kw, n_step=2, batch_fn=lambda c, n, rng: _repeated_tail_batch(c, n, rng, kind),
              **{"execution.merge_tails": False})
+
+
+def test_host_arrays_are_checked_chunk_by_chunk():
+    """Host index arrays are checked, re-ordered and uploaded in chunks of 2, 4, 8, ... steps beside
+    the device's work.  An index out of range raises as before; the chunks in front of the
+    offending one have been applied by then (the reference checks shapes and types only,
+    src/poplar_kge.cpp:69-106), and the engine stays usable."""
+    import libpoplar_kge
+
+    c = K.cfg_dict(feature=0, n_shard=2, batch=6, a2a=5, dim=8, n_entity=90, n_relation=12)
+    rng = np.random.default_rng(5)
+    st0 = K.make_state(c, rng)
+    n_step = 7                                   # chunks of 2, 4 and 1 steps
+    batch = K.random_batch(c, n_step, rng)
+    engine = libpoplar_kge.Engine(H.engine_settings(c, n_step), "")
+    H.load_state(engine, c, st0)
+    bad = {k: v.copy() for k, v in batch.items()}
+    bad["a2a"][1, 6, 0, 2] = 10**6               # in the last chunk
+    with pytest.raises(ValueError, match=r"'a2a' holds index 1000000 out of range \[0, 16\) \(step 6\)"):
+        H.train(engine, c, 0.05, bad)
+    st = H.read_state(engine, c)
+    assert st["step"] == st0["step"] + 6         # the first two chunks ran
+    # the same six steps through the oracle, then a whole good call on top: the engine is intact
+    ref = K.copy_state(st0)
+    from oracle.kge_oracle import Oracle
+    orc = Oracle("f64")
+    orc.train_step_loop(make_cfg(**c), ref, 0.05, {k: v[:, :6] for k, v in batch.items()})
+    assert K.rel_l2(st["entity_data"], ref["entity_data"]) < 1e-5
+    loss_h = H.train(engine, c, 0.05, batch)
+    loss_o = orc.train_step_loop(make_cfg(**c), ref, 0.05, batch)
+    np.testing.assert_allclose(loss_h, loss_o, rtol=1e-5)
+    assert K.rel_l2(H.read_state(engine, c)["entity_data"], ref["entity_data"]) < 1e-5
+    # an index out of range in the first chunk: nothing has run
+    bad = {k: v.copy() for k, v in batch.items()}
+    bad["remote"][0, 1, 3] = 90
+    with pytest.raises(ValueError, match="'remote' holds index 90 out of range"):
+        H.train(engine, c, 0.05, bad)
+    assert H.read_state(engine, c)["step"] == st0["step"] + 6 + n_step
