@@ -560,15 +560,16 @@ void parse_settings(kge_engine& E, const Items& s) {
     E.T = E.S * E.A;
     E.NR = E.B + E.T;
     E.R = E.S * E.NR;
-    // additive: merged tails.  Not with TransH (its L1 part has kernels of its own), the norm
-    // regularisers (they count a row's members that carry no gradient as its gathered slots) or
-    // bfloat16 scoring, and for tail lists that fit one workgroup's sort.
+    // additive: merged tails.  Not with TransH (its L1 part has kernels of its own) or the norm
+    // regularisers (they count a row's members that carry no gradient as its gathered slots),
+    // and for tail lists that fit one workgroup's sort.
     E.keep_gradients = s.find("execution.keep_gradients") ? s.boolean("execution.keep_gradients") : false;
     if (E.keep_gradients && (E.F || contributions_read_tables(E)))
         throw std::invalid_argument("'execution.keep_gradients' is implemented for score functions whose gradient "
                                     "contributions are used as stored (TransE, TransH) without entity features");
     E.merge_tails = s.find("execution.merge_tails") ? s.boolean("execution.merge_tails") : true;
-    if (E.score_fn == SCORE_TRANSH || E.reg_on || E.score_bf16 || E.T > kMergeMaxT) E.merge_tails = false;
+    if (E.score_fn == SCORE_TRANSH || E.reg_on || E.T > kMergeMaxT) E.merge_tails = false;
+    E.tpad = E.score_bf16 ? 128 : 64;  // the bfloat16 products work in tiles of 128
     E.Dp = round_up(E.D, (emb_et == ET_F32 && mom_et == ET_F32) ? 4 : 8);
     E.Fp = E.F ? round_up(E.F, feat_et == ET_F32 ? 4 : 8) : 0;
     RowLayout& L = E.L;
@@ -1194,12 +1195,17 @@ void run_step(kge_engine& E, int i) {
         const size_t head_n = SB * (size_t)Dp;
         GemmNT g = {};
         g.batches = E.S;
+        // merged tails: block d's live tail columns end at its distinct count (whole tiles)
+        const uint32_t* const tc = sh.tcount;
+        g.limit_stride = 1;
         { KernelTimer t(E, K_FWD);
           g.A = E.opnd16.p; g.lda = Dp; g.a_batch = (int64_t)Bn * Dp;
           g.Bt = E.opnd16.p + head_n; g.ldb = Dp; g.b_batch = (int64_t)Tn * Dp;
           g.C = E.coef.p; g.ldc = Tn; g.c_batch = (int64_t)Bn * Tn;
           g.M = Bn; g.N = Tn; g.K = Dp;
-          launch_gemm_nt_bf16(g, st); }
+          g.n_limit = tc;
+          launch_gemm_nt_bf16(g, st);
+          g.n_limit = nullptr; }
         // only the bfloat16 coefficients are read from here on
         { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, nullptr, loss_part, E.coef16.p, st, false); }
         // q^T and tails^T: one launch over all operand rows when there is a single block
@@ -1207,25 +1213,32 @@ void run_step(kge_engine& E, int i) {
         const bool one_block = E.S == 1;
         const int64_t ldT = one_block ? Bn + Tn : 0;
         { KernelTimer t(E, K_BWD);
+          TransposeLimit tails, coefs;   // dead tail columns are neither transposed nor multiplied
+          tails.rows = tc; tails.stride = 1; tails.pad = E.tpad;
+          coefs.cols = tc; coefs.stride = 1; coefs.pad = E.tpad;
           if (one_block) {
-              launch_transpose_bf16(E.opnd16.p, false, 1, Bn + Tn, Dp, Dp, 0, E.opndT16.p, nullptr, st);
+              tails.row_base = Bn;
+              launch_transpose_bf16(E.opnd16.p, false, 1, Bn + Tn, Dp, Dp, 0, E.opndT16.p, nullptr, st, tails);
           } else {
               launch_transpose_bf16(E.opnd16.p, false, E.S, Bn, Dp, Dp, (int64_t)Bn * Dp, E.opndT16.p, nullptr, st);
               launch_transpose_bf16(E.opnd16.p + head_n, false, E.S, Tn, Dp, Dp, (int64_t)Tn * Dp,
-                                    E.opndT16.p + head_n, nullptr, st);
+                                    E.opndT16.p + head_n, nullptr, st, tails);
           }
-          launch_transpose_bf16(E.coef16.p, false, E.S, Bn, Tn, Tn, (int64_t)Bn * Tn, E.coefT16.p, nullptr, st);
+          launch_transpose_bf16(E.coef16.p, false, E.S, Bn, Tn, Tn, (int64_t)Bn * Tn, E.coefT16.p, nullptr, st, coefs);
           // d q [B, Dp] = c [B, T] . tails [T, Dp]
           g.A = E.coef16.p; g.lda = Tn; g.a_batch = (int64_t)Bn * Tn;
           g.Bt = one_block ? E.opndT16.p + Bn : E.opndT16.p + head_n; g.ldb = one_block ? (int)ldT : Tn; g.b_batch = (int64_t)Dp * Tn;
           g.C = E.grad.p; g.ldc = Dp; g.c_batch = (int64_t)Bn * Dp;
           g.M = Bn; g.N = Dp; g.K = Tn; g.part = E.gemm_part.p;
+          g.k_limit = tc;
           launch_gemm_nt_bf16(g, st);
+          g.k_limit = nullptr;
           // d tails [T, Dp] = c^T [T, B] . q [B, Dp]
           g.A = E.coefT16.p; g.lda = Bn; g.a_batch = (int64_t)Tn * Bn;
           g.Bt = E.opndT16.p; g.ldb = one_block ? (int)ldT : Bn; g.b_batch = (int64_t)Dp * Bn;
           g.C = E.grad.p + head_n; g.ldc = Dp; g.c_batch = (int64_t)Tn * Dp;
           g.M = Tn; g.N = Dp; g.K = Bn;
+          g.m_limit = tc;
           launch_gemm_nt_bf16(g, st); }
     } else if (transh) {
         // transHScore (:551-565): c = n . tail and its backward are dot-product scoring on

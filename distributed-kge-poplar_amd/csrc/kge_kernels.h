@@ -208,19 +208,29 @@ struct GemmNT {
     float* part; int ksplit;                    // scratch for split contractions (or null); set by the launcher
     const char* add_base; int64_t add_pitch; int add_etype;
     const uint32_t* add_index; const uint32_t* add_count;
-    // device-side row counts (or null): output rows from *m_limit on are not computed;
-    // contraction columns from *k_limit (rounded up to the slab) on are taken as zero
-    const uint32_t* m_limit; const uint32_t* k_limit;
+    // device-side counts (or null), one per batch limit_stride words apart (0: one for all):
+    // output rows from the m_limit on and output columns from the n_limit on are not computed
+    // (whole tiles: a tile that starts below the limit is computed in full); contraction columns
+    // from the k_limit (rounded up to the slab) on are taken as zero
+    const uint32_t* m_limit; const uint32_t* k_limit; const uint32_t* n_limit;
+    int limit_stride;
 };
 bool gemm_nt_bf16_ok(int M, int N, int K);
 int gemm_nt_bf16_ksplit(int M, int N, int K, int batches);  // partials needed: batches * ksplit * M * N floats
 void launch_gemm_nt_bf16(const GemmNT& g, hipStream_t stream);
 // in[z][rows, cols] (float32 or bfloat16) -> out_t[z][cols, rows] bfloat16 and, unless null,
 // out[z][rows, cols] bfloat16; rows % 64 == 0, cols % 64 == 0
-// With `row_limit` (device-side count) input rows from *row_limit (rounded up to 64) on are skipped.
+// Device-side limits (or null; one count per batch `stride` words apart): input rows from
+// row_base + count (rounded up to `pad`) on, input columns from the column count (rounded up to
+// `pad`) on are skipped.
+struct TransposeLimit {
+    const uint32_t* rows = nullptr;
+    const uint32_t* cols = nullptr;
+    int row_base = 0, stride = 0, pad = 64;
+};
 void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, int cols, int64_t ld_in,
                            int64_t in_batch, uint16_t* out_t, uint16_t* out, hipStream_t stream,
-                           const uint32_t* row_limit = nullptr);
+                           const TransposeLimit& limit = TransposeLimit());
 
 // Scores of every block: a-operand row (d,b) = entity row of contribution
 // d*B+b combined with relation crel[d*B+b]; b-operand row (d,t) = entity row of

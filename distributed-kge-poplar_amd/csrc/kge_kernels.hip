@@ -876,10 +876,12 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     const TileId tile = xcd_tile(g.N / GB_T, g.M / GB_T, g.batches * g.ksplit);
     const int zb = tile.z / g.ksplit, zs = tile.z - zb * g.ksplit;
     const int m0 = tile.y * GB_T, n0 = tile.x * GB_T;
-    if (g.m_limit && (uint32_t)m0 >= *g.m_limit) return;
+    const int lim = zb * g.limit_stride;
+    if (g.m_limit && (uint32_t)m0 >= g.m_limit[lim]) return;
+    if (g.n_limit && (uint32_t)n0 >= g.n_limit[lim]) return;
     int K = g.K / g.ksplit;
     if (g.k_limit) {  // this split's share of the live columns, in whole slabs
-        const int live = (int)((*g.k_limit + GB_K - 1) / GB_K) * GB_K;
+        const int live = (int)((g.k_limit[lim] + GB_K - 1) / GB_K) * GB_K;
         K = max(0, min(K, live - zs * K));
     }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1027,12 +1029,12 @@ void launch_gemm_nt_bf16(const GemmNT& g0, hipStream_t stream) {
 __global__ __launch_bounds__(256) void k_transpose_bf16(const void* __restrict__ in, int in_f32,
                                                         int rows, int cols, int64_t ld_in,
                                                         int64_t in_batch, uint16_t* __restrict__ out_t,
-                                                        uint16_t* __restrict__ out,
-                                                        const uint32_t* __restrict__ row_limit) {
+                                                        uint16_t* __restrict__ out, TransposeLimit limit) {
     // pitch of 66 elements: a column walk (the transposed read) steps 33 banks per row
     __shared__ __attribute__((aligned(4))) uint16_t tile[64][66];
     const int z = blockIdx.z, r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-    if (row_limit && (uint32_t)r0 >= *row_limit) return;
+    if (limit.rows && r0 >= limit.row_base + (int)((limit.rows[z * limit.stride] + limit.pad - 1) / limit.pad) * limit.pad) return;
+    if (limit.cols && c0 >= (int)((limit.cols[z * limit.stride] + limit.pad - 1) / limit.pad) * limit.pad) return;
     const int q = (threadIdx.x & 15) * 4, lr = threadIdx.x >> 4;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -1063,9 +1065,9 @@ __global__ __launch_bounds__(256) void k_transpose_bf16(const void* __restrict__
 
 void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, int cols, int64_t ld_in,
                            int64_t in_batch, uint16_t* out_t, uint16_t* out, hipStream_t stream,
-                           const uint32_t* row_limit) {
+                           const TransposeLimit& limit) {
     hipLaunchKernelGGL(k_transpose_bf16, dim3(cols / 64, rows / 64, batches), dim3(256), 0, stream, in,
-                       in_f32 ? 1 : 0, rows, cols, ld_in, in_batch, out_t, out, row_limit);
+                       in_f32 ? 1 : 0, rows, cols, ld_in, in_batch, out_t, out, limit);
 }
 
 // --------------------------------------------------------------------------
@@ -1576,10 +1578,14 @@ template <int NW, bool XF>
 __global__ __launch_bounds__(NW * 64) void k_reduce_chunks(ReduceArgs a0, ReduceArgs a1) {
     __shared__ __attribute__((aligned(16))) float part[NW - 1][256];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // two reductions share the launch: blocks [0, a0.max_chunks) serve the first
-    const bool second = (int)blockIdx.x >= a0.max_chunks;
+    // two reductions share the launch: blocks [0, a0.max_chunks * slabs) serve the first; a
+    // workgroup takes one slab of 256 columns of one chunk (rows wider than 256 columns: the
+    // slabs' chains of dependent loads run side by side instead of one after the other)
+    const int slabs = (max(a0.Dp, a1.Dp) + 255) / 256;
+    const int b = blockIdx.x / slabs, slab = blockIdx.x - b * slabs;
+    const bool second = b >= a0.max_chunks;
     const ReduceArgs& a = second ? a1 : a0;
-    const int q = second ? blockIdx.x - a0.max_chunks : blockIdx.x;
+    const int q = second ? b - a0.max_chunks : b;
     // fetched together with the chunk count (entries past it are stale but inside the arrays):
     // one round trip less in front of every chunk
     const uint32_t pos = a.chunk_pos[q], len = a.chunk_len[q];
@@ -1587,7 +1593,7 @@ __global__ __launch_bounds__(NW * 64) void k_reduce_chunks(ReduceArgs a0, Reduce
     const int Dp = a.Dp;
     if (Dp & 3) {  // unaligned rows (stand-alone scatter-add on arbitrary widths): wave 0 only
         if (wave == 0)
-            for (int k = lane; k < Dp; k += 64) {
+            for (int k = slab * 256 + lane; k < min(Dp, (slab + 1) * 256); k += 64) {
                 float acc = 0.f;
                 for (uint32_t j = 0; j < len; ++j)
                     acc += a.src.grad[(size_t)a.src.sorted_item[pos + j] * Dp + k];
@@ -1597,24 +1603,21 @@ __global__ __launch_bounds__(NW * 64) void k_reduce_chunks(ReduceArgs a0, Reduce
     }
     const uint32_t share = (len + NW - 1) / NW;
     const uint32_t w0 = min(len, wave * share), w1 = min(len, w0 + share);
-    for (int k0 = 0; k0 < Dp; k0 += 256) {
-        const int k = k0 + lane * 4;
-        // sixteen loads in flight: a wave's share of a 64-item chunk in one round (same order of
-        // additions as any other round size)
-        float4 acc = sum_contribs<16, XF>(a.src, pos + w0, w1 - w0, k, Dp, lane, k < Dp);
-        if (wave > 0) *reinterpret_cast<float4*>(&part[wave - 1][lane * 4]) = acc;
-        __syncthreads();
-        if (wave == 0 && k < Dp) {
+    const int k = slab * 256 + lane * 4;
+    // sixteen loads in flight: a wave's share of a 64-item chunk in one round (same order of
+    // additions as any other round size)
+    float4 acc = sum_contribs<16, XF>(a.src, pos + w0, w1 - w0, k, Dp, lane, k < Dp);
+    if (wave > 0) *reinterpret_cast<float4*>(&part[wave - 1][lane * 4]) = acc;
+    __syncthreads();
+    if (wave == 0 && k < Dp) {
 #pragma unroll
-            for (int w = 0; w < NW - 1; ++w) acc = f4add(acc, *reinterpret_cast<const float4*>(&part[w][lane * 4]));
-            *reinterpret_cast<float4*>(a.partial + (size_t)q * Dp + k) = acc;
-        }
-        __syncthreads();
+        for (int w = 0; w < NW - 1; ++w) acc = f4add(acc, *reinterpret_cast<const float4*>(&part[w][lane * 4]));
+        *reinterpret_cast<float4*>(a.partial + (size_t)q * Dp + k) = acc;
     }
 }
 
 static void launch_reduce_kernel(const ReduceArgs& a0, const ReduceArgs& a1, hipStream_t stream) {
-    const int n = a0.max_chunks + a1.max_chunks;
+    const int n = (a0.max_chunks + a1.max_chunks) * ((std::max(a0.Dp, a1.Dp) + 255) / 256);
     if (n == 0) return;
     const bool xf = (a0.max_chunks && a0.src.transform >= 3) || (a1.max_chunks && a1.src.transform >= 3);
     if (std::max(a0.chunk, a1.chunk) > 64) {
@@ -1655,11 +1658,14 @@ DEVINL void adam4(float4& p, float4& m, float4& v, float4 g, const AdamArgs& a, 
 template <bool MF32, bool XF>
 __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
     const int lane = threadIdx.x & 63;
-    // two tables share the launch: blocks [0, ceil(a0.max_rows / 4)) serve the first
-    const int blocks0 = (a0.max_rows + 3) / 4;
+    // two tables share the launch: blocks [0, ceil(a0.max_rows * slabs / 4)) serve the first; a
+    // wave takes one slab of 256 columns of one row
+    const int slabs = (max(a0.Dp, a1.Dp) + 255) / 256;
+    const int blocks0 = (a0.max_rows * slabs + 3) / 4;
     const bool second = (int)blockIdx.x >= blocks0;
     const AdamArgs& a = second ? a1 : a0;
-    const int u = (second ? blockIdx.x - blocks0 : blockIdx.x) * 4 + (threadIdx.x >> 6);
+    const int g = (second ? blockIdx.x - blocks0 : blockIdx.x) * 4 + (threadIdx.x >> 6);
+    const int u = g / slabs, slab = g - u * slabs;
     // the row's plan entries are fetched together with the row count (entries past it are stale
     // but inside the arrays): one round trip less in front of every row
     const int uc = min(u, a.max_rows - 1);
@@ -1675,13 +1681,13 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
     char* prow = a.p_base + (int64_t)key * a.pitch;
     char* mrow = a.m_base + (int64_t)key * a.pitch;
     char* vrow = a.v_base + (int64_t)key * a.pitch;
-    for (int k0 = 0; k0 < Dp; k0 += 256) {
-        const int k = k0 + lane * 4;
+    {
+        const int k = slab * 256 + lane * 4;
         const bool active = k < Dp;
         float4 g = make_float4(0, 0, 0, 0);
         if (!a.grad_direct && q1 == q0 && n_real)  // wave-uniform: all lanes take part in the shuffles
             g = sum_contribs<8, XF>(a.src, pos, n_real, k, Dp, lane, active);
-        if (!active) continue;
+        if (!active) return;
         float4 p = load4(prow, k, a.p_etype);
         float4 m, v;
         if constexpr (MF32) {
@@ -1709,7 +1715,7 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
             if (a.grad_out_add) go = f4add(go, *reinterpret_cast<const float4*>(a.grad_out_add + (size_t)u * Dp + k));
             *reinterpret_cast<float4*>(a.grad_out + (size_t)u * Dp + k) = go;
         }
-        if (a.no_update) continue;
+        if (a.no_update) return;
         if (a.grad_add) g = f4add(g, *reinterpret_cast<const float4*>(a.grad_add + (size_t)u * Dp + k));
         adam4(p, m, v, g, a, alpha);
         store4(prow, k, a.p_etype, p);
@@ -1808,10 +1814,12 @@ __global__ __launch_bounds__(kHotWaves * 64) void k_adam_rows_hot(AdamArgs a0, H
         return;
     }
     b -= hot0 + hot1;
-    const int blocks0 = (a0.max_rows + kHotWaves - 1) / kHotWaves;
+    const int slabs = (max(a0.Dp, a1.Dp) + 255) / 256;   // a wave takes one slab of 256 columns of one row
+    const int blocks0 = (a0.max_rows * slabs + kHotWaves - 1) / kHotWaves;
     const bool second = b >= blocks0;
     const AdamArgs& a = second ? a1 : a0;
-    const int u = (second ? b - blocks0 : b) * kHotWaves + wave;
+    const int g = (second ? b - blocks0 : b) * kHotWaves + wave;
+    const int u = g / slabs, slab = g - u * slabs;
     const int uc = min(u, a.max_rows - 1);
     const uint32_t key = a.uniq_key[uc];
     const uint32_t q0 = a.chunk_off[uc], q1 = a.chunk_off[uc + 1];
@@ -1822,13 +1830,13 @@ __global__ __launch_bounds__(kHotWaves * 64) void k_adam_rows_hot(AdamArgs a0, H
     char* prow = a.p_base + (int64_t)key * a.pitch;
     char* mrow = a.m_base + (int64_t)key * a.pitch;
     char* vrow = a.v_base + (int64_t)key * a.pitch;
-    for (int k0 = 0; k0 < Dp; k0 += 256) {
-        const int k = k0 + lane * 4;
+    {
+        const int k = slab * 256 + lane * 4;
         const bool active = k < Dp;
         float4 g = make_float4(0, 0, 0, 0);
         if (n_real)  // wave-uniform: all lanes take part in the shuffles
             g = sum_contribs<8, false>(a.src, pos, n_real, k, Dp, lane, active);
-        if (!active) continue;
+        if (!active) return;
         float4 p = load4(prow, k, a.p_etype);
         float4 m, v;
         if constexpr (MF32) {
@@ -1843,7 +1851,7 @@ __global__ __launch_bounds__(kHotWaves * 64) void k_adam_rows_hot(AdamArgs a0, H
             if (a.grad_out_add) go = f4add(go, *reinterpret_cast<const float4*>(a.grad_out_add + (size_t)u * Dp + k));
             *reinterpret_cast<float4*>(a.grad_out + (size_t)u * Dp + k) = go;
         }
-        if (a.no_update) continue;
+        if (a.no_update) return;
         if (a.grad_add) g = f4add(g, *reinterpret_cast<const float4*>(a.grad_add + (size_t)u * Dp + k));
         adam4(p, m, v, g, a, alpha);
         store4(prow, k, a.p_etype, p);
@@ -1861,7 +1869,8 @@ void launch_adam_rows_hot2(const AdamArgs& a0, const HotRows& h0, const AdamArgs
                            hipStream_t stream) {
     const int hot = ((a0.Dp + kHotColumns - 1) / kHotColumns) * h0.max_hot +
                     ((a1.Dp + kHotColumns - 1) / kHotColumns) * h1.max_hot;
-    const dim3 grid(hot + (a0.max_rows + kHotWaves - 1) / kHotWaves + (a1.max_rows + kHotWaves - 1) / kHotWaves);
+    const int slabs = (std::max(a0.Dp, a1.Dp) + 255) / 256;
+    const dim3 grid(hot + (a0.max_rows * slabs + kHotWaves - 1) / kHotWaves + (a1.max_rows * slabs + kHotWaves - 1) / kHotWaves);
     if (grid.x == 0) return;
     const bool f32 = (a0.max_rows == 0 || a0.m_etype == ET_F32) && (a1.max_rows == 0 || a1.m_etype == ET_F32);
     if (f32) hipLaunchKernelGGL((k_adam_rows_hot<true>), grid, dim3(kHotWaves * 64), 0, stream, a0, h0, a1, h1);
@@ -1869,7 +1878,8 @@ void launch_adam_rows_hot2(const AdamArgs& a0, const HotRows& h0, const AdamArgs
 }
 
 static void launch_adam_kernel(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream) {
-    const dim3 grid((a0.max_rows + 3) / 4 + (a1.max_rows + 3) / 4);
+    const int slabs = (std::max(a0.Dp, a1.Dp) + 255) / 256;
+    const dim3 grid((a0.max_rows * slabs + 3) / 4 + (a1.max_rows * slabs + 3) / 4);
     if (grid.x == 0) return;
     const bool f32 = (a0.max_rows == 0 || a0.m_etype == ET_F32) && (a1.max_rows == 0 || a1.m_etype == ET_F32);
     const bool xf = (a0.max_rows && a0.src.transform >= 3) || (a1.max_rows && a1.src.transform >= 3);
@@ -2158,8 +2168,10 @@ void launch_proj_grad(const FeatureArgs& a, const float* grad_rows, float* gproj
         // rows past the distinct count are zero in the features and finite in grad_rows
         // (the contraction stops at the distinct count, so neither those rows nor their
         // transposes are touched)
-        launch_transpose_bf16(a.feat16, false, 1, a.max_rows, a.Fp, a.Fp, 0, a.featT16, nullptr, stream, a.counts);
-        launch_transpose_bf16(grad_rows, true, 1, a.max_rows, a.Dp, a.Dp, 0, a.gT16, nullptr, stream, a.counts);
+        TransposeLimit live_rows;   // rows past the step's distinct count are skipped
+        live_rows.rows = a.counts;
+        launch_transpose_bf16(a.feat16, false, 1, a.max_rows, a.Fp, a.Fp, 0, a.featT16, nullptr, stream, live_rows);
+        launch_transpose_bf16(grad_rows, true, 1, a.max_rows, a.Dp, a.Dp, 0, a.gT16, nullptr, stream, live_rows);
         GemmNT g = {};
         g.A = a.featT16; g.lda = a.max_rows; g.Bt = a.gT16; g.ldb = a.max_rows; g.C = gproj; g.ldc = a.Dp;
         g.M = a.Fp; g.N = a.Dp; g.K = a.max_rows; g.batches = 1;
