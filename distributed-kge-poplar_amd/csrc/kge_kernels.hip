@@ -1655,8 +1655,12 @@ DEVINL void adam4(float4& p, float4& m, float4& v, float4 g, const AdamArgs& a, 
 // One wave per distinct row: gather its gradient (directly from its few
 // contributions, or from its chunk partials), Adam, write the row back.
 // MF32: both moments float32 (the usual layout), accessed as plain 16-byte words
+// A wave's life is a chain of dependent loads (plan entry, item list, contribution rows and the
+// row itself, stores): what the kernel gets through is the number of resident waves over that
+// chain's length, so the plain form is compiled for eight waves per SIMD (four contribution
+// loads in flight instead of eight buy the registers).
 template <bool MF32, bool XF>
-__global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
+DEVINL void adam_rows_body(const AdamArgs& a0, const AdamArgs& a1) {
     const int lane = threadIdx.x & 63;
     // two tables share the launch: blocks [0, ceil(a0.max_rows * slabs / 4)) serve the first; a
     // wave takes one slab of 256 columns of one row
@@ -1686,7 +1690,7 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
         const bool active = k < Dp;
         float4 g = make_float4(0, 0, 0, 0);
         if (!a.grad_direct && q1 == q0 && n_real)  // wave-uniform: all lanes take part in the shuffles
-            g = sum_contribs<8, XF>(a.src, pos, n_real, k, Dp, lane, active);
+            g = sum_contribs<XF ? 8 : 4, XF>(a.src, pos, n_real, k, Dp, lane, active);
         if (!active) return;
         float4 p = load4(prow, k, a.p_etype);
         float4 m, v;
@@ -1700,14 +1704,15 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
         if (a.grad_direct) {
             g = *reinterpret_cast<const float4*>(a.grad_direct + (size_t)u * Dp + k);
         } else if (q1 > q0) {
-            for (uint32_t q = q0; q < q1; q += 8) {
-                float4 t[8];
+            constexpr int NP = XF ? 8 : 4;  // partial sums in flight
+            for (uint32_t q = q0; q < q1; q += NP) {
+                float4 t[NP];
 #pragma unroll
-                for (int x = 0; x < 8; ++x)
+                for (int x = 0; x < NP; ++x)
                     t[x] = (q + x < q1) ? *reinterpret_cast<const float4*>(a.partial + (size_t)(q + x) * Dp + k)
                                         : make_float4(0, 0, 0, 0);
 #pragma unroll
-                for (int x = 0; x < 8; ++x) g = f4add(g, t[x]);
+                for (int x = 0; x < NP; ++x) g = f4add(g, t[x]);
             }
         }
         if (a.grad_out) {
@@ -1729,6 +1734,15 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
     }
 }
 
+template <bool MF32>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
+    adam_rows_body<MF32, false>(a0, a1);
+}
+template <bool MF32>  // with the ComplEx / RotatE transforms of the contributions compiled in
+__global__ __launch_bounds__(256) void k_adam_rows_xf(AdamArgs a0, AdamArgs a1) {
+    adam_rows_body<MF32, true>(a0, a1);
+}
+
 // One launch for both tables without a first-level reduction before it.
 //   blocks [0, NS0 * max_hot0), [.., + NS1 * max_hot1): hot rows, one workgroup per (row, 32 columns).
 //     Lane = (slot, column group): eight contributions per load instruction (128 bytes of each),
@@ -1739,12 +1753,14 @@ __global__ __launch_bounds__(256) void k_adam_rows(AdamArgs a0, AdamArgs a1) {
 // columns per hot-row workgroup: 32 (128 bytes of every contribution per load; 16 and 8 columns
 // measured slower: the same rows are then fetched by two and four times as many workgroups)
 constexpr int kHotColumns = 32;
-// loads in flight per lane: 16 (the update of a 1M-row table's step measured 22.4 / 20.5 / 20.8 /
-// 23.6 us with 8 / 16 / 24 / 32; the registers of the larger ones cost the other rows' waves
-// their residency); four waves per workgroup (2, 8 and 16 measured slower)
-constexpr int kHotLoads = 16, kHotWaves = 4;
+// loads in flight per lane: 8, and the kernel compiled for eight waves per SIMD (56 registers): the
+// ordinary rows, one wave each, are bound by resident waves over the length of a wave's chain of
+// dependent loads (22.8M-row workload 38.9 -> 33.8 us, 91.2M-row 32.2 -> 26.3 us against 16 loads
+// and five waves; 4 and 16 loads at eight waves measured the same within a microsecond);
+// four waves per workgroup (2, 8 and 16 measured slower)
+constexpr int kHotLoads = 8, kHotWaves = 4;
 template <bool MF32>
-__global__ __launch_bounds__(kHotWaves * 64) void k_adam_rows_hot(AdamArgs a0, HotRows h0, AdamArgs a1, HotRows h1) {
+__global__ __launch_bounds__(kHotWaves * 64) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_adam_rows_hot(AdamArgs a0, HotRows h0, AdamArgs a1, HotRows h1) {
     constexpr int HC = kHotColumns, HS = 64 / (HC / 4);  // columns per workgroup, slots per wave
     __shared__ __attribute__((aligned(16))) float part[kHotWaves - 1][HC];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1835,7 +1851,7 @@ __global__ __launch_bounds__(kHotWaves * 64) void k_adam_rows_hot(AdamArgs a0, H
         const bool active = k < Dp;
         float4 g = make_float4(0, 0, 0, 0);
         if (n_real)  // wave-uniform: all lanes take part in the shuffles
-            g = sum_contribs<8, false>(a.src, pos, n_real, k, Dp, lane, active);
+            g = sum_contribs<4, false>(a.src, pos, n_real, k, Dp, lane, active);
         if (!active) return;
         float4 p = load4(prow, k, a.p_etype);
         float4 m, v;
@@ -1883,10 +1899,10 @@ static void launch_adam_kernel(const AdamArgs& a0, const AdamArgs& a1, hipStream
     if (grid.x == 0) return;
     const bool f32 = (a0.max_rows == 0 || a0.m_etype == ET_F32) && (a1.max_rows == 0 || a1.m_etype == ET_F32);
     const bool xf = (a0.max_rows && a0.src.transform >= 3) || (a1.max_rows && a1.src.transform >= 3);
-    if (f32 && !xf) hipLaunchKernelGGL((k_adam_rows<true, false>), grid, dim3(256), 0, stream, a0, a1);
-    else if (f32) hipLaunchKernelGGL((k_adam_rows<true, true>), grid, dim3(256), 0, stream, a0, a1);
-    else if (!xf) hipLaunchKernelGGL((k_adam_rows<false, false>), grid, dim3(256), 0, stream, a0, a1);
-    else hipLaunchKernelGGL((k_adam_rows<false, true>), grid, dim3(256), 0, stream, a0, a1);
+    if (f32 && !xf) hipLaunchKernelGGL((k_adam_rows<true>), grid, dim3(256), 0, stream, a0, a1);
+    else if (f32) hipLaunchKernelGGL((k_adam_rows_xf<true>), grid, dim3(256), 0, stream, a0, a1);
+    else if (!xf) hipLaunchKernelGGL((k_adam_rows<false>), grid, dim3(256), 0, stream, a0, a1);
+    else hipLaunchKernelGGL((k_adam_rows_xf<false>), grid, dim3(256), 0, stream, a0, a1);
 }
 void launch_adam_rows(const AdamArgs& a, hipStream_t stream) {
     AdamArgs none = a;
