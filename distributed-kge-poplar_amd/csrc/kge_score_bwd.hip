@@ -597,16 +597,32 @@ constexpr int L1P_WAVES = 16;
 constexpr int L1P_MAX_T = 512;  // tails per block at most (32 per wave)
 
 // the work of one wave with exactly TW tails (TW a multiple of 4): straight-line code over
-// its tails, their values and sums in registers
+// its tails, their values and sums in registers.
+// signum(a - b) with signum(0) = 0 (poplar_extensions l1distance.codelet.cpp:76-79) from
+// instructions of the fast class only (subtract, fused multiply-add): the difference times 2^126
+// plus one half, clamped to [0, 1] by the instruction's own output modifier, is p = 1 / 0.5 / 0
+// for a positive / zero / negative difference (any normal float times 2^126 is at least 1 in
+// magnitude), and signum = 2 p - 1.  The inner loop accumulates c p (four instructions per pair
+// and column: subtract, clamped fma, one fma for either side's sum) and the linear part is taken
+// off in small pieces, before the sums grow and rounding with them:
+//   tails   after every chunk of 8 heads, half the chunk's column sums: the running value is
+//           sum c (p - 1/2) = (1/2) sum c signum;
+//   heads   each wave's partial 2 sum_j c p minus the sum of the coefficients of its own TW
+//           columns, before the 16 waves' values are added.
+// The column and row-part sums of a chunk come from the coefficient rows staged in LDS, by waves
+// 8 .. 15 while waves 0 .. 7 add the head partials of the chunk before.
 template <int TW>
 DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restrict__ b_rows,
                          const float* __restrict__ cblk, float* __restrict__ grad_a, float* __restrict__ grad_b,
-                         int B, int T, int Dp, int t0, int t4, int w, int lane,
-                         float (*part)[L1P_WAVES][L1P_CB][64], float (*cs)[L1P_CB][L1P_MAX_T]) {
-    const int tid = threadIdx.x;
+                         int B, int T, int Dp, int t0, int t_live, int w, int lane,
+                         float (*part)[L1P_WAVES][L1P_CB][64], float (*cs)[L1P_CB][L1P_MAX_T],
+                         float (*col_half)[L1P_MAX_T], float (*row_part)[L1P_CB][L1P_WAVES]) {
+    const int tid = threadIdx.x, t4 = t_live / 4;
     // staging: thread -> (head, four columns) of a chunk's coefficient rows
     const bool stager = tid < L1P_CB * t4;
     const int s_head = tid / t4, s_col = (tid - s_head * t4) * 4;
+    // linear parts: thread 512 + t -> column t; threads 512 .. 639 -> (head, wave)
+    const int u = tid - 512;
     float4 c_next = make_float4(0.f, 0.f, 0.f, 0.f);
     if (stager) {
         c_next = *reinterpret_cast<const float4*>(cblk + (size_t)s_head * T + s_col);
@@ -622,6 +638,28 @@ DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restri
     for (int b0 = 0, buf = 0; b0 < B; b0 += L1P_CB, buf ^= 1) {
         const bool more = b0 + L1P_CB < B;
         if (stager && more) c_next = *reinterpret_cast<const float4*>(cblk + (size_t)(b0 + L1P_CB + s_head) * T + s_col);
+        if (b0 > 0) {
+#pragma unroll
+            for (int j4 = 0; j4 < TW; j4 += 4) {
+                const float4 h4 = *reinterpret_cast<const float4*>(&col_half[buf ^ 1][t0 + j4]);
+                gt[j4] -= h4.x, gt[j4 + 1] -= h4.y, gt[j4 + 2] -= h4.z, gt[j4 + 3] -= h4.w;
+            }
+        }
+        if (u >= 0) {
+            if (u < t_live) {
+                float sum = 0.f;
+#pragma unroll
+                for (int h = 0; h < L1P_CB; ++h) sum += cs[buf][h][u];
+                col_half[buf][u] = 0.5f * sum;
+            }
+            if (u < L1P_CB * L1P_WAVES) {
+                const int h = u / L1P_WAVES, v = u % L1P_WAVES;
+                float sum = 0.f;
+#pragma unroll
+                for (int j = 0; j < TW; ++j) sum += cs[buf][h][v * TW + j];
+                row_part[buf][h][v] = sum;
+            }
+        }
         float a_next = a_rows[(size_t)b0 * Dp];
 #pragma unroll 1
         for (int bi = 0; bi < L1P_CB; ++bi) {
@@ -635,16 +673,9 @@ DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restri
                 const float cv[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
                 for (int x = 0; x < 4; ++x) {
-                    // signum(a - b) with signum(0) = 0 (poplar_extensions l1distance.codelet.cpp:76-79)
-                    // from instructions of the fast class only (subtract, fused multiply-add):
-                    // the difference times 2^126 plus one half, clamped to [0, 1] by the
-                    // instruction's own output modifier, is 1 / 0.5 / 0 for a positive / zero /
-                    // negative difference (any normal float times 2^126 is at least 1 in
-                    // magnitude); twice that minus one is the sign.
-                    const float half_step = __builtin_amdgcn_fmed3f(fmaf(a - bt[j4 + x], 0x1p126f, 0.5f), 0.f, 1.f);
-                    const float sg = fmaf(half_step, 2.f, -1.f);
-                    gp = fmaf(cv[x], sg, gp);
-                    gt[j4 + x] = fmaf(-cv[x], sg, gt[j4 + x]);
+                    const float p = __builtin_amdgcn_fmed3f(fmaf(a - bt[j4 + x], 0x1p126f, 0.5f), 0.f, 1.f);
+                    gp = fmaf(cv[x], p, gp);
+                    gt[j4 + x] = fmaf(cv[x], p, gt[j4 + x]);
                 }
             }
             part[buf][w][bi][lane] = gp;
@@ -655,12 +686,13 @@ DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restri
         if (w < L1P_CB) {
             float sum = 0.f;
 #pragma unroll
-            for (int v = 0; v < L1P_WAVES; ++v) sum += part[buf][v][w][lane];
+            for (int v = 0; v < L1P_WAVES; ++v) sum += fmaf(2.f, part[buf][v][w][lane], -row_part[buf][w][v]);
             grad_a[(size_t)(b0 + w) * Dp] = sum;
         }
     }
+    const int last = ((B / L1P_CB) - 1) & 1;
 #pragma unroll
-    for (int j = 0; j < TW; ++j) grad_b[(size_t)j * Dp] = gt[j];
+    for (int j = 0; j < TW; ++j) grad_b[(size_t)j * Dp] = -2.f * (gt[j] - col_half[last][t0 + j]);
 }
 
 __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restrict__ operands,
@@ -668,8 +700,14 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
                                                             float* __restrict__ grad, int B, int T,
                                                             int Dp, int a_c0, int b_c0,
                                                             const uint32_t* __restrict__ tcount, int tpad) {
-    __shared__ float part[2][L1P_WAVES][L1P_CB][64];
-    __shared__ __attribute__((aligned(16))) float cs[2][L1P_CB][L1P_MAX_T];
+    // the coefficient rows first: their reads in the inner loop then carry the whole address
+    // offset in the instruction
+    __shared__ __attribute__((aligned(16))) struct {
+        float cs[2][L1P_CB][L1P_MAX_T];
+        float col_half[2][L1P_MAX_T];
+        float row_part[2][L1P_CB][L1P_WAVES];
+        float part[2][L1P_WAVES][L1P_CB][64];
+    } lds;
     const TileId tile = xcd_tile(Dp / 64, 1, (int)gridDim.x / (Dp / 64));
     const int d = tile.z, lane = threadIdx.x & 63, k = tile.x * 64 + lane;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -682,7 +720,7 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
     float* grad_a = grad + (size_t)(a_c0 + d * B) * Dp + k;
     float* grad_b = grad + (size_t)(b_c0 + d * T + t0) * Dp + k;
 #define KGE_L1P(TW_) \
-    case TW_: l1_pair_wave<TW_>(a_rows, b_rows, cblk, grad_a, grad_b, B, T, Dp, t0, t_live / 4, w, lane, part, cs); break;
+    case TW_: l1_pair_wave<TW_>(a_rows, b_rows, cblk, grad_a, grad_b, B, T, Dp, t0, t_live, w, lane, lds.part, lds.cs, lds.col_half, lds.row_part); break;
     switch (tw) {  // one of eight copies of the loop, chosen per block
         KGE_L1P(4) KGE_L1P(8) KGE_L1P(12) KGE_L1P(16) KGE_L1P(20) KGE_L1P(24) KGE_L1P(28) KGE_L1P(32)
     }
