@@ -542,6 +542,244 @@ __global__ __launch_bounds__(NW * 64) void k_score_bwd_mfma_both(BwdParams p) {
     }
 }
 
+// --------------------------------------------------------------------------
+// The same sums from bfloat16 matrix instructions on three-piece operands (mfma_split6: six
+// v_mfma_f32_32x32x16_bf16 per sixteen rows of `other` in place of eight
+// v_mfma_f32_32x32x2_f32, float32 accuracy).  The sum runs over the rows of `other`, so both
+// operand tiles are laid down in LDS with that index innermost, as pieces:
+//   Ap[piece][self row][32 j]    Bp[piece][embedding column][32 j]
+// A thread stages eight consecutive j of one coefficient row (head side: two 16-byte loads along
+// the row; tail side: eight 4-byte loads down a column of the coefficient matrix, consecutive
+// lanes on consecutive columns) and four consecutive j of one embedding column of `other`.
+// A row's four 16-byte chunks sit at position chunk ^ ((row / 4) % 4), which spreads sixteen
+// consecutive rows' accesses to one chunk over all banks.
+// Workgroup tile 128 (self rows) x 64 (embedding columns), eight waves as 4 x 2, one 32 x 32
+// accumulator each; tile-aligned shapes and dense float32 operands only.
+
+constexpr int BS_TI = 128, BS_TK = 64, BS_KJ = 32;
+constexpr int kBwdSplitSmemBytes = 2 * 3 * BS_TI * BS_KJ * 2 + 2 * 3 * BS_TK * BS_KJ * 2 + 4 * BS_TI * 4 + BS_TI * 4;
+
+template <int DIST, int SIDE_B>
+DEVINL void bwd_split_body(const BwdParams& p, const int d, const int tile_x, const int tile_y, char* smem) {
+    typedef uint16_t ATile[3][BS_TI][BS_KJ];
+    typedef uint16_t BTile[3][BS_TK][BS_KJ];
+    ATile* Ap = reinterpret_cast<ATile*>(smem);
+    BTile* Bp = reinterpret_cast<BTile*>(smem + 2 * sizeof(ATile));
+    float* part = reinterpret_cast<float*>(smem + 2 * sizeof(ATile) + 2 * sizeof(BTile));  // [4][128]
+    float* csum_s = part + 4 * BS_TI;
+    const int i0 = tile_y * BS_TI, kt0 = tile_x * BS_TK;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hl = lane >> 5, cl = lane & 31;
+    const int wi = (wave >> 1) * 32, wk = (wave & 1) * 32;
+    const int B = p.B, T = p.T, Dp = p.Dp;
+    const int t_live = tail_limit(p.tcount, d, T, p.tpad);  // merged tails: the block's live columns
+    const int n_self = SIDE_B ? T : B, n_other = SIDE_B ? B : t_live;
+    if (i0 >= (SIDE_B ? t_live : n_self)) return;  // the grid is sized for the longer side
+    const int grad_c0 = SIDE_B ? p.b_c0 : p.a_c0;
+    const RowSource& self_src = SIDE_B ? p.ent_b : p.ent_a;
+    const RowSource& other_src = SIDE_B ? p.ent_a : p.ent_b;
+    const char* const self_rows = self_src.base + (int64_t)(SIDE_B ? p.b_c0 + d * T : p.a_c0 + d * B) * self_src.pitch;
+    const char* const other_rows = other_src.base + (int64_t)(SIDE_B ? p.a_c0 + d * B : p.b_c0 + d * T) * other_src.pitch;
+    const int64_t opitch = other_src.pitch;
+    const float* const coef = p.coef + (size_t)d * B * T;
+    const int kcol = kt0 + wk + cl;
+
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    // L2: this lane's `self` values, in accumulator layout (fetched where they are used: held
+    // through the loop they would cost the registers of a fourth wave per SIMD)
+    auto load_self = [&](float sv[16]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i = i0 + wi + 8 * (r >> 2) + 4 * hl + (r & 3);
+            sv[r] = reinterpret_cast<const float*>(self_rows + (int64_t)i * self_src.pitch)[kcol];
+        }
+    };
+    // staging: coefficient row a_row, its j-chunk a_kg (8 values); column b_n of `other`, rows
+    // 8 b_kg + 4 b_half .. + 3 of the slab.  What is the same for a whole wave stays in scalar
+    // registers, so that the loads take a scalar base and one 32-bit lane offset.
+    const int a_row = SIDE_B ? (wave & 1) * 64 + lane : wave * 16 + (lane >> 2), a_kg = SIDE_B ? (wave >> 1) : (lane & 3);
+    const int b_n = lane, b_kg = wave & 3, b_half = wave >> 2;
+    const int a_col = (a_kg ^ ((a_row >> 2) & 3)) << 3;
+    const int b_col = ((b_kg ^ ((b_n >> 2) & 3)) << 3) + 4 * b_half;
+    const uint32_t a_off = SIDE_B ? (uint32_t)a_row : (uint32_t)(a_row * T + 8 * a_kg);
+    // near-identical-pair flags of the (self sub-tile, slab of `other`) blocks (L2: the forward
+    // pass wrote them for the columns it visited)
+    const int MT = B >> 5, NTL = T >> 5;
+    const uint32_t* const nflag = DIST == DIST_L2 ? p.nearflag + (size_t)d * MT * NTL : nullptr;
+    auto flag_of = [&](int i_tile, int j_tile) -> uint32_t {
+        if constexpr (DIST != DIST_L2) return 0u;
+        const int mt = SIDE_B ? j_tile : i_tile, nt = SIDE_B ? i_tile : j_tile;
+        const uint32_t f = nflag[(size_t)mt * NTL + min(nt, NTL - 1)];
+        return 32 * nt < t_live ? f : 0u;  // no flags for columns the forward pass did not visit
+    };
+    float cs_acc = 0.f;
+    // a slab's operand loads take a round trip to the memory-side cache however little work a
+    // slab is: two register sets, each filled two slabs ahead of its use
+    struct Slab {
+        floatx4 a[2], b;
+        uint32_t nf_row;
+    } set0, set1;
+    auto prefetch = [&](Slab& s, int j_first) __attribute__((always_inline)) {
+        // (taken through a scalar register afresh: the row addresses are then formed by scalar
+        // instructions every slab, not carried along as one 64-bit vector pointer per row)
+        const int j0 = __builtin_amdgcn_readfirstlane(j_first);
+        s.nf_row = flag_of((i0 + a_row) >> 5, j0 >> 5);
+        if (!SIDE_B) {
+            const float* src = coef + (size_t)i0 * T + j0;
+            s.a[0] = *reinterpret_cast<const floatx4*>(src + a_off);
+            s.a[1] = *reinterpret_cast<const floatx4*>(src + a_off + 4);
+        } else {
+#pragma unroll
+            for (int x = 0; x < 8; ++x) s.a[x >> 2][x & 3] = (coef + (size_t)(j0 + 8 * a_kg + x) * T + i0)[a_off];
+        }
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            s.b[x] = (reinterpret_cast<const float*>(other_rows + (int64_t)(j0 + 8 * b_kg + 4 * b_half + x) * opitch) + kt0)[b_n];
+    };
+    // writes a prefetched slab into tile copy `nb` as pieces and adds the coefficients to the row
+    // sums.  `keep` = 0 for a slab past the end and where some pair of the row's 32 x 32 block is
+    // nearly identical: such a block's coefficients go into the tile as zeros (its products
+    // vanish, its rows' sums leave it out) and it is taken in the direct form after the loop.
+    auto stage = [&](const Slab& s, int nb, float live) __attribute__((always_inline)) {
+        const float keep = s.nf_row == 0u ? live : 0.f;
+        const floatx4 a0 = s.a[0] * keep, a1 = s.a[1] * keep;
+        uint2 lo[3], hi[3];
+        split4_bf16(a0, lo);
+        split4_bf16(a1, hi);
+#pragma unroll
+        for (int q = 0; q < 3; ++q)
+            *reinterpret_cast<uint4*>(&Ap[nb][q][a_row][a_col]) = make_uint4(lo[q].x, lo[q].y, hi[q].x, hi[q].y);
+        if (DIST == DIST_L2) {
+            const floatx4 s4 = a0 + a1;
+            cs_acc += (s4.x + s4.y) + (s4.z + s4.w);
+        }
+        uint2 pb[3];
+        split4_bf16(s.b, pb);
+#pragma unroll
+        for (int q = 0; q < 3; ++q) *reinterpret_cast<uint2*>(&Bp[nb][q][b_n][b_col]) = pb[q];
+    };
+    const int j_last = n_other - BS_KJ;  // loads past the end fetch the last slab again
+    // one slab: the matrix work on tile copy `buf`, the next slab (register set `s`) into the
+    // other copy (last read one slab ago, before the barrier), and `s` filled again
+    auto step = [&](Slab& s, int jbase, int buf) __attribute__((always_inline)) {
+        // two steps of sixteen rows of `other`; a lane supplies rows 8 * (lane / 32) .. + 7 of a
+        // step, for its self row and for its embedding column
+        floatx4 fa[2][3], fb[2][3];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int chunk = 2 * ks + hl;
+#pragma unroll
+            for (int q = 0; q < 3; ++q) {
+                const int ra = wi + cl, rb = wk + cl;
+                fa[ks][q] = *reinterpret_cast<const floatx4*>(&Ap[buf][q][ra][(chunk ^ ((ra >> 2) & 3)) << 3]);
+                fb[ks][q] = *reinterpret_cast<const floatx4*>(&Bp[buf][q][rb][(chunk ^ ((rb >> 2) & 3)) << 3]);
+            }
+        }
+        stage(s, buf ^ 1, jbase + BS_KJ < n_other ? 1.f : 0.f);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) acc = mfma_split6(fa[ks], fb[ks], acc);
+        // the order asked of the scheduler: the first step's LDS reads, then one matrix
+        // instruction (each depends on the one before it), a share of the vector work and an LDS
+        // access, in turn
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+        for (int i = 0; i < 12; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+            if (i < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+        prefetch(s, min(jbase + 3 * BS_KJ, j_last));
+        __syncthreads();
+    };
+    prefetch(set0, 0);
+    stage(set0, 0, 1.f);
+    prefetch(set0, min(BS_KJ, j_last));
+    prefetch(set1, min(2 * BS_KJ, j_last));
+    __syncthreads();
+    for (int jbase = 0; jbase < n_other; jbase += 2 * BS_KJ) {  // n_other % 64 == 0
+        step(set0, jbase, 0);
+        step(set1, jbase + BS_KJ, 1);
+    }
+    if (DIST == DIST_L2) {
+        // slabs in which some pair of this wave's sub-tile is nearly identical: c * (self - other)
+        // directly, as the reference codelet does, from the operands in memory (acc holds the
+        // negated sum).  Rare, and out of the loop above so that its registers stay out of it.
+        for (int jbase = 0; jbase < n_other; jbase += BS_KJ) {
+            if (flag_of((i0 + wi) >> 5, jbase >> 5) == 0u) continue;
+            float sv[16];
+            load_self(sv);
+            for (int jj = jbase; jj < jbase + BS_KJ; ++jj) {
+                const float o = reinterpret_cast<const float*>(other_rows + (int64_t)jj * opitch)[kcol];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int i = i0 + wi + 8 * (r >> 2) + 4 * hl + (r & 3);
+                    const float cc = SIDE_B ? coef[(size_t)jj * T + i] : coef[(size_t)i * T + jj];
+                    acc[r] = fmaf(-cc, sv[r] - o, acc[r]);
+                }
+            }
+        }
+    }
+    if (DIST == DIST_L2) {
+        // the four partial sums of a row, added in a fixed order
+        part[a_kg * BS_TI + a_row] = cs_acc;
+        __syncthreads();
+        if (tid < BS_TI) csum_s[tid] = ((part[tid] + part[BS_TI + tid]) + part[2 * BS_TI + tid]) + part[3 * BS_TI + tid];
+        __syncthreads();
+    }
+    float* __restrict__ const gout = p.grad;
+    if (DIST == DIST_DOT && p.add_base) {
+        // added rows: all row ids, then all values, then the stores, so that a tile's loads are
+        // in flight together
+        const char* __restrict__ const ab = p.add_base;
+        const uint32_t* __restrict__ const ai = p.add_index;
+        const uint32_t cnt = *p.add_count;
+        uint32_t row[16];
+        float addv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i = i0 + wi + 8 * (r >> 2) + 4 * hl + (r & 3);
+            row[r] = (uint32_t)i < cnt ? ai[i] : 0u;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) addv[r] = load1(ab + (int64_t)row[r] * p.add_pitch, kcol, p.add_etype);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i = i0 + wi + 8 * (r >> 2) + 4 * hl + (r & 3);
+            gout[(size_t)(grad_c0 + d * n_self + i) * Dp + kcol] = acc[r] + addv[r];
+        }
+        return;
+    }
+    float sv[16];
+    if (DIST == DIST_L2) load_self(sv);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int i_loc = wi + 8 * (r >> 2) + 4 * hl + (r & 3);
+        float o = acc[r];
+        if (DIST == DIST_L2) o = sv[r] * csum_s[i_loc] - o;
+        gout[(size_t)(grad_c0 + d * n_self + i0 + i_loc) * Dp + kcol] = o;
+    }
+}
+
+// both sides in one launch, in the order of k_score_bwd_mfma_both
+template <int DIST>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_score_bwd_split_both(BwdParams p) {
+    __shared__ __attribute__((aligned(16))) char smem[kBwdSplitSmemBytes];
+    const int gx = p.Dp / BS_TK, ga = p.B / BS_TI, gb = p.T / BS_TI;
+    const bool heads_first = p.T >= p.B;  // a head tile loops over T rows, a tail tile over B
+    const int n_first = gx * (heads_first ? ga : gb) * p.S;
+    const int L = blockIdx.x;
+    if ((L < n_first) == heads_first) {
+        const TileId tile = xcd_tile(gx, ga, p.S, heads_first ? L : L - n_first);
+        bwd_split_body<DIST, 0>(p, tile.z, tile.x, tile.y, smem);
+    } else {
+        const TileId tile = xcd_tile(gx, gb, p.S, heads_first ? L - n_first : L);
+        bwd_split_body<DIST, 1>(p, tile.z, tile.x, tile.y, smem);
+    }
+}
+
 void launch_bwd(const BwdParams& p, int dist_fn, hipStream_t stream) {
     const int n_self = p.side_b ? p.T : p.B;
     const bool mfma_ok = p.use_mfma && !p.coef_div && p.ent_a.vec && p.ent_b.vec && (p.Dp & 3) == 0 &&
@@ -755,7 +993,14 @@ void launch_score_bwd(const ScoreShape& sh, const RowSource& ent, const float* r
         const dim3 grid = tile_grid(sh.Dp / BM_TK, sh.B / BM_TI + sh.T / BM_TI, sh.S);
         // eight waves per workgroup (two per SIMD): measured faster than four at
         // every benchmark shape, few workgroups (1M-row workload) or many (22.8M-row workload)
-        if (dist_fn == DIST_L2)
+        // three-piece bfloat16 products where the forward pass uses them; whole slabs of 32 rows
+        // of `other` on either side (the merged tails' live counts are multiples of tpad)
+        const bool split = sh.use_mfma == 2 && (!sh.tcount || sh.tpad % (2 * BS_KJ) == 0);
+        if (split && dist_fn == DIST_L2)
+            hipLaunchKernelGGL(k_score_bwd_split_both<DIST_L2>, grid, dim3(512), 0, stream, p);
+        else if (split)
+            hipLaunchKernelGGL(k_score_bwd_split_both<DIST_DOT>, grid, dim3(512), 0, stream, p);
+        else if (dist_fn == DIST_L2)
             hipLaunchKernelGGL((k_score_bwd_mfma_both<DIST_L2, 32, true, 8>), grid, dim3(512), 0, stream, p);
         else
             hipLaunchKernelGGL((k_score_bwd_mfma_both<DIST_DOT, 32, true, 8>), grid, dim3(512), 0, stream, p);
