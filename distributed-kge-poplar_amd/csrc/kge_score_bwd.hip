@@ -615,6 +615,7 @@ DEVINL void bwd_split_body(const BwdParams& p, const int d, const int tile_x, co
         return 32 * nt < t_live ? f : 0u;  // no flags for columns the forward pass did not visit
     };
     float cs_acc = 0.f;
+    uint32_t flag_seen = 0u;  // any flagged block among those this thread staged
     // a slab's operand loads take a round trip to the memory-side cache however little work a
     // slab is: two register sets, each filled two slabs ahead of its use
     struct Slab {
@@ -644,6 +645,7 @@ DEVINL void bwd_split_body(const BwdParams& p, const int d, const int tile_x, co
     // vanish, its rows' sums leave it out) and it is taken in the direct form after the loop.
     auto stage = [&](const Slab& s, int nb, float live) __attribute__((always_inline)) {
         const float keep = s.nf_row == 0u ? live : 0.f;
+        flag_seen |= s.nf_row;
         const floatx4 a0 = s.a[0] * keep, a1 = s.a[1] * keep;
         uint2 lo[3], hi[3];
         split4_bf16(a0, lo);
@@ -687,7 +689,7 @@ DEVINL void bwd_split_body(const BwdParams& p, const int d, const int tile_x, co
 #pragma unroll
         for (int i = 0; i < 12; ++i) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
             if (i < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             else __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
@@ -703,31 +705,31 @@ DEVINL void bwd_split_body(const BwdParams& p, const int d, const int tile_x, co
         step(set0, jbase, 0);
         step(set1, jbase + BS_KJ, 1);
     }
+    float sv[16];
     if (DIST == DIST_L2) {
+        load_self(sv);  // (in flight across the barriers below)
+        // the four partial sums of a row, added in a fixed order; and whether any block of the
+        // tile was flagged at all
+        part[a_kg * BS_TI + a_row] = cs_acc;
+        const int any_flag = __syncthreads_or(flag_seen != 0u);
+        if (tid < BS_TI) csum_s[tid] = ((part[tid] + part[BS_TI + tid]) + part[2 * BS_TI + tid]) + part[3 * BS_TI + tid];
+        __syncthreads();
         // slabs in which some pair of this wave's sub-tile is nearly identical: c * (self - other)
         // directly, as the reference codelet does, from the operands in memory (acc holds the
         // negated sum).  Rare, and out of the loop above so that its registers stay out of it.
-        for (int jbase = 0; jbase < n_other; jbase += BS_KJ) {
-            if (flag_of((i0 + wi) >> 5, jbase >> 5) == 0u) continue;
-            float sv[16];
-            load_self(sv);
-            for (int jj = jbase; jj < jbase + BS_KJ; ++jj) {
-                const float o = reinterpret_cast<const float*>(other_rows + (int64_t)jj * opitch)[kcol];
+        if (any_flag)
+            for (int jbase = 0; jbase < n_other; jbase += BS_KJ) {
+                if (flag_of((i0 + wi) >> 5, jbase >> 5) == 0u) continue;
+                for (int jj = jbase; jj < jbase + BS_KJ; ++jj) {
+                    const float o = reinterpret_cast<const float*>(other_rows + (int64_t)jj * opitch)[kcol];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int i = i0 + wi + 8 * (r >> 2) + 4 * hl + (r & 3);
-                    const float cc = SIDE_B ? coef[(size_t)jj * T + i] : coef[(size_t)i * T + jj];
-                    acc[r] = fmaf(-cc, sv[r] - o, acc[r]);
+                    for (int r = 0; r < 16; ++r) {
+                        const int i = i0 + wi + 8 * (r >> 2) + 4 * hl + (r & 3);
+                        const float cc = SIDE_B ? coef[(size_t)jj * T + i] : coef[(size_t)i * T + jj];
+                        acc[r] = fmaf(-cc, sv[r] - o, acc[r]);
+                    }
                 }
             }
-        }
-    }
-    if (DIST == DIST_L2) {
-        // the four partial sums of a row, added in a fixed order
-        part[a_kg * BS_TI + a_row] = cs_acc;
-        __syncthreads();
-        if (tid < BS_TI) csum_s[tid] = ((part[tid] + part[BS_TI + tid]) + part[2 * BS_TI + tid]) + part[3 * BS_TI + tid];
-        __syncthreads();
     }
     float* __restrict__ const gout = p.grad;
     if (DIST == DIST_DOT && p.add_base) {
@@ -752,8 +754,6 @@ DEVINL void bwd_split_body(const BwdParams& p, const int d, const int tile_x, co
         }
         return;
     }
-    float sv[16];
-    if (DIST == DIST_L2) load_self(sv);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int i_loc = wi + 8 * (r >> 2) + 4 * hl + (r & 3);
