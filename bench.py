@@ -189,6 +189,11 @@ def split_forward(w):
             and w["batch"] % 128 == 0 and w["tails"] % 64 == 0 and w["dim"] % 64 == 0)
 
 
+def split_backward(w):
+    """The same for the backward kernel (its tiles are 128 rows on either side)."""
+    return split_forward(w) and w["tails"] % 128 == 0
+
+
 # kernels whose working set (a few tens of MB, just written by the kernel before) is served by the
 # memory-side caches: their rate is no HBM figure
 CACHE_SERVED = ("gather_operands", "reduce_entity")
@@ -239,11 +244,11 @@ def kernel_table(w, timing, n_steps, uniq_rows, contributions):
         else:
             # the published peak of the instruction the kernel issues: float32 matrix / vector
             # instructions 157.3; bfloat16 matrix instructions 2500, of which the float32-product
-            # forward kernel issues six per product (three-piece operands)
+            # kernels issue six per product (three-piece operands)
             peak, instr = PEAK_FP32_TFLOPS, "f32"
             if w.get("scoring_dtype") == "bfloat16":
                 peak, instr = PEAK_BF16_TFLOPS, "bf16"
-            elif name == "score_fwd" and split_forward(w):
+            elif (name == "score_fwd" and split_forward(w)) or (name == "score_bwd" and split_backward(w)):
                 peak, instr = PEAK_BF16_TFLOPS / 6.0, "bf16 x6 (float32 products)"
             entry.update(bound="mfma", achieved=amount / (ms * 1e-3) / 1e12, peak=peak, unit="TFLOP/s",
                          instructions=instr)
