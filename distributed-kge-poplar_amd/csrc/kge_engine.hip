@@ -295,7 +295,7 @@ struct kge_engine {
     // predict scratch (allocated by the first predict call)
     DevBuf<uint32_t> p_idx, p_rel, p_count, p_best_i;
     DevBuf<float> p_opnd, p_scores, p_best_s, p_hidden, p_featd, p_opnd_n, p_cmat;
-    DevBuf<uint16_t> opnd16, opndT16, coef16, coefT16, feat16, featT16, projT16, gT16;  // bfloat16 scoring operands
+    DevBuf<uint16_t> opnd16, coef16, feat16, projT16, gT16;  // bfloat16 scoring operands
     // norm regularisers (src/poplar_kge.cpp:430-437): per distinct row gradients and loss shares
     float reg_p[3] = {3.f, 3.f, 3.f}, reg_w[3] = {0.f, 0.f, 0.f};
     bool reg_on = false;
@@ -702,9 +702,7 @@ void allocate(kge_engine& E) {
     if (!fused && E.dist_fn == DIST_L2) E.dist.alloc(SB * E.T);
     if (E.score_bf16) {
         E.opnd16.alloc(R * E.Dp);
-        E.opndT16.alloc(R * E.Dp);
         E.coef16.alloc(SB * E.T);
-        E.coefT16.alloc(SB * E.T);
         // split-contraction partials of the two backward products
         const size_t p_head = (size_t)E.S * gemm_nt_bf16_ksplit(E.B, E.Dp, E.T, E.S) * E.B * E.Dp;
         const size_t p_tail = (size_t)E.S * gemm_nt_bf16_ksplit(E.T, E.Dp, E.B, E.S) * E.T * E.Dp;
@@ -740,7 +738,6 @@ void allocate(kge_engine& E) {
         E.gproj_part.alloc((size_t)16 * E.Fp * E.Dp);
         if (E.score_bf16) {
             E.feat16.alloc(R * E.Fp);
-            E.featT16.alloc(R * E.Fp);
             E.projT16.alloc((size_t)E.Fp * E.Dp);
             E.gT16.alloc(R * E.Dp);
             E.projR.alloc((size_t)E.Fp * E.Dp);
@@ -1129,7 +1126,7 @@ void run_step(kge_engine& E, int i) {
             f.Dp = E.Dp; f.Fp = E.Fp; f.proj = E.proj.p + (size_t)net * E.Fp * E.Dp;
             f.featd = E.featd.p; f.gproj_part = E.gproj_part.p; f.use_mfma = E.use_mfma;
             f.round_bf16 = E.score_bf16 ? 1 : 0; f.projR = E.projR.p;
-            f.feat16 = E.feat16.p; f.featT16 = E.featT16.p; f.projT16 = E.projT16.p; f.gT16 = E.gT16.p;
+            f.feat16 = E.feat16.p; f.projT16 = E.projT16.p; f.gT16 = E.gT16.p;
             FeatureArgs fp = f;  // the feature part alone, without the embedding
             fp.emb_base = nullptr;
             float* hid = E.hidden.p + net * rows_n;          // value + feature part
@@ -1187,7 +1184,6 @@ void run_step(kge_engine& E, int i) {
     float* loss_part = E.loss_part.p + (size_t)i * E.S * E.n_part;
     // bfloat16 dot-product scoring on the matrix cores: three batched products
     //   scores = q . tails^T,   d q = c . tails,   d tails = c^T . q
-    // each in the form C = A . Bt^T, which needs tails^T, q^T and c^T: transposing casts
     const int Bn = E.B, Tn = E.T, Dp = E.Dp;
     const bool bf16_fast = E.score_bf16 && E.use_mfma && gemm_nt_bf16_ok(Bn, Tn, Dp) &&
                            gemm_nt_bf16_ok(Bn, Dp, Tn) && gemm_nt_bf16_ok(Tn, Dp, Bn);
@@ -1208,34 +1204,20 @@ void run_step(kge_engine& E, int i) {
           g.n_limit = nullptr; }
         // only the bfloat16 coefficients are read from here on
         { KernelTimer t(E, K_LOSS); launch_loss_rows(sh, clabel, E.coef.p, nullptr, loss_part, E.coef16.p, st, false); }
-        // q^T and tails^T: one launch over all operand rows when there is a single block
-        // (rows [0, B) heads, [B, B + T) tails: the transposed matrix [Dp, B + T] holds both)
-        const bool one_block = E.S == 1;
-        const int64_t ldT = one_block ? Bn + Tn : 0;
+        // d q and d tails contract over the rows of their second operand (and d tails over the
+        // rows of the coefficients too): the product kernel takes such operands as they lie
         { KernelTimer t(E, K_BWD);
-          TransposeLimit tails, coefs;   // dead tail columns are neither transposed nor multiplied
-          tails.rows = tc; tails.stride = 1; tails.pad = E.tpad;
-          coefs.cols = tc; coefs.stride = 1; coefs.pad = E.tpad;
-          if (one_block) {
-              tails.row_base = Bn;
-              launch_transpose_bf16(E.opnd16.p, false, 1, Bn + Tn, Dp, Dp, 0, E.opndT16.p, nullptr, st, tails);
-          } else {
-              launch_transpose_bf16(E.opnd16.p, false, E.S, Bn, Dp, Dp, (int64_t)Bn * Dp, E.opndT16.p, nullptr, st);
-              launch_transpose_bf16(E.opnd16.p + head_n, false, E.S, Tn, Dp, Dp, (int64_t)Tn * Dp,
-                                    E.opndT16.p + head_n, nullptr, st, tails);
-          }
-          launch_transpose_bf16(E.coef16.p, false, E.S, Bn, Tn, Tn, (int64_t)Bn * Tn, E.coefT16.p, nullptr, st, coefs);
           // d q [B, Dp] = c [B, T] . tails [T, Dp]
           g.A = E.coef16.p; g.lda = Tn; g.a_batch = (int64_t)Bn * Tn;
-          g.Bt = one_block ? E.opndT16.p + Bn : E.opndT16.p + head_n; g.ldb = one_block ? (int)ldT : Tn; g.b_batch = (int64_t)Dp * Tn;
+          g.Bt = E.opnd16.p + head_n; g.ldb = Dp; g.b_batch = (int64_t)Tn * Dp; g.b_kmajor = 1;
           g.C = E.grad.p; g.ldc = Dp; g.c_batch = (int64_t)Bn * Dp;
           g.M = Bn; g.N = Dp; g.K = Tn; g.part = E.gemm_part.p;
           g.k_limit = tc;
           launch_gemm_nt_bf16(g, st);
           g.k_limit = nullptr;
           // d tails [T, Dp] = c^T [T, B] . q [B, Dp]
-          g.A = E.coefT16.p; g.lda = Bn; g.a_batch = (int64_t)Tn * Bn;
-          g.Bt = E.opndT16.p; g.ldb = one_block ? (int)ldT : Bn; g.b_batch = (int64_t)Dp * Bn;
+          g.A = E.coef16.p; g.lda = Tn; g.a_batch = (int64_t)Bn * Tn; g.a_kmajor = 1;
+          g.Bt = E.opnd16.p; g.ldb = Dp; g.b_batch = (int64_t)Bn * Dp;
           g.C = E.grad.p + head_n; g.ldc = Dp; g.c_batch = (int64_t)Tn * Dp;
           g.M = Tn; g.N = Dp; g.K = Bn;
           g.m_limit = tc;

@@ -201,8 +201,8 @@ void launch_gather_operands(const RowSource& ent, const float* rel, const uint32
 // Strides in elements.  Optional rows added to the output: output row m gets row
 // add_index[m] of add_base (row 0 for m >= *add_count), columns as C's.
 struct GemmNT {
-    const uint16_t* A;  int64_t lda, a_batch;   // [M, K]
-    const uint16_t* Bt; int64_t ldb, b_batch;   // [N, K]
+    const uint16_t* A;  int64_t lda, a_batch;   // [M, K], or [K, M] with a_kmajor
+    const uint16_t* Bt; int64_t ldb, b_batch;   // [N, K], or [K, N] with b_kmajor
     float* C;           int64_t ldc, c_batch;   // [M, N]
     int M, N, K, batches;
     float* part; int ksplit;                    // scratch for split contractions (or null); set by the launcher
@@ -214,6 +214,8 @@ struct GemmNT {
     // from the k_limit (rounded up to the slab) on are taken as zero
     const uint32_t* m_limit; const uint32_t* k_limit; const uint32_t* n_limit;
     int limit_stride;
+    // the operand lies with the contraction index outermost (even pitch, 4-byte aligned base)
+    int a_kmajor, b_kmajor;
 };
 bool gemm_nt_bf16_ok(int M, int N, int K);
 int gemm_nt_bf16_ksplit(int M, int N, int K, int batches);  // partials needed: batches * ksplit * M * N floats
@@ -394,7 +396,7 @@ struct FeatureArgs {
     int use_mfma;
     // bfloat16 products (null without bfloat16 scoring): features [max_rows, Fp] and their
     // transpose, W^T [Dp, Fp], grad_rows^T [Dp, max_rows]
-    uint16_t *feat16, *featT16, *projT16, *gT16;
+    uint16_t *feat16, *projT16, *gT16;
     int round_bf16;         // features and W enter their products rounded to bfloat16
     float* projR;           // scratch [Fp, Dp]: W rounded, for the float32 kernels
 };

@@ -830,6 +830,12 @@ void launch_score_fwd_rows(const ScoreShape& sh, const RowSource& a, const RowSo
 // Shapes: M % 128 == 0, N % 128 == 0, K % 64 == 0, rows 16-byte aligned.
 constexpr int GB_T = 128, GB_K = 64, GB_LD = GB_K + 8;
 
+// AK / BK: the operand lies with the contraction index outermost (A[k][m] / B[k][n], pitch lda /
+// ldb between k rows), as the other operand of a product whose result is needed transposed
+// does: a thread then fetches eight k of a pair of adjacent rows with eight 4-byte loads
+// (consecutive lanes on consecutive pairs) and regroups them into the two rows' 16-byte pieces
+// with byte permutes, so the LDS tiles and the matrix loop are the same in every form.
+template <bool AK, bool BK>
 __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     __shared__ __attribute__((aligned(16))) uint16_t As[GB_T][GB_LD];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[GB_T][GB_LD];
@@ -849,8 +855,9 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
     const int hl = lane >> 5, cl = lane & 31;
-    const uint16_t* A = g.A + (size_t)zb * g.a_batch + (size_t)m0 * g.lda + (size_t)zs * (g.K / g.ksplit);
-    const uint16_t* Bt = g.Bt + (size_t)zb * g.b_batch + (size_t)n0 * g.ldb + (size_t)zs * (g.K / g.ksplit);
+    const size_t ks0 = (size_t)zs * (g.K / g.ksplit);  // this split's first contraction index
+    const uint16_t* A = g.A + (size_t)zb * g.a_batch + (AK ? ks0 * g.lda + m0 : (size_t)m0 * g.lda + ks0);
+    const uint16_t* Bt = g.Bt + (size_t)zb * g.b_batch + (BK ? ks0 * g.ldb + n0 : (size_t)n0 * g.ldb + ks0);
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -860,23 +867,55 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // staging: 128 rows x 64 columns = 1024 16-byte pieces per operand, four per thread
+    // staging: 128 rows x 64 columns = 1024 16-byte pieces per operand, four per thread.
+    // Row-major operand: piece h = row (tid + 256 h) / 8, columns 8 ((tid + 256 h) % 8) .. + 7.
+    // k-outermost operand: task t = 0, 1: rows 2 lane, 2 lane + 1 of the tile, columns
+    // 8 (wave + 4 t) .. + 7; register 2 t + 0 / + 1 hold the eight loaded words' halves.
     floatx4 areg[4], breg[4];
+    auto load_kmajor = [&](const uint16_t* X, int64_t ld, int k0, floatx4* reg) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint16_t* src = X + (size_t)(k0 + 8 * (wave + 4 * t)) * ld + 2 * lane;
+#pragma unroll
+            for (int x = 0; x < 8; ++x)
+                reg[2 * t + (x >> 2)][x & 3] = __uint_as_float(*reinterpret_cast<const uint32_t*>(src + (size_t)x * ld));
+        }
+    };
+    auto store_kmajor = [&](uint16_t (*Xs)[GB_LD], const floatx4* reg) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            uint32_t w[8];
+#pragma unroll
+            for (int x = 0; x < 8; ++x) w[x] = __float_as_uint(reg[2 * t + (x >> 2)][x & 3]);
+            uint4 even, odd;  // the lower halves (row 2 lane) and the upper halves (row 2 lane + 1)
+            even.x = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u); odd.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
+            even.y = __builtin_amdgcn_perm(w[3], w[2], 0x05040100u); odd.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
+            even.z = __builtin_amdgcn_perm(w[5], w[4], 0x05040100u); odd.z = __builtin_amdgcn_perm(w[5], w[4], 0x07060302u);
+            even.w = __builtin_amdgcn_perm(w[7], w[6], 0x05040100u); odd.w = __builtin_amdgcn_perm(w[7], w[6], 0x07060302u);
+            const int col = 8 * (wave + 4 * t);
+            *reinterpret_cast<uint4*>(&Xs[2 * lane][col]) = even;
+            *reinterpret_cast<uint4*>(&Xs[2 * lane + 1][col]) = odd;
+        }
+    };
     auto prefetch = [&](int k0) __attribute__((always_inline)) {
+        if (AK) load_kmajor(A, g.lda, k0, areg);
+        if (BK) load_kmajor(Bt, g.ldb, k0, breg);
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
             const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
-            areg[h] = *reinterpret_cast<const floatx4*>(A + (size_t)row * g.lda + k0 + col);
-            breg[h] = *reinterpret_cast<const floatx4*>(Bt + (size_t)row * g.ldb + k0 + col);
+            if (!AK) areg[h] = *reinterpret_cast<const floatx4*>(A + (size_t)row * g.lda + k0 + col);
+            if (!BK) breg[h] = *reinterpret_cast<const floatx4*>(Bt + (size_t)row * g.ldb + k0 + col);
         }
     };
     if (K > 0) prefetch(0);
     for (int k0 = 0; k0 < K; k0 += GB_K) {
+        if (AK) store_kmajor(As, areg);
+        if (BK) store_kmajor(Bs, breg);
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
             const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
-            *reinterpret_cast<floatx4*>(&As[row][col]) = areg[h];
-            *reinterpret_cast<floatx4*>(&Bs[row][col]) = breg[h];
+            if (!AK) *reinterpret_cast<floatx4*>(&As[row][col]) = areg[h];
+            if (!BK) *reinterpret_cast<floatx4*>(&Bs[row][col]) = breg[h];
         }
         __syncthreads();
         if (k0 + GB_K < K) prefetch(k0 + GB_K);
@@ -976,8 +1015,11 @@ __global__ __launch_bounds__(256) void k_sum_split_batches(const float* __restri
 void launch_gemm_nt_bf16(const GemmNT& g0, hipStream_t stream) {
     GemmNT g = g0;
     g.ksplit = (g.part && g.ldc == g.N && !g.add_base) ? gemm_nt_bf16_ksplit(g.M, g.N, g.K, g.batches) : 1;
-    hipLaunchKernelGGL(k_gemm_nt_bf16, tile_grid(g.N / GB_T, g.M / GB_T, g.batches * g.ksplit), dim3(256), 0,
-                       stream, g);
+    const dim3 grid = tile_grid(g.N / GB_T, g.M / GB_T, g.batches * g.ksplit);
+    if (g.a_kmajor && g.b_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<true, true>), grid, dim3(256), 0, stream, g);
+    else if (g.a_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<true, false>), grid, dim3(256), 0, stream, g);
+    else if (g.b_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<false, true>), grid, dim3(256), 0, stream, g);
+    else hipLaunchKernelGGL((k_gemm_nt_bf16<false, false>), grid, dim3(256), 0, stream, g);
     if (g.ksplit > 1) {
         const int64_t n = (int64_t)g.M * g.N;
         hipLaunchKernelGGL(k_sum_split_batches, dim3((unsigned)((n / 4 + 255) / 256), g.batches), dim3(256), 0,
@@ -2142,16 +2184,16 @@ __global__ __launch_bounds__(256) void k_sum_splits(const float* __restrict__ pa
 void launch_proj_grad(const FeatureArgs& a, const float* grad_rows, float* gproj,
                       hipStream_t stream) {
     if (feature_bf16_ok(a)) {
-        // gproj [Fp, Dp] = features^T [Fp, U] . grad_rows [U, Dp]: A = features^T, Bt = grad_rows^T;
+        // gproj [Fp, Dp] = features^T [Fp, U] . grad_rows [U, Dp]: A = the features, read with the
+        // contraction index outermost, Bt = grad_rows^T (a transposing cast: they are float32);
         // rows past the distinct count are zero in the features and finite in grad_rows
-        // (the contraction stops at the distinct count, so neither those rows nor their
-        // transposes are touched)
+        // (the contraction stops at the distinct count, rounded up to a slab)
         TransposeLimit live_rows;   // rows past the step's distinct count are skipped
         live_rows.rows = a.counts;
-        launch_transpose_bf16(a.feat16, false, 1, a.max_rows, a.Fp, a.Fp, 0, a.featT16, nullptr, stream, live_rows);
         launch_transpose_bf16(grad_rows, true, 1, a.max_rows, a.Dp, a.Dp, 0, a.gT16, nullptr, stream, live_rows);
         GemmNT g = {};
-        g.A = a.featT16; g.lda = a.max_rows; g.Bt = a.gT16; g.ldb = a.max_rows; g.C = gproj; g.ldc = a.Dp;
+        g.A = a.feat16; g.lda = a.Fp; g.a_kmajor = 1;  // the features as they lie, [U, Fp]
+        g.Bt = a.gT16; g.ldb = a.max_rows; g.C = gproj; g.ldc = a.Dp;
         g.M = a.Fp; g.N = a.Dp; g.K = a.max_rows; g.batches = 1;
         g.part = a.gproj_part;  // [16, Fp, Dp]: room for every split
         g.k_limit = a.counts;
