@@ -748,3 +748,41 @@ def test_host_arrays_are_checked_chunk_by_chunk():
     with pytest.raises(ValueError, match="'remote' holds index 90 out of range"):
         H.train(engine, c, 0.05, bad)
     assert H.read_state(engine, c)["step"] == st0["step"] + 6 + n_step
+
+
+def test_staged_batch_in_one_call_or_in_pieces():
+    """A staged batch's steps run in one call or in several (`step_begin` / `step_count`: the
+    plan then covers each call's steps only) must leave bit-identical tables: 40 steps in one
+    call against the same 40 steps in two calls of 20 on a second engine, and both against the
+    oracle."""
+    import libpoplar_kge
+
+    c = K.cfg_dict(feature=0, n_shard=4, batch=32, a2a=8, dim=16, n_entity=400, n_relation=9, shared_table=True)
+    rng = np.random.default_rng(77)
+    st0 = K.make_state(c, rng)
+    n_step = 40
+    batch = K.raw_batch(c, n_step, rng)
+    lr = np.full(c["n_shard"], 0.02, np.float32)
+    results = []
+    for pieces in ([(0, 40)], [(0, 20), (20, 20)]):
+        engine = libpoplar_kge.Engine(H.engine_settings(c, n_step), "")
+        H.load_state(engine, c, st0)
+        engine.run("stage_batch", {k: np.ascontiguousarray(v) for k, v in batch.items()})
+        losses = []
+        for begin, count in pieces:
+            loss = np.full(c["n_shard"], np.nan, np.float32)
+            engine.run("train_step_loop", dict(learning_rate=lr, loss=loss, staged=True,
+                                               step_begin=int(begin), step_count=int(count)))
+            losses.append(loss * count)
+        results.append((sum(losses) / n_step, H.read_state(engine, c)))
+    (loss_a, st_a), (loss_b, st_b) = results
+    assert st_a["step"] == st_b["step"] == st0["step"] + n_step
+    np.testing.assert_allclose(loss_a, loss_b, rtol=1e-6)   # (a mean over 40 against two means over 20)
+    for name in ("entity_data", "relation_embedding", "relation_embedding/adam_m", "relation_embedding/adam_v"):
+        np.testing.assert_array_equal(st_a[name], st_b[name])
+    # and against the oracle
+    from oracle.kge_oracle import Oracle
+    ref = K.copy_state(st0)
+    loss_o = Oracle("f64").train_step_loop(make_cfg(**c), ref, 0.02, batch)
+    np.testing.assert_allclose(loss_a, loss_o, rtol=1e-5)
+    assert K.rel_l2(st_a["entity_data"], ref["entity_data"]) < 1e-5
