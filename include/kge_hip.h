@@ -140,7 +140,10 @@ int kge_buffer_write(void* buf, const uint32_t* idx, const void* data, int64_t n
  * grad_out[i,:] -- every row of grad_t is overwritten (rows nobody indexes
  * become zero, as the reference's zeroed table leaves them), duplicates are
  * summed deterministically (sort by index + segmented reduce).  `workspace`
- * must hold kge_scatter_add_workspace_bytes(n, rows, cols) bytes (16-byte aligned). */
+ * must hold kge_scatter_add_workspace_bytes(n, rows, cols) bytes (16-byte aligned).
+ * Indices are expected in [0, rows); an index outside that range adds nothing (its
+ * gradient row is dropped, no row of grad_t is touched by it) where the reference
+ * would address memory outside the table.  n + rows must be below 2^31. */
 size_t kge_scatter_add_workspace_bytes(int64_t n, int64_t rows, int64_t cols);
 int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* idx, int64_t n,
                     const float* grad_out, void* workspace, void* stream);
@@ -153,7 +156,10 @@ int kge_scatter_add(float* grad_t, int64_t rows, int64_t cols, const uint32_t* i
  * runs on holds until the process ends.  Sizes whose workspace
  * (kge_scatter_add_workspace_bytes) exceeds that are rejected with
  * KGE_INVALID_ARGUMENT and a message in `err`.  The call allocates and frees
- * nothing.  All calls on one GPU share that GPU's array: calls that overlap in
+ * nothing (the runtime itself sets a stream's queue up, scratch for the kernels'
+ * private segments included, when kernels first run on that stream: issue one
+ * call on the stream beforehand where even that matters).  All calls on one GPU
+ * share that GPU's array: calls that overlap in
  * time on one GPU (different streams, or host threads) race; issue them in
  * order on one stream. */
 size_t kge_scatter_add_static_max_bytes(void);

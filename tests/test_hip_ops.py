@@ -202,9 +202,11 @@ def test_multislice_kat():
                                rtol=1e-6)
 
 
+# (the last case: 1.36M keys to sort = 332 sort tiles, where the histogram scan is a launch of its
+# own instead of a part of the scatter)
 @pytest.mark.parametrize("rows,cols,n,zipf", [(100, 8, 1000, True), (5000, 256, 20000, True),
                                               (300, 64, 300, False), (17, 3, 0, False),
-                                              (70000, 4, 5000, False)])
+                                              (70000, 4, 5000, False), (60000, 4, 1_300_000, False)])
 def test_scatter_add_vs_oracle_and_deterministic(oracle64, rows, cols, n, zipf):
     rng = np.random.default_rng(n + rows)
     idx = (K.zipf_ids(rng, rows, n) if zipf else rng.integers(0, rows, n)).astype(np.uint32)

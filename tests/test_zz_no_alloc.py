@@ -77,3 +77,47 @@ def test_static_scatter_add_rejects_what_does_not_fit():
     assert "more than the 16777216 bytes of the static scratch array" in msg
     _, msg = _static(0, 4, idx[:1], g[:1, :4], expect=1)
     assert "out of range" in msg
+
+
+def test_static_scatter_add_allocates_nothing_and_takes_any_stream(oracle64):
+    """The entry point's claim: no device memory is allocated or freed by a call.  After a
+    warm-up call (the first call on a device looks the array's address up, the first on a stream
+    lets the runtime set that stream's queue up) the device's free memory is the same before and
+    after a series of calls whose operands were prepared beforehand, on the null stream and on a
+    stream of the caller's, whose result is bit-identical to the null stream's."""
+    lib = H.lib()
+    rng = np.random.default_rng(5)
+    rows, cols, n = 4000, 128, 30000
+    idx = K.zipf_ids(rng, rows, n).astype(np.uint32)
+    g = rng.normal(size=(n, cols)).astype(np.float32)
+    ti, tg = _operands(idx, g, cols)
+    out = torch.full((rows, cols), float("nan"), device="cuda")
+    err = C.create_string_buffer(512)
+
+    def call(stream):
+        rc = lib.kge_scatter_add_static(H.dptr(out), C.c_int64(rows), C.c_int64(cols), H.dptr(ti), C.c_int64(n),
+                                        H.dptr(tg), stream, err, C.c_size_t(512))
+        assert rc == 0, err.value
+
+    call(None)                                   # warm-up
+    torch.cuda.synchronize()
+    first = out.cpu().numpy()
+    free_before, _ = torch.cuda.mem_get_info()   # (hipMemGetInfo)
+    for _ in range(5):
+        call(None)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before   # nothing allocated, nothing freed
+    # a stream of the caller's (default priority).  Its first call is not measured: the runtime
+    # sets a new stream's queue up when kernels first run on it (among other things the scratch
+    # memory for their private segments), which takes device memory once per queue.
+    side = torch.cuda.Stream()
+    call(C.c_void_p(side.cuda_stream))
+    side.synchronize()
+    out.fill_(float("nan"))
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    call(C.c_void_p(side.cuda_stream))
+    side.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    np.testing.assert_array_equal(out.cpu().numpy(), first)
+    assert K.rel_l2(first, oracle64.multi_update_add(rows, idx, g)) < 1e-6
