@@ -295,7 +295,7 @@ struct kge_engine {
     // predict scratch (allocated by the first predict call)
     DevBuf<uint32_t> p_idx, p_rel, p_count, p_best_i;
     DevBuf<float> p_opnd, p_scores, p_best_s, p_hidden, p_featd, p_opnd_n, p_cmat;
-    DevBuf<uint16_t> opnd16, coef16, feat16, projT16, gT16;  // bfloat16 scoring operands
+    DevBuf<uint16_t> opnd16, coef16, feat16;  // bfloat16 scoring operands
     // norm regularisers (src/poplar_kge.cpp:430-437): per distinct row gradients and loss shares
     float reg_p[3] = {3.f, 3.f, 3.f}, reg_w[3] = {0.f, 0.f, 0.f};
     bool reg_on = false;
@@ -738,8 +738,6 @@ void allocate(kge_engine& E) {
         E.gproj_part.alloc((size_t)16 * E.Fp * E.Dp);
         if (E.score_bf16) {
             E.feat16.alloc(R * E.Fp);
-            E.projT16.alloc((size_t)E.Fp * E.Dp);
-            E.gT16.alloc(R * E.Dp);
             E.projR.alloc((size_t)E.Fp * E.Dp);
         }
         E.gproj.alloc(E.nets * proj_n);
@@ -1126,7 +1124,7 @@ void run_step(kge_engine& E, int i) {
             f.Dp = E.Dp; f.Fp = E.Fp; f.proj = E.proj.p + (size_t)net * E.Fp * E.Dp;
             f.featd = E.featd.p; f.gproj_part = E.gproj_part.p; f.use_mfma = E.use_mfma;
             f.round_bf16 = E.score_bf16 ? 1 : 0; f.projR = E.projR.p;
-            f.feat16 = E.feat16.p; f.projT16 = E.projT16.p; f.gT16 = E.gT16.p;
+            f.feat16 = E.feat16.p;
             FeatureArgs fp = f;  // the feature part alone, without the embedding
             fp.emb_base = nullptr;
             float* hid = E.hidden.p + net * rows_n;          // value + feature part

@@ -214,26 +214,14 @@ struct GemmNT {
     // from the k_limit (rounded up to the slab) on are taken as zero
     const uint32_t* m_limit; const uint32_t* k_limit; const uint32_t* n_limit;
     int limit_stride;
-    // the operand lies with the contraction index outermost (even pitch, 4-byte aligned base)
+    // the operand lies with the contraction index outermost (even pitch, 4-byte aligned base);
+    // b_kmajor = 2: and Bt points to float32 values (pitch and batch stride in floats, 8-byte
+    // aligned base), rounded to bfloat16 while staged
     int a_kmajor, b_kmajor;
 };
 bool gemm_nt_bf16_ok(int M, int N, int K);
 int gemm_nt_bf16_ksplit(int M, int N, int K, int batches);  // partials needed: batches * ksplit * M * N floats
 void launch_gemm_nt_bf16(const GemmNT& g, hipStream_t stream);
-// in[z][rows, cols] (float32 or bfloat16) -> out_t[z][cols, rows] bfloat16 and, unless null,
-// out[z][rows, cols] bfloat16; rows % 64 == 0, cols % 64 == 0
-// Device-side limits (or null; one count per batch `stride` words apart): input rows from
-// row_base + count (rounded up to `pad`) on, input columns from the column count (rounded up to
-// `pad`) on are skipped.
-struct TransposeLimit {
-    const uint32_t* rows = nullptr;
-    const uint32_t* cols = nullptr;
-    int row_base = 0, stride = 0, pad = 64;
-};
-void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, int cols, int64_t ld_in,
-                           int64_t in_batch, uint16_t* out_t, uint16_t* out, hipStream_t stream,
-                           const TransposeLimit& limit = TransposeLimit());
-
 // Scores of every block: a-operand row (d,b) = entity row of contribution
 // d*B+b combined with relation crel[d*B+b]; b-operand row (d,t) = entity row of
 // contribution S*B + d*T + t.  With `fused_loss` the logsigmoid loss and the
@@ -396,7 +384,7 @@ struct FeatureArgs {
     int use_mfma;
     // bfloat16 products (null without bfloat16 scoring): features [max_rows, Fp] and their
     // transpose, W^T [Dp, Fp], grad_rows^T [Dp, max_rows]
-    uint16_t *feat16, *projT16, *gT16;
+    uint16_t* feat16;
     int round_bf16;         // features and W enter their products rounded to bfloat16
     float* projR;           // scratch [Fp, Dp]: W rounded, for the float32 kernels
 };

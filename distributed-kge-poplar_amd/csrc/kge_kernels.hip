@@ -835,7 +835,9 @@ constexpr int GB_T = 128, GB_K = 64, GB_LD = GB_K + 8;
 // does: a thread then fetches eight k of a pair of adjacent rows with eight 4-byte loads
 // (consecutive lanes on consecutive pairs) and regroups them into the two rows' 16-byte pieces
 // with byte permutes, so the LDS tiles and the matrix loop are the same in every form.
-template <bool AK, bool BK>
+// BK = 2: such a B operand in float32 (8-byte loads of a pair's two values), rounded to bfloat16
+// (to nearest even) while it is regrouped.
+template <bool AK, int BK>
 __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     __shared__ __attribute__((aligned(16))) uint16_t As[GB_T][GB_LD];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[GB_T][GB_LD];
@@ -857,7 +859,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     const int hl = lane >> 5, cl = lane & 31;
     const size_t ks0 = (size_t)zs * (g.K / g.ksplit);  // this split's first contraction index
     const uint16_t* A = g.A + (size_t)zb * g.a_batch + (AK ? ks0 * g.lda + m0 : (size_t)m0 * g.lda + ks0);
-    const uint16_t* Bt = g.Bt + (size_t)zb * g.b_batch + (BK ? ks0 * g.ldb + n0 : (size_t)n0 * g.ldb + ks0);
+    const uint16_t* Bt = g.Bt + (BK == 2 ? 2 : 1) * ((size_t)zb * g.b_batch + (BK ? ks0 * g.ldb + n0 : (size_t)n0 * g.ldb + ks0));
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -871,7 +873,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     // Row-major operand: piece h = row (tid + 256 h) / 8, columns 8 ((tid + 256 h) % 8) .. + 7.
     // k-outermost operand: task t = 0, 1: rows 2 lane, 2 lane + 1 of the tile, columns
     // 8 (wave + 4 t) .. + 7; register 2 t + 0 / + 1 hold the eight loaded words' halves.
-    floatx4 areg[4], breg[4];
+    floatx4 areg[4], breg[BK == 2 ? 8 : 4];
     auto load_kmajor = [&](const uint16_t* X, int64_t ld, int k0, floatx4* reg) __attribute__((always_inline)) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -897,9 +899,37 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
             *reinterpret_cast<uint4*>(&Xs[2 * lane + 1][col]) = odd;
         }
     };
+    // float32 source: task t's eight rows of two floats in registers 4 t .. 4 t + 3
+    auto load_kmajor_f32 = [&](const float* X, int64_t ld, int k0, floatx4* reg) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const float* src = X + (size_t)(k0 + 8 * (wave + 4 * t)) * ld + 2 * lane;
+#pragma unroll
+            for (int x = 0; x < 8; ++x) {
+                const float2 v = *reinterpret_cast<const float2*>(src + (size_t)x * ld);
+                reg[4 * t + (x >> 1)][2 * (x & 1)] = v.x;
+                reg[4 * t + (x >> 1)][2 * (x & 1) + 1] = v.y;
+            }
+        }
+    };
+    auto store_kmajor_f32 = [&](uint16_t (*Xs)[GB_LD], const floatx4* reg) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            uint32_t even[4], odd[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {  // rows 2 q, 2 q + 1 of the eight: (x, y) (x, y)
+                even[q] = pack_bf16(reg[4 * t + q][0], reg[4 * t + q][2]);
+                odd[q] = pack_bf16(reg[4 * t + q][1], reg[4 * t + q][3]);
+            }
+            const int col = 8 * (wave + 4 * t);
+            *reinterpret_cast<uint4*>(&Xs[2 * lane][col]) = make_uint4(even[0], even[1], even[2], even[3]);
+            *reinterpret_cast<uint4*>(&Xs[2 * lane + 1][col]) = make_uint4(odd[0], odd[1], odd[2], odd[3]);
+        }
+    };
     auto prefetch = [&](int k0) __attribute__((always_inline)) {
         if (AK) load_kmajor(A, g.lda, k0, areg);
-        if (BK) load_kmajor(Bt, g.ldb, k0, breg);
+        if (BK == 1) load_kmajor(Bt, g.ldb, k0, breg);
+        if (BK == 2) load_kmajor_f32(reinterpret_cast<const float*>(Bt), g.ldb, k0, breg);
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
             const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
@@ -910,7 +940,8 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
     if (K > 0) prefetch(0);
     for (int k0 = 0; k0 < K; k0 += GB_K) {
         if (AK) store_kmajor(As, areg);
-        if (BK) store_kmajor(Bs, breg);
+        if (BK == 1) store_kmajor(Bs, breg);
+        if (BK == 2) store_kmajor_f32(Bs, breg);
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
             const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
@@ -1016,62 +1047,17 @@ void launch_gemm_nt_bf16(const GemmNT& g0, hipStream_t stream) {
     GemmNT g = g0;
     g.ksplit = (g.part && g.ldc == g.N && !g.add_base) ? gemm_nt_bf16_ksplit(g.M, g.N, g.K, g.batches) : 1;
     const dim3 grid = tile_grid(g.N / GB_T, g.M / GB_T, g.batches * g.ksplit);
-    if (g.a_kmajor && g.b_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<true, true>), grid, dim3(256), 0, stream, g);
-    else if (g.a_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<true, false>), grid, dim3(256), 0, stream, g);
-    else if (g.b_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<false, true>), grid, dim3(256), 0, stream, g);
-    else hipLaunchKernelGGL((k_gemm_nt_bf16<false, false>), grid, dim3(256), 0, stream, g);
+    if (g.a_kmajor && g.b_kmajor == 2) hipLaunchKernelGGL((k_gemm_nt_bf16<true, 2>), grid, dim3(256), 0, stream, g);
+    else if (g.a_kmajor && g.b_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<true, 1>), grid, dim3(256), 0, stream, g);
+    else if (g.a_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<true, 0>), grid, dim3(256), 0, stream, g);
+    else if (g.b_kmajor == 2) hipLaunchKernelGGL((k_gemm_nt_bf16<false, 2>), grid, dim3(256), 0, stream, g);
+    else if (g.b_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<false, 1>), grid, dim3(256), 0, stream, g);
+    else hipLaunchKernelGGL((k_gemm_nt_bf16<false, 0>), grid, dim3(256), 0, stream, g);
     if (g.ksplit > 1) {
         const int64_t n = (int64_t)g.M * g.N;
         hipLaunchKernelGGL(k_sum_split_batches, dim3((unsigned)((n / 4 + 255) / 256), g.batches), dim3(256), 0,
                            stream, g.part, g.ksplit, n, g.C, g.c_batch);
     }
-}
-
-// Transposing cast: in[z][r, c] (float32 or bfloat16, row pitch ld_in) ->
-// out_t[z][c, r] bfloat16 (dense) and, if asked, out[z][r, c] bfloat16 (dense).
-// 64 x 64 tiles through LDS; rows and cols multiples of 64.
-__global__ __launch_bounds__(256) void k_transpose_bf16(const void* __restrict__ in, int in_f32,
-                                                        int rows, int cols, int64_t ld_in,
-                                                        int64_t in_batch, uint16_t* __restrict__ out_t,
-                                                        uint16_t* __restrict__ out, TransposeLimit limit) {
-    // pitch of 66 elements: a column walk (the transposed read) steps 33 banks per row
-    __shared__ __attribute__((aligned(4))) uint16_t tile[64][66];
-    const int z = blockIdx.z, r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-    if (limit.rows && r0 >= limit.row_base + (int)((limit.rows[z * limit.stride] + limit.pad - 1) / limit.pad) * limit.pad) return;
-    if (limit.cols && c0 >= (int)((limit.cols[z * limit.stride] + limit.pad - 1) / limit.pad) * limit.pad) return;
-    const int q = (threadIdx.x & 15) * 4, lr = threadIdx.x >> 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = lr + 16 * i;
-        const size_t off = (size_t)z * in_batch + (size_t)(r0 + r) * ld_in + c0 + q;
-        uint2 raw;
-        if (in_f32) {
-            const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(in) + off);
-            raw.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
-            raw.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
-        } else {
-            raw = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(in) + off);
-        }
-        *reinterpret_cast<uint32_t*>(&tile[r][q]) = raw.x;
-        *reinterpret_cast<uint32_t*>(&tile[r][q + 2]) = raw.y;
-        if (out) *reinterpret_cast<uint2*>(out + ((size_t)z * rows + r0 + r) * cols + c0 + q) = raw;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int c = lr + 16 * i;
-        uint2 raw;
-        raw.x = (uint32_t)tile[q][c] | ((uint32_t)tile[q + 1][c] << 16);
-        raw.y = (uint32_t)tile[q + 2][c] | ((uint32_t)tile[q + 3][c] << 16);
-        *reinterpret_cast<uint2*>(out_t + ((size_t)z * cols + c0 + c) * rows + r0 + q) = raw;
-    }
-}
-
-void launch_transpose_bf16(const void* in, bool in_f32, int batches, int rows, int cols, int64_t ld_in,
-                           int64_t in_batch, uint16_t* out_t, uint16_t* out, hipStream_t stream,
-                           const TransposeLimit& limit) {
-    hipLaunchKernelGGL(k_transpose_bf16, dim3(cols / 64, rows / 64, batches), dim3(256), 0, stream, in,
-                       in_f32 ? 1 : 0, rows, cols, ld_in, in_batch, out_t, out, limit);
 }
 
 // --------------------------------------------------------------------------
@@ -2115,9 +2101,9 @@ void launch_hidden_fwd(const FeatureArgs& a, float* hidden, hipStream_t stream) 
         // hidden [U, Dp] = features [U, Fp] . W [Fp, Dp] + embedding: A = features, Bt = W^T
         hipLaunchKernelGGL(k_gather_features, dim3((a.max_rows + 3) / 4), dim3(256), 0, stream, a,
                            (float*)nullptr, a.feat16);
-        launch_transpose_bf16(a.proj, true, 1, a.Fp, a.Dp, a.Dp, 0, a.projT16, nullptr, stream);
         GemmNT g = {};
-        g.A = a.feat16; g.lda = a.Fp; g.Bt = a.projT16; g.ldb = a.Fp; g.C = hidden; g.ldc = a.Dp;
+        g.A = a.feat16; g.lda = a.Fp; g.C = hidden; g.ldc = a.Dp;
+        g.Bt = reinterpret_cast<const uint16_t*>(a.proj); g.ldb = a.Dp; g.b_kmajor = 2;  // W [Fp, Dp] float32 as it lies
         g.M = a.max_rows; g.N = a.Dp; g.K = a.Fp; g.batches = 1;
         g.add_base = a.emb_base; g.add_pitch = a.pitch; g.add_etype = a.emb_etype;
         g.add_index = a.uniq_key; g.add_count = a.counts;
@@ -2184,16 +2170,14 @@ __global__ __launch_bounds__(256) void k_sum_splits(const float* __restrict__ pa
 void launch_proj_grad(const FeatureArgs& a, const float* grad_rows, float* gproj,
                       hipStream_t stream) {
     if (feature_bf16_ok(a)) {
-        // gproj [Fp, Dp] = features^T [Fp, U] . grad_rows [U, Dp]: A = the features, read with the
-        // contraction index outermost, Bt = grad_rows^T (a transposing cast: they are float32);
+        // gproj [Fp, Dp] = features^T [Fp, U] . grad_rows [U, Dp]: both operands read as they lie,
+        // with the contraction index outermost (the float32 gradient rows rounded while staged);
         // rows past the distinct count are zero in the features and finite in grad_rows
         // (the contraction stops at the distinct count, rounded up to a slab)
-        TransposeLimit live_rows;   // rows past the step's distinct count are skipped
-        live_rows.rows = a.counts;
-        launch_transpose_bf16(grad_rows, true, 1, a.max_rows, a.Dp, a.Dp, 0, a.gT16, nullptr, stream, live_rows);
         GemmNT g = {};
         g.A = a.feat16; g.lda = a.Fp; g.a_kmajor = 1;  // the features as they lie, [U, Fp]
-        g.Bt = a.gT16; g.ldb = a.max_rows; g.C = gproj; g.ldc = a.Dp;
+        g.Bt = reinterpret_cast<const uint16_t*>(grad_rows); g.ldb = a.Dp; g.b_kmajor = 2;  // [U, Dp] float32 as they lie
+        g.C = gproj; g.ldc = a.Dp;
         g.M = a.Fp; g.N = a.Dp; g.K = a.max_rows; g.batches = 1;
         g.part = a.gproj_part;  // [16, Fp, Dp]: room for every split
         g.k_limit = a.counts;

@@ -732,28 +732,6 @@ DEVINL void bwd_split_body(const BwdParams& p, const int d, const int tile_x, co
             }
     }
     float* __restrict__ const gout = p.grad;
-    if (DIST == DIST_DOT && p.add_base) {
-        // added rows: all row ids, then all values, then the stores, so that a tile's loads are
-        // in flight together
-        const char* __restrict__ const ab = p.add_base;
-        const uint32_t* __restrict__ const ai = p.add_index;
-        const uint32_t cnt = *p.add_count;
-        uint32_t row[16];
-        float addv[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int i = i0 + wi + 8 * (r >> 2) + 4 * hl + (r & 3);
-            row[r] = (uint32_t)i < cnt ? ai[i] : 0u;
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) addv[r] = load1(ab + (int64_t)row[r] * p.add_pitch, kcol, p.add_etype);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int i = i0 + wi + 8 * (r >> 2) + 4 * hl + (r & 3);
-            gout[(size_t)(grad_c0 + d * n_self + i) * Dp + kcol] = acc[r] + addv[r];
-        }
-        return;
-    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int i_loc = wi + 8 * (r >> 2) + 4 * hl + (r & 3);
