@@ -598,7 +598,6 @@ def main():
         "dtype": head.pop("dtype"),
         "data": "synthetic",
     }
-    out.update(head)
     # the other table sizes, same protocol (W warm-up, K timed steps, kernel pass), one after the other
     extra = {}
     for x in also:
@@ -609,6 +608,11 @@ def main():
         extra[x] = measure(x, args, kge, torch, full=False)
     if extra:
         out["workloads"] = extra
+    # the headline workload's details behind the other workloads, its workload description, roofline
+    # and CPU baseline last: whoever reads only the end of this one long line still sees them
+    last = ("config", "roofline", "cpu_baseline", "speedup_over_cpu_baseline")
+    out.update({k: v for k, v in head.items() if k not in last})
+    out.update({k: head[k] for k in last if k in head})
 
     def plain(o):  # numpy scalars -> Python numbers
         if isinstance(o, np.generic):
