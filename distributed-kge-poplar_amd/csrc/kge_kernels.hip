@@ -823,12 +823,15 @@ void launch_score_fwd_rows(const ScoreShape& sh, const RowSource& a, const RowSo
 //   C[z][m, n] = sum_k A[z][m, k] * Bt[z][n, k],  bfloat16 in, float32 out,
 // with v_mfma_f32_32x32x16_bf16 (lane l supplies row l%32, columns
 // 8*(l/32) .. +7 of the 16-column step, for both operands).  Workgroup tile
-// 128 x 128, four waves as 2 x 2, each 2 x 2 accumulators of 32 x 32; K slabs of
-// 64 staged through LDS with 16-byte copies, the next slab in registers while
-// the current one is multiplied.  LDS rows are padded to 72 elements (144 B) so
-// that eight consecutive rows' 16-byte reads fall in different banks.
-// Shapes: M % 128 == 0, N % 128 == 0, K % 64 == 0, rows 16-byte aligned.
-constexpr int GB_T = 128, GB_K = 64, GB_LD = GB_K + 8;
+// TM x TN (128 or 64 each), four waves as 2 x 2, each (TM/64) x (TN/64)
+// accumulators of 32 x 32; K slabs of 64 staged through LDS with 16-byte copies, the
+// next slab in registers while the current one is multiplied.  LDS rows are padded to
+// 72 elements (144 B) so that eight consecutive rows' 16-byte reads fall in different
+// banks.  The launcher takes the largest tile that still gives the chip enough
+// workgroups: the step's products are small, and a launch with fewer workgroups than
+// CUs is bound by the latency of its slabs, not by the matrix cores.
+// Shapes: M % 64 == 0, N % 64 == 0, K % 64 == 0, rows 16-byte aligned.
+constexpr int GB_K = 64, GB_LD = GB_K + 8;
 
 // AK / BK: the operand lies with the contraction index outermost (A[k][m] / B[k][n], pitch lda /
 // ldb between k rows), as the other operand of a product whose result is needed transposed
@@ -837,15 +840,17 @@ constexpr int GB_T = 128, GB_K = 64, GB_LD = GB_K + 8;
 // with byte permutes, so the LDS tiles and the matrix loop are the same in every form.
 // BK = 2: such a B operand in float32 (8-byte loads of a pair's two values), rounded to bfloat16
 // (to nearest even) while it is regrouped.
-template <bool AK, int BK>
+template <bool AK, int BK, int TM, int TN>
 __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[GB_T][GB_LD];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[GB_T][GB_LD];
+    static_assert((TM == 128 || TM == 64) && (TN == 128 || TN == 64), "tile sizes");
+    constexpr int NI = TM / 64, NJ = TN / 64;  // 32 x 32 accumulators per wave
+    __shared__ __attribute__((aligned(16))) uint16_t As[TM][GB_LD];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[TN][GB_LD];
     // z = batch * ksplit + split: with ksplit > 1 every split multiplies its own K / ksplit
     // columns into its own partial output [batch][split][M, N]
-    const TileId tile = xcd_tile(g.N / GB_T, g.M / GB_T, g.batches * g.ksplit);
+    const TileId tile = xcd_tile(g.N / TN, g.M / TM, g.batches * g.ksplit);
     const int zb = tile.z / g.ksplit, zs = tile.z - zb * g.ksplit;
-    const int m0 = tile.y * GB_T, n0 = tile.x * GB_T;
+    const int m0 = tile.y * TM, n0 = tile.x * TN;
     const int lim = zb * g.limit_stride;
     if (g.m_limit && (uint32_t)m0 >= g.m_limit[lim]) return;
     if (g.n_limit && (uint32_t)n0 >= g.n_limit[lim]) return;
@@ -855,55 +860,61 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
         K = max(0, min(K, live - zs * K));
     }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * (TN / 2);
     const int hl = lane >> 5, cl = lane & 31;
     const size_t ks0 = (size_t)zs * (g.K / g.ksplit);  // this split's first contraction index
     const uint16_t* A = g.A + (size_t)zb * g.a_batch + (AK ? ks0 * g.lda + m0 : (size_t)m0 * g.lda + ks0);
     const uint16_t* Bt = g.Bt + (BK == 2 ? 2 : 1) * ((size_t)zb * g.b_batch + (BK ? ks0 * g.ldb + n0 : (size_t)n0 * g.ldb + ks0));
 
-    floatx16 acc[2][2];
+    floatx16 acc[NI][NJ];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // staging: 128 rows x 64 columns = 1024 16-byte pieces per operand, four per thread.
+    // staging: a T x 64 operand tile = 8 T 16-byte pieces, T / 32 per thread.
     // Row-major operand: piece h = row (tid + 256 h) / 8, columns 8 ((tid + 256 h) % 8) .. + 7.
-    // k-outermost operand: task t = 0, 1: rows 2 lane, 2 lane + 1 of the tile, columns
-    // 8 (wave + 4 t) .. + 7; register 2 t + 0 / + 1 hold the eight loaded words' halves.
-    floatx4 areg[4], breg[BK == 2 ? 8 : 4];
-    auto load_kmajor = [&](const uint16_t* X, int64_t ld, int k0, floatx4* reg) __attribute__((always_inline)) {
+    // k-outermost operand: T / 2 pairs of adjacent rows times eight 8-column groups = T / 64
+    // tasks per thread; a task's lanes take consecutive pairs (all 64 of one group for T = 128,
+    // 32 of each of two groups for T = 64), registers 2 t, 2 t + 1 hold its eight loaded words.
+    floatx4 areg[TM / 32], breg[BK == 2 ? TN / 16 : TN / 32];
+    auto task_pair = [&](int T) { return T == 128 ? lane : (lane & 31); };
+    auto task_group = [&](int T, int t) { return T == 128 ? wave + 4 * t : 2 * wave + (lane >> 5); };
+    auto load_kmajor = [&](auto tc, const uint16_t* X, int64_t ld, int k0, floatx4* reg) __attribute__((always_inline)) {
+        constexpr int T = decltype(tc)::value;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const uint16_t* src = X + (size_t)(k0 + 8 * (wave + 4 * t)) * ld + 2 * lane;
+        for (int t = 0; t < T / 64; ++t) {
+            const uint16_t* src = X + (size_t)(k0 + 8 * task_group(T, t)) * ld + 2 * task_pair(T);
 #pragma unroll
             for (int x = 0; x < 8; ++x)
                 reg[2 * t + (x >> 2)][x & 3] = __uint_as_float(*reinterpret_cast<const uint32_t*>(src + (size_t)x * ld));
         }
     };
-    auto store_kmajor = [&](uint16_t (*Xs)[GB_LD], const floatx4* reg) __attribute__((always_inline)) {
+    auto store_kmajor = [&](auto tc, uint16_t (*Xs)[GB_LD], const floatx4* reg) __attribute__((always_inline)) {
+        constexpr int T = decltype(tc)::value;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < T / 64; ++t) {
             uint32_t w[8];
 #pragma unroll
             for (int x = 0; x < 8; ++x) w[x] = __float_as_uint(reg[2 * t + (x >> 2)][x & 3]);
-            uint4 even, odd;  // the lower halves (row 2 lane) and the upper halves (row 2 lane + 1)
+            uint4 even, odd;  // the lower halves (row 2 pair) and the upper halves (row 2 pair + 1)
             even.x = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u); odd.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
             even.y = __builtin_amdgcn_perm(w[3], w[2], 0x05040100u); odd.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
             even.z = __builtin_amdgcn_perm(w[5], w[4], 0x05040100u); odd.z = __builtin_amdgcn_perm(w[5], w[4], 0x07060302u);
             even.w = __builtin_amdgcn_perm(w[7], w[6], 0x05040100u); odd.w = __builtin_amdgcn_perm(w[7], w[6], 0x07060302u);
-            const int col = 8 * (wave + 4 * t);
-            *reinterpret_cast<uint4*>(&Xs[2 * lane][col]) = even;
-            *reinterpret_cast<uint4*>(&Xs[2 * lane + 1][col]) = odd;
+            const int col = 8 * task_group(T, t), row = 2 * task_pair(T);
+            *reinterpret_cast<uint4*>(&Xs[row][col]) = even;
+            *reinterpret_cast<uint4*>(&Xs[row + 1][col]) = odd;
         }
     };
-    // float32 source: task t's eight rows of two floats in registers 4 t .. 4 t + 3
-    auto load_kmajor_f32 = [&](const float* X, int64_t ld, int k0, floatx4* reg) __attribute__((always_inline)) {
+    // float32 source: a task's eight rows of two floats in registers 4 t .. 4 t + 3
+    auto load_kmajor_f32 = [&](auto tc, const float* X, int64_t ld, int k0, floatx4* reg) __attribute__((always_inline)) {
+        constexpr int T = decltype(tc)::value;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const float* src = X + (size_t)(k0 + 8 * (wave + 4 * t)) * ld + 2 * lane;
+        for (int t = 0; t < T / 64; ++t) {
+            const float* src = X + (size_t)(k0 + 8 * task_group(T, t)) * ld + 2 * task_pair(T);
 #pragma unroll
             for (int x = 0; x < 8; ++x) {
                 const float2 v = *reinterpret_cast<const float2*>(src + (size_t)x * ld);
@@ -912,51 +923,69 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
             }
         }
     };
-    auto store_kmajor_f32 = [&](uint16_t (*Xs)[GB_LD], const floatx4* reg) __attribute__((always_inline)) {
+    auto store_kmajor_f32 = [&](auto tc, uint16_t (*Xs)[GB_LD], const floatx4* reg) __attribute__((always_inline)) {
+        constexpr int T = decltype(tc)::value;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < T / 64; ++t) {
             uint32_t even[4], odd[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {  // rows 2 q, 2 q + 1 of the eight: (x, y) (x, y)
                 even[q] = pack_bf16(reg[4 * t + q][0], reg[4 * t + q][2]);
                 odd[q] = pack_bf16(reg[4 * t + q][1], reg[4 * t + q][3]);
             }
-            const int col = 8 * (wave + 4 * t);
-            *reinterpret_cast<uint4*>(&Xs[2 * lane][col]) = make_uint4(even[0], even[1], even[2], even[3]);
-            *reinterpret_cast<uint4*>(&Xs[2 * lane + 1][col]) = make_uint4(odd[0], odd[1], odd[2], odd[3]);
+            const int col = 8 * task_group(T, t), row = 2 * task_pair(T);
+            *reinterpret_cast<uint4*>(&Xs[row][col]) = make_uint4(even[0], even[1], even[2], even[3]);
+            *reinterpret_cast<uint4*>(&Xs[row + 1][col]) = make_uint4(odd[0], odd[1], odd[2], odd[3]);
         }
     };
+    using TMc = std::integral_constant<int, TM>;
+    using TNc = std::integral_constant<int, TN>;
     auto prefetch = [&](int k0) __attribute__((always_inline)) {
-        if (AK) load_kmajor(A, g.lda, k0, areg);
-        if (BK == 1) load_kmajor(Bt, g.ldb, k0, breg);
-        if (BK == 2) load_kmajor_f32(reinterpret_cast<const float*>(Bt), g.ldb, k0, breg);
+        if (AK) load_kmajor(TMc{}, A, g.lda, k0, areg);
+        if (BK == 1) load_kmajor(TNc{}, Bt, g.ldb, k0, breg);
+        if (BK == 2) load_kmajor_f32(TNc{}, reinterpret_cast<const float*>(Bt), g.ldb, k0, breg);
+        if (!AK) {
 #pragma unroll
-        for (int h = 0; h < 4; ++h) {
-            const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
-            if (!AK) areg[h] = *reinterpret_cast<const floatx4*>(A + (size_t)row * g.lda + k0 + col);
-            if (!BK) breg[h] = *reinterpret_cast<const floatx4*>(Bt + (size_t)row * g.ldb + k0 + col);
+            for (int h = 0; h < TM / 32; ++h) {
+                const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
+                areg[h] = *reinterpret_cast<const floatx4*>(A + (size_t)row * g.lda + k0 + col);
+            }
+        }
+        if (!BK) {
+#pragma unroll
+            for (int h = 0; h < TN / 32; ++h) {
+                const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
+                breg[h] = *reinterpret_cast<const floatx4*>(Bt + (size_t)row * g.ldb + k0 + col);
+            }
         }
     };
     if (K > 0) prefetch(0);
     for (int k0 = 0; k0 < K; k0 += GB_K) {
-        if (AK) store_kmajor(As, areg);
-        if (BK == 1) store_kmajor(Bs, breg);
-        if (BK == 2) store_kmajor_f32(Bs, breg);
+        if (AK) store_kmajor(TMc{}, As, areg);
+        if (BK == 1) store_kmajor(TNc{}, Bs, breg);
+        if (BK == 2) store_kmajor_f32(TNc{}, Bs, breg);
+        if (!AK) {
 #pragma unroll
-        for (int h = 0; h < 4; ++h) {
-            const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
-            if (!AK) *reinterpret_cast<floatx4*>(&As[row][col]) = areg[h];
-            if (!BK) *reinterpret_cast<floatx4*>(&Bs[row][col]) = breg[h];
+            for (int h = 0; h < TM / 32; ++h) {
+                const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
+                *reinterpret_cast<floatx4*>(&As[row][col]) = areg[h];
+            }
+        }
+        if (!BK) {
+#pragma unroll
+            for (int h = 0; h < TN / 32; ++h) {
+                const int idx = tid + 256 * h, row = idx >> 3, col = (idx & 7) * 8;
+                *reinterpret_cast<floatx4*>(&Bs[row][col]) = breg[h];
+            }
         }
         __syncthreads();
         if (k0 + GB_K < K) prefetch(k0 + GB_K);
-        floatx4 fa[2][2], fb[2][2];
+        floatx4 fa[2][NI], fb[2][NJ];
         auto fetch = [&](int buf, int ks) __attribute__((always_inline)) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                fa[buf][i] = *reinterpret_cast<const floatx4*>(&As[wm + 32 * i + cl][16 * ks + 8 * hl]);
-                fb[buf][i] = *reinterpret_cast<const floatx4*>(&Bs[wn + 32 * i + cl][16 * ks + 8 * hl]);
-            }
+            for (int i = 0; i < NI; ++i) fa[buf][i] = *reinterpret_cast<const floatx4*>(&As[wm + 32 * i + cl][16 * ks + 8 * hl]);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) fb[buf][j] = *reinterpret_cast<const floatx4*>(&Bs[wn + 32 * j + cl][16 * ks + 8 * hl]);
         };
         fetch(0, 0);
 #pragma unroll
@@ -964,9 +993,9 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
             if (ks + 1 < GB_K / 16) fetch((ks + 1) & 1, ks + 1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < NI; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < NJ; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                         __builtin_bit_cast(bf16x8, fa[ks & 1][i]), __builtin_bit_cast(bf16x8, fb[ks & 1][j]),
                         acc[i][j], 0, 0, 0);
@@ -986,47 +1015,74 @@ __global__ __launch_bounds__(256) void k_gemm_nt_bf16(GemmNT g) {
         const uint32_t* __restrict__ const ai = g.add_index;
         const uint32_t cnt = *g.add_count;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < NI; ++i) {
             uint32_t add_row[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + wm + 32 * i + 8 * (r >> 2) + 4 * hl + (r & 3);
                 add_row[r] = (uint32_t)m < cnt ? ai[m] : 0u;
             }
-            float addv[16][2];
+            float addv[16][NJ];
 #pragma unroll
             for (int r = 0; r < 16; ++r)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < NJ; ++j)
                     addv[r][j] = load1(ab + (int64_t)add_row[r] * g.add_pitch, n0 + wn + 32 * j + cl, g.add_etype);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + wm + 32 * i + 8 * (r >> 2) + 4 * hl + (r & 3);
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < NJ; ++j)
                     Cr[(size_t)m * g.ldc + n0 + wn + 32 * j + cl] = acc[i][j][r] + addv[r][j];
             }
         }
         return;
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int m = m0 + wm + 32 * i + 8 * (r >> 2) + 4 * hl + (r & 3);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) Cr[(size_t)m * g.ldc + n0 + wn + 32 * j + cl] = acc[i][j][r];
+            for (int j = 0; j < NJ; ++j) Cr[(size_t)m * g.ldc + n0 + wn + 32 * j + cl] = acc[i][j][r];
         }
 }
 
-bool gemm_nt_bf16_ok(int M, int N, int K) { return M % GB_T == 0 && N % GB_T == 0 && K % GB_K == 0; }
+bool gemm_nt_bf16_ok(int M, int N, int K) { return M % 128 == 0 && N % 128 == 0 && K % GB_K == 0; }
 
-// How many ways to split the contraction so that the launch has at least two
-// workgroups per CU (a power of two, at most 16, each split at least 256 columns).
+// The tile and the contraction split of a product, from the workgroups that will find work
+// (`live`: a device-side limit on rows or columns is taken to leave half the tiles, one on the
+// contraction half the splits).  Without a split where some tile makes two live workgroups per
+// CU: the largest such tile.  Else, where the caller has room for partial products, the largest
+// tile that reaches one live workgroup per CU with at most 16 splits (powers of two, at least
+// 256 columns each) and the fewest splits that do; else the smallest tile, unsplit.
+// Measured on the 8192 x 2048 x 512 workload with 768 features (us per step, the product's
+// kernel group): d q 128 x 64 unsplit 60.7 against 66.0 (128 x 128, 2 splits); d tails 8 splits
+// 60 at any tile against 64.5 (16) and 72.9 (4); hidden 64 x 64 28.0 against 35.3 (128 x 128);
+// d W 128 x 64 with 16 splits 31.1 against 33.0 (128 x 128) and 37.4 (64 x 64).
+struct GemmPlan { int tm, tn, ks; };
+static GemmPlan gemm_nt_bf16_plan(int M, int N, int K, int batches, bool mn_limited, bool k_limited, bool may_split) {
+    const int cand[3][2] = {{128, 128}, {128, 64}, {64, 64}};
+    auto tiles = [&](const int* t) { return (long)(M / t[0]) * (N / t[1]) * batches / (mn_limited ? 2 : 1); };
+    for (const auto& t : cand)
+        if (tiles(t) >= 512) return {t[0], t[1], 1};
+    if (may_split) {
+        const int k_div = k_limited ? 2 : 1;
+        for (const auto& t : cand) {
+            GemmPlan p = {t[0], t[1], 1};
+            auto can_double = [&]() { return p.ks < 16 && K % (2 * p.ks * GB_K) == 0 && K / (2 * p.ks) >= 256; };
+            while (tiles(t) * p.ks / k_div < 256 && can_double()) p.ks *= 2;
+            if (tiles(t) * p.ks / k_div >= 256) return p;
+        }
+    }
+    return {64, 64, 1};
+}
+
+// Room for the partial products of a split contraction: the largest split any combination of
+// limits may choose (batches * ksplit * M * N floats).
 int gemm_nt_bf16_ksplit(int M, int N, int K, int batches) {
-    const long tiles = (long)(M / GB_T) * (N / GB_T) * batches;
     int ks = 1;
-    while (ks < 16 && tiles * ks < 512 && K % (2 * ks * GB_K) == 0 && K / (2 * ks) >= 256) ks *= 2;
+    for (int f = 0; f < 4; ++f) ks = std::max(ks, gemm_nt_bf16_plan(M, N, K, batches, f & 1, f & 2, true).ks);
     return ks;
 }
 
@@ -1045,14 +1101,23 @@ __global__ __launch_bounds__(256) void k_sum_split_batches(const float* __restri
 // products are added in split order.  Splitting needs ldc == N (dense partials).
 void launch_gemm_nt_bf16(const GemmNT& g0, hipStream_t stream) {
     GemmNT g = g0;
-    g.ksplit = (g.part && g.ldc == g.N && !g.add_base) ? gemm_nt_bf16_ksplit(g.M, g.N, g.K, g.batches) : 1;
-    const dim3 grid = tile_grid(g.N / GB_T, g.M / GB_T, g.batches * g.ksplit);
-    if (g.a_kmajor && g.b_kmajor == 2) hipLaunchKernelGGL((k_gemm_nt_bf16<true, 2>), grid, dim3(256), 0, stream, g);
-    else if (g.a_kmajor && g.b_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<true, 1>), grid, dim3(256), 0, stream, g);
-    else if (g.a_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<true, 0>), grid, dim3(256), 0, stream, g);
-    else if (g.b_kmajor == 2) hipLaunchKernelGGL((k_gemm_nt_bf16<false, 2>), grid, dim3(256), 0, stream, g);
-    else if (g.b_kmajor) hipLaunchKernelGGL((k_gemm_nt_bf16<false, 1>), grid, dim3(256), 0, stream, g);
-    else hipLaunchKernelGGL((k_gemm_nt_bf16<false, 0>), grid, dim3(256), 0, stream, g);
+    const GemmPlan t = gemm_nt_bf16_plan(g.M, g.N, g.K, g.batches, g.m_limit || g.n_limit, g.k_limit != nullptr,
+                                         g.part && g.ldc == g.N && !g.add_base);
+    g.ksplit = t.ks;
+    const dim3 grid = tile_grid(g.N / t.tn, g.M / t.tm, g.batches * g.ksplit);
+#define KGE_GEMM_TILE(AK_, BK_)                                                                              \
+    do {                                                                                                     \
+        if (t.tm == 128 && t.tn == 128) hipLaunchKernelGGL((k_gemm_nt_bf16<AK_, BK_, 128, 128>), grid, dim3(256), 0, stream, g); \
+        else if (t.tm == 128) hipLaunchKernelGGL((k_gemm_nt_bf16<AK_, BK_, 128, 64>), grid, dim3(256), 0, stream, g);           \
+        else hipLaunchKernelGGL((k_gemm_nt_bf16<AK_, BK_, 64, 64>), grid, dim3(256), 0, stream, g);          \
+    } while (0)
+    if (g.a_kmajor && g.b_kmajor == 2) KGE_GEMM_TILE(true, 2);
+    else if (g.a_kmajor && g.b_kmajor) KGE_GEMM_TILE(true, 1);
+    else if (g.a_kmajor) KGE_GEMM_TILE(true, 0);
+    else if (g.b_kmajor == 2) KGE_GEMM_TILE(false, 2);
+    else if (g.b_kmajor) KGE_GEMM_TILE(false, 1);
+    else KGE_GEMM_TILE(false, 0);
+#undef KGE_GEMM_TILE
     if (g.ksplit > 1) {
         const int64_t n = (int64_t)g.M * g.N;
         hipLaunchKernelGGL(k_sum_split_batches, dim3((unsigned)((n / 4 + 255) / 256), g.batches), dim3(256), 0,
