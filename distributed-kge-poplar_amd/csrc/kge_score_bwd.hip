@@ -812,7 +812,7 @@ constexpr int L1P_WAVES = 16;
 
 constexpr int L1P_MAX_T = 512;  // tails per block at most (32 per wave)
 
-// the work of one wave with exactly TW tails (TW a multiple of 4): straight-line code over
+// the work of one wave with exactly TW tails (TW even): straight-line code over
 // its tails, their values and sums in registers.
 // signum(a - b) with signum(0) = 0 (poplar_extensions l1distance.codelet.cpp:76-79) from
 // instructions of the fast class only (subtract, fused multiply-add): the difference times 2^126
@@ -830,19 +830,29 @@ constexpr int L1P_MAX_T = 512;  // tails per block at most (32 per wave)
 template <int TW>
 DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restrict__ b_rows,
                          const float* __restrict__ cblk, float* __restrict__ grad_a, float* __restrict__ grad_b,
-                         int B, int T, int Dp, int t0, int t_live, int w, int lane,
+                         int B, int T, int Dp, int t_live, int w, int lane,
                          float (*part)[L1P_WAVES][L1P_CB][64], float (*cs)[L1P_CB][L1P_MAX_T],
                          float (*col_half)[L1P_MAX_T], float (*row_part)[L1P_CB][L1P_WAVES]) {
-    const int tid = threadIdx.x, t4 = t_live / 4;
-    // staging: thread -> (head, four columns) of a chunk's coefficient rows
+    // In LDS a wave's TW columns start at a multiple of four (TWS apart): its reads stay 16-byte
+    // ones when TW is not a multiple of four.  Column c lies at lds_col(c).
+    constexpr int TWS = (TW + 3) & ~3;
+    auto lds_col = [](int c) { return (c / TW) * TWS + c % TW; };
+    const int tid = threadIdx.x, t4 = t_live / 4, l0 = w * TWS;
+    // staging: thread -> (head, four columns) of a chunk's coefficient rows, stored as two pairs
+    // (TW is even, so a pair never straddles two waves' columns)
     const bool stager = tid < L1P_CB * t4;
     const int s_head = tid / t4, s_col = (tid - s_head * t4) * 4;
+    const int s_lo = lds_col(s_col), s_hi = lds_col(s_col + 2);
+    auto stage = [&](int buf, float4 v) __attribute__((always_inline)) {
+        *reinterpret_cast<float2*>(&cs[buf][s_head][s_lo]) = make_float2(v.x, v.y);
+        *reinterpret_cast<float2*>(&cs[buf][s_head][s_hi]) = make_float2(v.z, v.w);
+    };
     // linear parts: thread 512 + t -> column t; threads 512 .. 639 -> (head, wave)
-    const int u = tid - 512;
+    const int u = tid - 512, u_lds = u >= 0 ? lds_col(u) : 0;
     float4 c_next = make_float4(0.f, 0.f, 0.f, 0.f);
     if (stager) {
         c_next = *reinterpret_cast<const float4*>(cblk + (size_t)s_head * T + s_col);
-        *reinterpret_cast<float4*>(&cs[0][s_head][s_col]) = c_next;
+        stage(0, c_next);
     }
     float bt[TW], gt[TW];
 #pragma unroll
@@ -861,22 +871,25 @@ DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restri
         if (b0 > 0) {
 #pragma unroll
             for (int j4 = 0; j4 < TW; j4 += 4) {
-                const float4 h4 = *reinterpret_cast<const float4*>(&col_half[buf ^ 1][t0 + j4]);
-                gt[j4] -= h4.x, gt[j4 + 1] -= h4.y, gt[j4 + 2] -= h4.z, gt[j4 + 3] -= h4.w;
+                const float4 h4 = *reinterpret_cast<const float4*>(&col_half[buf ^ 1][l0 + j4]);
+                const float hv[4] = {h4.x, h4.y, h4.z, h4.w};
+#pragma unroll
+                for (int x = 0; x < 4; ++x)
+                    if (j4 + x < TW) gt[j4 + x] -= hv[x];
             }
         }
         if (u >= 0) {
             if (u < t_live) {
                 float sum = 0.f;
 #pragma unroll
-                for (int h = 0; h < L1P_CB; ++h) sum += cs[buf][h][u];
-                col_half[buf][u] = 0.5f * sum;
+                for (int h = 0; h < L1P_CB; ++h) sum += cs[buf][h][u_lds];
+                col_half[buf][u_lds] = 0.5f * sum;
             }
             if (u < L1P_CB * L1P_WAVES) {
                 const int h = u / L1P_WAVES, v = u % L1P_WAVES;
                 float sum = 0.f;
 #pragma unroll
-                for (int j = 0; j < TW; ++j) sum += cs[buf][h][v * TW + j];
+                for (int j = 0; j < TW; ++j) sum += cs[buf][h][v * TWS + j];
                 row_part[buf][h][v] = sum;
             }
         }
@@ -885,7 +898,7 @@ DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restri
             const float a = a_q0;
             a_q0 = a_q1;
             a_q1 = a_rows[(size_t)min(b0 + bi + 2, B - 1) * Dp];
-            const float* c = &cs[buf][bi][t0];
+            const float* c = &cs[buf][bi][l0];
             float gp = 0.f;
 #pragma unroll
             for (int j4 = 0; j4 < TW; j4 += 4) {
@@ -893,6 +906,7 @@ DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restri
                 const float cv[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
                 for (int x = 0; x < 4; ++x) {
+                    if (j4 + x >= TW) continue;
                     const float p = __builtin_amdgcn_fmed3f(fmaf(a - bt[j4 + x], 0x1p126f, 0.5f), 0.f, 1.f);
                     gp = fmaf(cv[x], p, gp);
                     gt[j4 + x] = fmaf(cv[x], p, gt[j4 + x]);
@@ -900,7 +914,7 @@ DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restri
             }
             part[buf][w][bi][lane] = gp;
         }
-        if (stager && more) *reinterpret_cast<float4*>(&cs[buf ^ 1][s_head][s_col]) = c_next;
+        if (stager && more) stage(buf ^ 1, c_next);
         __syncthreads();
         // waves 0 .. 7 add the 16 partials of head b0 + w
         if (w < L1P_CB) {
@@ -912,7 +926,7 @@ DEVINL void l1_pair_wave(const float* __restrict__ a_rows, const float* __restri
     }
     const int last = ((B / L1P_CB) - 1) & 1;
 #pragma unroll
-    for (int j = 0; j < TW; ++j) grad_b[(size_t)j * Dp] = -2.f * (gt[j] - col_half[last][t0 + j]);
+    for (int j = 0; j < TW; ++j) grad_b[(size_t)j * Dp] = -2.f * (gt[j] - col_half[last][l0 + j]);
 }
 
 __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restrict__ operands,
@@ -931,8 +945,13 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
     const TileId tile = xcd_tile(Dp / 64, 1, (int)gridDim.x / (Dp / 64));
     const int d = tile.z, lane = threadIdx.x & 63, k = tile.x * 64 + lane;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // merged tails: the block's live columns (a multiple of 64), split evenly over the waves
-    const int t_live = __builtin_amdgcn_readfirstlane(tail_limit(tcount, d, T, tpad));
+    // merged tails: the block's distinct tails in whole groups of 32 (two per wave), split evenly
+    // over the waves.  The columns between that and the forward pass's limit (whole groups of
+    // `tpad`) stand for no tail position: their coefficients are zero and nothing reads their
+    // gradient rows.  331 instead of 343 columns per block on average on the 22.8M-row workload,
+    // and the launch's time follows that average (158.6 -> 155 us), not its largest block.
+    const int t_fwd = tail_limit(tcount, d, T, tpad);
+    const int t_live = __builtin_amdgcn_readfirstlane(tcount ? min(t_fwd, ((int)tcount[d] + 31) & ~31) : t_fwd);
     const int tw = t_live / L1P_WAVES, t0 = w * tw;
     const float* a_rows = operands + (size_t)(a_c0 + d * B) * Dp + k;
     const float* b_rows = operands + (size_t)(b_c0 + d * T + t0) * Dp + k;
@@ -940,9 +959,10 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
     float* grad_a = grad + (size_t)(a_c0 + d * B) * Dp + k;
     float* grad_b = grad + (size_t)(b_c0 + d * T + t0) * Dp + k;
 #define KGE_L1P(TW_) \
-    case TW_: l1_pair_wave<TW_>(a_rows, b_rows, cblk, grad_a, grad_b, B, T, Dp, t0, t_live, w, lane, lds.part, lds.cs, lds.col_half, lds.row_part); break;
-    switch (tw) {  // one of eight copies of the loop, chosen per block
-        KGE_L1P(4) KGE_L1P(8) KGE_L1P(12) KGE_L1P(16) KGE_L1P(20) KGE_L1P(24) KGE_L1P(28) KGE_L1P(32)
+    case TW_: l1_pair_wave<TW_>(a_rows, b_rows, cblk, grad_a, grad_b, B, T, Dp, t_live, w, lane, lds.part, lds.cs, lds.col_half, lds.row_part); break;
+    switch (tw) {  // one of sixteen copies of the loop, chosen per block
+        KGE_L1P(2) KGE_L1P(4) KGE_L1P(6) KGE_L1P(8) KGE_L1P(10) KGE_L1P(12) KGE_L1P(14) KGE_L1P(16)
+        KGE_L1P(18) KGE_L1P(20) KGE_L1P(22) KGE_L1P(24) KGE_L1P(26) KGE_L1P(28) KGE_L1P(30) KGE_L1P(32)
     }
 #undef KGE_L1P
 }
@@ -950,7 +970,7 @@ __global__ __launch_bounds__(1024) void k_score_bwd_l1_pair(const float* __restr
 // shapes the paired L1 kernel takes: tails split evenly over 16 waves, whole
 // chunks of heads, whole 64-column slices, and enough workgroups for the chip
 static bool l1_pair_ok(const ScoreShape& sh) {
-    // (T % 64 == 0: every live count is a multiple of 64, 4 tails per wave at least)
+    // (T % 64 == 0: every live count is a multiple of 32, 2 tails per wave at least)
     return sh.T % 64 == 0 && sh.T >= 128 && sh.T <= L1P_MAX_T && sh.B % L1P_CB == 0 &&
            sh.Dp % 64 == 0 && sh.S * (sh.Dp / 64) >= 128 && (!sh.tcount || sh.tpad == 64);
 }
