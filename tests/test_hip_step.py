@@ -712,6 +712,32 @@ def test_step_repeated_tails(oracle64, name, kind):
              **{"execution.merge_tails": False})
 
 
+def _tails_with_distinct_counts(c, n_step, rng):
+    """Raw-id batches (kge_synthetic.raw_batch) in which block d's T tail positions hold exactly
+    counts[d] distinct rows: each of them once, then repeats."""
+    S, A, B = c["n_shard"], c["a2a"], c["batch"]
+    T = S * A
+    batch = K.raw_batch(c, n_step, rng, zipf=False)
+    counts = np.concatenate([[1, 20, 33, 64, 90, 100, 129, 150, 190, 200, 230, 256, 280, 300, 320, 330, 352, 370,
+                              385, 400, 416, 440, 449, 470, 480, 490, 500, 512], rng.integers(1, T + 1, S)])[:S]
+    for step in range(n_step):
+        for d in range(S):
+            n = int(min(counts[(d + step) % S], T))
+            pool = rng.choice(np.arange(1, c["n_entity"]), n, replace=False).astype(np.uint32)
+            rows = np.concatenate([pool, pool[rng.integers(0, n, T - n)]])
+            rng.shuffle(rows)
+            # block d's tails: slots B + d A .. + A - 1 of every source shard's `remote`
+            batch["remote"][:, step, B + d * A:B + (d + 1) * A] = rows.reshape(S, A)
+    return batch
+
+
+def test_step_paired_l1_distinct_tail_counts(oracle64):
+    """The paired L1 backward splits a block's distinct tails, in whole groups of 32, over its 16
+    waves and has one copy of its loop per tails-per-wave count (2, 4, ... 32): blocks with 1 to
+    512 distinct tails of 512 positions, against the oracle."""
+    run_case(oracle64, dict(CASES["paired_l1_t512"]), n_step=2, batch_fn=_tails_with_distinct_counts)
+
+
 def test_host_arrays_are_checked_chunk_by_chunk():
     """Host index arrays are checked, re-ordered and uploaded in chunks of 2, 4, 8, ... steps beside
     the device's work.  An index out of range raises as before; the chunks in front of the
