@@ -309,14 +309,22 @@ __global__ __launch_bounds__(256) void k_sort_scatter(SortJob j0, SortJob j1, in
                 tot[q] = d < DIG ? hseg[(size_t)n_tiles * DIG + d] : 0u;
             }
         } else
-        for (int t = 0; t < n_tiles; ++t) {
+        for (int t0 = 0; t0 < n_tiles; t0 += 8) {  // eight tiles' rows in flight: one round trip per eight tiles
+            uint32_t c[8][DPT];
 #pragma unroll
-            for (int q = 0; q < DPT; ++q) {
-                const int d = q * 256 + tid;
-                const uint32_t c = d < DIG ? hseg[(size_t)t * DIG + d] : 0u;
-                tot[q] += c;
-                pre[q] += t < tile ? c : 0u;
-            }
+            for (int x = 0; x < 8; ++x)
+#pragma unroll
+                for (int q = 0; q < DPT; ++q) {
+                    const int d = q * 256 + tid;
+                    c[x][q] = (t0 + x < n_tiles && d < DIG) ? hseg[(size_t)(t0 + x) * DIG + d] : 0u;
+                }
+#pragma unroll
+            for (int x = 0; x < 8; ++x)
+#pragma unroll
+                for (int q = 0; q < DPT; ++q) {
+                    tot[q] += c[x][q];
+                    pre[q] += t0 + x < tile ? c[x][q] : 0u;
+                }
         }
 #pragma unroll
         for (int q = 0; q < DPT; ++q) s_tot[q * 256 + tid] = tot[q];
