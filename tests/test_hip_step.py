@@ -35,6 +35,10 @@ CASES = {
     # tile-aligned shapes (positives % 128, tails % 128, dim % 64): the matrix-core fast path
     "aligned_l2": dict(distance_fn="L2", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
                        n_entity=3000, n_relation=8, gamma=6.0),
+    # L1 on whole 64 x 64 tiles and 32-column slabs: the vector forward kernel's form with the next
+    # slab's loads in flight
+    "aligned_l1": dict(distance_fn="L1", n_shard=2, batch=128, a2a=64, dim=64, feature=0,
+                       n_entity=3000, n_relation=8, gamma=6.0),
     "aligned_l2_wide": dict(distance_fn="L2", n_shard=4, batch=256, a2a=64, dim=128, feature=0,
                             n_entity=5000, n_relation=8, gamma=6.0, shared_table=True),
     "aligned_distmult": dict(score_fn="DistMult", distance_fn="MatMul", loss_fn="softmax",
@@ -300,7 +304,7 @@ def test_step_vs_oracle(oracle64, name):
 
 
 @pytest.mark.parametrize("name", ["l2_logsigmoid", "l2_softmax", "distmult_softmax_feat", "mid_l2",
-                                  "transe_matmul", "shared_l2", "paired_l1_t256"])
+                                  "transe_matmul", "shared_l2", "paired_l1_t256", "aligned_l2", "aligned_l1"])
 def test_step_vs_oracle_valu_scoring(oracle64, name):
     # the same cases on the VALU scoring kernels (default: matrix cores)
     run_case(oracle64, CASES[name], **{"execution.scoring": "valu"})
