@@ -277,6 +277,7 @@ struct kge_engine {
     DevBuf<uint32_t> e_uniq, e_seg, e_coff, e_cpos, e_clen, e_counts, e_item_row, e_real;
     DevBuf<uint32_t> r_uniq, r_seg, r_coff, r_cpos, r_clen, r_counts, r_real;
     DevBuf<uint32_t> e_hot, e_hot_count, r_hot, r_hot_count;  // the rows with chunks, per step
+    DevBuf<uint32_t> e_crow, r_crow;                          // the row of every chunk, per step
     DevBuf<uint32_t> nearflag;
     // additive setting execution.merge_tails (default true): a block scores one column per distinct
     // tail row, weighted by how many of its tail positions hold that row
@@ -683,6 +684,7 @@ void allocate(kge_engine& E) {
     E.e_clen.alloc(ns * E.e_cstride);
     E.e_counts.alloc(ns * 2);
     E.e_hot.alloc(ns * E.e_cstride);
+    E.e_crow.alloc(ns * E.e_cstride);
     E.e_hot_count.alloc(ns * 2);
     if (E.F) E.e_item_row.alloc(ns * R);
     E.r_ustride = E.n_rel_rows;
@@ -695,6 +697,7 @@ void allocate(kge_engine& E) {
     E.r_clen.alloc(ns * E.r_cstride);
     E.r_counts.alloc(ns * 2);
     E.r_hot.alloc(ns * E.r_cstride);
+    E.r_crow.alloc(ns * E.r_cstride);
     E.r_hot_count.alloc(ns * 2);
 
     E.coef.alloc(SB * E.T);
@@ -1042,6 +1045,7 @@ void run_plan(kge_engine& E, int s0, int sn, hipStream_t st) {
     ep.item_row = E.F ? E.e_item_row.p + s0 * R : nullptr;
     ep.seg_real = E.e_real.p + (size_t)s0 * ep.u_stride;
     ep.hot_rows = E.e_hot.p + (size_t)s0 * ep.c_stride; ep.hot_count = E.e_hot_count.p + 2 * s0;
+    ep.chunk_row = E.e_crow.p + (size_t)s0 * ep.c_stride;
     ep.host_counts = E.d_e_counts + 4 * (size_t)s0;
 
     const uint32_t* rk = rs.result_in_b ? E.rk_b.p : E.rk_a.p;
@@ -1060,6 +1064,7 @@ void run_plan(kge_engine& E, int s0, int sn, hipStream_t st) {
     rp.item_row = nullptr;
     rp.seg_real = E.r_real.p + (size_t)s0 * rp.u_stride;
     rp.hot_rows = E.r_hot.p + (size_t)s0 * rp.c_stride; rp.hot_count = E.r_hot_count.p + 2 * s0;
+    rp.chunk_row = E.r_crow.p + (size_t)s0 * rp.c_stride;
     rp.host_counts = E.d_r_counts + 4 * (size_t)s0;
     launch_find_segments2(ej, &rj, sn, E.seg_scratch.p, st);  // both plans' segments in one launch
     HIP_CHECK(hipGetLastError());
@@ -1412,6 +1417,8 @@ void run_step(kge_engine& E, int i) {
         he.max_hot = (int)E.h_e_counts[4 * (size_t)i + 2];
         hr.hot_rows = E.r_hot.p + (size_t)i * E.r_cstride; hr.hot_count = E.r_hot_count.p + 2 * i;
         hr.max_hot = (int)E.h_r_counts[4 * (size_t)i + 2];
+        he.chunk_row = E.e_crow.p + (size_t)i * E.e_cstride; he.n_chunks = (int)E.h_e_counts[4 * (size_t)i + 1];
+        hr.chunk_row = E.r_crow.p + (size_t)i * E.r_cstride; hr.n_chunks = (int)E.h_r_counts[4 * (size_t)i + 1];
         launch_adam_rows_hot2(ar, hr, ae, he, st);
     } else {
         // the relation rows first: they are few and slow (a dozen contributions each, two rounds

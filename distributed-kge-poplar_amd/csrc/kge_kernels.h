@@ -128,6 +128,7 @@ struct SegPlan {
     // row with the most}
     uint32_t* hot_rows;
     uint32_t* hot_count;
+    uint32_t* chunk_row = nullptr;  // or null: [n_seg, c_stride] distinct-row index of each chunk
     // or null: [n_seg, 4] {distinct rows, chunks, rows with chunks, real items of the biggest row}
     // once more, in device-visible host memory (the host sizes its launches from them)
     uint32_t* host_counts;
@@ -333,6 +334,11 @@ struct HotRows {
     const uint32_t* hot_rows;
     const uint32_t* hot_count;
     int max_hot;
+    // or null / 0: the row of every chunk (SegPlan::chunk_row) and an upper bound of the step's
+    // chunks: the launch then has one workgroup per chunk, and the first 1, 2, 4 or 8 of a row's
+    // chunk workgroups share its columns
+    const uint32_t* chunk_row = nullptr;
+    int n_chunks = 0;
 };
 void launch_adam_rows_hot2(const AdamArgs& a0, const HotRows& h0, const AdamArgs& a1, const HotRows& h1,
                            hipStream_t stream);

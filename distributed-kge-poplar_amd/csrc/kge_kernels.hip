@@ -1835,25 +1835,45 @@ constexpr int kHotColumns = 32;
 // and five waves; 4 and 16 loads at eight waves measured the same within a microsecond);
 // four waves per workgroup (2, 8 and 16 measured slower)
 constexpr int kHotLoads = 8, kHotWaves = 4;
-template <bool MF32>
+// BYCHUNK: one hot workgroup per chunk of the plan instead of one per (row with chunks, 32
+// columns).  A row of nch chunks has nch consecutive chunk workgroups; the first 1, 2, 4 or 8
+// of them (the largest power of two <= min(nch, 8)) split its columns evenly and each sums all
+// of the row's contributions over its share, the others return.  Rows with one chunk
+// (17 .. 64 contributions) then cost one workgroup instead of eight.
+template <bool MF32, bool BYCHUNK>
 __global__ __launch_bounds__(kHotWaves * 64) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_adam_rows_hot(AdamArgs a0, HotRows h0, AdamArgs a1, HotRows h1) {
-    constexpr int HC = kHotColumns, HS = 64 / (HC / 4);  // columns per workgroup, slots per wave
-    __shared__ __attribute__((aligned(16))) float part[kHotWaves - 1][HC];
+    __shared__ __attribute__((aligned(16))) float part[kHotWaves - 1][BYCHUNK ? 256 : kHotColumns];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int ns0 = (a0.Dp + HC - 1) / HC, ns1 = (a1.Dp + HC - 1) / HC;
-    const int hot0 = ns0 * h0.max_hot, hot1 = ns1 * h1.max_hot;
+    const int ns0 = (a0.Dp + kHotColumns - 1) / kHotColumns, ns1 = (a1.Dp + kHotColumns - 1) / kHotColumns;
+    const int hot0 = BYCHUNK ? (a0.max_rows ? h0.n_chunks : 0) : ns0 * h0.max_hot;
+    const int hot1 = BYCHUNK ? (a1.max_rows ? h1.n_chunks : 0) : ns1 * h1.max_hot;
     int b = blockIdx.x;
     if (b < hot0 + hot1) {
         const bool second = b >= hot0;
         const AdamArgs& a = second ? a1 : a0;
         const HotRows& h = second ? h1 : h0;
         if (second) b -= hot0;
-        const int ns = second ? ns1 : ns0, hb = b / ns, cb = b - hb * ns;
-        if (hb >= (int)h.hot_count[0]) return;
-        const int u = (int)h.hot_rows[hb], Dp = a.Dp;
+        const int Dp = a.Dp;
+        int u, col0, ncg;  // the row, this workgroup's first column and its groups of four columns
+        if constexpr (BYCHUNK) {
+            if (b >= (int)a.counts[1]) return;
+            u = (int)h.chunk_row[b];
+            const int q0 = (int)a.chunk_off[u], nch = (int)a.chunk_off[u + 1] - q0;
+            const int shares = nch >= 8 ? 8 : nch >= 4 ? 4 : nch >= 2 ? 2 : 1;
+            const int cb = b - q0;
+            if (cb >= shares) return;
+            const int HC = Dp / shares;
+            col0 = cb * HC; ncg = HC / 4;
+        } else {
+            const int ns = second ? ns1 : ns0, hb = b / ns, cb = b - hb * ns;
+            if (hb >= (int)h.hot_count[0]) return;
+            u = (int)h.hot_rows[hb];
+            col0 = cb * kHotColumns; ncg = kHotColumns / 4;
+        }
+        const int HS = 64 / ncg;  // contributions per load instruction (slots of a wave)
         const uint32_t key = a.uniq_key[u], pos = a.seg_start[u], n = a.seg_real[u];
         const float alpha = a.alpha[a.rows_per_alpha ? key / a.rows_per_alpha : 0u];
-        const int cg = lane & (HC / 4 - 1), slot = lane / (HC / 4), col = cb * HC + cg * 4;
+        const int cg = lane & (ncg - 1), slot = lane / ncg, col = col0 + cg * 4;
         const bool active = col < Dp;
         // this wave's quarter of the contributions, in whole groups of HS
         const uint32_t groups = (n + HS - 1) / HS, gshare = (groups + kHotWaves - 1) / kHotWaves;
@@ -1876,10 +1896,17 @@ __global__ __launch_bounds__(kHotWaves * 64) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
             for (int x = 0; x < kHotLoads; ++x) acc = f4add(acc, v[x]);
         }
+        if constexpr (BYCHUNK) {
+            for (int off = ncg; off < 64; off <<= 1) {
+                acc.x += __shfl_xor(acc.x, off, 64); acc.y += __shfl_xor(acc.y, off, 64);
+                acc.z += __shfl_xor(acc.z, off, 64); acc.w += __shfl_xor(acc.w, off, 64);
+            }
+        } else {
 #pragma unroll
-        for (int off = HC / 4; off < 64; off <<= 1) {
-            acc.x += __shfl_xor(acc.x, off, 64); acc.y += __shfl_xor(acc.y, off, 64);
-            acc.z += __shfl_xor(acc.z, off, 64); acc.w += __shfl_xor(acc.w, off, 64);
+            for (int off = kHotColumns / 4; off < 64; off <<= 1) {
+                acc.x += __shfl_xor(acc.x, off, 64); acc.y += __shfl_xor(acc.y, off, 64);
+                acc.z += __shfl_xor(acc.z, off, 64); acc.w += __shfl_xor(acc.w, off, 64);
+            }
         }
         if (wave > 0 && slot == 0) *reinterpret_cast<float4*>(&part[wave - 1][cg * 4]) = acc;
         __syncthreads();
@@ -1957,16 +1984,25 @@ __global__ __launch_bounds__(kHotWaves * 64) __attribute__((amdgpu_waves_per_eu(
     }
 }
 
+// the per-chunk form takes row widths that split evenly into 1 .. 8 shares of whole 16-byte groups
+static bool hot_by_chunk_ok(const AdamArgs& a, const HotRows& h) {
+    return a.max_rows == 0 || (h.chunk_row && a.Dp >= 32 && a.Dp <= 256 && (a.Dp & (a.Dp - 1)) == 0);
+}
+
 void launch_adam_rows_hot2(const AdamArgs& a0, const HotRows& h0, const AdamArgs& a1, const HotRows& h1,
                            hipStream_t stream) {
-    const int hot = ((a0.Dp + kHotColumns - 1) / kHotColumns) * h0.max_hot +
-                    ((a1.Dp + kHotColumns - 1) / kHotColumns) * h1.max_hot;
+    const bool by_chunk = hot_by_chunk_ok(a0, h0) && hot_by_chunk_ok(a1, h1);
+    const int hot = by_chunk ? (a0.max_rows ? h0.n_chunks : 0) + (a1.max_rows ? h1.n_chunks : 0)
+                             : ((a0.Dp + kHotColumns - 1) / kHotColumns) * h0.max_hot +
+                               ((a1.Dp + kHotColumns - 1) / kHotColumns) * h1.max_hot;
     const int slabs = (std::max(a0.Dp, a1.Dp) + 255) / 256;
     const dim3 grid(hot + (a0.max_rows * slabs + kHotWaves - 1) / kHotWaves + (a1.max_rows * slabs + kHotWaves - 1) / kHotWaves);
     if (grid.x == 0) return;
     const bool f32 = (a0.max_rows == 0 || a0.m_etype == ET_F32) && (a1.max_rows == 0 || a1.m_etype == ET_F32);
-    if (f32) hipLaunchKernelGGL((k_adam_rows_hot<true>), grid, dim3(kHotWaves * 64), 0, stream, a0, h0, a1, h1);
-    else hipLaunchKernelGGL((k_adam_rows_hot<false>), grid, dim3(kHotWaves * 64), 0, stream, a0, h0, a1, h1);
+    if (by_chunk && f32) hipLaunchKernelGGL((k_adam_rows_hot<true, true>), grid, dim3(kHotWaves * 64), 0, stream, a0, h0, a1, h1);
+    else if (by_chunk) hipLaunchKernelGGL((k_adam_rows_hot<false, true>), grid, dim3(kHotWaves * 64), 0, stream, a0, h0, a1, h1);
+    else if (f32) hipLaunchKernelGGL((k_adam_rows_hot<true, false>), grid, dim3(kHotWaves * 64), 0, stream, a0, h0, a1, h1);
+    else hipLaunchKernelGGL((k_adam_rows_hot<false, false>), grid, dim3(kHotWaves * 64), 0, stream, a0, h0, a1, h1);
 }
 
 static void launch_adam_kernel(const AdamArgs& a0, const AdamArgs& a1, hipStream_t stream) {

@@ -675,6 +675,7 @@ __global__ __launch_bounds__(256) void k_seg_chunks(SegJob j0, SegJob j1, int n_
     uint32_t* __restrict__ chunk_pos = plan.chunk_pos + (size_t)seg * plan.c_stride;
     uint32_t* __restrict__ chunk_len = plan.chunk_len + (size_t)seg * plan.c_stride;
     uint32_t* __restrict__ hot = plan.hot_rows ? plan.hot_rows + (size_t)seg * plan.c_stride : nullptr;
+    uint32_t* __restrict__ crow = plan.chunk_row ? plan.chunk_row + (size_t)seg * plan.c_stride : nullptr;
     const uint32_t* info_seg = tile_info + (size_t)w.slot * max_tiles * kSegInfo;
 
     // chunks and rows with chunks that the earlier tiles own
@@ -713,6 +714,7 @@ __global__ __launch_bounds__(256) void k_seg_chunks(SegJob j0, SegJob j1, int n_
                 for (uint32_t l = 0; l < nch[x]; ++l) {
                     chunk_pos[cb + l] = s + l * chunk;
                     chunk_len[cb + l] = min(chunk, real[x] - l * chunk);
+                    if (crow) crow[cb + l] = u;
                 }
                 cb += nch[x];
                 if (hot) hot[hb] = u;
