@@ -93,15 +93,29 @@ __global__ __launch_bounds__(256) void k_gather_operands_multi(RowSource ent, co
                                                                float* __restrict__ out, TailCols tc) {
     const int lane = threadIdx.x & 63;
     const int c0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW;
+    if (c0 >= n_rows) return;
+    // the row numbers are asked for together with the block's tail count (rows past it are
+    // never used, but their slots hold valid numbers): one round trip instead of two in front
+    // of the rows themselves
+    uint32_t key[RPW], rkey[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        const int c = min(c0 + r, n_rows - 1);  // a row past the end repeats the last one
+        key[r] = ent.index ? ent.index[c] : (uint32_t)c;
+        rkey[r] = (c < n_head && rel_mode) ? crel[c] : 0u;
+    }
     // (limits are multiples of RPW: the rows of a wave are live or not together)
-    if (c0 >= n_rows || !tc.live(c0 - n_head)) return;
+    const bool live = tc.live(c0 - n_head);
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) asm volatile("" : "+v"(key[r]), "+v"(rkey[r]));
+    if (!live) return;
     const char* row[RPW];
     const float* rrow[RPW];
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
-        const int c = min(c0 + r, n_rows - 1);  // a row past the end repeats the last one
-        row[r] = row_ptr(ent, c);
-        rrow[r] = (c < n_head && rel_mode) ? rel + (size_t)crel[c] * Dp : nullptr;
+        const int c = min(c0 + r, n_rows - 1);
+        row[r] = ent.base + (int64_t)key[r] * ent.pitch;
+        rrow[r] = (c < n_head && rel_mode) ? rel + (size_t)rkey[r] * Dp : nullptr;
     }
     for (int k = lane * 4; k < Dp; k += 256) {
         float4 v[RPW], q[RPW];
